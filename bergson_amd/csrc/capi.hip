@@ -1,0 +1,87 @@
+// extern "C" entry points of libbergson_amd.so (declared in include/bergson_amd.h).
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "common.hpp"
+
+namespace bgx {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  set_error("%s failed: %s (%d)", what, hipGetErrorString(e), (int)e);
+  return (int)e;
+}
+
+size_t collect_workspace_bytes(int n_modules, int N, int S, int p);
+int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules, int N, int S, int p, int in_dtype,
+                 const int32_t* lengths, const int64_t* rows_or_offsets, void* out, int64_t out_row_stride,
+                 int out_dtype, float lo, float hi, void* ws, size_t ws_bytes, void* stream);
+int adafactor_scales_impl(const float* row, int O, const float* col, int I, int dtype, float* row_scale,
+                          float* col_scale, void* stream);
+int unit_normalize_impl(void* rows, int64_t n_rows, int64_t D, int64_t stride, int dtype, void* stream);
+size_t scan_workspace_bytes(int Q, int k, int64_t chunk_rows);
+int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int dtype, const void* queries, int Q,
+              float query_scale, int unit_norm, int k, int64_t row_base, float* topk_val, int64_t* topk_idx,
+              float* row_max, float* scores, float* sumsq, void* ws, size_t ws_bytes, int64_t chunk_rows,
+              void* stream);
+
+}  // namespace bgx
+
+extern "C" {
+
+int bgx_abi_version(void) { return BGX_ABI_VERSION; }
+
+const char* bgx_last_error(void) { return bgx::g_err; }
+
+int bgx_adafactor_scales(const float* row_dev, int32_t O, const float* col_dev, int32_t I, int32_t dtype,
+                         float* row_scale_dev, float* col_scale_dev, void* stream) {
+  return bgx::adafactor_scales_impl(row_dev, O, col_dev, I, dtype, row_scale_dev, col_scale_dev, stream);
+}
+
+size_t bgx_collect_workspace_bytes(int32_t n_modules, int32_t N, int32_t S, int32_t p) {
+  return bgx::collect_workspace_bytes(n_modules, N, S, p);
+}
+
+int bgx_collect_seq(const bgx_module_desc* mods_host, int32_t n_modules, int32_t N, int32_t S, int32_t p,
+                    int32_t in_dtype, const int32_t* lengths_dev, const int64_t* out_rows_dev, void* out_dev,
+                    int64_t out_row_stride, int32_t out_dtype, float clamp_lo, float clamp_hi, void* workspace_dev,
+                    size_t workspace_bytes, void* stream) {
+  return bgx::collect_impl(false, mods_host, n_modules, N, S, p, in_dtype, lengths_dev, out_rows_dev, out_dev,
+                           out_row_stride, out_dtype, clamp_lo, clamp_hi, workspace_dev, workspace_bytes, stream);
+}
+
+int bgx_collect_tok(const bgx_module_desc* mods_host, int32_t n_modules, int32_t N, int32_t S, int32_t p,
+                    int32_t in_dtype, const int32_t* lengths_dev, const int64_t* row_offsets_dev, void* out_dev,
+                    int64_t out_row_stride, int32_t out_dtype, float clamp_lo, float clamp_hi, void* workspace_dev,
+                    size_t workspace_bytes, void* stream) {
+  return bgx::collect_impl(true, mods_host, n_modules, N, S, p, in_dtype, lengths_dev, row_offsets_dev, out_dev,
+                           out_row_stride, out_dtype, clamp_lo, clamp_hi, workspace_dev, workspace_bytes, stream);
+}
+
+int bgx_unit_normalize_rows(void* rows_dev, int64_t n_rows, int64_t D, int64_t row_stride, int32_t dtype,
+                            void* stream) {
+  return bgx::unit_normalize_impl(rows_dev, n_rows, D, row_stride, dtype, stream);
+}
+
+size_t bgx_scan_workspace_bytes(int32_t Q, int32_t k, int64_t chunk_rows) {
+  return bgx::scan_workspace_bytes(Q, k, chunk_rows);
+}
+
+int bgx_scan(const void* store_dev, int64_t n_rows, int64_t D, int64_t store_row_stride, int32_t dtype,
+             const void* queries_dev, int32_t Q, float query_scale, int32_t unit_norm, int32_t k, int64_t row_base,
+             float* topk_val_dev, int64_t* topk_idx_dev, float* row_max_dev, float* scores_dev, float* sumsq_dev,
+             void* workspace_dev, size_t workspace_bytes, int64_t chunk_rows, void* stream) {
+  return bgx::scan_impl(store_dev, n_rows, D, store_row_stride, dtype, queries_dev, Q, query_scale, unit_norm, k,
+                        row_base, topk_val_dev, topk_idx_dev, row_max_dev, scores_dev, sumsq_dev, workspace_dev,
+                        workspace_bytes, chunk_rows, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,524 @@
+// Fused per-module gradient collection for gfx950 (MI355X).
+//
+// One workgroup owns a tile of 64 tokens of one sequence of one module and
+//   1. projects the activations  a'[t, j] = sum_k a[t, k] * (R_in[j, k] * col_scale[k])
+//   2. projects the output grads g'[t, i] = sum_k g[t, k] * (R_out[i, k] * row_scale[k])
+//      both with MFMA tiles fed straight from global memory (a and g are read
+//      exactly once; the p x K projection matrices come from L2),
+//   3. per-sequence: reduces P[i, j] = sum_t g'[t, i] * a'[t, j] over its tokens
+//      and writes one fp32 partial; a second tiny kernel adds the partials of a
+//      sequence in a fixed order, clamps, casts and writes the store row.
+//      per-token: writes flatten(g'[t] (x) a'[t]) for every valid token.
+//
+// Reference op sequence: bergson/collector/collector.py:518-543 (forward
+// hook), :646-742 (backward hook), bergson/builder.py:17-32 (concatenation).
+//
+// The 4 waves of a workgroup split the K dimension (I, then O) between them,
+// so no barrier is needed in the streaming loop; their partial projections
+// are combined through LDS in a fixed pairwise order (w0+w2)+(w1+w3).
+
+#include "common.hpp"
+
+namespace bgx {
+
+constexpr int TILE_T = 64;  // tokens per workgroup
+constexpr int MT = TILE_T / 16;
+constexpr int COLLECT_THREADS = 256;
+
+// ---- MFMA step per element type ---------------------------------------------
+// A "k-step" of one wave covers KS consecutive k; lane (r = lane%16, q = lane/16)
+// holds EPL consecutive elements starting at k0 + q*EPL of row r (16 bytes).
+template <typename T>
+struct Mma;
+
+template <>
+struct Mma<bf16_t> {
+  static constexpr int EPL = 8;
+  static constexpr int KS = 32;
+  __device__ static void mma(const uint4& a, const uint4& b, f32x4& c) {
+    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  __device__ static float get(const uint4& v, int e) {
+    const uint32_t w = (&v.x)[e >> 1];
+    return bf16_bits_to_f32((e & 1) ? (w >> 16) : (w & 0xffffu));
+  }
+  __device__ static void set(uint4& v, int e, float f) {
+    uint32_t& w = (&v.x)[e >> 1];
+    const uint32_t b = f32_to_bf16_bits(f);
+    w = (e & 1) ? ((w & 0x0000ffffu) | (b << 16)) : ((w & 0xffff0000u) | b);
+  }
+};
+
+template <>
+struct Mma<f16_t> {
+  static constexpr int EPL = 8;
+  static constexpr int KS = 32;
+  __device__ static void mma(const uint4& a, const uint4& b, f32x4& c) {
+    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                               __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  __device__ static float get(const uint4& v, int e) {
+    const uint32_t w = (&v.x)[e >> 1];
+    return f16_bits_to_f32((e & 1) ? (w >> 16) : (w & 0xffffu));
+  }
+  __device__ static void set(uint4& v, int e, float f) {
+    uint32_t& w = (&v.x)[e >> 1];
+    const uint32_t b = f32_to_f16_bits(f);
+    w = (e & 1) ? ((w & 0x0000ffffu) | (b << 16)) : ((w & 0xffff0000u) | b);
+  }
+};
+
+template <>
+struct Mma<float> {
+  static constexpr int EPL = 4;
+  static constexpr int KS = 16;
+  // four K=4 MFMAs; MFMA e consumes element e of every lane, i.e. the k set
+  // {k0 + 4q + e : q = 0..3}; A and B use the same assignment so the sum over
+  // k is complete.
+  __device__ static void mma(const uint4& a, const uint4& b, f32x4& c) {
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
+  }
+  __device__ static float get(const uint4& v, int e) { return __uint_as_float((&v.x)[e]); }
+  __device__ static void set(uint4& v, int e, float f) { (&v.x)[e] = __float_as_uint(f); }
+};
+
+// 16-byte fragment of row `row` starting at element k0 (zero beyond K).
+template <typename T, bool ALIGNED>
+__device__ inline uint4 load_frag(const T* __restrict__ row, int k0, int K) {
+  using M = Mma<T>;
+  uint4 v = make_uint4(0u, 0u, 0u, 0u);
+  if (ALIGNED) {
+    if (k0 < K) v = *reinterpret_cast<const uint4*>(row + k0);
+  } else {
+#pragma unroll
+    for (int e = 0; e < M::EPL; ++e)
+      if (k0 + e < K) M::set(v, e, Elem<T>::load(row + k0 + e));
+  }
+  return v;
+}
+
+// x' = x @ (R * scale)^T for the 64 tokens of the tile, this wave's share of K.
+//   xrow0: pointer to token s0 of the sequence; rows s >= s_limit read as zero.
+//   acc[mt][pb][i] belongs to token mt*16 + (lane/16)*4 + i, column pb*16 + lane%16.
+template <typename T, int PB, bool ALIGNED>
+__device__ inline void project_tile(const T* __restrict__ xrow0, int64_t tok_stride, int rows_valid,
+                                    int K, const T* __restrict__ R, int p,
+                                    const float* __restrict__ scale, int wave, int lane,
+                                    f32x4 (&acc)[MT][PB]) {
+  using M = Mma<T>;
+  constexpr int U = 2;  // k-steps kept in flight per wave
+  const int r = lane & 15;
+  const int q = lane >> 4;
+
+  const T* xrow[MT];
+  bool xok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int t = mt * 16 + r;
+    xok[mt] = t < rows_valid;
+    xrow[mt] = xrow0 + (int64_t)t * tok_stride;
+  }
+  const T* rrow[PB];
+  bool rok[PB];
+#pragma unroll
+  for (int pb = 0; pb < PB; ++pb) {
+    const int j = pb * 16 + r;
+    rok[pb] = j < p;
+    rrow[pb] = R + (int64_t)j * K;
+  }
+
+  const int nsteps = (K + M::KS - 1) / M::KS;
+  for (int ks0 = wave; ks0 < nsteps; ks0 += 4 * U) {
+    uint4 xf[U][MT];
+    uint4 rf[U][PB];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k0 = (ks0 + 4 * u) * M::KS + q * M::EPL;  // >= K when the step is past the end
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        xf[u][mt] = make_uint4(0u, 0u, 0u, 0u);
+        if (mt * 16 < rows_valid && xok[mt]) xf[u][mt] = load_frag<T, ALIGNED>(xrow[mt], k0, K);
+      }
+#pragma unroll
+      for (int pb = 0; pb < PB; ++pb) {
+        rf[u][pb] = make_uint4(0u, 0u, 0u, 0u);
+        if (rok[pb]) rf[u][pb] = load_frag<T, ALIGNED>(rrow[pb], k0, K);
+      }
+    }
+    if (scale != nullptr) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int k0 = (ks0 + 4 * u) * M::KS + q * M::EPL;
+#pragma unroll
+        for (int e = 0; e < M::EPL; ++e) {
+          const float sc = (k0 + e < K) ? scale[k0 + e] : 0.f;
+#pragma unroll
+          for (int pb = 0; pb < PB; ++pb) M::set(rf[u][pb], e, M::get(rf[u][pb], e) * sc);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        if (mt * 16 < rows_valid) {
+#pragma unroll
+          for (int pb = 0; pb < PB; ++pb) M::mma(xf[u][mt], rf[u][pb], acc[mt][pb]);
+        }
+      }
+  }
+}
+
+struct CollectArgs {
+  const bgx_module_desc* mods;  // device copy
+  const int32_t* lengths;
+  int N, S, p, tiles_per_seq;
+  // per-sequence
+  float* partials;  // [n_modules][N][tiles_per_seq][p*p]
+  // per-token
+  const int64_t* row_offsets;
+  void* out;
+  int64_t out_row_stride;
+  int out_dtype;
+  float lo, hi;
+};
+
+__device__ inline int seq_token_limit(const int32_t* lengths, int n, int S) {
+  if (lengths == nullptr) return S;
+  const int l = lengths[n] - 1;
+  return l < S ? (l < 0 ? 0 : l) : S;
+}
+
+template <typename T, int PB, bool ALIGNED, bool PER_TOKEN>
+__global__ __launch_bounds__(COLLECT_THREADS) void collect_kernel(CollectArgs args) {
+  constexpr int PP = PB * 16;   // padded projection dim
+  constexpr int LDP = PP + 1;   // LDS row stride (floats)
+  __shared__ float sm[2][2][TILE_T][LDP];  // [a/g][slot][token][col]
+
+  const int tile = blockIdx.x;
+  const int m = blockIdx.y;
+  const int n = tile / args.tiles_per_seq;
+  const int ts = tile - n * args.tiles_per_seq;
+  const int s0 = ts * TILE_T;
+  const int s_limit = seq_token_limit(args.lengths, n, args.S);
+  if (s0 >= s_limit) return;  // whole tile is padding: g is exactly zero there
+  const int rows_valid = min(TILE_T, s_limit - s0);
+
+  const bgx_module_desc d = args.mods[m];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int p = args.p;
+
+  f32x4 accA[MT][PB];
+  f32x4 accG[MT][PB];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int pb = 0; pb < PB; ++pb) {
+      accA[mt][pb] = f32x4{0.f, 0.f, 0.f, 0.f};
+      accG[mt][pb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+  const T* a0 = (const T*)d.a + (int64_t)n * d.a_seq_stride + (int64_t)s0 * d.a_tok_stride;
+  const T* g0 = (const T*)d.g + (int64_t)n * d.g_seq_stride + (int64_t)s0 * d.g_tok_stride;
+  project_tile<T, PB, ALIGNED>(a0, d.a_tok_stride, rows_valid, d.I, (const T*)d.r_in, p,
+                               d.col_scale, wave, lane, accA);
+  project_tile<T, PB, ALIGNED>(g0, d.g_tok_stride, rows_valid, d.O, (const T*)d.r_out, p,
+                               d.row_scale, wave, lane, accG);
+
+  // ---- combine the 4 K-slices: (w0 + w2) + (w1 + w3), fixed order ----------
+  const int r = lane & 15;
+  const int q = lane >> 4;
+  if (wave >= 2) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int pb = 0; pb < PB; ++pb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int t = mt * 16 + q * 4 + i;
+          sm[0][wave - 2][t][pb * 16 + r] = accA[mt][pb][i];
+          sm[1][wave - 2][t][pb * 16 + r] = accG[mt][pb][i];
+        }
+  }
+  __syncthreads();
+  if (wave < 2) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int pb = 0; pb < PB; ++pb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int t = mt * 16 + q * 4 + i;
+          sm[0][wave][t][pb * 16 + r] += accA[mt][pb][i];
+          sm[1][wave][t][pb * 16 + r] += accG[mt][pb][i];
+        }
+  }
+  __syncthreads();
+  for (int e = tid; e < TILE_T * PP; e += COLLECT_THREADS) {
+    const int t = e / PP, c = e - t * PP;
+    sm[0][0][t][c] += sm[0][1][t][c];
+    sm[1][0][t][c] += sm[1][1][t][c];
+  }
+  __syncthreads();
+
+  const int pp = p * p;
+  if (!PER_TOKEN) {
+    // P[i, j] = sum_t g'[t, i] * a'[t, j]; tokens past rows_valid hold zeros.
+    float* dst = args.partials + (((int64_t)m * args.N + n) * args.tiles_per_seq + ts) * pp;
+    for (int e = tid; e < pp; e += COLLECT_THREADS) {
+      const int i = e / p, j = e - i * p;
+      float s = 0.f;
+#pragma unroll 8
+      for (int t = 0; t < TILE_T; ++t) s = fmaf(sm[1][0][t][i], sm[0][0][t][j], s);
+      dst[e] = s;
+    }
+  } else {
+    const int64_t row0 = args.row_offsets[n] + s0;
+    for (int t = wave; t < rows_valid; t += COLLECT_THREADS / WAVE) {
+      const int64_t base = (row0 + t) * args.out_row_stride + d.out_col;
+      for (int e = lane; e < pp; e += WAVE) {
+        const int i = e / p, j = e - i * p;
+        const float v = clampf(sm[1][0][t][i] * sm[0][0][t][j], args.lo, args.hi);
+        store_as(args.out, base + e, v, args.out_dtype);
+      }
+    }
+  }
+}
+
+// Adds the per-tile partials of each (module, sequence) in tile order, clamps,
+// casts and writes the module's block of the output row.
+__global__ __launch_bounds__(256) void collect_finalize_kernel(
+    const bgx_module_desc* __restrict__ mods, const float* __restrict__ partials,
+    const int32_t* __restrict__ lengths, const int64_t* __restrict__ out_rows, int N, int S, int p,
+    int tiles_per_seq, void* out, int64_t out_row_stride, int out_dtype, float lo, float hi) {
+  const int n = blockIdx.x;
+  const int m = blockIdx.y;
+  const int pp = p * p;
+  const int s_limit = seq_token_limit(lengths, n, S);
+  const int ntiles = (s_limit + TILE_T - 1) / TILE_T;
+  const float* src = partials + ((int64_t)m * N + n) * tiles_per_seq * pp;
+  const int64_t row = out_rows ? out_rows[n] : (int64_t)n;
+  const int64_t base = row * out_row_stride + mods[m].out_col;
+  for (int e = threadIdx.x; e < pp; e += blockDim.x) {
+    float s = 0.f;
+    for (int t = 0; t < ntiles; ++t) s += src[(int64_t)t * pp + e];
+    store_as(out, base + e, clampf(s, lo, hi), out_dtype);
+  }
+}
+
+// ---- Adafactor factors ---------------------------------------------------------
+__global__ __launch_bounds__(256) void adafactor_scales_kernel(const float* __restrict__ row, int O,
+                                                               const float* __restrict__ col, int I,
+                                                               int dtype, float* row_scale,
+                                                               float* col_scale) {
+  __shared__ double red[256];
+  const int tid = threadIdx.x;
+  if (col != nullptr) {
+    for (int i = tid; i < I; i += 256)
+      col_scale[i] = round_to_dtype(1.0f / sqrtf(col[i] + 1e-30f), dtype);
+  }
+  if (row != nullptr) {
+    // mean(row + eps) accumulated in double so the result does not depend on
+    // the reduction tree beyond fp32 rounding of the final mean.
+    double s = 0.0;
+    for (int o = tid; o < O; o += 256) s += (double)(row[o] + 1e-30f);
+    red[tid] = s;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+      if (tid < w) red[tid] += red[tid + w];
+      __syncthreads();
+    }
+    const float mean = (float)(red[0] / (double)O);
+    const float sq = sqrtf(mean);
+    for (int o = tid; o < O; o += 256)
+      row_scale[o] = round_to_dtype(sq * (1.0f / sqrtf(row[o] + 1e-30f)), dtype);
+  }
+}
+
+// ---- in-place row unit normalisation ----------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void unit_normalize_kernel(T* rows, int64_t n_rows, int64_t D,
+                                                             int64_t stride, float eps_sq) {
+  __shared__ float red[256];
+  const int64_t rowi = blockIdx.x;
+  T* x = rows + rowi * stride;
+  float s = 0.f;
+  for (int64_t d = threadIdx.x; d < D; d += 256) {
+    const float v = Elem<T>::load(x + d);
+    s = fmaf(v, v, s);
+  }
+  red[threadIdx.x] = s;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if (threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+    __syncthreads();
+  }
+  // the reference forms rsqrt in the gradient dtype and multiplies there
+  const float inv = Elem<T>::round(1.0f / sqrtf(fmaxf(Elem<T>::round(red[0]), eps_sq)));
+  for (int64_t d = threadIdx.x; d < D; d += 256) {
+    const float v = Elem<T>::load(x + d) * inv;
+    if constexpr (sizeof(T) == 4)
+      *(float*)(x + d) = v;
+    else if constexpr (Elem<T>::code == BGX_F16)
+      ((uint16_t*)x)[d] = (uint16_t)f32_to_f16_bits(v);
+    else
+      ((uint16_t*)x)[d] = (uint16_t)f32_to_bf16_bits(v);
+  }
+}
+
+// ---- host side ------------------------------------------------------------------------
+static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+static size_t desc_bytes(int n_modules) {
+  return align_up((size_t)n_modules * sizeof(bgx_module_desc), 256);
+}
+
+size_t collect_workspace_bytes(int n_modules, int N, int S, int p) {
+  if (n_modules <= 0 || N <= 0 || S <= 0 || p <= 0) return 0;
+  const size_t tiles = (size_t)((S + TILE_T - 1) / TILE_T);
+  return desc_bytes(n_modules) + (size_t)n_modules * N * tiles * p * p * sizeof(float);
+}
+
+template <typename T, int PB, bool ALIGNED>
+static void launch_collect(bool per_token, dim3 grid, hipStream_t st, const CollectArgs& args) {
+  if (per_token)
+    hipLaunchKernelGGL((collect_kernel<T, PB, ALIGNED, true>), grid, dim3(COLLECT_THREADS), 0, st, args);
+  else
+    hipLaunchKernelGGL((collect_kernel<T, PB, ALIGNED, false>), grid, dim3(COLLECT_THREADS), 0, st, args);
+}
+
+template <typename T>
+static void launch_collect_pb(int pb, bool aligned, bool per_token, dim3 grid, hipStream_t st,
+                              const CollectArgs& args) {
+  if (pb == 1) {
+    aligned ? launch_collect<T, 1, true>(per_token, grid, st, args)
+            : launch_collect<T, 1, false>(per_token, grid, st, args);
+  } else if (pb == 2) {
+    aligned ? launch_collect<T, 2, true>(per_token, grid, st, args)
+            : launch_collect<T, 2, false>(per_token, grid, st, args);
+  } else {
+    aligned ? launch_collect<T, 4, true>(per_token, grid, st, args)
+            : launch_collect<T, 4, false>(per_token, grid, st, args);
+  }
+}
+
+int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules, int N, int S,
+                 int p, int in_dtype, const int32_t* lengths, const int64_t* rows_or_offsets,
+                 void* out, int64_t out_row_stride, int out_dtype, float lo, float hi, void* ws,
+                 size_t ws_bytes, void* stream) {
+  BGX_REQUIRE(mods_host && out && ws, BGX_E_ARG, "collect: null mods/out/workspace");
+  BGX_REQUIRE(n_modules > 0 && N > 0 && S > 0, BGX_E_ARG, "collect: n_modules=%d N=%d S=%d", n_modules, N, S);
+  BGX_REQUIRE(n_modules <= 65535, BGX_E_SHAPE, "collect: n_modules=%d exceeds 65535", n_modules);
+  BGX_REQUIRE(p >= 1 && p <= 64, BGX_E_SHAPE, "collect: projection dim p=%d outside 1..64", p);
+  BGX_REQUIRE(in_dtype >= BGX_F32 && in_dtype <= BGX_BF16, BGX_E_DTYPE, "collect: in_dtype=%d", in_dtype);
+  BGX_REQUIRE(out_dtype >= BGX_F32 && out_dtype <= BGX_BF16, BGX_E_DTYPE, "collect: out_dtype=%d", out_dtype);
+  BGX_REQUIRE(out_row_stride > 0, BGX_E_ARG, "collect: out_row_stride=%lld", (long long)out_row_stride);
+  if (per_token)
+    BGX_REQUIRE(lengths && rows_or_offsets, BGX_E_ARG, "collect_tok: lengths and row_offsets are required");
+  const size_t need = collect_workspace_bytes(n_modules, N, S, p);
+  BGX_REQUIRE(ws_bytes >= need, BGX_E_WORKSPACE, "collect: workspace %zu < %zu bytes", ws_bytes, need);
+  BGX_REQUIRE(((uintptr_t)ws & 255) == 0, BGX_E_ALIGN, "collect: workspace must be 256-byte aligned");
+
+  const int epl = in_dtype == BGX_F32 ? 4 : 8;
+  bool aligned = true;
+  for (int m = 0; m < n_modules; ++m) {
+    const bgx_module_desc& d = mods_host[m];
+    BGX_REQUIRE(d.a && d.g && d.r_in && d.r_out, BGX_E_ARG, "collect: module %d has a null a/g/r_in/r_out", m);
+    BGX_REQUIRE(d.I > 0 && d.O > 0, BGX_E_ARG, "collect: module %d I=%d O=%d", m, d.I, d.O);
+    BGX_REQUIRE(d.out_col >= 0 && d.out_col + (int64_t)p * p <= out_row_stride, BGX_E_ARG,
+                "collect: module %d columns [%lld, +%d) do not fit a row of %lld", m, (long long)d.out_col,
+                p * p, (long long)out_row_stride);
+    BGX_REQUIRE(d.bias_col == nullptr && d.bias_scale == nullptr, BGX_E_SHAPE,
+                "collect: bias column is not supported by this build");
+    const bool ok = ((uintptr_t)d.a % 16 == 0) && ((uintptr_t)d.g % 16 == 0) &&
+                    ((uintptr_t)d.r_in % 16 == 0) && ((uintptr_t)d.r_out % 16 == 0) &&
+                    (d.I % epl == 0) && (d.O % epl == 0) && (d.a_seq_stride % epl == 0) &&
+                    (d.a_tok_stride % epl == 0) && (d.g_seq_stride % epl == 0) &&
+                    (d.g_tok_stride % epl == 0);
+    aligned = aligned && ok;
+  }
+
+  hipStream_t st = (hipStream_t)stream;
+  bgx_module_desc* mods_dev = (bgx_module_desc*)ws;
+  BGX_HIP(hipMemcpyAsync(mods_dev, mods_host, (size_t)n_modules * sizeof(bgx_module_desc),
+                         hipMemcpyHostToDevice, st));
+
+  CollectArgs args;
+  args.mods = mods_dev;
+  args.lengths = lengths;
+  args.N = N;
+  args.S = S;
+  args.p = p;
+  args.tiles_per_seq = (S + TILE_T - 1) / TILE_T;
+  args.partials = (float*)((char*)ws + desc_bytes(n_modules));
+  args.row_offsets = per_token ? rows_or_offsets : nullptr;
+  args.out = out;
+  args.out_row_stride = out_row_stride;
+  args.out_dtype = out_dtype;
+  args.lo = lo;
+  args.hi = hi;
+
+  const int64_t tiles = (int64_t)N * args.tiles_per_seq;
+  BGX_REQUIRE(tiles <= 0x7fffffffLL, BGX_E_SHAPE, "collect: %lld tiles exceed the grid limit", (long long)tiles);
+  const dim3 grid((unsigned)tiles, (unsigned)n_modules);
+  const int pb = (p + 15) / 16;
+  if (in_dtype == BGX_F32)
+    launch_collect_pb<float>(pb, aligned, per_token, grid, st, args);
+  else if (in_dtype == BGX_F16)
+    launch_collect_pb<f16_t>(pb, aligned, per_token, grid, st, args);
+  else
+    launch_collect_pb<bf16_t>(pb, aligned, per_token, grid, st, args);
+  BGX_HIP(hipGetLastError());
+
+  if (!per_token) {
+    hipLaunchKernelGGL(collect_finalize_kernel, dim3((unsigned)N, (unsigned)n_modules), dim3(256), 0, st,
+                       mods_dev, args.partials, lengths, rows_or_offsets, N, S, p, args.tiles_per_seq, out,
+                       out_row_stride, out_dtype, lo, hi);
+    BGX_HIP(hipGetLastError());
+  }
+  return 0;
+}
+
+int adafactor_scales_impl(const float* row, int O, const float* col, int I, int dtype, float* row_scale,
+                          float* col_scale, void* stream) {
+  BGX_REQUIRE(dtype >= BGX_F32 && dtype <= BGX_BF16, BGX_E_DTYPE, "adafactor_scales: dtype=%d", dtype);
+  BGX_REQUIRE((row == nullptr) == (row_scale == nullptr), BGX_E_ARG, "adafactor_scales: row / row_scale mismatch");
+  BGX_REQUIRE((col == nullptr) == (col_scale == nullptr), BGX_E_ARG, "adafactor_scales: col / col_scale mismatch");
+  BGX_REQUIRE(row == nullptr || O > 0, BGX_E_ARG, "adafactor_scales: O=%d", O);
+  BGX_REQUIRE(col == nullptr || I > 0, BGX_E_ARG, "adafactor_scales: I=%d", I);
+  if (row == nullptr && col == nullptr) return 0;
+  hipLaunchKernelGGL(adafactor_scales_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, row, O, col, I,
+                     dtype, row_scale, col_scale);
+  BGX_HIP(hipGetLastError());
+  return 0;
+}
+
+int unit_normalize_impl(void* rows, int64_t n_rows, int64_t D, int64_t stride, int dtype, void* stream) {
+  BGX_REQUIRE(rows != nullptr, BGX_E_ARG, "unit_normalize_rows: null rows");
+  BGX_REQUIRE(n_rows >= 0 && D > 0 && stride >= D, BGX_E_ARG, "unit_normalize_rows: n_rows=%lld D=%lld stride=%lld",
+              (long long)n_rows, (long long)D, (long long)stride);
+  BGX_REQUIRE(n_rows <= 0x7fffffffLL, BGX_E_SHAPE, "unit_normalize_rows: too many rows");
+  if (n_rows == 0) return 0;
+  // eps of fp32, squared (bergson/builder.py:14)
+  const float eps_sq = 1.1920928955078125e-07f * 1.1920928955078125e-07f;
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid((unsigned)n_rows), block(256);
+  if (dtype == BGX_F32)
+    hipLaunchKernelGGL(unit_normalize_kernel<float>, grid, block, 0, st, (float*)rows, n_rows, D, stride, eps_sq);
+  else if (dtype == BGX_F16)
+    hipLaunchKernelGGL(unit_normalize_kernel<f16_t>, grid, block, 0, st, (f16_t*)rows, n_rows, D, stride, eps_sq);
+  else if (dtype == BGX_BF16)
+    hipLaunchKernelGGL(unit_normalize_kernel<bf16_t>, grid, block, 0, st, (bf16_t*)rows, n_rows, D, stride, eps_sq);
+  else
+    BGX_REQUIRE(false, BGX_E_DTYPE, "unit_normalize_rows: dtype=%d", dtype);
+  BGX_HIP(hipGetLastError());
+  return 0;
+}
+
+}  // namespace bgx

@@ -1,0 +1,129 @@
+// Shared device/host helpers of the gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "bergson_amd.h"
+
+namespace bgx {
+
+// ---- host-side error plumbing (defined in capi.hip) -----------------------
+void set_error(const char* fmt, ...);
+int hip_fail(hipError_t e, const char* what);
+
+#define BGX_HIP(call)                                  \
+  do {                                                 \
+    hipError_t e__ = (call);                           \
+    if (e__ != hipSuccess) return hip_fail(e__, #call); \
+  } while (0)
+
+#define BGX_REQUIRE(cond, code, ...) \
+  do {                               \
+    if (!(cond)) {                   \
+      set_error(__VA_ARGS__);        \
+      return (code);                 \
+    }                                \
+  } while (0)
+
+// ---- vector types for the MFMA builtins -----------------------------------
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+
+// Element tags: the kernels are templated on these; the 16-bit types are
+// carried as raw bits and only converted through the helpers below.
+struct bf16_t {
+  uint16_t bits;
+};
+struct f16_t {
+  uint16_t bits;
+};
+
+constexpr int WAVE = 64;
+
+__host__ __device__ inline size_t dtype_size(int dt) {
+  return dt == BGX_F32 ? 4 : 2;
+}
+
+// ---- scalar conversions ----------------------------------------------------
+__device__ inline float bf16_bits_to_f32(uint32_t b) {
+  return __uint_as_float(b << 16);
+}
+// round-to-nearest-even, NaN kept quiet
+__device__ inline uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+__device__ inline float f16_bits_to_f32(uint32_t b) {
+  union {
+    uint16_t u;
+    _Float16 h;
+  } c;
+  c.u = (uint16_t)b;
+  return (float)c.h;
+}
+__device__ inline uint32_t f32_to_f16_bits(float f) {
+  union {
+    uint16_t u;
+    _Float16 h;
+  } c;
+  c.h = (_Float16)f;
+  return c.u;
+}
+
+template <typename T>
+struct Elem;
+template <>
+struct Elem<float> {
+  static constexpr int code = BGX_F32;
+  __device__ static float load(const float* p) { return *p; }
+  __device__ static float round(float x) { return x; }
+};
+template <>
+struct Elem<bf16_t> {
+  static constexpr int code = BGX_BF16;
+  __device__ static float load(const bf16_t* p) { return bf16_bits_to_f32(p->bits); }
+  __device__ static float round(float x) { return bf16_bits_to_f32(f32_to_bf16_bits(x)); }
+};
+template <>
+struct Elem<f16_t> {
+  static constexpr int code = BGX_F16;
+  __device__ static float load(const f16_t* p) { return f16_bits_to_f32(p->bits); }
+  __device__ static float round(float x) { return f16_bits_to_f32(f32_to_f16_bits(x)); }
+};
+
+// value rounded to the representable set of dtype `dt`
+__device__ inline float round_to_dtype(float x, int dt) {
+  if (dt == BGX_BF16) return Elem<bf16_t>::round(x);
+  if (dt == BGX_F16) return Elem<f16_t>::round(x);
+  return x;
+}
+
+// store one value as dtype `dt` at element index idx of base
+__device__ inline void store_as(void* base, int64_t idx, float v, int dt) {
+  if (dt == BGX_F32) {
+    ((float*)base)[idx] = v;
+  } else if (dt == BGX_F16) {
+    ((uint16_t*)base)[idx] = (uint16_t)f32_to_f16_bits(v);
+  } else {
+    ((uint16_t*)base)[idx] = (uint16_t)f32_to_bf16_bits(v);
+  }
+}
+
+__device__ inline float load_as(const void* base, int64_t idx, int dt) {
+  if (dt == BGX_F32) return ((const float*)base)[idx];
+  if (dt == BGX_F16) return f16_bits_to_f32(((const uint16_t*)base)[idx]);
+  return bf16_bits_to_f32(((const uint16_t*)base)[idx]);
+}
+
+__device__ inline float clampf(float v, float lo, float hi) {
+  // NaN propagates like torch.clamp
+  return v < lo ? lo : (v > hi ? hi : v);
+}
+
+}  // namespace bgx

@@ -1,0 +1,645 @@
+// Gradient-store scan for gfx950 (MI355X): scores every store row against Q
+// queries, streaming the store once from HBM.
+//
+//   scan_gemm_kernel   LDS-tiled MFMA GEMM  scores[n, q] = <store[n], queries[q]>,
+//                      with the row sum of squares accumulated from the same
+//                      tiles, and a fused epilogue: unit-norm scaling, optional
+//                      dense score write, per-row max over queries, and a
+//                      per-query threshold filter that appends the few scores
+//                      that can still enter the top-k to a candidate list.
+//   scan_select_kernel per query: exact top-k of (running top-k U candidates) by
+//                      radix select on unique 64-bit keys, sorted; raises the
+//                      query's threshold for the next pass.
+//   scan_finish_kernel decodes keys into (value, row) and the row maxima.
+//
+// The store is processed in passes of at most `chunk_rows` rows so that the
+// candidate lists are bounded (a pass can never append more than chunk_rows
+// entries per query) and the thresholds tighten quickly.
+//
+// Reference op sequence: bergson/score/scorer.py:89-115 (per-module GEMMs,
+// sum of squares, division, max over queries) and
+// bergson/query/attributor.py:137-167, :229-235 (row normalisation, GEMM,
+// torch.topk).
+
+#include "common.hpp"
+
+namespace bgx {
+
+// ---- element traits for the 32x32 MFMA tiles ------------------------------------
+// One "substep" consumes a 16-byte fragment per lane for A and for B:
+// lane (r = lane%32, h = lane/32) holds EPL consecutive k starting at h*EPL.
+template <typename T>
+struct Mma32;
+
+template <>
+struct Mma32<f16_t> {
+  static constexpr int EPL = 8;
+  __device__ static void mma(const uint4& a, const uint4& b, f32x16& c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c,
+                                               0, 0, 0);
+  }
+  __device__ static float sumsq(const uint4& v, float s) {
+    typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+    s = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, v.x), __builtin_bit_cast(h2, v.x), s, false);
+    s = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, v.y), __builtin_bit_cast(h2, v.y), s, false);
+    s = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, v.z), __builtin_bit_cast(h2, v.z), s, false);
+    s = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, v.w), __builtin_bit_cast(h2, v.w), s, false);
+    return s;
+  }
+};
+
+template <>
+struct Mma32<bf16_t> {
+  static constexpr int EPL = 8;
+  __device__ static void mma(const uint4& a, const uint4& b, f32x16& c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
+                                                c, 0, 0, 0);
+  }
+  __device__ static float sumsq(const uint4& v, float s) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float lo = __uint_as_float(w[i] << 16);
+      const float hi = __uint_as_float(w[i] & 0xffff0000u);
+      s = fmaf(lo, lo, s);
+      s = fmaf(hi, hi, s);
+    }
+    return s;
+  }
+};
+
+template <>
+struct Mma32<float> {
+  static constexpr int EPL = 4;
+  // four K=2 MFMAs; MFMA e consumes element e of both halves of the wave.
+  __device__ static void mma(const uint4& a, const uint4& b, f32x16& c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
+  }
+  __device__ static float sumsq(const uint4& v, float s) {
+    const float x = __uint_as_float(v.x), y = __uint_as_float(v.y), z = __uint_as_float(v.z),
+                w = __uint_as_float(v.w);
+    s = fmaf(x, x, s);
+    s = fmaf(y, y, s);
+    s = fmaf(z, z, s);
+    s = fmaf(w, w, s);
+    return s;
+  }
+};
+
+// ---- order-preserving float <-> uint32 ------------------------------------------------
+__host__ __device__ inline uint32_t f32_ordered(float f) {
+  union {
+    float f;
+    uint32_t u;
+  } c;
+  c.f = f;
+  return (c.u & 0x80000000u) ? ~c.u : (c.u | 0x80000000u);
+}
+__host__ __device__ inline float ordered_f32(uint32_t o) {
+  union {
+    float f;
+    uint32_t u;
+  } c;
+  c.u = (o & 0x80000000u) ? (o & 0x7fffffffu) : ~o;
+  return c.f;
+}
+// Unique key: larger score first, then lower row number.
+__device__ inline uint64_t make_key(float score, uint32_t row) {
+  return ((uint64_t)f32_ordered(score) << 32) | (uint64_t)(0xffffffffu - row);
+}
+
+constexpr int SCAN_KMAX = 2048;
+constexpr int TILE_ROW_BYTES = 128;  // bytes of K per LDS row (BK elements)
+constexpr int TILE_CHUNKS = TILE_ROW_BYTES / 16;
+constexpr int LDS_ROW_BYTES = TILE_ROW_BYTES + 16;  // padded against bank conflicts
+
+struct ScanArgs {
+  const void* store;
+  const void* queries;
+  int64_t row0;          // first store row of this pass
+  int64_t rows;          // rows in this pass
+  int64_t D;
+  int64_t store_stride;  // elements
+  int Q;
+  int row_tiles;         // ceil(rows / BM)
+  int q_tiles;           // ceil(Q / BN)
+  float query_scale;
+  int unit_norm;
+  // outputs / state (may be null)
+  float* scores;         // [n_rows, Q]
+  float* sumsq;          // [n_rows]
+  uint32_t* row_max_enc; // [n_rows] ordered-uint encoding
+  const float* thr;      // [Q] current k-th best per query
+  uint32_t* cand_count;  // [Q]
+  uint64_t* cand;        // [Q][cand_cap]
+  int64_t cand_cap;
+};
+
+template <typename T, bool ALIGNED>
+__device__ inline uint4 load_chunk(const T* __restrict__ base, int64_t row, int64_t n_rows, int64_t stride,
+                                   int64_t k, int64_t K) {
+  constexpr int EPL = Mma32<T>::EPL;
+  uint4 v = make_uint4(0u, 0u, 0u, 0u);
+  if (row >= n_rows || k >= K) return v;
+  const T* p = base + row * stride + k;
+  if (ALIGNED) {
+    v = *reinterpret_cast<const uint4*>(p);
+  } else {
+    if constexpr (sizeof(T) == 4) {
+      uint32_t* w = &v.x;
+      for (int e = 0; e < EPL; ++e)
+        if (k + e < K) w[e] = *reinterpret_cast<const uint32_t*>(p + e);
+    } else {
+      uint32_t* w = &v.x;
+      for (int e = 0; e < EPL; ++e)
+        if (k + e < K) {
+          const uint32_t b = *reinterpret_cast<const uint16_t*>(p + e);
+          w[e >> 1] |= (e & 1) ? (b << 16) : b;
+        }
+    }
+  }
+  return v;
+}
+
+// Workgroup tile BM x BN, WM x WN waves, each wave (BM/WM) x (BN/WN) as 32x32 MFMA blocks.
+template <typename T, int BM, int BN, int WM, int WN, bool ALIGNED>
+__global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
+  using M = Mma32<T>;
+  constexpr int NT = WM * WN * 64;
+  constexpr int EPL = M::EPL;
+  constexpr int BK = TILE_CHUNKS * EPL;  // elements of K per tile
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int GCH = BM * TILE_CHUNKS / NT;  // store chunks per thread
+  constexpr int QCH = BN * TILE_CHUNKS / NT;  // query chunks per thread
+  static_assert(BM * TILE_CHUNKS % NT == 0 && BN * TILE_CHUNKS % NT == 0, "loader mapping");
+  static_assert(NT % TILE_CHUNKS == 0, "loader mapping");
+  constexpr int ROWS_PER_PASS = NT / TILE_CHUNKS;
+
+  extern __shared__ __align__(16) unsigned char smem[];
+  // [buf][BM + BN rows][LDS_ROW_BYTES]
+  constexpr int BUF_BYTES = (BM + BN) * LDS_ROW_BYTES;
+  __shared__ float s_inv[BM];
+
+  // XCD-aware tile order: workgroup b runs on XCD b % 8; the q_tiles
+  // workgroups of one row tile share that XCD's L2.
+  const int b = blockIdx.x;
+  const int xcd = b & 7;
+  const int slot = b >> 3;
+  const int rt_local = slot / args.q_tiles;
+  const int qt = slot - rt_local * args.q_tiles;
+  const int rt = rt_local * 8 + xcd;
+  if (rt >= args.row_tiles) return;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+
+  const T* store = (const T*)args.store + args.row0 * args.store_stride;
+  const T* queries = (const T*)args.queries;
+  const int64_t g_row0 = (int64_t)rt * BM;  // pass-local first row
+  const int64_t q_row0 = (int64_t)qt * BN;
+  const int64_t D = args.D;
+
+  const int lrow = tid / TILE_CHUNKS;
+  const int lcol = tid % TILE_CHUNKS;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  float ss[GCH];
+#pragma unroll
+  for (int i = 0; i < GCH; ++i) ss[i] = 0.f;
+
+  uint4 gr[GCH], qr[QCH];
+  auto gload = [&](int kt) {
+    const int64_t k = (int64_t)kt * BK + lcol * EPL;
+#pragma unroll
+    for (int i = 0; i < GCH; ++i)
+      gr[i] = load_chunk<T, ALIGNED>(store, g_row0 + lrow + i * ROWS_PER_PASS, args.rows, args.store_stride, k, D);
+#pragma unroll
+    for (int i = 0; i < QCH; ++i)
+      qr[i] = load_chunk<T, ALIGNED>(queries, q_row0 + lrow + i * ROWS_PER_PASS, args.Q, D, k, D);
+  };
+  auto lstore = [&](int buf) {
+    unsigned char* base = smem + buf * BUF_BYTES;
+#pragma unroll
+    for (int i = 0; i < GCH; ++i) {
+      *reinterpret_cast<uint4*>(base + (lrow + i * ROWS_PER_PASS) * LDS_ROW_BYTES + lcol * 16) = gr[i];
+      ss[i] = M::sumsq(gr[i], ss[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < QCH; ++i)
+      *reinterpret_cast<uint4*>(base + (BM + lrow + i * ROWS_PER_PASS) * LDS_ROW_BYTES + lcol * 16) = qr[i];
+  };
+
+  const int KT = (int)((D + BK - 1) / BK);
+  gload(0);
+  lstore(0);
+  __syncthreads();
+
+  const int fr = lane & 31;
+  const int fh = lane >> 5;
+  for (int kt = 0; kt < KT; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < KT) gload(kt + 1);
+    const unsigned char* gb = smem + buf * BUF_BYTES + (wm * WTM + fr) * LDS_ROW_BYTES + fh * 16;
+    const unsigned char* qb = smem + buf * BUF_BYTES + (BM + wn * WTN + fr) * LDS_ROW_BYTES + fh * 16;
+#pragma unroll
+    for (int kk = 0; kk < TILE_CHUNKS / 2; ++kk) {
+      uint4 af[TM], bf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        af[i] = *reinterpret_cast<const uint4*>(gb + i * 32 * LDS_ROW_BYTES + kk * 32);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        bf[j] = *reinterpret_cast<const uint4*>(qb + j * 32 * LDS_ROW_BYTES + kk * 32);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) M::mma(af[i], bf[j], acc[i][j]);
+    }
+    if (kt + 1 < KT) lstore(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- row sum of squares -> per-row multiplier ------------------------------------
+#pragma unroll
+  for (int i = 0; i < GCH; ++i) {
+    float s = ss[i];
+    s += __shfl_xor(s, 1);
+    s += __shfl_xor(s, 2);
+    s += __shfl_xor(s, 4);
+    if (lcol == 0) {
+      const int row = lrow + i * ROWS_PER_PASS;
+      float w = args.query_scale;
+      if (args.unit_norm) w = s > 0.f ? args.query_scale / sqrtf(s) : 0.f;
+      s_inv[row] = w;
+      const int64_t grow = g_row0 + row;
+      if (qt == 0 && args.sumsq != nullptr && grow < args.rows) args.sumsq[args.row0 + grow] = s;
+    }
+  }
+  __syncthreads();
+
+  // ---- epilogue -----------------------------------------------------------------------
+  float thr[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int64_t q = q_row0 + wn * WTN + j * 32 + fr;
+    thr[j] = (args.thr != nullptr && q < args.Q) ? args.thr[q] : INFINITY;
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int row = wm * WTM + i * 32 + (e >> 2) * 8 + fh * 4 + (e & 3);
+      const int64_t prow = g_row0 + row;  // pass-local row
+      const bool row_ok = prow < args.rows;
+      const int64_t grow = args.row0 + prow;
+      const float w = s_inv[row];
+      float rmax = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int64_t q = q_row0 + wn * WTN + j * 32 + fr;
+        const float v = acc[i][j][e] * w;
+        if (row_ok && q < args.Q) {
+          rmax = fmaxf(rmax, v);
+          if (args.scores != nullptr) args.scores[grow * args.Q + q] = v;
+          if (v > thr[j]) {
+            const uint32_t pos = atomicAdd(&args.cand_count[q], 1u);
+            if ((int64_t)pos < args.cand_cap) args.cand[q * args.cand_cap + pos] = make_key(v, (uint32_t)grow);
+          }
+        }
+      }
+      if (args.row_max_enc != nullptr) {
+        rmax = fmaxf(rmax, __shfl_xor(rmax, 1));
+        rmax = fmaxf(rmax, __shfl_xor(rmax, 2));
+        rmax = fmaxf(rmax, __shfl_xor(rmax, 4));
+        rmax = fmaxf(rmax, __shfl_xor(rmax, 8));
+        rmax = fmaxf(rmax, __shfl_xor(rmax, 16));
+        if (fr == 0 && row_ok) atomicMax(&args.row_max_enc[grow], f32_ordered(rmax));
+      }
+    }
+  }
+}
+
+// ---- per-query exact selection ---------------------------------------------------------------
+struct SelectArgs {
+  uint64_t* top;         // [Q][k] sorted descending
+  uint32_t* top_count;   // [Q]
+  uint64_t* cand;        // [Q][cand_cap]
+  uint32_t* cand_count;  // [Q]
+  float* thr;            // [Q]
+  int64_t cand_cap;
+  int k;
+};
+
+__global__ __launch_bounds__(256) void scan_select_kernel(SelectArgs a) {
+  __shared__ uint64_t keys[SCAN_KMAX];
+  __shared__ uint32_t hist[256];
+  __shared__ uint64_t s_prefix;
+  __shared__ uint32_t s_rank;
+  __shared__ uint32_t s_fill;
+
+  const int q = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int k = a.k;
+  uint64_t* top = a.top + (int64_t)q * k;
+  const uint64_t* cand = a.cand + (int64_t)q * a.cand_cap;
+  const uint32_t ntop = a.top_count[q];
+  uint32_t ncand = a.cand_count[q];
+  if ((int64_t)ncand > a.cand_cap) ncand = (uint32_t)a.cand_cap;
+  const uint32_t total = ntop + ncand;
+  if (ncand == 0) return;  // nothing new for this query
+
+  auto elem = [&](uint32_t i) -> uint64_t { return i < ntop ? top[i] : cand[i - ntop]; };
+
+  uint64_t kth = 0;  // keep keys >= kth
+  if (total > (uint32_t)k) {
+    // radix select of the k-th largest key, 8 bits per pass from the top
+    if (tid == 0) {
+      s_prefix = 0;
+      s_rank = (uint32_t)k;  // rank (1-based, from the largest) inside the current bucket
+    }
+    __syncthreads();
+    for (int shift = 56; shift >= 0; shift -= 8) {
+      hist[tid] = 0;
+      __syncthreads();
+      const uint64_t prefix = s_prefix;
+      const uint64_t mask = shift == 56 ? 0ull : (~0ull << (shift + 8));
+      for (uint32_t i = tid; i < total; i += 256) {
+        const uint64_t key = elem(i);
+        if ((key & mask) == prefix) atomicAdd(&hist[(uint32_t)(key >> shift) & 255u], 1u);
+      }
+      __syncthreads();
+      if (tid == 0) {
+        uint32_t rank = s_rank;
+        int d = 255;
+        for (; d > 0; --d) {
+          if (hist[d] >= rank) break;
+          rank -= hist[d];
+        }
+        s_rank = rank;
+        s_prefix = prefix | ((uint64_t)d << shift);
+      }
+      __syncthreads();
+    }
+    kth = s_prefix;
+  }
+
+  if (tid == 0) s_fill = 0;
+  __syncthreads();
+  for (uint32_t i = tid; i < total; i += 256) {
+    const uint64_t key = elem(i);
+    if (key >= kth) {
+      const uint32_t pos = atomicAdd(&s_fill, 1u);
+      if (pos < SCAN_KMAX) keys[pos] = key;
+    }
+  }
+  __syncthreads();
+  const uint32_t kept = min(s_fill, (uint32_t)k);
+  // bitonic sort, descending, padded with zeros (below every real key)
+  uint32_t n2 = 1;
+  while (n2 < kept) n2 <<= 1;
+  for (uint32_t i = kept + tid; i < n2; i += 256) keys[i] = 0;
+  __syncthreads();
+  for (uint32_t size = 2; size <= n2; size <<= 1) {
+    for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+      for (uint32_t i = tid; i < n2 / 2; i += 256) {
+        const uint32_t lo = 2 * i - (i & (stride - 1));
+        const uint32_t hi = lo + stride;
+        const bool desc = (lo & size) == 0;
+        const uint64_t x = keys[lo], y = keys[hi];
+        if ((x < y) == desc) {
+          keys[lo] = y;
+          keys[hi] = x;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  for (uint32_t i = tid; i < kept; i += 256) top[i] = keys[i];
+  if (tid == 0) {
+    a.top_count[q] = kept;
+    a.cand_count[q] = 0;
+    if (kept == (uint32_t)k) a.thr[q] = ordered_f32((uint32_t)(keys[k - 1] >> 32));
+  }
+}
+
+__global__ void scan_init_kernel(uint32_t* top_count, uint32_t* cand_count, float* thr, int Q, uint32_t* row_max_enc,
+                                 int64_t n_rows) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < Q) {
+    if (top_count) top_count[i] = 0;
+    if (cand_count) cand_count[i] = 0;
+    if (thr) thr[i] = -INFINITY;
+  }
+  if (row_max_enc && i < n_rows) row_max_enc[i] = 0;  // below every encoded float
+}
+
+__global__ void scan_finish_kernel(const uint64_t* top, int Q, int k, int64_t row_base, float* topk_val,
+                                   int64_t* topk_idx, const uint32_t* row_max_enc, float* row_max, int64_t n_rows) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (top != nullptr && i < (int64_t)Q * k) {
+    const uint64_t key = top[i];
+    topk_val[i] = ordered_f32((uint32_t)(key >> 32));
+    topk_idx[i] = (int64_t)(0xffffffffu - (uint32_t)key) + row_base;
+  }
+  if (row_max != nullptr && i < n_rows) row_max[i] = ordered_f32(row_max_enc[i]);
+}
+
+// ---- host side --------------------------------------------------------------------------------
+constexpr int64_t SCAN_DEFAULT_CHUNK = 65536;
+constexpr int64_t SCAN_FIRST_CHUNK = 4096;
+
+static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+struct ScanLayout {
+  size_t top, top_count, cand_count, thr, cand, total;
+};
+
+static ScanLayout scan_layout(int Q, int k, int64_t chunk_rows) {
+  ScanLayout l;
+  size_t off = 0;
+  l.top = off;
+  off += align_up((size_t)Q * (size_t)(k > 0 ? k : 0) * 8, 256);
+  l.top_count = off;
+  off += align_up((size_t)Q * 4, 256);
+  l.cand_count = off;
+  off += align_up((size_t)Q * 4, 256);
+  l.thr = off;
+  off += align_up((size_t)Q * 4, 256);
+  l.cand = off;
+  off += k > 0 ? align_up((size_t)Q * (size_t)chunk_rows * 8, 256) : 0;
+  l.total = off;
+  return l;
+}
+
+static int64_t effective_chunk(int64_t chunk_rows) { return chunk_rows > 0 ? chunk_rows : SCAN_DEFAULT_CHUNK; }
+
+size_t scan_workspace_bytes(int Q, int k, int64_t chunk_rows) {
+  if (Q <= 0 || k < 0) return 0;
+  return scan_layout(Q, k, effective_chunk(chunk_rows)).total;
+}
+
+template <typename T, int BM, int BN, int WM, int WN>
+static int launch_gemm(const ScanArgs& a, bool aligned, hipStream_t st) {
+  constexpr int NT = WM * WN * 64;
+  constexpr size_t smem = 2 * (size_t)(BM + BN) * LDS_ROW_BYTES;
+  const int row_tiles_pad = (a.row_tiles + 7) / 8 * 8;
+  const dim3 grid((unsigned)(row_tiles_pad * a.q_tiles));
+  if (aligned) {
+    auto kern = scan_gemm_kernel<T, BM, BN, WM, WN, true>;
+    BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL(kern, grid, dim3(NT), smem, st, a);
+  } else {
+    auto kern = scan_gemm_kernel<T, BM, BN, WM, WN, false>;
+    BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL(kern, grid, dim3(NT), smem, st, a);
+  }
+  BGX_HIP(hipGetLastError());
+  return 0;
+}
+
+template <typename T>
+static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
+  // large tiles when there is enough work to fill the chip with them
+  if (a.Q > 64 && a.rows >= 4096) {
+    constexpr int BM = 256, BN = 256;
+    a.row_tiles = (int)((a.rows + BM - 1) / BM);
+    a.q_tiles = (a.Q + BN - 1) / BN;
+    return launch_gemm<T, BM, BN, 2, 2>(a, aligned, st);
+  } else if (a.Q > 32) {
+    constexpr int BM = 128, BN = 64;
+    a.row_tiles = (int)((a.rows + BM - 1) / BM);
+    a.q_tiles = (a.Q + BN - 1) / BN;
+    return launch_gemm<T, BM, BN, 4, 1>(a, aligned, st);
+  } else {
+    constexpr int BM = 128, BN = 32;
+    a.row_tiles = (int)((a.rows + BM - 1) / BM);
+    a.q_tiles = (a.Q + BN - 1) / BN;
+    return launch_gemm<T, BM, BN, 4, 1>(a, aligned, st);
+  }
+}
+
+int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int dtype, const void* queries, int Q,
+              float query_scale, int unit_norm, int k, int64_t row_base, float* topk_val, int64_t* topk_idx,
+              float* row_max, float* scores, float* sumsq, void* ws, size_t ws_bytes, int64_t chunk_rows,
+              void* stream) {
+  BGX_REQUIRE(store && queries, BGX_E_ARG, "scan: null store/queries");
+  BGX_REQUIRE(n_rows > 0 && D > 0 && Q > 0 && stride >= D, BGX_E_ARG, "scan: n_rows=%lld D=%lld Q=%d stride=%lld",
+              (long long)n_rows, (long long)D, Q, (long long)stride);
+  BGX_REQUIRE(dtype >= BGX_F32 && dtype <= BGX_BF16, BGX_E_DTYPE, "scan: dtype=%d", dtype);
+  BGX_REQUIRE(row_base >= 0 && n_rows + row_base <= 0xffffffffLL, BGX_E_SHAPE,
+              "scan: row numbers must fit 32 bits (n_rows=%lld row_base=%lld)", (long long)n_rows, (long long)row_base);
+  const bool want_topk = topk_val != nullptr || topk_idx != nullptr;
+  if (want_topk) {
+    BGX_REQUIRE(topk_val && topk_idx, BGX_E_ARG, "scan: topk_val and topk_idx go together");
+    BGX_REQUIRE(k >= 1 && k <= SCAN_KMAX && k <= n_rows, BGX_E_SHAPE, "scan: k=%d outside 1..min(%d, n_rows=%lld)", k,
+                SCAN_KMAX, (long long)n_rows);
+  } else {
+    k = 0;
+  }
+  const int64_t chunk = effective_chunk(chunk_rows);
+  const ScanLayout lay = scan_layout(Q, k, chunk);
+  const bool need_init = want_topk || row_max != nullptr;
+  if (want_topk) {
+    BGX_REQUIRE(ws != nullptr, BGX_E_WORKSPACE, "scan: workspace required for top-k");
+    BGX_REQUIRE(((uintptr_t)ws & 255) == 0, BGX_E_ALIGN, "scan: workspace must be 256-byte aligned");
+    BGX_REQUIRE(ws_bytes >= lay.total, BGX_E_WORKSPACE, "scan: workspace %zu < %zu bytes", ws_bytes, lay.total);
+  }
+  hipStream_t st = (hipStream_t)stream;
+  char* w = (char*)ws;
+  uint64_t* top = want_topk ? (uint64_t*)(w + lay.top) : nullptr;
+  uint32_t* top_count = want_topk ? (uint32_t*)(w + lay.top_count) : nullptr;
+  uint32_t* cand_count = want_topk ? (uint32_t*)(w + lay.cand_count) : nullptr;
+  float* thr = want_topk ? (float*)(w + lay.thr) : nullptr;
+  uint64_t* cand = want_topk ? (uint64_t*)(w + lay.cand) : nullptr;
+  // the row maxima are accumulated in place in an order-preserving integer
+  // encoding and decoded by the finish kernel
+  uint32_t* row_max_enc = (uint32_t*)row_max;
+
+  if (need_init) {
+    const int64_t n_init = (row_max ? n_rows : 0) > Q ? n_rows : Q;
+    hipLaunchKernelGGL(scan_init_kernel, dim3((unsigned)((n_init + 255) / 256)), dim3(256), 0, st, top_count,
+                       cand_count, thr, Q, row_max_enc, row_max ? n_rows : 0);
+    BGX_HIP(hipGetLastError());
+  }
+
+  const size_t esz = dtype_size(dtype);
+  const int epl = dtype == BGX_F32 ? 4 : 8;
+  const bool aligned = ((uintptr_t)store % 16 == 0) && ((uintptr_t)queries % 16 == 0) && (D % epl == 0) &&
+                       (stride % epl == 0);
+  (void)esz;
+
+  int64_t done = 0;
+  while (done < n_rows) {
+    int64_t rows = n_rows - done;
+    if (want_topk) {
+      int64_t lim = done == 0 ? SCAN_FIRST_CHUNK : done * 4;
+      if (lim < k) lim = k;
+      if (lim > chunk) lim = chunk;
+      if (rows > lim) rows = lim;
+    }
+    ScanArgs a;
+    a.store = store;
+    a.queries = queries;
+    a.row0 = done;
+    a.rows = rows;
+    a.D = D;
+    a.store_stride = stride;
+    a.Q = Q;
+    a.row_tiles = 0;
+    a.q_tiles = 0;
+    a.query_scale = query_scale;
+    a.unit_norm = unit_norm;
+    a.scores = scores;
+    a.sumsq = sumsq;
+    a.row_max_enc = row_max_enc;
+    a.thr = thr;
+    a.cand_count = cand_count;
+    a.cand = cand;
+    a.cand_cap = chunk;
+    int rc;
+    if (dtype == BGX_F16)
+      rc = launch_gemm_t<f16_t>(a, aligned, st);
+    else if (dtype == BGX_BF16)
+      rc = launch_gemm_t<bf16_t>(a, aligned, st);
+    else
+      rc = launch_gemm_t<float>(a, aligned, st);
+    if (rc != 0) return rc;
+    if (want_topk) {
+      SelectArgs s;
+      s.top = top;
+      s.top_count = top_count;
+      s.cand = cand;
+      s.cand_count = cand_count;
+      s.thr = thr;
+      s.cand_cap = chunk;
+      s.k = k;
+      hipLaunchKernelGGL(scan_select_kernel, dim3((unsigned)Q), dim3(256), 0, st, s);
+      BGX_HIP(hipGetLastError());
+    }
+    done += rows;
+  }
+
+  if (need_init) {
+    const int64_t n_fin = ((int64_t)Q * k > (row_max ? n_rows : 0)) ? (int64_t)Q * k : n_rows;
+    hipLaunchKernelGGL(scan_finish_kernel, dim3((unsigned)((n_fin + 255) / 256)), dim3(256), 0, st,
+                       (const uint64_t*)top, Q, k, row_base, topk_val, topk_idx, (const uint32_t*)row_max_enc, row_max,
+                       row_max ? n_rows : 0);
+    BGX_HIP(hipGetLastError());
+  }
+  return 0;
+}
+
+}  // namespace bgx

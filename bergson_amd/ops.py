@@ -1,0 +1,216 @@
+"""Tensor-level wrappers over the C ABI: argument checks, workspace and stream plumbing.
+
+Every function here enqueues HIP kernels on torch's current stream and returns
+without synchronising.  Tensors must live on the GPU; there is no CPU path.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import torch
+from torch import Tensor
+
+from . import _lib
+from ._lib import BGX_BF16, BGX_F16, BGX_F32, ModuleDesc
+
+DTYPE_CODE = {torch.float32: BGX_F32, torch.float16: BGX_F16, torch.bfloat16: BGX_BF16}
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return DTYPE_CODE[dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {dtype}; the kernels take float32, float16 and bfloat16") from None
+
+
+def _need_gpu(t: Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a GPU tensor: bergson_amd has no CPU path (got device {t.device})")
+
+
+def _stream() -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: Tensor | None) -> C.c_void_p | None:
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+_workspaces: dict[tuple[int, str], Tensor] = {}
+
+
+def _workspace(device: torch.device, nbytes: int, tag: str) -> Tensor:
+    """Per-device scratch buffer, grown on demand and reused between calls (stream-ordered)."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), tag)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def adafactor_scales(row: Tensor | None, col: Tensor | None, dtype: torch.dtype) -> tuple[Tensor | None, Tensor | None]:
+    """(row_scale [O], col_scale [I]) fp32 vectors of Adafactor factors rounded to `dtype`."""
+    lib = _lib.load()
+    ref = row if row is not None else col
+    assert ref is not None
+    _need_gpu(ref, "row/col")
+    row32 = row.detach().to(torch.float32).contiguous() if row is not None else None
+    col32 = col.detach().to(torch.float32).contiguous() if col is not None else None
+    row_scale = torch.empty_like(row32) if row32 is not None else None
+    col_scale = torch.empty_like(col32) if col32 is not None else None
+    rc = lib.bgx_adafactor_scales(
+        _ptr(row32), 0 if row32 is None else row32.numel(), _ptr(col32), 0 if col32 is None else col32.numel(),
+        dtype_code(dtype), _ptr(row_scale), _ptr(col_scale), _stream(),
+    )
+    _lib.check(rc, "bgx_adafactor_scales")
+    return row_scale, col_scale
+
+
+@dataclass
+class ModuleInput:
+    """One hooked module of one batch, as the collection kernels see it."""
+
+    a: Tensor  # [N, S, I]
+    g: Tensor  # [N, S, O]
+    r_in: Tensor  # [p, I], dtype of a
+    r_out: Tensor  # [p, O]
+    out_col: int
+    col_scale: Tensor | None = None  # [I] fp32
+    row_scale: Tensor | None = None  # [O] fp32
+
+
+def _rows_view(t: Tensor, name: str) -> Tensor:
+    if t.dim() != 3:
+        raise ValueError(f"{name} must be [N, S, features], got {tuple(t.shape)}")
+    return t if t.stride(2) == 1 else t.contiguous()
+
+
+def _collect(per_token: bool, modules: list[ModuleInput], p: int, out: Tensor, lengths: Tensor | None,
+             rows: Tensor | None, lo: float, hi: float) -> None:
+    lib = _lib.load()
+    if not modules:
+        raise ValueError("no modules to collect")
+    _need_gpu(out, "out")
+    if out.dim() != 2 or out.stride(1) != 1:
+        raise ValueError("out must be a 2-D tensor with contiguous rows")
+    N, S = modules[0].a.shape[:2]
+    in_dtype = modules[0].a.dtype
+    keep = []  # tensors that must stay alive until the launch is enqueued
+    descs = (ModuleDesc * len(modules))()
+    for d, m in zip(descs, modules):
+        a = _rows_view(m.a, "a")
+        g = _rows_view(m.g, "g")
+        _need_gpu(a, "a")
+        _need_gpu(g, "g")
+        if a.shape[:2] != (N, S) or g.shape[:2] != (N, S):
+            raise ValueError(f"all modules of a launch share [N, S]; got a {tuple(a.shape)} g {tuple(g.shape)}")
+        if a.dtype != in_dtype or g.dtype != in_dtype:
+            raise TypeError(f"all a/g of a launch share one dtype; got {a.dtype} and {g.dtype} vs {in_dtype}")
+        I, O = a.shape[2], g.shape[2]
+        r_in = m.r_in.contiguous()
+        r_out = m.r_out.contiguous()
+        if r_in.shape != (p, I) or r_out.shape != (p, O):
+            raise ValueError(f"projection shapes {tuple(r_in.shape)} / {tuple(r_out.shape)} do not match p={p} I={I} O={O}")
+        if r_in.dtype != in_dtype or r_out.dtype != in_dtype:
+            raise TypeError("projection matrices must have the dtype of the activations")
+        for s, n, k in ((m.col_scale, "col_scale", I), (m.row_scale, "row_scale", O)):
+            if s is not None and (s.dtype != torch.float32 or s.numel() != k or not s.is_contiguous()):
+                raise ValueError(f"{n} must be a contiguous fp32 vector of {k} elements")
+        keep += [a, g, r_in, r_out]
+        d.a, d.g, d.r_in, d.r_out = a.data_ptr(), g.data_ptr(), r_in.data_ptr(), r_out.data_ptr()
+        d.col_scale = None if m.col_scale is None else m.col_scale.data_ptr()
+        d.row_scale = None if m.row_scale is None else m.row_scale.data_ptr()
+        d.bias_col = None
+        d.bias_scale = None
+        d.a_seq_stride, d.a_tok_stride = a.stride(0), a.stride(1)
+        d.g_seq_stride, d.g_tok_stride = g.stride(0), g.stride(1)
+        d.out_col = m.out_col
+        d.I, d.O = I, O
+    if lengths is not None:
+        if lengths.dtype != torch.int32 or lengths.numel() != N or not lengths.is_contiguous():
+            raise ValueError("lengths must be a contiguous int32 vector of N elements")
+        _need_gpu(lengths, "lengths")
+    if rows is not None:
+        if rows.dtype != torch.int64 or rows.numel() != N or not rows.is_contiguous():
+            raise ValueError("row indices / offsets must be a contiguous int64 vector of N elements")
+        _need_gpu(rows, "rows")
+    nbytes = lib.bgx_collect_workspace_bytes(len(modules), N, S, p)
+    ws = _workspace(out.device, nbytes, "collect")
+    fn = lib.bgx_collect_tok if per_token else lib.bgx_collect_seq
+    rc = fn(descs, len(modules), N, S, p, dtype_code(in_dtype), _ptr(lengths), _ptr(rows), _ptr(out),
+            out.stride(0), dtype_code(out.dtype), lo, hi, _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "bgx_collect_tok" if per_token else "bgx_collect_seq")
+    del keep
+
+
+def collect_seq(modules: list[ModuleInput], p: int, out: Tensor, *, lengths: Tensor | None = None,
+                out_rows: Tensor | None = None, lo: float = float("-inf"), hi: float = float("inf")) -> None:
+    """out[row(n), m.out_col : m.out_col + p*p] = clamp(sum_s g'[n,s] (x) a'[n,s]) for every module m."""
+    _collect(False, modules, p, out, lengths, out_rows, lo, hi)
+
+
+def collect_tok(modules: list[ModuleInput], p: int, out: Tensor, *, lengths: Tensor, row_offsets: Tensor,
+                lo: float = float("-inf"), hi: float = float("inf")) -> None:
+    """out[row_offsets[n] + s, block(m)] = clamp(g'[n,s] (x) a'[n,s]) for s < lengths[n] - 1."""
+    _collect(True, modules, p, out, lengths, row_offsets, lo, hi)
+
+
+def unit_normalize_rows_(rows: Tensor) -> Tensor:
+    """In-place g * rsqrt(max(sum g^2, eps^2)) per row."""
+    lib = _lib.load()
+    _need_gpu(rows, "rows")
+    if rows.dim() != 2 or rows.stride(1) != 1:
+        raise ValueError("rows must be 2-D with contiguous rows")
+    rc = lib.bgx_unit_normalize_rows(_ptr(rows), rows.shape[0], rows.shape[1], rows.stride(0), dtype_code(rows.dtype),
+                                     _stream())
+    _lib.check(rc, "bgx_unit_normalize_rows")
+    return rows
+
+
+@dataclass
+class ScanResult:
+    topk_values: Tensor | None = None  # [Q, k] fp32
+    topk_indices: Tensor | None = None  # [Q, k] int64
+    row_max: Tensor | None = None  # [n_rows] fp32
+    scores: Tensor | None = None  # [n_rows, Q] fp32
+    sumsq: Tensor | None = None  # [n_rows] fp32
+
+
+def scan(store: Tensor, queries: Tensor, *, unit_norm: bool, k: int = 0, query_scale: float = 1.0, row_base: int = 0,
+         want_row_max: bool = False, want_scores: bool = False, want_sumsq: bool = False,
+         chunk_rows: int = 0) -> ScanResult:
+    """Score store rows [n, D] against queries [Q, D] (same dtype); see bgx_scan in include/bergson_amd.h."""
+    lib = _lib.load()
+    _need_gpu(store, "store")
+    _need_gpu(queries, "queries")
+    if store.dim() != 2 or store.stride(1) != 1:
+        raise ValueError("store must be 2-D with contiguous rows")
+    if queries.dim() != 2 or queries.shape[1] != store.shape[1]:
+        raise ValueError(f"queries {tuple(queries.shape)} do not match store {tuple(store.shape)}")
+    if queries.dtype != store.dtype:
+        raise TypeError("queries must have the store dtype")
+    queries = queries.contiguous()
+    n, D = store.shape
+    Q = queries.shape[0]
+    dev = store.device
+    res = ScanResult()
+    if k:
+        res.topk_values = torch.empty((Q, k), dtype=torch.float32, device=dev)
+        res.topk_indices = torch.empty((Q, k), dtype=torch.int64, device=dev)
+    if want_row_max:
+        res.row_max = torch.empty((n,), dtype=torch.float32, device=dev)
+    if want_scores:
+        res.scores = torch.empty((n, Q), dtype=torch.float32, device=dev)
+    if want_sumsq:
+        res.sumsq = torch.empty((n,), dtype=torch.float32, device=dev)
+    ws = None
+    if k:
+        ws = _workspace(dev, lib.bgx_scan_workspace_bytes(Q, k, chunk_rows), "scan")
+    rc = lib.bgx_scan(_ptr(store), n, D, store.stride(0), dtype_code(store.dtype), _ptr(queries), Q, query_scale,
+                      int(unit_norm), k, row_base, _ptr(res.topk_values), _ptr(res.topk_indices), _ptr(res.row_max),
+                      _ptr(res.scores), _ptr(res.sumsq), _ptr(ws), 0 if ws is None else ws.numel(), chunk_rows,
+                      _stream())
+    _lib.check(rc, "bgx_scan")
+    return res

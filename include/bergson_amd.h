@@ -1,0 +1,177 @@
+/*
+ * bergson_amd.h -- C ABI of the MI355X (gfx950) hot path for projected
+ * per-example gradient collection and gradient-store scoring.
+ *
+ * The reference (EleutherAI/bergson) is pure Python on PyTorch: it has no FFI
+ * of its own.  Every entry point below replaces a *sequence of PyTorch ops*
+ * that the reference issues from module hooks or from its scorer; the comment
+ * on each entry point names that sequence as bergson/<file>:<lines>.
+ *
+ * Conventions
+ *   - every function returns 0 on success, a positive hipError_t when a HIP
+ *     call failed, or a negative BGX_E_* code when an argument was rejected
+ *     before anything was enqueued.  bgx_last_error() gives the message of
+ *     the last failure on the calling thread.
+ *   - all pointers named *_dev are device pointers owned by the caller; the
+ *     library allocates nothing and never synchronises the host: all work is
+ *     enqueued on `stream` (a hipStream_t passed as void*; NULL = the null
+ *     stream).
+ *   - "rows" are store rows; "tokens" are (sequence, position) pairs.
+ *   - dtypes are BGX_F32 / BGX_F16 / BGX_BF16.
+ */
+#ifndef BERGSON_AMD_H
+#define BERGSON_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BGX_ABI_VERSION 1
+
+enum bgx_dtype { BGX_F32 = 0, BGX_F16 = 1, BGX_BF16 = 2 };
+
+enum bgx_error {
+  BGX_E_ARG = -1,       /* null / negative / inconsistent argument          */
+  BGX_E_DTYPE = -2,     /* dtype code not supported by this entry point     */
+  BGX_E_SHAPE = -3,     /* shape outside what the kernels are built for     */
+  BGX_E_WORKSPACE = -4, /* workspace smaller than bgx_*_workspace_bytes()   */
+  BGX_E_ALIGN = -5      /* pointer / stride alignment requirement violated  */
+};
+
+/* One hooked module (nn.Linear / Conv1D) of one batch.
+ *   a      [N, S, I]  module input   (bergson/collector/collector.py:453-458)
+ *   g      [N, S, O]  grad wrt module output (collector.py:460-472)
+ * both in the model dtype, last dimension contiguous, element strides given.
+ *   r_in   [p, I] row-major, model dtype: the "right" projection without its
+ *          bias column (collector.py:336-362, :1029-1063)
+ *   r_out  [p, O] row-major: the "left" projection
+ *   col_scale [I] fp32 or NULL: Adafactor input-side factor
+ *          rsqrt(col + 1e-30) already rounded to the model dtype
+ *          (collector.py:532-535)
+ *   row_scale [O] fp32 or NULL: Adafactor output-side factor
+ *          sqrt(mean(row+1e-30)) * rsqrt(row+1e-30), rounded likewise
+ *          (collector.py:655-658)
+ *   bias_col [p] fp32 or NULL: column I of the [p, I+1] right projection when
+ *          the bias gradient is collected (collector.py:552-590)
+ *   bias_scale [O] fp32 or NULL: factor applied to g for the bias column only
+ *          (rsqrt(bias_avg_sq + 1e-8), gradients.py:339-349); NULL = 1
+ *   out_col  first column of this module's p*p block in an output row
+ *          (bergson/data.py:380-389)
+ */
+typedef struct bgx_module_desc {
+  const void* a;
+  const void* g;
+  const void* r_in;
+  const void* r_out;
+  const float* col_scale;
+  const float* row_scale;
+  const float* bias_col;
+  const float* bias_scale;
+  int64_t a_seq_stride;
+  int64_t a_tok_stride;
+  int64_t g_seq_stride;
+  int64_t g_tok_stride;
+  int64_t out_col;
+  int32_t I;
+  int32_t O;
+} bgx_module_desc;
+
+int bgx_abi_version(void);
+const char* bgx_last_error(void);
+
+/* Adafactor factors of one module, computed once per module.
+ * Replaces collector.py:532-535 and :655-658 (closed form in
+ * bergson/gradients.py:300-337, eps = 1e-30):
+ *   col_scale[i] = round_dtype(rsqrt(col[i] + 1e-30))
+ *   row_scale[o] = round_dtype(sqrt(mean(row + 1e-30)) * rsqrt(row[o] + 1e-30))
+ * row/col are fp32 device vectors; outputs are fp32 vectors holding values
+ * representable in `dtype`.  Either pair may be NULL/0 to skip it. */
+int bgx_adafactor_scales(const float* row_dev, int32_t O, const float* col_dev,
+                         int32_t I, int32_t dtype, float* row_scale_dev,
+                         float* col_scale_dev, void* stream);
+
+/* Bytes of device workspace bgx_collect_seq / bgx_collect_tok need. */
+size_t bgx_collect_workspace_bytes(int32_t n_modules, int32_t N, int32_t S,
+                                   int32_t p);
+
+/* Per-sequence projected gradients of n_modules modules of one batch in ONE
+ * launch (plus a small deterministic reduction launch).
+ * Replaces, per module: the forward-hook scale + `a @ R_in^T`
+ * (collector.py:518-543), the backward-hook scale + `g @ R_out^T`, the token
+ * reduction `g'.mT @ a'`, `flatten(1).clamp_(lo, hi)` and the cast to the
+ * store dtype (collector.py:646-742; gradient_collectors.py:96-112), and the
+ * concatenation of modules into one row (bergson/builder.py:17-32).
+ *   out[row(n), mods[m].out_col + i*p + j] =
+ *       cast(clamp(sum_s g'[n,s,i] * a'[n,s,j]))
+ *   row(n) = out_rows_dev ? out_rows_dev[n] : n
+ * mods_host is a HOST array; it is copied into the workspace on `stream`
+ * (pageable memory is staged before return; pinned memory must stay valid
+ * until the stream reaches the copy).
+ * lengths_dev [N] int32 or NULL: document lengths; positions s >= len-1 carry
+ * an exactly-zero g (right padding, causal model, labels -100;
+ * bergson/data.py:800-804) and are skipped.
+ * p in 1..64. */
+int bgx_collect_seq(const bgx_module_desc* mods_host, int32_t n_modules,
+                    int32_t N, int32_t S, int32_t p, int32_t in_dtype,
+                    const int32_t* lengths_dev, const int64_t* out_rows_dev,
+                    void* out_dev, int64_t out_row_stride, int32_t out_dtype,
+                    float clamp_lo, float clamp_hi, void* workspace_dev,
+                    size_t workspace_bytes, void* stream);
+
+/* Per-token variant (attribute_tokens): no token reduction; row
+ * row_offsets_dev[n] + s of `out` receives flatten(g'[n,s] (x) a'[n,s]) for
+ * s < lengths_dev[n] - 1.  Replaces collector.py:660-683 / :730-736 (the
+ * [N,S,p,p] product and the boolean-mask gather) and the ragged scatter of
+ * bergson/builder.py:174-188.  lengths_dev and row_offsets_dev are required. */
+int bgx_collect_tok(const bgx_module_desc* mods_host, int32_t n_modules,
+                    int32_t N, int32_t S, int32_t p, int32_t in_dtype,
+                    const int32_t* lengths_dev, const int64_t* row_offsets_dev,
+                    void* out_dev, int64_t out_row_stride, int32_t out_dtype,
+                    float clamp_lo, float clamp_hi, void* workspace_dev,
+                    size_t workspace_bytes, void* stream);
+
+/* In-place unit normalisation of rows: g * rsqrt(max(sum g^2, eps_fp32^2)),
+ * replaces bergson/builder.py:14,:28-30.  rows_dev [n_rows, D], row stride in
+ * elements. */
+int bgx_unit_normalize_rows(void* rows_dev, int64_t n_rows, int64_t D,
+                            int64_t row_stride, int32_t dtype, void* stream);
+
+/* ---- gradient-store scoring ------------------------------------------- */
+
+/* Bytes of device workspace bgx_scan needs for Q queries, top-k of k and at
+ * most chunk_rows store rows per internal pass (0 = library default). */
+size_t bgx_scan_workspace_bytes(int32_t Q, int32_t k, int64_t chunk_rows);
+
+/* Scores n_rows store rows [n_rows, D] (row stride in elements) against Q
+ * queries [Q, D] of the same dtype, streaming the store once.
+ *   score[n, q] = query_scale * <store[n], queries[q]> * w[n]
+ *   w[n] = unit_norm ? (sumsq[n] > 0 ? 1/sqrt(sumsq[n]) : 0) : 1
+ * which is the index-side normalisation of bergson/score/scorer.py:89-115
+ * (scores / clamp_min(sqrt(sum g^2), 1e-12)) and of
+ * bergson/query/attributor.py:137-167 (g / ||g||, nan -> 0); queries are
+ * normalised by the caller as the reference does before scoring
+ * (attributor.py:202-206, bergson/process_grads.py:156-164).
+ * Outputs, each optional (NULL to skip):
+ *   topk_val_dev [Q, k] fp32, topk_idx_dev [Q, k] int64: per query the k
+ *     largest scores in descending order, ties broken by lower row index
+ *     (torch.topk, attributor.py:229-235); requires k <= n_rows, k <= 2048
+ *   row_max_dev [n_rows] fp32: max over queries (score_mode "nearest",
+ *     scorer.py:111-113)
+ *   scores_dev [n_rows, Q] fp32 row-major: every score (scorer.py:89-115)
+ *   sumsq_dev [n_rows] fp32: sum of squares of each row
+ * row_base is added to the row numbers reported in topk_idx_dev. */
+int bgx_scan(const void* store_dev, int64_t n_rows, int64_t D,
+             int64_t store_row_stride, int32_t dtype, const void* queries_dev,
+             int32_t Q, float query_scale, int32_t unit_norm, int32_t k,
+             int64_t row_base, float* topk_val_dev, int64_t* topk_idx_dev,
+             float* row_max_dev, float* scores_dev, float* sumsq_dev,
+             void* workspace_dev, size_t workspace_bytes, int64_t chunk_rows,
+             void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BERGSON_AMD_H */

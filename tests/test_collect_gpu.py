@@ -1,0 +1,222 @@
+"""HIP collection kernels against the CPU oracle (the reference's op sequence).
+
+Tolerances: relative L2 <= 1e-5 for fp32 inputs, <= 1e-2 for bf16 / fp16 inputs.
+"""
+import pytest
+import torch
+
+from helpers import TOL, rel_l2
+from oracle import hooks as ohooks
+from oracle.projection import module_projections
+
+pytestmark = pytest.mark.gpu
+
+
+def make_case(N, S, I, O, p, dtype, seed, normalizer=None, name="layers.0.mlp.dense_h_to_4h"):
+    gen = torch.Generator().manual_seed(seed)
+    a = torch.randn(N, S, I, generator=gen).to(dtype)
+    g = (torch.randn(N, S, O, generator=gen) * 0.1).to(dtype)
+    left, right = module_projections(name, p, O, I, dtype)
+    norm = None
+    if normalizer == "adafactor":
+        row = torch.randn(O, generator=gen).abs() * 1e-4
+        col = torch.randn(I, generator=gen).abs() * 1e-4
+        norm = ohooks.Adafactor(row=row, col=col)
+    return a, g, left, right, norm
+
+
+def run_kernel(device, cases, p, out_dtype, *, lengths=None, per_token=False, row_offsets=None, n_rows=None,
+               out_rows=None, lo=float("-inf"), hi=float("inf")):
+    from bergson_amd import ops
+
+    mods = []
+    col = 0
+    for a, g, left, right, norm in cases:
+        cs = rs = None
+        if norm is not None:
+            rs, cs = ops.adafactor_scales(norm.row.to(device), norm.col.to(device), a.dtype)
+        mods.append(ops.ModuleInput(a=a.to(device), g=g.to(device), r_in=right.to(device), r_out=left.to(device),
+                                    out_col=col, col_scale=cs, row_scale=rs))
+        col += p * p
+    N = cases[0][0].shape[0]
+    rows = n_rows if n_rows is not None else N
+    out = torch.zeros(rows, col, dtype=out_dtype, device=device)
+    ldev = None if lengths is None else torch.tensor(lengths, dtype=torch.int32, device=device)
+    if per_token:
+        ops.collect_tok(mods, p, out, lengths=ldev, row_offsets=torch.tensor(row_offsets, dtype=torch.int64, device=device),
+                        lo=lo, hi=hi)
+    else:
+        odev = None if out_rows is None else torch.tensor(out_rows, dtype=torch.int64, device=device)
+        ops.collect_seq(mods, p, out, lengths=ldev, out_rows=odev, lo=lo, hi=hi)
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+def oracle_rows(cases, out_dtype, **kw):
+    lo, hi = torch.finfo(out_dtype).min, torch.finfo(out_dtype).max
+    outs = [ohooks.module_gradient(a, g, norm, left, right, lo=lo, hi=hi, **kw).to(out_dtype)
+            for a, g, left, right, norm in cases]
+    return torch.cat(outs, dim=1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(2, 64, 128, 384, 16), (3, 100, 256, 128, 16), (1, 7, 64, 64, 16),
+                                   (2, 130, 128, 128, 32), (2, 70, 96, 160, 8), (2, 33, 64, 32, 5),
+                                   (1, 65, 128, 64, 48)])
+def test_seq_no_normalizer(device, dtype, shape):
+    N, S, I, O, p = shape
+    case = make_case(N, S, I, O, p, dtype, seed=1)
+    out_dtype = dtype
+    got = run_kernel(device, [case], p, out_dtype, lo=torch.finfo(out_dtype).min, hi=torch.finfo(out_dtype).max)
+    want = oracle_rows([case], out_dtype)
+    assert got.shape == want.shape
+    assert rel_l2(got, want) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_seq_unaligned_features(device, dtype):
+    # odd feature counts take the element-wise loader
+    case = make_case(2, 50, 100, 37, 16, dtype, seed=2)
+    got = run_kernel(device, [case], 16, dtype)
+    want = oracle_rows([case], dtype)
+    assert rel_l2(got, want) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_seq_adafactor(device, dtype):
+    a, g, left, right, norm = make_case(3, 150, 256, 512, 16, dtype, seed=3, normalizer="adafactor")
+    case = (a, g * 1e-3, left, right, norm)  # keeps every value inside the fp16 range of the store
+    out_dtype = torch.float16 if dtype == torch.bfloat16 else dtype
+    lo, hi = torch.finfo(out_dtype).min, torch.finfo(out_dtype).max
+    got = run_kernel(device, [case], 16, out_dtype, lo=lo, hi=hi)
+    want = oracle_rows([case], out_dtype)
+    assert torch.isfinite(got.float()).all()
+    assert rel_l2(got, want) <= TOL[dtype]
+
+
+def test_seq_adafactor_matches_closed_form_fp32(device):
+    # independent of the hook formulation: L @ normalize_weight(G^T A) @ R^T per sequence
+    a, g, left, right, norm = make_case(2, 40, 64, 96, 16, torch.float32, seed=4, normalizer="adafactor")
+    got = run_kernel(device, [(a, g, left, right, norm)], 16, torch.float32)
+    full = g.mT.double() @ a.double()  # [N, O, I]
+    r = norm.row.double() + 1e-30
+    c = norm.col.double() + 1e-30
+    full = full * (r.mean().sqrt() * r.rsqrt())[:, None] * c.rsqrt()[None, :]
+    want = (left.double() @ full @ right.double().T).flatten(1)
+    assert rel_l2(got, want) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_seq_multi_module_and_lengths(device, dtype):
+    N, S = 4, 200
+    lengths = [200, 131, 64, 2]
+    cases = []
+    for i, (I, O) in enumerate([(128, 384), (128, 128), (128, 512), (512, 128)]):
+        a, g, left, right, norm = make_case(N, S, I, O, 16, dtype, seed=10 + i, normalizer="adafactor",
+                                            name=f"layers.{i}.x")
+        # a causal model with right padding yields an exactly-zero g from position len-1 on
+        for n, l in enumerate(lengths):
+            g[n, l - 1:] = 0
+        cases.append((a, g, left, right, norm))
+    out_rows = [5, 0, 3, 1]
+    got = run_kernel(device, cases, 16, dtype, lengths=lengths, out_rows=out_rows, n_rows=6)
+    want = oracle_rows(cases, dtype)
+    assert rel_l2(got[out_rows], want) <= TOL[dtype]
+    assert got[[2, 4]].abs().sum() == 0
+    # without lengths the padded positions are read and contribute exactly zero
+    got_dense = run_kernel(device, cases, 16, dtype)
+    assert rel_l2(got_dense, want) <= TOL[dtype]
+
+
+def test_seq_bf16_to_fp16_store_saturates_finite(device):
+    # A bf16 model writing an fp16 store: the kernel clamps in fp32 at +-65504 and stays finite.  (The
+    # reference's clamp_ runs on the bf16 tensor, where the bound rounds up to 65536 and the cast gives inf.)
+    a, g, left, right, norm = make_case(2, 128, 256, 256, 16, torch.bfloat16, seed=6, normalizer="adafactor")
+    hi = torch.finfo(torch.float16).max
+    got = run_kernel(device, [(a, g, left, right, norm)], 16, torch.float16, lo=-hi, hi=hi)
+    want = ohooks.module_gradient(a, g, norm, left, right).float()
+    assert torch.isfinite(got.float()).all()
+    big = want.abs() > 7e4
+    assert big.any() and (got.float().abs()[big] == hi).all()
+    small = want.abs() < 6e4
+    assert rel_l2(got.float()[small], want[small]) <= 1e-2
+
+
+def test_seq_clamp_to_store_dtype(device):
+    a, g, left, right, _ = make_case(1, 64, 64, 64, 16, torch.float32, seed=5)
+    g = g * 1e6
+    lo, hi = torch.finfo(torch.float16).min, torch.finfo(torch.float16).max
+    got = run_kernel(device, [(a, g, left, right, None)], 16, torch.float16, lo=lo, hi=hi)
+    want = ohooks.module_gradient(a, g, None, left, right, lo=lo, hi=hi).to(torch.float16)
+    assert torch.isfinite(got.float()).all()
+    assert (got.float().abs() == hi).any()
+    assert rel_l2(got, want) <= 1e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("p", [16, 32, 8])
+def test_tok(device, dtype, p):
+    N, S = 3, 90
+    lengths = [90, 33, 70]
+    cases = []
+    for i, (I, O) in enumerate([(128, 256), (256, 64)]):
+        cases.append(make_case(N, S, I, O, p, dtype, seed=20 + i, normalizer="adafactor" if i else None,
+                               name=f"layers.{i}.y"))
+    mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+    # documents are stored in a different order than they sit in the batch
+    counts = [l - 1 for l in lengths]
+    doc_order = [2, 0, 1]
+    offs = {}
+    r = 0
+    for d in doc_order:
+        offs[d] = r
+        r += counts[d]
+    row_offsets = [offs[n] for n in range(N)]
+    got = run_kernel(device, cases, p, dtype, lengths=lengths, per_token=True, row_offsets=row_offsets, n_rows=r)
+    want_batch_order = oracle_rows(cases, dtype, attribute_tokens=True, collection_mask=mask)
+    want = torch.zeros_like(want_batch_order)
+    src = 0
+    for n in range(N):
+        want[row_offsets[n]:row_offsets[n] + counts[n]] = want_batch_order[src:src + counts[n]]
+        src += counts[n]
+    assert got.shape == want.shape
+    assert rel_l2(got, want) <= TOL[dtype]
+
+
+def test_tok_rows_sum_to_seq_row(device):
+    # sum over tokens of the per-token rows equals the per-sequence row (fp32)
+    N, S, p = 2, 77, 16
+    lengths = [77, 40]
+    a, g, left, right, _ = make_case(N, S, 128, 64, p, torch.float32, seed=30)
+    for n, l in enumerate(lengths):
+        g[n, l - 1:] = 0
+    case = (a, g, left, right, None)
+    seq = run_kernel(device, [case], p, torch.float32, lengths=lengths)
+    tok = run_kernel(device, [case], p, torch.float32, lengths=lengths, per_token=True, row_offsets=[0, 76], n_rows=76 + 39)
+    assert rel_l2(tok[:76].sum(0), seq[0]) <= 1e-5
+    assert rel_l2(tok[76:].sum(0), seq[1]) <= 1e-5
+
+
+def test_noncontiguous_views(device):
+    # g arriving as a slice of a wider tensor (fused qkv) keeps its strides
+    from bergson_amd import ops
+
+    N, S, I, O, p = 2, 64, 128, 128, 16
+    a, g_full, left, right, _ = make_case(N, S, I, 3 * O, p, torch.bfloat16, seed=40)
+    left = left[:, :O].contiguous()
+    gd = g_full.to(device)[:, :, O:2 * O]
+    assert not gd.is_contiguous()
+    out = torch.zeros(N, p * p, dtype=torch.bfloat16, device=device)
+    ops.collect_seq([ops.ModuleInput(a=a.to(device), g=gd, r_in=right.to(device), r_out=left.to(device), out_col=0)],
+                    p, out)
+    want = ohooks.module_gradient(a, g_full[:, :, O:2 * O], None, left, right)
+    assert rel_l2(out.cpu(), want) <= 1e-2
+
+
+def test_rejects_cpu_tensors():
+    from bergson_amd import ops
+
+    a = torch.zeros(1, 4, 8)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.collect_seq([ops.ModuleInput(a=a, g=a, r_in=torch.zeros(16, 8), r_out=torch.zeros(16, 8), out_col=0)], 16,
+                        torch.zeros(1, 256))

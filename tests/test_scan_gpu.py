@@ -1,0 +1,158 @@
+"""HIP store scan against the CPU oracle: scores within 1e-3 absolute cosine,
+top-k indices identical except where scores tie within that tolerance."""
+import pytest
+import torch
+
+from oracle import scan as oscan
+
+pytestmark = pytest.mark.gpu
+
+COS_TOL = 1e-3
+
+
+def make_store(n, D, Q, dtype, seed, outliers=True):
+    gen = torch.Generator().manual_seed(seed)
+    store = torch.randn(n, D, generator=gen)
+    if outliers:
+        idx = torch.randperm(n, generator=gen)[: max(1, n // 20)]
+        store[idx] *= 10
+    queries = torch.randn(Q, D, generator=gen)
+    return store.to(dtype), queries.to(dtype)
+
+
+def unit_queries(queries, dtype):
+    q = queries.float()
+    q = q / (q.norm(dim=1, keepdim=True) + torch.finfo(torch.float32).eps)
+    return q
+
+
+def check_topk(vals, idx, ref_scores, k, tol=COS_TOL):
+    """vals/idx [Q, k] from the kernel; ref_scores [Q, n] from the oracle."""
+    ref_v, ref_i = torch.topk(ref_scores, k, dim=1)
+    assert (vals - ref_v).abs().max().item() <= tol
+    assert (vals[:, :-1] >= vals[:, 1:]).all(), "values must be sorted descending"
+    # reported values are the scores of the reported rows
+    assert (torch.gather(ref_scores, 1, idx) - vals).abs().max().item() <= tol
+    for q in range(vals.shape[0]):
+        got, want = set(idx[q].tolist()), set(ref_i[q].tolist())
+        if got == want:
+            continue
+        kth = ref_v[q, -1].item()
+        for r in got ^ want:  # may differ only among rows tied with the k-th score
+            assert abs(ref_scores[q, r].item() - kth) <= tol, (q, r)
+        assert len(got) == k
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(300, 256, 7, 10), (1000, 512, 40, 100), (5000, 1024, 130, 100)])
+def test_scan_cosine_topk(device, dtype, shape):
+    from bergson_amd import ops
+
+    n, D, Q, k = shape
+    store, queries = make_store(n, D, Q, dtype, seed=n)
+    qn = unit_queries(queries, dtype)
+    # the oracle scores what the kernel is given: store rows in `dtype`, unit queries rounded to `dtype`
+    qd = qn.to(dtype)
+    ref = oscan.scorer_score({"m": store}, {"m": qd}, ["m"], dtype=torch.float32, unit_normalize=True).T  # [Q, n]
+    res = ops.scan(store.to(device), qd.to(device), unit_norm=True, k=k, want_row_max=True, want_scores=True,
+                   want_sumsq=True, chunk_rows=1024)
+    torch.cuda.synchronize()
+    scores = res.scores.cpu().T
+    assert (scores - ref).abs().max().item() <= COS_TOL
+    assert torch.allclose(res.sumsq.cpu(), store.float().pow(2).sum(1), rtol=1e-4)
+    assert (res.row_max.cpu() - ref.max(0).values).abs().max().item() <= COS_TOL
+    check_topk(res.topk_values.cpu(), res.topk_indices.cpu(), ref, k)
+
+
+def test_scan_matches_attributor_search(device):
+    from bergson_amd import ops
+
+    n, Q, k = 2000, 16, 50
+    sizes = {"a": 256, "b": 256, "c": 512}
+    gen = torch.Generator().manual_seed(7)
+    index = {m: torch.randn(n, d, generator=gen).to(torch.float16) for m, d in sizes.items()}
+    queries = {m: torch.randn(Q, d, generator=gen) for m, d in sizes.items()}
+    mods = list(sizes)
+    ref_v, ref_i = oscan.attributor_search(index, queries, mods, k, unit_norm=True)
+    store = torch.cat([index[m] for m in mods], 1)
+    qcat = torch.cat([queries[m] for m in mods], 1)
+    qn = qcat / (qcat.norm(dim=1, keepdim=True) + torch.finfo(torch.float32).eps)
+    res = ops.scan(store.to(device), qn.to(torch.float16).to(device), unit_norm=True, k=k)
+    torch.cuda.synchronize()
+    assert (res.topk_values.cpu() - ref_v).abs().max().item() <= COS_TOL
+    same = (res.topk_indices.cpu() == ref_i).float().mean().item()
+    assert same > 0.98  # neighbours closer than the tolerance may swap places
+
+
+def test_scan_self_match_and_zero_rows(device):
+    from bergson_amd import ops
+
+    n, D = 700, 384
+    store, _ = make_store(n, D, 1, torch.float16, seed=3)
+    store[5] = 0  # documents with fewer than 2 tokens are stored as zero rows
+    picks = [0, 5, 123, 699]
+    q = store[picks].float()
+    qn = q / (q.norm(dim=1, keepdim=True) + torch.finfo(torch.float32).eps)
+    res = ops.scan(store.to(device), qn.to(torch.float16).to(device), unit_norm=True, k=3, want_scores=True)
+    torch.cuda.synchronize()
+    idx, vals, scores = res.topk_indices.cpu(), res.topk_values.cpu(), res.scores.cpu()
+    assert torch.isfinite(scores).all()
+    assert (scores[5] == 0).all()  # zero row scores 0 against everything
+    for j, r in enumerate(picks):
+        if r == 5:
+            continue
+        assert idx[j, 0].item() == r and vals[j, 0].item() > 0.99
+        assert vals[j, 1].item() < 0.5
+
+
+def test_scan_raw_inner_product_and_reverse(device):
+    from bergson_amd import ops
+
+    store, queries = make_store(900, 256, 5, torch.bfloat16, seed=11, outliers=False)
+    ref = queries.float() @ store.float().T
+    res = ops.scan(store.to(device), queries.to(device), unit_norm=False, k=20, want_scores=True)
+    neg = ops.scan(store.to(device), (-queries).to(device), unit_norm=False, k=20)
+    torch.cuda.synchronize()
+    assert torch.allclose(res.scores.cpu().T, ref, rtol=1e-4, atol=1e-3)
+    rv, ri = torch.topk(ref, 20, dim=1)
+    assert torch.equal(res.topk_indices.cpu(), ri)
+    lv, li = torch.topk(ref, 20, dim=1, largest=False)
+    assert torch.equal(neg.topk_indices.cpu(), li)
+    assert torch.allclose(-neg.topk_values.cpu(), lv, rtol=1e-4, atol=1e-3)
+
+
+def test_scan_chunking_invariance(device):
+    # the chunk size of the internal passes changes neither scores nor the selected rows
+    from bergson_amd import ops
+
+    store, queries = make_store(6000, 512, 33, torch.float16, seed=5)
+    qd = unit_queries(queries, torch.float16).to(torch.float16)
+    a = ops.scan(store.to(device), qd.to(device), unit_norm=True, k=64, chunk_rows=512)
+    b = ops.scan(store.to(device), qd.to(device), unit_norm=True, k=64, chunk_rows=0)
+    torch.cuda.synchronize()
+    assert torch.equal(a.topk_indices.cpu(), b.topk_indices.cpu())
+    assert torch.equal(a.topk_values.cpu(), b.topk_values.cpu())
+
+
+def test_scan_ties_pick_lowest_rows(device):
+    from bergson_amd import ops
+
+    row = torch.randn(128)
+    store = row.repeat(50, 1).to(torch.float16)
+    res = ops.scan(store.to(device), row[None].to(torch.float16).to(device), unit_norm=True, k=10)
+    torch.cuda.synchronize()
+    assert res.topk_indices.cpu()[0].tolist() == list(range(10))
+
+
+def test_scan_k_equals_rows_and_unaligned_dim(device):
+    from bergson_amd import ops
+
+    store, queries = make_store(37, 100, 3, torch.float32, seed=13, outliers=False)
+    store = store[:, :99].contiguous()
+    queries = queries[:, :99].contiguous()
+    ref = queries @ store.T
+    res = ops.scan(store.to(device), queries.to(device), unit_norm=False, k=37)
+    torch.cuda.synchronize()
+    rv, ri = torch.topk(ref, 37, dim=1)
+    assert torch.equal(res.topk_indices.cpu(), ri)
+    assert torch.allclose(res.topk_values.cpu(), rv, rtol=1e-5, atol=1e-5)
