@@ -1,0 +1,137 @@
+"""Query an existing gradient store (bergson/query/attributor.py).
+
+The store stays in HBM in its on-disk dtype (e.g. 24.6 GB for 10^6 fp16 rows of
+12288); `search` streams it once through `bgx_scan`, which folds the row
+normalisation (attributor.py:137-167), the GEMM against the queries and the
+per-query top-k (attributor.py:229-235) into one pass.
+"""
+from __future__ import annotations
+
+import math
+from contextlib import contextmanager
+from pathlib import Path
+from typing import Generator
+
+import numpy as np
+import torch
+import torch.nn as nn
+from torch import Tensor
+
+from . import ops
+from .data import column_offsets, load_gradients, load_info, store_base_dtype
+from .gradient_collectors import TraceCollector
+from .gradients import GradientProcessor
+from .utils import numpy_to_tensor, torch_dtype_from_name
+
+
+class TraceResult:
+    """Holds the top-k of a `trace()` block once it has exited (attributor.py:22-44)."""
+
+    def __init__(self):
+        self._indices: Tensor | None = None
+        self._scores: Tensor | None = None
+
+    @property
+    def indices(self) -> Tensor:
+        if self._indices is None:
+            raise ValueError("No indices available. Exit the context manager first.")
+        return self._indices
+
+    @property
+    def scores(self) -> Tensor:
+        if self._scores is None:
+            raise ValueError("No scores available. Exit the context manager first.")
+        return self._scores
+
+
+def upload_store(mmap: np.ndarray, base_dtype: str, device: torch.device, chunk_bytes: int = 1 << 30) -> Tensor:
+    """Copies a mapped store to the device in row chunks, keeping its dtype and bits."""
+    n, D = mmap.shape
+    out = torch.empty((n, D), dtype=torch_dtype_from_name(base_dtype), device=device)
+    step = max(1, chunk_bytes // max(1, D * mmap.dtype.itemsize))
+    for lo in range(0, n, step):
+        hi = min(n, lo + step)
+        out[lo:hi].copy_(numpy_to_tensor(mmap[lo:hi], base_dtype), non_blocking=False)
+    return out
+
+
+class Attributor:
+    """`Attributor(index_path, device, dtype, unit_norm).search(queries, k)` (attributor.py:47-235)."""
+
+    def __init__(self, index_path: str | Path, device: str = "cuda", dtype: torch.dtype = torch.float32,
+                 unit_norm: bool = False, faiss_cfg=None, inversion_cfg=None, hessian_path: str | Path | None = None,
+                 ev_correction: bool = False):
+        if faiss_cfg is not None:
+            raise NotImplementedError("FAISS search is outside this package; the exact scan replaces the Flat index")
+        if hessian_path is not None:
+            raise NotImplementedError("preconditioned search (hessian_path) is outside this package")
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise RuntimeError("bergson_amd has no CPU path: Attributor needs a GPU device")
+        self.dtype = dtype
+        self.unit_norm = unit_norm
+        self.precondition = "none"
+        self.preconditioner = None
+        self.faiss_index = None
+        index_path = Path(index_path)
+        self.processor = GradientProcessor.load(index_path, map_location=device)
+        info = load_info(index_path)
+        self.grad_sizes: dict[str, int] = info["grad_sizes"]
+        self.ordered_modules = list(self.grad_sizes)
+        self._columns = column_offsets(self.grad_sizes)
+        base = store_base_dtype(info)
+        if base == "float64":
+            raise TypeError("float64 stores are not supported by the scan kernels")
+        self.store = upload_store(load_gradients(index_path), base, self.device)
+        self.N = self.store.shape[0]
+
+    @property
+    def grads(self) -> dict[str, Tensor]:
+        """Per-module column views of the device store (raw rows; normalisation happens inside the scan)."""
+        return {name: self.store[:, lo:hi] for name, (lo, hi) in self._columns.items()}
+
+    def search(self, queries: dict[str, Tensor], k: int | None, modules: set[str] | None = None,
+               reverse: bool = False):
+        """Top-k rows per query by inner product (cosine when unit_norm); returns (values, indices) [..., k]."""
+        q = torch.cat([queries[name].to(self.device, torch.float32) for name in self.ordered_modules], dim=1)
+        if self.unit_norm:
+            norm = q.norm(dim=1, keepdim=True)
+            q = q / (norm + torch.finfo(norm.dtype).eps)
+        if modules:
+            for name, (lo, hi) in self._columns.items():
+                if name not in modules:
+                    q[:, lo:hi] = 0
+        if reverse:
+            q = -q
+        k = min(k or self.N, self.N)
+        # a power-of-two rescale keeps small query entries clear of the fp16 subnormal range
+        qmax = float(q.abs().max().item())
+        shift = 0 if qmax == 0 or not math.isfinite(qmax) else -math.frexp(qmax)[1]
+        qd = (q * (2.0 ** shift)).to(self.store.dtype)
+        res = ops.scan(self.store, qd, unit_norm=self.unit_norm, k=k, query_scale=2.0 ** (-shift))
+        values = res.topk_values
+        if reverse:
+            values = -values
+        return torch.return_types.topk((values.to(self.dtype), res.topk_indices))
+
+    @contextmanager
+    def trace(self, module: nn.Module, k: int | None, *, modules: set[str] | None = None, reverse: bool = False
+              ) -> Generator[TraceResult, None, None]:
+        """Collects the gradients of whatever is back-propagated through `module` inside the block and
+        searches the store with them (attributor.py:237-282)."""
+        result = TraceResult()
+        collector = TraceCollector(model=module, processor=self.processor, target_modules=modules,
+                                   device=self.device, dtype=self.dtype)
+        mod_grads = collector.mod_grads
+        with collector:
+            yield result
+        if not mod_grads:
+            raise ValueError("No grads collected. Did you forget to call backward?")
+        queries = {name: torch.cat(mod_grads[name], dim=1) for name in self.ordered_modules if name in mod_grads}
+        if any(q.isnan().any() for q in queries.values()):
+            raise ValueError("NaN found in queries.")
+        for name in self.ordered_modules:  # modules that were not traced contribute nothing
+            if name not in queries:
+                rows = next(iter(queries.values())).shape[0]
+                queries[name] = torch.zeros((rows, self.grad_sizes[name]), device=self.device, dtype=self.dtype)
+        result._scores, result._indices = self.search(queries, k, modules, reverse)

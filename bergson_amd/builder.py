@@ -1,0 +1,195 @@
+"""Gradient-store writer.
+
+Same role and call signature as bergson/builder.py (`Builder.__init__`
+:61-139, `__call__` :141-165, scatter :167-188, `teardown` :196-232) and the
+same on-disk result.  The difference is where rows live while the store is
+being built: when the whole store fits the HBM budget it is kept in a device
+buffer -- the collection kernels write finished store-dtype rows straight
+into it -- and it is copied to the memory-mapped file once, in `flush()`.
+Otherwise each batch goes through one device buffer and one D2H copy.
+"""
+from __future__ import annotations
+
+from pathlib import Path
+
+import numpy as np
+import torch
+import torch.distributed as dist
+from torch import Tensor
+
+from . import ops
+from .config import PreprocessConfig
+from .data import compute_num_token_grads, create_index, create_token_index
+from .utils import dtype_name, storage_np_dtype, tensor_to_numpy
+
+
+class RowBlock(dict):
+    """`mod_grads` whose per-module tensors are column views of one [rows, D] device buffer.
+
+    `rows` is that buffer; `committed` says the rows already sit in the builder's device store (written
+    there directly by the collection kernel), so `Builder.__call__` has nothing left to move.
+    """
+
+    rows: Tensor | None = None
+    committed: bool = False
+
+
+class Builder:
+    """Writes per-sequence or ragged per-token gradient rows to disk (`path`) or memory (`path=None`)."""
+
+    grad_buffer: np.ndarray
+
+    def __init__(self, data, grad_sizes: dict[str, int], dtype: torch.dtype, preprocess_cfg: PreprocessConfig, *,
+                 attribute_tokens: bool = False, path: Path | None = None, device: torch.device | None = None,
+                 device_store_bytes: int | None = None):
+        self.grad_sizes = grad_sizes
+        self.num_items = len(data)
+        self.preprocess_cfg = preprocess_cfg
+        self.dtype = dtype
+        self.attribute_tokens = attribute_tokens
+        self.total_grad_dim = sum(grad_sizes.values())
+        if preprocess_cfg.hessian_path is not None:
+            raise NotImplementedError("preconditioning (preprocess_cfg.hessian_path) is outside this package")
+        if device is None:
+            device = torch.device("cuda", torch.cuda.current_device()) if torch.cuda.is_available() else None
+        self.device = device
+
+        if preprocess_cfg.aggregation != "none":
+            store_name = "float32"
+            num_grads = 1
+            self.in_memory_grad_buffer: Tensor | None = torch.zeros((1, self.total_grad_dim), dtype=torch.float32,
+                                                                    device=device)
+        else:
+            store_name = dtype_name(dtype)
+            num_grads = self.num_items
+            self.in_memory_grad_buffer = None
+        self.base_dtype = store_name
+        np_dtype = storage_np_dtype(store_name)
+
+        if attribute_tokens:
+            self.num_token_grads = compute_num_token_grads(data)
+            if path is not None:
+                self.grad_buffer, self.offsets = create_token_index(path, self.num_token_grads, grad_sizes, store_name)
+            else:
+                self.offsets = np.zeros(len(self.num_token_grads) + 1, dtype=np.int64)
+                np.cumsum(self.num_token_grads, out=self.offsets[1:])
+                self.grad_buffer = np.zeros((int(self.offsets[-1]), self.total_grad_dim), dtype=np_dtype)
+        else:
+            self.num_token_grads = None
+            self.offsets = None
+            if path is not None:
+                self.grad_buffer = create_index(path, num_grads=num_grads, grad_sizes=grad_sizes, dtype=store_name)
+            else:
+                self.grad_buffer = np.zeros((num_grads, self.total_grad_dim), dtype=np_dtype)
+
+        # ---- device-resident store ---------------------------------------------------------
+        self.device_rows: Tensor | None = None
+        self._offsets_dev: Tensor | None = None
+        self._dirty = False
+        if self.in_memory_grad_buffer is None and device is not None and device.type == "cuda":
+            nbytes = int(self.grad_buffer.shape[0]) * self.total_grad_dim * np_dtype.itemsize
+            if device_store_bytes is None:
+                free, _ = torch.cuda.mem_get_info(device)
+                device_store_bytes = free // 4
+            if 0 < nbytes <= device_store_bytes:
+                self.device_rows = torch.zeros((self.grad_buffer.shape[0], self.total_grad_dim), dtype=dtype,
+                                               device=device)
+            if self.offsets is not None:
+                self._offsets_dev = torch.from_numpy(self.offsets).to(device)
+
+    # ---- direct-write protocol used by the collectors ----------------------------------------
+    @property
+    def direct(self) -> bool:
+        """True when collection kernels may write finished rows straight into the device store."""
+        return self.device_rows is not None and not self.preprocess_cfg.unit_normalize
+
+    def token_row_offsets(self, indices: list[int]) -> Tensor:
+        """int64 [len(indices)] first store row of each document of a per-token store."""
+        assert self._offsets_dev is not None
+        idx = torch.as_tensor(indices, dtype=torch.int64).to(self._offsets_dev.device, non_blocking=True)
+        return self._offsets_dev[idx].contiguous()
+
+    def mark_written(self) -> None:
+        self._dirty = True
+
+    # ---- __call__ -------------------------------------------------------------------------------
+    def __call__(self, indices: list[int], mod_grads: dict[str, Tensor]) -> None:
+        """Concatenate the modules of a batch, optionally unit-normalise, and place the rows."""
+        if isinstance(mod_grads, RowBlock) and mod_grads.committed:
+            self._dirty = True
+            return
+        if isinstance(mod_grads, RowBlock) and mod_grads.rows is not None:
+            grads = mod_grads.rows
+        else:
+            grads = torch.cat([mod_grads[m] for m in self.grad_sizes.keys()], dim=-1)
+        if self.preprocess_cfg.unit_normalize:
+            if not grads.is_cuda:
+                raise RuntimeError("unit_normalize runs on the GPU: pass GPU tensors (bergson_amd has no CPU path)")
+            if grads.dtype not in ops.DTYPE_CODE:
+                grads = grads.to(torch.float32)
+            ops.unit_normalize_rows_(grads)
+
+        if self.preprocess_cfg.aggregation != "none":
+            assert self.in_memory_grad_buffer is not None
+            self.in_memory_grad_buffer[0] += grads.sum(dim=0).to(dtype=torch.float32,
+                                                                 device=self.in_memory_grad_buffer.device)
+            return
+        self._scatter(indices, grads)
+
+    def _scatter(self, indices: list[int], grads: Tensor) -> None:
+        if self.device_rows is not None and grads.is_cuda:
+            idx = torch.as_tensor(indices, dtype=torch.int64).to(grads.device, non_blocking=True)
+            if self.attribute_tokens:
+                assert self._offsets_dev is not None
+                starts = self._offsets_dev[idx]
+                counts = self._offsets_dev[idx + 1] - starts
+                rows = torch.repeat_interleave(starts - (torch.cumsum(counts, 0) - counts), counts) + torch.arange(
+                    grads.shape[0], device=grads.device)
+                self.device_rows.index_copy_(0, rows, grads.to(self.device_rows.dtype))
+            else:
+                self.device_rows.index_copy_(0, idx, grads.to(self.device_rows.dtype))
+            self._dirty = True
+            return
+        host = tensor_to_numpy(grads.to(self.dtype).cpu())
+        if self.attribute_tokens:
+            assert self.num_token_grads is not None and self.offsets is not None
+            row = 0
+            for idx, sl in zip(indices, self.num_token_grads[indices]):
+                self.grad_buffer[int(self.offsets[idx]):int(self.offsets[idx + 1])] = host[row:row + sl]
+                row += sl
+        else:
+            self.grad_buffer[indices] = host
+
+    # ---- lifecycle -------------------------------------------------------------------------------
+    def flush(self) -> None:
+        """Copy the device store to the host buffer (once) and flush the memory map."""
+        if self.device_rows is not None and self._dirty:
+            n = self.device_rows.shape[0]
+            row_bytes = max(1, self.total_grad_dim * self.device_rows.element_size())
+            step = max(1, (1 << 30) // row_bytes)
+            for lo in range(0, n, step):
+                hi = min(n, lo + step)
+                self.grad_buffer[lo:hi] = tensor_to_numpy(self.device_rows[lo:hi].cpu())
+            self._dirty = False
+        if isinstance(self.grad_buffer, np.memmap):
+            self.grad_buffer.flush()
+
+    def teardown(self) -> None:
+        self.flush()
+        if self.preprocess_cfg.aggregation == "none":
+            if dist.is_initialized() and not isinstance(self.grad_buffer, np.memmap):
+                if self.grad_buffer.dtype == np.uint16:
+                    raise NotImplementedError("gathering an in-memory bfloat16 store across ranks")
+                dist.all_reduce(torch.from_numpy(self.grad_buffer), op=dist.ReduceOp.SUM)
+            return
+        assert self.in_memory_grad_buffer is not None
+        if dist.is_initialized():
+            dist.reduce(self.in_memory_grad_buffer, dst=0, op=dist.ReduceOp.SUM)
+        if self.preprocess_cfg.aggregation == "mean":
+            self.in_memory_grad_buffer /= self.num_items
+        if self.preprocess_cfg.normalize_aggregated_grad:
+            ops.unit_normalize_rows_(self.in_memory_grad_buffer)
+        self.in_memory_grad_buffer = self.in_memory_grad_buffer.cpu()
+        rank = dist.get_rank() if dist.is_initialized() else 0
+        if rank == 0:
+            self.grad_buffer[:] = self.in_memory_grad_buffer.numpy().astype(self.grad_buffer.dtype)

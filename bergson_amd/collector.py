@@ -1,0 +1,459 @@
+"""Hook layer of gradient collection, backed by the fused HIP kernels.
+
+Mirrors the interface of bergson/collector/collector.py: `HookCollectorBase`
+(:44-768: target discovery, per-head splitting, hook registration, the
+`with collector.with_batch(mask):` protocol, `shapes()`), `CollectorComputer`
+(:771-923), `fwd_bwd_factory` (:926-985) and `create_projection_matrix`
+(:1029-1063).
+
+What differs from the reference is where the arithmetic happens.  The
+reference's forward hook scales and projects the activations and its backward
+hook scales, projects and reduces the output gradients, each as a handful of
+PyTorch ops per module.  Here the forward hook only keeps a reference to the
+module input; the backward hook hands (a, g) to one fused kernel launch --
+either immediately (`_compute_gradient`, one module per launch, returns the
+tensor the reference would) or deferred (`defer_module` + `launch_deferred`,
+all modules of the batch in one launch writing straight into a row buffer).
+"""
+from __future__ import annotations
+
+import functools
+import hashlib
+import math
+import os
+from abc import ABC, abstractmethod
+from contextlib import ContextDecorator, nullcontext
+from dataclasses import astuple, dataclass, field
+from fnmatch import fnmatchcase
+from typing import Callable, Literal, Mapping, Optional
+
+import numpy as np
+import torch
+import torch.distributed as dist
+import torch.nn as nn
+import torch.nn.functional as F
+from torch import Tensor
+from torch.utils.hooks import RemovableHandle
+
+from . import ops
+from .config import AttentionConfig, IndexConfig
+from .data import compute_num_token_grads, pad_and_tensor
+from .gradients import AdafactorNormalizer, AdamNormalizer, GradientProcessor, LayerAdapter
+
+
+def create_projection_matrix(identifier: str, m: int, n: int, dtype: torch.dtype, device: torch.device | str,
+                             projection_type: Literal["normal", "rademacher"] = "normal",
+                             projection_scale: Literal["jl", "row_norm"] = "jl") -> Tensor:
+    """Deterministic [m, n] projection matrix named by `identifier` (collector.py:1029-1063).
+
+    The seed is md5(identifier) mod 2**63-1.  `normal` draws `torch.randn` in `dtype`; the draw always
+    uses the CPU generator and is uploaded afterwards, so a matrix depends on (identifier, shape, dtype)
+    only and equals what the reference produces with device='cpu' on any machine.  `rademacher` uses
+    numpy's PCG64 bit stream exactly as the reference does.
+    """
+    digest = hashlib.md5(bytes(identifier, "utf-8")).digest()
+    seed = int.from_bytes(digest, byteorder="big") % (2**63 - 1)
+    if projection_type == "normal":
+        prng = torch.Generator("cpu").manual_seed(seed)
+        A = torch.randn(m, n, dtype=dtype, generator=prng)
+    elif projection_type == "rademacher":
+        random_bytes = np.random.Generator(np.random.PCG64(seed)).bytes((m * n + 7) // 8)
+        bits = np.unpackbits(np.frombuffer(random_bytes, dtype=np.uint8))[: m * n].reshape((m, n))
+        A = torch.from_numpy(bits).to(dtype=dtype)
+        A = A.add_(-0.5).mul_(2)
+    else:
+        raise ValueError(f"Unknown projection type: {projection_type}")
+    if projection_scale == "row_norm":
+        A /= A.norm(dim=1, keepdim=True)
+    else:
+        A /= math.sqrt(m)  # variance 1/m
+    return A.to(device)
+
+
+@dataclass
+class HookCollectorBase(ContextDecorator, ABC):
+    """Attaches forward and backward hooks to the supported layers of `model`.
+
+    Activations are [N, S, I], activation gradients [N, S, O].  Subclasses implement `setup`, `teardown`,
+    `backward_hook` and `process_batch` (collector.py:493-516, :745-768).
+    """
+
+    model: nn.Module
+    filter_modules: str | None = None
+    target_modules: set[str] | None = None
+    processor: GradientProcessor = field(default_factory=GradientProcessor)
+    attention_cfgs: dict[str, AttentionConfig] = field(default_factory=dict)
+    attribute_tokens: bool = False
+    lo: float = float("-inf")
+    hi: float = float("inf")
+    mod_grads: dict = field(default_factory=dict)
+    save_dtype: torch.dtype = torch.float32
+
+    def __post_init__(self):
+        self.rank = dist.get_rank() if dist.is_initialized() else 0
+        self.world_size = dist.get_world_size() if dist.is_initialized() else 1
+        self._fwd_hooks: list[RemovableHandle] = []
+        self._bwd_hooks: list[RemovableHandle] = []
+        self._current_collection_mask: Tensor | None = None
+        self._deferred: list[ops.ModuleInput] = []
+        self._scale_cache: dict[str, tuple[Tensor | None, Tensor | None]] = {}
+        self.target_info = self.discover_targets(self.model, self.target_modules, self.processor.include_bias,
+                                                 self.filter_modules)
+        if unknown := set(self.attention_cfgs) - set(self.target_info):
+            raise ValueError(f"attention_cfgs contains module names not found in the model: {unknown}. "
+                             f"Available modules: {set(self.target_info)}")
+        self.setup()
+
+    # ---- discovery and naming (collector.py:133-241) -----------------------------------
+    @staticmethod
+    def discover_targets(model: nn.Module, target_modules: set[str] | None = None, include_bias: bool = False,
+                         filter_modules: str | None = None) -> dict[str, tuple[torch.device, torch.Size, bool]]:
+        """name -> (device, weight shape [O, I], collect_bias) for every supported layer."""
+        target_info = {}
+        for name, layer in model.named_modules():
+            if not isinstance(layer, LayerAdapter.supported_modules):
+                continue
+            if target_modules is not None and name not in target_modules:
+                continue
+            if filter_modules and any(fnmatchcase(name, pat.strip()) for pat in filter_modules.split(",")):
+                continue
+            collect_bias = getattr(layer, "bias", None) is not None and include_bias
+            o = getattr(layer, LayerAdapter.out_attr(layer))
+            i = getattr(layer, LayerAdapter.in_attr(layer))
+            target_info[name] = (layer.weight.device, torch.Size([o, i]), collect_bias)
+        return target_info
+
+    @staticmethod
+    def get_head_name(name: str, head_idx: int) -> str:
+        return f"{name}.head_{head_idx}"
+
+    @staticmethod
+    def split_head_name(name: str) -> tuple[str, int] | None:
+        base, sep, suffix = name.rpartition(".head_")
+        if not sep or not suffix.isdigit():
+            return None
+        return base, int(suffix)
+
+    @staticmethod
+    def split_attention_heads(fn):
+        """Decorator: calls `fn(self, module, g_head)` once per head for modules in `attention_cfgs`
+        (collector.py:191-233).  The head's slice of g is a strided view; nothing is copied."""
+
+        @functools.wraps(fn)
+        def wrapper(self, module, g):
+            name = module._name
+            if name not in self.attention_cfgs:
+                return fn(self, module, g)
+            num_heads, head_size, head_dim = astuple(self.attention_cfgs[name])
+            orig_out = getattr(module, LayerAdapter.out_attr(module))
+            assert num_heads * head_size == orig_out, (
+                f"{name}: num_heads * head_size = {num_heads * head_size} does not cover the module's "
+                f"{orig_out} output features")
+            setattr(module, LayerAdapter.out_attr(module), head_size)
+            try:
+                for h in range(num_heads):
+                    module._name = self.get_head_name(name, h)
+                    try:
+                        head_g = torch.narrow(g, head_dim, h * head_size, head_size)
+                    except Exception:
+                        print(f"Error processing gradient of shape {g.shape} for head {h} in module {name}. "
+                              f"Provided head config may be incorrect. Head config: head dim {head_dim}, "
+                              f"head size {head_size}, num heads {num_heads}.")
+                        raise
+                    fn(self, module, head_g)
+            finally:
+                module._name = name
+                setattr(module, LayerAdapter.out_attr(module), orig_out)
+
+        return wrapper
+
+    def normalizer_for(self, name: str):
+        """Normalizer of module `name`; a split head takes its rows of the parent's (collector.py:243-279)."""
+        normalizer = self.processor.normalizers.get(name)
+        if normalizer is not None:
+            return normalizer
+        split = self.split_head_name(name)
+        if split is None:
+            return None
+        base, head_idx = split
+        normalizer = self.processor.normalizers.get(base)
+        if normalizer is None or base not in self.attention_cfgs:
+            return normalizer
+        head_size = self.attention_cfgs[base].head_size
+        lo, hi = head_idx * head_size, (head_idx + 1) * head_size
+        if isinstance(normalizer, AdamNormalizer):
+            bias = normalizer.bias_avg_sq
+            return AdamNormalizer(normalizer.weight_avg_sq[lo:hi], bias[lo:hi] if bias is not None else None)
+        if isinstance(normalizer, AdafactorNormalizer):
+            bias = normalizer.bias_avg_sq
+            return AdafactorNormalizer(normalizer.row[lo:hi], normalizer.col,
+                                       bias[lo:hi] if bias is not None else None)
+        return normalizer
+
+    @property
+    def per_module_projection_dim(self) -> int | None:
+        if self.processor.projection_target == "global":
+            return None
+        return self.processor.projection_dim or None
+
+    def shapes(self) -> Mapping[str, torch.Size]:
+        """Shapes of the collected gradients; their order is the column order of the store
+        (collector.py:288-334)."""
+        if self.processor.projection_target == "global":
+            assert self.processor.projection_dim is not None
+            return {"gradients": torch.Size((self.processor.projection_dim,))}
+        p_dim = self.per_module_projection_dim
+        proj_shape = torch.Size((p_dim, p_dim)) if p_dim is not None else None
+        shapes = {}
+        for name, (_, target_shape, collect_bias) in self.target_info.items():
+            if name in self.attention_cfgs:
+                cfg = self.attention_cfgs[name]
+                if proj_shape:
+                    head_shape = proj_shape
+                else:
+                    attention_shape = list(target_shape)
+                    attention_shape[cfg.head_dim - 2] = cfg.head_size
+                    if collect_bias:
+                        attention_shape[-1] += 1
+                    head_shape = torch.Size(attention_shape)
+                shapes.update({self.get_head_name(name, h): head_shape for h in range(cfg.num_heads)})
+            elif proj_shape:
+                shapes[name] = proj_shape
+            else:
+                grad_shape = list(target_shape)
+                if collect_bias:
+                    grad_shape[-1] += 1
+                shapes[name] = torch.Size(grad_shape)
+        return shapes
+
+    def projection(self, name: str, m: int, n: int, role: Literal["left", "right", "single"],
+                   device: torch.device, dtype: torch.dtype) -> Tensor:
+        """The cached `role` projection matrix [m, n] of parameter `name` (collector.py:336-362)."""
+        key = (name, role, device)
+        cache = self.processor._projection_matrices
+        if key in cache:
+            return cache[key]
+        A = create_projection_matrix(f"{name}/{role}", m, n, dtype, device, self.processor.projection_type,
+                                     self.processor.projection_scale)
+        cache[key] = A
+        return A
+
+    def num_rows(self, data) -> int:
+        if self.attribute_tokens:
+            return int(compute_num_token_grads(data).sum())
+        return len(data)
+
+    # ---- batch protocol (collector.py:413-491) -------------------------------------------
+    def with_batch(self, collection_mask: Tensor | None = None) -> "HookCollectorBase":
+        """Sets the [N, S] mask of collected positions (every real position but each sequence's last)."""
+        self._current_collection_mask = collection_mask
+        return self
+
+    def __enter__(self):
+        for name in self.target_info:
+            layer = self.model.get_submodule(name)
+            layer._name = name  # type: ignore[attr-defined]
+            layer._collect_bias = self.target_info[name][2]  # type: ignore[attr-defined]
+            self._fwd_hooks.append(layer.register_forward_hook(self._process_input))
+            self._bwd_hooks.append(layer.register_full_backward_hook(self._process_grad))
+        return self
+
+    def _process_input(self, module: nn.Module, inp: tuple, _):
+        x = inp[0].detach()
+        assert x.ndim == 3, f"Expected input of shape [N, S, I], got {x.shape}"
+        self.forward_hook(module, x)
+
+    def _process_grad(self, module: nn.Module, _, grad_out):
+        assert isinstance(module, LayerAdapter.supported_modules), (
+            f"Expected a module of type {LayerAdapter.supported_modules}, got {type(module)}")
+        g = grad_out[0].detach()
+        self.backward_hook(module, g)
+        if hasattr(module, "_inputs"):
+            del module._inputs
+
+    def __exit__(self, exc_type, exc, tb):
+        for layer in self.model.modules():
+            if hasattr(layer, "_inputs"):
+                del layer._inputs
+            if hasattr(layer, "_name"):
+                del layer._name
+        for h in self._fwd_hooks:
+            h.remove()
+        for h in self._bwd_hooks:
+            h.remove()
+        self._fwd_hooks.clear()
+        self._bwd_hooks.clear()
+        if exc_type is not None:
+            self._deferred.clear()  # a failed batch leaves nothing queued; otherwise process_batch launches
+        return False
+
+    # ---- the hook pair -----------------------------------------------------------------------
+    def forward_hook(self, module: nn.Module, a: Tensor) -> None:
+        """Keeps the module input for the backward hook (collector.py:518-543).
+
+        The reference scales and projects `a` here; the fused kernel does both when it also has g, so the
+        raw input is kept alive until then.
+        """
+        module._inputs = a
+
+    def _batch_lengths(self, device: torch.device) -> Tensor | None:
+        """int32 [N] document lengths implied by the collection mask (mask[n, s] = s + 1 < len[n])."""
+        mask = self._current_collection_mask
+        if mask is None:
+            return None
+        cached = getattr(self, "_lengths_cache", None)
+        if cached is not None and cached[0] is mask:
+            return cached[1]
+        lengths = (mask.sum(dim=1) + 1).to(device=device, dtype=torch.int32)
+        self._lengths_cache = (mask, lengths)
+        return lengths
+
+    def _scales(self, name: str, normalizer: AdafactorNormalizer, dtype: torch.dtype, device: torch.device):
+        key = f"{name}|{dtype}|{device}"
+        if key not in self._scale_cache:
+            self._scale_cache[key] = ops.adafactor_scales(normalizer.row.to(device), normalizer.col.to(device), dtype)
+        return self._scale_cache[key]
+
+    def module_input(self, module: nn.Module, g: Tensor, out_col: int = 0) -> ops.ModuleInput:
+        """Kernel operands of `module` for the current batch: its kept input, g, the two projection matrices
+        and, with an Adafactor normalizer, the two factor vectors."""
+        a = module._inputs
+        assert isinstance(a, Tensor), "Activation cache missing for module"
+        name: str = module._name  # type: ignore[assignment]
+        p = self.per_module_projection_dim
+        i = getattr(module, LayerAdapter.in_attr(module))
+        o = getattr(module, LayerAdapter.out_attr(module))
+        normalizer = self.normalizer_for(name)
+        if p is None:
+            raise NotImplementedError(
+                "bergson_amd collects projected gradients only: set processor.projection_dim "
+                "(projection_target='per_module'); unprojected [O, I] gradients have no HIP kernel here")
+        if module._collect_bias:
+            raise NotImplementedError(f"{name}: include_bias=True has no HIP kernel in this build")
+        if isinstance(normalizer, AdamNormalizer):
+            raise NotImplementedError(f"{name}: AdamNormalizer has no HIP kernel in this build; "
+                                      "convert with .to_adafactor() or drop the normalizer")
+        if not a.is_cuda or not g.is_cuda:
+            raise RuntimeError("bergson_amd has no CPU path: the model must run on the GPU")
+        # an attention head shares the parent's input and right projection (collector.py:527, :540)
+        parent = self.split_head_name(name)
+        right_name = parent[0] if parent is not None and parent[0] in self.attention_cfgs else name
+        r_in = self.projection(right_name, p, i, "right", a.device, a.dtype)
+        r_out = self.projection(name, p, o, "left", g.device, g.dtype)
+        row_scale = col_scale = None
+        if isinstance(normalizer, AdafactorNormalizer):
+            row_scale, col_scale = self._scales(name, normalizer, g.dtype, g.device)
+        return ops.ModuleInput(a=a, g=g, r_in=r_in, r_out=r_out, out_col=out_col, col_scale=col_scale,
+                               row_scale=row_scale)
+
+    def _compute_gradient(self, module: nn.Module, g: Tensor) -> Tensor:
+        """Per-sample [N, p*p] (or per-token [n_valid, p*p]) projected gradient of one module, clamped to
+        [lo, hi], in the model dtype (collector.py:592-743) -- one fused launch."""
+        mi = self.module_input(module, g, 0)
+        p = self.per_module_projection_dim
+        assert p is not None
+        N, S = g.shape[:2]
+        if self.attribute_tokens:
+            lengths = self._batch_lengths(g.device)
+            assert lengths is not None, "attribute_tokens needs a collection mask (with_batch)"
+            counts = (lengths.to(torch.int64) - 1).clamp_min_(0)
+            offsets = torch.cumsum(counts, 0) - counts
+            total = int(counts.sum().item())
+            out = torch.empty((total, p * p), dtype=g.dtype, device=g.device)
+            if total:
+                ops.collect_tok([mi], p, out, lengths=lengths, row_offsets=offsets, lo=self.lo, hi=self.hi)
+            return out
+        out = torch.empty((N, p * p), dtype=g.dtype, device=g.device)
+        ops.collect_seq([mi], p, out, lo=self.lo, hi=self.hi)
+        return out
+
+    # ---- deferred (one launch per batch) -----------------------------------------------------
+    def defer_module(self, module: nn.Module, g: Tensor, out_col: int) -> None:
+        """Queue `module` for `launch_deferred`; keeps a and g alive until then."""
+        self._deferred.append(self.module_input(module, g, out_col))
+
+    def launch_deferred(self, out: Tensor, *, lengths: Tensor | None = None, out_rows: Tensor | None = None,
+                        row_offsets: Tensor | None = None) -> None:
+        """One fused launch over every queued module, writing each module's block of `out`."""
+        if not self._deferred:
+            return
+        p = self.per_module_projection_dim
+        assert p is not None
+        try:
+            if self.attribute_tokens:
+                assert lengths is not None and row_offsets is not None
+                ops.collect_tok(self._deferred, p, out, lengths=lengths, row_offsets=row_offsets, lo=self.lo,
+                                hi=self.hi)
+            else:
+                ops.collect_seq(self._deferred, p, out, lengths=lengths, out_rows=out_rows, lo=self.lo, hi=self.hi)
+        finally:
+            self._deferred.clear()
+
+    @abstractmethod
+    def setup(self) -> None: ...
+
+    @abstractmethod
+    def teardown(self) -> None: ...
+
+    @abstractmethod
+    def backward_hook(self, module: nn.Module, g: Tensor) -> None: ...
+
+    @abstractmethod
+    def process_batch(self, indices: list[int], **kwargs) -> None: ...
+
+
+class CollectorComputer:
+    """Runs forward/backward over the batches and feeds the collector (collector.py:771-923)."""
+
+    def __init__(self, model, data, *, collector: HookCollectorBase, batches: list[list[int]] | None = None,
+                 cfg: IndexConfig):
+        self.model = model
+        self.device = torch.device(model.device)
+        self.data = data
+        self.batches = batches if batches is not None else [[idx] for idx in range(len(data))]
+        self.forward_backward = fwd_bwd_factory(cfg)
+        self.collector = collector
+        self.cfg = cfg
+        self.rank = dist.get_rank() if dist.is_initialized() else 0
+        self.world_size = dist.get_world_size() if dist.is_initialized() else 1
+
+    def run_with_collector_hooks(self, desc: Optional[str] = None):
+        """For each batch: pad, forward, loss, backward (hooks fire), `collector.process_batch`; then
+        `collector.teardown()`.  No host synchronisation happens inside the loop."""
+        total_processed = torch.tensor(0, device=self.device)
+        for indices in self.batches:
+            batch = self.data[indices]
+            x, y, _, collection_mask = pad_and_tensor(batch["input_ids"], labels=batch.get("labels"),
+                                                      device=self.device, sync_max_len=False)
+            total_processed += collection_mask.sum()
+            with self.collector.with_batch(collection_mask):
+                losses = self.forward_backward(self.model, x, y, batch)
+            self.collector.process_batch(indices, losses=losses)
+        self.collector.teardown()
+        if dist.is_initialized():
+            dist.all_reduce(total_processed, op=dist.ReduceOp.SUM)
+        if self.rank == 0 and self.cfg.run_path:
+            os.makedirs(self.cfg.partial_run_path, exist_ok=True)
+            torch.save(total_processed, os.path.join(self.cfg.partial_run_path, "total_processed.pt"))
+        self.total_processed = total_processed
+
+
+def fwd_bwd_factory(cfg: IndexConfig) -> Callable:
+    """fwd_bwd(model, x, y, batch) -> per-sample losses [N] (collector.py:926-985, cross-entropy branch)."""
+    if cfg.loss_fn != "ce":
+        raise NotImplementedError("only the cross-entropy loss is supported (loss_fn='kl' needs PEFT)")
+
+    def fwd_bwd(model, x: Tensor, y: Tensor, batch: dict):
+        logits = model(x).logits[:, :-1]
+        masks = y[:, 1:] != -100
+        denoms = masks.sum(dim=1, dtype=model.dtype) if cfg.loss_reduction == "mean" else 1.0
+        losses = F.cross_entropy(logits.reshape(-1, logits.size(-1)), y[:, 1:].flatten(), reduction="none",
+                                 label_smoothing=cfg.label_smoothing).reshape_as(y[:, 1:])
+        losses = losses.sum(1) / denoms
+        if "advantage" in batch:
+            losses *= torch.tensor(batch["advantage"], device=losses.device)
+        losses.sum().backward()
+        model.zero_grad()
+        return losses
+
+    return fwd_bwd

@@ -1,0 +1,358 @@
+"""On-disk gradient / score stores, batch allocation and padding.
+
+Byte-compatible with the reference's formats (bergson/data.py): `gradients.bin`
+is a raw row-major [num_grads, sum(grad_sizes)] array of `base_dtype`,
+`info.json` carries {attribute_tokens, num_items, num_grads, grad_sizes,
+base_dtype}, per-token stores add `offsets.npy`.  numpy has no bfloat16, so a
+bfloat16 store is mapped as uint16 bit patterns; `info.json` still says
+"bfloat16" and the bytes are the same.
+"""
+from __future__ import annotations
+
+import heapq
+import json
+import os
+import random
+from pathlib import Path
+from typing import Any, Iterator
+
+import numpy as np
+import torch
+import torch.distributed as dist
+from numpy.lib.recfunctions import structured_to_unstructured
+
+from .utils import BF16_NAME, storage_np_dtype
+
+
+def _dtype_name(dtype) -> str:
+    """Accepts a numpy dtype, a dtype name or torch.bfloat16 / 'bfloat16'."""
+    if isinstance(dtype, str):
+        return dtype
+    if isinstance(dtype, torch.dtype):
+        from .utils import dtype_name
+
+        return dtype_name(dtype)
+    return np.dtype(dtype).name
+
+
+def _lengths_of(data) -> np.ndarray:
+    cols = data.column_names
+    if "length" in cols:
+        return np.asarray(data["length"], dtype=np.int64)
+    if "input_ids" in cols:
+        return np.asarray([len(x) for x in data["input_ids"]], dtype=np.int64)
+    return np.asarray([len(x) for x in data["labels"]], dtype=np.int64)
+
+
+def compute_num_token_grads(data) -> np.ndarray:
+    """Per-token rows stored per example: max(length - 1, 0) (bergson/data.py:37-62)."""
+    return np.maximum(_lengths_of(data) - 1, 0)
+
+
+def _rank() -> int:
+    return dist.get_rank() if dist.is_initialized() else 0
+
+
+def _allocate_file(path: Path, nbytes: int) -> None:
+    with open(path, "wb") as f:
+        f.truncate(nbytes)
+        os.fsync(f.fileno())
+
+
+def create_token_index(root: Path, num_token_grads: np.ndarray, grad_sizes: dict[str, int], dtype
+                       ) -> tuple[np.memmap, np.ndarray]:
+    """Ragged per-token store: gradients.bin + offsets.npy + info.json (bergson/data.py:65-137)."""
+    root = Path(root)
+    name = _dtype_name(dtype)
+    np_dtype = storage_np_dtype(name)
+    total_grad_dim = sum(grad_sizes.values())
+    offsets = np.zeros(len(num_token_grads) + 1, dtype=np.int64)
+    np.cumsum(num_token_grads, out=offsets[1:])
+    total_tokens = int(offsets[-1])
+    grad_path = root / "gradients.bin"
+    if _rank() == 0:
+        root.mkdir(parents=True, exist_ok=True)
+        _allocate_file(grad_path, np_dtype.itemsize * total_tokens * total_grad_dim)
+        np.save(root / "offsets.npy", offsets)
+        with (root / "info.json").open("w") as f:
+            json.dump({"attribute_tokens": True, "num_items": len(num_token_grads), "num_grads": total_tokens,
+                       "grad_sizes": grad_sizes, "base_dtype": name}, f, indent=2)
+    if dist.is_initialized():
+        dist.barrier()
+    if total_tokens == 0:
+        return np.zeros((0, total_grad_dim), dtype=np_dtype), offsets  # type: ignore[return-value]
+    mmap = np.memmap(grad_path, dtype=np_dtype, mode="r+", shape=(total_tokens, total_grad_dim))
+    return mmap, offsets
+
+
+def create_index(root: Path, num_grads: int, grad_sizes: dict[str, int], dtype) -> np.memmap:
+    """Flat [num_grads, total_grad_dim] store: gradients.bin + info.json (bergson/data.py:392-445)."""
+    root = Path(root)
+    name = _dtype_name(dtype)
+    np_dtype = storage_np_dtype(name)
+    total = sum(grad_sizes.values())
+    grad_path = root / "gradients.bin"
+    if _rank() == 0:
+        root.mkdir(parents=True, exist_ok=True)
+        _allocate_file(grad_path, np_dtype.itemsize * total * num_grads)
+        with (root / "info.json").open("w") as f:
+            json.dump({"attribute_tokens": False, "num_items": num_grads, "num_grads": num_grads,
+                       "grad_sizes": grad_sizes, "base_dtype": name}, f, indent=2)
+    if dist.is_initialized():
+        dist.barrier()
+    return np.memmap(grad_path, dtype=np_dtype, mode="r+", shape=(num_grads, total))
+
+
+def column_offsets(grad_sizes: dict[str, int]) -> dict[str, tuple[int, int]]:
+    """(start, end) columns of each module in grad_sizes order (bergson/data.py:380-389)."""
+    offsets, start = {}, 0
+    for name, size in grad_sizes.items():
+        offsets[name] = (start, start + size)
+        start += size
+    return offsets
+
+
+def load_info(root_dir: Path | str) -> dict:
+    with (Path(root_dir) / "info.json").open("r") as f:
+        return json.load(f)
+
+
+def store_base_dtype(info: dict) -> str:
+    """`base_dtype`, or the scalar dtype of an old structured store (bergson/data.py:508-512)."""
+    if "base_dtype" in info:
+        return info["base_dtype"]
+    fmt = info["dtype"]["formats"][0]
+    return BF16_NAME if "bfloat16" in str(fmt) or str(fmt) == "|V2" else np.dtype(fmt).base.name
+
+
+def load_gradients(root_dir: Path | str) -> np.memmap:
+    """Read-only map of the flat [num_grads, total_grad_dim] array (bergson/data.py:492-519).
+
+    A bfloat16 store comes back as uint16 bit patterns; `utils.numpy_to_tensor(arr, 'bfloat16')` reinterprets them.
+    """
+    root_dir = Path(root_dir)
+    info = load_info(root_dir)
+    np_dtype = storage_np_dtype(store_base_dtype(info))
+    return np.memmap(root_dir / "gradients.bin", dtype=np_dtype, mode="r",
+                     shape=(info["num_grads"], sum(info["grad_sizes"].values())))
+
+
+def load_token_gradients(root_dir: Path | str) -> tuple[np.memmap, np.ndarray, np.ndarray]:
+    """(mmap, num_token_grads, offsets) of a per-token store (bergson/data.py:138-156)."""
+    root_dir = Path(root_dir)
+    mmap = load_gradients(root_dir)
+    offsets = np.load(root_dir / "offsets.npy")
+    return mmap, np.diff(offsets).astype(np.int64), offsets
+
+
+class TokenGradients:
+    """`tg[i]` = example i's [num_token_grads[i], grad_dim] rows (bergson/data.py:159-183)."""
+
+    def __init__(self, root_dir: Path | str):
+        self.mmap, self._num_token_grads, self._offsets = load_token_gradients(root_dir)
+
+    @property
+    def num_token_grads(self) -> np.ndarray:
+        return self._num_token_grads
+
+    def __len__(self) -> int:
+        return len(self._num_token_grads)
+
+    def __getitem__(self, i: int) -> np.ndarray:
+        return np.asarray(self.mmap[self._offsets[i]:self._offsets[i + 1]])
+
+
+class ModuleGradients:
+    """Module-name-keyed column views over a flat store (bergson/data.py:522-548)."""
+
+    def __init__(self, mmap: np.memmap, grad_sizes: dict[str, int]):
+        self.mmap = mmap
+        self.offsets = column_offsets(grad_sizes)
+
+    def __getitem__(self, name: str) -> np.ndarray:
+        lo, hi = self.offsets[name]
+        return self.mmap[:, lo:hi]
+
+    def __len__(self) -> int:
+        return len(self.mmap)
+
+    def __iter__(self) -> Iterator[str]:
+        return iter(self.offsets)
+
+    def __contains__(self, name: str) -> bool:
+        return name in self.offsets
+
+    def keys(self):
+        return self.offsets.keys()
+
+
+def load_module_gradients(root_dir: Path | str) -> ModuleGradients:
+    root_dir = Path(root_dir)
+    return ModuleGradients(load_gradients(root_dir), load_info(root_dir)["grad_sizes"])
+
+
+class Scores:
+    """A score store: structured (score_i, written_i) rows (bergson/data.py:587-644)."""
+
+    def __init__(self, mmap: np.memmap, info: dict[str, Any], offsets: np.ndarray | None = None):
+        self.mmap = mmap
+        self.info = info
+        self.offsets = offsets
+        self.num_scores = info["num_scores"]
+        self._score_fields = [f"score_{i}" for i in range(self.num_scores)]
+
+    def __len__(self) -> int:
+        return self.info["num_items"]
+
+    def __getitem__(self, key: Any) -> np.ndarray:
+        return structured_to_unstructured(self.mmap[key][self._score_fields])
+
+    def get(self, key: Any, score_idx: int = 0) -> np.ndarray:
+        return self.mmap[key][f"score_{score_idx}"]
+
+    def is_written(self) -> bool:
+        return all(np.all(self.mmap[f"written_{i}"]) for i in range(self.num_scores))
+
+    def to_grid(self) -> torch.Tensor:
+        """Per-token store -> zero-padded [docs, seq_len(, num_scores)] grid."""
+        assert self.offsets is not None, "to_grid() requires a per-token store"
+        tokens_per_doc = np.diff(self.offsets).astype(np.int64)
+        seq_len = int(tokens_per_doc.max()) + 1
+        grid = np.zeros((len(self), seq_len, self.num_scores), dtype=np.float32)
+        for doc in range(len(self)):
+            grid[doc, :tokens_per_doc[doc]] = self[self.offsets[doc]:self.offsets[doc + 1]]
+        scores = torch.from_numpy(grid)
+        return scores[..., 0] if self.num_scores == 1 else scores
+
+
+def score_np_dtype(info_dtype: dict) -> np.dtype:
+    """numpy structured dtype from the JSON spec; bfloat16 score fields map as 2-byte voids."""
+    formats = ["V2" if f == BF16_NAME else f for f in info_dtype["formats"]]
+    return np.dtype({"names": info_dtype["names"], "formats": formats, "offsets": info_dtype["offsets"],
+                     "itemsize": info_dtype["itemsize"]})
+
+
+def load_scores(path: Path | str) -> Scores:
+    """bergson/data.py:647-664."""
+    path = Path(path)
+    info = load_info(path)
+    mmap = np.memmap(path / "scores.bin", dtype=score_np_dtype(info["dtype"]), mode="r", shape=(info["num_rows"],))
+    offsets = np.load(path / "offsets.npy") if info.get("attribute_tokens") else None
+    return Scores(mmap, info, offsets)
+
+
+# ---- batching ---------------------------------------------------------------------------
+
+def allocate_batches(doc_lengths: list[int], N: int, seed: int = 42, max_batch_size: int | None = None
+                     ) -> list[list[int]]:
+    """This rank's batches under `max_len_in_batch * batch_size <= N` (bergson/data.py:190-236)."""
+    rank = dist.get_rank() if dist.is_initialized() else 0
+    world_size = dist.get_world_size() if dist.is_initialized() else 1
+    (batches,) = _allocate_batches_world(doc_lengths, N, world_size, seed, ranks=[rank],
+                                         max_batch_size=max_batch_size)
+    return batches
+
+
+def _allocate_batches_world(doc_lengths: list[int], N: int, world_size: int, seed: int = 42,
+                            ranks: list[int] | None = None, max_batch_size: int | None = None
+                            ) -> list[list[list[int]]]:
+    """Greedy length-sorted bin packing, split to a multiple of the world size, dealt round-robin,
+    shuffled per rank with `random.seed(seed)` (bergson/data.py:239-377).  Documents shorter than two
+    tokens are left out (their store rows stay zero)."""
+    doc_lengths = list(doc_lengths)
+    if ranks is None:
+        ranks = list(range(world_size))
+    docs_sorted = sorted(((i, l) for i, l in enumerate(doc_lengths) if l >= 2), key=lambda x: x[1], reverse=True)
+    n_skipped = len(doc_lengths) - len(docs_sorted)
+    if n_skipped > 0 and _rank() == 0:
+        print(f"Skipping {n_skipped} documents with fewer than 2 tokens (no valid next-token labels).")
+    if len(docs_sorted) < world_size:
+        raise RuntimeError("Not enough documents (with 2+ tokens) to distribute across workers.")
+    if docs_sorted[0][1] > N:
+        raise RuntimeError(f"At least one document is too long for the token batch size {N}.")
+
+    batches: list[list[int]] = []
+    cur: list[int] = []
+    for idx, length in docs_sorted:
+        if not cur:
+            cur.append(idx)
+            continue
+        new_cost = max(length, doc_lengths[cur[0]]) * (len(cur) + 1)
+        within_count = max_batch_size is None or len(cur) + 1 <= max_batch_size
+        if new_cost <= N and within_count:
+            cur.append(idx)
+        else:
+            batches.append(cur)
+            cur = [idx]
+    if cur:
+        batches.append(cur)
+
+    if len(batches) < world_size:  # every worker needs at least one batch
+        counter = 0
+        heap: list[tuple[int, int, list[int]]] = []
+        for batch in batches:
+            heapq.heappush(heap, (-len(batch), counter, batch))
+            counter += 1
+        while len(heap) < world_size:
+            _, _, big = heapq.heappop(heap)
+            if len(big) == 1:
+                raise RuntimeError("Not enough documents to give each worker at least one batch.")
+            singleton = [big.pop()]
+            heapq.heappush(heap, (-len(big), counter, big))
+            counter += 1
+            heapq.heappush(heap, (-1, counter, singleton))
+            counter += 1
+        batches = [b for _, _, b in heap]
+
+    k = -(-len(batches) // world_size)
+    target_batches = world_size * k
+    i = 0
+    while len(batches) < target_batches and i < len(batches):
+        batch = batches[i % len(batches)]
+        if len(batch) == 1:
+            i += 1
+            continue
+        batches.append([batch.pop()])
+        i += 1
+    assert len(batches) == target_batches, (
+        "Could not construct a number of batches divisible by the world size."
+        " If variability of item lengths in your dataset is low "
+        "consider using a different dataset size or token batch size.")
+    assert all(max(doc_lengths[i] for i in batch) * len(batch) <= N for batch in batches)
+
+    allocation: list[list[list[int]]] = [[] for _ in range(world_size)]
+    for b_idx, batch in enumerate(batches):
+        allocation[b_idx % world_size].append(batch)
+    assert len({len(b) for b in allocation}) == 1
+    for rank in ranks:
+        random.seed(seed)
+        random.shuffle(allocation[rank])
+    return [allocation[rank] for rank in ranks]
+
+
+def pad_and_tensor(sequences: list[list[int]], labels: list[list[int]] | None = None, *, padding_value: int = 0,
+                   dtype: torch.dtype | None = torch.long, device: torch.device | None = None,
+                   sync_max_len: bool = True) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(padded ids, padded labels (-100), shift_loss_masks, collection_masks) (bergson/data.py:743-806).
+
+    collection_masks[n, s] = s + 1 < len(sequences[n]): every real position but the last.
+    """
+    if labels is None:
+        labels = sequences
+    max_len = max(len(seq) for seq in sequences)
+    if sync_max_len and dist.is_initialized():
+        t = torch.tensor(max_len, device=device)
+        dist.all_reduce(t, op=dist.ReduceOp.MAX)
+        max_len = int(t)
+    padded = [list(seq) + [padding_value] * (max_len - len(seq)) for seq in sequences]
+    padded_labels = [list(label) + [-100] * (max_len - len(label)) for label in labels]
+    # built on the host and moved once: one H2D copy per tensor instead of device-side construction
+    tokens = torch.tensor(padded, dtype=dtype).to(device, non_blocking=True)
+    labels_t = torch.tensor(padded_labels, dtype=dtype).to(device, non_blocking=True)
+    N, S = tokens.shape
+    shift_loss_masks = torch.zeros(N, S, dtype=torch.bool, device=device)
+    shift_loss_masks[:, :-1] = labels_t[:, 1:] != -100
+    lengths = torch.tensor([len(seq) for seq in sequences]).to(device, non_blocking=True)
+    positions = torch.arange(S, device=device)
+    collection_masks = (positions.unsqueeze(0) + 1) < lengths.unsqueeze(1)
+    return tokens, labels_t, shift_loss_masks, collection_masks

@@ -1,0 +1,132 @@
+"""The whole collection loop on the GPU against the CPU oracle.
+
+Two kinds of comparison:
+  * fp32, Pythia-14m shape: the product loop on the GPU against the oracle's loop on the CPU.  Both
+    run the same transformers model; the model's own forward/backward differs between devices at
+    fp32 rounding level, so the store rows are compared at rel-L2 <= 1e-3 (the kernels alone are held
+    to 1e-5 on identical inputs in test_collect_gpu.py).
+  * bf16, Pythia-160m shape: the (a, g) pairs the hooks saw on the GPU are captured and pushed through
+    the oracle's hook arithmetic on the CPU; the store rows must agree within rel-L2 <= 1e-2.
+"""
+import json
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import rel_l2
+from oracle import hooks as ohooks
+from oracle import loop as oloop
+from oracle.projection import module_projections
+
+pytestmark = pytest.mark.gpu
+
+
+def _processor(p, normalizers=None):
+    from bergson_amd import GradientProcessor
+
+    return GradientProcessor(normalizers=normalizers or {}, projection_dim=p, projection_type="normal")
+
+
+def test_pythia14m_fp32_store_matches_cpu_loop(device, tmp_path):
+    from bergson_amd import IndexConfig, allocate_batches, collect_gradients, load_gradients
+    from bergson_amd.synthetic import ListDataset, make_gpt_neox, random_docs
+
+    lengths = [64, 64, 40, 33, 17, 64, 2, 50, 1, 29]
+    docs = random_docs(lengths, seed=3)
+    batches = allocate_batches(lengths, 128)
+    assert batches == oloop.allocate_batches(lengths, 128)
+    model_cpu = make_gpt_neox("pythia-14m", torch.float32, "cpu", seed=0)
+    want, want_losses = oloop.collect(model_cpu, model_cpu.base_model, docs, batches, p=16)
+
+    model = make_gpt_neox("pythia-14m", torch.float32, device, seed=0)
+    cfg = IndexConfig(run_path=str(tmp_path / "run"), projection_dim=16, projection_type="normal")
+    col = collect_gradients(model, ListDataset(docs), _processor(16), cfg, batches=batches)
+    torch.cuda.synchronize()
+    part = cfg.partial_run_path
+    info = json.loads((part / "info.json").read_text())
+    assert info["base_dtype"] == "float32" and info["num_grads"] == len(docs) and not info["attribute_tokens"]
+    assert list(info["grad_sizes"].values()) == [256] * 24
+    assert list(info["grad_sizes"])[0] == "layers.0.attention.query_key_value"
+    got = torch.from_numpy(np.array(load_gradients(part)))
+    assert got.shape == (len(docs), 24 * 256)
+    assert got[8].abs().sum() == 0  # a one-token document is never batched; its row stays zero
+    assert rel_l2(got, want) <= 1e-3
+    assert torch.allclose(col.per_doc_losses.cpu(), want_losses, rtol=1e-4, atol=1e-4)
+    assert int(col.total_processed) == sum(l - 1 for l in lengths if l >= 2)
+    assert (part / "processor_config.yaml").exists() and (part / "total_processed.pt").exists()
+
+
+def test_pythia14m_fp32_per_token_store(device, tmp_path):
+    from bergson_amd import IndexConfig, TokenGradients, allocate_batches, collect_gradients
+    from bergson_amd.synthetic import ListDataset, make_gpt_neox, random_docs
+
+    lengths = [30, 12, 1, 25, 7]
+    docs = random_docs(lengths, seed=5)
+    batches = allocate_batches(lengths, 64)
+    model_cpu = make_gpt_neox("pythia-14m", torch.float32, "cpu", seed=0, layers=2)
+    want, _ = oloop.collect(model_cpu, model_cpu.base_model, docs, batches, p=16, attribute_tokens=True)
+    want_seq, _ = oloop.collect(model_cpu, model_cpu.base_model, docs, batches, p=16)
+
+    model = make_gpt_neox("pythia-14m", torch.float32, device, seed=0, layers=2)
+    cfg = IndexConfig(run_path=str(tmp_path / "tok"), projection_dim=16, projection_type="normal",
+                      attribute_tokens=True)
+    collect_gradients(model, ListDataset(docs), _processor(16), cfg, batches=batches)
+    tg = TokenGradients(cfg.partial_run_path)
+    assert tg.num_token_grads.tolist() == [29, 11, 0, 24, 6]
+    got = torch.from_numpy(np.array(tg.mmap))
+    assert got.shape == want.shape
+    assert rel_l2(got, want) <= 1e-3
+    # the rows of a document add up to its per-sequence gradient
+    assert rel_l2(torch.from_numpy(tg[0]).sum(0), want_seq[0]) <= 1e-3
+
+
+@pytest.mark.parametrize("store_dtype", [None, torch.float16])
+def test_pythia160m_bf16_adafactor_against_captured_hooks(device, store_dtype):
+    from bergson_amd import AdafactorNormalizer, GradientCollector, IndexConfig
+    from bergson_amd.collector import CollectorComputer
+    from bergson_amd.synthetic import ListDataset, adafactor_moments, make_gpt_neox, random_docs
+
+    lengths = [300, 180, 260]
+    docs = random_docs(lengths, seed=7)
+    model = make_gpt_neox("pythia-160m", torch.bfloat16, device, seed=0, layers=3)
+    moments = adafactor_moments(model.base_model, seed=0)
+    normalizers = {n: AdafactorNormalizer(row=r.to(device), col=c.to(device)) for n, (r, c) in moments.items()}
+
+    captured = {}
+    handles = []
+    for name, mod in model.base_model.named_modules():
+        if isinstance(mod, torch.nn.Linear):
+            handles.append(mod.register_forward_hook(
+                lambda m, inp, out, name=name: captured.setdefault(name, {}).__setitem__("a", inp[0].detach().cpu())))
+            handles.append(mod.register_full_backward_hook(
+                lambda m, gin, gout, name=name: captured[name].__setitem__("g", gout[0].detach().cpu())))
+
+    cfg = IndexConfig(run_path="", projection_dim=16, projection_type="normal")
+    kw = {} if store_dtype is None else {"store_dtype": store_dtype}
+    col = GradientCollector(model=model.base_model, cfg=cfg, data=ListDataset(docs), processor=_processor(16, normalizers),
+                            **kw)
+    CollectorComputer(model=model, data=ListDataset(docs), collector=col, batches=[[0, 1, 2]], cfg=cfg
+                      ).run_with_collector_hooks()
+    for h in handles:
+        h.remove()
+    out_dtype = store_dtype or torch.bfloat16
+    assert col.builder.base_dtype == {torch.bfloat16: "bfloat16", torch.float16: "float16"}[out_dtype]
+    buf = col.builder.grad_buffer
+    got = torch.from_numpy(buf.astype(np.float32)) if out_dtype == torch.float16 else \
+        torch.from_numpy(buf.copy()).view(torch.bfloat16).float()
+    assert got.shape == (3, 12 * 256)
+
+    lo, hi = torch.finfo(out_dtype).min, torch.finfo(out_dtype).max
+    blocks = []
+    for name, (row, col_m) in moments.items():
+        a, g = captured[name]["a"], captured[name]["g"]
+        left, right = module_projections(name, 16, g.shape[-1], a.shape[-1], torch.bfloat16)
+        P = ohooks.module_gradient(a, g, ohooks.Adafactor(row=row, col=col_m), left, right)
+        blocks.append(P.float().clamp(lo, hi))
+    want = torch.cat(blocks, 1)
+    assert torch.isfinite(got).all()
+    assert rel_l2(got, want) <= 1e-2
+    # every module on its own, so that a small block cannot hide behind a large one
+    for b in range(12):
+        assert rel_l2(got[:, b * 256:(b + 1) * 256], want[:, b * 256:(b + 1) * 256]) <= 1e-2
