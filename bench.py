@@ -1,0 +1,271 @@
+#!/usr/bin/env python3
+"""Benchmark of the collection path on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+Workload (N=1): Pythia-160m-shaped GPT-NeoX, random-init bf16; 2048 documents with lengths
+lognormal(6, 1) clipped to [16, 2048], bin-packed into 4096-token batches, uniform-random ids;
+projection_dim 16 Gaussian projections on all 48 Linear modules; Adafactor normalizer with second
+moments |N(0,1)| * 1e-4; per-sequence gradients written to an fp16 store.
+
+A step is one batch through the whole path: forward, loss, backward (hooks queue the modules), one
+fused collection launch into the device-resident fp16 store.  The store is copied to its memory-mapped
+file once after the last timed step, inside the timed region.  Padded batches are staged in HBM
+before the timed region starts.  value = documents' tokens / wall seconds.
+
+One JSON line is printed.  It also carries
+  roofline      the fused collection kernel: algorithmic bytes (a and g read once) per launch over its
+                duration measured with events on the launch stream, against 8 TB/s;
+  cpu_baseline  the CPU oracle (the reference's op sequence on PyTorch CPU) on a bounded sample;
+  store_scan    the second half of the metric: 10^6 fp16 rows of 12288 scanned against 1024 queries
+                with unit-norm cosine, top-100 per query and the per-row max.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=40)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--docs", type=int, default=2048)
+    ap.add_argument("--token-batch-size", type=int, default=4096)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-scan", action="store_true")
+    ap.add_argument("--scan-rows", type=int, default=1_000_000)
+    ap.add_argument("--scan-queries", type=int, default=1024)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=32768)
+    return ap.parse_args()
+
+
+def collection_leg(args, torch, device):
+    import bergson_amd as B
+    from bergson_amd import ops
+    from bergson_amd.synthetic import ListDataset, adafactor_moments, lognormal_lengths, make_gpt_neox, random_docs
+
+    lengths = lognormal_lengths(args.docs, seed=0)
+    docs = random_docs(lengths, seed=0)
+    data = ListDataset(docs)
+    batches = B.allocate_batches(lengths, args.token_batch_size)
+    need = args.warmup + args.steps
+    if len(batches) < need:
+        raise SystemExit(f"{len(batches)} batches < warmup + steps = {need}: lower --steps or raise --docs")
+    model = make_gpt_neox("pythia-160m", torch.bfloat16, device, seed=0)
+    moments = adafactor_moments(model.base_model, seed=0)
+    normalizers = {n: B.AdafactorNormalizer(row=r.to(device), col=c.to(device)) for n, (r, c) in moments.items()}
+    processor = B.GradientProcessor(normalizers=normalizers, projection_dim=16, projection_type="normal")
+    run_dir = tempfile.mkdtemp(prefix="bgx_bench_")
+    cfg = B.IndexConfig(run_path=os.path.join(run_dir, "store"), projection_dim=16, projection_type="normal",
+                        token_batch_size=args.token_batch_size)
+    collector = B.GradientCollector(model=model.base_model, cfg=cfg, data=data, processor=processor,
+                                    store_dtype=torch.float16)
+    fwd_bwd = B.fwd_bwd_factory(cfg)
+
+    staged = []
+    for indices in batches[:need]:
+        b = data[indices]
+        x, y, _, mask = B.pad_and_tensor(b["input_ids"], device=device, sync_max_len=False)
+        staged.append((indices, b, x, y, mask))
+    torch.cuda.synchronize()
+
+    def step(item):
+        indices, b, x, y, mask = item
+        with collector.with_batch(mask):
+            losses = fwd_bwd(model, x, y, b)
+        collector.process_batch(indices, losses=losses)
+
+    for item in staged[:args.warmup]:
+        step(item)
+    torch.cuda.synchronize()
+    ops.collect_timer = []
+    t0 = time.perf_counter()
+    for item in staged[args.warmup:need]:
+        step(item)
+    collector.builder.flush()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    timer, ops.collect_timer = ops.collect_timer, None
+
+    tokens = sum(lengths[i] for item in staged[args.warmup:need] for i in item[0])
+    padded = sum(int(item[2].numel()) for item in staged[args.warmup:need])
+    kernel_ms = sum(e0.elapsed_time(e1) for e0, e1, _ in timer)
+    kernel_bytes = sum(nb for _, _, nb in timer)
+    achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
+    store = collector.builder.grad_buffer
+    out = {
+        "seconds": t1 - t0,
+        "tokens": tokens,
+        "padded_tokens": padded,
+        "launches": len(timer),
+        "kernel_ms_per_launch": kernel_ms / max(1, len(timer)),
+        "kernel_bytes_per_launch": kernel_bytes / max(1, len(timer)),
+        "achieved_gbs": achieved,
+        "n_batches_total": len(batches),
+        "store_rows_nonzero": int((abs(store[:, :256].astype("float32")).sum(axis=1) > 0).sum()),
+        "total_tokens_all_docs": int(sum(lengths)),
+    }
+    del collector, model
+    torch.cuda.empty_cache()
+    return out, docs, lengths
+
+
+def scan_leg(args, torch, device):
+    from bergson_amd import ops
+
+    n, D, Q, k = args.scan_rows, 12288, args.scan_queries, 100
+    gen = torch.Generator(device=device).manual_seed(1)
+    store = torch.empty((n, D), dtype=torch.float16, device=device)
+    step = 65536
+    for lo in range(0, n, step):
+        hi = min(n, lo + step)
+        blk = torch.randn((hi - lo, D), generator=gen, device=device)
+        heavy = torch.rand((hi - lo, 1), generator=gen, device=device) < 0.05
+        store[lo:hi] = (blk * torch.where(heavy, 10.0, 1.0)).to(torch.float16)
+    q = torch.randn((Q, D), generator=gen, device=device)
+    q = q / q.norm(dim=1, keepdim=True)
+    q = torch.cat([q, q.mean(dim=0, keepdim=True)], dim=0)  # last row: mean query -> mean-over-queries score
+    qd = (q * 64.0).to(torch.float16)
+
+    def run():
+        return ops.scan(store, qd, unit_norm=True, k=k, query_scale=1.0 / 64.0, want_row_max=True)
+
+    run()
+    torch.cuda.synchronize()
+    reps = 3
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        res = run()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / reps
+    flops = 2.0 * n * D * (Q + 1)
+    out = {
+        "rows": n, "dim": D, "queries": Q, "k": k, "ms": ms, "rows_per_s": n / (ms * 1e-3),
+        "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": MFMA_F16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, "traffic": None},
+        "hbm_gbs": n * D * 2 / (ms * 1e-3) / 1e9,
+        "top1_mean": float(res.topk_values[:Q, 0].mean().item()),
+    }
+    # the HBM-bound regime of the same kernel family: few queries per pass
+    q32 = qd[:32].contiguous()
+    ops.scan(store, q32, unit_norm=True, k=k, query_scale=1.0 / 64.0)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        ops.scan(store, q32, unit_norm=True, k=k, query_scale=1.0 / 64.0)
+    e1.record()
+    torch.cuda.synchronize()
+    ms32 = e0.elapsed_time(e1) / reps
+    gbs = n * D * 2 / (ms32 * 1e-3) / 1e9
+    out["q32"] = {"ms": ms32, "rows_per_s": n / (ms32 * 1e-3),
+                  "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                               "frac": gbs / HBM_PEAK_GBS, "traffic": None}}
+    del store
+    torch.cuda.empty_cache()
+    return out
+
+
+def cpu_baseline_leg(args, torch, docs, lengths):
+    """The CPU oracle on the first documents of the same workload, about `cpu_sample_tokens` tokens."""
+    from bergson_amd.synthetic import adafactor_moments, make_gpt_neox
+    from oracle import hooks as ohooks
+    from oracle import loop as oloop
+
+    picked, tok = [], 0
+    for i, l in enumerate(lengths):
+        if tok + l > args.cpu_sample_tokens and picked:
+            break
+        picked.append(i)
+        tok += l
+    sub_docs = [docs[i] for i in picked]
+    sub_len = [lengths[i] for i in picked]
+    batches = oloop.allocate_batches(sub_len, args.token_batch_size)
+    model = make_gpt_neox("pythia-160m", torch.bfloat16, "cpu", seed=0)
+    moments = adafactor_moments(model.base_model, seed=0)
+    norms = {n: ohooks.Adafactor(row=r, col=c) for n, (r, c) in moments.items()}
+    t0 = time.perf_counter()
+    rows, _ = oloop.collect(model, model.base_model, sub_docs, batches, p=16, normalizers=norms,
+                            save_dtype=torch.float16)
+    dt = time.perf_counter() - t0
+    return {"value": tok / dt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{len(picked)} documents / {tok} tokens of the same workload in {dt:.1f} s "
+                      f"(reference op sequence on PyTorch CPU, bf16 model, fp16 rows)"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported in this build "
+              "(collection shards by documents with no exchange, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (there is no CPU path)", file=sys.stderr)
+        sys.exit(1)
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    coll, docs, lengths = collection_leg(args, torch, device)
+    scan = None if args.no_scan else scan_leg(args, torch, device)
+    cpu = None if args.no_cpu_baseline else cpu_baseline_leg(args, torch, docs, lengths)
+
+    value = coll["tokens"] / coll["seconds"]
+    line = {
+        "metric": "grad-collection tokens/sec (Pythia-160m shape, p=16)",
+        "value": value,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": coll["seconds"] / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[1]: Pythia-160m-shaped GPT-NeoX bf16, lognormal(6,1) lengths in [16,2048], "
+                        "4096-token batches, p=16 normal projections on 48 modules, Adafactor normalizer, "
+                        "per-sequence rows into an fp16 store",
+            "documents": args.docs,
+            "token_batch_size": args.token_batch_size,
+            "tokens_timed": coll["tokens"],
+            "padded_tokens_timed": coll["padded_tokens"],
+            "batches_total": coll["n_batches_total"],
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "collect_kernel<bf16, p<=16> (+ its finalize launch inside the bracket)",
+            "achieved": coll["achieved_gbs"],
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": coll["achieved_gbs"] / HBM_PEAK_GBS,
+            "traffic": None,
+            "bytes_per_launch": coll["kernel_bytes_per_launch"],
+            "ms_per_launch": coll["kernel_ms_per_launch"],
+            "launches": coll["launches"],
+        },
+        "cpu_baseline": cpu,
+        "store_scan": scan,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -39,6 +39,10 @@ def _ptr(t: Tensor | None) -> C.c_void_p | None:
 
 _workspaces: dict[tuple[int, str], Tensor] = {}
 
+# When set to a list, every collection launch appends (start_event, stop_event, algorithmic_bytes): the
+# events bracket the launch on the stream it runs on.  Used by the benchmark; None costs nothing.
+collect_timer: list | None = None
+
 
 def _workspace(device: torch.device, nbytes: int, tag: str) -> Tensor:
     """Per-device scratch buffer, grown on demand and reused between calls (stream-ordered)."""
@@ -139,9 +143,17 @@ def _collect(per_token: bool, modules: list[ModuleInput], p: int, out: Tensor, l
     nbytes = lib.bgx_collect_workspace_bytes(len(modules), N, S, p)
     ws = _workspace(out.device, nbytes, "collect")
     fn = lib.bgx_collect_tok if per_token else lib.bgx_collect_seq
+    timer = collect_timer
+    if timer is not None:
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
     rc = fn(descs, len(modules), N, S, p, dtype_code(in_dtype), _ptr(lengths), _ptr(rows), _ptr(out),
             out.stride(0), dtype_code(out.dtype), lo, hi, _ptr(ws), ws.numel(), _stream())
     _lib.check(rc, "bgx_collect_tok" if per_token else "bgx_collect_seq")
+    if timer is not None:
+        ev1.record()
+        esz = 4 if in_dtype == torch.float32 else 2
+        timer.append((ev0, ev1, sum(int(N) * int(S) * (d.I + d.O) * esz for d in descs)))
     del keep
 
 

@@ -1,0 +1,73 @@
+"""The C-ABI library: it loads without a GPU, exports every symbol the header declares, and rejects bad
+arguments with the documented codes before touching the device."""
+import ctypes as C
+import re
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def _declared():
+    text = (ROOT / "include" / "bergson_amd.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(bgx_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound():
+    from bergson_amd import _lib
+
+    lib = _lib.load()
+    names = _declared()
+    assert "bgx_collect_seq" in names and "bgx_scan" in names and len(names) >= 9
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in the header but not exported"
+    assert sorted(_lib.SIGNATURES) == names, "ctypes bindings and header disagree"
+    assert lib.bgx_abi_version() == 1
+
+
+def test_module_desc_layout_matches_header():
+    from bergson_amd._lib import ModuleDesc
+
+    # 8 pointers, 5 int64, 2 int32
+    assert C.sizeof(ModuleDesc) == 8 * 8 + 5 * 8 + 2 * 4
+    assert ModuleDesc.out_col.offset == 8 * 8 + 4 * 8 and ModuleDesc.I.offset == 8 * 8 + 5 * 8
+
+
+def test_workspace_sizes():
+    from bergson_amd import _lib
+
+    lib = _lib.load()
+    # descriptors rounded to 256 B + one fp32 p*p partial per (module, sequence, 64-token tile)
+    assert lib.bgx_collect_workspace_bytes(48, 2, 2048, 16) == -(-48 * 112 // 256) * 256 + 48 * 2 * 32 * 256 * 4
+    assert lib.bgx_collect_workspace_bytes(0, 2, 64, 16) == 0
+    small = lib.bgx_scan_workspace_bytes(8, 10, 1024)
+    assert small >= 8 * 10 * 8 + 8 * 1024 * 8
+    assert lib.bgx_scan_workspace_bytes(1024, 100, 0) >= 1024 * 65536 * 8
+
+
+def test_argument_errors_before_any_launch():
+    from bergson_amd import _lib
+
+    lib = _lib.load()
+    descs = (_lib.ModuleDesc * 1)()
+    rc = lib.bgx_collect_seq(descs, 1, 1, 8, 16, 2, None, None, None, 256, 2, 0.0, 0.0, None, 0, None)
+    assert rc == -1 and b"null" in lib.bgx_last_error()
+    rc = lib.bgx_collect_seq(descs, 1, 1, 8, 65, 2, None, None, C.c_void_p(256), 256, 2, 0.0, 0.0, C.c_void_p(256), 0, None)
+    assert rc == -3 and b"p=65" in lib.bgx_last_error()
+    rc = lib.bgx_collect_seq(descs, 1, 1, 8, 16, 7, None, None, C.c_void_p(256), 256, 2, 0.0, 0.0, C.c_void_p(256), 0, None)
+    assert rc == -2
+    rc = lib.bgx_collect_seq(descs, 1, 1, 8, 16, 2, None, None, C.c_void_p(256), 256, 2, 0.0, 0.0, C.c_void_p(256), 16, None)
+    assert rc == -4 and b"workspace" in lib.bgx_last_error()
+    rc = lib.bgx_collect_tok(descs, 1, 1, 8, 16, 2, None, None, C.c_void_p(256), 256, 2, 0.0, 0.0, C.c_void_p(256), 1 << 20, None)
+    assert rc == -1 and b"lengths" in lib.bgx_last_error()
+    rc = lib.bgx_scan(None, 10, 8, 8, 1, None, 2, 1.0, 1, 1, 0, None, None, None, None, None, None, 0, 0, None)
+    assert rc == -1
+    rc = lib.bgx_scan(C.c_void_p(256), 10, 8, 8, 1, C.c_void_p(256), 2, 1.0, 1, 11, 0, C.c_void_p(256), C.c_void_p(256),
+                      None, None, None, C.c_void_p(256), 1 << 30, 0, None)
+    assert rc == -3 and b"k=11" in lib.bgx_last_error()
+    rc = lib.bgx_unit_normalize_rows(None, 1, 1, 1, 0, None)
+    assert rc == -1
+    with pytest.raises(_lib.BergsonAmdError, match="code -1"):
+        _lib.check(rc, "bgx_unit_normalize_rows")

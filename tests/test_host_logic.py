@@ -1,0 +1,176 @@
+"""Host-side logic that needs no GPU: batching, padding, target discovery, shapes, head splitting,
+processor files, and that the product refuses to run without a GPU instead of falling back."""
+import pytest
+import torch
+import torch.nn as nn
+
+from oracle import loop as oloop
+
+
+def test_allocate_batches_budget_order_and_oracle():
+    from bergson_amd import allocate_batches
+    from bergson_amd.data import _allocate_batches_world
+    from bergson_amd.synthetic import lognormal_lengths
+
+    lengths = lognormal_lengths(300, seed=0)
+    assert min(lengths) >= 16 and max(lengths) <= 2048
+    batches = allocate_batches(lengths, 4096)
+    assert batches == oloop.allocate_batches(lengths, 4096)
+    seen = sorted(i for b in batches for i in b)
+    assert seen == list(range(300))
+    assert all(max(lengths[i] for i in b) * len(b) <= 4096 for b in batches)
+    assert batches == allocate_batches(lengths, 4096)  # deterministic: shuffled with a fixed seed
+    # short documents are left out; a document longer than the budget is an error
+    assert sorted(i for b in allocate_batches([5, 1, 0, 7], 16) for i in b) == [0, 3]
+    with pytest.raises(RuntimeError, match="too long"):
+        allocate_batches([10, 50], 20)
+    # two workers get the same number of batches and disjoint documents
+    w = _allocate_batches_world(lengths, 4096, 2)
+    assert len(w[0]) == len(w[1])
+    assert not set(i for b in w[0] for i in b) & set(i for b in w[1] for i in b)
+    assert max(len(b) for b in allocate_batches(lengths, 4096, max_batch_size=3)) <= 3
+
+
+def test_pad_and_tensor_masks():
+    from bergson_amd import pad_and_tensor
+
+    x, y, shift, coll = pad_and_tensor([[5, 6, 7], [8]], sync_max_len=False)
+    assert x.tolist() == [[5, 6, 7], [8, 0, 0]]
+    assert y.tolist() == [[5, 6, 7], [8, -100, -100]]
+    assert coll.tolist() == [[True, True, False], [False, False, False]]
+    assert shift.tolist() == [[True, True, False], [False, False, False]]
+    ox, oy, om = oloop.pad_and_tensor([[5, 6, 7], [8]])
+    assert torch.equal(ox, x) and torch.equal(oy, y) and torch.equal(om, coll)
+    _, y2, shift2, coll2 = pad_and_tensor([[1, 2, 3, 4]], labels=[[-100, -100, 3, 4]], sync_max_len=False)
+    assert shift2.tolist() == [[False, True, True, False]] and coll2.tolist() == [[True, True, True, False]]
+
+
+class _Toy(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.attn = nn.Linear(8, 12)
+        self.mlp = nn.Sequential(nn.Linear(8, 16, bias=False), nn.GELU(), nn.Linear(16, 8))
+        self.norm = nn.LayerNorm(8)
+        self.device = torch.device("cpu")
+
+
+def _stub(model, **kw):
+    from bergson_amd import HookCollectorBase
+
+    class Stub(HookCollectorBase):
+        def setup(self): ...
+        def teardown(self): ...
+        def backward_hook(self, module, g): ...
+        def process_batch(self, indices, **k): ...
+
+    return Stub(model=model, **kw)
+
+
+def test_discover_targets_filters_and_bias():
+    from bergson_amd import GradientProcessor, HookCollectorBase
+
+    m = _Toy()
+    info = HookCollectorBase.discover_targets(m)
+    assert list(info) == ["attn", "mlp.0", "mlp.2"]
+    assert info["mlp.0"][1] == torch.Size([16, 8]) and info["attn"][2] is False
+    assert HookCollectorBase.discover_targets(m, include_bias=True)["attn"][2] is True
+    assert HookCollectorBase.discover_targets(m, include_bias=True)["mlp.0"][2] is False
+    assert list(HookCollectorBase.discover_targets(m, filter_modules="mlp.*")) == ["attn"]
+    assert list(HookCollectorBase.discover_targets(m, target_modules={"mlp.2"})) == ["mlp.2"]
+    with pytest.raises(ValueError, match="attention_cfgs"):
+        from bergson_amd import AttentionConfig
+        _stub(m, processor=GradientProcessor(projection_dim=4), attention_cfgs={"nope": AttentionConfig(2, 6, 2)})
+
+
+def test_shapes_and_head_normalizers():
+    from bergson_amd import AdafactorNormalizer, AdamNormalizer, AttentionConfig, GradientProcessor
+
+    m = _Toy()
+    c = _stub(m, processor=GradientProcessor(projection_dim=4), attention_cfgs={"attn": AttentionConfig(3, 4, 2)})
+    assert list(c.shapes()) == ["attn.head_0", "attn.head_1", "attn.head_2", "mlp.0", "mlp.2"]
+    assert all(s == torch.Size([4, 4]) for s in c.shapes().values())
+    full = _stub(m, processor=GradientProcessor(include_bias=True), attention_cfgs={"attn": AttentionConfig(3, 4, 2)})
+    assert full.shapes()["attn.head_1"] == torch.Size([4, 9]) and full.shapes()["mlp.0"] == torch.Size([16, 8])
+    assert full.shapes()["mlp.2"] == torch.Size([8, 17])
+    row, col = torch.arange(12.0), torch.arange(8.0)
+    c.processor.normalizers = {"attn": AdafactorNormalizer(row, col), "mlp.0": AdamNormalizer(torch.ones(16, 8))}
+    h1 = c.normalizer_for("attn.head_1")
+    assert h1.row.tolist() == [4.0, 5.0, 6.0, 7.0] and torch.equal(h1.col, col)
+    assert c.normalizer_for("mlp.2") is None and c.normalizer_for("mlp.0").weight_avg_sq.shape == (16, 8)
+    assert c.split_head_name("attn.head_2") == ("attn", 2) and c.split_head_name("attn") is None
+    c.processor.normalizers = {"attn": AdamNormalizer(torch.arange(96.0).reshape(12, 8), torch.arange(12.0))}
+    h2 = c.normalizer_for("attn.head_2")
+    assert h2.weight_avg_sq.shape == (4, 8) and h2.bias_avg_sq.tolist() == [8.0, 9.0, 10.0, 11.0]
+
+
+def test_projection_cache_and_roles():
+    from bergson_amd import GradientProcessor
+
+    c = _stub(_Toy(), processor=GradientProcessor(projection_dim=4, projection_type="normal"))
+    a = c.projection("attn", 4, 8, "right", torch.device("cpu"), torch.float32)
+    assert c.projection("attn", 4, 8, "right", torch.device("cpu"), torch.float32) is a
+    b = c.projection("attn", 4, 12, "left", torch.device("cpu"), torch.float32)
+    assert a.shape == (4, 8) and b.shape == (4, 12)
+    assert ("attn", "right", torch.device("cpu")) in c.processor._projection_matrices
+
+
+def test_processor_roundtrip(tmp_path):
+    from bergson_amd import AdafactorNormalizer, AdamNormalizer, GradientProcessor
+
+    p = GradientProcessor(normalizers={"a": AdafactorNormalizer(torch.ones(3), torch.ones(2) * 2),
+                                       "b": AdamNormalizer(torch.ones(3, 2), torch.ones(3))},
+                          projection_dim=16, projection_type="normal")
+    p.save(tmp_path)
+    for f in ["processor_config.yaml", "normalizers.pth", "hessians.pth", "hessians_eigen.pth"]:
+        assert (tmp_path / f).exists()
+    q = GradientProcessor.load(tmp_path)
+    assert q.projection_dim == 16 and q.projection_type == "normal" and q.projection_scale == "jl"
+    assert isinstance(q.normalizers["a"], AdafactorNormalizer) and q.normalizers["a"].col.tolist() == [2.0, 2.0]
+    assert isinstance(q.normalizers["b"], AdamNormalizer) and q.normalizers["b"].bias_avg_sq.shape == (3,)
+    ada = q.normalizers["b"].to_adafactor()
+    assert ada.row.shape == (3,) and ada.col.shape == (2,)
+    torch.testing.assert_close(q.normalizers["a"].to_adam().weight_avg_sq, torch.full((3, 2), 2.0))
+
+
+def test_config_defaults_follow_the_reference():
+    from bergson_amd import IndexConfig, PreprocessConfig, QueryConfig, ScoreConfig
+
+    c = IndexConfig(run_path="runs/x")
+    assert (c.projection_dim, c.projection_type, c.projection_scale, c.token_batch_size, c.loss_reduction,
+            c.attribute_tokens, c.include_bias) == (0, "rademacher", "jl", 2048, "sum", False, False)
+    assert str(c.partial_run_path) == "runs/x.part"
+    assert PreprocessConfig().aggregation == "none" and not PreprocessConfig().unit_normalize
+    assert ScoreConfig().precision == "fp32" and ScoreConfig().score == "individual"
+    assert QueryConfig().unit_norm is True and QueryConfig().top_k == 5
+
+
+def test_no_cpu_fallback():
+    """The product path refuses CPU tensors and CPU devices."""
+    from bergson_amd import Attributor, GradientProcessor, Scorer, ops
+    from bergson_amd.score_writer import InMemorySequenceScoreWriter
+
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.scan(torch.zeros(4, 8), torch.zeros(2, 8), unit_norm=True, k=1)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.unit_normalize_rows_(torch.zeros(4, 8))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        Scorer({"m": torch.zeros(2, 8)}, ["m"], InMemorySequenceScoreWriter(4, 2), torch.device("cpu"), torch.float32)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        Attributor("/nonexistent", device="cpu")
+    m = _Toy()
+    c = _stub(m, processor=GradientProcessor(projection_dim=4, projection_type="normal"))
+    with c:
+        m.attn(torch.randn(1, 3, 8)).sum().backward()  # hooks fire; nothing computed for the stub
+        mod = m.attn
+        mod._inputs = torch.randn(1, 3, 8)
+        with pytest.raises(RuntimeError, match="no CPU path"):
+            c._compute_gradient(mod, torch.randn(1, 3, 12))
+
+
+def test_product_does_not_import_the_oracle():
+    import pathlib
+    import re
+
+    root = pathlib.Path(__file__).resolve().parent.parent / "bergson_amd"
+    for f in root.rglob("*.py"):
+        assert not re.search(r"^\s*(from|import)\s+oracle\b", f.read_text(), re.M), f
