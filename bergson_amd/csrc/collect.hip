@@ -17,12 +17,13 @@
 // so no barrier is needed in the streaming loop; their partial projections
 // are combined through LDS in a fixed pairwise order (w0+w2)+(w1+w3).
 
+#include <algorithm>
+#include <vector>
+
 #include "common.hpp"
 
 namespace bgx {
 
-constexpr int TILE_T = 64;  // tokens per workgroup
-constexpr int MT = TILE_T / 16;
 constexpr int COLLECT_THREADS = 256;
 
 // ---- MFMA step per element type ---------------------------------------------
@@ -104,13 +105,12 @@ __device__ inline uint4 load_frag(const T* __restrict__ row, int k0, int K) {
 // x' = x @ (R * scale)^T for the 64 tokens of the tile, this wave's share of K.
 //   xrow0: pointer to token s0 of the sequence; rows s >= s_limit read as zero.
 //   acc[mt][pb][i] belongs to token mt*16 + (lane/16)*4 + i, column pb*16 + lane%16.
-template <typename T, int PB, bool ALIGNED>
+template <typename T, int PB, bool ALIGNED, int MT, int U>
 __device__ inline void project_tile(const T* __restrict__ xrow0, int64_t tok_stride, int rows_valid,
                                     int K, const T* __restrict__ R, int p,
                                     const float* __restrict__ scale, int wave, int lane,
                                     f32x4 (&acc)[MT][PB]) {
-  using M = Mma<T>;
-  constexpr int U = 2;  // k-steps kept in flight per wave
+  using M = Mma<T>;  // U = k-steps kept in flight per wave
   const int r = lane & 15;
   const int q = lane >> 4;
 
@@ -176,7 +176,7 @@ __device__ inline void project_tile(const T* __restrict__ xrow0, int64_t tok_str
 struct CollectArgs {
   const bgx_module_desc* mods;  // device copy
   const int32_t* lengths;
-  int N, S, p, tiles_per_seq;
+  int N, S, p, tiles_per_seq;  // tiles_per_seq = ceil(S / tokens per workgroup)
   // per-sequence
   float* partials;  // [n_modules][N][tiles_per_seq][p*p]
   // per-token
@@ -193,10 +193,11 @@ __device__ inline int seq_token_limit(const int32_t* lengths, int n, int S) {
   return l < S ? (l < 0 ? 0 : l) : S;
 }
 
-template <typename T, int PB, bool ALIGNED, bool PER_TOKEN>
+template <typename T, int PB, bool ALIGNED, bool PER_TOKEN, int MT, int U>
 __global__ __launch_bounds__(COLLECT_THREADS) void collect_kernel(CollectArgs args) {
-  constexpr int PP = PB * 16;   // padded projection dim
-  constexpr int LDP = PP + 1;   // LDS row stride (floats)
+  constexpr int TILE_T = 16 * MT;  // tokens per workgroup
+  constexpr int PP = PB * 16;      // padded projection dim
+  constexpr int LDP = PP + 1;      // LDS row stride (floats)
   __shared__ float sm[2][2][TILE_T][LDP];  // [a/g][slot][token][col]
 
   const int tile = blockIdx.x;
@@ -226,10 +227,10 @@ __global__ __launch_bounds__(COLLECT_THREADS) void collect_kernel(CollectArgs ar
 
   const T* a0 = (const T*)d.a + (int64_t)n * d.a_seq_stride + (int64_t)s0 * d.a_tok_stride;
   const T* g0 = (const T*)d.g + (int64_t)n * d.g_seq_stride + (int64_t)s0 * d.g_tok_stride;
-  project_tile<T, PB, ALIGNED>(a0, d.a_tok_stride, rows_valid, d.I, (const T*)d.r_in, p,
-                               d.col_scale, wave, lane, accA);
-  project_tile<T, PB, ALIGNED>(g0, d.g_tok_stride, rows_valid, d.O, (const T*)d.r_out, p,
-                               d.row_scale, wave, lane, accG);
+  project_tile<T, PB, ALIGNED, MT, U>(a0, d.a_tok_stride, rows_valid, d.I, (const T*)d.r_in, p,
+                                      d.col_scale, wave, lane, accA);
+  project_tile<T, PB, ALIGNED, MT, U>(g0, d.g_tok_stride, rows_valid, d.O, (const T*)d.r_out, p,
+                                      d.row_scale, wave, lane, accG);
 
   // ---- combine the 4 K-slices: (w0 + w2) + (w1 + w3), fixed order ----------
   const int r = lane & 15;
@@ -291,24 +292,32 @@ __global__ __launch_bounds__(COLLECT_THREADS) void collect_kernel(CollectArgs ar
   }
 }
 
-// Adds the per-tile partials of each (module, sequence) in tile order, clamps,
-// casts and writes the module's block of the output row.
+// Adds the per-tile partials of each (module, sequence) in a fixed order (four interleaved running
+// sums combined at the end, so that consecutive loads do not wait on each other), clamps, casts and
+// writes the module's block of the output row.
 __global__ __launch_bounds__(256) void collect_finalize_kernel(
     const bgx_module_desc* __restrict__ mods, const float* __restrict__ partials,
     const int32_t* __restrict__ lengths, const int64_t* __restrict__ out_rows, int N, int S, int p,
-    int tiles_per_seq, void* out, int64_t out_row_stride, int out_dtype, float lo, float hi) {
+    int tiles_per_seq, int tile_tokens, void* out, int64_t out_row_stride, int out_dtype, float lo, float hi) {
   const int n = blockIdx.x;
   const int m = blockIdx.y;
   const int pp = p * p;
   const int s_limit = seq_token_limit(lengths, n, S);
-  const int ntiles = (s_limit + TILE_T - 1) / TILE_T;
+  const int ntiles = (s_limit + tile_tokens - 1) / tile_tokens;
   const float* src = partials + ((int64_t)m * N + n) * tiles_per_seq * pp;
   const int64_t row = out_rows ? out_rows[n] : (int64_t)n;
   const int64_t base = row * out_row_stride + mods[m].out_col;
   for (int e = threadIdx.x; e < pp; e += blockDim.x) {
-    float s = 0.f;
-    for (int t = 0; t < ntiles; ++t) s += src[(int64_t)t * pp + e];
-    store_as(out, base + e, clampf(s, lo, hi), out_dtype);
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    int t = 0;
+    for (; t + 4 <= ntiles; t += 4) {
+      s0 += src[(int64_t)(t + 0) * pp + e];
+      s1 += src[(int64_t)(t + 1) * pp + e];
+      s2 += src[(int64_t)(t + 2) * pp + e];
+      s3 += src[(int64_t)(t + 3) * pp + e];
+    }
+    for (; t < ntiles; ++t) s0 += src[(int64_t)t * pp + e];
+    store_as(out, base + e, clampf((s0 + s1) + (s2 + s3), lo, hi), out_dtype);
   }
 }
 
@@ -379,32 +388,37 @@ static size_t desc_bytes(int n_modules) {
   return align_up((size_t)n_modules * sizeof(bgx_module_desc), 256);
 }
 
+constexpr int MIN_TILE_T = 64;  // smallest token tile any kernel variant uses: bounds the partials
+
 size_t collect_workspace_bytes(int n_modules, int N, int S, int p) {
   if (n_modules <= 0 || N <= 0 || S <= 0 || p <= 0) return 0;
-  const size_t tiles = (size_t)((S + TILE_T - 1) / TILE_T);
+  const size_t tiles = (size_t)((S + MIN_TILE_T - 1) / MIN_TILE_T);
   return desc_bytes(n_modules) + (size_t)n_modules * N * tiles * p * p * sizeof(float);
 }
 
-template <typename T, int PB, bool ALIGNED>
+template <typename T, int PB, bool ALIGNED, int MT, int U>
 static void launch_collect(bool per_token, dim3 grid, hipStream_t st, const CollectArgs& args) {
   if (per_token)
-    hipLaunchKernelGGL((collect_kernel<T, PB, ALIGNED, true>), grid, dim3(COLLECT_THREADS), 0, st, args);
+    hipLaunchKernelGGL((collect_kernel<T, PB, ALIGNED, true, MT, U>), grid, dim3(COLLECT_THREADS), 0, st, args);
   else
-    hipLaunchKernelGGL((collect_kernel<T, PB, ALIGNED, false>), grid, dim3(COLLECT_THREADS), 0, st, args);
+    hipLaunchKernelGGL((collect_kernel<T, PB, ALIGNED, false, MT, U>), grid, dim3(COLLECT_THREADS), 0, st, args);
 }
+
+// tokens per workgroup: 128 for the common case (p <= 16, aligned operands), else 64
+static int tile_tokens_for(int pb, bool aligned) { return (pb == 1 && aligned) ? 128 : 64; }
 
 template <typename T>
 static void launch_collect_pb(int pb, bool aligned, bool per_token, dim3 grid, hipStream_t st,
                               const CollectArgs& args) {
   if (pb == 1) {
-    aligned ? launch_collect<T, 1, true>(per_token, grid, st, args)
-            : launch_collect<T, 1, false>(per_token, grid, st, args);
+    aligned ? launch_collect<T, 1, true, 8, 2>(per_token, grid, st, args)
+            : launch_collect<T, 1, false, 4, 2>(per_token, grid, st, args);
   } else if (pb == 2) {
-    aligned ? launch_collect<T, 2, true>(per_token, grid, st, args)
-            : launch_collect<T, 2, false>(per_token, grid, st, args);
+    aligned ? launch_collect<T, 2, true, 4, 2>(per_token, grid, st, args)
+            : launch_collect<T, 2, false, 4, 2>(per_token, grid, st, args);
   } else {
-    aligned ? launch_collect<T, 4, true>(per_token, grid, st, args)
-            : launch_collect<T, 4, false>(per_token, grid, st, args);
+    aligned ? launch_collect<T, 4, true, 4, 1>(per_token, grid, st, args)
+            : launch_collect<T, 4, false, 4, 1>(per_token, grid, st, args);
   }
 }
 
@@ -446,7 +460,14 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
 
   hipStream_t st = (hipStream_t)stream;
   bgx_module_desc* mods_dev = (bgx_module_desc*)ws;
-  BGX_HIP(hipMemcpyAsync(mods_dev, mods_host, (size_t)n_modules * sizeof(bgx_module_desc),
+  // Workgroups are dispatched module by module; putting the modules with the most columns first
+  // leaves the cheapest tiles for the end of the launch, which shortens its tail.  The order has no
+  // effect on the result: every descriptor carries its own output column.
+  std::vector<bgx_module_desc> sorted(mods_host, mods_host + n_modules);
+  std::stable_sort(sorted.begin(), sorted.end(), [](const bgx_module_desc& x, const bgx_module_desc& y) {
+    return (int64_t)x.I + x.O > (int64_t)y.I + y.O;
+  });
+  BGX_HIP(hipMemcpyAsync(mods_dev, sorted.data(), (size_t)n_modules * sizeof(bgx_module_desc),
                          hipMemcpyHostToDevice, st));
 
   CollectArgs args;
@@ -455,7 +476,9 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   args.N = N;
   args.S = S;
   args.p = p;
-  args.tiles_per_seq = (S + TILE_T - 1) / TILE_T;
+  const int pb = (p + 15) / 16;
+  const int tile_tokens = tile_tokens_for(pb, aligned);
+  args.tiles_per_seq = (S + tile_tokens - 1) / tile_tokens;
   args.partials = (float*)((char*)ws + desc_bytes(n_modules));
   args.row_offsets = per_token ? rows_or_offsets : nullptr;
   args.out = out;
@@ -467,7 +490,6 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   const int64_t tiles = (int64_t)N * args.tiles_per_seq;
   BGX_REQUIRE(tiles <= 0x7fffffffLL, BGX_E_SHAPE, "collect: %lld tiles exceed the grid limit", (long long)tiles);
   const dim3 grid((unsigned)tiles, (unsigned)n_modules);
-  const int pb = (p + 15) / 16;
   if (in_dtype == BGX_F32)
     launch_collect_pb<float>(pb, aligned, per_token, grid, st, args);
   else if (in_dtype == BGX_F16)
@@ -478,8 +500,8 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
 
   if (!per_token) {
     hipLaunchKernelGGL(collect_finalize_kernel, dim3((unsigned)N, (unsigned)n_modules), dim3(256), 0, st,
-                       mods_dev, args.partials, lengths, rows_or_offsets, N, S, p, args.tiles_per_seq, out,
-                       out_row_stride, out_dtype, lo, hi);
+                       mods_dev, args.partials, lengths, rows_or_offsets, N, S, p, args.tiles_per_seq, tile_tokens,
+                       out, out_row_stride, out_dtype, lo, hi);
     BGX_HIP(hipGetLastError());
   }
   return 0;
