@@ -89,13 +89,19 @@ class HookCollectorBase(ContextDecorator, ABC):
     mod_grads: dict = field(default_factory=dict)
     save_dtype: torch.dtype = torch.float32
 
+    persistent_hooks = False
+    """When True the forward hooks stay registered between `with` blocks (they do nothing while no block is
+    open) and are removed by `remove_hooks()`; saves re-registering every hook for every batch."""
+
     def __post_init__(self):
         self.rank = dist.get_rank() if dist.is_initialized() else 0
         self.world_size = dist.get_world_size() if dist.is_initialized() else 1
         self._fwd_hooks: list[RemovableHandle] = []
         self._bwd_hooks: list[RemovableHandle] = []
         self._current_collection_mask: Tensor | None = None
-        self._deferred: list[ops.ModuleInput] = []
+        self._deferred: list = []
+        self._prepared: dict[str, ops.PreparedModule] = {}
+        self._active = False
         self._scale_cache: dict[str, tuple[Tensor | None, Tensor | None]] = {}
         self.target_info = self.discover_targets(self.model, self.target_modules, self.processor.include_bias,
                                                  self.filter_modules)
@@ -250,18 +256,32 @@ class HookCollectorBase(ContextDecorator, ABC):
         return self
 
     def __enter__(self):
-        for name in self.target_info:
-            layer = self.model.get_submodule(name)
-            layer._name = name  # type: ignore[attr-defined]
-            layer._collect_bias = self.target_info[name][2]  # type: ignore[attr-defined]
-            self._fwd_hooks.append(layer.register_forward_hook(self._process_input))
-            self._bwd_hooks.append(layer.register_full_backward_hook(self._process_grad))
+        """Activates collection.  A forward hook on every target keeps the module input and attaches a
+        tensor hook to the module output; that hook receives the gradient with respect to the output --
+        what the reference's full backward hook passes as grad_output[0] (collector.py:435-472) -- without
+        the extra autograd nodes a module-level backward hook inserts around every call."""
+        if not self._fwd_hooks:
+            for name in self.target_info:
+                layer = self.model.get_submodule(name)
+                layer._name = name  # type: ignore[attr-defined]
+                layer._collect_bias = self.target_info[name][2]  # type: ignore[attr-defined]
+                self._fwd_hooks.append(layer.register_forward_hook(self._process_input))
+            self._target_layers = [self.model.get_submodule(name) for name in self.target_info]
+        self._active = True
         return self
 
-    def _process_input(self, module: nn.Module, inp: tuple, _):
+    def _process_input(self, module: nn.Module, inp: tuple, out):
+        if not self._active:
+            return
         x = inp[0].detach()
         assert x.ndim == 3, f"Expected input of shape [N, S, I], got {x.shape}"
         self.forward_hook(module, x)
+        if isinstance(out, Tensor) and out.requires_grad:
+            out.register_hook(functools.partial(self._on_output_grad, module))
+
+    def _on_output_grad(self, module: nn.Module, grad: Tensor) -> None:
+        if self._active:
+            self._process_grad(module, None, (grad,))
 
     def _process_grad(self, module: nn.Module, _, grad_out):
         assert isinstance(module, LayerAdapter.supported_modules), (
@@ -271,18 +291,24 @@ class HookCollectorBase(ContextDecorator, ABC):
         if hasattr(module, "_inputs"):
             del module._inputs
 
-    def __exit__(self, exc_type, exc, tb):
-        for layer in self.model.modules():
-            if hasattr(layer, "_inputs"):
-                del layer._inputs
-            if hasattr(layer, "_name"):
-                del layer._name
+    def remove_hooks(self) -> None:
+        """Detach from the model: remove the hooks and the attributes set on the target layers."""
         for h in self._fwd_hooks:
             h.remove()
-        for h in self._bwd_hooks:
-            h.remove()
         self._fwd_hooks.clear()
-        self._bwd_hooks.clear()
+        for layer in getattr(self, "_target_layers", []):
+            for attr in ("_inputs", "_name", "_collect_bias"):
+                if hasattr(layer, attr):
+                    delattr(layer, attr)
+        self._active = False
+
+    def __exit__(self, exc_type, exc, tb):
+        self._active = False
+        for layer in getattr(self, "_target_layers", []):
+            if hasattr(layer, "_inputs"):
+                del layer._inputs
+        if not self.persistent_hooks:
+            self.remove_hooks()
         if exc_type is not None:
             self._deferred.clear()  # a failed batch leaves nothing queued; otherwise process_batch launches
         return False
@@ -369,8 +395,17 @@ class HookCollectorBase(ContextDecorator, ABC):
 
     # ---- deferred (one launch per batch) -----------------------------------------------------
     def defer_module(self, module: nn.Module, g: Tensor, out_col: int) -> None:
-        """Queue `module` for `launch_deferred`; keeps a and g alive until then."""
-        self._deferred.append(self.module_input(module, g, out_col))
+        """Queue `module` for `launch_deferred`; keeps a and g alive until then.  Everything about the
+        module that does not change between batches (projection matrices, factor vectors, output column)
+        is resolved and checked on its first batch only."""
+        name: str = module._name  # type: ignore[assignment]
+        prepared = self._prepared.get(name)
+        if prepared is None or prepared.dtype != g.dtype or prepared.out_col != out_col:
+            prepared = ops.PreparedModule(self.module_input(module, g, out_col), self.per_module_projection_dim)
+            self._prepared[name] = prepared
+        a = module._inputs
+        assert isinstance(a, Tensor), "Activation cache missing for module"
+        self._deferred.append((prepared, a, g))
 
     def launch_deferred(self, out: Tensor, *, lengths: Tensor | None = None, out_rows: Tensor | None = None,
                         row_offsets: Tensor | None = None) -> None:
@@ -382,10 +417,9 @@ class HookCollectorBase(ContextDecorator, ABC):
         try:
             if self.attribute_tokens:
                 assert lengths is not None and row_offsets is not None
-                ops.collect_tok(self._deferred, p, out, lengths=lengths, row_offsets=row_offsets, lo=self.lo,
-                                hi=self.hi)
+                ops.collect_prepared(True, self._deferred, p, out, lengths, row_offsets, self.lo, self.hi)
             else:
-                ops.collect_seq(self._deferred, p, out, lengths=lengths, out_rows=out_rows, lo=self.lo, hi=self.hi)
+                ops.collect_prepared(False, self._deferred, p, out, lengths, out_rows, self.lo, self.hi)
         finally:
             self._deferred.clear()
 
@@ -430,6 +464,7 @@ class CollectorComputer:
                 losses = self.forward_backward(self.model, x, y, batch)
             self.collector.process_batch(indices, losses=losses)
         self.collector.teardown()
+        self.collector.remove_hooks()
         if dist.is_initialized():
             dist.all_reduce(total_processed, op=dist.ReduceOp.SUM)
         if self.rank == 0 and self.cfg.run_path:
@@ -443,6 +478,8 @@ def fwd_bwd_factory(cfg: IndexConfig) -> Callable:
     if cfg.loss_fn != "ce":
         raise NotImplementedError("only the cross-entropy loss is supported (loss_fn='kl' needs PEFT)")
 
+    trainable: dict[int, list] = {}
+
     def fwd_bwd(model, x: Tensor, y: Tensor, batch: dict):
         logits = model(x).logits[:, :-1]
         masks = y[:, 1:] != -100
@@ -453,7 +490,12 @@ def fwd_bwd_factory(cfg: IndexConfig) -> Callable:
         if "advantage" in batch:
             losses *= torch.tensor(batch["advantage"], device=losses.device)
         losses.sum().backward()
-        model.zero_grad()
+        # model.zero_grad(): only parameters that require grad can hold one; the list is built once
+        params = trainable.get(id(model))
+        if params is None:
+            params = trainable[id(model)] = [q for q in model.parameters() if q.requires_grad]
+        for q in params:
+            q.grad = None
         return losses
 
     return fwd_bwd

@@ -26,6 +26,8 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
                  int out_dtype, float lo, float hi, void* ws, size_t ws_bytes, void* stream);
 int adafactor_scales_impl(const float* row, int O, const float* col, int I, int dtype, float* row_scale,
                           float* col_scale, void* stream);
+int collect_timing_enable(int max_launches);
+int collect_timing_read(float* ms_out, int capacity, int* count_out);
 int unit_normalize_impl(void* rows, int64_t n_rows, int64_t D, int64_t stride, int dtype, void* stream);
 size_t scan_workspace_bytes(int Q, int k, int64_t chunk_rows);
 int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int dtype, const void* queries, int Q,
@@ -64,6 +66,12 @@ int bgx_collect_tok(const bgx_module_desc* mods_host, int32_t n_modules, int32_t
                     size_t workspace_bytes, void* stream) {
   return bgx::collect_impl(true, mods_host, n_modules, N, S, p, in_dtype, lengths_dev, row_offsets_dev, out_dev,
                            out_row_stride, out_dtype, clamp_lo, clamp_hi, workspace_dev, workspace_bytes, stream);
+}
+
+int bgx_collect_timing_enable(int32_t max_launches) { return bgx::collect_timing_enable(max_launches); }
+
+int bgx_collect_timing_read(float* ms_out, int32_t capacity, int32_t* count_out) {
+  return bgx::collect_timing_read(ms_out, capacity, count_out);
 }
 
 int bgx_unit_normalize_rows(void* rows_dev, int64_t n_rows, int64_t D, int64_t row_stride, int32_t dtype,

@@ -382,6 +382,34 @@ __global__ __launch_bounds__(256) void unit_normalize_kernel(T* rows, int64_t n_
 }
 
 // ---- host side ------------------------------------------------------------------------
+// Optional event pairs around collect_kernel (benchmark support).
+static std::vector<hipEvent_t> g_timing_events;  // start0, stop0, start1, stop1, ...
+static int g_timing_used = 0;
+
+int collect_timing_enable(int max_launches) {
+  for (hipEvent_t e : g_timing_events) (void)hipEventDestroy(e);
+  g_timing_events.clear();
+  g_timing_used = 0;
+  BGX_REQUIRE(max_launches >= 0, BGX_E_ARG, "collect_timing_enable: max_launches=%d", max_launches);
+  for (int i = 0; i < 2 * max_launches; ++i) {
+    hipEvent_t e;
+    BGX_HIP(hipEventCreate(&e));
+    g_timing_events.push_back(e);
+  }
+  return 0;
+}
+
+int collect_timing_read(float* ms_out, int capacity, int* count_out) {
+  BGX_REQUIRE(ms_out && count_out && capacity >= 0, BGX_E_ARG, "collect_timing_read: null output");
+  const int n = g_timing_used < capacity ? g_timing_used : capacity;
+  for (int i = 0; i < n; ++i) {
+    BGX_HIP(hipEventSynchronize(g_timing_events[2 * i + 1]));
+    BGX_HIP(hipEventElapsedTime(&ms_out[i], g_timing_events[2 * i], g_timing_events[2 * i + 1]));
+  }
+  *count_out = n;
+  return 0;
+}
+
 static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 static size_t desc_bytes(int n_modules) {
@@ -490,6 +518,8 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   const int64_t tiles = (int64_t)N * args.tiles_per_seq;
   BGX_REQUIRE(tiles <= 0x7fffffffLL, BGX_E_SHAPE, "collect: %lld tiles exceed the grid limit", (long long)tiles);
   const dim3 grid((unsigned)tiles, (unsigned)n_modules);
+  const bool timed = 2 * (g_timing_used + 1) <= (int)g_timing_events.size();
+  if (timed) BGX_HIP(hipEventRecord(g_timing_events[2 * g_timing_used], st));
   if (in_dtype == BGX_F32)
     launch_collect_pb<float>(pb, aligned, per_token, grid, st, args);
   else if (in_dtype == BGX_F16)
@@ -497,6 +527,10 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   else
     launch_collect_pb<bf16_t>(pb, aligned, per_token, grid, st, args);
   BGX_HIP(hipGetLastError());
+  if (timed) {
+    BGX_HIP(hipEventRecord(g_timing_events[2 * g_timing_used + 1], st));
+    ++g_timing_used;
+  }
 
   if (!per_token) {
     hipLaunchKernelGGL(collect_finalize_kernel, dim3((unsigned)N, (unsigned)n_modules), dim3(256), 0, st,

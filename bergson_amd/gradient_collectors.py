@@ -47,8 +47,8 @@ class _DeferredBatchMixin:
         block = RowBlock()
         if not self._deferred:
             return block
-        dev = self._deferred[0].g.device
-        N = self._deferred[0].g.shape[0]
+        dev = self._deferred[0][2].device
+        N = self._deferred[0][2].shape[0]
         assert N == len(indices), f"batch of {N} sequences but {len(indices)} indices"
         lengths = self._batch_lengths(dev) if (self.attribute_tokens or self.skip_padding) else None
         direct = builder is not None and builder.direct and not need_rows
@@ -84,6 +84,8 @@ class _DeferredBatchMixin:
 @dataclass(kw_only=True)
 class GradientCollector(_DeferredBatchMixin, HookCollectorBase):
     """Collects per-sample (or per-token) projected gradients and writes them to a store, or scores them."""
+
+    persistent_hooks = True
 
     data: object
     cfg: IndexConfig
@@ -147,6 +149,7 @@ class GradientCollector(_DeferredBatchMixin, HookCollectorBase):
     def teardown(self):
         if dist.is_initialized():
             dist.reduce(self.per_doc_losses, dst=0)
+        self.remove_hooks()
         if self.builder:
             self.builder.teardown()
         if self.rank == 0 and self.cfg.run_path:

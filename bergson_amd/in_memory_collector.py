@@ -24,6 +24,8 @@ from .utils import get_gradient_dtype, numpy_to_tensor
 
 @dataclass(kw_only=True)
 class InMemoryCollector(_DeferredBatchMixin, HookCollectorBase):
+    persistent_hooks = True
+
     data: object
     cfg: IndexConfig
     skip_hessians: bool = True
@@ -78,6 +80,7 @@ class InMemoryCollector(_DeferredBatchMixin, HookCollectorBase):
         self.per_doc_losses[indices] = losses.detach().type_as(self.per_doc_losses)
 
     def teardown(self) -> None:
+        self.remove_hooks()
         if dist.is_initialized():
             dist.reduce(self.per_doc_losses, dst=0)
         grad_sizes = {name: math.prod(s) for name, s in self.shapes().items()}

@@ -54,6 +54,23 @@ def _workspace(device: torch.device, nbytes: int, tag: str) -> Tensor:
     return ws
 
 
+def collect_timing_start(max_launches: int) -> None:
+    """Record an event pair around the collection kernel of the next `max_launches` launches."""
+    _lib.check(_lib.load().bgx_collect_timing_enable(max_launches), "bgx_collect_timing_enable")
+
+
+def collect_timing_stop() -> list[float]:
+    """Kernel-only durations (ms) of the launches recorded since `collect_timing_start`."""
+    lib = _lib.load()
+    cap = 1 << 16
+    buf = (C.c_float * cap)()
+    n = C.c_int32(0)
+    _lib.check(lib.bgx_collect_timing_read(buf, cap, C.byref(n)), "bgx_collect_timing_read")
+    out = [float(buf[i]) for i in range(n.value)]
+    _lib.check(lib.bgx_collect_timing_enable(0), "bgx_collect_timing_enable")
+    return out
+
+
 def adafactor_scales(row: Tensor | None, col: Tensor | None, dtype: torch.dtype) -> tuple[Tensor | None, Tensor | None]:
     """(row_scale [O], col_scale [I]) fp32 vectors of Adafactor factors rounded to `dtype`."""
     lib = _lib.load()
@@ -154,6 +171,88 @@ def _collect(per_token: bool, modules: list[ModuleInput], p: int, out: Tensor, l
         ev1.record()
         esz = 4 if in_dtype == torch.float32 else 2
         timer.append((ev0, ev1, sum(int(N) * int(S) * (d.I + d.O) * esz for d in descs)))
+    del keep
+
+
+class PreparedModule:
+    """The batch-independent part of a module's descriptor, validated once.
+
+    `fill` completes a descriptor with the (a, g) of one batch; only what can change between batches is
+    checked there.
+    """
+
+    def __init__(self, m: ModuleInput, p: int):
+        I, O = m.a.shape[2], m.g.shape[2]
+        self.dtype = m.a.dtype
+        self.I, self.O, self.p, self.out_col = I, O, p, m.out_col
+        self.r_in = m.r_in.contiguous()
+        self.r_out = m.r_out.contiguous()
+        if self.r_in.shape != (p, I) or self.r_out.shape != (p, O):
+            raise ValueError(f"projection shapes {tuple(self.r_in.shape)} / {tuple(self.r_out.shape)} do not match "
+                             f"p={p} I={I} O={O}")
+        if self.r_in.dtype != self.dtype or self.r_out.dtype != self.dtype or m.g.dtype != self.dtype:
+            raise TypeError("activations, gradients and projection matrices must share one dtype")
+        for s, n, k in ((m.col_scale, "col_scale", I), (m.row_scale, "row_scale", O)):
+            if s is not None and (s.dtype != torch.float32 or s.numel() != k or not s.is_contiguous()):
+                raise ValueError(f"{n} must be a contiguous fp32 vector of {k} elements")
+        for t in (m.a, m.g, self.r_in, self.r_out):
+            _need_gpu(t, "module operand")
+        self.col_scale, self.row_scale = m.col_scale, m.row_scale
+        d = ModuleDesc()
+        d.r_in, d.r_out = self.r_in.data_ptr(), self.r_out.data_ptr()
+        d.col_scale = None if m.col_scale is None else m.col_scale.data_ptr()
+        d.row_scale = None if m.row_scale is None else m.row_scale.data_ptr()
+        d.bias_col = None
+        d.bias_scale = None
+        d.out_col, d.I, d.O = m.out_col, I, O
+        self.template = d
+
+
+def collect_prepared(per_token: bool, items: list, p: int, out: Tensor, lengths: Tensor | None,
+                     rows: Tensor | None, lo: float, hi: float) -> None:
+    """Fused launch over `items` = [(PreparedModule, a, g), ...] of one batch."""
+    lib = _lib.load()
+    _need_gpu(out, "out")
+    if out.dim() != 2 or out.stride(1) != 1:
+        raise ValueError("out must be a 2-D tensor with contiguous rows")
+    n = len(items)
+    N, S = items[0][1].shape[:2]
+    in_dtype = items[0][0].dtype
+    descs = (ModuleDesc * n)()
+    keep = []
+    nbytes_alg = 0
+    for i, (pm, a, g) in enumerate(items):
+        if a.stride(2) != 1:
+            a = a.contiguous()
+        if g.stride(2) != 1:
+            g = g.contiguous()
+        if a.shape != (N, S, pm.I) or g.shape != (N, S, pm.O) or a.dtype != in_dtype or g.dtype != in_dtype \
+                or pm.p != p:
+            raise ValueError(f"module {i}: a {tuple(a.shape)} {a.dtype} / g {tuple(g.shape)} {g.dtype} do not match "
+                             f"[N={N}, S={S}], I={pm.I}, O={pm.O}, {in_dtype}")
+        keep.append(a)
+        keep.append(g)
+        C.memmove(C.byref(descs[i]), C.byref(pm.template), C.sizeof(ModuleDesc))
+        d = descs[i]
+        d.a, d.g = a.data_ptr(), g.data_ptr()
+        d.a_seq_stride, d.a_tok_stride = a.stride(0), a.stride(1)
+        d.g_seq_stride, d.g_tok_stride = g.stride(0), g.stride(1)
+        nbytes_alg += pm.I + pm.O
+    for t, name, dt in ((lengths, "lengths", torch.int32), (rows, "rows", torch.int64)):
+        if t is not None and (t.dtype != dt or t.numel() != N or not t.is_contiguous() or not t.is_cuda):
+            raise ValueError(f"{name} must be a contiguous {dt} GPU vector of N={N} elements")
+    ws = _workspace(out.device, lib.bgx_collect_workspace_bytes(n, N, S, p), "collect")
+    fn = lib.bgx_collect_tok if per_token else lib.bgx_collect_seq
+    timer = collect_timer
+    if timer is not None:
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+    rc = fn(descs, n, N, S, p, dtype_code(in_dtype), _ptr(lengths), _ptr(rows), _ptr(out), out.stride(0),
+            dtype_code(out.dtype), lo, hi, _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "bgx_collect_tok" if per_token else "bgx_collect_seq")
+    if timer is not None:
+        ev1.record()
+        timer.append((ev0, ev1, int(N) * int(S) * nbytes_alg * (4 if in_dtype == torch.float32 else 2)))
     del keep
 
 

@@ -133,6 +133,17 @@ int bgx_collect_tok(const bgx_module_desc* mods_host, int32_t n_modules,
                     float clamp_lo, float clamp_hi, void* workspace_dev,
                     size_t workspace_bytes, void* stream);
 
+/* Benchmark support (no counterpart in the reference): while enabled, every
+ * bgx_collect_seq / bgx_collect_tok call records a HIP event pair immediately
+ * around its collect_kernel launch, on the launch stream, so that the kernel's
+ * own duration can be read without a profiler.
+ *   bgx_collect_timing_enable(n)  n > 0: start recording, at most n launches;
+ *                                 n = 0: stop and release the events
+ *   bgx_collect_timing_read(ms, capacity, &count): waits for the recorded
+ *       events and writes each launch's kernel time in milliseconds. */
+int bgx_collect_timing_enable(int32_t max_launches);
+int bgx_collect_timing_read(float* ms_out, int32_t capacity, int32_t* count_out);
+
 /* In-place unit normalisation of rows: g * rsqrt(max(sum g^2, eps_fp32^2)),
  * replaces bergson/builder.py:14,:28-30.  rows_dev [n_rows, D], row stride in
  * elements. */
