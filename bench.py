@@ -34,6 +34,9 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes moved per algorithmic byte by collect_kernel on this workload, from the FETCH_SIZE and
+# WRITE_SIZE hardware counters (profiles/collect_kernel_pythia160m_pmc_traffic.txt)
+COLLECT_TRAFFIC_RATIO = 1.066
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
@@ -49,6 +52,9 @@ def parse_args():
     ap.add_argument("--scan-rows", type=int, default=1_000_000)
     ap.add_argument("--scan-queries", type=int, default=1024)
     ap.add_argument("--cpu-sample-tokens", type=int, default=32768)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 1 GiB device copy (reads 1 GiB, writes 1 GiB): the known-size "
+                         "kernel that hardware byte counters are scaled by")
     return ap.parse_args()
 
 
@@ -226,6 +232,13 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
+    if args.copy_calibration:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=device)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
     coll, docs, lengths = collection_leg(args, torch, device)
     scan = None if args.no_scan else scan_leg(args, torch, device)
     cpu = None if args.no_cpu_baseline else cpu_baseline_leg(args, torch, docs, lengths)
@@ -261,7 +274,8 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": coll["achieved_gbs"] / HBM_PEAK_GBS,
-            "traffic": None,
+            "traffic": coll["kernel_bytes_per_launch"] * COLLECT_TRAFFIC_RATIO,
+            "traffic_source": "bytes_per_launch x 1.066 (rocprofv3 FETCH_SIZE + WRITE_SIZE, profiles/)",
             "bytes_per_launch": coll["kernel_bytes_per_launch"],
             "ms_per_launch": coll["kernel_ms_per_launch"],
             "ms_per_launch_with_descriptor_copy_and_finalize": coll["bracket_ms_per_launch"],

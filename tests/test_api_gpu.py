@@ -1,0 +1,179 @@
+"""The reference-shaped classes (Scorer, Attributor, InMemoryCollector, head splitting, Builder options)
+on the GPU against the CPU oracle."""
+import json
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import rel_l2
+from oracle import hooks as ohooks
+from oracle import loop as oloop
+from oracle import scan as oscan
+from oracle import store as ostore
+from oracle.projection import module_projections, projection_matrix
+
+pytestmark = pytest.mark.gpu
+
+
+def _proc(p, normalizers=None):
+    from bergson_amd import GradientProcessor
+
+    return GradientProcessor(normalizers=normalizers or {}, projection_dim=p, projection_type="normal")
+
+
+def _setup(device, lengths, layers=2, seed=11):
+    from bergson_amd import allocate_batches
+    from bergson_amd.synthetic import ListDataset, make_gpt_neox, random_docs
+
+    docs = random_docs(lengths, seed=seed)
+    batches = allocate_batches(lengths, 96)
+    cpu = make_gpt_neox("pythia-14m", torch.float32, "cpu", seed=0, layers=layers)
+    gpu = make_gpt_neox("pythia-14m", torch.float32, device, seed=0, layers=layers)
+    return docs, ListDataset(docs), batches, cpu, gpu
+
+
+def test_in_memory_collector_and_unit_normalize(device):
+    from bergson_amd import IndexConfig, InMemoryCollector, PreprocessConfig
+    from bergson_amd.collector import CollectorComputer
+
+    lengths = [40, 22, 31, 17, 48]
+    docs, data, batches, cpu, gpu = _setup(device, lengths)
+    want, _ = oloop.collect(cpu, cpu.base_model, docs, batches, p=16, unit_normalize=True)
+    cfg = IndexConfig(projection_dim=16, projection_type="normal")
+    col = InMemoryCollector(model=gpu.base_model, cfg=cfg, data=data, processor=_proc(16),
+                            preprocess_cfg=PreprocessConfig(unit_normalize=True))
+    CollectorComputer(model=gpu, data=data, collector=col, batches=batches, cfg=cfg).run_with_collector_hooks()
+    assert list(col.gradients) == list(oloop.target_linears(cpu.base_model))
+    got = torch.cat([col.gradients[n] for n in col.gradients], 1)
+    assert got.shape == want.shape
+    torch.testing.assert_close(got.norm(dim=1), torch.ones(5), rtol=1e-4, atol=1e-4)
+    assert rel_l2(got, want) <= 1e-3
+
+
+@pytest.mark.parametrize("aggregation", ["mean", "sum"])
+def test_aggregated_store(device, tmp_path, aggregation):
+    from bergson_amd import IndexConfig, PreprocessConfig, collect_gradients, load_gradients
+
+    lengths = [40, 22, 31, 17]
+    docs, data, batches, cpu, gpu = _setup(device, lengths)
+    rows, _ = oloop.collect(cpu, cpu.base_model, docs, batches, p=16)
+    want = rows.sum(0, keepdim=True) if aggregation == "sum" else rows.mean(0, keepdim=True)
+    cfg = IndexConfig(run_path=str(tmp_path / "agg"), projection_dim=16, projection_type="normal")
+    collect_gradients(gpu, data, _proc(16), cfg, batches=batches,
+                      preprocess_cfg=PreprocessConfig(aggregation=aggregation))
+    info = json.loads((cfg.partial_run_path / "info.json").read_text())
+    assert info["num_grads"] == 1 and info["base_dtype"] == "float32"
+    got = torch.from_numpy(np.array(load_gradients(cfg.partial_run_path)))
+    assert rel_l2(got, want) <= 1e-3
+
+
+def test_attention_head_split(device):
+    """Per-head rows: each head projects its slice of g with its own left matrix and shares the
+    parent's input-side matrix; with Adafactor its row factor uses the mean over its own rows."""
+    from bergson_amd import AdafactorNormalizer, AttentionConfig, GradientCollector, IndexConfig
+    from bergson_amd.collector import CollectorComputer
+
+    lengths = [30, 30]
+    docs, data, batches, cpu, gpu = _setup(device, lengths, layers=1)
+    name = "layers.0.attention.dense"
+    heads, hs = 4, 32
+    gen = torch.Generator().manual_seed(0)
+    row, colm = torch.rand(128, generator=gen) + 0.1, torch.rand(128, generator=gen) + 0.1
+    cap = {}
+    mod = gpu.base_model.get_submodule(name)
+    h1 = mod.register_forward_hook(lambda m, i, o: cap.__setitem__("a", i[0].detach().cpu()))
+    h2 = mod.register_full_backward_hook(lambda m, gi, go: cap.__setitem__("g", go[0].detach().cpu()))
+    cfg = IndexConfig(projection_dim=16, projection_type="normal")
+    col = GradientCollector(model=gpu.base_model, cfg=cfg, data=data, target_modules={name},
+                            processor=_proc(16, {name: AdafactorNormalizer(row.to(device), colm.to(device))}),
+                            attention_cfgs={name: AttentionConfig(heads, hs, 2)})
+    assert list(col.shapes()) == [f"{name}.head_{h}" for h in range(heads)]
+    CollectorComputer(model=gpu, data=data, collector=col, batches=[[0, 1]], cfg=cfg).run_with_collector_hooks()
+    h1.remove(), h2.remove()
+    got = torch.from_numpy(np.array(col.builder.grad_buffer))
+    assert got.shape == (2, heads * 256)
+    a, g = cap["a"], cap["g"]
+    right = projection_matrix(f"{name}/right", 16, 128, torch.float32)
+    stash = ohooks.forward_hook(a, ohooks.Adafactor(row, colm), right)
+    for h in range(heads):
+        left = projection_matrix(f"{name}.head_{h}/left", 16, hs, torch.float32)
+        norm_h = ohooks.Adafactor(row[h * hs:(h + 1) * hs], colm)
+        want = ohooks.backward_hook(stash, g[:, :, h * hs:(h + 1) * hs], norm_h, left, right)
+        assert rel_l2(got[:, h * 256:(h + 1) * 256], want) <= 1e-4
+
+
+def test_scorer_on_the_fly_matches_oracle(device, tmp_path):
+    from bergson_amd import IndexConfig, Scorer, collect_gradients
+    from bergson_amd.data import load_scores
+    from bergson_amd.score_writer import MemmapSequenceScoreWriter
+
+    lengths = [40, 22, 31, 17, 48, 12]
+    docs, data, batches, cpu, gpu = _setup(device, lengths)
+    rows, _ = oloop.collect(cpu, cpu.base_model, docs, batches, p=16)
+    mods = list(oloop.target_linears(cpu.base_model))
+    sizes = {m: 256 for m in mods}
+    cols = ostore.column_offsets(sizes)
+    index = {m: rows[:, lo:hi] for m, (lo, hi) in cols.items()}
+    gen = torch.Generator().manual_seed(5)
+    queries = {m: torch.randn(3, 256, generator=gen) for m in mods}
+    qn = oscan.normalize_and_aggregate_queries(queries, mods, unit_normalize=True)
+    want = oscan.scorer_score(index, qn, mods, unit_normalize=True)
+    want_near = oscan.scorer_score(index, qn, mods, unit_normalize=True, score_mode="nearest")
+
+    for mode, ref, width in (("individual", want, 3), ("nearest", want_near, 1)):
+        path = tmp_path / mode
+        writer = MemmapSequenceScoreWriter(path, len(docs), width)
+        scorer = Scorer(qn, mods, writer, device, torch.float32, unit_normalize=True, score_mode=mode)
+        cfg = IndexConfig(projection_dim=16, projection_type="normal")
+        collect_gradients(gpu, data, _proc(16), cfg, batches=batches, scorer=scorer)
+        writer.flush()
+        sc = load_scores(path)
+        assert sc.is_written()
+        got = torch.from_numpy(np.array(sc[:]))
+        assert got.shape == ref.shape
+        assert (got - ref).abs().max().item() <= 1e-3
+
+
+def test_attributor_search_and_trace(device, tmp_path):
+    from bergson_amd import Attributor, IndexConfig, collect_gradients
+
+    lengths = [40, 22, 31, 17, 48, 12, 25, 36]
+    docs, data, batches, cpu, gpu = _setup(device, lengths)
+    cfg = IndexConfig(run_path=str(tmp_path / "idx"), projection_dim=16, projection_type="normal")
+    collect_gradients(gpu, data, _proc(16), cfg, batches=batches)
+    rows, _ = oloop.collect(cpu, cpu.base_model, docs, batches, p=16)
+    mods = list(oloop.target_linears(cpu.base_model))
+    cols = ostore.column_offsets({m: 256 for m in mods})
+    index = {m: rows[:, lo:hi] for m, (lo, hi) in cols.items()}
+
+    attr = Attributor(cfg.partial_run_path, device="cuda:0", unit_norm=True)
+    assert attr.N == len(docs) and attr.ordered_modules == mods
+    queries = {m: index[m][[1, 6]] for m in mods}
+    vals, idx = attr.search({m: q.to(device) for m, q in queries.items()}, k=3)
+    ref_v, ref_i = oscan.attributor_search(index, queries, mods, 3, unit_norm=True)
+    assert idx[:, 0].tolist() == [1, 6] and (vals[:, 0] > 0.999).all()
+    assert torch.equal(idx.cpu(), ref_i)
+    assert (vals.cpu() - ref_v).abs().max().item() <= 1e-3
+    rv, ri = attr.search({m: q.to(device) for m, q in queries.items()}, k=2, reverse=True)
+    ref_rv, ref_ri = oscan.attributor_search(index, queries, mods, 2, unit_norm=True, reverse=True)
+    assert torch.equal(ri.cpu(), ref_ri) and (rv.cpu() - ref_rv).abs().max().item() <= 1e-3
+    # a subset of modules: the other modules' query columns do not contribute
+    sub = set(mods[:3])
+    sv, si = attr.search({m: q.to(device) for m, q in queries.items()}, k=4, modules=sub)
+    norm_i = oscan.attributor_normalize_index({m: index[m] for m in mods}, mods)
+    qcat = torch.cat([queries[m] for m in mods], 1)
+    qnorm = {m: queries[m] / (qcat.norm(dim=1, keepdim=True) + torch.finfo(torch.float32).eps) for m in mods}
+    ref_sub = sum(qnorm[m] @ norm_i[m].T for m in mods[:3])
+    rsv, rsi = torch.topk(ref_sub, 4, dim=1)
+    assert torch.equal(si.cpu(), rsi) and (sv.cpu() - rsv).abs().max().item() <= 1e-3
+
+    # trace(): the gradient of document 3's loss finds document 3
+    from bergson_amd import pad_and_tensor
+    with attr.trace(gpu.base_model, 2) as result:
+        x, y, _, _ = pad_and_tensor([docs[3]], device=device, sync_max_len=False)
+        logits = gpu(x).logits[:, :-1]
+        loss = torch.nn.functional.cross_entropy(logits.reshape(-1, logits.size(-1)), y[:, 1:].flatten(), reduction="sum")
+        loss.backward()
+        gpu.zero_grad()
+    assert result.indices[0, 0].item() == 3 and result.scores[0, 0].item() > 0.99
