@@ -243,32 +243,35 @@ __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
   };
 
   const int KT = (int)((D + BK - 1) / BK);
+  // Pipeline: while the MFMAs of K tile kt run from LDS buffer kt&1, the registers that hold tile kt+1
+  // are written to the other buffer and the global loads of tile kt+2 are issued; one barrier per tile.
   gload(0);
   lstore(0);
+  if (KT > 1) gload(1);
   __syncthreads();
 
   const int fr = lane & 31;
   const int fh = lane >> 5;
+  auto mma_step = [&](const unsigned char* gb, const unsigned char* qb, int kk) {
+    uint4 af[TM], bf[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const uint4*>(gb + i * 32 * LDS_ROW_BYTES + kk * 32);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const uint4*>(qb + j * 32 * LDS_ROW_BYTES + kk * 32);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) M::mma(af[i], bf[j], acc[i][j]);
+  };
   for (int kt = 0; kt < KT; ++kt) {
     const int buf = kt & 1;
-    if (kt + 1 < KT) gload(kt + 1);
     const unsigned char* gb = smem + buf * BUF_BYTES + (wm * WTM + fr) * LDS_ROW_BYTES + fh * 16;
     const unsigned char* qb = smem + buf * BUF_BYTES + (BM + wn * WTN + fr) * LDS_ROW_BYTES + fh * 16;
-#pragma unroll
-    for (int kk = 0; kk < TILE_CHUNKS / 2; ++kk) {
-      uint4 af[TM], bf[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        af[i] = *reinterpret_cast<const uint4*>(gb + i * 32 * LDS_ROW_BYTES + kk * 32);
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        bf[j] = *reinterpret_cast<const uint4*>(qb + j * 32 * LDS_ROW_BYTES + kk * 32);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) M::mma(af[i], bf[j], acc[i][j]);
-    }
+    mma_step(gb, qb, 0);
     if (kt + 1 < KT) lstore(buf ^ 1);
+    if (kt + 2 < KT) gload(kt + 2);
+#pragma unroll
+    for (int kk = 1; kk < TILE_CHUNKS / 2; ++kk) mma_step(gb, qb, kk);
     __syncthreads();
   }
 
@@ -514,10 +517,11 @@ template <typename T>
 static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
   // large tiles when there is enough work to fill the chip with them
   if (a.Q > 64 && a.rows >= 4096) {
+    // 8 waves, each 128 x 64: two waves per SIMD hide each other's LDS and barrier stalls
     constexpr int BM = 256, BN = 256;
     a.row_tiles = (int)((a.rows + BM - 1) / BM);
     a.q_tiles = (a.Q + BN - 1) / BN;
-    return launch_gemm<T, BM, BN, 2, 2>(a, aligned, st);
+    return launch_gemm<T, BM, BN, 2, 4>(a, aligned, st);
   } else if (a.Q > 32) {
     constexpr int BM = 128, BN = 64;
     a.row_tiles = (int)((a.rows + BM - 1) / BM);
