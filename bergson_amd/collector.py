@@ -101,6 +101,8 @@ class HookCollectorBase(ContextDecorator, ABC):
         self._current_collection_mask: Tensor | None = None
         self._deferred: list = []
         self._prepared: dict[str, ops.PreparedModule] = {}
+        self._adam_prepared: dict[str, ops.AdamPrepared] = {}
+        self._deferred_adam: list = []
         self._active = False
         self._scale_cache: dict[str, tuple[Tensor | None, Tensor | None]] = {}
         self.target_info = self.discover_targets(self.model, self.target_modules, self.processor.include_bias,
@@ -309,8 +311,9 @@ class HookCollectorBase(ContextDecorator, ABC):
                 del layer._inputs
         if not self.persistent_hooks:
             self.remove_hooks()
-        if exc_type is not None:
-            self._deferred.clear()  # a failed batch leaves nothing queued; otherwise process_batch launches
+        if exc_type is not None:  # a failed batch leaves nothing queued; otherwise process_batch launches
+            self._deferred.clear()
+            self._deferred_adam.clear()
         return False
 
     # ---- the hook pair -----------------------------------------------------------------------
@@ -357,8 +360,7 @@ class HookCollectorBase(ContextDecorator, ABC):
         if module._collect_bias:
             raise NotImplementedError(f"{name}: include_bias=True has no HIP kernel in this build")
         if isinstance(normalizer, AdamNormalizer):
-            raise NotImplementedError(f"{name}: AdamNormalizer has no HIP kernel in this build; "
-                                      "convert with .to_adafactor() or drop the normalizer")
+            raise AssertionError("Adam modules go through adam_prepared()")
         if not a.is_cuda or not g.is_cuda:
             raise RuntimeError("bergson_amd has no CPU path: the model must run on the GPU")
         # an attention head shares the parent's input and right projection (collector.py:527, :540)
@@ -372,13 +374,55 @@ class HookCollectorBase(ContextDecorator, ABC):
         return ops.ModuleInput(a=a, g=g, r_in=r_in, r_out=r_out, out_col=out_col, col_scale=col_scale,
                                row_scale=row_scale)
 
+    def adam_prepared(self, module: nn.Module, g: Tensor, out_col: int) -> "ops.AdamPrepared":
+        """The module's Adam table and projections, built on its first batch (collector.py:609-644)."""
+        name: str = module._name  # type: ignore[assignment]
+        key = f"{name}|{g.dtype}|{out_col}"
+        prep = self._adam_prepared.get(key)
+        if prep is not None:
+            return prep
+        p = self.per_module_projection_dim
+        if p is None:
+            raise NotImplementedError("bergson_amd collects projected gradients only: set processor.projection_dim")
+        if module._collect_bias:
+            raise NotImplementedError(f"{name}: include_bias=True has no HIP kernel in this build")
+        if not g.is_cuda:
+            raise RuntimeError("bergson_amd has no CPU path: the model must run on the GPU")
+        normalizer = self.normalizer_for(name)
+        assert isinstance(normalizer, AdamNormalizer)
+        i = getattr(module, LayerAdapter.in_attr(module))
+        o = getattr(module, LayerAdapter.out_attr(module))
+        parent = self.split_head_name(name)
+        right_name = parent[0] if parent is not None and parent[0] in self.attention_cfgs else name
+        r_in = self.projection(right_name, p, i, "right", g.device, g.dtype)
+        r_out = self.projection(name, p, o, "left", g.device, g.dtype)
+        prep = ops.AdamPrepared(r_in, r_out, normalizer.weight_avg_sq, out_col)
+        self._adam_prepared[key] = prep
+        return prep
+
     def _compute_gradient(self, module: nn.Module, g: Tensor) -> Tensor:
         """Per-sample [N, p*p] (or per-token [n_valid, p*p]) projected gradient of one module, clamped to
         [lo, hi], in the model dtype (collector.py:592-743) -- one fused launch."""
-        mi = self.module_input(module, g, 0)
         p = self.per_module_projection_dim
-        assert p is not None
         N, S = g.shape[:2]
+        if isinstance(self.normalizer_for(module._name), AdamNormalizer):
+            prep = self.adam_prepared(module, g, 0)
+            a = module._inputs
+            if self.attribute_tokens:
+                lengths = self._batch_lengths(g.device)
+                assert lengths is not None, "attribute_tokens needs a collection mask (with_batch)"
+                counts = (lengths.to(torch.int64) - 1).clamp_min_(0)
+                offsets = torch.cumsum(counts, 0) - counts
+                out = torch.empty((int(counts.sum().item()), p * p), dtype=g.dtype, device=g.device)
+                if out.shape[0]:
+                    ops.collect_adam(prep, a, g, out, per_token=True, lengths=lengths, rows=offsets, lo=self.lo,
+                                     hi=self.hi)
+                return out
+            out = torch.empty((N, p * p), dtype=g.dtype, device=g.device)
+            ops.collect_adam(prep, a, g, out, per_token=False, lengths=None, rows=None, lo=self.lo, hi=self.hi)
+            return out
+        mi = self.module_input(module, g, 0)
+        assert p is not None
         if self.attribute_tokens:
             lengths = self._batch_lengths(g.device)
             assert lengths is not None, "attribute_tokens needs a collection mask (with_batch)"
@@ -399,6 +443,11 @@ class HookCollectorBase(ContextDecorator, ABC):
         module that does not change between batches (projection matrices, factor vectors, output column)
         is resolved and checked on its first batch only."""
         name: str = module._name  # type: ignore[assignment]
+        if isinstance(self.normalizer_for(name), AdamNormalizer):
+            a = module._inputs
+            assert isinstance(a, Tensor), "Activation cache missing for module"
+            self._deferred_adam.append((self.adam_prepared(module, g, out_col), a, g))
+            return
         prepared = self._prepared.get(name)
         if prepared is None or prepared.dtype != g.dtype or prepared.out_col != out_col:
             prepared = ops.PreparedModule(self.module_input(module, g, out_col), self.per_module_projection_dim)
@@ -409,19 +458,29 @@ class HookCollectorBase(ContextDecorator, ABC):
 
     def launch_deferred(self, out: Tensor, *, lengths: Tensor | None = None, out_rows: Tensor | None = None,
                         row_offsets: Tensor | None = None) -> None:
-        """One fused launch over every queued module, writing each module's block of `out`."""
-        if not self._deferred:
+        """One fused launch over every queued module (one launch sequence per module with an Adam
+        normaliser), writing each module's block of `out`."""
+        if not self._deferred and not self._deferred_adam:
             return
         p = self.per_module_projection_dim
         assert p is not None
         try:
             if self.attribute_tokens:
                 assert lengths is not None and row_offsets is not None
-                ops.collect_prepared(True, self._deferred, p, out, lengths, row_offsets, self.lo, self.hi)
+                if self._deferred:
+                    ops.collect_prepared(True, self._deferred, p, out, lengths, row_offsets, self.lo, self.hi)
+                for prep, a, g in self._deferred_adam:
+                    ops.collect_adam(prep, a, g, out, per_token=True, lengths=lengths, rows=row_offsets, lo=self.lo,
+                                     hi=self.hi)
             else:
-                ops.collect_prepared(False, self._deferred, p, out, lengths, out_rows, self.lo, self.hi)
+                if self._deferred:
+                    ops.collect_prepared(False, self._deferred, p, out, lengths, out_rows, self.lo, self.hi)
+                for prep, a, g in self._deferred_adam:
+                    ops.collect_adam(prep, a, g, out, per_token=False, lengths=lengths, rows=out_rows, lo=self.lo,
+                                     hi=self.hi)
         finally:
             self._deferred.clear()
+            self._deferred_adam.clear()
 
     @abstractmethod
     def setup(self) -> None: ...

@@ -1,0 +1,290 @@
+// Adam second-moment normalisation on the collection path.
+//
+// The reference forms, per sequence or per token, the full weight-shaped gradient, divides it by
+// sqrt(v) + 1e-8 and projects it from both sides (bergson/collector/collector.py:609-644,
+// bergson/gradients.py:380-388).  Per token t that is
+//     P_t[i, j] = sum_o L[i, o] g_t[o] * H_t[o, j],
+//     H_t[o, j] = sum_k a_t[k] * C[(o, j), k],      C[(o, j), k] = R[j, k] / (sqrt(v[o, k]) + 1e-8)
+// so nothing weight-shaped is formed per token: H is one GEMM of the activations against a table C that
+// depends on the module only (built once by adam_table_kernel), and P_t is a small contraction of H_t with
+// L and g_t.  The per-sequence gradient is the sum of its tokens' P_t (the normalisation is linear).
+//
+// This build materialises H for a chunk of tokens at a time (GEMM on the scan kernel's main loop, then
+// adam_contract_kernel).  H is O*p values per token, which makes the path HBM-heavy for large modules;
+// fusing the contraction into the GEMM is the planned next step.
+
+#include "common.hpp"
+
+namespace bgx {
+
+int gemm_scores(const void* rows, int64_t n_rows, int64_t D, int64_t stride, int dtype, const void* queries, int Q,
+                float* scores, hipStream_t st);
+
+// table[(o * p + j) * I + k] = round_T(R[j, k] / (sqrt(v[o, k]) + 1e-8))
+template <typename T>
+__global__ __launch_bounds__(256) void adam_table_kernel(const T* __restrict__ r_in, const float* __restrict__ v, int O,
+                                                         int I, int p, T* __restrict__ table) {
+  const int64_t total = (int64_t)O * p * I;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int k = (int)(idx % I);
+    const int64_t oj = idx / I;
+    const int j = (int)(oj % p);
+    const int o = (int)(oj / p);
+    const float w = 1.0f / (sqrtf(v[(int64_t)o * I + k]) + 1e-8f);
+    const float val = Elem<T>::load(r_in + (int64_t)j * I + k) * w;
+    if constexpr (sizeof(T) == 4)
+      *(float*)(table + idx) = val;
+    else if constexpr (Elem<T>::code == BGX_F16)
+      ((uint16_t*)table)[idx] = (uint16_t)f32_to_f16_bits(val);
+    else
+      ((uint16_t*)table)[idx] = (uint16_t)f32_to_bf16_bits(val);
+  }
+}
+
+struct ContractArgs {
+  const float* H;        // [chunk_tokens, O * p]
+  const void* g;         // [N, S, O]
+  const void* r_out;     // [p, O]
+  int64_t g_seq_stride, g_tok_stride;
+  int64_t t0;            // first flattened token of the chunk
+  int chunk_tokens;
+  int S, O, p;
+  const int32_t* lengths;
+  // per-token output
+  const int64_t* row_offsets;
+  void* out;
+  int64_t out_row_stride, out_col;
+  int out_dtype;
+  float lo, hi;
+  // per-sequence: per-token fp32 rows of the chunk
+  float* ptok;           // [chunk_tokens, p * p]
+};
+
+constexpr int CONTRACT_OC = 32;  // output features staged per step
+
+// One workgroup per token of the chunk: P_t[i, j] = sum_o L[i, o] g_t[o] H_t[o, j].
+template <typename T, bool PER_TOKEN>
+__global__ __launch_bounds__(256) void adam_contract_kernel(ContractArgs a) {
+  __shared__ float s_lg[CONTRACT_OC][65];  // [o][i]  L[i, o] * g_t[o]
+  __shared__ float s_h[CONTRACT_OC][65];   // [o][j]
+  const int tl = blockIdx.x;
+  const int64_t t = a.t0 + tl;
+  const int n = (int)(t / a.S);
+  const int s = (int)(t - (int64_t)n * a.S);
+  const int p = a.p, pp = p * p;
+  bool valid = true;
+  if (a.lengths != nullptr) valid = s < a.lengths[n] - 1;
+  if (PER_TOKEN && !valid) return;
+  const int tid = threadIdx.x;
+  float acc[16];  // p*p <= 4096 outputs over 256 threads
+#pragma unroll
+  for (int c = 0; c < 16; ++c) acc[c] = 0.f;
+  if (valid) {
+    const T* g = (const T*)a.g + (int64_t)n * a.g_seq_stride + (int64_t)s * a.g_tok_stride;
+    const T* L = (const T*)a.r_out;
+    const float* H = a.H + (int64_t)tl * a.O * p;
+    for (int o0 = 0; o0 < a.O; o0 += CONTRACT_OC) {
+      const int oc = min(CONTRACT_OC, a.O - o0);
+      __syncthreads();
+      for (int e = tid; e < oc * p; e += 256) {
+        const int oo = e / p, x = e - oo * p;
+        s_lg[oo][x] = Elem<T>::load(L + (int64_t)x * a.O + o0 + oo) * Elem<T>::load(g + o0 + oo);
+        s_h[oo][x] = H[(int64_t)(o0 + oo) * p + x];
+      }
+      __syncthreads();
+#pragma unroll
+      for (int c = 0; c < 16; ++c) {
+        const int e = tid + c * 256;
+        if (e < pp) {
+          const int i = e / p, j = e - i * p;
+          float sum = acc[c];
+          for (int oo = 0; oo < oc; ++oo) sum = fmaf(s_lg[oo][i], s_h[oo][j], sum);
+          acc[c] = sum;
+        }
+      }
+    }
+  }
+  if (PER_TOKEN) {
+    const int64_t base = (a.row_offsets[n] + s) * a.out_row_stride + a.out_col;
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+      const int e = tid + c * 256;
+      if (e < pp) store_as(a.out, base + e, clampf(acc[c], a.lo, a.hi), a.out_dtype);
+    }
+  } else {
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+      const int e = tid + c * 256;
+      if (e < pp) a.ptok[(int64_t)tl * pp + e] = acc[c];
+    }
+  }
+}
+
+// acc[n, e] += sum over the chunk's tokens of sequence n, in token order.
+__global__ __launch_bounds__(256) void adam_seq_sum_kernel(const float* __restrict__ ptok, float* __restrict__ acc,
+                                                           int64_t t0, int chunk_tokens, int S, int pp, int n_first) {
+  const int n = n_first + blockIdx.x;
+  const int64_t lo = (int64_t)n * S > t0 ? (int64_t)n * S : t0;
+  const int64_t hi_seq = (int64_t)(n + 1) * S;
+  const int64_t hi = hi_seq < t0 + chunk_tokens ? hi_seq : t0 + chunk_tokens;
+  for (int e = threadIdx.x; e < pp; e += blockDim.x) {
+    float s = acc[(int64_t)n * pp + e];
+    for (int64_t t = lo; t < hi; ++t) s += ptok[(t - t0) * pp + e];
+    acc[(int64_t)n * pp + e] = s;
+  }
+}
+
+__global__ __launch_bounds__(256) void adam_seq_finalize_kernel(const float* __restrict__ acc,
+                                                                const int64_t* __restrict__ out_rows, int pp,
+                                                                void* out, int64_t out_row_stride, int64_t out_col,
+                                                                int out_dtype, float lo, float hi) {
+  const int n = blockIdx.x;
+  const int64_t row = out_rows ? out_rows[n] : (int64_t)n;
+  for (int e = threadIdx.x; e < pp; e += blockDim.x)
+    store_as(out, row * out_row_stride + out_col + e, clampf(acc[(int64_t)n * pp + e], lo, hi), out_dtype);
+}
+
+__global__ void adam_zero_kernel(float* x, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] = 0.f;
+}
+
+// ---- host ---------------------------------------------------------------------------------------
+static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+size_t adam_table_bytes(int O, int I, int p, int dtype) {
+  if (O <= 0 || I <= 0 || p <= 0) return 0;
+  return (size_t)O * p * I * dtype_size(dtype);
+}
+
+int adam_prepare_impl(const void* r_in, const float* v, int O, int I, int p, int dtype, void* table, void* stream) {
+  BGX_REQUIRE(r_in && v && table, BGX_E_ARG, "adam_prepare: null pointer");
+  BGX_REQUIRE(O > 0 && I > 0 && p >= 1 && p <= 64, BGX_E_SHAPE, "adam_prepare: O=%d I=%d p=%d", O, I, p);
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t total = (int64_t)O * p * I;
+  const unsigned blocks = (unsigned)((total + 255) / 256 > 65536 * 16 ? 65536 * 16 : (total + 255) / 256);
+  if (dtype == BGX_F32)
+    hipLaunchKernelGGL(adam_table_kernel<float>, dim3(blocks), dim3(256), 0, st, (const float*)r_in, v, O, I, p,
+                       (float*)table);
+  else if (dtype == BGX_F16)
+    hipLaunchKernelGGL(adam_table_kernel<f16_t>, dim3(blocks), dim3(256), 0, st, (const f16_t*)r_in, v, O, I, p,
+                       (f16_t*)table);
+  else if (dtype == BGX_BF16)
+    hipLaunchKernelGGL(adam_table_kernel<bf16_t>, dim3(blocks), dim3(256), 0, st, (const bf16_t*)r_in, v, O, I, p,
+                       (bf16_t*)table);
+  else
+    BGX_REQUIRE(false, BGX_E_DTYPE, "adam_prepare: dtype=%d", dtype);
+  BGX_HIP(hipGetLastError());
+  return 0;
+}
+
+static int64_t adam_chunk(int64_t T, int O, int p, int64_t chunk_tokens) {
+  if (chunk_tokens <= 0) {
+    // keep H (fp32, O*p per token) near 512 MB
+    chunk_tokens = ((int64_t)512 << 20) / ((int64_t)O * p * 4);
+    chunk_tokens = chunk_tokens / 256 * 256;
+    if (chunk_tokens < 256) chunk_tokens = 256;
+  }
+  return chunk_tokens < T ? chunk_tokens : T;
+}
+
+size_t collect_adam_workspace_bytes(int N, int S, int O, int p, int64_t chunk_tokens) {
+  if (N <= 0 || S <= 0 || O <= 0 || p <= 0) return 0;
+  const int64_t T = (int64_t)N * S;
+  const int64_t tc = adam_chunk(T, O, p, chunk_tokens);
+  return align_up((size_t)tc * O * p * 4, 256) + align_up((size_t)tc * p * p * 4, 256) +
+         align_up((size_t)N * p * p * 4, 256);
+}
+
+int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_t a_tok_stride, int64_t g_seq_stride,
+                      int64_t g_tok_stride, int N, int S, int I, int O, int p, int dtype, const void* table,
+                      const void* r_out, int per_token, const int32_t* lengths, const int64_t* rows, void* out,
+                      int64_t out_row_stride, int64_t out_col, int out_dtype, float lo, float hi, void* ws,
+                      size_t ws_bytes, int64_t chunk_tokens, void* stream) {
+  BGX_REQUIRE(a && g && table && r_out && out && ws, BGX_E_ARG, "collect_adam: null pointer");
+  BGX_REQUIRE(N > 0 && S > 0 && I > 0 && O > 0, BGX_E_ARG, "collect_adam: N=%d S=%d I=%d O=%d", N, S, I, O);
+  BGX_REQUIRE(p >= 1 && p <= 64, BGX_E_SHAPE, "collect_adam: p=%d outside 1..64", p);
+  BGX_REQUIRE(dtype >= BGX_F32 && dtype <= BGX_BF16 && out_dtype >= BGX_F32 && out_dtype <= BGX_BF16, BGX_E_DTYPE,
+              "collect_adam: dtype=%d out_dtype=%d", dtype, out_dtype);
+  BGX_REQUIRE(a_seq_stride == (int64_t)S * a_tok_stride, BGX_E_ALIGN,
+              "collect_adam: activations must be uniformly strided over the flattened tokens");
+  BGX_REQUIRE((int64_t)O * p <= 0x7fffffffLL, BGX_E_SHAPE, "collect_adam: O*p too large");
+  BGX_REQUIRE(out_col >= 0 && out_col + (int64_t)p * p <= out_row_stride, BGX_E_ARG, "collect_adam: columns do not fit");
+  if (per_token) BGX_REQUIRE(lengths && rows, BGX_E_ARG, "collect_adam: per-token mode needs lengths and row_offsets");
+  const size_t need = collect_adam_workspace_bytes(N, S, O, p, chunk_tokens);
+  BGX_REQUIRE(ws_bytes >= need, BGX_E_WORKSPACE, "collect_adam: workspace %zu < %zu bytes", ws_bytes, need);
+  BGX_REQUIRE(((uintptr_t)ws & 255) == 0, BGX_E_ALIGN, "collect_adam: workspace must be 256-byte aligned");
+
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t T = (int64_t)N * S;
+  const int64_t tc = adam_chunk(T, O, p, chunk_tokens);
+  const int pp = p * p;
+  char* w = (char*)ws;
+  float* H = (float*)w;
+  float* ptok = (float*)(w + align_up((size_t)tc * O * p * 4, 256));
+  float* acc = (float*)((char*)ptok + align_up((size_t)tc * pp * 4, 256));
+  const size_t esz = dtype_size(dtype);
+
+  if (!per_token) {
+    const int64_t nacc = (int64_t)N * pp;
+    hipLaunchKernelGGL(adam_zero_kernel, dim3((unsigned)((nacc + 255) / 256)), dim3(256), 0, st, acc, nacc);
+    BGX_HIP(hipGetLastError());
+  }
+  for (int64_t t0 = 0; t0 < T; t0 += tc) {
+    const int64_t rows_c = T - t0 < tc ? T - t0 : tc;
+    const char* a_chunk = (const char*)a + (size_t)t0 * a_tok_stride * esz;
+    const int rc = gemm_scores(a_chunk, rows_c, I, a_tok_stride, dtype, table, O * p, H, st);
+    if (rc != 0) return rc;
+    ContractArgs c;
+    c.H = H;
+    c.g = g;
+    c.r_out = r_out;
+    c.g_seq_stride = g_seq_stride;
+    c.g_tok_stride = g_tok_stride;
+    c.t0 = t0;
+    c.chunk_tokens = (int)rows_c;
+    c.S = S;
+    c.O = O;
+    c.p = p;
+    c.lengths = lengths;
+    c.row_offsets = per_token ? rows : nullptr;
+    c.out = out;
+    c.out_row_stride = out_row_stride;
+    c.out_col = out_col;
+    c.out_dtype = out_dtype;
+    c.lo = lo;
+    c.hi = hi;
+    c.ptok = ptok;
+    const dim3 grid((unsigned)rows_c), block(256);
+#define BGX_CONTRACT(T_)                                                                         \
+  if (per_token)                                                                                 \
+    hipLaunchKernelGGL((adam_contract_kernel<T_, true>), grid, block, 0, st, c);                 \
+  else                                                                                           \
+    hipLaunchKernelGGL((adam_contract_kernel<T_, false>), grid, block, 0, st, c);
+    if (dtype == BGX_F32) {
+      BGX_CONTRACT(float)
+    } else if (dtype == BGX_F16) {
+      BGX_CONTRACT(f16_t)
+    } else {
+      BGX_CONTRACT(bf16_t)
+    }
+#undef BGX_CONTRACT
+    BGX_HIP(hipGetLastError());
+    if (!per_token) {
+      const int n_first = (int)(t0 / S);
+      const int n_last = (int)((t0 + rows_c - 1) / S);
+      hipLaunchKernelGGL(adam_seq_sum_kernel, dim3((unsigned)(n_last - n_first + 1)), dim3(256), 0, st, ptok, acc, t0,
+                         (int)rows_c, S, pp, n_first);
+      BGX_HIP(hipGetLastError());
+    }
+  }
+  if (!per_token) {
+    hipLaunchKernelGGL(adam_seq_finalize_kernel, dim3((unsigned)N), dim3(256), 0, st, acc, rows, pp, out,
+                       out_row_stride, out_col, out_dtype, lo, hi);
+    BGX_HIP(hipGetLastError());
+  }
+  return 0;
+}
+
+}  // namespace bgx

@@ -26,6 +26,14 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
                  int out_dtype, float lo, float hi, void* ws, size_t ws_bytes, void* stream);
 int adafactor_scales_impl(const float* row, int O, const float* col, int I, int dtype, float* row_scale,
                           float* col_scale, void* stream);
+size_t adam_table_bytes(int O, int I, int p, int dtype);
+int adam_prepare_impl(const void* r_in, const float* v, int O, int I, int p, int dtype, void* table, void* stream);
+size_t collect_adam_workspace_bytes(int N, int S, int O, int p, int64_t chunk_tokens);
+int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_t a_tok_stride, int64_t g_seq_stride,
+                      int64_t g_tok_stride, int N, int S, int I, int O, int p, int dtype, const void* table,
+                      const void* r_out, int per_token, const int32_t* lengths, const int64_t* rows, void* out,
+                      int64_t out_row_stride, int64_t out_col, int out_dtype, float lo, float hi, void* ws,
+                      size_t ws_bytes, int64_t chunk_tokens, void* stream);
 int collect_timing_enable(int max_launches);
 int collect_timing_read(float* ms_out, int capacity, int* count_out);
 int unit_normalize_impl(void* rows, int64_t n_rows, int64_t D, int64_t stride, int dtype, void* stream);
@@ -66,6 +74,31 @@ int bgx_collect_tok(const bgx_module_desc* mods_host, int32_t n_modules, int32_t
                     size_t workspace_bytes, void* stream) {
   return bgx::collect_impl(true, mods_host, n_modules, N, S, p, in_dtype, lengths_dev, row_offsets_dev, out_dev,
                            out_row_stride, out_dtype, clamp_lo, clamp_hi, workspace_dev, workspace_bytes, stream);
+}
+
+size_t bgx_adam_table_bytes(int32_t O, int32_t I, int32_t p, int32_t dtype) {
+  return bgx::adam_table_bytes(O, I, p, dtype);
+}
+
+int bgx_adam_prepare(const void* r_in_dev, const float* weight_avg_sq_dev, int32_t O, int32_t I, int32_t p,
+                     int32_t dtype, void* table_dev, void* stream) {
+  return bgx::adam_prepare_impl(r_in_dev, weight_avg_sq_dev, O, I, p, dtype, table_dev, stream);
+}
+
+size_t bgx_collect_adam_workspace_bytes(int32_t N, int32_t S, int32_t O, int32_t p, int64_t chunk_tokens) {
+  return bgx::collect_adam_workspace_bytes(N, S, O, p, chunk_tokens);
+}
+
+int bgx_collect_adam(const void* a_dev, const void* g_dev, int64_t a_seq_stride, int64_t a_tok_stride,
+                     int64_t g_seq_stride, int64_t g_tok_stride, int32_t N, int32_t S, int32_t I, int32_t O, int32_t p,
+                     int32_t dtype, const void* table_dev, const void* r_out_dev, int32_t per_token,
+                     const int32_t* lengths_dev, const int64_t* rows_dev, void* out_dev, int64_t out_row_stride,
+                     int64_t out_col, int32_t out_dtype, float clamp_lo, float clamp_hi, void* workspace_dev,
+                     size_t workspace_bytes, int64_t chunk_tokens, void* stream) {
+  return bgx::collect_adam_impl(a_dev, g_dev, a_seq_stride, a_tok_stride, g_seq_stride, g_tok_stride, N, S, I, O, p,
+                                dtype, table_dev, r_out_dev, per_token, lengths_dev, rows_dev, out_dev, out_row_stride,
+                                out_col, out_dtype, clamp_lo, clamp_hi, workspace_dev, workspace_bytes, chunk_tokens,
+                                stream);
 }
 
 int bgx_collect_timing_enable(int32_t max_launches) { return bgx::collect_timing_enable(max_launches); }

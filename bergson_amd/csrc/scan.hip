@@ -516,7 +516,8 @@ static int launch_gemm(const ScanArgs& a, bool aligned, hipStream_t st) {
 template <typename T>
 static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
   // large tiles when there is enough work to fill the chip with them
-  if (a.Q > 64 && a.rows >= 4096) {
+  const int64_t big_tiles = ((a.rows + 255) / 256) * ((a.Q + 255) / 256);
+  if (a.Q > 64 && a.rows >= 256 && big_tiles >= 256) {
     // 8 waves, each 128 x 64: two waves per SIMD hide each other's LDS and barrier stalls
     constexpr int BM = 256, BN = 256;
     a.row_tiles = (int)((a.rows + BM - 1) / BM);
@@ -533,6 +534,36 @@ static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
     a.q_tiles = (a.Q + BN - 1) / BN;
     return launch_gemm<T, BM, BN, 4, 1>(a, aligned, st);
   }
+}
+
+// scores[n, q] = <rows[n], queries[q]> for every (n, q): the GEMM alone, no norms, no selection.
+int gemm_scores(const void* rows, int64_t n_rows, int64_t D, int64_t stride, int dtype, const void* queries, int Q,
+                float* scores, hipStream_t st) {
+  ScanArgs a;
+  a.store = rows;
+  a.queries = queries;
+  a.row0 = 0;
+  a.rows = n_rows;
+  a.D = D;
+  a.store_stride = stride;
+  a.Q = Q;
+  a.row_tiles = 0;
+  a.q_tiles = 0;
+  a.query_scale = 1.0f;
+  a.unit_norm = 0;
+  a.scores = scores;
+  a.sumsq = nullptr;
+  a.row_max_enc = nullptr;
+  a.thr = nullptr;
+  a.cand_count = nullptr;
+  a.cand = nullptr;
+  a.cand_cap = 0;
+  const int epl = dtype == BGX_F32 ? 4 : 8;
+  const bool aligned = ((uintptr_t)rows % 16 == 0) && ((uintptr_t)queries % 16 == 0) && (D % epl == 0) &&
+                       (stride % epl == 0);
+  if (dtype == BGX_F16) return launch_gemm_t<f16_t>(a, aligned, st);
+  if (dtype == BGX_BF16) return launch_gemm_t<bf16_t>(a, aligned, st);
+  return launch_gemm_t<float>(a, aligned, st);
 }
 
 int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int dtype, const void* queries, int Q,

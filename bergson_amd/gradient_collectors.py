@@ -45,10 +45,11 @@ class _DeferredBatchMixin:
         them and nobody else needs them; otherwise into a fresh batch buffer whose column views are
         returned as mod_grads."""
         block = RowBlock()
-        if not self._deferred:
+        queued = self._deferred or self._deferred_adam
+        if not queued:
             return block
-        dev = self._deferred[0][2].device
-        N = self._deferred[0][2].shape[0]
+        dev = queued[0][2].device
+        N = queued[0][2].shape[0]
         assert N == len(indices), f"batch of {N} sequences but {len(indices)} indices"
         lengths = self._batch_lengths(dev) if (self.attribute_tokens or self.skip_padding) else None
         direct = builder is not None and builder.direct and not need_rows
@@ -67,6 +68,7 @@ class _DeferredBatchMixin:
                 self.launch_deferred(rows, lengths=lengths, row_offsets=offsets)
             else:
                 self._deferred.clear()
+                self._deferred_adam.clear()
         elif direct:
             idx = torch.as_tensor(indices, dtype=torch.int64).to(dev, non_blocking=True)
             self.launch_deferred(builder.device_rows, lengths=lengths, out_rows=idx)

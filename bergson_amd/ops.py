@@ -256,6 +256,58 @@ def collect_prepared(per_token: bool, items: list, p: int, out: Tensor, lengths:
     del keep
 
 
+class AdamPrepared:
+    """Per-module state of the Adam path: the [(O*p), I] table built from the right projection and the
+    second moments, and the left projection."""
+
+    def __init__(self, r_in: Tensor, r_out: Tensor, weight_avg_sq: Tensor, out_col: int):
+        lib = _lib.load()
+        _need_gpu(r_in, "r_in")
+        p, I = r_in.shape
+        O = r_out.shape[1]
+        if r_out.shape[0] != p or tuple(weight_avg_sq.shape) != (O, I):
+            raise ValueError(f"Adam shapes: r_in {tuple(r_in.shape)}, r_out {tuple(r_out.shape)}, "
+                             f"weight_avg_sq {tuple(weight_avg_sq.shape)}")
+        self.dtype = r_in.dtype
+        self.p, self.I, self.O, self.out_col = p, I, O, out_col
+        self.r_in = r_in.contiguous()
+        self.r_out = r_out.contiguous()
+        v = weight_avg_sq.detach().to(device=r_in.device, dtype=torch.float32).contiguous()
+        nbytes = lib.bgx_adam_table_bytes(O, I, p, dtype_code(self.dtype))
+        self.table = torch.empty(nbytes // self.r_in.element_size(), dtype=self.dtype, device=r_in.device)
+        rc = lib.bgx_adam_prepare(_ptr(self.r_in), _ptr(v), O, I, p, dtype_code(self.dtype), _ptr(self.table), _stream())
+        _lib.check(rc, "bgx_adam_prepare")
+
+
+def collect_adam(prep: AdamPrepared, a: Tensor, g: Tensor, out: Tensor, *, per_token: bool, lengths: Tensor | None,
+                 rows: Tensor | None, lo: float, hi: float, chunk_tokens: int = 0) -> None:
+    """One module with an Adam normaliser: writes its p*p block of every output row (see bgx_collect_adam)."""
+    lib = _lib.load()
+    for t, name in ((a, "a"), (g, "g"), (out, "out")):
+        _need_gpu(t, name)
+    if a.dim() != 3 or g.dim() != 3 or a.shape[:2] != g.shape[:2]:
+        raise ValueError(f"a {tuple(a.shape)} / g {tuple(g.shape)} must be [N, S, I] and [N, S, O]")
+    N, S, I = a.shape
+    O = g.shape[2]
+    if (I, O) != (prep.I, prep.O) or a.dtype != prep.dtype or g.dtype != prep.dtype:
+        raise ValueError("a / g do not match the prepared module")
+    if a.stride(2) != 1 or a.stride(0) != S * a.stride(1):
+        a = a.contiguous()
+    if g.stride(2) != 1:
+        g = g.contiguous()
+    if out.dim() != 2 or out.stride(1) != 1:
+        raise ValueError("out must be a 2-D tensor with contiguous rows")
+    if per_token and (lengths is None or rows is None):
+        raise ValueError("per-token collection needs lengths and row offsets")
+    nbytes = lib.bgx_collect_adam_workspace_bytes(N, S, O, prep.p, chunk_tokens)
+    ws = _workspace(out.device, nbytes, "adam")
+    rc = lib.bgx_collect_adam(_ptr(a), _ptr(g), a.stride(0), a.stride(1), g.stride(0), g.stride(1), N, S, I, O, prep.p,
+                              dtype_code(prep.dtype), _ptr(prep.table), _ptr(prep.r_out), int(per_token), _ptr(lengths),
+                              _ptr(rows), _ptr(out), out.stride(0), prep.out_col, dtype_code(out.dtype), lo, hi,
+                              _ptr(ws), ws.numel(), chunk_tokens, _stream())
+    _lib.check(rc, "bgx_collect_adam")
+
+
 def collect_seq(modules: list[ModuleInput], p: int, out: Tensor, *, lengths: Tensor | None = None,
                 out_rows: Tensor | None = None, lo: float = float("-inf"), hi: float = float("inf")) -> None:
     """out[row(n), m.out_col : m.out_col + p*p] = clamp(sum_s g'[n,s] (x) a'[n,s]) for every module m."""

@@ -133,6 +133,40 @@ int bgx_collect_tok(const bgx_module_desc* mods_host, int32_t n_modules,
                     float clamp_lo, float clamp_hi, void* workspace_dev,
                     size_t workspace_bytes, void* stream);
 
+/* ---- Adam second-moment normaliser on the collection path ---------------
+ * Replaces bergson/collector/collector.py:609-644 with
+ * bergson/gradients.py:380-388 (grad / (sqrt(weight_avg_sq) + 1e-8), eps
+ * outside the root) and the double-sided projection of collector.py:545-550.
+ *
+ * bgx_adam_prepare builds, once per module, the table
+ *   table[(o*p + j), k] = round_dtype(r_in[j, k] / (sqrt(weight_avg_sq[o, k]) + 1e-8))
+ * of bgx_adam_table_bytes(O, I, p, dtype) bytes.
+ * bgx_collect_adam then computes, for one module of one batch,
+ *   P_t[i, j] = sum_o r_out[i, o] g_t[o] * sum_k a_t[k] table[(o*p + j), k]
+ * per token t and writes either every valid token's row (per_token != 0:
+ * row row_offsets[n] + s, s < lengths[n] - 1) or the sum over each sequence
+ * (per_token == 0: row rows[n], or n when rows is NULL), clamped and cast.
+ * a must be uniformly strided over the flattened tokens
+ * (a_seq_stride == S * a_tok_stride).  chunk_tokens = 0 picks the number of
+ * tokens per internal pass. */
+size_t bgx_adam_table_bytes(int32_t O, int32_t I, int32_t p, int32_t dtype);
+int bgx_adam_prepare(const void* r_in_dev, const float* weight_avg_sq_dev,
+                     int32_t O, int32_t I, int32_t p, int32_t dtype,
+                     void* table_dev, void* stream);
+size_t bgx_collect_adam_workspace_bytes(int32_t N, int32_t S, int32_t O,
+                                        int32_t p, int64_t chunk_tokens);
+int bgx_collect_adam(const void* a_dev, const void* g_dev,
+                     int64_t a_seq_stride, int64_t a_tok_stride,
+                     int64_t g_seq_stride, int64_t g_tok_stride, int32_t N,
+                     int32_t S, int32_t I, int32_t O, int32_t p, int32_t dtype,
+                     const void* table_dev, const void* r_out_dev,
+                     int32_t per_token, const int32_t* lengths_dev,
+                     const int64_t* rows_dev, void* out_dev,
+                     int64_t out_row_stride, int64_t out_col,
+                     int32_t out_dtype, float clamp_lo, float clamp_hi,
+                     void* workspace_dev, size_t workspace_bytes,
+                     int64_t chunk_tokens, void* stream);
+
 /* Benchmark support (no counterpart in the reference): while enabled, every
  * bgx_collect_seq / bgx_collect_tok call records a HIP event pair immediately
  * around its collect_kernel launch, on the launch stream, so that the kernel's

@@ -45,8 +45,9 @@ def adafactor_normalize_bias(grad: Tensor, n: Adafactor, eps: float = 1e-8) -> T
 
 
 def adam_normalize_weight(grad: Tensor, n: Adam, eps: float = 1e-8) -> Tensor:
-    """eps outside the square root (gradients.py:380-388)."""
-    return grad / (n.weight_avg_sq.sqrt() + eps)
+    """eps outside the square root; in place in the reference, so the result keeps grad's dtype
+    (gradients.py:380-388)."""
+    return grad.clone().div_(n.weight_avg_sq.sqrt().add_(eps))
 
 
 def adam_normalize_bias(grad: Tensor, n: Adam, eps: float = 1e-8) -> Tensor:

@@ -220,3 +220,62 @@ def test_rejects_cpu_tensors():
     with pytest.raises(RuntimeError, match="no CPU path"):
         ops.collect_seq([ops.ModuleInput(a=a, g=a, r_in=torch.zeros(16, 8), r_out=torch.zeros(16, 8), out_col=0)], 16,
                         torch.zeros(1, 256))
+
+
+# ---- Adam second-moment normaliser -----------------------------------------------------------------------
+
+def _adam_case(N, S, I, O, p, dtype, seed):
+    gen = torch.Generator().manual_seed(seed)
+    a = torch.randn(N, S, I, generator=gen).to(dtype)
+    g = (torch.randn(N, S, O, generator=gen) * 0.1).to(dtype)
+    left, right = module_projections("layers.1.attention.dense", p, O, I, dtype)
+    v = (torch.randn(O, I, generator=gen).abs() * 1e-5) + 1e-9
+    return a, g, left, right, ohooks.Adam(weight_avg_sq=v)
+
+
+def _run_adam(device, case, p, out_dtype, *, per_token=False, lengths=None, row_offsets=None, n_rows=None,
+              chunk_tokens=0, out_col=0, width=None):
+    from bergson_amd import ops
+
+    a, g, left, right, norm = case
+    prep = ops.AdamPrepared(right.to(device), left.to(device), norm.weight_avg_sq.to(device), out_col)
+    rows = n_rows if n_rows is not None else a.shape[0]
+    out = torch.zeros(rows, width or p * p, dtype=out_dtype, device=device)
+    ldev = None if lengths is None else torch.tensor(lengths, dtype=torch.int32, device=device)
+    rdev = None if row_offsets is None else torch.tensor(row_offsets, dtype=torch.int64, device=device)
+    ops.collect_adam(prep, a.to(device), g.to(device), out, per_token=per_token, lengths=ldev, rows=rdev,
+                     lo=torch.finfo(out_dtype).min, hi=torch.finfo(out_dtype).max, chunk_tokens=chunk_tokens)
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 40, 64, 96, 16), (3, 70, 128, 64, 32), (1, 33, 96, 40, 8)])
+def test_adam_seq(device, dtype, shape):
+    N, S, I, O, p = shape
+    case = _adam_case(N, S, I, O, p, dtype, seed=50)
+    got = _run_adam(device, case, p, dtype, chunk_tokens=64)  # several internal passes
+    a, g, left, right, norm = case
+    want = ohooks.module_gradient(a, g, norm, left, right)
+    assert got.shape == want.shape
+    assert rel_l2(got, want) <= TOL[dtype]
+    if dtype == torch.float32:
+        # and against the closed form L @ (G^T A / (sqrt(v) + 1e-8)) @ R^T in fp64
+        full = (g.mT.double() @ a.double()) / (norm.weight_avg_sq.double().sqrt() + 1e-8)
+        assert rel_l2(got, (left.double() @ full @ right.double().T).flatten(1)) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_adam_tok(device, dtype):
+    N, S, I, O, p = 3, 50, 64, 96, 16
+    lengths = [50, 21, 37]
+    case = _adam_case(N, S, I, O, p, dtype, seed=51)
+    a, g, left, right, norm = case
+    mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+    counts = [l - 1 for l in lengths]
+    offs = [0, counts[0], counts[0] + counts[1]]
+    got = _run_adam(device, case, p, dtype, per_token=True, lengths=lengths, row_offsets=offs, n_rows=sum(counts),
+                    chunk_tokens=64, out_col=256, width=768)
+    want = ohooks.module_gradient(a, g, norm, left, right, attribute_tokens=True, collection_mask=mask)
+    assert rel_l2(got[:, 256:512], want) <= TOL[dtype]
+    assert got[:, :256].abs().sum() == 0 and got[:, 512:].abs().sum() == 0

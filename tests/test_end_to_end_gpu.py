@@ -130,3 +130,50 @@ def test_pythia160m_bf16_adafactor_against_captured_hooks(device, store_dtype):
     # every module on its own, so that a small block cannot hide behind a large one
     for b in range(12):
         assert rel_l2(got[:, b * 256:(b + 1) * 256], want[:, b * 256:(b + 1) * 256]) <= 1e-2
+
+
+def test_pythia14m_fp32_adam_and_mixed_normalizers(device):
+    """Adam on some modules, Adafactor on others, none on the rest: every module's block against the
+    oracle's hook arithmetic on the captured (a, g)."""
+    from bergson_amd import AdafactorNormalizer, AdamNormalizer, GradientCollector, IndexConfig
+    from bergson_amd.collector import CollectorComputer
+    from bergson_amd.synthetic import ListDataset, make_gpt_neox, random_docs
+
+    lengths = [40, 25, 33]
+    docs = random_docs(lengths, seed=9)
+    model = make_gpt_neox("pythia-14m", torch.float32, device, seed=0, layers=2)
+    names = [n for n, m in model.base_model.named_modules() if isinstance(m, torch.nn.Linear)]
+    gen = torch.Generator().manual_seed(1)
+    onorm, norms = {}, {}
+    for k, n in enumerate(names):
+        mod = model.base_model.get_submodule(n)
+        O, I = mod.out_features, mod.in_features
+        if k % 3 == 0:
+            v = torch.rand(O, I, generator=gen) * 1e-4 + 1e-8
+            onorm[n], norms[n] = ohooks.Adam(v), AdamNormalizer(v.to(device))
+        elif k % 3 == 1:
+            r, c = torch.rand(O, generator=gen) * 1e-4 + 1e-8, torch.rand(I, generator=gen) * 1e-4 + 1e-8
+            onorm[n], norms[n] = ohooks.Adafactor(r, c), AdafactorNormalizer(r.to(device), c.to(device))
+    captured = {}
+    handles = []
+    for name in names:
+        mod = model.base_model.get_submodule(name)
+        handles.append(mod.register_forward_hook(
+            lambda m, inp, out, name=name: captured.setdefault(name, {}).__setitem__("a", inp[0].detach().cpu())))
+        handles.append(mod.register_full_backward_hook(
+            lambda m, gin, gout, name=name: captured[name].__setitem__("g", gout[0].detach().cpu())))
+    for attribute_tokens in (False, True):
+        cfg = IndexConfig(run_path="", projection_dim=16, projection_type="normal", attribute_tokens=attribute_tokens)
+        col = GradientCollector(model=model.base_model, cfg=cfg, data=ListDataset(docs), processor=_processor(16, norms))
+        CollectorComputer(model=model, data=ListDataset(docs), collector=col, batches=[[0, 1, 2]], cfg=cfg
+                          ).run_with_collector_hooks()
+        got = torch.from_numpy(np.array(col.builder.grad_buffer))
+        mask = (torch.arange(40).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+        for b, name in enumerate(names):
+            a, g = captured[name]["a"], captured[name]["g"]
+            left, right = module_projections(name, 16, g.shape[-1], a.shape[-1], torch.float32)
+            want = ohooks.module_gradient(a, g, onorm.get(name), left, right, attribute_tokens=attribute_tokens,
+                                          collection_mask=mask if attribute_tokens else None)
+            assert rel_l2(got[:, b * 256:(b + 1) * 256], want) <= 1e-4, (attribute_tokens, name)
+    for h in handles:
+        h.remove()
