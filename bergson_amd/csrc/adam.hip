@@ -121,16 +121,33 @@ __global__ __launch_bounds__(256) void adam_contract_kernel(ContractArgs a) {
   }
 }
 
-// acc[n, e] += sum over the chunk's tokens of sequence n, in token order.
-__global__ __launch_bounds__(256) void adam_seq_sum_kernel(const float* __restrict__ ptok, float* __restrict__ acc,
-                                                           int64_t t0, int chunk_tokens, int S, int pp, int n_first) {
+constexpr int SEQ_SLICES = 32;
+
+// part[n - n_first, slice, e] = sum over one slice of the chunk's tokens of sequence n, in token order.
+__global__ __launch_bounds__(256) void adam_seq_slice_kernel(const float* __restrict__ ptok, float* __restrict__ part,
+                                                             int64_t t0, int chunk_tokens, int S, int pp, int n_first) {
   const int n = n_first + blockIdx.x;
+  const int sl = blockIdx.y;
   const int64_t lo = (int64_t)n * S > t0 ? (int64_t)n * S : t0;
   const int64_t hi_seq = (int64_t)(n + 1) * S;
   const int64_t hi = hi_seq < t0 + chunk_tokens ? hi_seq : t0 + chunk_tokens;
+  const int64_t per = (hi - lo + SEQ_SLICES - 1) / SEQ_SLICES;
+  const int64_t a = lo + sl * per;
+  const int64_t b = a + per < hi ? a + per : hi;
+  for (int e = threadIdx.x; e < pp; e += blockDim.x) {
+    float s = 0.f;
+    for (int64_t t = a; t < b; ++t) s += ptok[(t - t0) * pp + e];
+    part[((int64_t)blockIdx.x * SEQ_SLICES + sl) * pp + e] = s;
+  }
+}
+
+// acc[n, e] += the slices of sequence n, in slice order.
+__global__ __launch_bounds__(256) void adam_seq_sum_kernel(const float* __restrict__ part, float* __restrict__ acc, int pp,
+                                                           int n_first) {
+  const int n = n_first + blockIdx.x;
   for (int e = threadIdx.x; e < pp; e += blockDim.x) {
     float s = acc[(int64_t)n * pp + e];
-    for (int64_t t = lo; t < hi; ++t) s += ptok[(t - t0) * pp + e];
+    for (int sl = 0; sl < SEQ_SLICES; ++sl) s += part[((int64_t)blockIdx.x * SEQ_SLICES + sl) * pp + e];
     acc[(int64_t)n * pp + e] = s;
   }
 }
@@ -194,7 +211,7 @@ size_t collect_adam_workspace_bytes(int N, int S, int O, int p, int64_t chunk_to
   const int64_t T = (int64_t)N * S;
   const int64_t tc = adam_chunk(T, O, p, chunk_tokens);
   return align_up((size_t)tc * O * p * 4, 256) + align_up((size_t)tc * p * p * 4, 256) +
-         align_up((size_t)N * p * p * 4, 256);
+         align_up((size_t)N * p * p * 4, 256) + align_up((size_t)N * SEQ_SLICES * p * p * 4, 256);
 }
 
 int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_t a_tok_stride, int64_t g_seq_stride,
@@ -224,6 +241,7 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
   float* H = (float*)w;
   float* ptok = (float*)(w + align_up((size_t)tc * O * p * 4, 256));
   float* acc = (float*)((char*)ptok + align_up((size_t)tc * pp * 4, 256));
+  float* part = (float*)((char*)acc + align_up((size_t)N * pp * 4, 256));
   const size_t esz = dtype_size(dtype);
 
   if (!per_token) {
@@ -274,8 +292,10 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
     if (!per_token) {
       const int n_first = (int)(t0 / S);
       const int n_last = (int)((t0 + rows_c - 1) / S);
-      hipLaunchKernelGGL(adam_seq_sum_kernel, dim3((unsigned)(n_last - n_first + 1)), dim3(256), 0, st, ptok, acc, t0,
-                         (int)rows_c, S, pp, n_first);
+      const unsigned nseq = (unsigned)(n_last - n_first + 1);
+      hipLaunchKernelGGL(adam_seq_slice_kernel, dim3(nseq, SEQ_SLICES), dim3(256), 0, st, ptok, part, t0, (int)rows_c, S,
+                         pp, n_first);
+      hipLaunchKernelGGL(adam_seq_sum_kernel, dim3(nseq), dim3(256), 0, st, part, acc, pp, n_first);
       BGX_HIP(hipGetLastError());
     }
   }
