@@ -357,22 +357,38 @@ class HookCollectorBase(ContextDecorator, ABC):
             raise NotImplementedError(
                 "bergson_amd collects projected gradients only: set processor.projection_dim "
                 "(projection_target='per_module'); unprojected [O, I] gradients have no HIP kernel here")
-        if module._collect_bias:
-            raise NotImplementedError(f"{name}: include_bias=True has no HIP kernel in this build")
         if isinstance(normalizer, AdamNormalizer):
             raise AssertionError("Adam modules go through adam_prepared()")
         if not a.is_cuda or not g.is_cuda:
             raise RuntimeError("bergson_amd has no CPU path: the model must run on the GPU")
-        # an attention head shares the parent's input and right projection (collector.py:527, :540)
-        parent = self.split_head_name(name)
-        right_name = parent[0] if parent is not None and parent[0] in self.attention_cfgs else name
-        r_in = self.projection(right_name, p, i, "right", a.device, a.dtype)
         r_out = self.projection(name, p, o, "left", g.device, g.dtype)
+        bias_col = bias_scale = None
+        if module._collect_bias:
+            # with a bias the right projection has I + 1 columns and is named after the (head) module
+            # itself (collector.py:552-590); its last column multiplies the bias gradient
+            right = self.projection(name, p, i + 1, "right", a.device, a.dtype)
+            key = f"{name}|split|{a.dtype}"
+            if key not in self._scale_cache:
+                self._scale_cache[key] = (right[:, :i].contiguous(), right[:, i].float().contiguous())
+            r_in, bias_col = self._scale_cache[key]
+        else:
+            # an attention head shares the parent's input and right projection (collector.py:527, :540)
+            parent = self.split_head_name(name)
+            right_name = parent[0] if parent is not None and parent[0] in self.attention_cfgs else name
+            r_in = self.projection(right_name, p, i, "right", a.device, a.dtype)
         row_scale = col_scale = None
         if isinstance(normalizer, AdafactorNormalizer):
             row_scale, col_scale = self._scales(name, normalizer, g.dtype, g.device)
+            if module._collect_bias:
+                assert normalizer.bias_avg_sq is not None, f"{name}: bias collected but the normalizer has no bias_avg_sq"
+                key = f"{name}|bias|{g.device}"
+                if key not in self._scale_cache:
+                    # rsqrt(bias_avg_sq + 1e-8), eps inside the root (gradients.py:339-349)
+                    self._scale_cache[key] = (normalizer.bias_avg_sq.to(g.device, torch.float32).add(1e-8).rsqrt()
+                                              .contiguous(), None)
+                bias_scale = self._scale_cache[key][0]
         return ops.ModuleInput(a=a, g=g, r_in=r_in, r_out=r_out, out_col=out_col, col_scale=col_scale,
-                               row_scale=row_scale)
+                               row_scale=row_scale, bias_col=bias_col, bias_scale=bias_scale)
 
     def adam_prepared(self, module: nn.Module, g: Tensor, out_col: int) -> "ops.AdamPrepared":
         """The module's Adam table and projections, built on its first batch (collector.py:609-644)."""

@@ -193,12 +193,15 @@ __device__ inline int seq_token_limit(const int32_t* lengths, int n, int S) {
   return l < S ? (l < 0 ? 0 : l) : S;
 }
 
-template <typename T, int PB, bool ALIGNED, bool PER_TOKEN, int MT, int U>
+// BIAS: the launch contains modules whose bias gradient is collected (bias_col != NULL).  The bias adds
+// (sum_t gb'_t) (x) bias_col to P, where gb' = g' when the module has no bias_scale and otherwise a second
+// projection of g scaled by bias_scale (the Adafactor bias factor applies to the unscaled g).
+template <typename T, int PB, bool ALIGNED, bool PER_TOKEN, int MT, int U, bool BIAS = false>
 __global__ __launch_bounds__(COLLECT_THREADS) void collect_kernel(CollectArgs args) {
   constexpr int TILE_T = 16 * MT;  // tokens per workgroup
   constexpr int PP = PB * 16;      // padded projection dim
   constexpr int LDP = PP + 1;      // LDS row stride (floats)
-  __shared__ float sm[2][2][TILE_T][LDP];  // [a/g][slot][token][col]
+  __shared__ float sm[BIAS ? 3 : 2][2][TILE_T][LDP];  // [a/g/gb][slot][token][col]
 
   const int tile = blockIdx.x;
   const int m = blockIdx.y;
@@ -232,9 +235,46 @@ __global__ __launch_bounds__(COLLECT_THREADS) void collect_kernel(CollectArgs ar
   project_tile<T, PB, ALIGNED, MT, U>(g0, d.g_tok_stride, rows_valid, d.O, (const T*)d.r_out, p,
                                       d.row_scale, wave, lane, accG);
 
-  // ---- combine the 4 K-slices: (w0 + w2) + (w1 + w3), fixed order ----------
   const int r = lane & 15;
   const int q = lane >> 4;
+  const bool has_bias = BIAS && d.bias_col != nullptr;
+  const bool own_gb = has_bias && d.bias_scale != nullptr;  // bias needs its own projection of g
+  if constexpr (BIAS) {
+    if (own_gb) {
+      f32x4 accB[MT][PB];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int pb = 0; pb < PB; ++pb) accB[mt][pb] = f32x4{0.f, 0.f, 0.f, 0.f};
+      project_tile<T, PB, ALIGNED, MT, U>(g0, d.g_tok_stride, rows_valid, d.O, (const T*)d.r_out, p,
+                                          d.bias_scale, wave, lane, accB);
+      // the same pairwise combination as below, for the bias projection only
+      if (wave >= 2) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int pb = 0; pb < PB; ++pb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sm[2][wave - 2][mt * 16 + q * 4 + i][pb * 16 + r] = accB[mt][pb][i];
+      }
+      __syncthreads();
+      if (wave < 2) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int pb = 0; pb < PB; ++pb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sm[2][wave][mt * 16 + q * 4 + i][pb * 16 + r] += accB[mt][pb][i];
+      }
+      __syncthreads();
+      for (int e = tid; e < TILE_T * PP; e += COLLECT_THREADS) {
+        const int t = e / PP, c = e - t * PP;
+        sm[2][0][t][c] += sm[2][1][t][c];
+      }
+    }
+  }
+
+  // ---- combine the 4 K-slices: (w0 + w2) + (w1 + w3), fixed order ----------
   if (wave >= 2) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -263,20 +303,30 @@ __global__ __launch_bounds__(COLLECT_THREADS) void collect_kernel(CollectArgs ar
   __syncthreads();
   for (int e = tid; e < TILE_T * PP; e += COLLECT_THREADS) {
     const int t = e / PP, c = e - t * PP;
-    sm[0][0][t][c] += sm[0][1][t][c];
+    float av = sm[0][0][t][c] + sm[0][1][t][c];
+    // without a bias factor the bias shares g': (g'_t) (x) (a'_t + bias_col)
+    if (has_bias && !own_gb && c < p) av += d.bias_col[c];
+    sm[0][0][t][c] = av;
     sm[1][0][t][c] += sm[1][1][t][c];
   }
   __syncthreads();
 
   const int pp = p * p;
   if (!PER_TOKEN) {
-    // P[i, j] = sum_t g'[t, i] * a'[t, j]; tokens past rows_valid hold zeros.
+    // P[i, j] = sum_t g'[t, i] * a'[t, j] (+ gb'[t, i] * bias_col[j]); tokens past rows_valid hold zeros.
     float* dst = args.partials + (((int64_t)m * args.N + n) * args.tiles_per_seq + ts) * pp;
     for (int e = tid; e < pp; e += COLLECT_THREADS) {
       const int i = e / p, j = e - i * p;
       float s = 0.f;
 #pragma unroll 8
       for (int t = 0; t < TILE_T; ++t) s = fmaf(sm[1][0][t][i], sm[0][0][t][j], s);
+      if constexpr (BIAS) {
+        if (own_gb) {
+          float sb = 0.f;
+          for (int t = 0; t < TILE_T; ++t) sb += sm[2][0][t][i];
+          s = fmaf(sb, d.bias_col[j], s);
+        }
+      }
       dst[e] = s;
     }
   } else {
@@ -285,8 +335,11 @@ __global__ __launch_bounds__(COLLECT_THREADS) void collect_kernel(CollectArgs ar
       const int64_t base = (row0 + t) * args.out_row_stride + d.out_col;
       for (int e = lane; e < pp; e += WAVE) {
         const int i = e / p, j = e - i * p;
-        const float v = clampf(sm[1][0][t][i] * sm[0][0][t][j], args.lo, args.hi);
-        store_as(args.out, base + e, v, args.out_dtype);
+        float v = sm[1][0][t][i] * sm[0][0][t][j];
+        if constexpr (BIAS) {
+          if (own_gb) v = fmaf(sm[2][0][t][i], d.bias_col[j], v);
+        }
+        store_as(args.out, base + e, clampf(v, args.lo, args.hi), args.out_dtype);
       }
     }
   }
@@ -425,28 +478,36 @@ size_t collect_workspace_bytes(int n_modules, int N, int S, int p) {
 }
 
 template <typename T, int PB, bool ALIGNED, int MT, int U>
-static void launch_collect(bool per_token, dim3 grid, hipStream_t st, const CollectArgs& args) {
-  if (per_token)
-    hipLaunchKernelGGL((collect_kernel<T, PB, ALIGNED, true, MT, U>), grid, dim3(COLLECT_THREADS), 0, st, args);
-  else
-    hipLaunchKernelGGL((collect_kernel<T, PB, ALIGNED, false, MT, U>), grid, dim3(COLLECT_THREADS), 0, st, args);
+static void launch_collect(bool per_token, bool bias, dim3 grid, hipStream_t st, const CollectArgs& args) {
+  const dim3 block(COLLECT_THREADS);
+  if (bias) {
+    // the rarely used bias variant runs on 64-token tiles whatever MT says, to bound its LDS footprint
+    if (per_token)
+      hipLaunchKernelGGL((collect_kernel<T, PB, ALIGNED, true, 4, 1, true>), grid, block, 0, st, args);
+    else
+      hipLaunchKernelGGL((collect_kernel<T, PB, ALIGNED, false, 4, 1, true>), grid, block, 0, st, args);
+  } else if (per_token) {
+    hipLaunchKernelGGL((collect_kernel<T, PB, ALIGNED, true, MT, U>), grid, block, 0, st, args);
+  } else {
+    hipLaunchKernelGGL((collect_kernel<T, PB, ALIGNED, false, MT, U>), grid, block, 0, st, args);
+  }
 }
 
 // tokens per workgroup: 128 for the common case (p <= 16, aligned operands), else 64
-static int tile_tokens_for(int pb, bool aligned) { return (pb == 1 && aligned) ? 128 : 64; }
+static int tile_tokens_for(int pb, bool aligned, bool bias) { return (pb == 1 && aligned && !bias) ? 128 : 64; }
 
 template <typename T>
-static void launch_collect_pb(int pb, bool aligned, bool per_token, dim3 grid, hipStream_t st,
+static void launch_collect_pb(int pb, bool aligned, bool per_token, bool bias, dim3 grid, hipStream_t st,
                               const CollectArgs& args) {
   if (pb == 1) {
-    aligned ? launch_collect<T, 1, true, 8, 2>(per_token, grid, st, args)
-            : launch_collect<T, 1, false, 4, 2>(per_token, grid, st, args);
+    aligned ? launch_collect<T, 1, true, 8, 2>(per_token, bias, grid, st, args)
+            : launch_collect<T, 1, false, 4, 2>(per_token, bias, grid, st, args);
   } else if (pb == 2) {
-    aligned ? launch_collect<T, 2, true, 4, 2>(per_token, grid, st, args)
-            : launch_collect<T, 2, false, 4, 2>(per_token, grid, st, args);
+    aligned ? launch_collect<T, 2, true, 4, 2>(per_token, bias, grid, st, args)
+            : launch_collect<T, 2, false, 4, 2>(per_token, bias, grid, st, args);
   } else {
-    aligned ? launch_collect<T, 4, true, 4, 1>(per_token, grid, st, args)
-            : launch_collect<T, 4, false, 4, 1>(per_token, grid, st, args);
+    aligned ? launch_collect<T, 4, true, 4, 1>(per_token, bias, grid, st, args)
+            : launch_collect<T, 4, false, 4, 1>(per_token, bias, grid, st, args);
   }
 }
 
@@ -469,6 +530,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
 
   const int epl = in_dtype == BGX_F32 ? 4 : 8;
   bool aligned = true;
+  bool any_bias = false;
   for (int m = 0; m < n_modules; ++m) {
     const bgx_module_desc& d = mods_host[m];
     BGX_REQUIRE(d.a && d.g && d.r_in && d.r_out, BGX_E_ARG, "collect: module %d has a null a/g/r_in/r_out", m);
@@ -476,8 +538,9 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     BGX_REQUIRE(d.out_col >= 0 && d.out_col + (int64_t)p * p <= out_row_stride, BGX_E_ARG,
                 "collect: module %d columns [%lld, +%d) do not fit a row of %lld", m, (long long)d.out_col,
                 p * p, (long long)out_row_stride);
-    BGX_REQUIRE(d.bias_col == nullptr && d.bias_scale == nullptr, BGX_E_SHAPE,
-                "collect: bias column is not supported by this build");
+    BGX_REQUIRE(d.bias_col != nullptr || d.bias_scale == nullptr, BGX_E_ARG,
+                "collect: module %d has a bias_scale but no bias_col", m);
+    any_bias = any_bias || d.bias_col != nullptr;
     const bool ok = ((uintptr_t)d.a % 16 == 0) && ((uintptr_t)d.g % 16 == 0) &&
                     ((uintptr_t)d.r_in % 16 == 0) && ((uintptr_t)d.r_out % 16 == 0) &&
                     (d.I % epl == 0) && (d.O % epl == 0) && (d.a_seq_stride % epl == 0) &&
@@ -505,7 +568,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   args.S = S;
   args.p = p;
   const int pb = (p + 15) / 16;
-  const int tile_tokens = tile_tokens_for(pb, aligned);
+  const int tile_tokens = tile_tokens_for(pb, aligned, any_bias);
   args.tiles_per_seq = (S + tile_tokens - 1) / tile_tokens;
   args.partials = (float*)((char*)ws + desc_bytes(n_modules));
   args.row_offsets = per_token ? rows_or_offsets : nullptr;
@@ -521,11 +584,11 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   const bool timed = 2 * (g_timing_used + 1) <= (int)g_timing_events.size();
   if (timed) BGX_HIP(hipEventRecord(g_timing_events[2 * g_timing_used], st));
   if (in_dtype == BGX_F32)
-    launch_collect_pb<float>(pb, aligned, per_token, grid, st, args);
+    launch_collect_pb<float>(pb, aligned, per_token, any_bias, grid, st, args);
   else if (in_dtype == BGX_F16)
-    launch_collect_pb<f16_t>(pb, aligned, per_token, grid, st, args);
+    launch_collect_pb<f16_t>(pb, aligned, per_token, any_bias, grid, st, args);
   else
-    launch_collect_pb<bf16_t>(pb, aligned, per_token, grid, st, args);
+    launch_collect_pb<bf16_t>(pb, aligned, per_token, any_bias, grid, st, args);
   BGX_HIP(hipGetLastError());
   if (timed) {
     BGX_HIP(hipEventRecord(g_timing_events[2 * g_timing_used + 1], st));

@@ -100,6 +100,8 @@ class ModuleInput:
     out_col: int
     col_scale: Tensor | None = None  # [I] fp32
     row_scale: Tensor | None = None  # [O] fp32
+    bias_col: Tensor | None = None  # [p] fp32: column I of the [p, I+1] right projection
+    bias_scale: Tensor | None = None  # [O] fp32: factor of g for the bias column (None = 1)
 
 
 def _rows_view(t: Tensor, name: str) -> Tensor:
@@ -143,8 +145,11 @@ def _collect(per_token: bool, modules: list[ModuleInput], p: int, out: Tensor, l
         d.a, d.g, d.r_in, d.r_out = a.data_ptr(), g.data_ptr(), r_in.data_ptr(), r_out.data_ptr()
         d.col_scale = None if m.col_scale is None else m.col_scale.data_ptr()
         d.row_scale = None if m.row_scale is None else m.row_scale.data_ptr()
-        d.bias_col = None
-        d.bias_scale = None
+        for t_, n_, k_ in ((m.bias_col, "bias_col", p), (m.bias_scale, "bias_scale", O)):
+            if t_ is not None and (t_.dtype != torch.float32 or t_.numel() != k_ or not t_.is_contiguous()):
+                raise ValueError(f"{n_} must be a contiguous fp32 vector of {k_} elements")
+        d.bias_col = None if m.bias_col is None else m.bias_col.data_ptr()
+        d.bias_scale = None if m.bias_scale is None else m.bias_scale.data_ptr()
         d.a_seq_stride, d.a_tok_stride = a.stride(0), a.stride(1)
         d.g_seq_stride, d.g_tok_stride = g.stride(0), g.stride(1)
         d.out_col = m.out_col
@@ -197,13 +202,17 @@ class PreparedModule:
                 raise ValueError(f"{n} must be a contiguous fp32 vector of {k} elements")
         for t in (m.a, m.g, self.r_in, self.r_out):
             _need_gpu(t, "module operand")
+        for s, n, k in ((m.bias_col, "bias_col", p), (m.bias_scale, "bias_scale", O)):
+            if s is not None and (s.dtype != torch.float32 or s.numel() != k or not s.is_contiguous()):
+                raise ValueError(f"{n} must be a contiguous fp32 vector of {k} elements")
         self.col_scale, self.row_scale = m.col_scale, m.row_scale
+        self.bias_col, self.bias_scale = m.bias_col, m.bias_scale
         d = ModuleDesc()
         d.r_in, d.r_out = self.r_in.data_ptr(), self.r_out.data_ptr()
         d.col_scale = None if m.col_scale is None else m.col_scale.data_ptr()
         d.row_scale = None if m.row_scale is None else m.row_scale.data_ptr()
-        d.bias_col = None
-        d.bias_scale = None
+        d.bias_col = None if m.bias_col is None else m.bias_col.data_ptr()
+        d.bias_scale = None if m.bias_scale is None else m.bias_scale.data_ptr()
         d.out_col, d.I, d.O = m.out_col, I, O
         self.template = d
 

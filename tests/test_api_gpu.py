@@ -177,3 +177,33 @@ def test_attributor_search_and_trace(device, tmp_path):
         loss.backward()
         gpu.zero_grad()
     assert result.indices[0, 0].item() == 3 and result.scores[0, 0].item() > 0.99
+
+
+def test_include_bias_end_to_end(device):
+    """include_bias=True through the collector: every module's block against the oracle on captured (a, g)."""
+    from bergson_amd import GradientCollector, GradientProcessor, IndexConfig
+    from bergson_amd.collector import CollectorComputer
+
+    lengths = [30, 22]
+    docs, data, batches, cpu, gpu = _setup(device, lengths, layers=1)
+    names = list(oloop.target_linears(cpu.base_model))
+    captured = {}
+    handles = []
+    for name in names:
+        mod = gpu.base_model.get_submodule(name)
+        handles.append(mod.register_forward_hook(
+            lambda m, inp, out, name=name: captured.setdefault(name, {}).__setitem__("a", inp[0].detach().cpu())))
+        handles.append(mod.register_full_backward_hook(
+            lambda m, gin, gout, name=name: captured[name].__setitem__("g", gout[0].detach().cpu())))
+    cfg = IndexConfig(projection_dim=16, projection_type="normal", include_bias=True)
+    proc = GradientProcessor(projection_dim=16, projection_type="normal", include_bias=True)
+    col = GradientCollector(model=gpu.base_model, cfg=cfg, data=data, processor=proc)
+    CollectorComputer(model=gpu, data=data, collector=col, batches=[[0, 1]], cfg=cfg).run_with_collector_hooks()
+    for h in handles:
+        h.remove()
+    got = torch.from_numpy(np.array(col.builder.grad_buffer))
+    for b, name in enumerate(names):
+        a, g = captured[name]["a"], captured[name]["g"]
+        left, right = module_projections(name, 16, g.shape[-1], a.shape[-1], torch.float32, collect_bias=True)
+        want = ohooks.module_gradient(a, g, None, left, right, collect_bias=True)
+        assert rel_l2(got[:, b * 256:(b + 1) * 256], want) <= 1e-4, name

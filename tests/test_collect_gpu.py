@@ -279,3 +279,48 @@ def test_adam_tok(device, dtype):
     want = ohooks.module_gradient(a, g, norm, left, right, attribute_tokens=True, collection_mask=mask)
     assert rel_l2(got[:, 256:512], want) <= TOL[dtype]
     assert got[:, :256].abs().sum() == 0 and got[:, 512:].abs().sum() == 0
+
+
+# ---- bias column -------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("normalizer", [None, "adafactor"])
+@pytest.mark.parametrize("per_token", [False, True])
+def test_bias_column(device, dtype, normalizer, per_token):
+    from bergson_amd import ops
+
+    N, S, I, O, p = 2, 90, 96, 64, 16
+    gen = torch.Generator().manual_seed(60)
+    a = torch.randn(N, S, I, generator=gen).to(dtype)
+    g = (torch.randn(N, S, O, generator=gen) * 0.1).to(dtype)
+    lengths = [90, 47]
+    for n, l in enumerate(lengths):
+        g[n, l - 1:] = 0
+    left, right = module_projections("layers.0.mlp.dense_4h_to_h", p, O, I, dtype, collect_bias=True)
+    assert right.shape == (p, I + 1)
+    norm = None
+    rs = cs = bs = None
+    if normalizer:
+        # second moments in the model dtype, as the reference's arithmetic needs for a bias with a 16-bit model
+        row = (torch.rand(O, generator=gen) + 0.1).to(dtype)
+        col = (torch.rand(I, generator=gen) + 0.1).to(dtype)
+        bsq = (torch.rand(O, generator=gen) + 0.1).to(dtype)
+        norm = ohooks.Adafactor(row=row, col=col, bias_avg_sq=bsq)
+        rs, cs = ops.adafactor_scales(row.to(device), col.to(device), dtype)
+        bs = (bsq.to(device).float() + 1e-8).rsqrt().contiguous()
+    mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+    want = ohooks.module_gradient(a, g, norm, left, right, collect_bias=True, attribute_tokens=per_token,
+                                  collection_mask=mask if per_token else None)
+    mi = ops.ModuleInput(a=a.to(device), g=g.to(device), r_in=right[:, :I].contiguous().to(device),
+                         r_out=left.to(device), out_col=0, col_scale=cs, row_scale=rs,
+                         bias_col=right[:, I].float().contiguous().to(device), bias_scale=bs)
+    if per_token:
+        out = torch.zeros(sum(l - 1 for l in lengths), p * p, dtype=dtype, device=device)
+        ops.collect_tok([mi], p, out, lengths=torch.tensor(lengths, dtype=torch.int32, device=device),
+                        row_offsets=torch.tensor([0, lengths[0] - 1], dtype=torch.int64, device=device))
+    else:
+        out = torch.zeros(N, p * p, dtype=dtype, device=device)
+        ops.collect_seq([mi], p, out)
+    torch.cuda.synchronize()
+    assert out.shape == want.shape
+    assert rel_l2(out.cpu(), want) <= TOL[dtype]
