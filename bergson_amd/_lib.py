@@ -62,8 +62,9 @@ SIGNATURES: dict[str, tuple] = {
     "bgx_collect_adam": (
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32,
-         C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p,
-         C.c_int64, C.c_int64, C.c_int32, C.c_float, C.c_float, C.c_void_p, C.c_size_t, C.c_int64, C.c_void_p],
+         C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p,
+         C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int32, C.c_float, C.c_float, C.c_void_p, C.c_size_t,
+         C.c_int64, C.c_void_p],
     ),
     "bgx_collect_timing_enable": (C.c_int, [C.c_int32]),
     "bgx_collect_timing_read": (C.c_int, [C.POINTER(C.c_float), C.c_int32, C.POINTER(C.c_int32)]),

@@ -400,19 +400,25 @@ class HookCollectorBase(ContextDecorator, ABC):
         p = self.per_module_projection_dim
         if p is None:
             raise NotImplementedError("bergson_amd collects projected gradients only: set processor.projection_dim")
-        if module._collect_bias:
-            raise NotImplementedError(f"{name}: include_bias=True has no HIP kernel in this build")
         if not g.is_cuda:
             raise RuntimeError("bergson_amd has no CPU path: the model must run on the GPU")
         normalizer = self.normalizer_for(name)
         assert isinstance(normalizer, AdamNormalizer)
         i = getattr(module, LayerAdapter.in_attr(module))
         o = getattr(module, LayerAdapter.out_attr(module))
-        parent = self.split_head_name(name)
-        right_name = parent[0] if parent is not None and parent[0] in self.attention_cfgs else name
-        r_in = self.projection(right_name, p, i, "right", g.device, g.dtype)
         r_out = self.projection(name, p, o, "left", g.device, g.dtype)
-        prep = ops.AdamPrepared(r_in, r_out, normalizer.weight_avg_sq, out_col)
+        if module._collect_bias:
+            # the projection runs on [grad | bias_grad]: I + 1 columns, named after the module itself
+            # (collector.py:626-644)
+            assert normalizer.bias_avg_sq is not None, f"{name}: bias collected but the normalizer has no bias_avg_sq"
+            right = self.projection(name, p, i + 1, "right", g.device, g.dtype)
+            prep = ops.AdamPrepared(right[:, :i].contiguous(), r_out, normalizer.weight_avg_sq, out_col,
+                                    bias_col=right[:, i], bias_avg_sq=normalizer.bias_avg_sq)
+        else:
+            parent = self.split_head_name(name)
+            right_name = parent[0] if parent is not None and parent[0] in self.attention_cfgs else name
+            r_in = self.projection(right_name, p, i, "right", g.device, g.dtype)
+            prep = ops.AdamPrepared(r_in, r_out, normalizer.weight_avg_sq, out_col)
         self._adam_prepared[key] = prep
         return prep
 

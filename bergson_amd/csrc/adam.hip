@@ -59,6 +59,9 @@ struct ContractArgs {
   float lo, hi;
   // per-sequence: per-token fp32 rows of the chunk
   float* ptok;           // [chunk_tokens, p * p]
+  // bias column (both NULL when the bias is not collected)
+  const float* bias_col;    // [p]  column I of the [p, I+1] right projection
+  const float* bias_scale;  // [O]  1 / (sqrt(bias_avg_sq) + 1e-8)
 };
 
 constexpr int CONTRACT_OC = 32;  // output features staged per step
@@ -68,6 +71,7 @@ template <typename T, bool PER_TOKEN>
 __global__ __launch_bounds__(256) void adam_contract_kernel(ContractArgs a) {
   __shared__ float s_lg[CONTRACT_OC][65];  // [o][i]  L[i, o] * g_t[o]
   __shared__ float s_h[CONTRACT_OC][65];   // [o][j]
+  __shared__ float s_bs[CONTRACT_OC];      // bias factor of the staged output features
   const int tl = blockIdx.x;
   const int64_t t = a.t0 + tl;
   const int n = (int)(t / a.S);
@@ -77,9 +81,13 @@ __global__ __launch_bounds__(256) void adam_contract_kernel(ContractArgs a) {
   if (a.lengths != nullptr) valid = s < a.lengths[n] - 1;
   if (PER_TOKEN && !valid) return;
   const int tid = threadIdx.x;
-  float acc[16];  // p*p <= 4096 outputs over 256 threads
+  float acc[16];   // p*p <= 4096 outputs over 256 threads
+  float accb[16];  // sum_o L[i, o] g[o] bias_scale[o] of each output's row i
 #pragma unroll
-  for (int c = 0; c < 16; ++c) acc[c] = 0.f;
+  for (int c = 0; c < 16; ++c) {
+    acc[c] = 0.f;
+    accb[c] = 0.f;
+  }
   if (valid) {
     const T* g = (const T*)a.g + (int64_t)n * a.g_seq_stride + (int64_t)s * a.g_tok_stride;
     const T* L = (const T*)a.r_out;
@@ -92,6 +100,7 @@ __global__ __launch_bounds__(256) void adam_contract_kernel(ContractArgs a) {
         s_lg[oo][x] = Elem<T>::load(L + (int64_t)x * a.O + o0 + oo) * Elem<T>::load(g + o0 + oo);
         s_h[oo][x] = H[(int64_t)(o0 + oo) * p + x];
       }
+      if (a.bias_col != nullptr && tid < oc) s_bs[tid] = a.bias_scale[o0 + tid];
       __syncthreads();
 #pragma unroll
       for (int c = 0; c < 16; ++c) {
@@ -101,8 +110,20 @@ __global__ __launch_bounds__(256) void adam_contract_kernel(ContractArgs a) {
           float sum = acc[c];
           for (int oo = 0; oo < oc; ++oo) sum = fmaf(s_lg[oo][i], s_h[oo][j], sum);
           acc[c] = sum;
+          if (a.bias_col != nullptr) {
+            float sb = accb[c];
+            for (int oo = 0; oo < oc; ++oo) sb = fmaf(s_lg[oo][i], s_bs[oo], sb);
+            accb[c] = sb;
+          }
         }
       }
+    }
+  }
+  if (a.bias_col != nullptr) {
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+      const int e = tid + c * 256;
+      if (e < pp) acc[c] = fmaf(accb[c], a.bias_col[e % p], acc[c]);
     }
   }
   if (PER_TOKEN) {
@@ -216,10 +237,13 @@ size_t collect_adam_workspace_bytes(int N, int S, int O, int p, int64_t chunk_to
 
 int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_t a_tok_stride, int64_t g_seq_stride,
                       int64_t g_tok_stride, int N, int S, int I, int O, int p, int dtype, const void* table,
-                      const void* r_out, int per_token, const int32_t* lengths, const int64_t* rows, void* out,
-                      int64_t out_row_stride, int64_t out_col, int out_dtype, float lo, float hi, void* ws,
-                      size_t ws_bytes, int64_t chunk_tokens, void* stream) {
+                      const void* r_out, const float* bias_col, const float* bias_scale, int per_token,
+                      const int32_t* lengths, const int64_t* rows, void* out, int64_t out_row_stride, int64_t out_col,
+                      int out_dtype, float lo, float hi, void* ws, size_t ws_bytes, int64_t chunk_tokens,
+                      void* stream) {
   BGX_REQUIRE(a && g && table && r_out && out && ws, BGX_E_ARG, "collect_adam: null pointer");
+  BGX_REQUIRE((bias_col == nullptr) == (bias_scale == nullptr), BGX_E_ARG,
+              "collect_adam: bias_col and bias_scale go together");
   BGX_REQUIRE(N > 0 && S > 0 && I > 0 && O > 0, BGX_E_ARG, "collect_adam: N=%d S=%d I=%d O=%d", N, S, I, O);
   BGX_REQUIRE(p >= 1 && p <= 64, BGX_E_SHAPE, "collect_adam: p=%d outside 1..64", p);
   BGX_REQUIRE(dtype >= BGX_F32 && dtype <= BGX_BF16 && out_dtype >= BGX_F32 && out_dtype <= BGX_BF16, BGX_E_DTYPE,
@@ -274,6 +298,8 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
     c.lo = lo;
     c.hi = hi;
     c.ptok = ptok;
+    c.bias_col = bias_col;
+    c.bias_scale = bias_scale;
     const dim3 grid((unsigned)rows_c), block(256);
 #define BGX_CONTRACT(T_)                                                                         \
   if (per_token)                                                                                 \

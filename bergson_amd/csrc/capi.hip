@@ -31,9 +31,10 @@ int adam_prepare_impl(const void* r_in, const float* v, int O, int I, int p, int
 size_t collect_adam_workspace_bytes(int N, int S, int O, int p, int64_t chunk_tokens);
 int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_t a_tok_stride, int64_t g_seq_stride,
                       int64_t g_tok_stride, int N, int S, int I, int O, int p, int dtype, const void* table,
-                      const void* r_out, int per_token, const int32_t* lengths, const int64_t* rows, void* out,
-                      int64_t out_row_stride, int64_t out_col, int out_dtype, float lo, float hi, void* ws,
-                      size_t ws_bytes, int64_t chunk_tokens, void* stream);
+                      const void* r_out, const float* bias_col, const float* bias_scale, int per_token,
+                      const int32_t* lengths, const int64_t* rows, void* out, int64_t out_row_stride, int64_t out_col,
+                      int out_dtype, float lo, float hi, void* ws, size_t ws_bytes, int64_t chunk_tokens,
+                      void* stream);
 int collect_timing_enable(int max_launches);
 int collect_timing_read(float* ms_out, int capacity, int* count_out);
 int unit_normalize_impl(void* rows, int64_t n_rows, int64_t D, int64_t stride, int dtype, void* stream);
@@ -91,12 +92,14 @@ size_t bgx_collect_adam_workspace_bytes(int32_t N, int32_t S, int32_t O, int32_t
 
 int bgx_collect_adam(const void* a_dev, const void* g_dev, int64_t a_seq_stride, int64_t a_tok_stride,
                      int64_t g_seq_stride, int64_t g_tok_stride, int32_t N, int32_t S, int32_t I, int32_t O, int32_t p,
-                     int32_t dtype, const void* table_dev, const void* r_out_dev, int32_t per_token,
-                     const int32_t* lengths_dev, const int64_t* rows_dev, void* out_dev, int64_t out_row_stride,
+                     int32_t dtype, const void* table_dev, const void* r_out_dev, const float* bias_col_dev,
+                     const float* bias_scale_dev, int32_t per_token, const int32_t* lengths_dev,
+                     const int64_t* rows_dev, void* out_dev, int64_t out_row_stride,
                      int64_t out_col, int32_t out_dtype, float clamp_lo, float clamp_hi, void* workspace_dev,
                      size_t workspace_bytes, int64_t chunk_tokens, void* stream) {
   return bgx::collect_adam_impl(a_dev, g_dev, a_seq_stride, a_tok_stride, g_seq_stride, g_tok_stride, N, S, I, O, p,
-                                dtype, table_dev, r_out_dev, per_token, lengths_dev, rows_dev, out_dev, out_row_stride,
+                                dtype, table_dev, r_out_dev, bias_col_dev, bias_scale_dev, per_token, lengths_dev,
+                                rows_dev, out_dev, out_row_stride,
                                 out_col, out_dtype, clamp_lo, clamp_hi, workspace_dev, workspace_bytes, chunk_tokens,
                                 stream);
 }

@@ -269,7 +269,8 @@ class AdamPrepared:
     """Per-module state of the Adam path: the [(O*p), I] table built from the right projection and the
     second moments, and the left projection."""
 
-    def __init__(self, r_in: Tensor, r_out: Tensor, weight_avg_sq: Tensor, out_col: int):
+    def __init__(self, r_in: Tensor, r_out: Tensor, weight_avg_sq: Tensor, out_col: int,
+                 bias_col: Tensor | None = None, bias_avg_sq: Tensor | None = None):
         lib = _lib.load()
         _need_gpu(r_in, "r_in")
         p, I = r_in.shape
@@ -281,6 +282,14 @@ class AdamPrepared:
         self.p, self.I, self.O, self.out_col = p, I, O, out_col
         self.r_in = r_in.contiguous()
         self.r_out = r_out.contiguous()
+        self.bias_col = self.bias_scale = None
+        if bias_col is not None:
+            if bias_avg_sq is None:
+                raise ValueError("the bias column needs bias_avg_sq")
+            self.bias_col = bias_col.detach().to(device=r_in.device, dtype=torch.float32).contiguous()
+            # 1 / (sqrt(bias_avg_sq) + 1e-8): eps outside the root
+            self.bias_scale = (bias_avg_sq.detach().to(device=r_in.device, dtype=torch.float32).sqrt() + 1e-8
+                               ).reciprocal().contiguous()
         v = weight_avg_sq.detach().to(device=r_in.device, dtype=torch.float32).contiguous()
         nbytes = lib.bgx_adam_table_bytes(O, I, p, dtype_code(self.dtype))
         self.table = torch.empty(nbytes // self.r_in.element_size(), dtype=self.dtype, device=r_in.device)
@@ -311,7 +320,8 @@ def collect_adam(prep: AdamPrepared, a: Tensor, g: Tensor, out: Tensor, *, per_t
     nbytes = lib.bgx_collect_adam_workspace_bytes(N, S, O, prep.p, chunk_tokens)
     ws = _workspace(out.device, nbytes, "adam")
     rc = lib.bgx_collect_adam(_ptr(a), _ptr(g), a.stride(0), a.stride(1), g.stride(0), g.stride(1), N, S, I, O, prep.p,
-                              dtype_code(prep.dtype), _ptr(prep.table), _ptr(prep.r_out), int(per_token), _ptr(lengths),
+                              dtype_code(prep.dtype), _ptr(prep.table), _ptr(prep.r_out), _ptr(prep.bias_col),
+                              _ptr(prep.bias_scale), int(per_token), _ptr(lengths),
                               _ptr(rows), _ptr(out), out.stride(0), prep.out_col, dtype_code(out.dtype), lo, hi,
                               _ptr(ws), ws.numel(), chunk_tokens, _stream())
     _lib.check(rc, "bgx_collect_adam")

@@ -146,6 +146,10 @@ int bgx_collect_tok(const bgx_module_desc* mods_host, int32_t n_modules,
  * per token t and writes either every valid token's row (per_token != 0:
  * row row_offsets[n] + s, s < lengths[n] - 1) or the sum over each sequence
  * (per_token == 0: row rows[n], or n when rows is NULL), clamped and cast.
+ * bias_col_dev [p] / bias_scale_dev [O] (both or neither): when the bias
+ * gradient is collected, column I of the [p, I+1] right projection and
+ * 1 / (sqrt(bias_avg_sq) + 1e-8) (gradients.py:390-400); they add
+ * (sum_o r_out[i, o] g_t[o] bias_scale[o]) * bias_col[j] to P_t[i, j].
  * a must be uniformly strided over the flattened tokens
  * (a_seq_stride == S * a_tok_stride).  chunk_tokens = 0 picks the number of
  * tokens per internal pass. */
@@ -160,6 +164,7 @@ int bgx_collect_adam(const void* a_dev, const void* g_dev,
                      int64_t g_seq_stride, int64_t g_tok_stride, int32_t N,
                      int32_t S, int32_t I, int32_t O, int32_t p, int32_t dtype,
                      const void* table_dev, const void* r_out_dev,
+                     const float* bias_col_dev, const float* bias_scale_dev,
                      int32_t per_token, const int32_t* lengths_dev,
                      const int64_t* rows_dev, void* out_dev,
                      int64_t out_row_stride, int64_t out_col,

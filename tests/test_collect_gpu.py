@@ -324,3 +324,35 @@ def test_bias_column(device, dtype, normalizer, per_token):
     torch.cuda.synchronize()
     assert out.shape == want.shape
     assert rel_l2(out.cpu(), want) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("per_token", [False, True])
+def test_adam_with_bias(device, per_token):
+    from bergson_amd import ops
+
+    N, S, I, O, p = 2, 40, 64, 48, 16
+    lengths = [40, 19]
+    gen = torch.Generator().manual_seed(70)
+    a = torch.randn(N, S, I, generator=gen)
+    g = torch.randn(N, S, O, generator=gen) * 0.1
+    for n, l in enumerate(lengths):
+        g[n, l - 1:] = 0
+    left, right = module_projections("layers.2.attention.dense", p, O, I, torch.float32, collect_bias=True)
+    norm = ohooks.Adam(weight_avg_sq=torch.rand(O, I, generator=gen) * 1e-4 + 1e-8,
+                       bias_avg_sq=torch.rand(O, generator=gen) * 1e-4 + 1e-8)
+    mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+    want = ohooks.module_gradient(a, g, norm, left, right, collect_bias=True, attribute_tokens=per_token,
+                                  collection_mask=mask if per_token else None)
+    prep = ops.AdamPrepared(right[:, :I].contiguous().to(device), left.to(device), norm.weight_avg_sq.to(device), 0,
+                            bias_col=right[:, I].to(device), bias_avg_sq=norm.bias_avg_sq.to(device))
+    ldev = torch.tensor(lengths, dtype=torch.int32, device=device)
+    if per_token:
+        out = torch.zeros(sum(l - 1 for l in lengths), p * p, device=device)
+        ops.collect_adam(prep, a.to(device), g.to(device), out, per_token=True, lengths=ldev,
+                         rows=torch.tensor([0, lengths[0] - 1], dtype=torch.int64, device=device), lo=-3e38, hi=3e38)
+    else:
+        out = torch.zeros(N, p * p, device=device)
+        ops.collect_adam(prep, a.to(device), g.to(device), out, per_token=False, lengths=None, rows=None, lo=-3e38,
+                         hi=3e38)
+    torch.cuda.synchronize()
+    assert rel_l2(out.cpu(), want) <= 1e-5
