@@ -18,6 +18,7 @@
 // are combined through LDS in a fixed pairwise order (w0+w2)+(w1+w3).
 
 #include <algorithm>
+#include <type_traits>
 #include <vector>
 
 #include "common.hpp"
@@ -102,9 +103,14 @@ __device__ inline uint4 load_frag(const T* __restrict__ row, int k0, int K) {
   return v;
 }
 
-// x' = x @ (R * scale)^T for the 64 tokens of the tile, this wave's share of K.
-//   xrow0: pointer to token s0 of the sequence; rows s >= s_limit read as zero.
+// x' = x @ (R * scale)^T for the 16*MT tokens of the tile, this wave's share of K (k-steps wave, wave+4, ...).
+//   xrow0: pointer to the tile's first token.
 //   acc[mt][pb][i] belongs to token mt*16 + (lane/16)*4 + i, column pb*16 + lane%16.
+// ALIGNED (the fast path; K is a multiple of the k-step and everything is 16-byte aligned): every load is
+// unconditional.  Token rows past rows_valid and projection rows past p re-read a valid row instead of
+// being masked -- a select on loaded data would make the wave wait for each load before issuing the
+// next -- so those accumulator entries hold garbage; the caller zeroes the token rows, and columns >= p
+// are never read.  !ALIGNED: element-wise guarded loads, rows and columns out of range read as zero.
 template <typename T, int PB, bool ALIGNED, int MT, int U>
 __device__ inline void project_tile(const T* __restrict__ xrow0, int64_t tok_stride, int rows_valid,
                                     int K, const T* __restrict__ R, int p,
@@ -120,7 +126,7 @@ __device__ inline void project_tile(const T* __restrict__ xrow0, int64_t tok_str
   for (int mt = 0; mt < MT; ++mt) {
     const int t = mt * 16 + r;
     xok[mt] = t < rows_valid;
-    xrow[mt] = xrow0 + (int64_t)t * tok_stride;
+    xrow[mt] = xrow0 + (int64_t)(ALIGNED ? min(t, rows_valid - 1) : t) * tok_stride;
   }
   const T* rrow[PB];
   bool rok[PB];
@@ -128,49 +134,73 @@ __device__ inline void project_tile(const T* __restrict__ xrow0, int64_t tok_str
   for (int pb = 0; pb < PB; ++pb) {
     const int j = pb * 16 + r;
     rok[pb] = j < p;
-    rrow[pb] = R + (int64_t)j * K;
+    rrow[pb] = R + (int64_t)(ALIGNED ? min(j, p - 1) : j) * K;
   }
 
   const int nsteps = (K + M::KS - 1) / M::KS;
-  for (int ks0 = wave; ks0 < nsteps; ks0 += 4 * U) {
-    uint4 xf[U][MT];
-    uint4 rf[U][PB];
+
+  // UU consecutive k-steps of this wave starting at step ks0: all loads first, then the MFMAs
+  auto run = [&](int ks0, auto uu_tag) {
+    constexpr int UU = decltype(uu_tag)::value;
+    uint4 xf[UU][MT];
+    uint4 rf[UU][PB];
+    float sc[UU][M::EPL];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int k0 = (ks0 + 4 * u) * M::KS + q * M::EPL;  // >= K when the step is past the end
+    for (int u = 0; u < UU; ++u) {
+      const int k0 = (ks0 + 4 * u) * M::KS + q * M::EPL;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        xf[u][mt] = make_uint4(0u, 0u, 0u, 0u);
-        if (mt * 16 < rows_valid && xok[mt]) xf[u][mt] = load_frag<T, ALIGNED>(xrow[mt], k0, K);
+        if (ALIGNED) {
+          xf[u][mt] = *reinterpret_cast<const uint4*>(xrow[mt] + k0);
+        } else {
+          xf[u][mt] = make_uint4(0u, 0u, 0u, 0u);
+          if (xok[mt]) xf[u][mt] = load_frag<T, false>(xrow[mt], k0, K);
+        }
       }
 #pragma unroll
       for (int pb = 0; pb < PB; ++pb) {
-        rf[u][pb] = make_uint4(0u, 0u, 0u, 0u);
-        if (rok[pb]) rf[u][pb] = load_frag<T, ALIGNED>(rrow[pb], k0, K);
+        if (ALIGNED) {
+          rf[u][pb] = *reinterpret_cast<const uint4*>(rrow[pb] + k0);
+        } else {
+          rf[u][pb] = make_uint4(0u, 0u, 0u, 0u);
+          if (rok[pb]) rf[u][pb] = load_frag<T, false>(rrow[pb], k0, K);
+        }
+      }
+      if (scale != nullptr) {
+        if (ALIGNED) {
+#pragma unroll
+          for (int e = 0; e < M::EPL; e += 4) {
+            const float4 v = *reinterpret_cast<const float4*>(scale + k0 + e);
+            sc[u][e] = v.x;
+            sc[u][e + 1] = v.y;
+            sc[u][e + 2] = v.z;
+            sc[u][e + 3] = v.w;
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < M::EPL; ++e) sc[u][e] = (k0 + e < K) ? scale[k0 + e] : 0.f;
+        }
       }
     }
     if (scale != nullptr) {
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int k0 = (ks0 + 4 * u) * M::KS + q * M::EPL;
+      for (int u = 0; u < UU; ++u)
 #pragma unroll
-        for (int e = 0; e < M::EPL; ++e) {
-          const float sc = (k0 + e < K) ? scale[k0 + e] : 0.f;
+        for (int e = 0; e < M::EPL; ++e)
 #pragma unroll
-          for (int pb = 0; pb < PB; ++pb) M::set(rf[u][pb], e, M::get(rf[u][pb], e) * sc);
-        }
-      }
+          for (int pb = 0; pb < PB; ++pb) M::set(rf[u][pb], e, M::get(rf[u][pb], e) * sc[u][e]);
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int u = 0; u < UU; ++u)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        if (mt * 16 < rows_valid) {
+      for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-          for (int pb = 0; pb < PB; ++pb) M::mma(xf[u][mt], rf[u][pb], acc[mt][pb]);
-        }
-      }
-  }
+        for (int pb = 0; pb < PB; ++pb) M::mma(xf[u][mt], rf[u][pb], acc[mt][pb]);
+  };
+
+  int ks0 = wave;
+  for (; ks0 + 4 * (U - 1) < nsteps; ks0 += 4 * U) run(ks0, std::integral_constant<int, U>{});
+  for (; ks0 < nsteps; ks0 += 4) run(ks0, std::integral_constant<int, 1>{});
 }
 
 struct CollectArgs {
@@ -255,7 +285,8 @@ __global__ __launch_bounds__(COLLECT_THREADS) void collect_kernel(CollectArgs ar
 #pragma unroll
           for (int pb = 0; pb < PB; ++pb)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) sm[2][wave - 2][mt * 16 + q * 4 + i][pb * 16 + r] = accB[mt][pb][i];
+            for (int i = 0; i < 4; ++i)
+              sm[2][wave - 2][mt * 16 + q * 4 + i][pb * 16 + r] = (mt * 16 + q * 4 + i < rows_valid) ? accB[mt][pb][i] : 0.f;
       }
       __syncthreads();
       if (wave < 2) {
@@ -264,7 +295,8 @@ __global__ __launch_bounds__(COLLECT_THREADS) void collect_kernel(CollectArgs ar
 #pragma unroll
           for (int pb = 0; pb < PB; ++pb)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) sm[2][wave][mt * 16 + q * 4 + i][pb * 16 + r] += accB[mt][pb][i];
+            for (int i = 0; i < 4; ++i)
+              sm[2][wave][mt * 16 + q * 4 + i][pb * 16 + r] += (mt * 16 + q * 4 + i < rows_valid) ? accB[mt][pb][i] : 0.f;
       }
       __syncthreads();
       for (int e = tid; e < TILE_T * PP; e += COLLECT_THREADS) {
@@ -283,8 +315,9 @@ __global__ __launch_bounds__(COLLECT_THREADS) void collect_kernel(CollectArgs ar
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int t = mt * 16 + q * 4 + i;
-          sm[0][wave - 2][t][pb * 16 + r] = accA[mt][pb][i];
-          sm[1][wave - 2][t][pb * 16 + r] = accG[mt][pb][i];
+          const bool live = t < rows_valid;  // rows past the tile's last token hold garbage on the fast path
+          sm[0][wave - 2][t][pb * 16 + r] = live ? accA[mt][pb][i] : 0.f;
+          sm[1][wave - 2][t][pb * 16 + r] = live ? accG[mt][pb][i] : 0.f;
         }
   }
   __syncthreads();
@@ -296,8 +329,9 @@ __global__ __launch_bounds__(COLLECT_THREADS) void collect_kernel(CollectArgs ar
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int t = mt * 16 + q * 4 + i;
-          sm[0][wave][t][pb * 16 + r] += accA[mt][pb][i];
-          sm[1][wave][t][pb * 16 + r] += accG[mt][pb][i];
+          const bool live = t < rows_valid;
+          sm[0][wave][t][pb * 16 + r] += live ? accA[mt][pb][i] : 0.f;
+          sm[1][wave][t][pb * 16 + r] += live ? accG[mt][pb][i] : 0.f;
         }
   }
   __syncthreads();
@@ -529,6 +563,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   BGX_REQUIRE(((uintptr_t)ws & 255) == 0, BGX_E_ALIGN, "collect: workspace must be 256-byte aligned");
 
   const int epl = in_dtype == BGX_F32 ? 4 : 8;
+  const int kstep = in_dtype == BGX_F32 ? 16 : 32;
   bool aligned = true;
   bool any_bias = false;
   for (int m = 0; m < n_modules; ++m) {
@@ -543,7 +578,10 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     any_bias = any_bias || d.bias_col != nullptr;
     const bool ok = ((uintptr_t)d.a % 16 == 0) && ((uintptr_t)d.g % 16 == 0) &&
                     ((uintptr_t)d.r_in % 16 == 0) && ((uintptr_t)d.r_out % 16 == 0) &&
-                    (d.I % epl == 0) && (d.O % epl == 0) && (d.a_seq_stride % epl == 0) &&
+                    (d.I % kstep == 0) && (d.O % kstep == 0) && (d.a_seq_stride % epl == 0) &&
+                    (d.col_scale == nullptr || (uintptr_t)d.col_scale % 16 == 0) &&
+                    (d.row_scale == nullptr || (uintptr_t)d.row_scale % 16 == 0) &&
+                    (d.bias_scale == nullptr || (uintptr_t)d.bias_scale % 16 == 0) &&
                     (d.a_tok_stride % epl == 0) && (d.g_seq_stride % epl == 0) &&
                     (d.g_tok_stride % epl == 0);
     aligned = aligned && ok;

@@ -487,11 +487,19 @@ static ScanLayout scan_layout(int Q, int k, int64_t chunk_rows) {
   return l;
 }
 
-static int64_t effective_chunk(int64_t chunk_rows) { return chunk_rows > 0 ? chunk_rows : SCAN_DEFAULT_CHUNK; }
+// Rows per pass: the candidate lists hold one entry per (query, row of a pass) in the worst case, so the
+// default keeps Q * chunk near 64 Mi entries (512 MB) -- 65536 rows at 1024 queries, more for fewer.
+static int64_t effective_chunk(int64_t chunk_rows, int Q) {
+  if (chunk_rows > 0) return chunk_rows;
+  int64_t c = ((int64_t)64 << 20) / (Q > 0 ? Q : 1);
+  if (c > ((int64_t)1 << 20)) c = (int64_t)1 << 20;
+  if (c < SCAN_DEFAULT_CHUNK) c = SCAN_DEFAULT_CHUNK;
+  return c / 256 * 256;
+}
 
 size_t scan_workspace_bytes(int Q, int k, int64_t chunk_rows) {
   if (Q <= 0 || k < 0) return 0;
-  return scan_layout(Q, k, effective_chunk(chunk_rows)).total;
+  return scan_layout(Q, k, effective_chunk(chunk_rows, Q)).total;
 }
 
 template <typename T, int BM, int BN, int WM, int WN>
@@ -584,7 +592,7 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
   } else {
     k = 0;
   }
-  const int64_t chunk = effective_chunk(chunk_rows);
+  const int64_t chunk = effective_chunk(chunk_rows, Q);
   const ScanLayout lay = scan_layout(Q, k, chunk);
   const bool need_init = want_topk || row_max != nullptr;
   if (want_topk) {
