@@ -5,6 +5,7 @@ The public names mirror the part of `bergson`'s surface that sits on that path
 HIP kernels behind the C ABI of `include/bergson_amd.h`; there is no CPU path.
 """
 from .attributor import Attributor
+from .build import build, create_processor
 from .builder import Builder
 from .collection import collect_gradients
 from .collector import CollectorComputer, HookCollectorBase, create_projection_matrix, fwd_bwd_factory
@@ -24,6 +25,7 @@ from .gradient_collectors import GradientCollector, StreamingGradientCollector, 
 from .gradients import AdafactorNormalizer, AdamNormalizer, GradientProcessor, LayerAdapter, Normalizer
 from .in_memory_collector import InMemoryCollector
 from .process_grads import normalize_and_aggregate_grads, normalize_flat_grad
+from .score import create_scorer, get_query_grads, score_dataset
 from .scorer import Scorer
 
 __all__ = [
@@ -33,5 +35,5 @@ __all__ = [
     "load_gradients", "load_module_gradients", "load_scores", "load_token_gradients", "pad_and_tensor",
     "GradientCollector", "StreamingGradientCollector", "TraceCollector", "AdafactorNormalizer", "AdamNormalizer",
     "GradientProcessor", "LayerAdapter", "Normalizer", "InMemoryCollector", "normalize_and_aggregate_grads",
-    "normalize_flat_grad", "Scorer",
+    "normalize_flat_grad", "Scorer", "build", "create_processor", "create_scorer", "get_query_grads", "score_dataset",
 ]

@@ -207,3 +207,44 @@ def test_include_bias_end_to_end(device):
         left, right = module_projections(name, 16, g.shape[-1], a.shape[-1], torch.float32, collect_bias=True)
         want = ohooks.module_gradient(a, g, None, left, right, collect_bias=True)
         assert rel_l2(got[:, b * 256:(b + 1) * 256], want) <= 1e-4, name
+
+
+def test_build_then_score_entry_points(device, tmp_path):
+    """`build` a query store and a training store, then `score_dataset` on the fly: the scores equal the
+    oracle's scorer applied to the oracle's rows; query slices give the same file."""
+    from bergson_amd import IndexConfig, PreprocessConfig, ScoreConfig, build, load_gradients, score_dataset
+    from bergson_amd.data import load_scores
+    from bergson_amd.synthetic import ListDataset, random_docs
+
+    lengths = [40, 22, 31, 17, 48, 12]
+    docs, data, batches, cpu, gpu = _setup(device, lengths)
+    qlengths = [20, 35, 28]
+    qdocs = random_docs(qlengths, seed=77)
+    qdata = ListDataset(qdocs)
+
+    qcfg = IndexConfig(run_path=str(tmp_path / "query"), projection_dim=16, projection_type="normal",
+                       token_batch_size=96)
+    build(qcfg, model=gpu, data=qdata)
+    assert (tmp_path / "query" / "gradients.bin").exists() and not (tmp_path / "query.part").exists()
+    assert (tmp_path / "query" / "processor_config.yaml").exists()
+    qrows = torch.from_numpy(np.array(load_gradients(tmp_path / "query")))
+    qwant, _ = oloop.collect(cpu, cpu.base_model, qdocs, oloop.allocate_batches(qlengths, 96), p=16)
+    assert rel_l2(qrows, qwant) <= 1e-3
+
+    rows, _ = oloop.collect(cpu, cpu.base_model, docs, batches, p=16)
+    mods = list(oloop.target_linears(cpu.base_model))
+    cols = ostore.column_offsets({m: 256 for m in mods})
+    index = {m: rows[:, lo:hi] for m, (lo, hi) in cols.items()}
+    queries = {m: qwant[:, lo:hi] for m, (lo, hi) in cols.items()}
+    qn = oscan.normalize_and_aggregate_queries(queries, mods, unit_normalize=True)
+    want = oscan.scorer_score(index, qn, mods, unit_normalize=True)
+
+    for name, qbs in (("scores_all", None), ("scores_sliced", 2)):
+        icfg = IndexConfig(run_path=str(tmp_path / name), projection_dim=16, projection_type="normal",
+                           token_batch_size=96)
+        scfg = ScoreConfig(query_path=str(tmp_path / "query"), query_batch_size=qbs)
+        score_dataset(icfg, scfg, PreprocessConfig(unit_normalize=True), model=gpu, data=data)
+        sc = load_scores(tmp_path / name)
+        assert sc.is_written() and sc.num_scores == 3
+        got = torch.from_numpy(np.array(sc[:]))
+        assert (got - want).abs().max().item() <= 1e-3
