@@ -628,6 +628,8 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
   while (done < n_rows) {
     int64_t rows = n_rows - done;
     if (want_topk) {
+      // the first pass has no threshold yet and appends every score: each query's list grows by one
+      // serialised atomic per row, so that pass stays small and later passes grow fourfold
       int64_t lim = done == 0 ? SCAN_FIRST_CHUNK : done * 4;
       if (lim < k) lim = k;
       if (lim > chunk) lim = chunk;
