@@ -528,13 +528,20 @@ static void launch_collect(bool per_token, bool bias, dim3 grid, hipStream_t st,
 }
 
 // tokens per workgroup: 128 for the common case (p <= 16, aligned operands), else 64
-static int tile_tokens_for(int pb, bool aligned, bool bias) { return (pb == 1 && aligned && !bias) ? 128 : 64; }
+// 128-token tiles halve the projection-matrix traffic per token, but a sequence whose length is just past
+// a multiple of 128 wastes most of its last tile; fall back to 64-token tiles when that waste exceeds 4 %.
+static int tile_tokens_for(int pb, bool aligned, bool bias, int S) {
+  if (!(pb == 1 && aligned && !bias)) return 64;
+  const int padded = (S + 127) / 128 * 128;
+  return (int64_t)padded * 100 <= (int64_t)S * 104 ? 128 : 64;
+}
 
 template <typename T>
-static void launch_collect_pb(int pb, bool aligned, bool per_token, bool bias, dim3 grid, hipStream_t st,
-                              const CollectArgs& args) {
+static void launch_collect_pb(int pb, bool aligned, bool per_token, bool bias, int tile_tokens, dim3 grid,
+                              hipStream_t st, const CollectArgs& args) {
   if (pb == 1) {
-    aligned ? launch_collect<T, 1, true, 8, 2>(per_token, bias, grid, st, args)
+    if (aligned && tile_tokens == 128) return launch_collect<T, 1, true, 8, 2>(per_token, bias, grid, st, args);
+    aligned ? launch_collect<T, 1, true, 4, 2>(per_token, bias, grid, st, args)
             : launch_collect<T, 1, false, 4, 2>(per_token, bias, grid, st, args);
   } else if (pb == 2) {
     aligned ? launch_collect<T, 2, true, 4, 2>(per_token, bias, grid, st, args)
@@ -606,7 +613,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   args.S = S;
   args.p = p;
   const int pb = (p + 15) / 16;
-  const int tile_tokens = tile_tokens_for(pb, aligned, any_bias);
+  const int tile_tokens = tile_tokens_for(pb, aligned, any_bias, S);
   args.tiles_per_seq = (S + tile_tokens - 1) / tile_tokens;
   args.partials = (float*)((char*)ws + desc_bytes(n_modules));
   args.row_offsets = per_token ? rows_or_offsets : nullptr;
@@ -622,11 +629,11 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   const bool timed = 2 * (g_timing_used + 1) <= (int)g_timing_events.size();
   if (timed) BGX_HIP(hipEventRecord(g_timing_events[2 * g_timing_used], st));
   if (in_dtype == BGX_F32)
-    launch_collect_pb<float>(pb, aligned, per_token, any_bias, grid, st, args);
+    launch_collect_pb<float>(pb, aligned, per_token, any_bias, tile_tokens, grid, st, args);
   else if (in_dtype == BGX_F16)
-    launch_collect_pb<f16_t>(pb, aligned, per_token, any_bias, grid, st, args);
+    launch_collect_pb<f16_t>(pb, aligned, per_token, any_bias, tile_tokens, grid, st, args);
   else
-    launch_collect_pb<bf16_t>(pb, aligned, per_token, any_bias, grid, st, args);
+    launch_collect_pb<bf16_t>(pb, aligned, per_token, any_bias, tile_tokens, grid, st, args);
   BGX_HIP(hipGetLastError());
   if (timed) {
     BGX_HIP(hipEventRecord(g_timing_events[2 * g_timing_used + 1], st));
