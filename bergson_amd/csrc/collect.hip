@@ -17,7 +17,11 @@
 // so no barrier is needed in the streaming loop; their partial projections
 // are combined through LDS in a fixed pairwise order (w0+w2)+(w1+w3).
 
+#include <stdlib.h>
+#include <string.h>
+
 #include <algorithm>
+#include <atomic>
 #include <type_traits>
 #include <vector>
 
@@ -379,6 +383,207 @@ __global__ __launch_bounds__(COLLECT_THREADS) void collect_kernel(CollectArgs ar
   }
 }
 
+// ---- persistent variant (p <= 16, aligned operands, no bias) -------------------------------------
+// One workgroup per CU walks a contiguous range of (module, tile) items; the host cuts the item list
+// into ranges of equal weight, so the launch has no tail.  The scaled projection matrices of the
+// current module sit in LDS in MFMA fragment order (k-step s, lane l -> 16 bytes at (s*64 + l)*16),
+// staged once per module change instead of being fetched from L2 by every tile.  Each wave owns a
+// quarter of the tile's tokens over the whole of K, so nothing has to be combined across waves before
+// the token reduction, and that reduction runs on the matrix cores as well: the accumulator registers
+// of g' and a' are exactly the A and B operands of v_mfma_f32_16x16x4_f32 (lane (c, q) holds token
+// 4q + e, column c), so P += g'^T a' takes four MFMAs per 16 tokens with fp32 products.
+struct PersistArgs {
+  CollectArgs c;
+  const int32_t* wg_first;  // [gridDim.x + 1] first item of each workgroup; item = module * tiles_pm + tile
+  int tiles_pm;             // tiles per module = N * tiles_per_seq
+  int r_steps;              // k-steps of LDS reserved for projection fragments
+};
+
+template <typename T>
+__device__ inline void stage_projection(const T* __restrict__ R, const float* __restrict__ scale, int K, int p,
+                                        uint4* __restrict__ dst, int tid) {
+  using M = Mma<T>;
+  const int nfrag = (K / M::KS) * WAVE;
+  constexpr int B = 6;  // fragments per thread in flight
+  for (int f0 = tid; f0 < nfrag; f0 += COLLECT_THREADS * B) {
+    uint4 v[B];
+    uint4 s4[B][M::EPL / 4];
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      const int f = min(f0 + b * COLLECT_THREADS, nfrag - 1);
+      const int ks = f >> 6, l = f & 63;
+      const int r = l & 15, q = l >> 4;
+      const int k0 = ks * M::KS + q * M::EPL;
+      v[b] = load16_global(R + (int64_t)min(r, p - 1) * K + k0);
+      if (scale != nullptr) {
+#pragma unroll
+        for (int e = 0; e < M::EPL / 4; ++e) s4[b][e] = load16_global(scale + k0 + 4 * e);
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      const int f = f0 + b * COLLECT_THREADS;
+      if (scale != nullptr) {
+#pragma unroll
+        for (int e = 0; e < M::EPL; ++e)
+          M::set(v[b], e, M::get(v[b], e) * __uint_as_float((&s4[b][e >> 2].x)[e & 3]));
+      }
+      if (f < nfrag) dst[f] = v[b];
+    }
+  }
+}
+
+// x' = x @ R'^T for this wave's 16*MTW tokens over all of K, R' fragments read from LDS.
+// acc[mt][i] belongs to token mt*16 + (lane/16)*4 + i, column lane%16.  Token rows past rows_valid
+// re-read a valid row (their accumulator entries are garbage; the caller discards them).
+template <typename T, int MTW, int U>
+__device__ inline void project_tokens_lds(const T* __restrict__ xrow0, int64_t tok_stride, int rows_valid, int K,
+                                          const uint4* __restrict__ rfrag, int lane, f32x4 (&acc)[MTW]) {
+  using M = Mma<T>;
+  const int r = lane & 15;
+  const int q = lane >> 4;
+  const T* xrow[MTW];
+#pragma unroll
+  for (int mt = 0; mt < MTW; ++mt)
+    xrow[mt] = xrow0 + (int64_t)min(mt * 16 + r, rows_valid - 1) * tok_stride + q * M::EPL;
+  const int nsteps = K / M::KS;
+
+  auto run = [&](int ks0, auto uu_tag) {
+    constexpr int UU = decltype(uu_tag)::value;
+    uint4 xf[UU][MTW];
+    uint4 rf[UU];
+#pragma unroll
+    for (int u = 0; u < UU; ++u) {
+#pragma unroll
+      for (int mt = 0; mt < MTW; ++mt) xf[u][mt] = load16_global(xrow[mt] + (ks0 + u) * M::KS);
+      rf[u] = rfrag[(ks0 + u) * WAVE + lane];
+    }
+    // keep every load of the block ahead of the first MFMA: with one wave per SIMD the loads in
+    // flight are all that hides the memory latency
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < UU; ++u)
+#pragma unroll
+      for (int mt = 0; mt < MTW; ++mt) M::mma(xf[u][mt], rf[u], acc[mt]);
+  };
+
+  int ks0 = 0;
+  for (; ks0 + U <= nsteps; ks0 += U) run(ks0, std::integral_constant<int, U>{});
+  if constexpr (U > 2) {
+    for (; ks0 + 2 <= nsteps; ks0 += 2) run(ks0, std::integral_constant<int, 2>{});
+  }
+  for (; ks0 < nsteps; ++ks0) run(ks0, std::integral_constant<int, 1>{});
+}
+
+template <typename T, bool PER_TOKEN, int MTW, int U>
+__global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(PersistArgs pa) {
+  using M = Mma<T>;
+  constexpr int WAVE_T = 16 * MTW;      // tokens per wave
+  constexpr int TILE_T = 4 * WAVE_T;    // tokens per workgroup
+  constexpr int LDP = 17;
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  uint4* rfrag = reinterpret_cast<uint4*>(smem_raw);
+  unsigned char* scratch = smem_raw + (size_t)pa.r_steps * WAVE * 16;
+  // per-sequence: the P blocks of waves 1..3, double-buffered by tile parity; per-token: a', g' of each wave
+  f32x4 (*pred)[3][WAVE] = reinterpret_cast<f32x4 (*)[3][WAVE]>(scratch);
+  float (*tok)[2][WAVE_T][LDP] = reinterpret_cast<float (*)[2][WAVE_T][LDP]>(scratch);
+
+  const CollectArgs& args = pa.c;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int c = lane & 15;
+  const int q = lane >> 4;
+  const int p = args.p;
+  const int pp = p * p;
+  const int item0 = pa.wg_first[blockIdx.x];
+  const int item1 = pa.wg_first[blockIdx.x + 1];
+
+  int cur_m = -1;
+  int parity = 0;
+  for (int item = item0; item < item1; ++item) {
+    const int m = item / pa.tiles_pm;
+    const int tile = item - m * pa.tiles_pm;
+    const int n = tile / args.tiles_per_seq;
+    const int ts = tile - n * args.tiles_per_seq;
+    const int s0 = ts * TILE_T;
+    const int s_limit = seq_token_limit(args.lengths, n, args.S);
+    if (s0 >= s_limit) continue;  // whole tile is padding (uniform over the workgroup)
+    const int rows_valid = min(WAVE_T, s_limit - s0 - wave * WAVE_T);  // of this wave; may be <= 0
+
+    const bgx_module_desc d = args.mods[m];  // uniform
+    const int nA = d.I / M::KS;
+    if (m != cur_m) {
+      __syncthreads();  // every wave has finished reading the previous module's fragments
+      stage_projection<T>((const T*)d.r_in, d.col_scale, d.I, p, rfrag, tid);
+      stage_projection<T>((const T*)d.r_out, d.row_scale, d.O, p, rfrag + (size_t)nA * WAVE, tid);
+      cur_m = m;
+      __syncthreads();
+    }
+
+    f32x4 accA[MTW];
+    f32x4 accG[MTW];
+#pragma unroll
+    for (int mt = 0; mt < MTW; ++mt) {
+      accA[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      accG[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    if (rows_valid > 0) {
+      const int64_t t0 = s0 + wave * WAVE_T;
+      const T* a0 = (const T*)d.a + (int64_t)n * d.a_seq_stride + t0 * d.a_tok_stride;
+      const T* g0 = (const T*)d.g + (int64_t)n * d.g_seq_stride + t0 * d.g_tok_stride;
+      project_tokens_lds<T, MTW, U>(a0, d.a_tok_stride, rows_valid, d.I, rfrag, lane, accA);
+      project_tokens_lds<T, MTW, U>(g0, d.g_tok_stride, rows_valid, d.O, rfrag + (size_t)nA * WAVE, lane, accG);
+      // token rows past the last valid one hold garbage: zero them in g' (that removes their products)
+#pragma unroll
+      for (int mt = 0; mt < MTW; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (mt * 16 + q * 4 + i >= rows_valid) accG[mt][i] = 0.f;
+    }
+
+    if constexpr (!PER_TOKEN) {
+      // P[i, j] = sum_t g'[t, i] * a'[t, j] over this wave's tokens; lane (c, q) gets P[4q + e][c]
+      f32x4 P = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int mt = 0; mt < MTW; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) P = __builtin_amdgcn_mfma_f32_16x16x4f32(accG[mt][i], accA[mt][i], P, 0, 0, 0);
+      if (wave > 0) pred[parity][wave - 1][lane] = P;
+      __syncthreads();
+      if (wave == 0) {
+        const f32x4 p1 = pred[parity][0][lane], p2 = pred[parity][1][lane], p3 = pred[parity][2][lane];
+        float* dst = args.partials + (((int64_t)m * args.N + n) * args.tiles_per_seq + ts) * pp;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int i = q * 4 + e;
+          if (i < p && c < p) dst[i * p + c] = (P[e] + p1[e]) + (p2[e] + p3[e]);
+        }
+      }
+      parity ^= 1;  // the next tile writes the other buffer, so one barrier per tile is enough
+    } else {
+      __syncthreads();  // the previous tile's readers are done with tok
+#pragma unroll
+      for (int mt = 0; mt < MTW; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          tok[wave][0][mt * 16 + q * 4 + i][c] = accA[mt][i];
+          tok[wave][1][mt * 16 + q * 4 + i][c] = accG[mt][i];
+        }
+      __syncthreads();
+      const int64_t row0 = args.row_offsets[n] + s0 + wave * WAVE_T;
+      for (int t = 0; t < rows_valid; ++t) {
+        const int64_t base = (row0 + t) * args.out_row_stride + d.out_col;
+        for (int e = lane; e < pp; e += WAVE) {
+          const int i = e / p, j = e - i * p;
+          store_as(args.out, base + e, clampf(tok[wave][1][t][i] * tok[wave][0][t][j], args.lo, args.hi),
+                   args.out_dtype);
+        }
+      }
+    }
+  }
+}
+
 // Adds the per-tile partials of each (module, sequence) in a fixed order (four interleaved running
 // sums combined at the end, so that consecutive loads do not wait on each other), clamps, casts and
 // writes the module's block of the output row.
@@ -499,8 +704,12 @@ int collect_timing_read(float* ms_out, int capacity, int* count_out) {
 
 static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+constexpr int PERSIST_MAX_WGS = 1024;        // upper bound on the workgroups of the persistent variant
+constexpr size_t LDS_PER_WG = 160 * 1024;    // LDS one workgroup may allocate on gfx950
+
+// head of the workspace: the descriptor table, then the item ranges of the persistent workgroups
 static size_t desc_bytes(int n_modules) {
-  return align_up((size_t)n_modules * sizeof(bgx_module_desc), 256);
+  return align_up((size_t)n_modules * sizeof(bgx_module_desc) + (PERSIST_MAX_WGS + 1) * sizeof(int32_t), 256);
 }
 
 constexpr int MIN_TILE_T = 64;  // smallest token tile any kernel variant uses: bounds the partials
@@ -550,6 +759,52 @@ static void launch_collect_pb(int pb, bool aligned, bool per_token, bool bias, i
     aligned ? launch_collect<T, 4, true, 4, 1>(per_token, bias, grid, st, args)
             : launch_collect<T, 4, false, 4, 1>(per_token, bias, grid, st, args);
   }
+}
+
+constexpr int MAX_DEVICES = 64;
+
+// CUs of the current device (cached per device)
+static int compute_units(int* out) {
+  static std::atomic<int> cached[MAX_DEVICES];
+  int dev = 0;
+  BGX_HIP(hipGetDevice(&dev));
+  int cus = (dev >= 0 && dev < MAX_DEVICES) ? cached[dev].load(std::memory_order_relaxed) : 0;
+  if (cus <= 0) {
+    BGX_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    if (dev >= 0 && dev < MAX_DEVICES) cached[dev].store(cus, std::memory_order_relaxed);
+  }
+  *out = cus;
+  return 0;
+}
+
+template <typename T, bool PER_TOKEN, int MTW, int U>
+static int launch_persist_one(int wgs, size_t lds, hipStream_t st, const PersistArgs& pa) {
+  auto kern = collect_persist_kernel<T, PER_TOKEN, MTW, U>;
+  // the opt-in to more than 64 KB of dynamic LDS is per kernel and per device; do it once for each
+  static std::atomic<bool> opted_in[MAX_DEVICES];
+  int dev = 0;
+  BGX_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= MAX_DEVICES || !opted_in[dev].load(std::memory_order_acquire)) {
+    BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_PER_WG));
+    if (dev >= 0 && dev < MAX_DEVICES) opted_in[dev].store(true, std::memory_order_release);
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(COLLECT_THREADS), lds, st, pa);
+  return 0;
+}
+
+template <typename T>
+static int launch_persist(bool per_token, int tile_tokens, int wgs, size_t lds, hipStream_t st,
+                          const PersistArgs& pa) {
+  if (tile_tokens == 128)
+    return per_token ? launch_persist_one<T, true, 2, 4>(wgs, lds, st, pa)
+                     : launch_persist_one<T, false, 2, 4>(wgs, lds, st, pa);
+  return per_token ? launch_persist_one<T, true, 1, 8>(wgs, lds, st, pa)
+                   : launch_persist_one<T, false, 1, 8>(wgs, lds, st, pa);
+}
+
+// LDS beside the projection fragments: the larger of the P exchange buffers and the per-token a', g' tiles
+static size_t persist_scratch_bytes(int tile_tokens) {
+  return std::max((size_t)2 * 3 * WAVE * 16, (size_t)2 * tile_tokens * 17 * sizeof(float));
 }
 
 int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules, int N, int S,
@@ -603,8 +858,6 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   std::stable_sort(sorted.begin(), sorted.end(), [](const bgx_module_desc& x, const bgx_module_desc& y) {
     return (int64_t)x.I + x.O > (int64_t)y.I + y.O;
   });
-  BGX_HIP(hipMemcpyAsync(mods_dev, sorted.data(), (size_t)n_modules * sizeof(bgx_module_desc),
-                         hipMemcpyHostToDevice, st));
 
   CollectArgs args;
   args.mods = mods_dev;
@@ -615,6 +868,52 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   const int pb = (p + 15) / 16;
   const int tile_tokens = tile_tokens_for(pb, aligned, any_bias, S);
   args.tiles_per_seq = (S + tile_tokens - 1) / tile_tokens;
+  const int64_t tiles = (int64_t)N * args.tiles_per_seq;
+  BGX_REQUIRE(tiles <= 0x7fffffffLL, BGX_E_SHAPE, "collect: %lld tiles exceed the grid limit", (long long)tiles);
+
+  // The persistent variant needs every module's projection fragments (16 rows x (I + O) elements) to
+  // fit in LDS beside its exchange buffers.
+  int r_steps = 0;
+  for (int m = 0; m < n_modules; ++m) r_steps = std::max(r_steps, (sorted[m].I + sorted[m].O) / kstep);
+  const size_t persist_lds = (size_t)r_steps * 1024 + persist_scratch_bytes(tile_tokens);
+  bool persist = pb == 1 && aligned && !any_bias && persist_lds <= LDS_PER_WG &&
+                 tiles * n_modules <= 0x7fffffffLL;
+  // BGX_COLLECT_PERSIST=0 in the environment forces the one-workgroup-per-tile kernel (tests, comparisons)
+  if (const char* e = getenv("BGX_COLLECT_PERSIST")) persist = persist && e[0] != '0';
+
+  std::vector<unsigned char> head((size_t)n_modules * sizeof(bgx_module_desc));
+  memcpy(head.data(), sorted.data(), head.size());
+  int wgs = 0;
+  if (persist) {
+    int cus = 0;
+    const int rc_cus = compute_units(&cus);
+    if (rc_cus != 0) return rc_cus;
+    const int64_t items = tiles * n_modules;
+    wgs = (int)std::min<int64_t>(std::min(std::max(cus, 1), PERSIST_MAX_WGS), items);
+    // equal-weight contiguous ranges; an item costs its k-steps plus a constant for the token reduction
+    std::vector<int32_t> first((size_t)wgs + 1, (int32_t)items);
+    first[0] = 0;
+    constexpr int REDUCE_STEPS = 2;
+    double total = 0.0;
+    for (int m = 0; m < n_modules; ++m)
+      total += (double)tiles * ((sorted[m].I + sorted[m].O) / kstep + REDUCE_STEPS);
+    double cum = 0.0;
+    int g = 0;
+    int64_t item = 0;
+    for (int m = 0; m < n_modules && g + 1 < wgs; ++m) {
+      const double w = (sorted[m].I + sorted[m].O) / kstep + REDUCE_STEPS;
+      for (int64_t t = 0; t < tiles && g + 1 < wgs; ++t) {
+        cum += w;
+        ++item;
+        while (g + 1 < wgs && cum >= total * (double)(g + 1) / (double)wgs) first[++g] = (int32_t)item;
+      }
+    }
+    first[wgs] = (int32_t)items;
+    const size_t off = head.size();
+    head.resize(off + first.size() * sizeof(int32_t));
+    memcpy(head.data() + off, first.data(), first.size() * sizeof(int32_t));
+  }
+  BGX_HIP(hipMemcpyAsync(mods_dev, head.data(), head.size(), hipMemcpyHostToDevice, st));
   args.partials = (float*)((char*)ws + desc_bytes(n_modules));
   args.row_offsets = per_token ? rows_or_offsets : nullptr;
   args.out = out;
@@ -623,17 +922,30 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   args.lo = lo;
   args.hi = hi;
 
-  const int64_t tiles = (int64_t)N * args.tiles_per_seq;
-  BGX_REQUIRE(tiles <= 0x7fffffffLL, BGX_E_SHAPE, "collect: %lld tiles exceed the grid limit", (long long)tiles);
   const dim3 grid((unsigned)tiles, (unsigned)n_modules);
   const bool timed = 2 * (g_timing_used + 1) <= (int)g_timing_events.size();
   if (timed) BGX_HIP(hipEventRecord(g_timing_events[2 * g_timing_used], st));
-  if (in_dtype == BGX_F32)
+  if (persist) {
+    PersistArgs pa;
+    pa.c = args;
+    pa.wg_first = (const int32_t*)((const char*)ws + (size_t)n_modules * sizeof(bgx_module_desc));
+    pa.tiles_pm = (int)tiles;
+    pa.r_steps = r_steps;
+    int rc;
+    if (in_dtype == BGX_F32)
+      rc = launch_persist<float>(per_token, tile_tokens, wgs, persist_lds, st, pa);
+    else if (in_dtype == BGX_F16)
+      rc = launch_persist<f16_t>(per_token, tile_tokens, wgs, persist_lds, st, pa);
+    else
+      rc = launch_persist<bf16_t>(per_token, tile_tokens, wgs, persist_lds, st, pa);
+    if (rc != 0) return rc;
+  } else if (in_dtype == BGX_F32) {
     launch_collect_pb<float>(pb, aligned, per_token, any_bias, tile_tokens, grid, st, args);
-  else if (in_dtype == BGX_F16)
+  } else if (in_dtype == BGX_F16) {
     launch_collect_pb<f16_t>(pb, aligned, per_token, any_bias, tile_tokens, grid, st, args);
-  else
+  } else {
     launch_collect_pb<bf16_t>(pb, aligned, per_token, any_bias, tile_tokens, grid, st, args);
+  }
   BGX_HIP(hipGetLastError());
   if (timed) {
     BGX_HIP(hipEventRecord(g_timing_events[2 * g_timing_used + 1], st));

@@ -44,6 +44,16 @@ struct f16_t {
 
 constexpr int WAVE = 64;
 
+// 16-byte load from device memory.  Pointers that come out of a descriptor table carry no address
+// space, and the compiler then falls back to generic ("flat") loads, which it cannot keep in flight
+// next to LDS traffic; this tells it the pointer is a plain global one.
+__device__ inline uint4 load16_global(const void* p) {
+  typedef uint32_t raw4 __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(1))) const raw4* global_ptr;
+  const raw4 v = *(global_ptr)(uintptr_t)p;
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 __host__ __device__ inline size_t dtype_size(int dt) {
   return dt == BGX_F32 ? 4 : 2;
 }

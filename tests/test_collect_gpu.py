@@ -12,6 +12,17 @@ from oracle.projection import module_projections
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(params=["persistent", "grid"], autouse=True)
+def kernel_variant(request, monkeypatch):
+    """Every case runs twice: with the persistent collection kernel where it applies (the default), and with
+    the one-workgroup-per-tile kernel forced through the library's environment switch."""
+    if request.param == "grid":
+        monkeypatch.setenv("BGX_COLLECT_PERSIST", "0")
+    else:
+        monkeypatch.delenv("BGX_COLLECT_PERSIST", raising=False)
+    return request.param
+
+
 def make_case(N, S, I, O, p, dtype, seed, normalizer=None, name="layers.0.mlp.dense_h_to_4h"):
     gen = torch.Generator().manual_seed(seed)
     a = torch.randn(N, S, I, generator=gen).to(dtype)
@@ -151,6 +162,42 @@ def test_seq_clamp_to_store_dtype(device):
     assert torch.isfinite(got.float()).all()
     assert (got.float().abs() == hi).any()
     assert rel_l2(got, want) <= 1e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("per_token", [False, True])
+def test_many_tiles_across_modules(device, dtype, per_token):
+    """More (module, tile) items than the GPU has CUs, modules of different widths and ragged lengths: a
+    persistent workgroup then walks several tiles and crosses module and sequence boundaries."""
+    N, S, p = 8, 640, 16
+    lengths = [640, 513, 129, 128, 400, 2, 77, 639]
+    shapes = [(64, 192), (128, 64), (64, 64), (256, 64), (64, 256), (128, 128), (192, 64), (64, 128)]
+    cases = []
+    for i, (I, O) in enumerate(shapes):
+        a, g, left, right, norm = make_case(N, S, I, O, p, dtype, seed=40 + i, normalizer="adafactor" if i % 2 else None,
+                                            name=f"layers.{i}.z")
+        for n, l in enumerate(lengths):
+            g[n, l - 1:] = 0
+        cases.append((a, g, left, right, norm))
+    if not per_token:
+        got = run_kernel(device, cases, p, dtype, lengths=lengths)
+        want = oracle_rows(cases, dtype)
+    else:
+        counts = [l - 1 for l in lengths]
+        row_offsets = [sum(counts[:n]) for n in range(N)]
+        mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+        got = run_kernel(device, cases, p, dtype, lengths=lengths, per_token=True, row_offsets=row_offsets,
+                         n_rows=sum(counts))
+        want = oracle_rows(cases, dtype, attribute_tokens=True, collection_mask=mask)
+    assert got.shape == want.shape
+    assert rel_l2(got, want) <= TOL[dtype]
+
+
+def test_wide_module_uses_the_tile_kernel(device):
+    """I + O too wide for the projection fragments to fit in LDS: the launch falls back to the tile kernel."""
+    cases = [make_case(2, 70, 4096, 1024, 16, torch.bfloat16, seed=50, normalizer="adafactor")]
+    got = run_kernel(device, cases, 16, torch.bfloat16)
+    assert rel_l2(got, oracle_rows(cases, torch.bfloat16)) <= TOL[torch.bfloat16]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
