@@ -39,8 +39,10 @@ def test_workspace_sizes():
     from bergson_amd import _lib
 
     lib = _lib.load()
-    # descriptors rounded to 256 B + one fp32 p*p partial per (module, sequence, 64-token tile)
-    assert lib.bgx_collect_workspace_bytes(48, 2, 2048, 16) == -(-48 * 112 // 256) * 256 + 48 * 2 * 32 * 256 * 4
+    # head (descriptors + 1025 int32 item ranges of the persistent workgroups) rounded to 256 B
+    # + one fp32 p*p partial per (module, sequence, 64-token tile)
+    head = -(-(48 * 112 + 1025 * 4) // 256) * 256
+    assert lib.bgx_collect_workspace_bytes(48, 2, 2048, 16) == head + 48 * 2 * 32 * 256 * 4
     assert lib.bgx_collect_workspace_bytes(0, 2, 64, 16) == 0
     small = lib.bgx_scan_workspace_bytes(8, 10, 1024)
     assert small >= 8 * 10 * 8 + 8 * 1024 * 8
