@@ -1,21 +1,24 @@
 // Fused per-module gradient collection for gfx950 (MI355X).
 //
-// One workgroup owns a tile of 64 tokens of one sequence of one module and
-//   1. projects the activations  a'[t, j] = sum_k a[t, k] * (R_in[j, k] * col_scale[k])
-//   2. projects the output grads g'[t, i] = sum_k g[t, k] * (R_out[i, k] * row_scale[k])
-//      both with MFMA tiles fed straight from global memory (a and g are read
-//      exactly once; the p x K projection matrices come from L2),
-//   3. per-sequence: reduces P[i, j] = sum_t g'[t, i] * a'[t, j] over its tokens
-//      and writes one fp32 partial; a second tiny kernel adds the partials of a
-//      sequence in a fixed order, clamps, casts and writes the store row.
-//      per-token: writes flatten(g'[t] (x) a'[t]) for every valid token.
+// For a tile of tokens of one sequence of one module the kernels
+//   1. project the activations  a'[t, j] = sum_k a[t, k] * (R_in[j, k] * col_scale[k])
+//   2. project the output grads g'[t, i] = sum_k g[t, k] * (R_out[i, k] * row_scale[k])
+//      both with MFMA tiles whose A operand is loaded straight from global memory (a and g are
+//      read exactly once),
+//   3. per-sequence: reduce P[i, j] = sum_t g'[t, i] * a'[t, j] over the tile's tokens and write one
+//      fp32 partial; a second tiny kernel adds the partials of a sequence in a fixed order, clamps,
+//      casts and writes the store row.
+//      per-token: write flatten(g'[t] (x) a'[t]) for every valid token.
 //
 // Reference op sequence: bergson/collector/collector.py:518-543 (forward
 // hook), :646-742 (backward hook), bergson/builder.py:17-32 (concatenation).
 //
-// The 4 waves of a workgroup split the K dimension (I, then O) between them,
-// so no barrier is needed in the streaming loop; their partial projections
-// are combined through LDS in a fixed pairwise order (w0+w2)+(w1+w3).
+// Two kernels share that arithmetic:
+//   collect_persist_kernel  p <= 16, aligned operands, no bias, projection matrices small enough for
+//                           LDS: one workgroup per CU walks an equal share of all (module, tile) items.
+//   collect_kernel          everything else: one workgroup per (module, tile); its 4 waves split K
+//                           and combine their partial projections through LDS in the fixed order
+//                           (w0+w2)+(w1+w3); the projection matrices come from L2.
 
 #include <stdlib.h>
 #include <string.h>
