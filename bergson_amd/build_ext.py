@@ -18,7 +18,7 @@ PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 INCLUDE = PKG.parent / "include"
 LIB = PKG / "libbergson_amd.so"
-SOURCES = ["capi.hip", "collect.hip", "scan.hip", "adam.hip"]
+SOURCES = ["capi.hip", "collect.hip", "scan.hip", "adam.hip", "fullgrad.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

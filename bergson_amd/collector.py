@@ -103,6 +103,8 @@ class HookCollectorBase(ContextDecorator, ABC):
         self._prepared: dict[str, ops.PreparedModule] = {}
         self._adam_prepared: dict[str, ops.AdamPrepared] = {}
         self._deferred_adam: list = []
+        self._deferred_full: list = []  # unprojected / global-projection modules: (FullGradModule, name, a, g)
+        self._full_prepared: dict = {}
         self._active = False
         self._scale_cache: dict[str, tuple[Tensor | None, Tensor | None]] = {}
         self.target_info = self.discover_targets(self.model, self.target_modules, self.processor.include_bias,
@@ -314,6 +316,7 @@ class HookCollectorBase(ContextDecorator, ABC):
         if exc_type is not None:  # a failed batch leaves nothing queued; otherwise process_batch launches
             self._deferred.clear()
             self._deferred_adam.clear()
+            self._deferred_full.clear()
         return False
 
     # ---- the hook pair -----------------------------------------------------------------------
@@ -390,6 +393,79 @@ class HookCollectorBase(ContextDecorator, ABC):
         return ops.ModuleInput(a=a, g=g, r_in=r_in, r_out=r_out, out_col=out_col, col_scale=col_scale,
                                row_scale=row_scale, bias_col=bias_col, bias_scale=bias_scale)
 
+    def full_prepared(self, module: nn.Module, g: Tensor, out_col: int) -> "ops.FullGradModule":
+        """Normaliser vectors of `module` for the unprojected path (collector.py:609-742 with p = None)."""
+        name: str = module._name  # type: ignore[assignment]
+        key = f"{name}|{g.dtype}|{out_col}"
+        prep = self._full_prepared.get(key)
+        if prep is not None:
+            return prep
+        if not g.is_cuda:
+            raise RuntimeError("bergson_amd has no CPU path: the model must run on the GPU")
+        i = getattr(module, LayerAdapter.in_attr(module))
+        o = g.shape[-1]  # an attention head sees its own slice of the output features
+        normalizer = self.normalizer_for(name)
+        bias = bool(module._collect_bias)
+        prep = ops.FullGradModule(O=o, I=i, out_col=out_col, collect_bias=bias)
+        f32 = dict(device=g.device, dtype=torch.float32)
+        if isinstance(normalizer, AdamNormalizer):
+            prep.adam_v = normalizer.weight_avg_sq.detach().to(**f32).contiguous()
+            if bias:
+                assert normalizer.bias_avg_sq is not None, f"{name}: bias collected but the normalizer has no bias_avg_sq"
+                # 1 / (sqrt(bias_avg_sq) + 1e-8), eps outside the root (gradients.py:390-400)
+                prep.bias_scale = (normalizer.bias_avg_sq.detach().to(**f32).sqrt() + 1e-8).reciprocal().contiguous()
+        elif isinstance(normalizer, AdafactorNormalizer):
+            prep.row_scale, prep.col_scale = self._scales(name, normalizer, g.dtype, g.device)
+            if bias:
+                assert normalizer.bias_avg_sq is not None, f"{name}: bias collected but the normalizer has no bias_avg_sq"
+                # rsqrt(bias_avg_sq + 1e-8), eps inside the root (gradients.py:339-349)
+                prep.bias_scale = normalizer.bias_avg_sq.detach().to(**f32).add(1e-8).rsqrt().contiguous()
+        self._full_prepared[key] = prep
+        return prep
+
+    def _token_rows(self, device: torch.device):
+        """(lengths, per-document token counts, offsets of each document's first row, total rows)."""
+        lengths = self._batch_lengths(device)
+        assert lengths is not None, "attribute_tokens needs a collection mask (with_batch)"
+        counts = (lengths.to(torch.int64) - 1).clamp_min_(0)
+        offsets = torch.cumsum(counts, 0) - counts
+        return lengths, counts, offsets, int(counts.sum().item())
+
+    def _global_projection(self, items: list, out: Tensor, lengths: Tensor | None, out_rows: Tensor | None,
+                           row_offsets: Tensor | None) -> None:
+        """projection_target = "global" (collector.py:364-402): every module's clamped, flattened gradient
+        times its block of the single projection matrix, summed over the modules into columns
+        [0, projection_dim) of the output rows.  The sum over modules is kept in fp32 (the reference adds
+        in the model dtype) and cast once."""
+        pd = self.processor.projection_dim
+        assert pd is not None
+        g0 = items[0][3]
+        N = g0.shape[0]
+        if self.attribute_tokens:
+            lens, counts, local, total = self._token_rows(g0.device)
+            n_rows = total
+        else:
+            lens, counts, local, n_rows = lengths, None, None, N
+        if n_rows == 0:
+            return
+        acc = torch.zeros((n_rows, pd), dtype=torch.float32, device=g0.device)
+        for prep, name, a, g in items:
+            tmp = torch.empty((n_rows, prep.width), dtype=g.dtype, device=g.device)
+            ops.full_gradient(prep, a, g, tmp, per_token=self.attribute_tokens, lengths=lens,
+                              rows=local if self.attribute_tokens else None, lo=self.lo, hi=self.hi)
+            R = self.projection(name, pd, prep.width, "single", g.device, g.dtype)
+            acc += (tmp @ R.T).float()
+        res = acc.to(out.dtype)
+        if self.attribute_tokens:
+            assert row_offsets is not None and counts is not None and local is not None
+            dst = torch.repeat_interleave(row_offsets.to(torch.int64) - local, counts) + torch.arange(
+                n_rows, device=out.device)
+            out[:, :pd].index_copy_(0, dst, res)
+        elif out_rows is not None:
+            out[:, :pd].index_copy_(0, out_rows, res)
+        else:
+            out[:n_rows, :pd].copy_(res)
+
     def adam_prepared(self, module: nn.Module, g: Tensor, out_col: int) -> "ops.AdamPrepared":
         """The module's Adam table and projections, built on its first batch (collector.py:609-644)."""
         name: str = module._name  # type: ignore[assignment]
@@ -427,6 +503,21 @@ class HookCollectorBase(ContextDecorator, ABC):
         [lo, hi], in the model dtype (collector.py:592-743) -- one fused launch."""
         p = self.per_module_projection_dim
         N, S = g.shape[:2]
+        if p is None:
+            # weight-shaped gradient [O, I (+1)] per sample or per token
+            fp = self.full_prepared(module, g, 0)
+            a = module._inputs
+            assert isinstance(a, Tensor), "Activation cache missing for module"
+            if self.attribute_tokens:
+                lengths, _, offsets, total = self._token_rows(g.device)
+                out = torch.empty((total, fp.width), dtype=g.dtype, device=g.device)
+                if total:
+                    ops.full_gradient(fp, a, g, out, per_token=True, lengths=lengths, rows=offsets, lo=self.lo,
+                                      hi=self.hi)
+                return out
+            out = torch.empty((N, fp.width), dtype=g.dtype, device=g.device)
+            ops.full_gradient(fp, a, g, out, per_token=False, lengths=None, rows=None, lo=self.lo, hi=self.hi)
+            return out
         if isinstance(self.normalizer_for(module._name), AdamNormalizer):
             prep = self.adam_prepared(module, g, 0)
             a = module._inputs
@@ -465,6 +556,11 @@ class HookCollectorBase(ContextDecorator, ABC):
         module that does not change between batches (projection matrices, factor vectors, output column)
         is resolved and checked on its first batch only."""
         name: str = module._name  # type: ignore[assignment]
+        if self.per_module_projection_dim is None:
+            a = module._inputs
+            assert isinstance(a, Tensor), "Activation cache missing for module"
+            self._deferred_full.append((self.full_prepared(module, g, out_col), name, a, g))
+            return
         if isinstance(self.normalizer_for(name), AdamNormalizer):
             a = module._inputs
             assert isinstance(a, Tensor), "Activation cache missing for module"
@@ -482,10 +578,21 @@ class HookCollectorBase(ContextDecorator, ABC):
                         row_offsets: Tensor | None = None) -> None:
         """One fused launch over every queued module (one launch sequence per module with an Adam
         normaliser), writing each module's block of `out`."""
-        if not self._deferred and not self._deferred_adam:
+        if not self._deferred and not self._deferred_adam and not self._deferred_full:
             return
         p = self.per_module_projection_dim
-        assert p is not None
+        if p is None:
+            try:
+                if self.processor.projection_target == "global":
+                    self._global_projection(self._deferred_full, out, lengths, out_rows, row_offsets)
+                else:
+                    for prep, _name, a, g in self._deferred_full:
+                        ops.full_gradient(prep, a, g, out, per_token=self.attribute_tokens, lengths=lengths,
+                                          rows=row_offsets if self.attribute_tokens else out_rows, lo=self.lo,
+                                          hi=self.hi)
+            finally:
+                self._deferred_full.clear()
+            return
         try:
             if self.attribute_tokens:
                 assert lengths is not None and row_offsets is not None
@@ -503,6 +610,7 @@ class HookCollectorBase(ContextDecorator, ABC):
         finally:
             self._deferred.clear()
             self._deferred_adam.clear()
+            self._deferred_full.clear()
 
     @abstractmethod
     def setup(self) -> None: ...

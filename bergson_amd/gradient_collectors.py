@@ -38,6 +38,8 @@ class _DeferredBatchMixin:
             cols = self._columns = {n: lo for n, (lo, _) in column_offsets(sizes).items()}
             self._row_width = sum(sizes.values())
             self._grad_sizes = sizes
+        if self.processor.projection_target == "global":
+            return 0  # every module adds into the single "gradients" block
         return cols[name]
 
     def _launch_batch(self, indices: list[int], builder: Builder | None, need_rows: bool) -> RowBlock:
@@ -45,11 +47,12 @@ class _DeferredBatchMixin:
         them and nobody else needs them; otherwise into a fresh batch buffer whose column views are
         returned as mod_grads."""
         block = RowBlock()
-        queued = self._deferred or self._deferred_adam
+        queued = self._deferred or self._deferred_adam or self._deferred_full
         if not queued:
             return block
-        dev = queued[0][2].device
-        N = queued[0][2].shape[0]
+        g0 = queued[0][-1]
+        dev = g0.device
+        N = g0.shape[0]
         assert N == len(indices), f"batch of {N} sequences but {len(indices)} indices"
         lengths = self._batch_lengths(dev) if (self.attribute_tokens or self.skip_padding) else None
         direct = builder is not None and builder.direct and not need_rows
@@ -69,6 +72,7 @@ class _DeferredBatchMixin:
             else:
                 self._deferred.clear()
                 self._deferred_adam.clear()
+                self._deferred_full.clear()
         elif direct:
             idx = torch.as_tensor(indices, dtype=torch.int64).to(dev, non_blocking=True)
             self.launch_deferred(builder.device_rows, lengths=lengths, out_rows=idx)
@@ -111,8 +115,6 @@ class GradientCollector(_DeferredBatchMixin, HookCollectorBase):
         self.attribute_tokens = self.cfg.attribute_tokens
         if self.cfg.attribute_tokens:
             assert self.preprocess_cfg.aggregation == "none", "attribute_tokens is incompatible with reduce mode."
-        if self.processor.projection_target == "global":
-            raise NotImplementedError("projection_target='global' has no HIP kernel in this build")
         self.save_dtype = self.store_dtype or get_gradient_dtype(self.model)
         self.lo = torch.finfo(self.save_dtype).min
         self.hi = torch.finfo(self.save_dtype).max

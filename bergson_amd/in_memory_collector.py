@@ -46,8 +46,6 @@ class InMemoryCollector(_DeferredBatchMixin, HookCollectorBase):
         assert isinstance(self.model.device, torch.device), "Model device is not set correctly"
         if not self.skip_hessians:
             raise NotImplementedError("autocorrelation statistics (skip_hessians=False) are outside this package")
-        if self.processor.projection_target == "global":
-            raise NotImplementedError("projection_target='global' has no HIP kernel in this build")
         self.attribute_tokens = self.cfg.attribute_tokens
         if self.cfg.attribute_tokens:
             assert self.preprocess_cfg.aggregation == "none", "attribute_tokens is incompatible with reduce mode."

@@ -327,6 +327,69 @@ def collect_adam(prep: AdamPrepared, a: Tensor, g: Tensor, out: Tensor, *, per_t
     _lib.check(rc, "bgx_collect_adam")
 
 
+@dataclass
+class FullGradModule:
+    """Per-module state of the unprojected path: the normaliser's vectors on the device and the output column."""
+
+    O: int
+    I: int
+    out_col: int
+    collect_bias: bool = False
+    row_scale: Tensor | None = None   # Adafactor, from adafactor_scales
+    col_scale: Tensor | None = None
+    adam_v: Tensor | None = None      # [O, I] fp32
+    bias_scale: Tensor | None = None  # [O] fp32, None = 1
+
+    @property
+    def width(self) -> int:
+        return self.O * (self.I + int(self.collect_bias))
+
+
+def full_gradient(mod: FullGradModule, a: Tensor, g: Tensor, out: Tensor, *, per_token: bool,
+                  lengths: Tensor | None, rows: Tensor | None, lo: float, hi: float) -> None:
+    """Weight-shaped gradient of one module written to its columns of `out` (see bgx_fullgrad_seq / _tok).
+
+    per_token=False: out[rows[n] (or n)] gets flatten(normalise(g[n]^T a[n])) -- the batched GEMM runs on
+    the BLAS, as the reference's `g.mT @ a` does; per_token=True: out[rows[n] + s] gets
+    flatten(normalise(g[n, s] (x) a[n, s])) for s < lengths[n] - 1.
+    """
+    lib = _lib.load()
+    for t, name in ((a, "a"), (g, "g"), (out, "out")):
+        _need_gpu(t, name)
+    if a.dim() != 3 or g.dim() != 3 or a.shape[:2] != g.shape[:2]:
+        raise ValueError(f"a {tuple(a.shape)} / g {tuple(g.shape)} must be [N, S, I] and [N, S, O]")
+    N, S, I = a.shape
+    O = g.shape[2]
+    if (I, O) != (mod.I, mod.O) or a.dtype != g.dtype:
+        raise ValueError("a / g do not match the prepared module")
+    if out.dim() != 2 or out.stride(1) != 1:
+        raise ValueError("out must be a 2-D tensor with contiguous rows")
+    if a.stride(2) != 1:
+        a = a.contiguous()
+    if g.stride(2) != 1:
+        g = g.contiguous()
+    code = dtype_code(a.dtype)
+    if per_token:
+        if lengths is None or rows is None:
+            raise ValueError("per-token collection needs lengths and row offsets")
+        rc = lib.bgx_fullgrad_tok(_ptr(a), _ptr(g), a.stride(0), a.stride(1), g.stride(0), g.stride(1), N, S, I, O, code,
+                                  _ptr(mod.row_scale), _ptr(mod.col_scale), _ptr(mod.adam_v), int(mod.collect_bias),
+                                  _ptr(mod.bias_scale), _ptr(lengths), _ptr(rows), _ptr(out), out.stride(0),
+                                  mod.out_col, dtype_code(out.dtype), lo, hi, _stream())
+        _lib.check(rc, "bgx_fullgrad_tok")
+        return
+    P = torch.bmm(g.transpose(1, 2), a)  # [N, O, I], the plain library GEMM of the path
+    bias_sum = None
+    if mod.collect_bias:
+        bias_sum = torch.empty((N, O), dtype=torch.float32, device=g.device)
+        rc = lib.bgx_token_sum(_ptr(g), g.stride(0), g.stride(1), N, S, O, code, _ptr(bias_sum), _stream())
+        _lib.check(rc, "bgx_token_sum")
+    rc = lib.bgx_fullgrad_seq(_ptr(P), N, O, I, code, _ptr(mod.row_scale), _ptr(mod.col_scale), _ptr(mod.adam_v),
+                              _ptr(bias_sum), _ptr(mod.bias_scale), _ptr(rows), _ptr(out), out.stride(0), mod.out_col,
+                              dtype_code(out.dtype), lo, hi, _stream())
+    _lib.check(rc, "bgx_fullgrad_seq")
+
+
 def collect_seq(modules: list[ModuleInput], p: int, out: Tensor, *, lengths: Tensor | None = None,
                 out_rows: Tensor | None = None, lo: float = float("-inf"), hi: float = float("inf")) -> None:
     """out[row(n), m.out_col : m.out_col + p*p] = clamp(sum_s g'[n,s] (x) a'[n,s]) for every module m."""

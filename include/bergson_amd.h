@@ -172,6 +172,51 @@ int bgx_collect_adam(const void* a_dev, const void* g_dev,
                      void* workspace_dev, size_t workspace_bytes,
                      int64_t chunk_tokens, void* stream);
 
+/* ---- weight-shaped (unprojected) gradients --------------------------------
+ * projection_dim 0 / None, and the input of projection_target = "global":
+ * bergson/collector/collector.py:609-742 with p = None.  Normalisers as in
+ * bergson/gradients.py: Adafactor factors row_scale [O] / col_scale [I] (from
+ * bgx_adafactor_scales), or Adam second moments adam_v [O, I]
+ * (grad / (sqrt(v) + 1e-8), gradients.py:380-388); the two are exclusive, all
+ * NULL = no normaliser.  With the bias gradient collected every row of the
+ * gradient has I + 1 entries, the last being the bias gradient times
+ * bias_scale [O] (NULL = 1): rsqrt(bias_avg_sq + 1e-8) for Adafactor
+ * (gradients.py:339-349), 1 / (sqrt(bias_avg_sq) + 1e-8) for Adam (:390-400).
+ *
+ * bgx_token_sum: sum_dev[n, o] = sum_s g[n, s, o] (fp32), the bias gradient of
+ *   a sequence before its factor (collector.py:612-615, :650-653, :704-707).
+ * bgx_fullgrad_seq: P_dev [N, O, I] (contiguous, dtype) is the batched GEMM
+ *   g^T a that the caller ran with its BLAS (`g.mT @ a`, collector.py:623,
+ *   :684, :735).  Writes out[row(n), out_col + o*(I+b) + i] =
+ *   cast(clamp(normalise(P[n, o, i]))), row(n) = out_rows[n] (n when NULL);
+ *   bias_sum_dev [N, O] non-NULL adds the bias column (b = 1).
+ * bgx_fullgrad_tok: per token s < lengths[n] - 1 writes row
+ *   row_offsets[n] + s with out_col + o*(I+b) + i = normalise(g[o] * a[i])
+ *   (collector.py:620-632, :668-683, :730-734), bias column g[o] *
+ *   bias_scale[o] when collect_bias != 0. */
+int bgx_token_sum(const void* g_dev, int64_t g_seq_stride, int64_t g_tok_stride,
+                  int32_t N, int32_t S, int32_t O, int32_t dtype,
+                  float* sum_dev, void* stream);
+int bgx_fullgrad_seq(const void* P_dev, int32_t N, int32_t O, int32_t I,
+                     int32_t dtype, const float* row_scale_dev,
+                     const float* col_scale_dev, const float* adam_v_dev,
+                     const float* bias_sum_dev, const float* bias_scale_dev,
+                     const int64_t* out_rows_dev, void* out_dev,
+                     int64_t out_row_stride, int64_t out_col,
+                     int32_t out_dtype, float clamp_lo, float clamp_hi,
+                     void* stream);
+int bgx_fullgrad_tok(const void* a_dev, const void* g_dev,
+                     int64_t a_seq_stride, int64_t a_tok_stride,
+                     int64_t g_seq_stride, int64_t g_tok_stride, int32_t N,
+                     int32_t S, int32_t I, int32_t O, int32_t dtype,
+                     const float* row_scale_dev, const float* col_scale_dev,
+                     const float* adam_v_dev, int32_t collect_bias,
+                     const float* bias_scale_dev, const int32_t* lengths_dev,
+                     const int64_t* row_offsets_dev, void* out_dev,
+                     int64_t out_row_stride, int64_t out_col,
+                     int32_t out_dtype, float clamp_lo, float clamp_hi,
+                     void* stream);
+
 /* Benchmark support (no counterpart in the reference): while enabled, every
  * bgx_collect_seq / bgx_collect_tok call records a HIP event pair immediately
  * around its collect_kernel launch, on the launch stream, so that the kernel's

@@ -167,3 +167,13 @@ def module_gradient(a: Tensor, g: Tensor, normalizer, left: Tensor | None, right
     """forward_hook followed by backward_hook for one module."""
     stash = forward_hook(a, normalizer, right, kw.get("collect_bias", False))
     return backward_hook(stash, g, normalizer, left, right, **kw)
+
+
+def accumulate_global_projection(acc: Tensor | None, P: Tensor, R_single: Tensor) -> Tensor:
+    """`accumulate_global_projection` (collector.py:364-390): P [rows, O*I(+O)] is the clamped, flattened
+    gradient of one module, R_single [proj_dim, P.shape[1]] that module's block of the global projection;
+    the projected blocks of all modules are added in the model dtype."""
+    projected = P @ R_single.T
+    if acc is None:
+        return projected
+    return acc.add_(projected)

@@ -14,7 +14,7 @@ import torch.nn.functional as F
 from torch import Tensor
 
 from . import hooks
-from .projection import module_projections
+from .projection import module_projections, projection_matrix
 
 
 def allocate_batches(doc_lengths: list[int], N: int, seed: int = 42, max_batch_size: int | None = None
@@ -79,10 +79,13 @@ def target_linears(base_model: nn.Module) -> dict[str, nn.Linear]:
 def collect(model, base_model: nn.Module, docs: list[list[int]], batches: list[list[int]], *, p: int | None,
             normalizers: dict | None = None, projection_type: str = "normal", attribute_tokens: bool = False,
             include_bias: bool = False, save_dtype: torch.dtype | None = None, loss_reduction: str = "sum",
-            unit_normalize: bool = False) -> tuple[Tensor, Tensor]:
+            unit_normalize: bool = False, global_dim: int | None = None) -> tuple[Tensor, Tensor]:
     """The whole reference loop on CPU: returns (rows, losses).
 
     rows is [num_docs, D] (per sequence) or [sum(max(len-1, 0)), D] (per token), in save_dtype.
+    global_dim (with p=None) is projection_target="global": every module's unprojected gradient goes through
+    its block of one [global_dim, sum of module sizes] projection and the blocks are summed
+    (collector.py:364-402), so D = global_dim.
     """
     from .store import preprocess, token_offsets
 
@@ -120,7 +123,11 @@ def collect(model, base_model: nn.Module, docs: list[list[int]], batches: list[l
             left, right = get_proj(name, mod, g.dtype)
             P = hooks.backward_hook(stash.pop(name), g, normalizers.get(name), left, right, collect_bias=bias,
                                     attribute_tokens=attribute_tokens, collection_mask=state["mask"], lo=lo, hi=hi)
-            mod_grads[name] = P.to(save_dtype)
+            if global_dim is not None:
+                R = projection_matrix(f"{name}/single", global_dim, P.shape[1], P.dtype, projection_type, "jl")
+                mod_grads["gradients"] = hooks.accumulate_global_projection(mod_grads.get("gradients"), P, R)
+            else:
+                mod_grads[name] = P.to(save_dtype)
         return hook
 
     handles = []
@@ -137,7 +144,11 @@ def collect(model, base_model: nn.Module, docs: list[list[int]], batches: list[l
             x, y, mask = pad_and_tensor([docs[i] for i in indices])
             state["mask"] = mask
             losses = losses_and_backward(model, x, y, loss_reduction)
-            grad_sizes = {n: mod_grads[n].shape[1] for n in targets}
+            if global_dim is not None:  # finalize_global_projection, collector.py:392-402
+                mod_grads["gradients"] = mod_grads["gradients"].to(save_dtype)
+                grad_sizes = {"gradients": global_dim}
+            else:
+                grad_sizes = {n: mod_grads[n].shape[1] for n in targets}
             g = preprocess(mod_grads, grad_sizes, unit_normalize)
             mod_grads.clear()
             if rows is None:

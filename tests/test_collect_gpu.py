@@ -403,3 +403,77 @@ def test_adam_with_bias(device, per_token):
                          hi=3e38)
     torch.cuda.synchronize()
     assert rel_l2(out.cpu(), want) <= 1e-5
+
+
+# ---- weight-shaped (unprojected) gradients ----------------------------------------------------------
+def _full_case(N, S, I, O, dtype, kind, bias, seed):
+    gen = torch.Generator().manual_seed(seed)
+    a = torch.randn(N, S, I, generator=gen).to(dtype)
+    g = (torch.randn(N, S, O, generator=gen) * 0.1).to(dtype)
+    norm = None
+    if kind == "adafactor":
+        norm = ohooks.Adafactor(torch.rand(O, generator=gen) + 0.1, torch.rand(I, generator=gen) + 0.1,
+                                torch.rand(O, generator=gen) + 0.1 if bias else None)
+    elif kind == "adam":
+        norm = ohooks.Adam(torch.rand(O, I, generator=gen) + 0.1, torch.rand(O, generator=gen) + 0.1 if bias else None)
+    return a, g, norm
+
+
+def _full_module(device, a, g, norm, bias, out_col):
+    from bergson_amd import ops
+
+    O, I = g.shape[2], a.shape[2]
+    mod = ops.FullGradModule(O=O, I=I, out_col=out_col, collect_bias=bias)
+    if isinstance(norm, ohooks.Adafactor):
+        mod.row_scale, mod.col_scale = ops.adafactor_scales(norm.row.to(device), norm.col.to(device), a.dtype)
+        if bias:
+            mod.bias_scale = norm.bias_avg_sq.to(device).add(1e-8).rsqrt()
+    elif isinstance(norm, ohooks.Adam):
+        mod.adam_v = norm.weight_avg_sq.to(device).contiguous()
+        if bias:
+            mod.bias_scale = (norm.bias_avg_sq.to(device).sqrt() + 1e-8).reciprocal()
+    return mod
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("kind", [None, "adafactor", "adam"])
+@pytest.mark.parametrize("bias", [False, True])
+def test_fullgrad_seq(device, dtype, kind, bias):
+    from bergson_amd import ops
+
+    N, S, I, O = 3, 37, 24, 40
+    a, g, norm = _full_case(N, S, I, O, dtype, kind, bias, seed=60)
+    lo, hi = torch.finfo(dtype).min, torch.finfo(dtype).max
+    want = ohooks.module_gradient(a, g, norm, None, None, collect_bias=bias, lo=lo, hi=hi)
+    width = O * (I + int(bias))
+    out = torch.zeros(5, 7 + width, dtype=dtype, device=device)
+    rows = torch.tensor([4, 0, 2], dtype=torch.int64, device=device)
+    ops.full_gradient(_full_module(device, a, g, norm, bias, 7), a.to(device), g.to(device), out, per_token=False,
+                      lengths=None, rows=rows, lo=lo, hi=hi)
+    torch.cuda.synchronize()
+    got = out.cpu()
+    assert rel_l2(got[[4, 0, 2], 7:], want) <= TOL[dtype]
+    assert got[:, :7].abs().sum() == 0 and got[[1, 3]].abs().sum() == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("kind", [None, "adafactor", "adam"])
+@pytest.mark.parametrize("bias", [False, True])
+def test_fullgrad_tok(device, dtype, kind, bias):
+    from bergson_amd import ops
+
+    N, S, I, O = 3, 21, 24, 20
+    lengths = [21, 2, 10]
+    a, g, norm = _full_case(N, S, I, O, dtype, kind, bias, seed=61)
+    mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+    lo, hi = torch.finfo(dtype).min, torch.finfo(dtype).max
+    want = ohooks.module_gradient(a, g, norm, None, None, collect_bias=bias, attribute_tokens=True,
+                                  collection_mask=mask, lo=lo, hi=hi)
+    counts = [l - 1 for l in lengths]
+    offs = [sum(counts[:n]) for n in range(N)]
+    out = torch.zeros(sum(counts), O * (I + int(bias)), dtype=dtype, device=device)
+    ops.full_gradient(_full_module(device, a, g, norm, bias, 0), a.to(device), g.to(device), out, per_token=True,
+                      lengths=torch.tensor(lengths, dtype=torch.int32, device=device),
+                      rows=torch.tensor(offs, dtype=torch.int64, device=device), lo=lo, hi=hi)
+    torch.cuda.synchronize()
+    assert rel_l2(out.cpu(), want) <= TOL[dtype]

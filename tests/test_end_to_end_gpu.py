@@ -177,3 +177,64 @@ def test_pythia14m_fp32_adam_and_mixed_normalizers(device):
             assert rel_l2(got[:, b * 256:(b + 1) * 256], want) <= 1e-4, (attribute_tokens, name)
     for h in handles:
         h.remove()
+
+
+@pytest.mark.parametrize("attribute_tokens", [False, True])
+def test_unprojected_gradients_match_cpu_loop(device, tmp_path, attribute_tokens):
+    """projection_dim=0: the store holds the weight-shaped gradients themselves."""
+    from bergson_amd import GradientProcessor, IndexConfig, allocate_batches, collect_gradients, load_gradients
+    from bergson_amd.synthetic import ListDataset, make_gpt_neox, random_docs
+
+    lengths = [20, 9, 1, 16, 5]
+    docs = random_docs(lengths, seed=7)
+    batches = allocate_batches(lengths, 40)
+    model_cpu = make_gpt_neox("pythia-14m", torch.float32, "cpu", seed=0, layers=1)
+    want, _ = oloop.collect(model_cpu, model_cpu.base_model, docs, batches, p=None, attribute_tokens=attribute_tokens)
+    model = make_gpt_neox("pythia-14m", torch.float32, device, seed=0, layers=1)
+    cfg = IndexConfig(run_path=str(tmp_path / "full"), projection_dim=0, attribute_tokens=attribute_tokens)
+    collect_gradients(model, ListDataset(docs), GradientProcessor(projection_dim=None), cfg, batches=batches)
+    torch.cuda.synchronize()
+    part = cfg.partial_run_path
+    info = json.loads((part / "info.json").read_text())
+    assert list(info["grad_sizes"].values()) == [384 * 128, 128 * 128, 512 * 128, 128 * 512]
+    if attribute_tokens:
+        from bergson_amd import TokenGradients
+
+        tg = TokenGradients(part)
+        got = torch.cat([torch.from_numpy(np.array(tg[i])) for i in range(len(docs))])
+    else:
+        got = torch.from_numpy(np.array(load_gradients(part)))
+    assert got.shape == want.shape
+    assert rel_l2(got, want) <= 1e-3
+
+
+@pytest.mark.parametrize("attribute_tokens", [False, True])
+def test_global_projection_matches_cpu_loop(device, tmp_path, attribute_tokens):
+    """projection_target="global": one [projection_dim] row per document (or token) over all modules."""
+    from bergson_amd import GradientProcessor, IndexConfig, allocate_batches, collect_gradients, load_gradients
+    from bergson_amd.synthetic import ListDataset, make_gpt_neox, random_docs
+
+    lengths = [20, 9, 1, 16, 5]
+    docs = random_docs(lengths, seed=8)
+    batches = allocate_batches(lengths, 40)
+    model_cpu = make_gpt_neox("pythia-14m", torch.float32, "cpu", seed=0, layers=1)
+    want, _ = oloop.collect(model_cpu, model_cpu.base_model, docs, batches, p=None, global_dim=32,
+                            attribute_tokens=attribute_tokens)
+    model = make_gpt_neox("pythia-14m", torch.float32, device, seed=0, layers=1)
+    cfg = IndexConfig(run_path=str(tmp_path / "glob"), projection_dim=32, projection_type="normal",
+                      attribute_tokens=attribute_tokens)
+    proc = GradientProcessor(projection_dim=32, projection_type="normal", projection_target="global")
+    collect_gradients(model, ListDataset(docs), proc, cfg, batches=batches)
+    torch.cuda.synchronize()
+    part = cfg.partial_run_path
+    info = json.loads((part / "info.json").read_text())
+    assert info["grad_sizes"] == {"gradients": 32}
+    if attribute_tokens:
+        from bergson_amd import TokenGradients
+
+        tg = TokenGradients(part)
+        got = torch.cat([torch.from_numpy(np.array(tg[i])) for i in range(len(docs))])
+    else:
+        got = torch.from_numpy(np.array(load_gradients(part)))
+    assert got.shape == want.shape
+    assert rel_l2(got, want) <= 1e-3

@@ -143,3 +143,28 @@ def test_normalizer_helpers_match_closed_forms():
     b = torch.randn(3, generator=gen)
     torch.testing.assert_close(H.adam_normalize_bias(b, m), b / (m.bias_avg_sq.sqrt() + 1e-8))
     torch.testing.assert_close(H.adafactor_normalize_bias(b, n), b / (n.bias_avg_sq + 1e-8).sqrt())
+
+
+def test_global_projection_is_the_projection_of_the_concatenated_gradient():
+    """projection_target="global" (collector.py:364-402): summing each module's block `P_m @ R_m^T` equals
+    projecting the concatenation of the per-sample autograd gradients with the concatenated blocks, and the
+    blocks are the matrices named "<module>/single"."""
+    from oracle.projection import projection_matrix
+
+    torch.manual_seed(0)
+    gen = torch.Generator().manual_seed(3)
+    N, S, pd = 3, 4, 5
+    lins = {"m.a": nn.Linear(6, 5), "m.b": nn.Linear(5, 7)}
+    acc = None
+    grads, blocks = [], []
+    for name, lin in lins.items():
+        x = torch.randn(N, S, lin.in_features, generator=gen)
+        a, g, wg, _ = _capture(lin, x, _loss)
+        P = H.module_gradient(a, g, None, None, None)
+        R = projection_matrix(f"{name}/single", pd, P.shape[1], torch.float32)
+        acc = H.accumulate_global_projection(acc, P, R)
+        grads.append(torch.stack([w.flatten() for w in wg]))
+        blocks.append(R)
+    want = torch.cat(grads, dim=1) @ torch.cat(blocks, dim=1).T
+    assert acc.shape == (N, pd)
+    torch.testing.assert_close(acc, want, rtol=1e-4, atol=1e-5)
