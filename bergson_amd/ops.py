@@ -290,11 +290,38 @@ class AdamPrepared:
             # 1 / (sqrt(bias_avg_sq) + 1e-8): eps outside the root
             self.bias_scale = (bias_avg_sq.detach().to(device=r_in.device, dtype=torch.float32).sqrt() + 1e-8
                                ).reciprocal().contiguous()
-        v = weight_avg_sq.detach().to(device=r_in.device, dtype=torch.float32).contiguous()
-        nbytes = lib.bgx_adam_table_bytes(O, I, p, dtype_code(self.dtype))
-        self.table = torch.empty(nbytes // self.r_in.element_size(), dtype=self.dtype, device=r_in.device)
-        rc = lib.bgx_adam_prepare(_ptr(self.r_in), _ptr(v), O, I, p, dtype_code(self.dtype), _ptr(self.table), _stream())
-        _lib.check(rc, "bgx_adam_prepare")
+        self.v = weight_avg_sq.detach().to(device=r_in.device, dtype=torch.float32).contiguous()
+        self._table: Tensor | None = None
+        self._seq_state = None
+
+    @property
+    def table(self) -> Tensor:
+        """[(O*p), I] table of the per-token path, built on first use."""
+        if self._table is None:
+            lib = _lib.load()
+            nbytes = lib.bgx_adam_table_bytes(self.O, self.I, self.p, dtype_code(self.dtype))
+            self._table = torch.empty(nbytes // self.r_in.element_size(), dtype=self.dtype, device=self.r_in.device)
+            rc = lib.bgx_adam_prepare(_ptr(self.r_in), _ptr(self.v), self.O, self.I, self.p, dtype_code(self.dtype),
+                                      _ptr(self._table), _stream())
+            _lib.check(rc, "bgx_adam_prepare")
+        return self._table
+
+    def seq_state(self):
+        """Operands of the per-sequence path that do not change between batches: the normaliser module of
+        the weight-shaped gradient, the right projection over [grad | bias] and L^T with an identity
+        projection (see collect_adam)."""
+        if self._seq_state is None:
+            dev = self.r_in.device
+            bias = self.bias_col is not None
+            full = FullGradModule(O=self.O, I=self.I, out_col=0, collect_bias=bias, adam_v=self.v,
+                                  bias_scale=self.bias_scale)
+            r_in = self.r_in
+            if bias:
+                r_in = torch.cat([self.r_in, self.bias_col.to(self.dtype).unsqueeze(1)], dim=1).contiguous()
+            lt = self.r_out.t().contiguous()  # [O, p]: row o is what output feature o contributes to every P[i, :]
+            eye = torch.eye(self.p, dtype=self.dtype, device=dev)
+            self._seq_state = (full, r_in, lt, eye)
+        return self._seq_state
 
 
 def collect_adam(prep: AdamPrepared, a: Tensor, g: Tensor, out: Tensor, *, per_token: bool, lengths: Tensor | None,
@@ -317,6 +344,9 @@ def collect_adam(prep: AdamPrepared, a: Tensor, g: Tensor, out: Tensor, *, per_t
         raise ValueError("out must be a 2-D tensor with contiguous rows")
     if per_token and (lengths is None or rows is None):
         raise ValueError("per-token collection needs lengths and row offsets")
+    if not per_token and chunk_tokens == 0:
+        _collect_adam_seq(prep, a, g, out, lengths, rows, lo, hi)
+        return
     nbytes = lib.bgx_collect_adam_workspace_bytes(N, S, O, prep.p, chunk_tokens)
     ws = _workspace(out.device, nbytes, "adam")
     rc = lib.bgx_collect_adam(_ptr(a), _ptr(g), a.stride(0), a.stride(1), g.stride(0), g.stride(1), N, S, I, O, prep.p,
@@ -388,6 +418,29 @@ def full_gradient(mod: FullGradModule, a: Tensor, g: Tensor, out: Tensor, *, per
                               _ptr(bias_sum), _ptr(mod.bias_scale), _ptr(rows), _ptr(out), out.stride(0), mod.out_col,
                               dtype_code(out.dtype), lo, hi, _stream())
     _lib.check(rc, "bgx_fullgrad_seq")
+
+
+def _collect_adam_seq(prep: AdamPrepared, a: Tensor, g: Tensor, out: Tensor, lengths: Tensor | None,
+                      rows: Tensor | None, lo: float, hi: float) -> None:
+    """Per-sequence Adam without anything per token: the normalisation is applied to the summed gradient, as
+    the reference does (collector.py:634-644):
+        Q[n] = (g[n]^T a[n]) / (sqrt(v) + 1e-8)  [| bias column]     batched GEMM + bgx_fullgrad_seq
+        P[n] = L Q[n] R^T                                            bgx_collect_seq with the output features
+    in the role of tokens: "a" = Q[n] ([O, I(+1)] rows), projected by R; "g" = L^T ([O, p], shared by all n,
+    sequence stride 0) with an identity projection; the token reduction is the sum over output features.
+    """
+    N, S, _ = a.shape
+    full, r_in, lt, eye = prep.seq_state()
+    if lengths is not None:
+        # positions from len-1 on carry no label; zero them instead of relying on the model's zeros
+        keep = (torch.arange(S, device=g.device).unsqueeze(0) + 1 < lengths.unsqueeze(1)).unsqueeze(-1)
+        g = g * keep
+    q = torch.empty((N, full.width), dtype=prep.dtype, device=a.device)
+    full_gradient(full, a, g, q, per_token=False, lengths=None, rows=None, lo=float("-inf"), hi=float("inf"))
+    Iw = full.width // prep.O
+    m = ModuleInput(a=q.view(N, prep.O, Iw), g=lt.unsqueeze(0).expand(N, prep.O, prep.p), r_in=r_in, r_out=eye,
+                    out_col=prep.out_col)
+    _collect(False, [m], prep.p, out, None, rows, lo, hi)
 
 
 def collect_seq(modules: list[ModuleInput], p: int, out: Tensor, *, lengths: Tensor | None = None,

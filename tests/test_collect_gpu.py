@@ -298,10 +298,13 @@ def _run_adam(device, case, p, out_dtype, *, per_token=False, lengths=None, row_
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(2, 40, 64, 96, 16), (3, 70, 128, 64, 32), (1, 33, 96, 40, 8)])
-def test_adam_seq(device, dtype, shape):
+@pytest.mark.parametrize("chunk_tokens", [0, 64])
+def test_adam_seq(device, dtype, shape, chunk_tokens):
+    """chunk_tokens = 0: the normalisation is applied to the summed gradient (batched GEMM, then the
+    collection kernel over output features); 64: the per-token formulation in several internal passes."""
     N, S, I, O, p = shape
     case = _adam_case(N, S, I, O, p, dtype, seed=50)
-    got = _run_adam(device, case, p, dtype, chunk_tokens=64)  # several internal passes
+    got = _run_adam(device, case, p, dtype, chunk_tokens=chunk_tokens)
     a, g, left, right, norm = case
     want = ohooks.module_gradient(a, g, norm, left, right)
     assert got.shape == want.shape
@@ -477,3 +480,19 @@ def test_fullgrad_tok(device, dtype, kind, bias):
                       rows=torch.tensor(offs, dtype=torch.int64, device=device), lo=lo, hi=hi)
     torch.cuda.synchronize()
     assert rel_l2(out.cpu(), want) <= TOL[dtype]
+
+
+def test_adam_seq_with_lengths_and_rows(device):
+    """Per-sequence Adam with positions past each document's last label skipped and rows scattered."""
+    N, S, I, O, p = 3, 48, 64, 96, 16
+    lengths = [48, 20, 33]
+    case = _adam_case(N, S, I, O, p, torch.float32, seed=52)
+    a, g, left, right, norm = case
+    gz = g.clone()
+    for n, l in enumerate(lengths):
+        gz[n, l - 1:] = 0
+    want = ohooks.module_gradient(a, gz, norm, left, right)
+    # g itself is NOT zeroed: the lengths must do it
+    got = _run_adam(device, case, p, torch.float32, lengths=lengths, row_offsets=[2, 0, 1], n_rows=4)
+    assert rel_l2(got[[2, 0, 1]], want) <= 1e-5
+    assert got[3].abs().sum() == 0
