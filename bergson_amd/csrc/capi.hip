@@ -52,8 +52,8 @@ int unit_normalize_impl(void* rows, int64_t n_rows, int64_t D, int64_t stride, i
 size_t scan_workspace_bytes(int Q, int k, int64_t chunk_rows);
 int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int dtype, const void* queries, int Q,
               float query_scale, int unit_norm, int k, int64_t row_base, float* topk_val, int64_t* topk_idx,
-              float* row_max, float* scores, float* sumsq, void* ws, size_t ws_bytes, int64_t chunk_rows,
-              void* stream);
+              float* row_max, float* row_mean, float* scores, float* sumsq, void* ws, size_t ws_bytes,
+              int64_t chunk_rows, void* stream);
 
 }  // namespace bgx
 
@@ -158,11 +158,11 @@ size_t bgx_scan_workspace_bytes(int32_t Q, int32_t k, int64_t chunk_rows) {
 
 int bgx_scan(const void* store_dev, int64_t n_rows, int64_t D, int64_t store_row_stride, int32_t dtype,
              const void* queries_dev, int32_t Q, float query_scale, int32_t unit_norm, int32_t k, int64_t row_base,
-             float* topk_val_dev, int64_t* topk_idx_dev, float* row_max_dev, float* scores_dev, float* sumsq_dev,
-             void* workspace_dev, size_t workspace_bytes, int64_t chunk_rows, void* stream) {
+             float* topk_val_dev, int64_t* topk_idx_dev, float* row_max_dev, float* row_mean_dev, float* scores_dev,
+             float* sumsq_dev, void* workspace_dev, size_t workspace_bytes, int64_t chunk_rows, void* stream) {
   return bgx::scan_impl(store_dev, n_rows, D, store_row_stride, dtype, queries_dev, Q, query_scale, unit_norm, k,
-                        row_base, topk_val_dev, topk_idx_dev, row_max_dev, scores_dev, sumsq_dev, workspace_dev,
-                        workspace_bytes, chunk_rows, stream);
+                        row_base, topk_val_dev, topk_idx_dev, row_max_dev, row_mean_dev, scores_dev, sumsq_dev,
+                        workspace_dev, workspace_bytes, chunk_rows, stream);
 }
 
 }  // extern "C"

@@ -132,6 +132,8 @@ struct ScanArgs {
   float* scores;         // [n_rows, Q]
   float* sumsq;          // [n_rows]
   uint32_t* row_max_enc; // [n_rows] ordered-uint encoding
+  float* row_sum_part;   // [rows of this pass][n_parts] sum over each wave column's queries, or null
+  int n_parts;           // q_tiles * (waves along the queries)
   const float* thr;      // [Q] current k-th best per query
   uint32_t* cand_count;  // [Q]
   uint64_t* cand;        // [Q][cand_cap]
@@ -310,12 +312,14 @@ __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
       const int64_t grow = args.row0 + prow;
       const float w = s_inv[row];
       float rmax = -INFINITY;
+      float rsum = 0.f;
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         const int64_t q = q_row0 + wn * WTN + j * 32 + fr;
         const float v = acc[i][j][e] * w;
         if (row_ok && q < args.Q) {
           rmax = fmaxf(rmax, v);
+          rsum += v;
           if (args.scores != nullptr) args.scores[grow * args.Q + q] = v;
           if (v > thr[j]) {
             const uint32_t pos = atomicAdd(&args.cand_count[q], 1u);
@@ -330,6 +334,15 @@ __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
         rmax = fmaxf(rmax, __shfl_xor(rmax, 8));
         rmax = fmaxf(rmax, __shfl_xor(rmax, 16));
         if (fr == 0 && row_ok) atomicMax(&args.row_max_enc[grow], f32_ordered(rmax));
+      }
+      if (args.row_sum_part != nullptr) {
+        // fixed-order butterfly over the 32 lanes that hold this row's scores; one writer per (row, part)
+        rsum += __shfl_xor(rsum, 1);
+        rsum += __shfl_xor(rsum, 2);
+        rsum += __shfl_xor(rsum, 4);
+        rsum += __shfl_xor(rsum, 8);
+        rsum += __shfl_xor(rsum, 16);
+        if (fr == 0 && row_ok) args.row_sum_part[prow * args.n_parts + qt * WN + wn] = rsum;
       }
     }
   }
@@ -460,6 +473,16 @@ __global__ void scan_finish_kernel(const uint64_t* top, int Q, int k, int64_t ro
   if (row_max != nullptr && i < n_rows) row_max[i] = ordered_f32(row_max_enc[i]);
 }
 
+// row_mean[row0 + r] = (sum of the row's partial sums, in part order) / Q
+__global__ void scan_row_mean_kernel(const float* __restrict__ part, int n_parts, int64_t rows, int64_t row0,
+                                     float inv_q, float* __restrict__ row_mean) {
+  const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= rows) return;
+  float s = 0.f;
+  for (int p = 0; p < n_parts; ++p) s += part[r * n_parts + p];
+  row_mean[row0 + r] = s * inv_q;
+}
+
 // ---- host side --------------------------------------------------------------------------------
 constexpr int64_t SCAN_DEFAULT_CHUNK = 65536;
 constexpr int64_t SCAN_FIRST_CHUNK = 4096;
@@ -467,7 +490,7 @@ constexpr int64_t SCAN_FIRST_CHUNK = 4096;
 static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 struct ScanLayout {
-  size_t top, top_count, cand_count, thr, cand, total;
+  size_t top, top_count, cand_count, thr, row_part, cand, total;
 };
 
 static ScanLayout scan_layout(int Q, int k, int64_t chunk_rows) {
@@ -481,6 +504,8 @@ static ScanLayout scan_layout(int Q, int k, int64_t chunk_rows) {
   off += align_up((size_t)Q * 4, 256);
   l.thr = off;
   off += align_up((size_t)Q * 4, 256);
+  l.row_part = off;  // per-pass partial row sums: at most 4 wave columns per 256-query tile
+  off += align_up((size_t)chunk_rows * (size_t)((Q + 255) / 256 * 4) * 4, 256);
   l.cand = off;
   off += k > 0 ? align_up((size_t)Q * (size_t)chunk_rows * 8, 256) : 0;
   l.total = off;
@@ -530,16 +555,19 @@ static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
     constexpr int BM = 256, BN = 256;
     a.row_tiles = (int)((a.rows + BM - 1) / BM);
     a.q_tiles = (a.Q + BN - 1) / BN;
+    a.n_parts = a.q_tiles * 4;
     return launch_gemm<T, BM, BN, 2, 4>(a, aligned, st);
   } else if (a.Q > 32) {
     constexpr int BM = 128, BN = 64;
     a.row_tiles = (int)((a.rows + BM - 1) / BM);
     a.q_tiles = (a.Q + BN - 1) / BN;
+    a.n_parts = a.q_tiles;
     return launch_gemm<T, BM, BN, 4, 1>(a, aligned, st);
   } else {
     constexpr int BM = 128, BN = 32;
     a.row_tiles = (int)((a.rows + BM - 1) / BM);
     a.q_tiles = (a.Q + BN - 1) / BN;
+    a.n_parts = a.q_tiles;
     return launch_gemm<T, BM, BN, 4, 1>(a, aligned, st);
   }
 }
@@ -562,6 +590,8 @@ int gemm_scores(const void* rows, int64_t n_rows, int64_t D, int64_t stride, int
   a.scores = scores;
   a.sumsq = nullptr;
   a.row_max_enc = nullptr;
+  a.row_sum_part = nullptr;
+  a.n_parts = 0;
   a.thr = nullptr;
   a.cand_count = nullptr;
   a.cand = nullptr;
@@ -576,8 +606,8 @@ int gemm_scores(const void* rows, int64_t n_rows, int64_t D, int64_t stride, int
 
 int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int dtype, const void* queries, int Q,
               float query_scale, int unit_norm, int k, int64_t row_base, float* topk_val, int64_t* topk_idx,
-              float* row_max, float* scores, float* sumsq, void* ws, size_t ws_bytes, int64_t chunk_rows,
-              void* stream) {
+              float* row_max, float* row_mean, float* scores, float* sumsq, void* ws, size_t ws_bytes,
+              int64_t chunk_rows, void* stream) {
   BGX_REQUIRE(store && queries, BGX_E_ARG, "scan: null store/queries");
   BGX_REQUIRE(n_rows > 0 && D > 0 && Q > 0 && stride >= D, BGX_E_ARG, "scan: n_rows=%lld D=%lld Q=%d stride=%lld",
               (long long)n_rows, (long long)D, Q, (long long)stride);
@@ -595,8 +625,8 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
   const int64_t chunk = effective_chunk(chunk_rows, Q);
   const ScanLayout lay = scan_layout(Q, k, chunk);
   const bool need_init = want_topk || row_max != nullptr;
-  if (want_topk) {
-    BGX_REQUIRE(ws != nullptr, BGX_E_WORKSPACE, "scan: workspace required for top-k");
+  if (want_topk || row_mean != nullptr) {
+    BGX_REQUIRE(ws != nullptr, BGX_E_WORKSPACE, "scan: workspace required for top-k and row means");
     BGX_REQUIRE(((uintptr_t)ws & 255) == 0, BGX_E_ALIGN, "scan: workspace must be 256-byte aligned");
     BGX_REQUIRE(ws_bytes >= lay.total, BGX_E_WORKSPACE, "scan: workspace %zu < %zu bytes", ws_bytes, lay.total);
   }
@@ -607,6 +637,7 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
   uint32_t* cand_count = want_topk ? (uint32_t*)(w + lay.cand_count) : nullptr;
   float* thr = want_topk ? (float*)(w + lay.thr) : nullptr;
   uint64_t* cand = want_topk ? (uint64_t*)(w + lay.cand) : nullptr;
+  float* row_part = row_mean != nullptr ? (float*)(w + lay.row_part) : nullptr;
   // the row maxima are accumulated in place in an order-preserving integer
   // encoding and decoded by the finish kernel
   uint32_t* row_max_enc = (uint32_t*)row_max;
@@ -635,6 +666,7 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
       if (lim > chunk) lim = chunk;
       if (rows > lim) rows = lim;
     }
+    if (row_part != nullptr && rows > chunk) rows = chunk;  // the partial sums of one pass fit the workspace
     ScanArgs a;
     a.store = store;
     a.queries = queries;
@@ -650,6 +682,8 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
     a.scores = scores;
     a.sumsq = sumsq;
     a.row_max_enc = row_max_enc;
+    a.row_sum_part = row_part;
+    a.n_parts = 0;
     a.thr = thr;
     a.cand_count = cand_count;
     a.cand = cand;
@@ -662,6 +696,11 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
     else
       rc = launch_gemm_t<float>(a, aligned, st);
     if (rc != 0) return rc;
+    if (row_part != nullptr) {
+      hipLaunchKernelGGL(scan_row_mean_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, row_part,
+                         a.n_parts, rows, done, 1.0f / (float)Q, row_mean);
+      BGX_HIP(hipGetLastError());
+    }
     if (want_topk) {
       SelectArgs s;
       s.top = top;

@@ -472,13 +472,14 @@ class ScanResult:
     topk_values: Tensor | None = None  # [Q, k] fp32
     topk_indices: Tensor | None = None  # [Q, k] int64
     row_max: Tensor | None = None  # [n_rows] fp32
+    row_mean: Tensor | None = None  # [n_rows] fp32
     scores: Tensor | None = None  # [n_rows, Q] fp32
     sumsq: Tensor | None = None  # [n_rows] fp32
 
 
 def scan(store: Tensor, queries: Tensor, *, unit_norm: bool, k: int = 0, query_scale: float = 1.0, row_base: int = 0,
-         want_row_max: bool = False, want_scores: bool = False, want_sumsq: bool = False,
-         chunk_rows: int = 0) -> ScanResult:
+         want_row_max: bool = False, want_row_mean: bool = False, want_scores: bool = False,
+         want_sumsq: bool = False, chunk_rows: int = 0) -> ScanResult:
     """Score store rows [n, D] against queries [Q, D] (same dtype); see bgx_scan in include/bergson_amd.h."""
     lib = _lib.load()
     _need_gpu(store, "store")
@@ -499,16 +500,18 @@ def scan(store: Tensor, queries: Tensor, *, unit_norm: bool, k: int = 0, query_s
         res.topk_indices = torch.empty((Q, k), dtype=torch.int64, device=dev)
     if want_row_max:
         res.row_max = torch.empty((n,), dtype=torch.float32, device=dev)
+    if want_row_mean:
+        res.row_mean = torch.empty((n,), dtype=torch.float32, device=dev)
     if want_scores:
         res.scores = torch.empty((n, Q), dtype=torch.float32, device=dev)
     if want_sumsq:
         res.sumsq = torch.empty((n,), dtype=torch.float32, device=dev)
     ws = None
-    if k:
+    if k or want_row_mean:
         ws = _workspace(dev, lib.bgx_scan_workspace_bytes(Q, k, chunk_rows), "scan")
     rc = lib.bgx_scan(_ptr(store), n, D, store.stride(0), dtype_code(store.dtype), _ptr(queries), Q, query_scale,
                       int(unit_norm), k, row_base, _ptr(res.topk_values), _ptr(res.topk_indices), _ptr(res.row_max),
-                      _ptr(res.scores), _ptr(res.sumsq), _ptr(ws), 0 if ws is None else ws.numel(), chunk_rows,
+                      _ptr(res.row_mean), _ptr(res.scores), _ptr(res.sumsq), _ptr(ws), 0 if ws is None else ws.numel(), chunk_rows,
                       _stream())
     _lib.check(rc, "bgx_scan")
     return res

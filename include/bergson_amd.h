@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define BGX_ABI_VERSION 1
+#define BGX_ABI_VERSION 2
 
 enum bgx_dtype { BGX_F32 = 0, BGX_F16 = 1, BGX_BF16 = 2 };
 
@@ -255,6 +255,11 @@ size_t bgx_scan_workspace_bytes(int32_t Q, int32_t k, int64_t chunk_rows);
  *     (torch.topk, attributor.py:229-235); requires k <= n_rows, k <= 2048
  *   row_max_dev [n_rows] fp32: max over queries (score_mode "nearest",
  *     scorer.py:111-113)
+ *   row_mean_dev [n_rows] fp32: mean over queries, summed in a fixed order.
+ *     By linearity this is the score against the mean of the queries, which
+ *     is how the reference obtains it (aggregation "mean",
+ *     bergson/process_grads.py:166-182, then scorer.py:89-115); needs the
+ *     workspace
  *   scores_dev [n_rows, Q] fp32 row-major: every score (scorer.py:89-115)
  *   sumsq_dev [n_rows] fp32: sum of squares of each row
  * row_base is added to the row numbers reported in topk_idx_dev. */
@@ -262,9 +267,9 @@ int bgx_scan(const void* store_dev, int64_t n_rows, int64_t D,
              int64_t store_row_stride, int32_t dtype, const void* queries_dev,
              int32_t Q, float query_scale, int32_t unit_norm, int32_t k,
              int64_t row_base, float* topk_val_dev, int64_t* topk_idx_dev,
-             float* row_max_dev, float* scores_dev, float* sumsq_dev,
-             void* workspace_dev, size_t workspace_bytes, int64_t chunk_rows,
-             void* stream);
+             float* row_max_dev, float* row_mean_dev, float* scores_dev,
+             float* sumsq_dev, void* workspace_dev, size_t workspace_bytes,
+             int64_t chunk_rows, void* stream);
 
 #ifdef __cplusplus
 }

@@ -54,11 +54,17 @@ def test_scan_cosine_topk(device, dtype, shape):
     # the oracle scores what the kernel is given: store rows in `dtype`, unit queries rounded to `dtype`
     qd = qn.to(dtype)
     ref = oscan.scorer_score({"m": store}, {"m": qd}, ["m"], dtype=torch.float32, unit_normalize=True).T  # [Q, n]
-    res = ops.scan(store.to(device), qd.to(device), unit_norm=True, k=k, want_row_max=True, want_scores=True,
-                   want_sumsq=True, chunk_rows=1024)
+    res = ops.scan(store.to(device), qd.to(device), unit_norm=True, k=k, want_row_max=True, want_row_mean=True,
+                   want_scores=True, want_sumsq=True, chunk_rows=1024)
     torch.cuda.synchronize()
     scores = res.scores.cpu().T
     assert (scores - ref).abs().max().item() <= COS_TOL
+    # mean over queries: the mean of the scores, which by linearity is the score against the mean query
+    # (how the reference gets it: aggregate the queries first, process_grads.py:166-182)
+    assert (res.row_mean.cpu() - ref.mean(0)).abs().max().item() <= COS_TOL
+    ref_mean_query = oscan.scorer_score({"m": store}, {"m": qd.float().mean(0, keepdim=True)}, ["m"],
+                                        dtype=torch.float32, unit_normalize=True)[:, 0]
+    assert (res.row_mean.cpu() - ref_mean_query).abs().max().item() <= COS_TOL
     assert torch.allclose(res.sumsq.cpu(), store.float().pow(2).sum(1), rtol=1e-4)
     assert (res.row_max.cpu() - ref.max(0).values).abs().max().item() <= COS_TOL
     check_topk(res.topk_values.cpu(), res.topk_indices.cpu(), ref, k)
@@ -156,3 +162,18 @@ def test_scan_k_equals_rows_and_unaligned_dim(device):
     rv, ri = torch.topk(ref, 37, dim=1)
     assert torch.equal(res.topk_indices.cpu(), ri)
     assert torch.allclose(res.topk_values.cpu(), rv, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("Q", [5, 48, 300])
+def test_scan_row_mean_alone(device, Q):
+    """Only the mean over queries is asked for (no top-k): several passes, every tile configuration."""
+    from bergson_amd import ops
+
+    n, D = 3000, 256
+    store, queries = make_store(n, D, Q, torch.float16, seed=77)
+    qd = unit_queries(queries, torch.float16).to(torch.float16)
+    ref = oscan.scorer_score({"m": store}, {"m": qd}, ["m"], dtype=torch.float32, unit_normalize=True)  # [n, Q]
+    res = ops.scan(store.to(device), qd.to(device), unit_norm=True, want_row_mean=True, chunk_rows=1024)
+    torch.cuda.synchronize()
+    assert res.topk_values is None
+    assert (res.row_mean.cpu() - ref.mean(1)).abs().max().item() <= COS_TOL
