@@ -64,10 +64,10 @@ def test_argument_errors_before_any_launch():
     assert rc == -4 and b"workspace" in lib.bgx_last_error()
     rc = lib.bgx_collect_tok(descs, 1, 1, 8, 16, 2, None, None, C.c_void_p(256), 256, 2, 0.0, 0.0, C.c_void_p(256), 1 << 20, None)
     assert rc == -1 and b"lengths" in lib.bgx_last_error()
-    rc = lib.bgx_scan(None, 10, 8, 8, 1, None, 2, 1.0, 1, 1, 0, None, None, None, None, None, None, 0, 0, None)
+    rc = lib.bgx_scan(None, 10, 8, 8, 1, None, 2, 1.0, 1, 1, 0, None, None, None, None, None, None, None, 0, 0, None)
     assert rc == -1
     rc = lib.bgx_scan(C.c_void_p(256), 10, 8, 8, 1, C.c_void_p(256), 2, 1.0, 1, 11, 0, C.c_void_p(256), C.c_void_p(256),
-                      None, None, None, C.c_void_p(256), 1 << 30, 0, None)
+                      None, None, None, None, C.c_void_p(256), 1 << 30, 0, None)
     assert rc == -3 and b"k=11" in lib.bgx_last_error()
     rc = lib.bgx_unit_normalize_rows(None, 1, 1, 1, 0, None)
     assert rc == -1
