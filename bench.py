@@ -223,7 +223,7 @@ def main():
     args = parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported in this build "
-              "(collection shards by documents with no exchange, see DESIGN.md)", file=sys.stderr)
+              "(collection shards by documents with no exchange; the scan shards by store rows)", file=sys.stderr)
         sys.exit(2)
     import torch
 

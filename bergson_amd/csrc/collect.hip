@@ -33,6 +33,7 @@
 namespace bgx {
 
 constexpr int COLLECT_THREADS = 256;
+constexpr int STAGE_B = 6;
 
 // ---- MFMA step per element type ---------------------------------------------
 // A "k-step" of one wave covers KS consecutive k; lane (r = lane%16, q = lane/16)
@@ -407,7 +408,7 @@ __device__ inline void stage_projection(const T* __restrict__ R, const float* __
                                         uint4* __restrict__ dst, int tid) {
   using M = Mma<T>;
   const int nfrag = (K / M::KS) * WAVE;
-  constexpr int B = 6;  // fragments per thread in flight
+  constexpr int B = STAGE_B;  // fragments per thread in flight
   for (int f0 = tid; f0 < nfrag; f0 += COLLECT_THREADS * B) {
     uint4 v[B];
     uint4 s4[B][M::EPL / 4];
