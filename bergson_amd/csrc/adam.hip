@@ -4,23 +4,26 @@
 // sqrt(v) + 1e-8 and projects it from both sides (bergson/collector/collector.py:609-644,
 // bergson/gradients.py:380-388).  Per token t that is
 //     P_t[i, j] = sum_o L[i, o] g_t[o] * H_t[o, j],
-//     H_t[o, j] = sum_k a_t[k] * C[(o, j), k],      C[(o, j), k] = R[j, k] / (sqrt(v[o, k]) + 1e-8)
+//     H_t[o, j] = sum_k a_t[k] * C[(j, o), k],      C[(j, o), k] = R[j, k] / (sqrt(v[o, k]) + 1e-8)
 // so nothing weight-shaped is formed per token: H is one GEMM of the activations against a table C that
 // depends on the module only (built once by adam_table_kernel), and P_t is a small contraction of H_t with
 // L and g_t.  The per-sequence gradient is the sum of its tokens' P_t (the normalisation is linear).
 //
-// This build materialises H for a chunk of tokens at a time (GEMM on the scan kernel's main loop, then
-// adam_contract_kernel).  H is O*p values per token, which makes the path HBM-heavy for large modules;
-// fusing the contraction into the GEMM is the planned next step.
+// This build materialises H for a chunk of tokens at a time (GEMM on the scan kernel's main loop), stored
+// per token as [j][o] so that the contraction over o reads it contiguously, and contracts it on the matrix
+// cores (adam_contract_mfma_kernel): P_t = L Z_t with Z_t[o, j] = g_t[o] H_t[o, j], L as the A operand shared
+// by the tokens of a wave, Z_t formed in registers as the B operand.  H is O*p values per token, which makes
+// the path HBM-heavy for large modules; fusing the contraction into the GEMM is the planned next step.
 
 #include "common.hpp"
+#include "mma16.hpp"
 
 namespace bgx {
 
 int gemm_scores(const void* rows, int64_t n_rows, int64_t D, int64_t stride, int dtype, const void* queries, int Q,
                 float* scores, hipStream_t st);
 
-// table[(o * p + j) * I + k] = round_T(R[j, k] / (sqrt(v[o, k]) + 1e-8))
+// table[(j * O + o) * I + k] = round_T(R[j, k] / (sqrt(v[o, k]) + 1e-8))
 template <typename T>
 __global__ __launch_bounds__(256) void adam_table_kernel(const T* __restrict__ r_in, const float* __restrict__ v, int O,
                                                          int I, int p, T* __restrict__ table) {
@@ -28,9 +31,9 @@ __global__ __launch_bounds__(256) void adam_table_kernel(const T* __restrict__ r
   for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
        idx += (int64_t)gridDim.x * blockDim.x) {
     const int k = (int)(idx % I);
-    const int64_t oj = idx / I;
-    const int j = (int)(oj % p);
-    const int o = (int)(oj / p);
+    const int64_t jo = idx / I;
+    const int o = (int)(jo % O);
+    const int j = (int)(jo / O);
     const float w = 1.0f / (sqrtf(v[(int64_t)o * I + k]) + 1e-8f);
     const float val = Elem<T>::load(r_in + (int64_t)j * I + k) * w;
     if constexpr (sizeof(T) == 4)
@@ -43,7 +46,7 @@ __global__ __launch_bounds__(256) void adam_table_kernel(const T* __restrict__ r
 }
 
 struct ContractArgs {
-  const float* H;        // [chunk_tokens, O * p]
+  const float* H;        // [chunk_tokens][p][O]
   const void* g;         // [N, S, O]
   const void* r_out;     // [p, O]
   int64_t g_seq_stride, g_tok_stride;
@@ -66,7 +69,8 @@ struct ContractArgs {
 
 constexpr int CONTRACT_OC = 32;  // output features staged per step
 
-// One workgroup per token of the chunk: P_t[i, j] = sum_o L[i, o] g_t[o] H_t[o, j].
+// Generic fallback (any O, any alignment): one workgroup per token of the chunk,
+// P_t[i, j] = sum_o L[i, o] g_t[o] H_t[o, j] on the vector ALUs.
 template <typename T, bool PER_TOKEN>
 __global__ __launch_bounds__(256) void adam_contract_kernel(ContractArgs a) {
   __shared__ float s_lg[CONTRACT_OC][65];  // [o][i]  L[i, o] * g_t[o]
@@ -98,7 +102,7 @@ __global__ __launch_bounds__(256) void adam_contract_kernel(ContractArgs a) {
       for (int e = tid; e < oc * p; e += 256) {
         const int oo = e / p, x = e - oo * p;
         s_lg[oo][x] = Elem<T>::load(L + (int64_t)x * a.O + o0 + oo) * Elem<T>::load(g + o0 + oo);
-        s_h[oo][x] = H[(int64_t)(o0 + oo) * p + x];
+        s_h[oo][x] = H[(int64_t)x * a.O + o0 + oo];
       }
       if (a.bias_col != nullptr && tid < oc) s_bs[tid] = a.bias_scale[o0 + tid];
       __syncthreads();
@@ -139,6 +143,130 @@ __global__ __launch_bounds__(256) void adam_contract_kernel(ContractArgs a) {
       const int e = tid + c * 256;
       if (e < pp) a.ptok[(int64_t)tl * pp + e] = acc[c];
     }
+  }
+}
+
+// The same contraction on the matrix cores.  A wave owns TT tokens of the chunk; per k-step (KS output
+// features) it loads the fragments of L once and, for every token, builds the B operand
+// Z_t[o, j] = g_t[o] * H_t[j][o] in registers (rounded to the model dtype, as the reference's normalised
+// gradient is) and accumulates P_t[16 it .. , 16 jt ..] += L[., o-slice] Z_t[o-slice, .].
+// Needs O % KS == 0 and 16-byte aligned g rows and L; PT = ceil(p / 16).
+template <typename T, bool PER_TOKEN, bool BIAS, int PT, int TT>
+__global__ __launch_bounds__(256) void adam_contract_mfma_kernel(ContractArgs a) {
+  using M = Mma<T>;
+  constexpr int HV = M::EPL / 4;  // 16-byte loads of fp32 values per fragment
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int c = lane & 15;
+  const int q = lane >> 4;
+  const int p = a.p, O = a.O, pp = p * p;
+  const int64_t tl0 = ((int64_t)blockIdx.x * 4 + wave) * TT;  // first chunk-local token of this wave
+  if (tl0 >= a.chunk_tokens) return;
+
+  const T* grow[TT];
+  const float* hrow[TT];
+  bool valid[TT];
+  int64_t out_base[TT];
+#pragma unroll
+  for (int u = 0; u < TT; ++u) {
+    const bool in_chunk = tl0 + u < a.chunk_tokens;
+    const int64_t tl = in_chunk ? tl0 + u : a.chunk_tokens - 1;
+    const int64_t t = a.t0 + tl;
+    const int n = (int)(t / a.S);
+    const int s = (int)(t - (int64_t)n * a.S);
+    valid[u] = in_chunk && (a.lengths == nullptr || s < a.lengths[n] - 1);
+    grow[u] = (const T*)a.g + (int64_t)n * a.g_seq_stride + (int64_t)s * a.g_tok_stride + q * M::EPL;
+    hrow[u] = a.H + tl * (int64_t)O * p + q * M::EPL;
+    out_base[u] = PER_TOKEN ? (a.row_offsets[n] + s) * a.out_row_stride + a.out_col : tl * pp;
+  }
+  const T* lrow[PT];
+  int64_t hcol[PT];
+#pragma unroll
+  for (int t = 0; t < PT; ++t) {
+    const int r = min(t * 16 + c, p - 1);  // rows / columns past p repeat the last one and are not stored
+    lrow[t] = (const T*)a.r_out + (int64_t)r * O + q * M::EPL;
+    hcol[t] = (int64_t)r * O;
+  }
+
+  f32x4 acc[TT][PT][PT];
+  f32x4 accb[BIAS ? TT : 1][PT];
+#pragma unroll
+  for (int u = 0; u < TT; ++u)
+#pragma unroll
+    for (int it = 0; it < PT; ++it) {
+      if (BIAS) accb[u][it] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int jt = 0; jt < PT; ++jt) acc[u][it][jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+  const int nsteps = O / M::KS;
+  for (int ks = 0; ks < nsteps; ++ks) {
+    const int k0 = ks * M::KS;
+    uint4 af[PT];
+#pragma unroll
+    for (int it = 0; it < PT; ++it) af[it] = load16_global(lrow[it] + k0);
+    float bs[M::EPL];
+    if (BIAS) {
+#pragma unroll
+      for (int h = 0; h < HV; ++h) {
+        const uint4 v = load16_global(a.bias_scale + k0 + q * M::EPL + 4 * h);
+        bs[4 * h] = __uint_as_float(v.x);
+        bs[4 * h + 1] = __uint_as_float(v.y);
+        bs[4 * h + 2] = __uint_as_float(v.z);
+        bs[4 * h + 3] = __uint_as_float(v.w);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < TT; ++u) {
+      const uint4 gv = load16_global(grow[u] + k0);
+      if (BIAS) {
+        uint4 bfb = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+        for (int e = 0; e < M::EPL; ++e) M::set(bfb, e, M::get(gv, e) * bs[e]);
+#pragma unroll
+        for (int it = 0; it < PT; ++it) M::mma(af[it], bfb, accb[u][it]);
+      }
+#pragma unroll
+      for (int jt = 0; jt < PT; ++jt) {
+        uint4 bf = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+        for (int h = 0; h < HV; ++h) {
+          const uint4 hv = load16_global(hrow[u] + hcol[jt] + k0 + 4 * h);
+          M::set(bf, 4 * h, M::get(gv, 4 * h) * __uint_as_float(hv.x));
+          M::set(bf, 4 * h + 1, M::get(gv, 4 * h + 1) * __uint_as_float(hv.y));
+          M::set(bf, 4 * h + 2, M::get(gv, 4 * h + 2) * __uint_as_float(hv.z));
+          M::set(bf, 4 * h + 3, M::get(gv, 4 * h + 3) * __uint_as_float(hv.w));
+        }
+#pragma unroll
+        for (int it = 0; it < PT; ++it) M::mma(af[it], bf, acc[u][it][jt]);
+      }
+    }
+  }
+
+  // acc[u][it][jt][e] = P_t[16 it + 4 q + e][16 jt + c]
+#pragma unroll
+  for (int u = 0; u < TT; ++u) {
+    if (tl0 + u >= a.chunk_tokens) continue;
+    if (PER_TOKEN && !valid[u]) continue;
+#pragma unroll
+    for (int it = 0; it < PT; ++it)
+#pragma unroll
+      for (int jt = 0; jt < PT; ++jt) {
+        const int j = jt * 16 + c;
+        const float bc = (BIAS && j < p) ? a.bias_col[j] : 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int i = it * 16 + q * 4 + e;
+          if (i < p && j < p) {
+            float v = acc[u][it][jt][e];
+            if (BIAS) v = fmaf(accb[u][it][e], bc, v);
+            if (PER_TOKEN)
+              store_as(a.out, out_base[u] + i * p + j, clampf(v, a.lo, a.hi), a.out_dtype);
+            else
+              a.ptok[out_base[u] + i * p + j] = valid[u] ? v : 0.f;
+          }
+        }
+      }
   }
 }
 
@@ -276,6 +404,8 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
   for (int64_t t0 = 0; t0 < T; t0 += tc) {
     const int64_t rows_c = T - t0 < tc ? T - t0 : tc;
     const char* a_chunk = (const char*)a + (size_t)t0 * a_tok_stride * esz;
+    // fp32 H: every store instruction of the GEMM epilogue then covers whole 128-byte lines (16-bit
+    // scores made that kernel three times slower)
     const int rc = gemm_scores(a_chunk, rows_c, I, a_tok_stride, dtype, table, O * p, H, st);
     if (rc != 0) return rc;
     ContractArgs c;
@@ -300,20 +430,61 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
     c.ptok = ptok;
     c.bias_col = bias_col;
     c.bias_scale = bias_scale;
-    const dim3 grid((unsigned)rows_c), block(256);
+    const int kstep = dtype == BGX_F32 ? 16 : 32;
+    const int epl = dtype == BGX_F32 ? 4 : 8;
+    const bool mfma_ok = O % kstep == 0 && (uintptr_t)g % 16 == 0 && (uintptr_t)r_out % 16 == 0 &&
+                         g_seq_stride % epl == 0 && g_tok_stride % epl == 0 &&
+                         (bias_scale == nullptr || (uintptr_t)bias_scale % 16 == 0);
+    const bool bias = bias_col != nullptr;
+    const dim3 block(256);
+    if (mfma_ok) {
+      const int pt = p <= 16 ? 1 : (p <= 32 ? 2 : 4);
+      // tokens per wave: L's fragments are shared by them, but a chunk is only a few thousand tokens and
+      // every wave of the chip needs some
+      const int tt = pt == 4 ? 1 : 2;
+      const dim3 grid((unsigned)((rows_c + 4 * tt - 1) / (4 * tt)));
+#define BGX_CONTRACT_M(T_, PT_, TT_)                                                                         \
+  if (per_token && bias)                                                                                     \
+    hipLaunchKernelGGL((adam_contract_mfma_kernel<T_, true, true, PT_, TT_>), grid, block, 0, st, c);       \
+  else if (per_token)                                                                                        \
+    hipLaunchKernelGGL((adam_contract_mfma_kernel<T_, true, false, PT_, TT_>), grid, block, 0, st, c);      \
+  else if (bias)                                                                                             \
+    hipLaunchKernelGGL((adam_contract_mfma_kernel<T_, false, true, PT_, TT_>), grid, block, 0, st, c);      \
+  else                                                                                                       \
+    hipLaunchKernelGGL((adam_contract_mfma_kernel<T_, false, false, PT_, TT_>), grid, block, 0, st, c);
+#define BGX_CONTRACT_P(T_)              \
+  if (pt == 1) {                        \
+    BGX_CONTRACT_M(T_, 1, 2)            \
+  } else if (pt == 2) {                 \
+    BGX_CONTRACT_M(T_, 2, 2)            \
+  } else {                              \
+    BGX_CONTRACT_M(T_, 4, 1)            \
+  }
+      if (dtype == BGX_F32) {
+        BGX_CONTRACT_P(float)
+      } else if (dtype == BGX_F16) {
+        BGX_CONTRACT_P(f16_t)
+      } else {
+        BGX_CONTRACT_P(bf16_t)
+      }
+#undef BGX_CONTRACT_P
+#undef BGX_CONTRACT_M
+    } else {
+      const dim3 grid((unsigned)rows_c);
 #define BGX_CONTRACT(T_)                                                                         \
   if (per_token)                                                                                 \
     hipLaunchKernelGGL((adam_contract_kernel<T_, true>), grid, block, 0, st, c);                 \
   else                                                                                           \
     hipLaunchKernelGGL((adam_contract_kernel<T_, false>), grid, block, 0, st, c);
-    if (dtype == BGX_F32) {
-      BGX_CONTRACT(float)
-    } else if (dtype == BGX_F16) {
-      BGX_CONTRACT(f16_t)
-    } else {
-      BGX_CONTRACT(bf16_t)
-    }
+      if (dtype == BGX_F32) {
+        BGX_CONTRACT(float)
+      } else if (dtype == BGX_F16) {
+        BGX_CONTRACT(f16_t)
+      } else {
+        BGX_CONTRACT(bf16_t)
+      }
 #undef BGX_CONTRACT
+    }
     BGX_HIP(hipGetLastError());
     if (!per_token) {
       const int n_first = (int)(t0 / S);

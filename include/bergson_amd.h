@@ -139,10 +139,10 @@ int bgx_collect_tok(const bgx_module_desc* mods_host, int32_t n_modules,
  * outside the root) and the double-sided projection of collector.py:545-550.
  *
  * bgx_adam_prepare builds, once per module, the table
- *   table[(o*p + j), k] = round_dtype(r_in[j, k] / (sqrt(weight_avg_sq[o, k]) + 1e-8))
+ *   table[(j*O + o), k] = round_dtype(r_in[j, k] / (sqrt(weight_avg_sq[o, k]) + 1e-8))
  * of bgx_adam_table_bytes(O, I, p, dtype) bytes.
  * bgx_collect_adam then computes, for one module of one batch,
- *   P_t[i, j] = sum_o r_out[i, o] g_t[o] * sum_k a_t[k] table[(o*p + j), k]
+ *   P_t[i, j] = sum_o r_out[i, o] g_t[o] * sum_k a_t[k] table[(j*O + o), k]
  * per token t and writes either every valid token's row (per_token != 0:
  * row row_offsets[n] + s, s < lengths[n] - 1) or the sum over each sequence
  * (per_token == 0: row rows[n], or n when rows is NULL), clamped and cast.
