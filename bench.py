@@ -35,8 +35,11 @@ sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes moved per algorithmic byte by collect_kernel on this workload, from the FETCH_SIZE and
-# WRITE_SIZE hardware counters (profiles/collect_kernel_pythia160m_pmc_traffic.txt)
+# WRITE_SIZE hardware counters (profiles/collect_and_scan_kernels_pmc_hbm_traffic.txt)
 COLLECT_TRAFFIC_RATIO = 1.035
+# the same for the store scan: 1024 queries (four query tiles re-read each row tile, half from L2), 32 queries
+SCAN_TRAFFIC_RATIO_Q1024 = 1.51
+SCAN_TRAFFIC_RATIO_Q32 = 1.007
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
@@ -169,7 +172,8 @@ def scan_leg(args, torch, device):
     out = {
         "rows": n, "dim": D, "queries": Q, "k": k, "ms": ms, "rows_per_s": n / (ms * 1e-3),
         "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": MFMA_F16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, "traffic": None},
+                     "unit": "TFLOP/s", "frac": flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
+                     "traffic": n * D * 2 * SCAN_TRAFFIC_RATIO_Q1024},
         "hbm_gbs": n * D * 2 / (ms * 1e-3) / 1e9,
         "top1_mean": float(res.topk_values[:Q, 0].mean().item()),
     }
@@ -186,7 +190,7 @@ def scan_leg(args, torch, device):
     gbs = n * D * 2 / (ms32 * 1e-3) / 1e9
     out["q32"] = {"ms": ms32, "rows_per_s": n / (ms32 * 1e-3),
                   "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                               "frac": gbs / HBM_PEAK_GBS, "traffic": None}}
+                               "frac": gbs / HBM_PEAK_GBS, "traffic": n * D * 2 * SCAN_TRAFFIC_RATIO_Q32}}
     del store
     torch.cuda.empty_cache()
     return out
