@@ -193,6 +193,16 @@ def test_many_tiles_across_modules(device, dtype, per_token):
     assert rel_l2(got, want) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("p", [5, 8, 13])
+def test_seq_small_projection_dims(device, dtype, p):
+    """p < 16: the unused rows / columns of the 16 x 16 MFMA tiles must not leak into the p x p block."""
+    cases = [make_case(3, 150, 96, 160, p, dtype, seed=45 + p, normalizer="adafactor" if p != 8 else None)]
+    got = run_kernel(device, cases, p, dtype)
+    assert got.shape == (3, p * p)
+    assert rel_l2(got, oracle_rows(cases, dtype)) <= TOL[dtype]
+
+
 def test_wide_module_uses_the_tile_kernel(device):
     """I + O too wide for the projection fragments to fit in LDS: the launch falls back to the tile kernel."""
     cases = [make_case(2, 70, 4096, 1024, 16, torch.bfloat16, seed=50, normalizer="adafactor")]
