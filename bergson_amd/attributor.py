@@ -108,11 +108,25 @@ class Attributor:
         qmax = float(q.abs().max().item())
         shift = 0 if qmax == 0 or not math.isfinite(qmax) else -math.frexp(qmax)[1]
         qd = (q * (2.0 ** shift)).to(self.store.dtype)
-        res = ops.scan(self.store, qd, unit_norm=self.unit_norm, k=k, query_scale=2.0 ** (-shift))
-        values = res.topk_values
+        if k <= ops.SCAN_KMAX:
+            res = ops.scan(self.store, qd, unit_norm=self.unit_norm, k=k, query_scale=2.0 ** (-shift))
+            values, indices = res.topk_values, res.topk_indices
+        else:
+            # beyond the fused selection's capacity (k = None asks for a full ranking of the store): the
+            # scan writes every score, in slices of queries so that [n, Q'] fp32 stays near 4 GB, and the
+            # ranking is the library's
+            step = max(1, (1 << 30) // max(1, self.N))
+            vals, idxs = [], []
+            for lo in range(0, qd.shape[0], step):
+                res = ops.scan(self.store, qd[lo:lo + step].contiguous(), unit_norm=self.unit_norm,
+                               query_scale=2.0 ** (-shift), want_scores=True)
+                v, i = torch.topk(res.scores.T, k, dim=1)
+                vals.append(v)
+                idxs.append(i)
+            values, indices = torch.cat(vals), torch.cat(idxs)
         if reverse:
             values = -values
-        return torch.return_types.topk((values.to(self.dtype), res.topk_indices))
+        return torch.return_types.topk((values.to(self.dtype), indices))
 
     @contextmanager
     def trace(self, module: nn.Module, k: int | None, *, modules: set[str] | None = None, reverse: bool = False

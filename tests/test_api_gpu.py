@@ -248,3 +248,29 @@ def test_build_then_score_entry_points(device, tmp_path):
         assert sc.is_written() and sc.num_scores == 3
         got = torch.from_numpy(np.array(sc[:]))
         assert (got - want).abs().max().item() <= 1e-3
+
+
+def test_attributor_full_ranking_beyond_the_fused_top_k(device, tmp_path):
+    """k = None ranks the whole store (attributor.py:229-235 with k = None -> N); past the fused selection's
+    2048 entries the scan writes every score and the ranking is torch.topk's."""
+    from bergson_amd import Attributor, GradientProcessor
+    from bergson_amd.data import create_index
+
+    n, sizes = 2500, {"a": 48, "b": 80}
+    gen = torch.Generator().manual_seed(9)
+    rows = torch.randn(n, 128, generator=gen)
+    path = tmp_path / "big"
+    mm = create_index(path, n, sizes, np.float32)
+    mm[:] = rows.numpy()
+    mm.flush()
+    GradientProcessor(projection_dim=None).save(path)
+    attr = Attributor(path, device="cuda:0", unit_norm=True)
+    q = rows[[7, 1900]]
+    vals, idx = attr.search({"a": q[:, :48].to(device), "b": q[:, 48:].to(device)}, k=None)
+    assert vals.shape == (2, n) and idx.shape == (2, n)
+    index = {"a": rows[:, :48], "b": rows[:, 48:]}
+    ref_v, ref_i = oscan.attributor_search(index, {"a": q[:, :48], "b": q[:, 48:]}, ["a", "b"], n, unit_norm=True)
+    assert idx[:, 0].tolist() == [7, 1900]
+    assert (vals.cpu() - ref_v).abs().max().item() <= 1e-3
+    assert (idx.cpu() == ref_i).float().mean().item() > 0.99  # neighbours closer than the tolerance may swap
+    assert all(sorted(r.tolist()) == list(range(n)) for r in idx.cpu())
