@@ -15,8 +15,11 @@
 // by the tokens of a wave, Z_t formed in registers as the B operand.  H is O*p values per token, which makes
 // the path HBM-heavy for large modules; fusing the contraction into the GEMM is the planned next step.
 
+#include <stdlib.h>
+
 #include "common.hpp"
 #include "mma16.hpp"
+#include "mma32.hpp"
 
 namespace bgx {
 
@@ -270,6 +273,199 @@ __global__ __launch_bounds__(256) void adam_contract_mfma_kernel(ContractArgs a)
   }
 }
 
+// ---- fused path: H never leaves the CU ------------------------------------------------------------
+// Workgroup (token tile of 256, column j of P) walks the output features in chunks of 256:
+//   1. the tile GEMM of the store scan (256 x 256, K = I): acc[t, o] = sum_k a[t, k] * table[(j, o), k],
+//   2. acc goes to LDS in the model dtype (the tile buffers are free by then),
+//   3. second MFMA pass, one wave per 32 tokens: pacc[t, i] += sum_o (acc[t, o] * g[t, o]) * L[i, o], the
+//      A operand read back from LDS and scaled by 16 bytes of the token's g row, the B operand 16 bytes
+//      of L's row i,
+// and finally writes ptok[t][i * p + j].  Needs a 16-bit model dtype, O % 256 == 0, I % 64 == 0,
+// p <= 32, aligned rows, no bias column; everything else takes the two-kernel path above.
+struct FusedArgs {
+  const void* a;  // activations of the chunk, [tokens, I]
+  int64_t a_tok_stride;
+  const void* table;  // [(p * O), I]
+  const void* g;
+  int64_t g_seq_stride, g_tok_stride;
+  const void* r_out;  // [p, O]
+  int64_t t0;         // first flattened token of the chunk
+  int tokens;
+  int S, I, O, p;
+  const int32_t* lengths;
+  float* ptok;  // [tokens][p * p]
+};
+
+constexpr int FUSED_TILE = 256;
+constexpr int FUSED_ZROW = FUSED_TILE * 2 + 16;  // bytes per token row of the staged tile (padded)
+
+template <typename T>
+__global__ __launch_bounds__(512) void adam_fused_kernel(FusedArgs a) {
+  using M = Mma32<T>;
+  static_assert(sizeof(T) == 2, "the fused Adam kernel is for 16-bit model dtypes");
+  constexpr int BM = FUSED_TILE, BN = FUSED_TILE, WN = 4, NT = 512;
+  constexpr int EPL = M::EPL;
+  constexpr int BK = TILE_CHUNKS * EPL;
+  constexpr int WTM = 128, WTN = 64, TM = 4, TN = 2;
+  constexpr int GCH = BM * TILE_CHUNKS / NT, QCH = BN * TILE_CHUNKS / NT;
+  constexpr int ROWS_PER_PASS = NT / TILE_CHUNKS;
+  constexpr int BUF_BYTES = (BM + BN) * LDS_ROW_BYTES;
+  static_assert(BM * FUSED_ZROW <= 2 * BUF_BYTES, "the staged tile reuses the GEMM's LDS buffers");
+  extern __shared__ __align__(16) unsigned char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  const int fr = lane & 31;
+  const int fh = lane >> 5;
+  const int lrow = tid / TILE_CHUNKS;
+  const int lcol = tid % TILE_CHUNKS;
+  const int t_row0 = blockIdx.x * BM;  // chunk-local first token of the tile
+  const int j = blockIdx.y;
+  const int p = a.p, O = a.O, pp = p * p;
+  const int64_t I = a.I;
+  const int rows_here = a.tokens - t_row0;  // valid tokens of this tile (may exceed BM)
+
+  const T* act = (const T*)a.a + (int64_t)t_row0 * a.a_tok_stride;
+  const T* Lmat = (const T*)a.r_out;
+
+  // this lane's token in the second pass and its g row
+  const int my_tl = t_row0 + wave * 32 + fr;
+  const int64_t my_t = a.t0 + (my_tl < a.tokens ? my_tl : a.tokens - 1);
+  const int my_n = (int)(my_t / a.S);
+  const int my_s = (int)(my_t - (int64_t)my_n * a.S);
+  const T* my_g = (const T*)a.g + (int64_t)my_n * a.g_seq_stride + (int64_t)my_s * a.g_tok_stride + fh * EPL;
+  const T* my_l = Lmat + (int64_t)min(fr, p - 1) * O + fh * EPL;
+
+  f32x16 pacc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) pacc[e] = 0.f;
+
+  const int KT = (int)(I / BK);
+  for (int oc = 0; oc < O; oc += BN) {
+    const T* tab = (const T*)a.table + ((int64_t)j * O + oc) * I;
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][jj][e] = 0.f;
+
+    uint4 gr[GCH], qr[QCH];
+    auto gload = [&](int kt) {
+      const int64_t k = (int64_t)kt * BK + lcol * EPL;
+#pragma unroll
+      for (int i = 0; i < GCH; ++i)
+        gr[i] = load_chunk<T, true>(act, lrow + i * ROWS_PER_PASS, rows_here, a.a_tok_stride, k, I);
+#pragma unroll
+      for (int i = 0; i < QCH; ++i) qr[i] = load_chunk<T, true>(tab, lrow + i * ROWS_PER_PASS, BN, I, k, I);
+    };
+    auto lstore = [&](int buf) {
+      unsigned char* base = smem + buf * BUF_BYTES;
+#pragma unroll
+      for (int i = 0; i < GCH; ++i)
+        *reinterpret_cast<uint4*>(base + (lrow + i * ROWS_PER_PASS) * LDS_ROW_BYTES + lcol * 16) = gr[i];
+#pragma unroll
+      for (int i = 0; i < QCH; ++i)
+        *reinterpret_cast<uint4*>(base + (BM + lrow + i * ROWS_PER_PASS) * LDS_ROW_BYTES + lcol * 16) = qr[i];
+    };
+    auto mma_step = [&](const unsigned char* gb, const unsigned char* qb, int kk) {
+      uint4 af[TM], bf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const uint4*>(gb + i * 32 * LDS_ROW_BYTES + kk * 32);
+#pragma unroll
+      for (int jj = 0; jj < TN; ++jj) bf[jj] = *reinterpret_cast<const uint4*>(qb + jj * 32 * LDS_ROW_BYTES + kk * 32);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int jj = 0; jj < TN; ++jj) M::mma(af[i], bf[jj], acc[i][jj]);
+    };
+
+    // same pipeline as the store scan: MFMAs of tile kt from buffer kt&1 while tile kt+1 goes to the
+    // other buffer and the loads of tile kt+2 are in flight; one barrier per tile
+    gload(0);
+    lstore(0);
+    if (KT > 1) gload(1);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+      const int buf = kt & 1;
+      const unsigned char* gb = smem + buf * BUF_BYTES + (wm * WTM + fr) * LDS_ROW_BYTES + fh * 16;
+      const unsigned char* qb = smem + buf * BUF_BYTES + (BM + wn * WTN + fr) * LDS_ROW_BYTES + fh * 16;
+      mma_step(gb, qb, 0);
+      if (kt + 1 < KT) lstore(buf ^ 1);
+      if (kt + 2 < KT) gload(kt + 2);
+#pragma unroll
+      for (int kk = 1; kk < TILE_CHUNKS / 2; ++kk) mma_step(gb, qb, kk);
+      __syncthreads();
+    }
+
+    // acc -> LDS as [token][o] in the model dtype
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int row = wm * WTM + i * 32 + (e >> 2) * 8 + fh * 4 + (e & 3);
+          const int col = wn * WTN + jj * 32 + fr;
+          uint16_t bits;
+          if constexpr (Elem<T>::code == BGX_F16)
+            bits = (uint16_t)f32_to_f16_bits(acc[i][jj][e]);
+          else
+            bits = (uint16_t)f32_to_bf16_bits(acc[i][jj][e]);
+          *reinterpret_cast<uint16_t*>(smem + row * FUSED_ZROW + col * 2) = bits;
+        }
+    __syncthreads();
+
+    // second pass: this wave's 32 tokens x 32 rows of L, K = the chunk's 256 output features
+    const unsigned char* zrow = smem + (wave * 32 + fr) * FUSED_ZROW + fh * 16;
+#pragma unroll 4
+    for (int ks = 0; ks < BN / 16; ++ks) {
+      const uint4 zf = *reinterpret_cast<const uint4*>(zrow + ks * 32);
+      const uint4 gf = load16_global(my_g + oc + ks * 16);
+      const uint4 lf = load16_global(my_l + oc + ks * 16);
+      uint4 af = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) Mma<T>::set(af, e, Mma<T>::get(zf, e) * Mma<T>::get(gf, e));
+      M::mma(af, lf, pacc);
+    }
+    __syncthreads();  // the next chunk's tiles overwrite the staged tile
+  }
+
+  // pacc[e] = P[token (e>>2)*8 + fh*4 + (e&3) of this wave][i = fr], column j
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const int tl = t_row0 + wave * 32 + (e >> 2) * 8 + fh * 4 + (e & 3);
+    if (tl < a.tokens && fr < p) {
+      bool valid = true;
+      if (a.lengths != nullptr) {
+        const int64_t t = a.t0 + tl;
+        const int n = (int)(t / a.S);
+        valid = (int)(t - (int64_t)n * a.S) < a.lengths[n] - 1;
+      }
+      a.ptok[(int64_t)tl * pp + fr * p + j] = valid ? pacc[e] : 0.f;
+    }
+  }
+}
+
+// per-token rows from ptok: clamp, cast, scatter to the rows of the valid tokens
+__global__ __launch_bounds__(256) void adam_tok_finalize_kernel(const float* __restrict__ ptok, int64_t t0, int tokens,
+                                                                int S, int pp, const int32_t* __restrict__ lengths,
+                                                                const int64_t* __restrict__ row_offsets, void* out,
+                                                                int64_t out_row_stride, int64_t out_col, int out_dtype,
+                                                                float lo, float hi) {
+  const int tl = blockIdx.x;
+  const int64_t t = t0 + tl;
+  const int n = (int)(t / S);
+  const int s = (int)(t - (int64_t)n * S);
+  if (s >= lengths[n] - 1) return;
+  const int64_t base = (row_offsets[n] + s) * out_row_stride + out_col;
+  for (int e = threadIdx.x; e < pp; e += blockDim.x)
+    store_as(out, base + e, clampf(ptok[(int64_t)tl * pp + e], lo, hi), out_dtype);
+}
+
 constexpr int SEQ_SLICES = 32;
 
 // part[n - n_first, slice, e] = sum over one slice of the chunk's tokens of sequence n, in token order.
@@ -401,6 +597,68 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
     hipLaunchKernelGGL(adam_zero_kernel, dim3((unsigned)((nacc + 255) / 256)), dim3(256), 0, st, acc, nacc);
     BGX_HIP(hipGetLastError());
   }
+  // ---- fused path ------------------------------------------------------------------------------
+  const bool fused = dtype != BGX_F32 && O % FUSED_TILE == 0 && I % 64 == 0 && p <= 32 && bias_col == nullptr &&
+                     (uintptr_t)a % 16 == 0 && (uintptr_t)g % 16 == 0 && (uintptr_t)r_out % 16 == 0 &&
+                     (uintptr_t)table % 16 == 0 && a_tok_stride % 8 == 0 && g_seq_stride % 8 == 0 &&
+                     g_tok_stride % 8 == 0 && getenv("BGX_ADAM_FUSED_OFF") == nullptr;
+  if (fused) {
+    // no H: the region reserved for it holds the per-token fp32 results, so a chunk can be much larger
+    int64_t fc = (int64_t)((size_t)tc * O * p * 4 / ((size_t)pp * 4));
+    fc = fc / FUSED_TILE * FUSED_TILE;
+    if (fc > T) fc = T;
+    float* ptok_f = (float*)w;
+    constexpr size_t smem = 2 * (size_t)(2 * FUSED_TILE) * LDS_ROW_BYTES;
+    for (int64_t t0 = 0; t0 < T; t0 += fc) {
+      const int64_t rows_c = T - t0 < fc ? T - t0 : fc;
+      FusedArgs f;
+      f.a = (const char*)a + (size_t)t0 * a_tok_stride * esz;
+      f.a_tok_stride = a_tok_stride;
+      f.table = table;
+      f.g = g;
+      f.g_seq_stride = g_seq_stride;
+      f.g_tok_stride = g_tok_stride;
+      f.r_out = r_out;
+      f.t0 = t0;
+      f.tokens = (int)rows_c;
+      f.S = S;
+      f.I = I;
+      f.O = O;
+      f.p = p;
+      f.lengths = lengths;
+      f.ptok = ptok_f;
+      const dim3 grid((unsigned)((rows_c + FUSED_TILE - 1) / FUSED_TILE), (unsigned)p);
+      if (dtype == BGX_F16) {
+        auto kern = adam_fused_kernel<f16_t>;
+        BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        hipLaunchKernelGGL(kern, grid, dim3(512), smem, st, f);
+      } else {
+        auto kern = adam_fused_kernel<bf16_t>;
+        BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        hipLaunchKernelGGL(kern, grid, dim3(512), smem, st, f);
+      }
+      BGX_HIP(hipGetLastError());
+      if (per_token) {
+        hipLaunchKernelGGL(adam_tok_finalize_kernel, dim3((unsigned)rows_c), dim3(256), 0, st, ptok_f, t0, (int)rows_c,
+                           S, pp, lengths, rows, out, out_row_stride, out_col, out_dtype, lo, hi);
+      } else {
+        const int n_first = (int)(t0 / S);
+        const int n_last = (int)((t0 + rows_c - 1) / S);
+        const unsigned nseq = (unsigned)(n_last - n_first + 1);
+        hipLaunchKernelGGL(adam_seq_slice_kernel, dim3(nseq, SEQ_SLICES), dim3(256), 0, st, ptok_f, part, t0,
+                           (int)rows_c, S, pp, n_first);
+        hipLaunchKernelGGL(adam_seq_sum_kernel, dim3(nseq), dim3(256), 0, st, part, acc, pp, n_first);
+      }
+      BGX_HIP(hipGetLastError());
+    }
+    if (!per_token) {
+      hipLaunchKernelGGL(adam_seq_finalize_kernel, dim3((unsigned)N), dim3(256), 0, st, acc, rows, pp, out,
+                         out_row_stride, out_col, out_dtype, lo, hi);
+      BGX_HIP(hipGetLastError());
+    }
+    return 0;
+  }
+
   for (int64_t t0 = 0; t0 < T; t0 += tc) {
     const int64_t rows_c = T - t0 < tc ? T - t0 : tc;
     const char* a_chunk = (const char*)a + (size_t)t0 * a_tok_stride * esz;

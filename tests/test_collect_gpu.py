@@ -506,3 +506,33 @@ def test_adam_seq_with_lengths_and_rows(device):
     got = _run_adam(device, case, p, torch.float32, lengths=lengths, row_offsets=[2, 0, 1], n_rows=4)
     assert rel_l2(got[[2, 0, 1]], want) <= 1e-5
     assert got[3].abs().sum() == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("p", [16, 32])
+@pytest.mark.parametrize("per_token", [False, True])
+def test_adam_fused_path(device, dtype, p, per_token, monkeypatch):
+    """Shapes the fused Adam kernel takes (16-bit, O % 256 == 0, I % 64 == 0, p <= 32): several token tiles,
+    two chunks of output features, ragged lengths; against the oracle and against the two-kernel path."""
+    N, S, I, O = 3, 200, 128, 512
+    lengths = [200, 77, 130]
+    case = _adam_case(N, S, I, O, p, dtype, seed=53)
+    a, g, left, right, norm = case
+    g = g.clone()
+    for n, l in enumerate(lengths):
+        g[n, l - 1:] = 0
+    case = (a, g, left, right, norm)
+    if per_token:
+        mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+        counts = [l - 1 for l in lengths]
+        offs = [sum(counts[:n]) for n in range(N)]
+        want = ohooks.module_gradient(a, g, norm, left, right, attribute_tokens=True, collection_mask=mask)
+        kw = dict(per_token=True, lengths=lengths, row_offsets=offs, n_rows=sum(counts))
+    else:
+        want = ohooks.module_gradient(a, g, norm, left, right)
+        kw = dict(chunk_tokens=256)  # the per-token formulation, summed per sequence
+    got = _run_adam(device, case, p, dtype, **kw)
+    assert rel_l2(got, want) <= TOL[dtype]
+    monkeypatch.setenv("BGX_ADAM_FUSED_OFF", "1")
+    other = _run_adam(device, case, p, dtype, **kw)
+    assert rel_l2(got, other) <= TOL[dtype]
