@@ -347,8 +347,15 @@ def collect_adam(prep: AdamPrepared, a: Tensor, g: Tensor, out: Tensor, *, per_t
     if per_token and (lengths is None or rows is None):
         raise ValueError("per-token collection needs lengths and row offsets")
     if not per_token and chunk_tokens == 0:
-        _collect_adam_seq(prep, a, g, out, lengths, rows, lo, hi)
-        return
+        # Two ways to the per-sequence rows.  Normalising the summed gradient costs ~ N * O * I (bound by the
+        # bytes of the [N, O, I] gradient); summing per-token results costs ~ N * S * p * O * I flops on the
+        # fused kernel.  Measured on Pythia-160m shapes the second wins once sequences are shorter than
+        # about 1500 / p tokens.
+        fused_ok = (a.dtype != torch.float32 and O % 256 == 0 and I % 64 == 0 and prep.p <= 32
+                    and prep.bias_col is None)
+        if not (fused_ok and S * prep.p < 1500):
+            _collect_adam_seq(prep, a, g, out, lengths, rows, lo, hi)
+            return
     nbytes = lib.bgx_collect_adam_workspace_bytes(N, S, O, prep.p, chunk_tokens)
     ws = _workspace(out.device, nbytes, "adam")
     rc = lib.bgx_collect_adam(_ptr(a), _ptr(g), a.stride(0), a.stride(1), g.stride(0), g.stride(1), N, S, I, O, prep.p,

@@ -536,3 +536,12 @@ def test_adam_fused_path(device, dtype, p, per_token, monkeypatch):
     monkeypatch.setenv("BGX_ADAM_FUSED_OFF", "1")
     other = _run_adam(device, case, p, dtype, **kw)
     assert rel_l2(got, other) <= TOL[dtype]
+
+
+def test_adam_seq_many_short_sequences(device):
+    """Many short sequences of a fused-eligible shape: the per-sequence rows come from the per-token kernel."""
+    N, S, I, O, p = 40, 24, 128, 256, 16
+    case = _adam_case(N, S, I, O, p, torch.bfloat16, seed=54)
+    a, g, left, right, norm = case
+    got = _run_adam(device, case, p, torch.bfloat16)
+    assert rel_l2(got, ohooks.module_gradient(a, g, norm, left, right)) <= TOL[torch.bfloat16]
