@@ -341,6 +341,7 @@ struct PersistArgs {
   const int32_t* wg_first;  // [gridDim.x + 1] first item of each workgroup; item = module * tiles_pm + tile
   int tiles_pm;             // tiles per module = N * tiles_per_seq
   int r_steps;              // k-steps of LDS reserved for projection fragments
+  int scratch_bytes;        // LDS between the fragments and the staging rings (exchange / per-token tiles)
 };
 
 template <typename T>
@@ -419,7 +420,152 @@ __device__ inline void project_tokens_lds(const T* __restrict__ xrow0, int64_t t
   for (; ks0 < nsteps; ++ks0) run(ks0, std::integral_constant<int, 1>{});
 }
 
-template <typename T, bool PER_TOKEN, int MTW, int U>
+// The same projection with the token rows streamed through registers and a wave-private LDS slot, so
+// that the global loads are fully coalesced: a load instruction covers 8 token rows x 128 bytes (8 lanes
+// per row) instead of 16 rows x 64 bytes, which is worth ~12 % of bandwidth by itself and -- because whole
+// lines are consumed at once -- allows the non-temporal hint (+13 %, and no write-back of other kernels'
+// dirty lines under this kernel).
+//
+// Unit = 8 rows x 128 bytes = one k-pair (two k-steps) of 8 tokens, written to LDS as it was loaded
+// (lane l -> 16 bytes at l*16: row l/8, slot l%8).  Slot s of row rho of row group rg holds chunk
+// s ^ rho ^ (rg & 1) of the pair, which makes the fragment reads (16 token rows x one chunk per lane
+// group) conflict-free.  Needs K % (2 * KS) == 0.
+//
+// A wave's input is one stream of k-pairs: a of its tile, g of its tile, a of its next tile, ...  The
+// stream is cut into blocks of up to STREAM_Q k-pairs (a block does not cross a segment), and the wave keeps
+// exactly one block ahead in registers: while k-pair j of a block goes to LDS and through the MFMAs,
+// k-pair j of the next block is already being loaded into the registers it leaves.  The loads therefore
+// never drain between the blocks, the segments or the tiles of a workgroup's range.
+constexpr int STREAM_Q = 4;
+
+// A load from memory that nothing writes while the kernel runs, at an address that is the same in every
+// lane: goes through the scalar unit, and so stays out of the vector memory queue (whose in-order
+// completion would otherwise tie a wait for this value to every stream load issued before it).
+template <typename V>
+__device__ inline V load_uniform(const V* p) {
+  static_assert(sizeof(V) % 4 == 0 && alignof(V) >= 4, "dword granularity");
+#if defined(__HIP_DEVICE_COMPILE__)
+  typedef __attribute__((address_space(4))) const uint32_t* const_ptr;
+  const const_ptr src = (const_ptr)(uintptr_t)p;
+  union {
+    V v;
+    uint32_t w[sizeof(V) / 4];
+  } u;
+#pragma unroll
+  for (size_t i = 0; i < sizeof(V) / 4; ++i) u.w[i] = src[i];
+  return u.v;
+#else
+  return *p;  // the host pass only parses device functions
+#endif
+}
+
+__device__ inline int seq_token_limit_uniform(const int32_t* lengths, int n, int S) {
+  return lengths ? min(max(load_uniform(lengths + n) - 1, 0), S) : S;
+}
+
+template <int MTW>
+struct Stream {
+  static constexpr int RG = 2 * MTW;            // row groups of 8 tokens
+  static constexpr int SLOT_BYTES = RG * 1024;  // one k-pair of the wave's tokens
+  static constexpr int NSLOT = 2;
+  static constexpr int BYTES_PER_WAVE = NSLOT * SLOT_BYTES;
+};
+
+// per-lane row pointers of a segment (at its first k-pair)
+template <typename T, int MTW>
+__device__ inline void stream_rows(const T* base, int64_t tok_stride, int rows_valid, int lane,
+                                   const T* (&urow)[2 * MTW]) {
+  const int rho = lane >> 3;
+  const int sig = lane & 7;
+#pragma unroll
+  for (int rg = 0; rg < 2 * MTW; ++rg)
+    urow[rg] = base + (int64_t)min(rg * 8 + rho, rows_valid - 1) * tok_stride + (sig ^ rho ^ (rg & 1)) * Mma<T>::EPL;
+}
+
+// Every block issues exactly STREAM_Q * RG loads, in k-pair order, whatever its length: a k-pair that does
+// not exist is replaced by a repeat of the block's first one, which is never used.  With that the number of
+// loads between the issue of a k-pair and its use is the same on every path through the code, so the
+// wait counts the compiler derives are exact (one that differed between two paths would have to be taken
+// at its worst case, a full drain).  For module widths that are multiples of STREAM_Q k-pairs the only
+// such repeats are at the end of a wave's last tile.
+//
+// loads the first block of a segment (only where nothing ran ahead of it)
+template <typename T, int MTW>
+__device__ inline void stream_prime(const T* const (&urow)[2 * MTW], int nkp, uint4 (&v)[STREAM_Q][2 * MTW]) {
+#pragma unroll
+  for (int j = 0; j < STREAM_Q; ++j) {
+    const int off = j < nkp ? j * 2 * Mma<T>::KS : 0;
+#pragma unroll
+    for (int rg = 0; rg < 2 * MTW; ++rg) v[j][rg] = load16_global_stream(urow[rg] + off);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+// Consumes one segment (nkp k-pairs of the rows `cur`, whose first block is in v) into acc, and loads
+// behind it: the later blocks of the segment, then the first block of the segment `nxt` (nkp_next = 0:
+// nothing follows; nxt must still point at readable rows).
+template <typename T, int MTW>
+__device__ inline void stream_segment(const T* const (&cur)[2 * MTW], int nkp, const T* const (&nxt)[2 * MTW],
+                                      int nkp_next, const uint4* __restrict__ rfrag,
+                                      unsigned char* __restrict__ stage, int lane, uint4 (&v)[STREAM_Q][2 * MTW],
+                                      f32x4 (&acc)[MTW]) {
+  using M = Mma<T>;
+  using St = Stream<MTW>;
+  constexpr int RG = St::RG;
+  constexpr int Q = STREAM_Q;
+  const int r = lane & 15;
+  const int q = lane >> 4;
+  int foff[MTW][2];  // fragment of 16-row block mt, k-step s of the pair, inside a slot
+#pragma unroll
+  for (int mt = 0; mt < MTW; ++mt)
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+      foff[mt][s] = (mt * 2 + (r >> 3)) * 1024 + (r & 7) * 128 + (((s * 4 + q) ^ (r & 7) ^ (r >> 3)) << 4);
+
+  for (int kp0 = 0; kp0 < nkp; kp0 += Q) {
+    const int len = min(Q, nkp - kp0);
+    const bool last = kp0 + Q >= nkp;
+    const int len_next = last ? min(Q, nkp_next) : min(Q, nkp - kp0 - Q);
+    const T* nptr[RG];
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg) nptr[rg] = last ? nxt[rg] : cur[rg] + (kp0 + Q) * 2 * M::KS;
+
+    auto step = [&](auto j_tag, auto full_tag) {
+      constexpr int j = decltype(j_tag)::value;
+      constexpr bool FULL = decltype(full_tag)::value;
+      unsigned char* slot = stage + (j % St::NSLOT) * St::SLOT_BYTES;
+      if (FULL || j < len) {
+#pragma unroll
+        for (int rg = 0; rg < RG; ++rg) *reinterpret_cast<uint4*>(slot + rg * 1024 + lane * 16) = v[j][rg];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      const int off = (FULL || j < len_next) ? j * 2 * M::KS : 0;
+#pragma unroll
+      for (int rg = 0; rg < RG; ++rg) v[j][rg] = load16_global_stream(nptr[rg] + off);
+      __builtin_amdgcn_sched_barrier(0);
+      if (FULL || j < len) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+          const uint4 rf = rfrag[((kp0 + j) * 2 + s) * WAVE + lane];
+#pragma unroll
+          for (int mt = 0; mt < MTW; ++mt) {
+            const uint4 xf = *reinterpret_cast<const uint4*>(slot + foff[mt][s]);
+            M::mma(xf, rf, acc[mt]);
+          }
+        }
+      }
+    };
+    // one code path for full and partial blocks: a second, unguarded copy of the steps would meet this one
+    // at a join, where the queue registers of the two have to be reconciled by moves that wait for the loads
+    step(std::integral_constant<int, 0>{}, std::false_type{});
+    step(std::integral_constant<int, 1>{}, std::false_type{});
+    step(std::integral_constant<int, 2>{}, std::false_type{});
+    step(std::integral_constant<int, 3>{}, std::false_type{});
+  }
+}
+static_assert(STREAM_Q == 4, "stream_segment spells out its four steps");
+
+template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED = false>
 __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(PersistArgs pa) {
   using M = Mma<T>;
   constexpr int WAVE_T = 16 * MTW;      // tokens per wave
@@ -435,33 +581,42 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
   const CollectArgs& args = pa.c;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  unsigned char* stage = scratch + pa.scratch_bytes + wave * Stream<MTW>::BYTES_PER_WAVE;  // STAGED only
   const int c = lane & 15;
   const int q = lane >> 4;
   const int p = args.p;
   const int pp = p * p;
-  const int item0 = pa.wg_first[blockIdx.x];
-  const int item1 = pa.wg_first[blockIdx.x + 1];
+  const int item0 = load_uniform(pa.wg_first + blockIdx.x);
+  const int item1 = load_uniform(pa.wg_first + blockIdx.x + 1);
 
   int cur_m = -1;
   int parity = 0;
+  // STAGED: the register queue of the wave's input stream, and whether it holds the first block of the
+  // tile that comes next
+  uint4 v[STAGED ? STREAM_Q : 1][2 * MTW];
+  bool primed = false;
   for (int item = item0; item < item1; ++item) {
     const int m = item / pa.tiles_pm;
     const int tile = item - m * pa.tiles_pm;
     const int n = tile / args.tiles_per_seq;
     const int ts = tile - n * args.tiles_per_seq;
     const int s0 = ts * TILE_T;
-    const int s_limit = seq_token_limit(args.lengths, n, args.S);
-    if (s0 >= s_limit) continue;  // whole tile is padding (uniform over the workgroup)
+    const int s_limit = seq_token_limit_uniform(args.lengths, n, args.S);
+    if (s0 >= s_limit) continue;  // whole tile is padding (uniform over the workgroup); nothing ran ahead into it
     const int rows_valid = min(WAVE_T, s_limit - s0 - wave * WAVE_T);  // of this wave; may be <= 0
 
-    const bgx_module_desc d = args.mods[m];  // uniform
+    const bgx_module_desc d = load_uniform(args.mods + m);
     const int nA = d.I / M::KS;
     if (m != cur_m) {
       __syncthreads();  // every wave has finished reading the previous module's fragments
       stage_projection<T>((const T*)d.r_in, d.col_scale, d.I, p, rfrag, tid);
       stage_projection<T>((const T*)d.r_out, d.row_scale, d.O, p, rfrag + (size_t)nA * WAVE, tid);
       cur_m = m;
+      // Staging has waited for its own loads, but not on every path the compiler sees (its guarded batches):
+      // without this explicit "no vector load outstanding", the tile code below would have to assume
+      // that staging loads may still be pending behind the stream's and wait for everything.
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), nothing else
       __syncthreads();
     }
 
@@ -476,14 +631,49 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
       const int64_t t0 = s0 + wave * WAVE_T;
       const T* a0 = (const T*)d.a + (int64_t)n * d.a_seq_stride + t0 * d.a_tok_stride;
       const T* g0 = (const T*)d.g + (int64_t)n * d.g_seq_stride + t0 * d.g_tok_stride;
-      project_tokens_lds<T, MTW, U>(a0, d.a_tok_stride, rows_valid, d.I, rfrag, lane, accA);
-      project_tokens_lds<T, MTW, U>(g0, d.g_tok_stride, rows_valid, d.O, rfrag + (size_t)nA * WAVE, lane, accG);
+      if constexpr (STAGED) {
+        constexpr int RG = 2 * MTW;
+        const int nkpA = d.I / (2 * M::KS), nkpG = d.O / (2 * M::KS);
+        const T* ua[RG];
+        const T* ug[RG];
+        const T* un[RG];
+        stream_rows<T, MTW>(a0, d.a_tok_stride, rows_valid, lane, ua);
+        stream_rows<T, MTW>(g0, d.g_tok_stride, rows_valid, lane, ug);
+        if (!primed) stream_prime<T, MTW>(ua, nkpA, v);
+        stream_segment<T, MTW>(ua, nkpA, ug, nkpG, rfrag, stage, lane, v, accA);
+        // what follows g: the a rows of the next tile of the range, where this wave has tokens in it
+        int nkpN = 0;
+#pragma unroll
+        for (int rg = 0; rg < RG; ++rg) un[rg] = ug[rg];
+        if (item + 1 < item1) {
+          const int m2 = (item + 1) / pa.tiles_pm;
+          const int tile2 = item + 1 - m2 * pa.tiles_pm;
+          const int n2 = tile2 / args.tiles_per_seq;
+          const int s02 = (tile2 - n2 * args.tiles_per_seq) * TILE_T;
+          const int rows2 = min(WAVE_T, seq_token_limit_uniform(args.lengths, n2, args.S) - s02 - wave * WAVE_T);
+          if (rows2 > 0) {  // implies that the tile is not all padding
+            const bgx_module_desc* d2 = args.mods + m2;
+            const int64_t stride2 = load_uniform(&d2->a_tok_stride);
+            const T* a2 = (const T*)load_uniform(&d2->a) + (int64_t)n2 * load_uniform(&d2->a_seq_stride) +
+                          (int64_t)(s02 + wave * WAVE_T) * stride2;
+            stream_rows<T, MTW>(a2, stride2, rows2, lane, un);
+            nkpN = load_uniform(&d2->I) / (2 * M::KS);
+          }
+        }
+        stream_segment<T, MTW>(ug, nkpG, un, nkpN, rfrag + (size_t)nA * WAVE, stage, lane, v, accG);
+        primed = nkpN > 0;
+      } else {
+        project_tokens_lds<T, MTW, U>(a0, d.a_tok_stride, rows_valid, d.I, rfrag, lane, accA);
+        project_tokens_lds<T, MTW, U>(g0, d.g_tok_stride, rows_valid, d.O, rfrag + (size_t)nA * WAVE, lane, accG);
+      }
       // token rows past the last valid one hold garbage: zero them in g' (that removes their products)
 #pragma unroll
       for (int mt = 0; mt < MTW; ++mt)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
           if (mt * 16 + q * 4 + i >= rows_valid) accG[mt][i] = 0.f;
+    } else {
+      primed = false;
     }
 
     if constexpr (!PER_TOKEN) {
@@ -721,9 +911,9 @@ static int compute_units(int* out) {
   return 0;
 }
 
-template <typename T, bool PER_TOKEN, int MTW, int U>
+template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED>
 static int launch_persist_one(int wgs, size_t lds, hipStream_t st, const PersistArgs& pa) {
-  auto kern = collect_persist_kernel<T, PER_TOKEN, MTW, U>;
+  auto kern = collect_persist_kernel<T, PER_TOKEN, MTW, U, STAGED>;
   // the opt-in to more than 64 KB of dynamic LDS is per kernel and per device; do it once for each
   static std::atomic<bool> opted_in[MAX_DEVICES];
   int dev = 0;
@@ -736,14 +926,21 @@ static int launch_persist_one(int wgs, size_t lds, hipStream_t st, const Persist
   return 0;
 }
 
-template <typename T>
-static int launch_persist(bool per_token, int tile_tokens, int wgs, size_t lds, hipStream_t st,
-                          const PersistArgs& pa) {
+template <typename T, bool STAGED>
+static int launch_persist_s(bool per_token, int tile_tokens, int wgs, size_t lds, hipStream_t st,
+                            const PersistArgs& pa) {
   if (tile_tokens == 128)
-    return per_token ? launch_persist_one<T, true, 2, 4>(wgs, lds, st, pa)
-                     : launch_persist_one<T, false, 2, 4>(wgs, lds, st, pa);
-  return per_token ? launch_persist_one<T, true, 1, 8>(wgs, lds, st, pa)
-                   : launch_persist_one<T, false, 1, 8>(wgs, lds, st, pa);
+    return per_token ? launch_persist_one<T, true, 2, 4, STAGED>(wgs, lds, st, pa)
+                     : launch_persist_one<T, false, 2, 4, STAGED>(wgs, lds, st, pa);
+  return per_token ? launch_persist_one<T, true, 1, 8, STAGED>(wgs, lds, st, pa)
+                   : launch_persist_one<T, false, 1, 8, STAGED>(wgs, lds, st, pa);
+}
+
+template <typename T>
+static int launch_persist(bool staged, bool per_token, int tile_tokens, int wgs, size_t lds, hipStream_t st,
+                          const PersistArgs& pa) {
+  return staged ? launch_persist_s<T, true>(per_token, tile_tokens, wgs, lds, st, pa)
+                : launch_persist_s<T, false>(per_token, tile_tokens, wgs, lds, st, pa);
 }
 
 // LDS beside the projection fragments: the larger of the P exchange buffers and the per-token a', g' tiles
@@ -819,9 +1016,17 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   // fit in LDS beside its exchange buffers.
   int r_steps = 0;
   for (int m = 0; m < n_modules; ++m) r_steps = std::max(r_steps, (sorted[m].I + sorted[m].O) / kstep);
-  const size_t persist_lds = (size_t)r_steps * 1024 + persist_scratch_bytes(tile_tokens);
+  const size_t scratch_bytes = per_token ? persist_scratch_bytes(tile_tokens) : (size_t)2 * 3 * WAVE * 16;
+  size_t persist_lds = (size_t)r_steps * 1024 + scratch_bytes;
   bool persist = pb == 1 && aligned && !any_bias && persist_lds <= LDS_PER_WG &&
                  tiles * n_modules <= 0x7fffffffLL;
+  // staging rings for fully coalesced loads: every K a multiple of two k-steps, and 32 KB more of LDS
+  const size_t stage_bytes = (size_t)4 * (tile_tokens == 128 ? Stream<2>::BYTES_PER_WAVE : Stream<1>::BYTES_PER_WAVE);
+  bool staged = persist && persist_lds + stage_bytes <= LDS_PER_WG;
+  for (int m = 0; m < n_modules && staged; ++m)
+    staged = sorted[m].I % (2 * kstep) == 0 && sorted[m].O % (2 * kstep) == 0;
+  if (const char* e = getenv("BGX_COLLECT_STAGED")) staged = staged && e[0] != '0';
+  if (staged) persist_lds += stage_bytes;
   // BGX_COLLECT_PERSIST=0 in the environment forces the one-workgroup-per-tile kernel (tests, comparisons)
   if (const char* e = getenv("BGX_COLLECT_PERSIST")) persist = persist && e[0] != '0';
 
@@ -875,13 +1080,14 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     pa.wg_first = (const int32_t*)((const char*)ws + (size_t)n_modules * sizeof(bgx_module_desc));
     pa.tiles_pm = (int)tiles;
     pa.r_steps = r_steps;
+    pa.scratch_bytes = (int)scratch_bytes;
     int rc;
     if (in_dtype == BGX_F32)
-      rc = launch_persist<float>(per_token, tile_tokens, wgs, persist_lds, st, pa);
+      rc = launch_persist<float>(staged, per_token, tile_tokens, wgs, persist_lds, st, pa);
     else if (in_dtype == BGX_F16)
-      rc = launch_persist<f16_t>(per_token, tile_tokens, wgs, persist_lds, st, pa);
+      rc = launch_persist<f16_t>(staged, per_token, tile_tokens, wgs, persist_lds, st, pa);
     else
-      rc = launch_persist<bf16_t>(per_token, tile_tokens, wgs, persist_lds, st, pa);
+      rc = launch_persist<bf16_t>(staged, per_token, tile_tokens, wgs, persist_lds, st, pa);
     if (rc != 0) return rc;
   } else if (in_dtype == BGX_F32) {
     launch_collect_pb<float>(pb, aligned, per_token, any_bias, tile_tokens, grid, st, args);

@@ -47,6 +47,17 @@ constexpr int WAVE = 64;
 // 16-byte load from device memory.  Pointers that come out of a descriptor table carry no address
 // space, and the compiler then falls back to generic ("flat") loads, which it cannot keep in flight
 // next to LDS traffic; this tells it the pointer is a plain global one.
+// The same with the non-temporal hint, for data that is read exactly once: it does not displace what the
+// caches hold, so the dirty lines earlier kernels left behind are not written back under this kernel.
+// Only for access patterns in which one load instruction consumes whole 128-byte lines -- a line that is
+// not retained is fetched again by the next instruction that touches its other half.
+__device__ inline uint4 load16_global_stream(const void* p) {
+  typedef uint32_t raw4 __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(1))) const raw4* global_ptr;
+  const raw4 v = __builtin_nontemporal_load((global_ptr)(uintptr_t)p);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 __device__ inline uint4 load16_global(const void* p) {
   typedef uint32_t raw4 __attribute__((ext_vector_type(4)));
   typedef __attribute__((address_space(1))) const raw4* global_ptr;
