@@ -608,6 +608,19 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
 
     const bgx_module_desc d = load_uniform(args.mods + m);
     const int nA = d.I / M::KS;
+    const int64_t t0 = s0 + wave * WAVE_T;
+    const T* a0 = (const T*)d.a + (int64_t)n * d.a_seq_stride + t0 * d.a_tok_stride;
+    const T* g0 = (const T*)d.g + (int64_t)n * d.g_seq_stride + t0 * d.g_tok_stride;
+    if constexpr (STAGED) {
+      // a tile nothing ran ahead into (the first of the range, or after padding): its first loads go out
+      // before the projections are staged
+      if (rows_valid > 0 && !primed) {
+        const T* ua[2 * MTW];
+        stream_rows<T, MTW>(a0, d.a_tok_stride, rows_valid, lane, ua);
+        stream_prime<T, MTW>(ua, d.I / (2 * M::KS), v);
+        primed = true;
+      }
+    }
     if (m != cur_m) {
       __syncthreads();  // every wave has finished reading the previous module's fragments
       stage_projection<T>((const T*)d.r_in, d.col_scale, d.I, p, rfrag, tid);
@@ -628,9 +641,6 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
       accG[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     if (rows_valid > 0) {
-      const int64_t t0 = s0 + wave * WAVE_T;
-      const T* a0 = (const T*)d.a + (int64_t)n * d.a_seq_stride + t0 * d.a_tok_stride;
-      const T* g0 = (const T*)d.g + (int64_t)n * d.g_seq_stride + t0 * d.g_tok_stride;
       if constexpr (STAGED) {
         constexpr int RG = 2 * MTW;
         const int nkpA = d.I / (2 * M::KS), nkpG = d.O / (2 * M::KS);
@@ -639,7 +649,6 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
         const T* un[RG];
         stream_rows<T, MTW>(a0, d.a_tok_stride, rows_valid, lane, ua);
         stream_rows<T, MTW>(g0, d.g_tok_stride, rows_valid, lane, ug);
-        if (!primed) stream_prime<T, MTW>(ua, nkpA, v);
         stream_segment<T, MTW>(ua, nkpA, ug, nkpG, rfrag, stage, lane, v, accA);
         // what follows g: the a rows of the next tile of the range, where this wave has tokens in it
         int nkpN = 0;
@@ -1039,24 +1048,52 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     if (rc_cus != 0) return rc_cus;
     const int64_t items = tiles * n_modules;
     wgs = (int)std::min<int64_t>(std::min(std::max(cus, 1), PERSIST_MAX_WGS), items);
-    // equal-weight contiguous ranges; an item costs its k-steps plus a constant for the token reduction
+    // Contiguous ranges with the smallest possible maximum cost.  An item costs its k-steps plus a constant
+    // for the token reduction; a range also pays for staging the projections of every module it touches
+    // (16 rows against the tile's tokens, counted twice because those loads come in dependent rounds).
     std::vector<int32_t> first((size_t)wgs + 1, (int32_t)items);
-    first[0] = 0;
     constexpr int REDUCE_STEPS = 2;
-    double total = 0.0;
-    for (int m = 0; m < n_modules; ++m)
-      total += (double)tiles * ((sorted[m].I + sorted[m].O) / kstep + REDUCE_STEPS);
-    double cum = 0.0;
-    int g = 0;
-    int64_t item = 0;
-    for (int m = 0; m < n_modules && g + 1 < wgs; ++m) {
-      const double w = (sorted[m].I + sorted[m].O) / kstep + REDUCE_STEPS;
-      for (int64_t t = 0; t < tiles && g + 1 < wgs; ++t) {
-        cum += w;
-        ++item;
-        while (g + 1 < wgs && cum >= total * (double)(g + 1) / (double)wgs) first[++g] = (int32_t)item;
-      }
+    std::vector<double> w(n_modules), sw(n_modules);
+    double total = 0.0, biggest = 0.0;
+    for (int m = 0; m < n_modules; ++m) {
+      const double ks = (double)((sorted[m].I + sorted[m].O) / kstep);
+      w[m] = ks + REDUCE_STEPS;
+      sw[m] = ks * 32.0 / (double)tile_tokens;
+      total += (double)tiles * w[m] + sw[m];
+      biggest = std::max(biggest, w[m] + sw[m]);
     }
+    // ranges filled in order up to `limit`: how many are needed (bounds != nullptr: also where they start)
+    auto fill = [&](double limit, int32_t* bounds) {
+      int64_t parts = 1;
+      double load = 0.0;
+      int staged_m = -1;
+      for (int m = 0; m < n_modules; ++m) {
+        int64_t left = tiles;
+        while (left > 0) {
+          const double extra = staged_m == m ? 0.0 : sw[m];
+          const int64_t fit = (int64_t)std::floor((limit - load - extra) / w[m] + 1e-9);
+          if (fit <= 0) {  // load > 0 here, since limit >= biggest
+            if (bounds && parts < wgs) bounds[parts] = (int32_t)((int64_t)m * tiles + (tiles - left));
+            ++parts;
+            load = 0.0;
+            staged_m = -1;
+            continue;
+          }
+          const int64_t take = std::min(fit, left);
+          load += extra + (double)take * w[m];
+          staged_m = m;
+          left -= take;
+        }
+      }
+      return parts;
+    };
+    double lo_l = std::max(biggest, total / (double)wgs), hi_l = total + biggest;
+    for (int it = 0; it < 48 && hi_l - lo_l > 1e-3 * lo_l; ++it) {
+      const double mid = 0.5 * (lo_l + hi_l);
+      if (fill(mid, nullptr) <= wgs) hi_l = mid; else lo_l = mid;
+    }
+    first[0] = 0;
+    fill(hi_l, first.data());
     first[wgs] = (int32_t)items;
     const size_t off = head.size();
     head.resize(off + first.size() * sizeof(int32_t));

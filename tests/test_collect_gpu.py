@@ -12,14 +12,17 @@ from oracle.projection import module_projections
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=["persistent", "grid"], autouse=True)
+@pytest.fixture(params=["streamed", "persistent", "grid"], autouse=True)
 def kernel_variant(request, monkeypatch):
-    """Every case runs twice: with the persistent collection kernel where it applies (the default), and with
-    the one-workgroup-per-tile kernel forced through the library's environment switch."""
+    """Every case runs three times: with the persistent collection kernel and its streamed loads where they
+    apply (the default), with the persistent kernel's direct fragment loads, and with the
+    one-workgroup-per-tile kernel, the latter two forced through the library's environment switches."""
+    monkeypatch.delenv("BGX_COLLECT_PERSIST", raising=False)
+    monkeypatch.delenv("BGX_COLLECT_STAGED", raising=False)
     if request.param == "grid":
         monkeypatch.setenv("BGX_COLLECT_PERSIST", "0")
-    else:
-        monkeypatch.delenv("BGX_COLLECT_PERSIST", raising=False)
+    elif request.param == "persistent":
+        monkeypatch.setenv("BGX_COLLECT_STAGED", "0")
     return request.param
 
 
@@ -178,6 +181,38 @@ def test_many_tiles_across_modules(device, dtype, per_token):
                                             name=f"layers.{i}.z")
         for n, l in enumerate(lengths):
             g[n, l - 1:] = 0
+        cases.append((a, g, left, right, norm))
+    if not per_token:
+        got = run_kernel(device, cases, p, dtype, lengths=lengths)
+        want = oracle_rows(cases, dtype)
+    else:
+        counts = [l - 1 for l in lengths]
+        row_offsets = [sum(counts[:n]) for n in range(N)]
+        mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+        got = run_kernel(device, cases, p, dtype, lengths=lengths, per_token=True, row_offsets=row_offsets,
+                         n_rows=sum(counts))
+        want = oracle_rows(cases, dtype, attribute_tokens=True, collection_mask=mask)
+    assert got.shape == want.shape
+    assert rel_l2(got, want) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("per_token", [False, True])
+def test_long_item_ranges_with_odd_widths(device, dtype, per_token):
+    """Several tiles per workgroup, module widths that are odd multiples of the streamed kernel's 128-byte
+    unit (so the last block of a segment is partial), sequences shorter than a tile (waves without tokens),
+    all-padding tiles in the middle of a range: the input stream runs ahead across all of these."""
+    N, S, p = 6, 1536, 16
+    lengths = [1536, 1, 700, 1409, 130, 1025]
+    unit = 64 if dtype == torch.bfloat16 else 32
+    shapes = [(5 * unit, 7 * unit), (unit, 9 * unit), (3 * unit, unit), (6 * unit, 2 * unit), (4 * unit, 11 * unit),
+              (13 * unit, 5 * unit), (unit, unit), (10 * unit, 3 * unit)]
+    cases = []
+    for i, (I, O) in enumerate(shapes):
+        a, g, left, right, norm = make_case(N, S, I, O, p, dtype, seed=140 + i, normalizer="adafactor" if i % 3 else None,
+                                            name=f"layers.{i}.w")
+        for n, l in enumerate(lengths):
+            g[n, max(l - 1, 0):] = 0
         cases.append((a, g, left, right, norm))
     if not per_token:
         got = run_kernel(device, cases, p, dtype, lengths=lengths)
