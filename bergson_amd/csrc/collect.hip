@@ -342,6 +342,7 @@ struct PersistArgs {
   int tiles_pm;             // tiles per module = N * tiles_per_seq
   int r_steps;              // k-steps of LDS reserved for projection fragments
   int scratch_bytes;        // LDS between the fragments and the staging rings (exchange / per-token tiles)
+  int out_vec8;             // per-token rows: every p x p block starts 16-byte aligned and p is 8 or 16
 };
 
 template <typename T>
@@ -467,7 +468,7 @@ template <int MTW>
 struct Stream {
   static constexpr int RG = 2 * MTW;            // row groups of 8 tokens
   static constexpr int SLOT_BYTES = RG * 1024;  // one k-pair of the wave's tokens
-  static constexpr int NSLOT = 2;
+  static constexpr int NSLOT = 1;
   static constexpr int BYTES_PER_WAVE = NSLOT * SLOT_BYTES;
 };
 
@@ -570,7 +571,7 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
   using M = Mma<T>;
   constexpr int WAVE_T = 16 * MTW;      // tokens per wave
   constexpr int TILE_T = 4 * WAVE_T;    // tokens per workgroup
-  constexpr int LDP = 17;
+  constexpr int LDP = 20;  // row of a' or g' in LDS: 16 floats, padded so that rows stay 16-byte aligned
   extern __shared__ __align__(16) unsigned char smem_raw[];
   uint4* rfrag = reinterpret_cast<uint4*>(smem_raw);
   unsigned char* scratch = smem_raw + (size_t)pa.r_steps * WAVE * 16;
@@ -705,7 +706,9 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
       }
       parity ^= 1;  // the next tile writes the other buffer, so one barrier per tile is enough
     } else {
-      __syncthreads();  // the previous tile's readers are done with tok
+      // tok[wave] is private to the wave, and a wave's LDS operations complete in order: no workgroup
+      // barrier, only the compiler must keep the writes, the reads and the next tile's writes in order
+      __builtin_amdgcn_wave_barrier();
 #pragma unroll
       for (int mt = 0; mt < MTW; ++mt)
 #pragma unroll
@@ -713,8 +716,36 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
           tok[wave][0][mt * 16 + q * 4 + i][c] = accA[mt][i];
           tok[wave][1][mt * 16 + q * 4 + i][c] = accG[mt][i];
         }
-      __syncthreads();
-      const int64_t row0 = args.row_offsets[n] + s0 + wave * WAVE_T;
+      __builtin_amdgcn_wave_barrier();
+      const int64_t row0 = load_uniform(args.row_offsets + n) + s0 + wave * WAVE_T;
+      if (pa.out_vec8) {
+        // a lane writes 8 consecutive columns of one row i of one token's block: 16 bytes in a 16-bit store
+        const int jg = p >> 3;                // 8-column groups per block row: 1 or 2
+        const int lt = p == 16 ? 5 : 3;       // log2 of the p * jg lane tasks per token
+        auto write_rows = [&](auto dt_tag) {  // one copy of the loop per output dtype, chosen outside it
+          constexpr int DT = decltype(dt_tag)::value;
+          for (int x = lane; x < (rows_valid << lt); x += WAVE) {
+            const int t = x >> lt;
+            const int rem = x & ((1 << lt) - 1);
+            const int i = rem >> (jg - 1);
+            const int j0 = (rem & (jg - 1)) << 3;
+            const float gv = tok[wave][1][t][i];
+            const float4 a_lo = *reinterpret_cast<const float4*>(&tok[wave][0][t][j0]);
+            const float4 a_hi = *reinterpret_cast<const float4*>(&tok[wave][0][t][j0 + 4]);
+            const float o[8] = {clampf(gv * a_lo.x, args.lo, args.hi), clampf(gv * a_lo.y, args.lo, args.hi),
+                                clampf(gv * a_lo.z, args.lo, args.hi), clampf(gv * a_lo.w, args.lo, args.hi),
+                                clampf(gv * a_hi.x, args.lo, args.hi), clampf(gv * a_hi.y, args.lo, args.hi),
+                                clampf(gv * a_hi.z, args.lo, args.hi), clampf(gv * a_hi.w, args.lo, args.hi)};
+            store8_as<DT>(args.out, (row0 + t) * args.out_row_stride + d.out_col + i * p + j0, o);
+          }
+        };
+        if (args.out_dtype == BGX_F32)
+          write_rows(std::integral_constant<int, BGX_F32>{});
+        else if (args.out_dtype == BGX_F16)
+          write_rows(std::integral_constant<int, BGX_F16>{});
+        else
+          write_rows(std::integral_constant<int, BGX_BF16>{});
+      } else
       for (int t = 0; t < rows_valid; ++t) {
         const int64_t base = (row0 + t) * args.out_row_stride + d.out_col;
         for (int e = lane; e < pp; e += WAVE) {
@@ -954,7 +985,7 @@ static int launch_persist(bool staged, bool per_token, int tile_tokens, int wgs,
 
 // LDS beside the projection fragments: the larger of the P exchange buffers and the per-token a', g' tiles
 static size_t persist_scratch_bytes(int tile_tokens) {
-  return std::max((size_t)2 * 3 * WAVE * 16, (size_t)2 * tile_tokens * 17 * sizeof(float));
+  return std::max((size_t)2 * 3 * WAVE * 16, (size_t)2 * tile_tokens * 20 * sizeof(float));
 }
 
 int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules, int N, int S,
@@ -1118,6 +1149,10 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     pa.tiles_pm = (int)tiles;
     pa.r_steps = r_steps;
     pa.scratch_bytes = (int)scratch_bytes;
+    const int64_t out_elem = out_dtype == BGX_F32 ? 4 : 2;
+    bool vec8 = per_token && (p == 8 || p == 16) && (uintptr_t)out % 16 == 0 && (out_row_stride * out_elem) % 16 == 0;
+    for (int m = 0; m < n_modules && vec8; ++m) vec8 = (sorted[m].out_col * out_elem) % 16 == 0;
+    pa.out_vec8 = vec8 ? 1 : 0;
     int rc;
     if (in_dtype == BGX_F32)
       rc = launch_persist<float>(staged, per_token, tile_tokens, wgs, persist_lds, st, pa);

@@ -136,6 +136,27 @@ __device__ inline void store_as(void* base, int64_t idx, float v, int dt) {
   }
 }
 
+// eight consecutive values at once; base + idx must be 16-byte aligned in the output dtype DT
+template <int DT>
+__device__ inline void store8_as(void* base, int64_t idx, const float (&v)[8]) {
+  if constexpr (DT == BGX_F32) {
+    typedef float raw4 __attribute__((ext_vector_type(4)));
+    raw4* dst = reinterpret_cast<raw4*>((float*)base + idx);
+    __builtin_nontemporal_store(raw4{v[0], v[1], v[2], v[3]}, dst);
+    __builtin_nontemporal_store(raw4{v[4], v[5], v[6], v[7]}, dst + 1);
+  } else {
+    uint32_t w[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t lo = DT == BGX_F16 ? f32_to_f16_bits(v[2 * k]) : f32_to_bf16_bits(v[2 * k]);
+      const uint32_t hi = DT == BGX_F16 ? f32_to_f16_bits(v[2 * k + 1]) : f32_to_bf16_bits(v[2 * k + 1]);
+      w[k] = (lo & 0xffffu) | (hi << 16);
+    }
+    typedef uint32_t raw4 __attribute__((ext_vector_type(4)));
+    __builtin_nontemporal_store(raw4{w[0], w[1], w[2], w[3]}, reinterpret_cast<raw4*>((uint16_t*)base + idx));
+  }
+}
+
 __device__ inline float load_as(const void* base, int64_t idx, int dt) {
   if (dt == BGX_F32) return ((const float*)base)[idx];
   if (dt == BGX_F16) return f16_bits_to_f32(((const uint16_t*)base)[idx]);
