@@ -36,7 +36,7 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBS = 8000.0
 # HBM bytes moved per algorithmic byte by collect_kernel on this workload, from the FETCH_SIZE and
 # WRITE_SIZE hardware counters (profiles/collect_and_scan_kernels_pmc_hbm_traffic.txt)
-COLLECT_TRAFFIC_RATIO = 1.035
+COLLECT_TRAFFIC_RATIO = 1.036
 # the same for the store scan: 1024 queries (four query tiles re-read each row tile, half from L2), 32 queries
 SCAN_TRAFFIC_RATIO_Q1024 = 1.51
 SCAN_TRAFFIC_RATIO_Q32 = 1.007
@@ -274,13 +274,13 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "bgx::collect_persist_kernel<bf16_t, false, 2, 4> and <bf16_t, false, 1, 8> (128- and 64-token tiles)",
+            "kernel": "bgx::collect_persist_kernel<bf16_t, false, 2, 4, true> and <bf16_t, false, 1, 8, true> (128- and 64-token tiles, streamed loads)",
             "achieved": coll["achieved_gbs"],
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": coll["achieved_gbs"] / HBM_PEAK_GBS,
             "traffic": coll["kernel_bytes_per_launch"] * COLLECT_TRAFFIC_RATIO,
-            "traffic_source": "bytes_per_launch x 1.035 (rocprofv3 FETCH_SIZE + WRITE_SIZE, profiles/)",
+            "traffic_source": "bytes_per_launch x 1.036 (rocprofv3 FETCH_SIZE + WRITE_SIZE, profiles/)",
             "bytes_per_launch": coll["kernel_bytes_per_launch"],
             "ms_per_launch": coll["kernel_ms_per_launch"],
             "ms_per_launch_with_descriptor_copy_and_finalize": coll["bracket_ms_per_launch"],
