@@ -9,7 +9,7 @@ from .build import build, create_processor
 from .builder import Builder
 from .collection import collect_gradients
 from .collector import CollectorComputer, HookCollectorBase, create_projection_matrix, fwd_bwd_factory
-from .config import AttentionConfig, IndexConfig, PreprocessConfig, QueryConfig, ScoreConfig
+from .config import AttentionConfig, IndexConfig, InversionConfig, PreprocessConfig, QueryConfig, ScoreConfig
 from .data import (
     TokenGradients,
     allocate_batches,
@@ -22,6 +22,7 @@ from .data import (
     pad_and_tensor,
 )
 from .gradient_collectors import GradientCollector, StreamingGradientCollector, TraceCollector
+from .hessians import DensePreconditioner, invert_psd_matrix, load_preconditioner
 from .gradients import AdafactorNormalizer, AdamNormalizer, GradientProcessor, LayerAdapter, Normalizer
 from .in_memory_collector import InMemoryCollector
 from .process_grads import normalize_and_aggregate_grads, normalize_flat_grad
@@ -35,5 +36,6 @@ __all__ = [
     "load_gradients", "load_module_gradients", "load_scores", "load_token_gradients", "pad_and_tensor",
     "GradientCollector", "StreamingGradientCollector", "TraceCollector", "AdafactorNormalizer", "AdamNormalizer",
     "GradientProcessor", "LayerAdapter", "Normalizer", "InMemoryCollector", "normalize_and_aggregate_grads",
-    "normalize_flat_grad", "Scorer", "build", "create_processor", "create_scorer", "get_query_grads", "score_dataset",
+    "normalize_flat_grad", "Scorer", "InversionConfig", "DensePreconditioner", "invert_psd_matrix",
+    "load_preconditioner", "build", "create_processor", "create_scorer", "get_query_grads", "score_dataset",
 ]

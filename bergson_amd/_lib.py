@@ -11,7 +11,7 @@ from pathlib import Path
 LIB_PATH = Path(__file__).resolve().parent / "libbergson_amd.so"
 
 BGX_F32, BGX_F16, BGX_BF16 = 0, 1, 2
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class ModuleDesc(C.Structure):
@@ -33,6 +33,17 @@ class ModuleDesc(C.Structure):
         ("out_col", C.c_int64),
         ("I", C.c_int32),
         ("O", C.c_int32),
+    ]
+
+
+class BlockDesc(C.Structure):
+    """bgx_block_desc: one module's fp32 matrix and its columns in a gradient row."""
+
+    _fields_ = [
+        ("h_dev", C.c_void_p),
+        ("col0", C.c_int64),
+        ("dim", C.c_int32),
+        ("reserved", C.c_int32),
     ]
 
 
@@ -82,6 +93,17 @@ SIGNATURES: dict[str, tuple] = {
     "bgx_collect_timing_enable": (C.c_int, [C.c_int32]),
     "bgx_collect_timing_read": (C.c_int, [C.POINTER(C.c_float), C.c_int32, C.POINTER(C.c_int32)]),
     "bgx_unit_normalize_rows": (C.c_int, [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p]),
+    "bgx_precond_workspace_bytes": (C.c_size_t, [C.c_int32]),
+    "bgx_block_gemm": (
+        C.c_int,
+        [C.c_void_p, C.c_int32, C.c_int64, C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.POINTER(BlockDesc), C.c_int32,
+         C.c_void_p, C.c_size_t, C.c_void_p],
+    ),
+    "bgx_gram_accumulate": (
+        C.c_int,
+        [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.POINTER(BlockDesc), C.c_int32, C.c_void_p, C.c_size_t,
+         C.c_void_p],
+    ),
     "bgx_scan_workspace_bytes": (C.c_size_t, [C.c_int32, C.c_int32, C.c_int64]),
     "bgx_scan": (
         C.c_int,

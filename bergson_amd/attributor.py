@@ -63,15 +63,23 @@ class Attributor:
                  ev_correction: bool = False):
         if faiss_cfg is not None:
             raise NotImplementedError("FAISS search is outside this package; the exact scan replaces the Flat index")
-        if hessian_path is not None:
-            raise NotImplementedError("preconditioned search (hessian_path) is outside this package")
         self.device = torch.device(device)
         if self.device.type != "cuda":
             raise RuntimeError("bergson_amd has no CPU path: Attributor needs a GPU device")
         self.dtype = dtype
         self.unit_norm = unit_norm
-        self.precondition = "none"
-        self.preconditioner = None
+        # `hessian_path` enables preconditioning: H^-1 on the queries, or -- with unit_norm -- H^-1/2 on the
+        # index rows as well as on the queries (attributor.py:73-89)
+        if hessian_path is None:
+            self.precondition = "none"
+            self.preconditioner = None
+        else:
+            from .hessians import load_preconditioner
+
+            self.precondition = "two-sided" if unit_norm else "one-sided"
+            self.preconditioner = load_preconditioner(hessian_path, inversion_cfg=inversion_cfg,
+                                                      power=-0.5 if unit_norm else -1.0, ev_correction=ev_correction,
+                                                      device=self.device)
         self.faiss_index = None
         index_path = Path(index_path)
         self.processor = GradientProcessor.load(index_path, map_location=device)
@@ -84,6 +92,13 @@ class Attributor:
             raise TypeError("float64 stores are not supported by the scan kernels")
         self.store = upload_store(load_gradients(index_path), base, self.device)
         self.N = self.store.shape[0]
+        if self.preconditioner is not None and unit_norm:
+            # split mode: the index rows are transformed once, before the scan normalises them.  The
+            # transformed store is fp32 (what g.float() @ H gives) when a second, fp32 copy fits in half of the
+            # free memory, else it keeps the store's dtype.
+            free, _ = torch.cuda.mem_get_info(self.device)
+            out_dtype = torch.float32 if self.store.numel() * 4 <= free // 2 else self.store.dtype
+            self.store = self.preconditioner.apply_rows(self.store, self.grad_sizes, out_dtype=out_dtype)
 
     @property
     def grads(self) -> dict[str, Tensor]:
@@ -94,6 +109,8 @@ class Attributor:
                reverse: bool = False):
         """Top-k rows per query by inner product (cosine when unit_norm); returns (values, indices) [..., k]."""
         q = torch.cat([queries[name].to(self.device, torch.float32) for name in self.ordered_modules], dim=1)
+        if self.preconditioner is not None:
+            q = self.preconditioner.apply_rows(q.contiguous(), self.grad_sizes)
         if self.unit_norm:
             norm = q.norm(dim=1, keepdim=True)
             q = q / (norm + torch.finfo(norm.dtype).eps)

@@ -18,7 +18,7 @@ PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 INCLUDE = PKG.parent / "include"
 LIB = PKG / "libbergson_amd.so"
-SOURCES = ["capi.hip", "collect.hip", "scan.hip", "adam.hip", "fullgrad.hip"]
+SOURCES = ["capi.hip", "collect.hip", "scan.hip", "adam.hip", "fullgrad.hip", "precond.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -54,7 +54,7 @@ def _compile(src: str, verbose: bool) -> Path:
 
 def build(verbose: bool = True) -> Path:
     """Compile every HIP source and link the shared library. Always rebuilds."""
-    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as ex:
+    with ThreadPoolExecutor(max_workers=min(6, len(SOURCES))) as ex:
         objs = list(ex.map(lambda s: _compile(s, verbose), SOURCES))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *map(str, objs), "-o", str(LIB)]
     if verbose:

@@ -48,11 +48,20 @@ class Builder:
         self.dtype = dtype
         self.attribute_tokens = attribute_tokens
         self.total_grad_dim = sum(grad_sizes.values())
-        if preprocess_cfg.hessian_path is not None:
-            raise NotImplementedError("preconditioning (preprocess_cfg.hessian_path) is outside this package")
         if device is None:
             device = torch.device("cuda", torch.cuda.current_device()) if torch.cuda.is_available() else None
         self.device = device
+        # H^-1, or H^-1/2 when the rows are unit-normalised afterwards (builder.py:75-83)
+        self.preconditioner = None
+        if preprocess_cfg.hessian_path is not None:
+            from .hessians import load_preconditioner
+
+            if device is None or device.type != "cuda":
+                raise RuntimeError("preconditioning runs on the GPU (bergson_amd has no CPU path)")
+            self.preconditioner = load_preconditioner(
+                preprocess_cfg.hessian_path, inversion_cfg=preprocess_cfg.inversion_cfg,
+                power=-0.5 if preprocess_cfg.unit_normalize else -1.0, ev_correction=preprocess_cfg.ev_correction,
+                device=device)
 
         if preprocess_cfg.aggregation != "none":
             store_name = "float32"
@@ -101,7 +110,8 @@ class Builder:
     @property
     def direct(self) -> bool:
         """True when collection kernels may write finished rows straight into the device store."""
-        return self.device_rows is not None and not self.preprocess_cfg.unit_normalize
+        return (self.device_rows is not None and not self.preprocess_cfg.unit_normalize
+                and self.preconditioner is None)
 
     def token_row_offsets(self, indices: list[int]) -> Tensor:
         """int64 [len(indices)] first store row of each document of a per-token store."""
@@ -122,6 +132,12 @@ class Builder:
             grads = mod_grads.rows
         else:
             grads = torch.cat([mod_grads[m] for m in self.grad_sizes.keys()], dim=-1)
+        if self.preconditioner is not None:
+            if not grads.is_cuda:
+                raise RuntimeError("preconditioning runs on the GPU: pass GPU tensors (bergson_amd has no CPU path)")
+            if grads.dtype not in ops.DTYPE_CODE:
+                grads = grads.to(torch.float32)
+            grads = self.preconditioner.apply_rows(grads.contiguous(), self.grad_sizes)  # fp32, as g.float() @ H^p
         if self.preprocess_cfg.unit_normalize:
             if not grads.is_cuda:
                 raise RuntimeError("unit_normalize runs on the GPU: pass GPU tensors (bergson_amd has no CPU path)")

@@ -55,12 +55,25 @@ class IndexConfig:
 
 
 @dataclass
+class InversionConfig:
+    """How to invert a Hessian with regularisation (bergson/config/config.py:78-96): `inversion` is one of
+    "damped_inverse" 1/(l + c mean(l)), "tikhonov_filtered" l/(l^2 + (c mean(l))^2), "pseudoinverse" 1/l where
+    l > c mean(l) else 0, "factored_tikhonov" (= damped_inverse for a dense Hessian); c = damping_factor."""
+
+    inversion: str = "damped_inverse"
+    damping_factor: float = 0.1
+
+
+@dataclass
 class PreprocessConfig:
     """Gradient preprocessing shared by build, reduce and score."""
 
     unit_normalize: bool = False
     hessian_path: str | None = None
+    """A saved GradientProcessor with dense autocorrelation Hessians: gradients are multiplied by H^-1, or by
+    H^-1/2 on both sides when unit_normalize is set."""
     ev_correction: bool = False
+    inversion_cfg: InversionConfig = field(default_factory=InversionConfig)
     aggregation: Literal["mean", "sum", "none"] = "none"
     normalize_aggregated_grad: bool = False
 

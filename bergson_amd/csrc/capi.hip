@@ -54,10 +54,32 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
               float query_scale, int unit_norm, int k, int64_t row_base, float* topk_val, int64_t* topk_idx,
               float* row_max, float* row_mean, float* scores, float* sumsq, void* ws, size_t ws_bytes,
               int64_t chunk_rows, void* stream);
+size_t precond_workspace_bytes(int n_blocks);
+int block_gemm_impl(const void* in, int in_dtype, int64_t in_stride, void* out, int out_dtype, int64_t out_stride,
+                    int64_t rows, const bgx_block_desc* blocks, int n_blocks, void* ws, size_t ws_bytes,
+                    void* stream);
+int gram_accumulate_impl(const void* rows_dev, int dtype, int64_t stride, int64_t rows, const bgx_block_desc* blocks,
+                         int n_blocks, void* ws, size_t ws_bytes, void* stream);
 
 }  // namespace bgx
 
 extern "C" {
+
+size_t bgx_precond_workspace_bytes(int32_t n_blocks) { return bgx::precond_workspace_bytes(n_blocks); }
+
+int bgx_block_gemm(const void* in_dev, int32_t in_dtype, int64_t in_row_stride, void* out_dev, int32_t out_dtype,
+                   int64_t out_row_stride, int64_t n_rows, const bgx_block_desc* blocks_host, int32_t n_blocks,
+                   void* workspace_dev, size_t workspace_bytes, void* stream) {
+  return bgx::block_gemm_impl(in_dev, in_dtype, in_row_stride, out_dev, out_dtype, out_row_stride, n_rows, blocks_host,
+                              n_blocks, workspace_dev, workspace_bytes, stream);
+}
+
+int bgx_gram_accumulate(const void* rows_dev, int32_t dtype, int64_t row_stride, int64_t n_rows,
+                        const bgx_block_desc* blocks_host, int32_t n_blocks, void* workspace_dev,
+                        size_t workspace_bytes, void* stream) {
+  return bgx::gram_accumulate_impl(rows_dev, dtype, row_stride, n_rows, blocks_host, n_blocks, workspace_dev,
+                                   workspace_bytes, stream);
+}
 
 int bgx_abi_version(void) { return BGX_ABI_VERSION; }
 

@@ -2,8 +2,9 @@
 
 Rows are written by the same fused launch as `GradientCollector`; after
 `teardown()` the per-module tensors are in `.gradients` and, with a scorer,
-the scores in `.scores`.  The autocorrelation statistics of the reference
-(`skip_hessians=False`) belong to Hessian fitting and are not provided.
+the scores in `.scores`.  With `skip_hessians=False` every batch's rows are also
+added into the per-module autocorrelation Grams `P^T P` (fp32, one fused launch
+for all modules), which `teardown()` normalises and attaches to the processor.
 """
 from __future__ import annotations
 
@@ -44,8 +45,9 @@ class InMemoryCollector(_DeferredBatchMixin, HookCollectorBase):
 
     def setup(self) -> None:
         assert isinstance(self.model.device, torch.device), "Model device is not set correctly"
-        if not self.skip_hessians:
-            raise NotImplementedError("autocorrelation statistics (skip_hessians=False) are outside this package")
+        if not self.skip_hessians and self.processor.projection_target == "global":
+            raise NotImplementedError("autocorrelation statistics of a global projection")
+        self._gram_blocks = None
         self.attribute_tokens = self.cfg.attribute_tokens
         if self.cfg.attribute_tokens:
             assert self.preprocess_cfg.aggregation == "none", "attribute_tokens is incompatible with reduce mode."
@@ -69,19 +71,54 @@ class InMemoryCollector(_DeferredBatchMixin, HookCollectorBase):
     def process_batch(self, indices: list[int], **kwargs) -> None:
         losses = kwargs.get("losses")
         assert losses is not None, "losses must be provided in kwargs"
-        need_rows = self.scorer is not None or self.preprocess_cfg.aggregation != "none"
+        need_rows = (self.scorer is not None or self.preprocess_cfg.aggregation != "none"
+                     or not self.skip_hessians)
         block = self._launch_batch(indices, self.builder, need_rows)
+        if not self.skip_hessians and block.rows is not None:
+            self._accumulate_grams(block.rows)
         if self.builder is not None:
             self.builder(indices, block)
         if self.scorer is not None:
             self.scorer(indices, block)
         self.per_doc_losses[indices] = losses.detach().type_as(self.per_doc_losses)
 
+    def _accumulate_grams(self, rows: Tensor) -> None:
+        """hessians[name] += P.float().T @ P.float() for every module (in_memory_collector.py:149-154)."""
+        from . import ops
+        from .data import column_offsets
+
+        if self._gram_blocks is None:
+            sizes = {name: math.prod(s) for name, s in self.shapes().items()}
+            self._gram_blocks = []
+            for name, (lo, hi) in column_offsets(sizes).items():
+                h = self.processor.hessians.get(name)
+                if h is None or h.device != rows.device or h.dtype != torch.float32 or not h.is_contiguous():
+                    h0 = torch.zeros((hi - lo, hi - lo), dtype=torch.float32, device=rows.device)
+                    if h is not None:
+                        h0.copy_(h)
+                    h = self.processor.hessians[name] = h0
+                self._gram_blocks.append((h, lo))
+        ops.gram_accumulate(rows, self._gram_blocks)
+
+    def num_rows(self) -> int:
+        """Rows summed into the Grams: documents, or gradient-carrying tokens with attribute_tokens."""
+        if self.cfg.attribute_tokens:
+            from .data import compute_num_token_grads
+
+            return int(compute_num_token_grads(self.data).sum())
+        return len(self.data)
+
     def teardown(self) -> None:
         self.remove_hooks()
         if dist.is_initialized():
             dist.reduce(self.per_doc_losses, dst=0)
         grad_sizes = {name: math.prod(s) for name, s in self.shapes().items()}
+        if not self.skip_hessians and self.processor.hessians:
+            from .hessians import process_autocorrelation_matrices
+
+            if dist.is_initialized() and dist.get_world_size() > 1:
+                raise NotImplementedError("autocorrelation statistics across ranks")
+            process_autocorrelation_matrices(self.processor, self.processor.hessians, self.num_rows(), grad_sizes)
         if self.builder is not None:
             self.builder.teardown()
             buf = self.builder.grad_buffer

@@ -12,7 +12,7 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from ._lib import BGX_BF16, BGX_F16, BGX_F32, ModuleDesc
+from ._lib import BGX_BF16, BGX_F16, BGX_F32, BlockDesc, ModuleDesc
 
 SCAN_KMAX = 2048  # largest k of the scan's fused top-k selection
 
@@ -474,6 +474,63 @@ def unit_normalize_rows_(rows: Tensor) -> Tensor:
                                      _stream())
     _lib.check(rc, "bgx_unit_normalize_rows")
     return rows
+
+
+def _block_descs(blocks: list[tuple[Tensor, int]], width: int) -> "C.Array":
+    """(matrix [d, d] fp32 on the GPU, first column) per module -> bgx_block_desc array."""
+    descs = (BlockDesc * len(blocks))()
+    for d, (h, col0) in zip(descs, blocks):
+        _need_gpu(h, "block matrix")
+        if h.dtype != torch.float32 or h.dim() != 2 or h.shape[0] != h.shape[1] or not h.is_contiguous():
+            raise ValueError("a block matrix must be a contiguous square fp32 tensor")
+        if col0 < 0 or col0 + h.shape[0] > width:
+            raise ValueError(f"block columns {col0}..{col0 + h.shape[0]} outside a row of {width}")
+        d.h_dev, d.col0, d.dim, d.reserved = h.data_ptr(), col0, h.shape[0], 0
+    return descs
+
+
+def block_gemm(rows: Tensor, blocks: list[tuple[Tensor, int]], out_dtype: torch.dtype = torch.float32,
+               out: Tensor | None = None) -> Tensor:
+    """out[:, c0:c0+d] = rows[:, c0:c0+d].float() @ H for every (H [d, d] fp32, c0) in `blocks`.
+
+    Columns that belong to no block are copied (cast) from `rows`, so that `out` is a complete row
+    block (DensePreconditioner.apply passes modules without a matrix through unchanged)."""
+    lib = _lib.load()
+    _need_gpu(rows, "rows")
+    if rows.dim() != 2 or rows.stride(1) != 1:
+        raise ValueError("rows must be 2-D with contiguous rows")
+    if out is None:
+        out = torch.empty(rows.shape, dtype=out_dtype, device=rows.device)
+    elif out.shape != rows.shape or out.stride(1) != 1 or out.data_ptr() == rows.data_ptr():
+        raise ValueError("out must be a separate [rows, width] tensor with contiguous rows")
+    covered = sum(h.shape[0] for h, _ in blocks)
+    if covered != rows.shape[1]:
+        out.copy_(rows)
+    if not blocks or rows.shape[0] == 0:
+        return out
+    descs = _block_descs(blocks, rows.shape[1])
+    nbytes = lib.bgx_precond_workspace_bytes(len(blocks))
+    ws = _workspace(rows.device, nbytes, "precond")
+    rc = lib.bgx_block_gemm(_ptr(rows), dtype_code(rows.dtype), rows.stride(0), _ptr(out), dtype_code(out.dtype),
+                            out.stride(0), rows.shape[0], descs, len(blocks), _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "bgx_block_gemm")
+    return out
+
+
+def gram_accumulate(rows: Tensor, blocks: list[tuple[Tensor, int]]) -> None:
+    """H += rows[:, c0:c0+d].float().T @ rows[:, c0:c0+d].float() for every (H, c0) in `blocks`, in place."""
+    lib = _lib.load()
+    _need_gpu(rows, "rows")
+    if rows.dim() != 2 or rows.stride(1) != 1:
+        raise ValueError("rows must be 2-D with contiguous rows")
+    if not blocks or rows.shape[0] == 0:
+        return
+    descs = _block_descs(blocks, rows.shape[1])
+    nbytes = lib.bgx_precond_workspace_bytes(len(blocks))
+    ws = _workspace(rows.device, nbytes, "precond")
+    rc = lib.bgx_gram_accumulate(_ptr(rows), dtype_code(rows.dtype), rows.stride(0), rows.shape[0], descs, len(blocks),
+                                 _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "bgx_gram_accumulate")
 
 
 @dataclass

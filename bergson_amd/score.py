@@ -3,7 +3,8 @@
 
 `get_query_grads` reads the query store, `create_scorer` normalises / aggregates the queries and builds
 the `Scorer` with its memory-mapped writer, `score_dataset` runs the collection loop with that scorer
-(one pass per query slice when `query_batch_size` is set).  Preconditioning is outside this package.
+(one pass per query slice when `query_batch_size` is set).  A dense Hessian at `preprocess_cfg.hessian_path`
+preconditions the queries once and, in split mode, every batch of index rows.
 """
 from __future__ import annotations
 
@@ -50,9 +51,19 @@ def create_scorer(path: Path, data, score_cfg: ScoreConfig, preprocess_cfg: Prep
                   dtype: torch.dtype, *, attribute_tokens: bool = False, query_range: tuple[int, int] | None = None,
                   num_queries_total: int | None = None) -> Scorer:
     """Scorer with a memory-mapped writer at `path` (score.py:138-256)."""
-    if preprocess_cfg.hessian_path is not None:
-        raise NotImplementedError("preconditioning (preprocess_cfg.hessian_path) is outside this package")
     query_grads = get_query_grads(score_cfg, query_range)
+    # H^-1/2 on both sides when the scores are cosines (split mode), H^-1 on the queries otherwise
+    # (score.py:167-192).  The query store is taken to hold raw gradients.
+    from .hessians import load_preconditioner, make_split_hessian
+
+    preconditioner = load_preconditioner(preprocess_cfg.hessian_path, inversion_cfg=preprocess_cfg.inversion_cfg,
+                                         power=-0.5 if preprocess_cfg.unit_normalize else -1.0,
+                                         ev_correction=preprocess_cfg.ev_correction, device=device)
+    index_transform = None
+    if preconditioner is not None:
+        query_grads = preconditioner.apply({m: g.to(device) for m, g in query_grads.items()})
+        if preprocess_cfg.unit_normalize:
+            index_transform = make_split_hessian(preconditioner.h_inv, score_cfg.modules, device, dtype)
     if query_range is not None and preprocess_cfg.aggregation != "none":
         raise ValueError("query_batch_size requires aggregation='none': aggregation mixes gradients across "
                          "queries, which a row slice would corrupt.")
@@ -75,7 +86,8 @@ def create_scorer(path: Path, data, score_cfg: ScoreConfig, preprocess_cfg: Prep
     return Scorer(query_grads=query_grads, modules=score_cfg.modules, writer=writer, device=device, dtype=dtype,
                   unit_normalize=preprocess_cfg.unit_normalize, score_mode=score_cfg.score,
                   attribute_tokens=attribute_tokens,
-                  query_offset=query_range[0] if query_range is not None else 0)
+                  query_offset=query_range[0] if query_range is not None else 0,
+                  **({"index_transform": index_transform} if index_transform is not None else {}))
 
 
 def score_dataset(index_cfg: IndexConfig, score_cfg: ScoreConfig, preprocess_cfg: PreprocessConfig | None = None, *,

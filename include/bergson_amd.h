@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define BGX_ABI_VERSION 2
+#define BGX_ABI_VERSION 3
 
 enum bgx_dtype { BGX_F32 = 0, BGX_F16 = 1, BGX_BF16 = 2 };
 
@@ -270,6 +270,43 @@ int bgx_scan(const void* store_dev, int64_t n_rows, int64_t D,
              float* row_max_dev, float* row_mean_dev, float* scores_dev,
              float* sumsq_dev, void* workspace_dev, size_t workspace_bytes,
              int64_t chunk_rows, void* stream);
+
+/* ---- dense per-module preconditioner --------------------------------------
+ * One fp32 matrix h_dev [dim, dim] (row-major) per module; the module's values
+ * are columns col0 .. col0 + dim of a gradient row.
+ *
+ * bgx_block_gemm: out[n, col0 + j] = sum_i fp32(in[n, col0 + i]) * h[i, j] for
+ *   every block, rows n < n_rows; fp32 accumulation, cast to out_dtype.  This
+ *   is DensePreconditioner.apply, `g @ H^p` per module
+ *   (bergson/hessians/preconditioner.py:77-92), as called by
+ *   bergson/builder.py:17-32 and bergson/query/attributor.py:138-145,
+ *   :195-200, and the batched `torch.bmm` of the split transform in
+ *   bergson/score/score.py:111-135.  out_dev must not alias in_dev; columns of
+ *   a row that belong to no block are left untouched in out_dev.
+ * bgx_gram_accumulate: h[i, j] += sum_n fp32(rows[n, col0 + i]) *
+ *   fp32(rows[n, col0 + j]) -- the autocorrelation Gram of
+ *   bergson/collector/in_memory_collector.py:149-154
+ *   (`hessians[name].addmm_(P.mT, P)` on `P.float()`).  Calls on one stream
+ *   accumulate in call order; every element has one writer (no atomics).
+ * blocks_host is read during the call; workspace_dev holds
+ * bgx_precond_workspace_bytes(n_blocks) bytes. */
+typedef struct bgx_block_desc {
+  float* h_dev;
+  int64_t col0;
+  int32_t dim;
+  int32_t reserved;
+} bgx_block_desc;
+
+size_t bgx_precond_workspace_bytes(int32_t n_blocks);
+int bgx_block_gemm(const void* in_dev, int32_t in_dtype, int64_t in_row_stride,
+                   void* out_dev, int32_t out_dtype, int64_t out_row_stride,
+                   int64_t n_rows, const bgx_block_desc* blocks_host,
+                   int32_t n_blocks, void* workspace_dev,
+                   size_t workspace_bytes, void* stream);
+int bgx_gram_accumulate(const void* rows_dev, int32_t dtype, int64_t row_stride,
+                        int64_t n_rows, const bgx_block_desc* blocks_host,
+                        int32_t n_blocks, void* workspace_dev,
+                        size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

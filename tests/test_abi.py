@@ -24,7 +24,7 @@ def test_header_symbols_are_exported_and_bound():
     for n in names:
         assert hasattr(lib, n), f"{n} is declared in the header but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes bindings and header disagree"
-    assert lib.bgx_abi_version() == _lib.ABI_VERSION == 2
+    assert lib.bgx_abi_version() == _lib.ABI_VERSION == 3
 
 
 def test_module_desc_layout_matches_header():
@@ -33,6 +33,27 @@ def test_module_desc_layout_matches_header():
     # 8 pointers, 5 int64, 2 int32
     assert C.sizeof(ModuleDesc) == 8 * 8 + 5 * 8 + 2 * 4
     assert ModuleDesc.out_col.offset == 8 * 8 + 4 * 8 and ModuleDesc.I.offset == 8 * 8 + 5 * 8
+
+
+def test_block_desc_layout_matches_header():
+    from bergson_amd._lib import BlockDesc
+
+    # pointer, int64, 2 int32
+    assert C.sizeof(BlockDesc) == 24 and BlockDesc.col0.offset == 8 and BlockDesc.dim.offset == 16
+
+
+def test_precond_argument_errors_before_any_launch():
+    from bergson_amd import _lib
+
+    lib = _lib.load()
+    assert lib.bgx_precond_workspace_bytes(48) >= 48 * 24
+    descs = (_lib.BlockDesc * 1)()
+    rc = lib.bgx_block_gemm(None, 0, 8, None, 0, 8, 4, descs, 1, None, 0, None)
+    assert rc == -1 and b"null" in lib.bgx_last_error()
+    rc = lib.bgx_gram_accumulate(C.c_void_p(256), 7, 8, 4, descs, 1, C.c_void_p(256), 1 << 20, None)
+    assert rc != 0 and b"dtype" in lib.bgx_last_error()
+    rc = lib.bgx_block_gemm(C.c_void_p(256), 0, 8, C.c_void_p(256), 0, 8, 4, descs, 1, C.c_void_p(512), 1 << 20, None)
+    assert rc != 0 and b"out" in lib.bgx_last_error()
 
 
 def test_workspace_sizes():
