@@ -25,6 +25,7 @@ from .gradient_collectors import GradientCollector, StreamingGradientCollector, 
 from .hessians import DensePreconditioner, invert_psd_matrix, load_preconditioner
 from .gradients import AdafactorNormalizer, AdamNormalizer, GradientProcessor, LayerAdapter, Normalizer
 from .in_memory_collector import InMemoryCollector
+from .optimizer_state import load_from_optimizer
 from .process_grads import normalize_and_aggregate_grads, normalize_flat_grad
 from .score import create_scorer, get_query_grads, score_dataset
 from .scorer import Scorer
@@ -37,5 +38,5 @@ __all__ = [
     "GradientCollector", "StreamingGradientCollector", "TraceCollector", "AdafactorNormalizer", "AdamNormalizer",
     "GradientProcessor", "LayerAdapter", "Normalizer", "InMemoryCollector", "normalize_and_aggregate_grads",
     "normalize_flat_grad", "Scorer", "InversionConfig", "DensePreconditioner", "invert_psd_matrix",
-    "load_preconditioner", "build", "create_processor", "create_scorer", "get_query_grads", "score_dataset",
+    "load_preconditioner", "load_from_optimizer", "build", "create_processor", "create_scorer", "get_query_grads", "score_dataset",
 ]
