@@ -40,3 +40,12 @@ __all__ = [
     "normalize_flat_grad", "Scorer", "InversionConfig", "DensePreconditioner", "invert_psd_matrix",
     "load_preconditioner", "load_from_optimizer", "build", "create_processor", "create_scorer", "get_query_grads", "score_dataset",
 ]
+
+
+def __getattr__(name: str):
+    # the Trainer callback pulls in transformers' trainer modules: imported on first use only
+    if name in ("GradientCollectorCallback", "prepare_for_gradient_collection"):
+        from . import huggingface
+
+        return getattr(huggingface, name)
+    raise AttributeError(f"module 'bergson_amd' has no attribute {name!r}")

@@ -295,6 +295,14 @@ class HookCollectorBase(ContextDecorator, ABC):
         if hasattr(module, "_inputs"):
             del module._inputs
 
+    def invalidate_prepared(self) -> None:
+        """Forget everything derived from the processor's normalizers (folded factor vectors, Adam tables):
+        call after replacing `processor.normalizers`, e.g. from live optimizer state."""
+        self._prepared.clear()
+        self._adam_prepared.clear()
+        self._full_prepared.clear()
+        self._scale_cache.clear()
+
     def remove_hooks(self) -> None:
         """Detach from the model: remove the hooks and the attributes set on the target layers."""
         for h in self._fwd_hooks:
