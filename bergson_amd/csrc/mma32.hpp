@@ -75,7 +75,9 @@ constexpr int TILE_CHUNKS = TILE_ROW_BYTES / 16;
 constexpr int LDS_ROW_BYTES = TILE_ROW_BYTES + 16;
 
 // 16 bytes of row `row` of a [n_rows, K] matrix starting at element k; zero outside the matrix.
-template <typename T, bool ALIGNED>
+// STREAM: the data is read once by the launch and every load instruction consumes whole 128-byte lines
+// (non-temporal hint; aligned rows only).
+template <typename T, bool ALIGNED, bool STREAM = false>
 __device__ inline uint4 load_chunk(const T* __restrict__ base, int64_t row, int64_t n_rows, int64_t stride,
                                    int64_t k, int64_t K) {
   constexpr int EPL = Mma32<T>::EPL;
@@ -83,7 +85,10 @@ __device__ inline uint4 load_chunk(const T* __restrict__ base, int64_t row, int6
   if (row >= n_rows || k >= K) return v;
   const T* p = base + row * stride + k;
   if (ALIGNED) {
-    v = *reinterpret_cast<const uint4*>(p);
+    if constexpr (STREAM)
+      v = load16_global_stream(p);
+    else
+      v = *reinterpret_cast<const uint4*>(p);
   } else {
     if constexpr (sizeof(T) == 4) {
       uint32_t* w = &v.x;

@@ -75,7 +75,10 @@ struct ScanArgs {
 };
 
 // Workgroup tile BM x BN, WM x WN waves, each wave (BM/WM) x (BN/WN) as 32x32 MFMA blocks.
-template <typename T, int BM, int BN, int WM, int WN, bool ALIGNED>
+// PF = how many K tiles the global loads run ahead of the LDS stores (one register set per tile in flight);
+// STREAM = non-temporal loads of the store rows, for launches with one query tile, where every store line
+// is wanted exactly once.
+template <typename T, int BM, int BN, int WM, int WN, bool ALIGNED, int PF = 1, bool STREAM = false>
 __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
   using M = Mma32<T>;
   constexpr int NT = WM * WN * 64;
@@ -130,34 +133,41 @@ __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
 #pragma unroll
   for (int i = 0; i < GCH; ++i) ss[i] = 0.f;
 
-  uint4 gr[GCH], qr[QCH];
-  auto gload = [&](int kt) {
+  uint4 gr[PF][GCH], qr[PF][QCH];  // K tile t travels in register set t % PF
+  auto gload = [&](int kt, auto set_tag) {
+    constexpr int SET = decltype(set_tag)::value;
     const int64_t k = (int64_t)kt * BK + lcol * EPL;
 #pragma unroll
     for (int i = 0; i < GCH; ++i)
-      gr[i] = load_chunk<T, ALIGNED>(store, g_row0 + lrow + i * ROWS_PER_PASS, args.rows, args.store_stride, k, D);
+      gr[SET][i] = load_chunk<T, ALIGNED, STREAM>(store, g_row0 + lrow + i * ROWS_PER_PASS, args.rows,
+                                                  args.store_stride, k, D);
 #pragma unroll
     for (int i = 0; i < QCH; ++i)
-      qr[i] = load_chunk<T, ALIGNED>(queries, q_row0 + lrow + i * ROWS_PER_PASS, args.Q, D, k, D);
+      qr[SET][i] = load_chunk<T, ALIGNED>(queries, q_row0 + lrow + i * ROWS_PER_PASS, args.Q, D, k, D);
   };
-  auto lstore = [&](int buf) {
+  auto lstore = [&](int buf, auto set_tag) {
+    constexpr int SET = decltype(set_tag)::value;
     unsigned char* base = smem + buf * BUF_BYTES;
 #pragma unroll
     for (int i = 0; i < GCH; ++i) {
-      *reinterpret_cast<uint4*>(base + (lrow + i * ROWS_PER_PASS) * LDS_ROW_BYTES + lcol * 16) = gr[i];
-      ss[i] = M::sumsq(gr[i], ss[i]);
+      *reinterpret_cast<uint4*>(base + (lrow + i * ROWS_PER_PASS) * LDS_ROW_BYTES + lcol * 16) = gr[SET][i];
+      ss[i] = M::sumsq(gr[SET][i], ss[i]);
     }
 #pragma unroll
     for (int i = 0; i < QCH; ++i)
-      *reinterpret_cast<uint4*>(base + (BM + lrow + i * ROWS_PER_PASS) * LDS_ROW_BYTES + lcol * 16) = qr[i];
+      *reinterpret_cast<uint4*>(base + (BM + lrow + i * ROWS_PER_PASS) * LDS_ROW_BYTES + lcol * 16) = qr[SET][i];
   };
 
   const int KT = (int)((D + BK - 1) / BK);
   // Pipeline: while the MFMAs of K tile kt run from LDS buffer kt&1, the registers that hold tile kt+1
-  // are written to the other buffer and the global loads of tile kt+2 are issued; one barrier per tile.
-  gload(0);
-  lstore(0);
-  if (KT > 1) gload(1);
+  // are written to the other buffer and the global loads of tile kt+1+PF are issued into the register set
+  // that has just been emptied; one barrier per tile.
+  gload(0, std::integral_constant<int, 0>{});
+  lstore(0, std::integral_constant<int, 0>{});
+  if (KT > 1) gload(1, std::integral_constant<int, 1 % PF>{});
+  if constexpr (PF > 1)
+    if (KT > 2) gload(2, std::integral_constant<int, 0>{});
+  static_assert(PF == 1 || PF == 2, "prologue spells out its loads");
   __syncthreads();
 
   const int fr = lane & 31;
@@ -173,16 +183,24 @@ __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) M::mma(af[i], bf[j], acc[i][j]);
   };
-  for (int kt = 0; kt < KT; ++kt) {
+  auto k_tile = [&](int kt, auto set_tag) {  // set_tag: the register set of tile kt + 1
     const int buf = kt & 1;
     const unsigned char* gb = smem + buf * BUF_BYTES + (wm * WTM + fr) * LDS_ROW_BYTES + fh * 16;
     const unsigned char* qb = smem + buf * BUF_BYTES + (BM + wn * WTN + fr) * LDS_ROW_BYTES + fh * 16;
     mma_step(gb, qb, 0);
-    if (kt + 1 < KT) lstore(buf ^ 1);
-    if (kt + 2 < KT) gload(kt + 2);
+    if (kt + 1 < KT) lstore(buf ^ 1, set_tag);
+    if (kt + 1 + PF < KT) gload(kt + 1 + PF, set_tag);
 #pragma unroll
     for (int kk = 1; kk < TILE_CHUNKS / 2; ++kk) mma_step(gb, qb, kk);
     __syncthreads();
+  };
+  if constexpr (PF == 1) {
+    for (int kt = 0; kt < KT; ++kt) k_tile(kt, std::integral_constant<int, 0>{});
+  } else {
+    for (int kt = 0; kt < KT; kt += 2) {
+      k_tile(kt, std::integral_constant<int, 1>{});
+      if (kt + 1 < KT) k_tile(kt + 1, std::integral_constant<int, 0>{});
+    }
   }
 
   // ---- row sum of squares -> per-row multiplier ------------------------------------
@@ -435,23 +453,27 @@ size_t scan_workspace_bytes(int Q, int k, int64_t chunk_rows) {
   return scan_layout(Q, k, effective_chunk(chunk_rows, Q)).total;
 }
 
-template <typename T, int BM, int BN, int WM, int WN>
-static int launch_gemm(const ScanArgs& a, bool aligned, hipStream_t st) {
+template <typename T, int BM, int BN, int WM, int WN, bool ALIGNED, int PF, bool STREAM>
+static int launch_gemm_v(const ScanArgs& a, hipStream_t st) {
   constexpr int NT = WM * WN * 64;
   constexpr size_t smem = 2 * (size_t)(BM + BN) * LDS_ROW_BYTES;
   const int row_tiles_pad = (a.row_tiles + 7) / 8 * 8;
   const dim3 grid((unsigned)(row_tiles_pad * a.q_tiles));
-  if (aligned) {
-    auto kern = scan_gemm_kernel<T, BM, BN, WM, WN, true>;
-    BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    hipLaunchKernelGGL(kern, grid, dim3(NT), smem, st, a);
-  } else {
-    auto kern = scan_gemm_kernel<T, BM, BN, WM, WN, false>;
-    BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    hipLaunchKernelGGL(kern, grid, dim3(NT), smem, st, a);
-  }
+  auto kern = scan_gemm_kernel<T, BM, BN, WM, WN, ALIGNED, PF, STREAM>;
+  BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+  hipLaunchKernelGGL(kern, grid, dim3(NT), smem, st, a);
   BGX_HIP(hipGetLastError());
   return 0;
+}
+
+// PF: see the kernel.  The small-tile variants are bound by HBM latency (a K tile is only 16 KB per
+// workgroup), so they run two tiles ahead, and stream the store past the caches when no other workgroup
+// will want the same rows.
+template <typename T, int BM, int BN, int WM, int WN, int PF = 1>
+static int launch_gemm(const ScanArgs& a, bool aligned, hipStream_t st) {
+  if (!aligned) return launch_gemm_v<T, BM, BN, WM, WN, false, PF, false>(a, st);
+  if (PF > 1 && a.q_tiles == 1) return launch_gemm_v<T, BM, BN, WM, WN, true, PF, true>(a, st);
+  return launch_gemm_v<T, BM, BN, WM, WN, true, PF, false>(a, st);
 }
 
 template <typename T>
@@ -470,13 +492,13 @@ static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
     a.row_tiles = (int)((a.rows + BM - 1) / BM);
     a.q_tiles = (a.Q + BN - 1) / BN;
     a.n_parts = a.q_tiles;
-    return launch_gemm<T, BM, BN, 4, 1>(a, aligned, st);
+    return launch_gemm<T, BM, BN, 4, 1, 2>(a, aligned, st);
   } else {
     constexpr int BM = 128, BN = 32;
     a.row_tiles = (int)((a.rows + BM - 1) / BM);
     a.q_tiles = (a.Q + BN - 1) / BN;
     a.n_parts = a.q_tiles;
-    return launch_gemm<T, BM, BN, 4, 1>(a, aligned, st);
+    return launch_gemm<T, BM, BN, 4, 1, 2>(a, aligned, st);
   }
 }
 
