@@ -11,7 +11,7 @@ from pathlib import Path
 LIB_PATH = Path(__file__).resolve().parent / "libbergson_amd.so"
 
 BGX_F32, BGX_F16, BGX_BF16 = 0, 1, 2
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 class ModuleDesc(C.Structure):
@@ -56,6 +56,8 @@ SIGNATURES: dict[str, tuple] = {
         [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p],
     ),
     "bgx_collect_workspace_bytes": (C.c_size_t, [C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
+    "bgx_collect_workspace_bytes_for": (C.c_size_t, [C.POINTER(ModuleDesc), C.c_int32, C.c_int32, C.c_int32, C.c_int32,
+                                                     C.c_int32]),
     "bgx_collect_seq": (
         C.c_int,
         [C.POINTER(ModuleDesc), C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p,

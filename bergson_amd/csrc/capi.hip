@@ -21,6 +21,7 @@ int hip_fail(hipError_t e, const char* what) {
 }
 
 size_t collect_workspace_bytes(int n_modules, int N, int S, int p);
+size_t collect_workspace_bytes_for(const bgx_module_desc* mods, int n_modules, int N, int S, int p, int in_dtype);
 int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules, int N, int S, int p, int in_dtype,
                  const int32_t* lengths, const int64_t* rows_or_offsets, void* out, int64_t out_row_stride,
                  int out_dtype, float lo, float hi, void* ws, size_t ws_bytes, void* stream);
@@ -92,6 +93,11 @@ int bgx_adafactor_scales(const float* row_dev, int32_t O, const float* col_dev, 
 
 size_t bgx_collect_workspace_bytes(int32_t n_modules, int32_t N, int32_t S, int32_t p) {
   return bgx::collect_workspace_bytes(n_modules, N, S, p);
+}
+
+size_t bgx_collect_workspace_bytes_for(const bgx_module_desc* mods_host, int32_t n_modules, int32_t N, int32_t S,
+                                       int32_t p, int32_t in_dtype) {
+  return bgx::collect_workspace_bytes_for(mods_host, n_modules, N, S, p, in_dtype);
 }
 
 int bgx_collect_seq(const bgx_module_desc* mods_host, int32_t n_modules, int32_t N, int32_t S, int32_t p,

@@ -343,15 +343,18 @@ struct PersistArgs {
   int r_steps;              // k-steps of LDS reserved for projection fragments
   int scratch_bytes;        // LDS between the fragments and the staging rings (exchange / per-token tiles)
   int out_vec8;             // per-token rows: every p x p block starts 16-byte aligned and p is 8 or 16
+  const uint4* frag;        // RFG: scaled projection fragments of every module in global memory
+  const int64_t* frag_off;  // RFG: [n_modules] first k-step of a module's fragments (r_in's, then r_out's)
 };
 
+// k-steps [ks0, ks1) of the matrix; the whole of it by default
 template <typename T>
 __device__ inline void stage_projection(const T* __restrict__ R, const float* __restrict__ scale, int K, int p,
-                                        uint4* __restrict__ dst, int tid) {
+                                        uint4* __restrict__ dst, int tid, int ks0 = 0, int ks1 = -1) {
   using M = Mma<T>;
-  const int nfrag = (K / M::KS) * WAVE;
+  const int nfrag = (ks1 < 0 ? K / M::KS : min(ks1, K / M::KS)) * WAVE;
   constexpr int B = STAGE_B;  // fragments per thread in flight
-  for (int f0 = tid; f0 < nfrag; f0 += COLLECT_THREADS * B) {
+  for (int f0 = ks0 * WAVE + tid; f0 < nfrag; f0 += COLLECT_THREADS * B) {
     uint4 v[B];
     uint4 s4[B][M::EPL / 4];
 #pragma unroll
@@ -490,26 +493,37 @@ __device__ inline void stream_rows(const T* base, int64_t tok_stride, int rows_v
 // at its worst case, a full drain).  For module widths that are multiples of STREAM_Q k-pairs the only
 // such repeats are at the end of a wave's last tile.
 //
+// With RFG the projection fragments do not sit in LDS (modules too wide for it) but in a table in global
+// memory, in the same fragment order, written by frag_prepare_kernel before the launch; they then travel
+// through the same queue: two 1 KB fragment loads per k-pair behind the wave's 2 * MTW row loads.  They are
+// ordinary cached loads -- every workgroup of a module reads the same table.
+//
 // loads the first block of a segment (only where nothing ran ahead of it)
-template <typename T, int MTW>
-__device__ inline void stream_prime(const T* const (&urow)[2 * MTW], int nkp, uint4 (&v)[STREAM_Q][2 * MTW]) {
+template <typename T, int MTW, bool RFG>
+__device__ inline void stream_prime(const T* const (&urow)[2 * MTW], int nkp, const uint4* __restrict__ rf, int lane,
+                                    uint4 (&v)[STREAM_Q][2 * MTW], uint4 (&rq)[RFG ? STREAM_Q : 1][2]) {
 #pragma unroll
   for (int j = 0; j < STREAM_Q; ++j) {
-    const int off = j < nkp ? j * 2 * Mma<T>::KS : 0;
+    const int jj = j < nkp ? j : 0;
 #pragma unroll
-    for (int rg = 0; rg < 2 * MTW; ++rg) v[j][rg] = load16_global_stream(urow[rg] + off);
+    for (int rg = 0; rg < 2 * MTW; ++rg) v[j][rg] = load16_global_stream(urow[rg] + jj * 2 * Mma<T>::KS);
+    if constexpr (RFG) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s) rq[j][s] = load16_global(rf + (jj * 2 + s) * WAVE + lane);
+    }
   }
   __builtin_amdgcn_sched_barrier(0);
 }
 
 // Consumes one segment (nkp k-pairs of the rows `cur`, whose first block is in v) into acc, and loads
 // behind it: the later blocks of the segment, then the first block of the segment `nxt` (nkp_next = 0:
-// nothing follows; nxt must still point at readable rows).
-template <typename T, int MTW>
+// nothing follows; nxt must still point at readable rows).  rf: the segment's fragments (LDS, or with RFG
+// the global table, whose first block is in rq); rf_next: with RFG the next segment's fragments.
+template <typename T, int MTW, bool RFG>
 __device__ inline void stream_segment(const T* const (&cur)[2 * MTW], int nkp, const T* const (&nxt)[2 * MTW],
-                                      int nkp_next, const uint4* __restrict__ rfrag,
+                                      int nkp_next, const uint4* __restrict__ rf, const uint4* __restrict__ rf_next,
                                       unsigned char* __restrict__ stage, int lane, uint4 (&v)[STREAM_Q][2 * MTW],
-                                      f32x4 (&acc)[MTW]) {
+                                      uint4 (&rq)[RFG ? STREAM_Q : 1][2], f32x4 (&acc)[MTW]) {
   using M = Mma<T>;
   using St = Stream<MTW>;
   constexpr int RG = St::RG;
@@ -530,44 +544,87 @@ __device__ inline void stream_segment(const T* const (&cur)[2 * MTW], int nkp, c
     const T* nptr[RG];
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg) nptr[rg] = last ? nxt[rg] : cur[rg] + (kp0 + Q) * 2 * M::KS;
+    const uint4* nrf = last ? rf_next : rf + (kp0 + Q) * 2 * WAVE;  // RFG only
 
-    auto step = [&](auto j_tag, auto full_tag) {
+    auto step = [&](auto j_tag) {
       constexpr int j = decltype(j_tag)::value;
-      constexpr bool FULL = decltype(full_tag)::value;
       unsigned char* slot = stage + (j % St::NSLOT) * St::SLOT_BYTES;
-      if (FULL || j < len) {
+      if (j < len) {
 #pragma unroll
         for (int rg = 0; rg < RG; ++rg) *reinterpret_cast<uint4*>(slot + rg * 1024 + lane * 16) = v[j][rg];
       }
       __builtin_amdgcn_sched_barrier(0);
-      const int off = (FULL || j < len_next) ? j * 2 * M::KS : 0;
+      const int jj = j < len_next ? j : 0;
+      auto refill = [&]() {
 #pragma unroll
-      for (int rg = 0; rg < RG; ++rg) v[j][rg] = load16_global_stream(nptr[rg] + off);
-      __builtin_amdgcn_sched_barrier(0);
-      if (FULL || j < len) {
+        for (int rg = 0; rg < RG; ++rg) v[j][rg] = load16_global_stream(nptr[rg] + jj * 2 * M::KS);
+        if constexpr (RFG) {
+#pragma unroll
+          for (int s = 0; s < 2; ++s) rq[j][s] = load16_global(nrf + (jj * 2 + s) * WAVE + lane);
+        }
+      };
+      // LDS fragments: the refill goes out before the MFMAs.  Table fragments: after them -- rq[j] is
+      // still needed by this step's MFMAs, and a refill issued earlier would have to land in other
+      // registers, which the loop could only hand over with moves that wait for the loads.
+      if constexpr (!RFG) {
+        refill();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (j < len) {
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-          const uint4 rf = rfrag[((kp0 + j) * 2 + s) * WAVE + lane];
+          uint4 rfv;
+          if constexpr (RFG)
+            rfv = rq[j][s];
+          else
+            rfv = rf[((kp0 + j) * 2 + s) * WAVE + lane];
 #pragma unroll
           for (int mt = 0; mt < MTW; ++mt) {
             const uint4 xf = *reinterpret_cast<const uint4*>(slot + foff[mt][s]);
-            M::mma(xf, rf, acc[mt]);
+            M::mma(xf, rfv, acc[mt]);
           }
         }
+      }
+      if constexpr (RFG) {
+        __builtin_amdgcn_sched_barrier(0);
+        refill();
+        __builtin_amdgcn_sched_barrier(0);
       }
     };
     // one code path for full and partial blocks: a second, unguarded copy of the steps would meet this one
     // at a join, where the queue registers of the two have to be reconciled by moves that wait for the loads
-    step(std::integral_constant<int, 0>{}, std::false_type{});
-    step(std::integral_constant<int, 1>{}, std::false_type{});
-    step(std::integral_constant<int, 2>{}, std::false_type{});
-    step(std::integral_constant<int, 3>{}, std::false_type{});
+    step(std::integral_constant<int, 0>{});
+    step(std::integral_constant<int, 1>{});
+    step(std::integral_constant<int, 2>{});
+    step(std::integral_constant<int, 3>{});
   }
 }
 static_assert(STREAM_Q == 4, "stream_segment spells out its four steps");
 
-template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED = false>
+// Fills the global fragment table of the RFG variant: block (m, 0, z) writes the scaled fragments of k-steps
+// [z, z + 1) * FRAG_STEPS_PER_WG of module m's r_in, block (m, 1, z) those of its r_out, in the order
+// stage_projection gives them in LDS.
+constexpr int FRAG_STEPS_PER_WG = 4 * STAGE_B;  // one round of loads per thread
+
+template <typename T>
+__global__ __launch_bounds__(COLLECT_THREADS) void frag_prepare_kernel(const bgx_module_desc* __restrict__ mods,
+                                                                       const int64_t* __restrict__ frag_off,
+                                                                       uint4* __restrict__ frag, int p) {
+  const bgx_module_desc d = mods[blockIdx.x];
+  const int ks0 = blockIdx.z * FRAG_STEPS_PER_WG;
+  const int K = blockIdx.y == 0 ? d.I : d.O;
+  if (ks0 * Mma<T>::KS >= K) return;
+  uint4* dst = frag + frag_off[blockIdx.x] * WAVE;
+  if (blockIdx.y == 0)
+    stage_projection<T>((const T*)d.r_in, d.col_scale, d.I, p, dst, threadIdx.x, ks0, ks0 + FRAG_STEPS_PER_WG);
+  else
+    stage_projection<T>((const T*)d.r_out, d.row_scale, d.O, p, dst + (size_t)(d.I / Mma<T>::KS) * WAVE, threadIdx.x,
+                        ks0, ks0 + FRAG_STEPS_PER_WG);
+}
+
+template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED = false, bool RFG = false>
 __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(PersistArgs pa) {
+  static_assert(STAGED || !RFG, "the global fragment table is read through the stream's queue");
   using M = Mma<T>;
   constexpr int WAVE_T = 16 * MTW;      // tokens per wave
   constexpr int TILE_T = 4 * WAVE_T;    // tokens per workgroup
@@ -596,6 +653,7 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
   // STAGED: the register queue of the wave's input stream, and whether it holds the first block of the
   // tile that comes next
   uint4 v[STAGED ? STREAM_Q : 1][2 * MTW];
+  uint4 rq[RFG ? STREAM_Q : 1][2];  // RFG: the fragments that go with v
   bool primed = false;
   for (int item = item0; item < item1; ++item) {
     const int m = item / pa.tiles_pm;
@@ -609,6 +667,9 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
 
     const bgx_module_desc d = load_uniform(args.mods + m);
     const int nA = d.I / M::KS;
+    const uint4* rfA = rfrag;  // fragments of r_in, then of r_out: in LDS, or (RFG) in the global table
+    if constexpr (RFG) rfA = pa.frag + load_uniform(pa.frag_off + m) * WAVE;
+    const uint4* rfG = rfA + (size_t)nA * WAVE;
     const int64_t t0 = s0 + wave * WAVE_T;
     const T* a0 = (const T*)d.a + (int64_t)n * d.a_seq_stride + t0 * d.a_tok_stride;
     const T* g0 = (const T*)d.g + (int64_t)n * d.g_seq_stride + t0 * d.g_tok_stride;
@@ -618,11 +679,11 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
       if (rows_valid > 0 && !primed) {
         const T* ua[2 * MTW];
         stream_rows<T, MTW>(a0, d.a_tok_stride, rows_valid, lane, ua);
-        stream_prime<T, MTW>(ua, d.I / (2 * M::KS), v);
+        stream_prime<T, MTW, RFG>(ua, d.I / (2 * M::KS), rfA, lane, v, rq);
         primed = true;
       }
     }
-    if (m != cur_m) {
+    if (!RFG && m != cur_m) {
       __syncthreads();  // every wave has finished reading the previous module's fragments
       stage_projection<T>((const T*)d.r_in, d.col_scale, d.I, p, rfrag, tid);
       stage_projection<T>((const T*)d.r_out, d.row_scale, d.O, p, rfrag + (size_t)nA * WAVE, tid);
@@ -650,9 +711,10 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
         const T* un[RG];
         stream_rows<T, MTW>(a0, d.a_tok_stride, rows_valid, lane, ua);
         stream_rows<T, MTW>(g0, d.g_tok_stride, rows_valid, lane, ug);
-        stream_segment<T, MTW>(ua, nkpA, ug, nkpG, rfrag, stage, lane, v, accA);
+        stream_segment<T, MTW, RFG>(ua, nkpA, ug, nkpG, rfA, rfG, stage, lane, v, rq, accA);
         // what follows g: the a rows of the next tile of the range, where this wave has tokens in it
         int nkpN = 0;
+        const uint4* rfN = rfG;  // RFG: the next tile's r_in fragments (any readable address when none follows)
 #pragma unroll
         for (int rg = 0; rg < RG; ++rg) un[rg] = ug[rg];
         if (item + 1 < item1) {
@@ -668,13 +730,14 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
                           (int64_t)(s02 + wave * WAVE_T) * stride2;
             stream_rows<T, MTW>(a2, stride2, rows2, lane, un);
             nkpN = load_uniform(&d2->I) / (2 * M::KS);
+            if constexpr (RFG) rfN = pa.frag + load_uniform(pa.frag_off + m2) * WAVE;
           }
         }
-        stream_segment<T, MTW>(ug, nkpG, un, nkpN, rfrag + (size_t)nA * WAVE, stage, lane, v, accG);
+        stream_segment<T, MTW, RFG>(ug, nkpG, un, nkpN, rfG, rfN, stage, lane, v, rq, accG);
         primed = nkpN > 0;
       } else {
-        project_tokens_lds<T, MTW, U>(a0, d.a_tok_stride, rows_valid, d.I, rfrag, lane, accA);
-        project_tokens_lds<T, MTW, U>(g0, d.g_tok_stride, rows_valid, d.O, rfrag + (size_t)nA * WAVE, lane, accG);
+        project_tokens_lds<T, MTW, U>(a0, d.a_tok_stride, rows_valid, d.I, rfA, lane, accA);
+        project_tokens_lds<T, MTW, U>(g0, d.g_tok_stride, rows_valid, d.O, rfG, lane, accG);
       }
       // token rows past the last valid one hold garbage: zero them in g' (that removes their products)
 #pragma unroll
@@ -881,9 +944,14 @@ static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 constexpr int PERSIST_MAX_WGS = 1024;        // upper bound on the workgroups of the persistent variant
 constexpr size_t LDS_PER_WG = 160 * 1024;    // LDS one workgroup may allocate on gfx950
 
-// head of the workspace: the descriptor table, then the item ranges of the persistent workgroups
+static size_t ranges_offset(int n_modules) { return (size_t)n_modules * sizeof(bgx_module_desc); }
+static size_t frag_off_offset(int n_modules) {
+  return align_up(ranges_offset(n_modules) + (PERSIST_MAX_WGS + 1) * sizeof(int32_t), 8);
+}
+// head of the workspace: the descriptor table, the item ranges of the persistent workgroups, and each
+// module's position in the global fragment table
 static size_t desc_bytes(int n_modules) {
-  return align_up((size_t)n_modules * sizeof(bgx_module_desc) + (PERSIST_MAX_WGS + 1) * sizeof(int32_t), 256);
+  return align_up(frag_off_offset(n_modules) + (size_t)n_modules * sizeof(int64_t), 256);
 }
 
 constexpr int MIN_TILE_T = 64;  // smallest token tile any kernel variant uses: bounds the partials
@@ -892,6 +960,27 @@ size_t collect_workspace_bytes(int n_modules, int N, int S, int p) {
   if (n_modules <= 0 || N <= 0 || S <= 0 || p <= 0) return 0;
   const size_t tiles = (size_t)((S + MIN_TILE_T - 1) / MIN_TILE_T);
   return desc_bytes(n_modules) + (size_t)n_modules * N * tiles * p * p * sizeof(float);
+}
+
+// Bytes of the global fragment table for these modules (1 KB per k-step of I + O), or 0 when the table
+// cannot be used: a width that is not a multiple of two k-steps, p > 16, a bias column.
+static size_t fragment_table_bytes(const bgx_module_desc* mods, int n_modules, int p, int in_dtype) {
+  if (p > 16) return 0;
+  const int kstep = in_dtype == BGX_F32 ? 16 : 32;
+  size_t steps = 0;
+  for (int m = 0; m < n_modules; ++m) {
+    if (mods[m].I <= 0 || mods[m].O <= 0 || mods[m].I % (2 * kstep) || mods[m].O % (2 * kstep) || mods[m].bias_col)
+      return 0;
+    steps += (size_t)(mods[m].I + mods[m].O) / kstep;
+  }
+  return steps * 1024;
+}
+
+// The workspace that also holds the fragment table, for launches whose modules are too wide for LDS.
+size_t collect_workspace_bytes_for(const bgx_module_desc* mods, int n_modules, int N, int S, int p, int in_dtype) {
+  const size_t base = collect_workspace_bytes(n_modules, N, S, p);
+  if (base == 0 || mods == nullptr) return base;
+  return align_up(base, 256) + fragment_table_bytes(mods, n_modules, p, in_dtype);
 }
 
 template <typename T, int PB, bool ALIGNED, int MT, int U>
@@ -951,9 +1040,9 @@ static int compute_units(int* out) {
   return 0;
 }
 
-template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED>
+template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED, bool RFG>
 static int launch_persist_one(int wgs, size_t lds, hipStream_t st, const PersistArgs& pa) {
-  auto kern = collect_persist_kernel<T, PER_TOKEN, MTW, U, STAGED>;
+  auto kern = collect_persist_kernel<T, PER_TOKEN, MTW, U, STAGED, RFG>;
   // the opt-in to more than 64 KB of dynamic LDS is per kernel and per device; do it once for each
   static std::atomic<bool> opted_in[MAX_DEVICES];
   int dev = 0;
@@ -966,21 +1055,23 @@ static int launch_persist_one(int wgs, size_t lds, hipStream_t st, const Persist
   return 0;
 }
 
-template <typename T, bool STAGED>
+template <typename T, bool STAGED, bool RFG>
 static int launch_persist_s(bool per_token, int tile_tokens, int wgs, size_t lds, hipStream_t st,
                             const PersistArgs& pa) {
   if (tile_tokens == 128)
-    return per_token ? launch_persist_one<T, true, 2, 4, STAGED>(wgs, lds, st, pa)
-                     : launch_persist_one<T, false, 2, 4, STAGED>(wgs, lds, st, pa);
-  return per_token ? launch_persist_one<T, true, 1, 8, STAGED>(wgs, lds, st, pa)
-                   : launch_persist_one<T, false, 1, 8, STAGED>(wgs, lds, st, pa);
+    return per_token ? launch_persist_one<T, true, 2, 4, STAGED, RFG>(wgs, lds, st, pa)
+                     : launch_persist_one<T, false, 2, 4, STAGED, RFG>(wgs, lds, st, pa);
+  return per_token ? launch_persist_one<T, true, 1, 8, STAGED, RFG>(wgs, lds, st, pa)
+                   : launch_persist_one<T, false, 1, 8, STAGED, RFG>(wgs, lds, st, pa);
 }
 
+// staged: streamed token rows; rfg: (staged only) projection fragments from the global table
 template <typename T>
-static int launch_persist(bool staged, bool per_token, int tile_tokens, int wgs, size_t lds, hipStream_t st,
+static int launch_persist(bool staged, bool rfg, bool per_token, int tile_tokens, int wgs, size_t lds, hipStream_t st,
                           const PersistArgs& pa) {
-  return staged ? launch_persist_s<T, true>(per_token, tile_tokens, wgs, lds, st, pa)
-                : launch_persist_s<T, false>(per_token, tile_tokens, wgs, lds, st, pa);
+  if (rfg) return launch_persist_s<T, true, true>(per_token, tile_tokens, wgs, lds, st, pa);
+  return staged ? launch_persist_s<T, true, false>(per_token, tile_tokens, wgs, lds, st, pa)
+                : launch_persist_s<T, false, false>(per_token, tile_tokens, wgs, lds, st, pa);
 }
 
 // LDS beside the projection fragments: the larger of the P exchange buffers and the per-token a', g' tiles
@@ -1067,8 +1158,23 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     staged = sorted[m].I % (2 * kstep) == 0 && sorted[m].O % (2 * kstep) == 0;
   if (const char* e = getenv("BGX_COLLECT_STAGED")) staged = staged && e[0] != '0';
   if (staged) persist_lds += stage_bytes;
+  // Modules too wide for LDS: the streamed kernel with the fragments in a global table, when the caller's
+  // workspace has room for it (bgx_collect_workspace_bytes_for) -- else the tile kernel.
+  const size_t frag_bytes = fragment_table_bytes(sorted.data(), n_modules, p, in_dtype);
+  const size_t frag_ws_off = align_up(need, 256);
+  bool rfg = !persist && pb == 1 && aligned && !any_bias && tiles * n_modules <= 0x7fffffffLL && frag_bytes > 0 &&
+             ws_bytes >= frag_ws_off + frag_bytes;
+  if (const char* e = getenv("BGX_COLLECT_STAGED")) rfg = rfg && e[0] != '0';
+  if (rfg) {
+    persist = staged = true;
+    r_steps = 0;
+    persist_lds = scratch_bytes + stage_bytes;
+  }
   // BGX_COLLECT_PERSIST=0 in the environment forces the one-workgroup-per-tile kernel (tests, comparisons)
-  if (const char* e = getenv("BGX_COLLECT_PERSIST")) persist = persist && e[0] != '0';
+  if (const char* e = getenv("BGX_COLLECT_PERSIST")) {
+    persist = persist && e[0] != '0';
+    rfg = rfg && persist;
+  }
 
   std::vector<unsigned char> head((size_t)n_modules * sizeof(bgx_module_desc));
   memcpy(head.data(), sorted.data(), head.size());
@@ -1089,7 +1195,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     for (int m = 0; m < n_modules; ++m) {
       const double ks = (double)((sorted[m].I + sorted[m].O) / kstep);
       w[m] = ks + REDUCE_STEPS;
-      sw[m] = ks * 32.0 / (double)tile_tokens;
+      sw[m] = rfg ? 0.0 : ks * 32.0 / (double)tile_tokens;  // nothing is staged when the fragments stay in global memory
       total += (double)tiles * w[m] + sw[m];
       biggest = std::max(biggest, w[m] + sw[m]);
     }
@@ -1126,11 +1232,33 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     first[0] = 0;
     fill(hi_l, first.data());
     first[wgs] = (int32_t)items;
-    const size_t off = head.size();
-    head.resize(off + first.size() * sizeof(int32_t));
-    memcpy(head.data() + off, first.data(), first.size() * sizeof(int32_t));
+    head.resize(desc_bytes(n_modules), 0);
+    memcpy(head.data() + ranges_offset(n_modules), first.data(), first.size() * sizeof(int32_t));
+    if (rfg) {  // where each module's fragments start, in k-steps
+      std::vector<int64_t> foff((size_t)n_modules);
+      int64_t steps = 0;
+      for (int m = 0; m < n_modules; ++m) {
+        foff[m] = steps;
+        steps += (sorted[m].I + sorted[m].O) / kstep;
+      }
+      memcpy(head.data() + frag_off_offset(n_modules), foff.data(), foff.size() * sizeof(int64_t));
+    }
   }
   BGX_HIP(hipMemcpyAsync(mods_dev, head.data(), head.size(), hipMemcpyHostToDevice, st));
+  uint4* frag_dev = (uint4*)((char*)ws + frag_ws_off);
+  const int64_t* frag_off_dev = (const int64_t*)((const char*)ws + frag_off_offset(n_modules));
+  if (rfg) {
+    int widest = 0;
+    for (int m = 0; m < n_modules; ++m) widest = std::max(widest, std::max(sorted[m].I, sorted[m].O) / kstep);
+    const dim3 pgrid((unsigned)n_modules, 2, (unsigned)((widest + FRAG_STEPS_PER_WG - 1) / FRAG_STEPS_PER_WG));
+    if (in_dtype == BGX_F32)
+      hipLaunchKernelGGL(frag_prepare_kernel<float>, pgrid, dim3(COLLECT_THREADS), 0, st, mods_dev, frag_off_dev, frag_dev, p);
+    else if (in_dtype == BGX_F16)
+      hipLaunchKernelGGL(frag_prepare_kernel<f16_t>, pgrid, dim3(COLLECT_THREADS), 0, st, mods_dev, frag_off_dev, frag_dev, p);
+    else
+      hipLaunchKernelGGL(frag_prepare_kernel<bf16_t>, pgrid, dim3(COLLECT_THREADS), 0, st, mods_dev, frag_off_dev, frag_dev, p);
+    BGX_HIP(hipGetLastError());
+  }
   args.partials = (float*)((char*)ws + desc_bytes(n_modules));
   args.row_offsets = per_token ? rows_or_offsets : nullptr;
   args.out = out;
@@ -1145,7 +1273,9 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   if (persist) {
     PersistArgs pa;
     pa.c = args;
-    pa.wg_first = (const int32_t*)((const char*)ws + (size_t)n_modules * sizeof(bgx_module_desc));
+    pa.wg_first = (const int32_t*)((const char*)ws + ranges_offset(n_modules));
+    pa.frag = frag_dev;
+    pa.frag_off = frag_off_dev;
     pa.tiles_pm = (int)tiles;
     pa.r_steps = r_steps;
     pa.scratch_bytes = (int)scratch_bytes;
@@ -1155,11 +1285,11 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     pa.out_vec8 = vec8 ? 1 : 0;
     int rc;
     if (in_dtype == BGX_F32)
-      rc = launch_persist<float>(staged, per_token, tile_tokens, wgs, persist_lds, st, pa);
+      rc = launch_persist<float>(staged, rfg, per_token, tile_tokens, wgs, persist_lds, st, pa);
     else if (in_dtype == BGX_F16)
-      rc = launch_persist<f16_t>(staged, per_token, tile_tokens, wgs, persist_lds, st, pa);
+      rc = launch_persist<f16_t>(staged, rfg, per_token, tile_tokens, wgs, persist_lds, st, pa);
     else
-      rc = launch_persist<bf16_t>(staged, per_token, tile_tokens, wgs, persist_lds, st, pa);
+      rc = launch_persist<bf16_t>(staged, rfg, per_token, tile_tokens, wgs, persist_lds, st, pa);
     if (rc != 0) return rc;
   } else if (in_dtype == BGX_F32) {
     launch_collect_pb<float>(pb, aligned, per_token, any_bias, tile_tokens, grid, st, args);

@@ -133,10 +133,17 @@ __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
 #pragma unroll
   for (int i = 0; i < GCH; ++i) ss[i] = 0.f;
 
+  const int KT = (int)((D + BK - 1) / BK);
+  // Streaming variants: row tiles start at different K tiles.  All rows of the store are the same number of
+  // bytes apart, so workgroups that walk K in step would ask the same few memory channels for every row at
+  // once.  The starting tile depends only on the row's position in the store, never on the pass.
+  const int k_rot = PF > 1 ? (int)((((args.row0 + g_row0) / BM) * 5) % KT) : 0;
   uint4 gr[PF][GCH], qr[PF][QCH];  // K tile t travels in register set t % PF
   auto gload = [&](int kt, auto set_tag) {
     constexpr int SET = decltype(set_tag)::value;
-    const int64_t k = (int64_t)kt * BK + lcol * EPL;
+    int kte = kt + k_rot;
+    if (kte >= KT) kte -= KT;
+    const int64_t k = (int64_t)kte * BK + lcol * EPL;
 #pragma unroll
     for (int i = 0; i < GCH; ++i)
       gr[SET][i] = load_chunk<T, ALIGNED, STREAM>(store, g_row0 + lrow + i * ROWS_PER_PASS, args.rows,
@@ -158,7 +165,6 @@ __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
       *reinterpret_cast<uint4*>(base + (BM + lrow + i * ROWS_PER_PASS) * LDS_ROW_BYTES + lcol * 16) = qr[SET][i];
   };
 
-  const int KT = (int)((D + BK - 1) / BK);
   // Pipeline: while the MFMAs of K tile kt run from LDS buffer kt&1, the registers that hold tile kt+1
   // are written to the other buffer and the global loads of tile kt+1+PF are issued into the register set
   // that has just been emptied; one barrier per tile.
@@ -166,7 +172,7 @@ __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
   lstore(0, std::integral_constant<int, 0>{});
   if (KT > 1) gload(1, std::integral_constant<int, 1 % PF>{});
   if constexpr (PF > 1)
-    if (KT > 2) gload(2, std::integral_constant<int, 0>{});
+    if (KT > 2) gload(2, std::integral_constant<int, 2 % PF>{});
   static_assert(PF == 1 || PF == 2, "prologue spells out its loads");
   __syncthreads();
 

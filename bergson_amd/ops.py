@@ -164,7 +164,7 @@ def _collect(per_token: bool, modules: list[ModuleInput], p: int, out: Tensor, l
         if rows.dtype != torch.int64 or rows.numel() != N or not rows.is_contiguous():
             raise ValueError("row indices / offsets must be a contiguous int64 vector of N elements")
         _need_gpu(rows, "rows")
-    nbytes = lib.bgx_collect_workspace_bytes(len(modules), N, S, p)
+    nbytes = lib.bgx_collect_workspace_bytes_for(descs, len(modules), N, S, p, dtype_code(in_dtype))
     ws = _workspace(out.device, nbytes, "collect")
     fn = lib.bgx_collect_tok if per_token else lib.bgx_collect_seq
     timer = collect_timer
@@ -252,7 +252,7 @@ def collect_prepared(per_token: bool, items: list, p: int, out: Tensor, lengths:
     for t, name, dt in ((lengths, "lengths", torch.int32), (rows, "rows", torch.int64)):
         if t is not None and (t.dtype != dt or t.numel() != N or not t.is_contiguous() or not t.is_cuda):
             raise ValueError(f"{name} must be a contiguous {dt} GPU vector of N={N} elements")
-    ws = _workspace(out.device, lib.bgx_collect_workspace_bytes(n, N, S, p), "collect")
+    ws = _workspace(out.device, lib.bgx_collect_workspace_bytes_for(descs, n, N, S, p, dtype_code(in_dtype)), "collect")
     fn = lib.bgx_collect_tok if per_token else lib.bgx_collect_seq
     timer = collect_timer
     if timer is not None:

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define BGX_ABI_VERSION 3
+#define BGX_ABI_VERSION 4
 
 enum bgx_dtype { BGX_F32 = 0, BGX_F16 = 1, BGX_BF16 = 2 };
 
@@ -93,9 +93,20 @@ int bgx_adafactor_scales(const float* row_dev, int32_t O, const float* col_dev,
                          int32_t I, int32_t dtype, float* row_scale_dev,
                          float* col_scale_dev, void* stream);
 
-/* Bytes of device workspace bgx_collect_seq / bgx_collect_tok need. */
+/* Bytes of device workspace bgx_collect_seq / bgx_collect_tok need.
+ * bgx_collect_workspace_bytes is the minimum for any modules of that count.
+ * bgx_collect_workspace_bytes_for looks at the modules (only I, O and bias_col
+ * of each descriptor are read) and adds room for a table of pre-scaled
+ * projection fragments, 32 bytes per input and output feature: with it,
+ * modules too wide for their projections to be kept on chip (Llama-3-8B's
+ * 4096 x 14336) still run through the streamed persistent kernel; without it
+ * such launches use the one-workgroup-per-tile kernel.  Both sizes are
+ * accepted by the collect entry points. */
 size_t bgx_collect_workspace_bytes(int32_t n_modules, int32_t N, int32_t S,
                                    int32_t p);
+size_t bgx_collect_workspace_bytes_for(const bgx_module_desc* mods_host,
+                                       int32_t n_modules, int32_t N, int32_t S,
+                                       int32_t p, int32_t in_dtype);
 
 /* Per-sequence projected gradients of n_modules modules of one batch in ONE
  * launch (plus a small deterministic reduction launch).

@@ -24,7 +24,7 @@ def test_header_symbols_are_exported_and_bound():
     for n in names:
         assert hasattr(lib, n), f"{n} is declared in the header but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes bindings and header disagree"
-    assert lib.bgx_abi_version() == _lib.ABI_VERSION == 3
+    assert lib.bgx_abi_version() == _lib.ABI_VERSION == 4
 
 
 def test_module_desc_layout_matches_header():
@@ -62,9 +62,18 @@ def test_workspace_sizes():
     lib = _lib.load()
     # head (descriptors + 1025 int32 item ranges of the persistent workgroups) rounded to 256 B
     # + one fp32 p*p partial per (module, sequence, 64-token tile)
-    head = -(-(48 * 112 + 1025 * 4) // 256) * 256
+    # + one int64 per module (its place in the fragment table), rounded to 256 B
+    head = -(-(-(-(48 * 112 + 1025 * 4) // 8) * 8 + 48 * 8) // 256) * 256
     assert lib.bgx_collect_workspace_bytes(48, 2, 2048, 16) == head + 48 * 2 * 32 * 256 * 4
     assert lib.bgx_collect_workspace_bytes(0, 2, 64, 16) == 0
+    # with the modules known: + 1 KB per k-step of I + O for the fragment table (bf16: 32 features per k-step)
+    descs = (_lib.ModuleDesc * 2)()
+    for d, (I, O) in zip(descs, [(4096, 14336), (4096, 1024)]):
+        d.I, d.O = I, O
+    base = lib.bgx_collect_workspace_bytes(2, 2, 2048, 16)
+    assert lib.bgx_collect_workspace_bytes_for(descs, 2, 2, 2048, 16, 2) == -(-base // 256) * 256 + (4096 + 14336 + 4096 + 1024) * 32
+    descs[1].O = 1000   # a width the streamed kernel cannot take: no table
+    assert lib.bgx_collect_workspace_bytes_for(descs, 2, 2, 2048, 16, 2) == -(-base // 256) * 256
     small = lib.bgx_scan_workspace_bytes(8, 10, 1024)
     assert small >= 8 * 10 * 8 + 8 * 1024 * 8
     assert lib.bgx_scan_workspace_bytes(1024, 100, 0) >= 1024 * 65536 * 8

@@ -238,11 +238,35 @@ def test_seq_small_projection_dims(device, dtype, p):
     assert rel_l2(got, oracle_rows(cases, dtype)) <= TOL[dtype]
 
 
-def test_wide_module_uses_the_tile_kernel(device):
-    """I + O too wide for the projection fragments to fit in LDS: the launch falls back to the tile kernel."""
-    cases = [make_case(2, 70, 4096, 1024, 16, torch.bfloat16, seed=50, normalizer="adafactor")]
-    got = run_kernel(device, cases, 16, torch.bfloat16)
-    assert rel_l2(got, oracle_rows(cases, torch.bfloat16)) <= TOL[torch.bfloat16]
+@pytest.mark.parametrize("per_token", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_wide_modules(device, dtype, per_token):
+    """I + O too wide for the projection fragments to fit in LDS: the streamed kernel reads them from a table in
+    global memory (the default variant), or the launch falls back to the tile kernel (the other two).  Several
+    tiles per workgroup, ragged lengths, a narrow module in the same launch."""
+    N, S, p = 3, 400, 16
+    lengths = [400, 130, 2]
+    wide = 4096 if dtype == torch.bfloat16 else 2048
+    shapes = [(wide, 1024), (512, wide + 512), (64, 64)]
+    cases = []
+    for i, (I, O) in enumerate(shapes):
+        a, g, left, right, norm = make_case(N, S, I, O, p, dtype, seed=50 + i, normalizer="adafactor" if i != 1 else None,
+                                            name=f"layers.{i}.wide")
+        for n, l in enumerate(lengths):
+            g[n, l - 1:] = 0
+        cases.append((a, g, left, right, norm))
+    if not per_token:
+        got = run_kernel(device, cases, p, dtype, lengths=lengths)
+        want = oracle_rows(cases, dtype)
+    else:
+        counts = [l - 1 for l in lengths]
+        row_offsets = [sum(counts[:n]) for n in range(N)]
+        mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+        got = run_kernel(device, cases, p, dtype, lengths=lengths, per_token=True, row_offsets=row_offsets,
+                         n_rows=sum(counts))
+        want = oracle_rows(cases, dtype, attribute_tokens=True, collection_mask=mask)
+    assert got.shape == want.shape
+    assert rel_l2(got, want) <= TOL[dtype]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
