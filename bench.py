@@ -39,7 +39,7 @@ HBM_PEAK_GBS = 8000.0
 COLLECT_TRAFFIC_RATIO = 1.036
 # the same for the store scan: 1024 queries (four query tiles re-read each row tile, half from L2), 32 queries
 SCAN_TRAFFIC_RATIO_Q1024 = 1.51
-SCAN_TRAFFIC_RATIO_Q32 = 1.007
+SCAN_TRAFFIC_RATIO_Q32 = 1.0014
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
@@ -274,7 +274,7 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "bgx::collect_persist_kernel<bf16_t, false, 2, 4, true> and <bf16_t, false, 1, 8, true> (128- and 64-token tiles, streamed loads)",
+            "kernel": "bgx::collect_persist_kernel<bf16_t, false, 2, 4, true, false> and <bf16_t, false, 1, 8, true, false> (128- and 64-token tiles, streamed loads, projections in LDS)",
             "achieved": coll["achieved_gbs"],
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",

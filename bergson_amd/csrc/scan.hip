@@ -134,10 +134,10 @@ __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
   for (int i = 0; i < GCH; ++i) ss[i] = 0.f;
 
   const int KT = (int)((D + BK - 1) / BK);
-  // Streaming variants: row tiles start at different K tiles.  All rows of the store are the same number of
+  // Streaming variant (one query tile): row tiles start at different K tiles.  All rows of the store are the same number of
   // bytes apart, so workgroups that walk K in step would ask the same few memory channels for every row at
   // once.  The starting tile depends only on the row's position in the store, never on the pass.
-  const int k_rot = PF > 1 ? (int)((((args.row0 + g_row0) / BM) * 5) % KT) : 0;
+  const int k_rot = STREAM ? (int)((((args.row0 + g_row0) / BM) * 5) % KT) : 0;
   uint4 gr[PF][GCH], qr[PF][QCH];  // K tile t travels in register set t % PF
   auto gload = [&](int kt, auto set_tag) {
     constexpr int SET = decltype(set_tag)::value;
