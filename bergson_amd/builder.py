@@ -10,6 +10,7 @@ Otherwise each batch goes through one device buffer and one D2H copy.
 """
 from __future__ import annotations
 
+import os
 from pathlib import Path
 
 import numpy as np
@@ -20,7 +21,7 @@ from torch import Tensor
 from . import ops
 from .config import PreprocessConfig
 from .data import compute_num_token_grads, create_index, create_token_index
-from .utils import dtype_name, storage_np_dtype, tensor_to_numpy
+from .utils import DeviceIndexRing, dtype_name, storage_np_dtype, tensor_to_numpy
 
 
 class RowBlock(dict):
@@ -32,6 +33,7 @@ class RowBlock(dict):
 
     rows: Tensor | None = None
     committed: bool = False
+    indices_dev: Tensor | None = None  # the batch's document indices, already on the device
 
 
 class Builder:
@@ -92,9 +94,12 @@ class Builder:
                 self.grad_buffer = np.zeros((num_grads, self.total_grad_dim), dtype=np_dtype)
 
         # ---- device-resident store ---------------------------------------------------------
+        self._index_ring = DeviceIndexRing()
         self.device_rows: Tensor | None = None
         self._offsets_dev: Tensor | None = None
         self._dirty = False
+        self._dirty_rows: np.ndarray | None = None  # which rows of the device store the host copy lacks
+        self._stage: Tensor | None = None           # pinned staging buffer of flush()
         if self.in_memory_grad_buffer is None and device is not None and device.type == "cuda":
             nbytes = int(self.grad_buffer.shape[0]) * self.total_grad_dim * np_dtype.itemsize
             if device_store_bytes is None:
@@ -103,6 +108,11 @@ class Builder:
             if 0 < nbytes <= device_store_bytes:
                 self.device_rows = torch.zeros((self.grad_buffer.shape[0], self.total_grad_dim), dtype=dtype,
                                                device=device)
+                self._dirty_rows = np.zeros(self.grad_buffer.shape[0], dtype=bool)
+                # the pinned staging buffer of flush(), allocated here: pinning memory takes tens of ms
+                row_bytes = max(1, self.total_grad_dim * self.device_rows.element_size())
+                rows = max(1, min(self.FLUSH_STAGE_BYTES // row_bytes, self.grad_buffer.shape[0]))
+                self._stage = torch.empty((rows, self.total_grad_dim), dtype=dtype, pin_memory=True)
             if self.offsets is not None:
                 self._offsets_dev = torch.from_numpy(self.offsets).to(device)
 
@@ -116,17 +126,27 @@ class Builder:
     def token_row_offsets(self, indices: list[int]) -> Tensor:
         """int64 [len(indices)] first store row of each document of a per-token store."""
         assert self._offsets_dev is not None
-        idx = torch.as_tensor(indices, dtype=torch.int64).to(self._offsets_dev.device, non_blocking=True)
+        idx = indices if isinstance(indices, Tensor) else self._index_ring.get(indices, self._offsets_dev.device)
         return self._offsets_dev[idx].contiguous()
 
-    def mark_written(self) -> None:
+    def mark_written(self, indices: list[int] | None = None) -> None:
+        """Rows of the device store have changed: those of the documents `indices`, or possibly all."""
         self._dirty = True
+        if self._dirty_rows is None:
+            return
+        if indices is None:
+            self._dirty_rows[:] = True
+        elif self.offsets is not None:
+            for i in indices:
+                self._dirty_rows[int(self.offsets[i]):int(self.offsets[i + 1])] = True
+        else:
+            self._dirty_rows[indices] = True
 
     # ---- __call__ -------------------------------------------------------------------------------
     def __call__(self, indices: list[int], mod_grads: dict[str, Tensor]) -> None:
         """Concatenate the modules of a batch, optionally unit-normalise, and place the rows."""
         if isinstance(mod_grads, RowBlock) and mod_grads.committed:
-            self._dirty = True
+            self.mark_written(indices)
             return
         if isinstance(mod_grads, RowBlock) and mod_grads.rows is not None:
             grads = mod_grads.rows
@@ -150,11 +170,11 @@ class Builder:
             self.in_memory_grad_buffer[0] += grads.sum(dim=0).to(dtype=torch.float32,
                                                                  device=self.in_memory_grad_buffer.device)
             return
-        self._scatter(indices, grads)
+        self._scatter(indices, grads, getattr(mod_grads, "indices_dev", None))
 
-    def _scatter(self, indices: list[int], grads: Tensor) -> None:
+    def _scatter(self, indices: list[int], grads: Tensor, indices_dev: Tensor | None = None) -> None:
         if self.device_rows is not None and grads.is_cuda:
-            idx = torch.as_tensor(indices, dtype=torch.int64).to(grads.device, non_blocking=True)
+            idx = indices_dev if indices_dev is not None else self._index_ring.get(indices, grads.device)
             if self.attribute_tokens:
                 assert self._offsets_dev is not None
                 starts = self._offsets_dev[idx]
@@ -164,7 +184,7 @@ class Builder:
                 self.device_rows.index_copy_(0, rows, grads.to(self.device_rows.dtype))
             else:
                 self.device_rows.index_copy_(0, idx, grads.to(self.device_rows.dtype))
-            self._dirty = True
+            self.mark_written(indices)
             return
         host = tensor_to_numpy(grads.to(self.dtype).cpu())
         if self.attribute_tokens:
@@ -177,15 +197,52 @@ class Builder:
             self.grad_buffer[indices] = host
 
     # ---- lifecycle -------------------------------------------------------------------------------
+    FLUSH_STAGE_BYTES = 64 << 20  # pinned staging buffer of flush()
+    FLUSH_MERGE_ROWS = 32         # runs of changed rows closer than this are written as one
+
+    def _dirty_runs(self) -> list[tuple[int, int]]:
+        """[lo, hi) runs of rows changed since the last flush, neighbours merged."""
+        assert self._dirty_rows is not None
+        idx = np.flatnonzero(self._dirty_rows)
+        if idx.size == 0:
+            return []
+        cut = np.flatnonzero(np.diff(idx) > self.FLUSH_MERGE_ROWS)
+        starts = np.concatenate(([idx[0]], idx[cut + 1]))
+        ends = np.concatenate((idx[cut], [idx[-1]])) + 1
+        return list(zip(starts.tolist(), ends.tolist()))
+
     def flush(self) -> None:
-        """Copy the device store to the host buffer (once) and flush the memory map."""
+        """Bring the host copy of the store up to date and flush the memory map.
+
+        Only rows written since the last flush travel: device -> pinned staging buffer -> the file (one
+        `pwrite` per run of rows; assigning through the memory map instead takes a page fault per 4 KB) or
+        the in-memory array."""
         if self.device_rows is not None and self._dirty:
-            n = self.device_rows.shape[0]
             row_bytes = max(1, self.total_grad_dim * self.device_rows.element_size())
-            step = max(1, (1 << 30) // row_bytes)
-            for lo in range(0, n, step):
-                hi = min(n, lo + step)
-                self.grad_buffer[lo:hi] = tensor_to_numpy(self.device_rows[lo:hi].cpu())
+            assert self._stage is not None
+            to_file = isinstance(self.grad_buffer, np.memmap)
+            fd = os.open(self.grad_buffer.filename, os.O_WRONLY) if to_file else -1
+            try:
+                for run_lo, run_hi in self._dirty_runs():
+                    for lo in range(run_lo, run_hi, self._stage.shape[0]):
+                        hi = min(run_hi, lo + self._stage.shape[0])
+                        stage = self._stage[:hi - lo]
+                        stage.copy_(self.device_rows[lo:hi], non_blocking=True)
+                        torch.cuda.current_stream(self.device_rows.device).synchronize()
+                        host = tensor_to_numpy(stage)
+                        if to_file:
+                            view = memoryview(host).cast("B")
+                            off = int(self.grad_buffer.offset) + lo * row_bytes
+                            done = 0
+                            while done < len(view):
+                                done += os.pwrite(fd, view[done:], off + done)
+                        else:
+                            self.grad_buffer[lo:hi] = host
+            finally:
+                if fd >= 0:
+                    os.close(fd)
+            assert self._dirty_rows is not None
+            self._dirty_rows[:] = False
             self._dirty = False
         if isinstance(self.grad_buffer, np.memmap):
             self.grad_buffer.flush()

@@ -25,7 +25,7 @@ from .builder import Builder, RowBlock
 from .collector import HookCollectorBase
 from .config import IndexConfig, PreprocessConfig
 from .data import column_offsets
-from .utils import get_gradient_dtype
+from .utils import DeviceIndexRing, get_gradient_dtype
 
 
 class _DeferredBatchMixin:
@@ -42,6 +42,17 @@ class _DeferredBatchMixin:
             return 0  # every module adds into the single "gradients" block
         return cols[name]
 
+    def _indices_dev(self, indices: list[int], device) -> Tensor:
+        ring = getattr(self, "_index_ring", None)
+        if ring is None:
+            ring = self._index_ring = DeviceIndexRing()
+        return ring.get(indices, torch.device(device))
+
+    def _record_losses(self, indices: list[int], losses: Tensor) -> None:
+        """per_doc_losses[indices] = losses, with the indices taken to the device without a host stall."""
+        idx = self._indices_dev(indices, self.per_doc_losses.device)
+        self.per_doc_losses.index_copy_(0, idx, losses.detach().to(self.per_doc_losses.dtype))
+
     def _launch_batch(self, indices: list[int], builder: Builder | None, need_rows: bool) -> RowBlock:
         """Runs the deferred launch.  Rows go straight into the builder's device store when it accepts
         them and nobody else needs them; otherwise into a fresh batch buffer whose column views are
@@ -52,6 +63,7 @@ class _DeferredBatchMixin:
             return block
         g0 = queued[0][-1]
         dev = g0.device
+        block.indices_dev = self._indices_dev(indices, dev)
         N = g0.shape[0]
         assert N == len(indices), f"batch of {N} sequences but {len(indices)} indices"
         lengths = self._batch_lengths(dev) if (self.attribute_tokens or self.skip_padding) else None
@@ -60,7 +72,7 @@ class _DeferredBatchMixin:
             assert lengths is not None, "attribute_tokens needs a collection mask (with_batch)"
             if direct:
                 self.launch_deferred(builder.device_rows, lengths=lengths,
-                                     row_offsets=builder.token_row_offsets(indices))
+                                     row_offsets=builder.token_row_offsets(block.indices_dev))
                 block.committed = True
                 return block
             counts = (lengths.to(torch.int64) - 1).clamp_min_(0)
@@ -74,8 +86,7 @@ class _DeferredBatchMixin:
                 self._deferred_adam.clear()
                 self._deferred_full.clear()
         elif direct:
-            idx = torch.as_tensor(indices, dtype=torch.int64).to(dev, non_blocking=True)
-            self.launch_deferred(builder.device_rows, lengths=lengths, out_rows=idx)
+            self.launch_deferred(builder.device_rows, lengths=lengths, out_rows=block.indices_dev)
             block.committed = True
             return block
         else:
@@ -148,7 +159,7 @@ class GradientCollector(_DeferredBatchMixin, HookCollectorBase):
             self.scorer(indices, block)
         if self.builder or self.scorer:
             self.mod_grads = {}
-        self.per_doc_losses[indices] = losses.detach().type_as(self.per_doc_losses)
+        self._record_losses(indices, losses)
 
     def teardown(self):
         if dist.is_initialized():

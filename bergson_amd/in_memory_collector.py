@@ -80,7 +80,7 @@ class InMemoryCollector(_DeferredBatchMixin, HookCollectorBase):
             self.builder(indices, block)
         if self.scorer is not None:
             self.scorer(indices, block)
-        self.per_doc_losses[indices] = losses.detach().type_as(self.per_doc_losses)
+        self._record_losses(indices, losses)
 
     def _accumulate_grams(self, rows: Tensor) -> None:
         """hessians[name] += P.float().T @ P.float() for every module (in_memory_collector.py:149-154)."""

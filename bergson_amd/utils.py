@@ -54,3 +54,42 @@ def numpy_to_tensor(arr: np.ndarray, base_dtype: str | None = None) -> Tensor:
 
 def convert_precision_to_torch(precision: str) -> torch.dtype:
     return {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[precision]
+
+
+class DeviceIndexRing:
+    """Document indices of a batch as an int64 device tensor without stalling the host.
+
+    A Python list handed to torch for indexing, or an unpinned CPU tensor moved to the GPU, is copied with a
+    stream synchronisation: the host then waits for the whole backward pass it has just queued.  The lists
+    go through a ring of pinned slots instead; a slot is reused only after the copy out of it has finished
+    (an event per slot, normally long since signalled)."""
+
+    def __init__(self, slots: int = 32):
+        self.slots = slots
+        self._buf: torch.Tensor | None = None
+        self._events: list = [None] * slots
+        self._next = 0
+        self._last: tuple | None = None  # (key, tensor) of the most recent list: a batch asks more than once
+
+    def get(self, indices, device: torch.device) -> torch.Tensor:
+        key = (tuple(indices), str(device))
+        if self._last is not None and self._last[0] == key:
+            return self._last[1]
+        n = len(indices)
+        if self._buf is None or self._buf.shape[1] < n:
+            if self._buf is not None:
+                torch.cuda.synchronize()  # copies out of the old ring
+            self._buf = torch.empty((self.slots, max(256, 2 * n)), dtype=torch.int64, pin_memory=True)
+            self._events = [None] * self.slots
+        i = self._next
+        self._next = (i + 1) % self.slots
+        if self._events[i] is not None:
+            self._events[i].synchronize()
+        row = self._buf[i, :n]
+        row.copy_(torch.as_tensor(indices, dtype=torch.int64))
+        out = row.to(device, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self._events[i] = ev
+        self._last = (key, out)
+        return out
