@@ -274,3 +274,48 @@ def test_attributor_full_ranking_beyond_the_fused_top_k(device, tmp_path):
     assert (vals.cpu() - ref_v).abs().max().item() <= 1e-3
     assert (idx.cpu() == ref_i).float().mean().item() > 0.99  # neighbours closer than the tolerance may swap
     assert all(sorted(r.tolist()) == list(range(n)) for r in idx.cpu())
+
+
+@pytest.mark.parametrize("attribute_tokens", [False, True])
+def test_builder_flushes_only_changed_rows(device, tmp_path, attribute_tokens):
+    """Device-resident store: rows reach the file at flush(), run by run of changed rows; a second flush after
+    more batches adds exactly those; rows never written stay zero; the memory map sees what was written."""
+    from bergson_amd import Builder, PreprocessConfig, load_gradients
+    from bergson_amd.builder import RowBlock
+    from bergson_amd.synthetic import ListDataset
+
+    lengths = [5, 3, 9, 2, 7, 4, 6, 8, 3, 5, 2, 9] * 20
+    data = ListDataset([[1] * l for l in lengths])
+    sizes = {"a": 64, "b": 32}
+    b = Builder(data, sizes, torch.float16, PreprocessConfig(), attribute_tokens=attribute_tokens,
+                path=tmp_path / "store", device=torch.device(device))
+    assert b.direct and b.device_rows is not None
+    n_rows = b.device_rows.shape[0]
+    want = torch.zeros((n_rows, 96), dtype=torch.float16)
+    gen = torch.Generator().manual_seed(3)
+
+    def write(docs):
+        if attribute_tokens:
+            rows = torch.cat([torch.arange(int(b.offsets[i]), int(b.offsets[i + 1])) for i in docs])
+        else:
+            rows = torch.tensor(docs)
+        vals = torch.randn(len(rows), 96, generator=gen).to(torch.float16)
+        want[rows] = vals
+        b.device_rows[rows.to(device)] = vals.to(device)      # what the collection kernel does on the direct path
+        block = RowBlock()
+        block.committed = True
+        b(docs, block)
+
+    write([0, 1, 2, 200, 201])
+    write([77])
+    runs = b._dirty_runs()
+    assert 2 <= len(runs) <= 3 and all(lo < hi for lo, hi in runs)
+    b.flush()
+    assert b._dirty_runs() == []
+    assert torch.equal(torch.from_numpy(np.array(b.grad_buffer)), want)          # through the memory map
+    assert torch.equal(torch.from_numpy(np.array(load_gradients(tmp_path / "store"))), want)  # through the file
+    write([5, 6, 239, 100])
+    b.teardown()
+    got = torch.from_numpy(np.array(load_gradients(tmp_path / "store")))
+    assert torch.equal(got, want)
+    assert (got.abs().sum(1) == 0).sum() >= n_rows // 2    # most rows were never written and are still zero
