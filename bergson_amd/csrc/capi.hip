@@ -51,6 +51,7 @@ int collect_timing_enable(int max_launches);
 int collect_timing_read(float* ms_out, int capacity, int* count_out);
 int unit_normalize_impl(void* rows, int64_t n_rows, int64_t D, int64_t stride, int dtype, void* stream);
 size_t scan_workspace_bytes(int Q, int k, int64_t chunk_rows);
+size_t scan_workspace_bytes_for(int Q, int k, int64_t chunk_rows, int64_t D, int dtype);
 int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int dtype, const void* queries, int Q,
               float query_scale, int unit_norm, int k, int64_t row_base, float* topk_val, int64_t* topk_idx,
               float* row_max, float* row_mean, float* scores, float* sumsq, void* ws, size_t ws_bytes,
@@ -178,6 +179,10 @@ int bgx_collect_timing_read(float* ms_out, int32_t capacity, int32_t* count_out)
 int bgx_unit_normalize_rows(void* rows_dev, int64_t n_rows, int64_t D, int64_t row_stride, int32_t dtype,
                             void* stream) {
   return bgx::unit_normalize_impl(rows_dev, n_rows, D, row_stride, dtype, stream);
+}
+
+size_t bgx_scan_workspace_bytes_for(int32_t Q, int32_t k, int64_t chunk_rows, int64_t D, int32_t dtype) {
+  return bgx::scan_workspace_bytes_for(Q, k, chunk_rows, D, dtype);
 }
 
 size_t bgx_scan_workspace_bytes(int32_t Q, int32_t k, int64_t chunk_rows) {

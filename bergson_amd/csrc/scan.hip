@@ -23,6 +23,7 @@
 
 #include "common.hpp"
 #include "mma32.hpp"
+#include "stream.hpp"
 
 namespace bgx {
 
@@ -72,6 +73,7 @@ struct ScanArgs {
   uint32_t* cand_count;  // [Q]
   uint64_t* cand;        // [Q][cand_cap]
   int64_t cand_cap;
+  int first_pass;        // streaming kernel, no thresholds yet: row r of the pass is entry r of every query's list
 };
 
 // Workgroup tile BM x BN, WM x WN waves, each wave (BM/WM) x (BN/WN) as 32x32 MFMA blocks.
@@ -280,6 +282,149 @@ __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
   }
 }
 
+// ---- few queries: the store streamed once, no tiles in LDS ---------------------------------------
+// With at most 32 queries the scan is a matter of reading the store once, and the tile kernel above -- a
+// barrier and an LDS round trip of the whole workgroup per 64 columns -- tops out at 5.3 TB/s.  This kernel
+// is the collection kernel's input stream pointed at the store: persistent workgroups, each wave streams 64
+// rows at a time over all of D with whole-line non-temporal loads through its register queue and its own
+// LDS slot, the queries come as MFMA fragments from a table in global memory (built once per scan; every
+// wave reads the same table, so it lives in L2), the row norms are summed from the data on its way to LDS.
+// No workgroup barrier anywhere.  Scores land in 16 x 16 accumulators: lane (c, q4) holds rows 4 q4 + e of
+// each 16-row block against query 16 qb + c.
+constexpr int SS_MTW = 4;                // 16-row blocks per wave
+constexpr int SS_WAVE_ROWS = 16 * SS_MTW;
+constexpr int SS_TILE_ROWS = 4 * SS_WAVE_ROWS;
+
+template <typename T>
+__global__ __launch_bounds__(COLLECT_THREADS) void scan_query_fragments_kernel(const T* __restrict__ queries, int Q,
+                                                                               int64_t D, int nblk,
+                                                                               uint4* __restrict__ table) {
+  const int blk = blockIdx.y;
+  const int ks0 = blockIdx.x * 4 * STAGE_B;
+  if ((int64_t)ks0 * Mma<T>::KS >= D) return;
+  stage_projection<T>(queries + (int64_t)blk * 16 * D, nullptr, (int)D, min(16, Q - blk * 16), table, threadIdx.x, ks0,
+                      ks0 + 4 * STAGE_B, blk, nblk);
+}
+
+template <typename T, int QB>
+__global__ __launch_bounds__(COLLECT_THREADS, 1) void scan_stream_kernel(ScanArgs args, const uint4* __restrict__ qfrag) {
+  using M = Mma<T>;
+  using St = Stream<SS_MTW>;
+  constexpr int RG = St::RG;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  unsigned char* stage = smem + wave * St::BYTES_PER_WAVE;
+  constexpr int SC_PITCH = 16 * QB + 1;  // floats per row of the wave's score block in LDS (odd: no bank conflicts)
+  float* sc = reinterpret_cast<float*>(smem + 4 * St::BYTES_PER_WAVE) + wave * (SS_WAVE_ROWS * SC_PITCH);
+  float* wrow = reinterpret_cast<float*>(smem + 4 * St::BYTES_PER_WAVE) + 4 * (SS_WAVE_ROWS * SC_PITCH) +
+                wave * SS_WAVE_ROWS;  // row multipliers
+  const int c = lane & 15;
+  const int q4 = lane >> 4;
+  const int rho = lane >> 3;
+  const int sig = lane & 7;
+
+  const T* store = (const T*)args.store + args.row0 * args.store_stride;
+  const int nkp = (int)(args.D / (2 * M::KS));
+  const int64_t n_tiles = (args.rows + SS_TILE_ROWS - 1) / SS_TILE_ROWS;
+  const int64_t t_first = n_tiles * blockIdx.x / gridDim.x;
+  const int64_t t_last = n_tiles * (blockIdx.x + 1) / gridDim.x;
+
+  if (args.first_pass && blockIdx.x == 0 && tid < args.Q) args.cand_count[tid] = (uint32_t)args.rows;
+
+  uint4 v[STREAM_Q][RG];
+  uint4 rq[STREAM_Q][2 * QB];
+  bool primed = false;
+  for (int64_t tile = t_first; tile < t_last; ++tile) {
+    const int64_t prow0 = tile * SS_TILE_ROWS + wave * SS_WAVE_ROWS;  // pass-local first row of this wave
+    const int rows_valid = (int)min((int64_t)SS_WAVE_ROWS, args.rows - prow0);
+    if (rows_valid <= 0) {
+      primed = false;
+      continue;
+    }
+    const T* ur[RG];
+    const T* un[RG];
+    stream_rows<T, SS_MTW>(store + prow0 * args.store_stride, args.store_stride, rows_valid, lane, ur);
+    if (!primed) stream_prime<T, SS_MTW, true, QB>(ur, nkp, qfrag, lane, v, rq);
+    int nkp_next = 0;
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg) un[rg] = ur[rg];
+    if (tile + 1 < t_last) {
+      const int64_t prow1 = prow0 + SS_TILE_ROWS;
+      const int rows1 = (int)min((int64_t)SS_WAVE_ROWS, args.rows - prow1);
+      if (rows1 > 0) {
+        stream_rows<T, SS_MTW>(store + prow1 * args.store_stride, args.store_stride, rows1, lane, un);
+        nkp_next = nkp;
+      }
+    }
+    f32x4 acc[SS_MTW * QB];
+#pragma unroll
+    for (int i = 0; i < SS_MTW * QB; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float ssq[RG];
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg) ssq[rg] = 0.f;
+    stream_segment<T, SS_MTW, true, QB, true>(ur, nkp, un, nkp_next, qfrag, qfrag, stage, lane, v, rq, acc, ssq);
+    primed = nkp_next > 0;
+
+    // ---- row norms: lane (rho, sig) carried slot sig of row rg * 8 + rho; a row's 8 lanes add up ----
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg) {
+      float s = ssq[rg];
+      s += __shfl_xor(s, 1);
+      s += __shfl_xor(s, 2);
+      s += __shfl_xor(s, 4);
+      const int row = rg * 8 + rho;
+      if (sig == 0) {
+        float w = args.query_scale;
+        if (args.unit_norm) w = s > 0.f ? args.query_scale / sqrtf(s) : 0.f;
+        wrow[row] = w;
+        if (args.sumsq != nullptr && row < rows_valid) args.sumsq[args.row0 + prow0 + row] = s;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+
+    // ---- scores: through LDS, so that lane l owns row l and walks the queries in a plain loop -------------
+#pragma unroll
+    for (int mt = 0; mt < SS_MTW; ++mt)
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sc[(mt * 16 + q4 * 4 + e) * SC_PITCH + qb * 16 + c] = acc[mt * QB + qb][e];
+    __builtin_amdgcn_wave_barrier();
+    {
+      const int row = lane;
+      const bool row_ok = row < rows_valid;
+      const int64_t prow = prow0 + row;
+      const int64_t grow = args.row0 + prow;
+      const float w = wrow[row];
+      float rmax = -INFINITY;
+      float rsum = 0.f;
+      for (int qi = 0; qi < args.Q; ++qi) {
+        const float val = sc[row * SC_PITCH + qi] * w;
+        const float thr = args.thr != nullptr ? args.thr[qi] : INFINITY;
+        if (row_ok) {
+          rmax = fmaxf(rmax, val);
+          rsum += val;  // queries in ascending order: a fixed sum
+          if (args.scores != nullptr) args.scores[grow * args.Q + qi] = val;
+          if (args.first_pass) {
+            args.cand[qi * args.cand_cap + prow] = make_key(val, (uint32_t)grow);
+          } else if (val > thr) {
+            const uint32_t pos = atomicAdd(&args.cand_count[qi], 1u);
+            if ((int64_t)pos < args.cand_cap) args.cand[qi * args.cand_cap + pos] = make_key(val, (uint32_t)grow);
+          }
+        }
+      }
+      if (row_ok) {
+        if (args.row_max_enc != nullptr) atomicMax(&args.row_max_enc[grow], f32_ordered(rmax));
+        if (args.row_sum_part != nullptr) args.row_sum_part[prow * args.n_parts] = rsum;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();  // sc and wrow are rewritten by the next tile
+  }
+}
+
 // ---- per-query exact selection ---------------------------------------------------------------
 struct SelectArgs {
   uint64_t* top;         // [Q][k] sorted descending
@@ -291,95 +436,191 @@ struct SelectArgs {
   int k;
 };
 
-__global__ __launch_bounds__(256) void scan_select_kernel(SelectArgs a) {
-  __shared__ uint64_t keys[SCAN_KMAX];
-  __shared__ uint32_t hist[256];
-  __shared__ uint64_t s_prefix;
-  __shared__ uint32_t s_rank;
-  __shared__ uint32_t s_fill;
+constexpr int SELECT_THREADS = 1024;
+constexpr uint32_t SELECT_SAMPLE = 4096;                     // > SCAN_KMAX
+constexpr uint32_t SELECT_PRESELECT_MIN = 4 * SELECT_SAMPLE;  // shorter lists go to the exact selection directly
+constexpr int SELECT_COMPACT_U = 4;                           // keys per thread and compaction step
+
+struct SelectShared {
+  uint64_t keys[SCAN_KMAX];
+  uint32_t hist[256];
+  uint32_t part[SELECT_COMPACT_U * SELECT_THREADS / 64 + 1];  // compaction: per (sub-block, wave) counts, then offsets
+  uint64_t prefix;
+  uint32_t rank;
+  uint32_t fill;
+};
+
+// The rank-th largest (rank from 1, rank <= n) of the n keys elem(0..n-1): radix select, 8 bits per pass from
+// the top.  Every thread of the workgroup calls it.
+template <typename F>
+__device__ uint64_t radix_kth(F elem, uint32_t n, uint32_t rank, SelectShared& sh) {
+  const int tid = threadIdx.x;
+  if (tid == 0) {
+    sh.prefix = 0;
+    sh.rank = rank;  // rank inside the current bucket
+  }
+  __syncthreads();
+  for (int shift = 56; shift >= 0; shift -= 8) {
+    if (tid < 256) sh.hist[tid] = 0;
+    __syncthreads();
+    const uint64_t prefix = sh.prefix;
+    const uint64_t mask = shift == 56 ? 0ull : (~0ull << (shift + 8));
+    for (uint32_t i = tid; i < n; i += SELECT_THREADS) {
+      const uint64_t key = elem(i);
+      if ((key & mask) == prefix) atomicAdd(&sh.hist[(uint32_t)(key >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    if (tid < 64) {
+      // wave 0: lane l owns bins 4l..4l+3; counts of all higher bins through a suffix sum over the lanes
+      const uint32_t h0 = sh.hist[4 * tid], h1 = sh.hist[4 * tid + 1], h2 = sh.hist[4 * tid + 2],
+                     h3 = sh.hist[4 * tid + 3];
+      const uint32_t own = h0 + h1 + h2 + h3;
+      uint32_t incl = own;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t o = __shfl_down(incl, d);
+        if (tid + d < 64) incl += o;
+      }
+      const uint32_t above = incl - own;
+      const uint32_t r = sh.rank;
+      if (above < r && r <= incl) {  // true for exactly one lane
+        uint32_t rr = r - above;
+        int d;
+        if (h3 >= rr) {
+          d = 3;
+        } else if (h3 + h2 >= rr) {
+          d = 2;
+          rr -= h3;
+        } else if (h3 + h2 + h1 >= rr) {
+          d = 1;
+          rr -= h3 + h2;
+        } else {
+          d = 0;
+          rr -= h3 + h2 + h1;
+        }
+        sh.rank = rr;
+        sh.prefix = prefix | ((uint64_t)(4 * tid + d) << shift);
+      }
+    }
+    __syncthreads();
+  }
+  const uint64_t kth = sh.prefix;
+  __syncthreads();  // the next call resets prefix and rank
+  return kth;
+}
+
+// Merges each query's candidate list into its running top-k.  A long list (a pass without a threshold
+// leaves one entry per row) is first cut down in place: the k-th largest of a strided sample of it is a
+// lower bound of the k-th largest overall, and only entries at or above that bound stay.
+__global__ __launch_bounds__(SELECT_THREADS) void scan_select_kernel(SelectArgs a) {
+  __shared__ SelectShared sh;
 
   const int q = blockIdx.x;
   const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
   const int k = a.k;
   uint64_t* top = a.top + (int64_t)q * k;
-  const uint64_t* cand = a.cand + (int64_t)q * a.cand_cap;
+  uint64_t* cand = a.cand + (int64_t)q * a.cand_cap;
   const uint32_t ntop = a.top_count[q];
   uint32_t ncand = a.cand_count[q];
   if ((int64_t)ncand > a.cand_cap) ncand = (uint32_t)a.cand_cap;
-  const uint32_t total = ntop + ncand;
   if (ncand == 0) return;  // nothing new for this query
 
+  if (ncand >= SELECT_PRESELECT_MIN) {
+    const uint32_t step = ncand / SELECT_SAMPLE;
+    const uint64_t bound =
+        radix_kth([&](uint32_t i) -> uint64_t { return cand[(uint64_t)i * step]; }, SELECT_SAMPLE, (uint32_t)k, sh);
+    // order-preserving compaction in place: a step reads SELECT_COMPACT_U * SELECT_THREADS entries, and writes
+    // its survivors only after every thread has read, at positions no later step reads from
+    constexpr int NW = SELECT_THREADS / 64;
+    constexpr uint32_t STEP = SELECT_COMPACT_U * SELECT_THREADS;
+    uint32_t w_base = 0;
+    for (uint32_t base = 0; base < ncand; base += STEP) {
+      uint64_t key[SELECT_COMPACT_U];
+      uint32_t lane_off[SELECT_COMPACT_U];
+      bool keep[SELECT_COMPACT_U];
+#pragma unroll
+      for (int j = 0; j < SELECT_COMPACT_U; ++j) {
+        const uint32_t i = base + j * SELECT_THREADS + tid;
+        key[j] = i < ncand ? cand[i] : 0ull;
+      }
+#pragma unroll
+      for (int j = 0; j < SELECT_COMPACT_U; ++j) {
+        const uint32_t i = base + j * SELECT_THREADS + tid;
+        keep[j] = i < ncand && key[j] >= bound;
+        const uint64_t ballot = __ballot(keep[j]);
+        lane_off[j] = __popcll(ballot & ((1ull << lane) - 1ull));
+        if (lane == 0) sh.part[j * NW + wave] = __popcll(ballot);
+      }
+      __syncthreads();
+      if (tid < 64) {
+        // exclusive prefix over the SELECT_COMPACT_U * NW = 64 counts, in (sub-block, wave) order
+        const uint32_t own = sh.part[tid];
+        uint32_t incl = own;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const uint32_t o = __shfl_up(incl, d);
+          if (tid >= d) incl += o;
+        }
+        sh.part[tid] = incl - own;
+        if (tid == 63) sh.part[64] = incl;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < SELECT_COMPACT_U; ++j)
+        if (keep[j]) cand[w_base + sh.part[j * NW + wave] + lane_off[j]] = key[j];
+      w_base += sh.part[64];
+      __syncthreads();
+    }
+    __threadfence_block();
+    __syncthreads();
+    ncand = w_base;
+  }
+  static_assert(SELECT_COMPACT_U * SELECT_THREADS / 64 == 64, "the compaction's offsets are one wave's prefix sum");
+
+  const uint32_t total = ntop + ncand;
   auto elem = [&](uint32_t i) -> uint64_t { return i < ntop ? top[i] : cand[i - ntop]; };
 
   uint64_t kth = 0;  // keep keys >= kth
-  if (total > (uint32_t)k) {
-    // radix select of the k-th largest key, 8 bits per pass from the top
-    if (tid == 0) {
-      s_prefix = 0;
-      s_rank = (uint32_t)k;  // rank (1-based, from the largest) inside the current bucket
-    }
-    __syncthreads();
-    for (int shift = 56; shift >= 0; shift -= 8) {
-      hist[tid] = 0;
-      __syncthreads();
-      const uint64_t prefix = s_prefix;
-      const uint64_t mask = shift == 56 ? 0ull : (~0ull << (shift + 8));
-      for (uint32_t i = tid; i < total; i += 256) {
-        const uint64_t key = elem(i);
-        if ((key & mask) == prefix) atomicAdd(&hist[(uint32_t)(key >> shift) & 255u], 1u);
-      }
-      __syncthreads();
-      if (tid == 0) {
-        uint32_t rank = s_rank;
-        int d = 255;
-        for (; d > 0; --d) {
-          if (hist[d] >= rank) break;
-          rank -= hist[d];
-        }
-        s_rank = rank;
-        s_prefix = prefix | ((uint64_t)d << shift);
-      }
-      __syncthreads();
-    }
-    kth = s_prefix;
-  }
+  if (total > (uint32_t)k) kth = radix_kth(elem, total, (uint32_t)k, sh);
 
-  if (tid == 0) s_fill = 0;
+  if (tid == 0) sh.fill = 0;
   __syncthreads();
-  for (uint32_t i = tid; i < total; i += 256) {
+  for (uint32_t i = tid; i < total; i += SELECT_THREADS) {
     const uint64_t key = elem(i);
     if (key >= kth) {
-      const uint32_t pos = atomicAdd(&s_fill, 1u);
-      if (pos < SCAN_KMAX) keys[pos] = key;
+      const uint32_t pos = atomicAdd(&sh.fill, 1u);
+      if (pos < SCAN_KMAX) sh.keys[pos] = key;
     }
   }
   __syncthreads();
-  const uint32_t kept = min(s_fill, (uint32_t)k);
+  const uint32_t kept = min(sh.fill, (uint32_t)k);
   // bitonic sort, descending, padded with zeros (below every real key)
   uint32_t n2 = 1;
   while (n2 < kept) n2 <<= 1;
-  for (uint32_t i = kept + tid; i < n2; i += 256) keys[i] = 0;
+  for (uint32_t i = kept + tid; i < n2; i += SELECT_THREADS) sh.keys[i] = 0;
   __syncthreads();
   for (uint32_t size = 2; size <= n2; size <<= 1) {
     for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
-      for (uint32_t i = tid; i < n2 / 2; i += 256) {
+      for (uint32_t i = tid; i < n2 / 2; i += SELECT_THREADS) {
         const uint32_t lo = 2 * i - (i & (stride - 1));
         const uint32_t hi = lo + stride;
         const bool desc = (lo & size) == 0;
-        const uint64_t x = keys[lo], y = keys[hi];
+        const uint64_t x = sh.keys[lo], y = sh.keys[hi];
         if ((x < y) == desc) {
-          keys[lo] = y;
-          keys[hi] = x;
+          sh.keys[lo] = y;
+          sh.keys[hi] = x;
         }
       }
       __syncthreads();
     }
   }
-  for (uint32_t i = tid; i < kept; i += 256) top[i] = keys[i];
+  for (uint32_t i = tid; i < kept; i += SELECT_THREADS) top[i] = sh.keys[i];
   if (tid == 0) {
     a.top_count[q] = kept;
     a.cand_count[q] = 0;
-    if (kept == (uint32_t)k) a.thr[q] = ordered_f32((uint32_t)(keys[k - 1] >> 32));
+    if (kept == (uint32_t)k) a.thr[q] = ordered_f32((uint32_t)(sh.keys[k - 1] >> 32));
   }
 }
 
@@ -459,6 +700,49 @@ size_t scan_workspace_bytes(int Q, int k, int64_t chunk_rows) {
   return scan_layout(Q, k, effective_chunk(chunk_rows, Q)).total;
 }
 
+// Bytes of the query fragment table of the streaming kernel (1 KB per k-step and block of 16 queries), or 0
+// where that kernel does not apply: more than 32 queries, a row length that is no multiple of two k-steps.
+static size_t query_table_bytes(int Q, int64_t D, int dtype) {
+  if (Q <= 0 || Q > 32) return 0;
+  const int kstep = dtype == BGX_F32 ? 16 : 32;
+  if (D <= 0 || D % (2 * kstep) != 0) return 0;
+  return (size_t)((Q + 15) / 16) * (size_t)(D / kstep) * 1024;
+}
+
+size_t scan_workspace_bytes_for(int Q, int k, int64_t chunk_rows, int64_t D, int dtype) {
+  const size_t base = scan_workspace_bytes(Q, k, chunk_rows);
+  return align_up(std::max<size_t>(base, 256), 256) + query_table_bytes(Q, D, dtype);
+}
+
+template <typename T>
+static int launch_stream(const ScanArgs& a, int blocks, const uint4* table, int wgs, hipStream_t st) {
+  // stage slots, score blocks (pitch 16 * blocks + 1 floats), row multipliers
+  const size_t smem = 4 * Stream<SS_MTW>::BYTES_PER_WAVE +
+                      4 * SS_WAVE_ROWS * (size_t)(16 * blocks + 1) * sizeof(float) + 4 * SS_WAVE_ROWS * sizeof(float);
+  if (blocks == 1) {
+    auto kern = scan_stream_kernel<T, 1>;
+    BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(COLLECT_THREADS), smem, st, a, table);
+  } else {
+    auto kern = scan_stream_kernel<T, 2>;
+    BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(COLLECT_THREADS), smem, st, a, table);
+  }
+  BGX_HIP(hipGetLastError());
+  return 0;
+}
+
+template <typename T>
+static int launch_query_fragments(const void* queries, int Q, int64_t D, uint4* table, hipStream_t st) {
+  const int blocks = (Q + 15) / 16;
+  const int64_t steps = D / Mma<T>::KS;
+  const dim3 grid((unsigned)((steps + 4 * STAGE_B - 1) / (4 * STAGE_B)), (unsigned)blocks);
+  hipLaunchKernelGGL(scan_query_fragments_kernel<T>, grid, dim3(COLLECT_THREADS), 0, st, (const T*)queries, Q, D, blocks,
+                     table);
+  BGX_HIP(hipGetLastError());
+  return 0;
+}
+
 template <typename T, int BM, int BN, int WM, int WN, bool ALIGNED, int PF, bool STREAM>
 static int launch_gemm_v(const ScanArgs& a, hipStream_t st) {
   constexpr int NT = WM * WN * 64;
@@ -532,6 +816,7 @@ int gemm_scores(const void* rows, int64_t n_rows, int64_t D, int64_t stride, int
   a.cand_count = nullptr;
   a.cand = nullptr;
   a.cand_cap = 0;
+  a.first_pass = 0;
   const int epl = dtype == BGX_F32 ? 4 : 8;
   const bool aligned = ((uintptr_t)rows % 16 == 0) && ((uintptr_t)queries % 16 == 0) && (D % epl == 0) &&
                        (stride % epl == 0);
@@ -591,6 +876,26 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
                        (stride % epl == 0);
   (void)esz;
 
+  // Few queries and a pass large enough to give every CU several tiles: the streaming kernel, if the
+  // workspace has room for its query fragment table (bgx_scan_workspace_bytes_for).
+  const size_t table_bytes = query_table_bytes(Q, D, dtype);
+  const size_t table_off = align_up(std::max<size_t>(lay.total, 256), 256);
+  int cus = 0;
+  {
+    int dev = 0;
+    BGX_HIP(hipGetDevice(&dev));
+    BGX_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  }
+  const bool stream_ok = table_bytes > 0 && aligned && ws != nullptr && ((uintptr_t)ws & 255) == 0 &&
+                         ws_bytes >= table_off + table_bytes && getenv("BGX_SCAN_STREAM_OFF") == nullptr;
+  // With top-k the streaming scan opens with one tile per workgroup and no thresholds (the select kernel
+  // cuts that pass's one-entry-per-row lists down); every later pass is as long as the workspace allows.
+  const int64_t stream_first = (int64_t)std::max(cus, 1) * SS_TILE_ROWS;
+  const int64_t stream_min_rows = 2 * stream_first;
+  const bool stream_scan = stream_ok && n_rows >= stream_min_rows && chunk >= stream_first;
+  uint4* qtable = stream_ok ? (uint4*)((char*)ws + table_off) : nullptr;
+  bool table_built = false;
+
   int64_t done = 0;
   while (done < n_rows) {
     int64_t rows = n_rows - done;
@@ -598,6 +903,7 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
       // the first pass has no threshold yet and appends every score: each query's list grows by one
       // serialised atomic per row, so that pass stays small and later passes grow fourfold
       int64_t lim = done == 0 ? SCAN_FIRST_CHUNK : done * 4;
+      if (stream_scan) lim = done == 0 ? stream_first : chunk;
       if (lim < k) lim = k;
       if (lim > chunk) lim = chunk;
       if (rows > lim) rows = lim;
@@ -624,8 +930,26 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
     a.cand_count = cand_count;
     a.cand = cand;
     a.cand_cap = chunk;
+    a.first_pass = 0;
     int rc;
-    if (dtype == BGX_F16)
+    if (stream_scan && rows >= 16 * SS_TILE_ROWS) {
+      a.first_pass = want_topk && done == 0;
+      if (!table_built) {
+        rc = dtype == BGX_F16    ? launch_query_fragments<f16_t>(queries, Q, D, qtable, st)
+             : dtype == BGX_BF16 ? launch_query_fragments<bf16_t>(queries, Q, D, qtable, st)
+                                 : launch_query_fragments<float>(queries, Q, D, qtable, st);
+        if (rc != 0) return rc;
+        table_built = true;
+      }
+      a.row_tiles = (int)((rows + SS_TILE_ROWS - 1) / SS_TILE_ROWS);
+      a.q_tiles = 1;
+      a.n_parts = 1;
+      const int wgs = (int)std::min<int64_t>(std::max(cus, 1), a.row_tiles);
+      const int blocks = (Q + 15) / 16;
+      rc = dtype == BGX_F16    ? launch_stream<f16_t>(a, blocks, qtable, wgs, st)
+           : dtype == BGX_BF16 ? launch_stream<bf16_t>(a, blocks, qtable, wgs, st)
+                               : launch_stream<float>(a, blocks, qtable, wgs, st);
+    } else if (dtype == BGX_F16)
       rc = launch_gemm_t<f16_t>(a, aligned, st);
     else if (dtype == BGX_BF16)
       rc = launch_gemm_t<bf16_t>(a, aligned, st);
@@ -646,7 +970,7 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
       s.thr = thr;
       s.cand_cap = chunk;
       s.k = k;
-      hipLaunchKernelGGL(scan_select_kernel, dim3((unsigned)Q), dim3(256), 0, st, s);
+      hipLaunchKernelGGL(scan_select_kernel, dim3((unsigned)Q), dim3(SELECT_THREADS), 0, st, s);
       BGX_HIP(hipGetLastError());
     }
     done += rows;

@@ -14,10 +14,12 @@ namespace bgx {
 constexpr int COLLECT_THREADS = 256;  // the workgroup size these helpers are written for (4 waves)
 constexpr int STAGE_B = 6;            // fragments a thread keeps in flight while staging a projection
 
-// k-steps [ks0, ks1) of the matrix; the whole of it by default
+// k-steps [ks0, ks1) of the matrix; the whole of it by default.  The fragment of k-step ks goes to
+// dst[(ks * nblk + blk) * 64 + lane]: nblk matrices of 16 rows interleaved per k-step (one by default).
 template <typename T>
 __device__ inline void stage_projection(const T* __restrict__ R, const float* __restrict__ scale, int K, int p,
-                                        uint4* __restrict__ dst, int tid, int ks0 = 0, int ks1 = -1) {
+                                        uint4* __restrict__ dst, int tid, int ks0 = 0, int ks1 = -1, int blk = 0,
+                                        int nblk = 1) {
   using M = Mma<T>;
   const int nfrag = (ks1 < 0 ? K / M::KS : min(ks1, K / M::KS)) * WAVE;
   constexpr int B = STAGE_B;  // fragments per thread in flight
@@ -44,7 +46,7 @@ __device__ inline void stage_projection(const T* __restrict__ R, const float* __
         for (int e = 0; e < M::EPL; ++e)
           M::set(v[b], e, M::get(v[b], e) * __uint_as_float((&s4[b][e >> 2].x)[e & 3]));
       }
-      if (f < nfrag) dst[f] = v[b];
+      if (f < nfrag) dst[((f >> 6) * nblk + blk) * WAVE + (f & 63)] = v[b];
     }
   }
 }

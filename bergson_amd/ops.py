@@ -573,8 +573,8 @@ def scan(store: Tensor, queries: Tensor, *, unit_norm: bool, k: int = 0, query_s
     if want_sumsq:
         res.sumsq = torch.empty((n,), dtype=torch.float32, device=dev)
     ws = None
-    if k or want_row_mean:
-        ws = _workspace(dev, lib.bgx_scan_workspace_bytes(Q, k, chunk_rows), "scan")
+    if k or want_row_mean or Q <= 32:  # few queries: the streaming kernel keeps its query fragments there
+        ws = _workspace(dev, lib.bgx_scan_workspace_bytes_for(Q, k, chunk_rows, D, dtype_code(store.dtype)), "scan")
     rc = lib.bgx_scan(_ptr(store), n, D, store.stride(0), dtype_code(store.dtype), _ptr(queries), Q, query_scale,
                       int(unit_norm), k, row_base, _ptr(res.topk_values), _ptr(res.topk_indices), _ptr(res.row_max),
                       _ptr(res.row_mean), _ptr(res.scores), _ptr(res.sumsq), _ptr(ws), 0 if ws is None else ws.numel(), chunk_rows,

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define BGX_ABI_VERSION 4
+#define BGX_ABI_VERSION 5
 
 enum bgx_dtype { BGX_F32 = 0, BGX_F16 = 1, BGX_BF16 = 2 };
 
@@ -250,6 +250,15 @@ int bgx_unit_normalize_rows(void* rows_dev, int64_t n_rows, int64_t D,
 /* Bytes of device workspace bgx_scan needs for Q queries, top-k of k and at
  * most chunk_rows store rows per internal pass (0 = library default). */
 size_t bgx_scan_workspace_bytes(int32_t Q, int32_t k, int64_t chunk_rows);
+/* The same plus room for a table of the queries as matrix-core fragments
+ * (1 KB per block of 16 queries and k-step: 32 elements of D at 16 bits, 16 at
+ * fp32): with it, scans with at most 32 queries over at least 512 rows per
+ * compute unit, D a multiple of two k-steps, stream the store with the
+ * few-queries kernel; without it they use the tiled kernel.  A workspace is then needed
+ * even when neither top-k nor row means are asked for.  bgx_scan accepts
+ * either size. */
+size_t bgx_scan_workspace_bytes_for(int32_t Q, int32_t k, int64_t chunk_rows,
+                                    int64_t D, int32_t dtype);
 
 /* Scores n_rows store rows [n_rows, D] (row stride in elements) against Q
  * queries [Q, D] of the same dtype, streaming the store once.

@@ -24,7 +24,7 @@ def test_header_symbols_are_exported_and_bound():
     for n in names:
         assert hasattr(lib, n), f"{n} is declared in the header but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes bindings and header disagree"
-    assert lib.bgx_abi_version() == _lib.ABI_VERSION == 4
+    assert lib.bgx_abi_version() == _lib.ABI_VERSION == 5
 
 
 def test_module_desc_layout_matches_header():
@@ -77,6 +77,13 @@ def test_workspace_sizes():
     small = lib.bgx_scan_workspace_bytes(8, 10, 1024)
     assert small >= 8 * 10 * 8 + 8 * 1024 * 8
     assert lib.bgx_scan_workspace_bytes(1024, 100, 0) >= 1024 * 65536 * 8
+    # the few-queries kernel's table: 1 KB per block of 16 queries and k-step (32 elements at 16 bits, 16 at fp32)
+    base = lib.bgx_scan_workspace_bytes(20, 100, 0)
+    padded = -(-base // 256) * 256
+    assert lib.bgx_scan_workspace_bytes_for(20, 100, 0, 12288, 1) == padded + 2 * (12288 // 32) * 1024
+    assert lib.bgx_scan_workspace_bytes_for(20, 100, 0, 12288, 0) == padded + 2 * (12288 // 16) * 1024
+    assert lib.bgx_scan_workspace_bytes_for(33, 100, 0, 12288, 1) == -(-lib.bgx_scan_workspace_bytes(33, 100, 0) // 256) * 256
+    assert lib.bgx_scan_workspace_bytes_for(20, 100, 0, 12288 + 32, 1) == padded   # not two k-steps: no table
 
 
 def test_argument_errors_before_any_launch():

@@ -177,3 +177,103 @@ def test_scan_row_mean_alone(device, Q):
     torch.cuda.synchronize()
     assert res.topk_values is None
     assert (res.row_mean.cpu() - ref.mean(1)).abs().max().item() <= COS_TOL
+
+
+# ---- few queries over a long store: the streaming kernel ------------------------------------------------
+# At most 32 queries, a row length that is a multiple of two MFMA k-steps and at least two tiles of 256 rows
+# per compute unit route the scan through the streaming kernel: a first pass of one tile per compute unit
+# without thresholds (one candidate per row, cut down by the select kernel's sample bound), then the rest.
+STREAM_ROWS = 2 * 256 * 256 + 9001  # past the minimum, with a ragged last tile
+
+
+@pytest.mark.parametrize("dtype,D,Q", [(torch.float16, 128, 5), (torch.float16, 320, 32), (torch.bfloat16, 192, 16),
+                                       (torch.bfloat16, 64, 23), (torch.float32, 96, 8), (torch.float32, 32, 32)])
+def test_scan_streamed_few_queries(device, dtype, D, Q):
+    from bergson_amd import ops
+
+    n, k = STREAM_ROWS, 100
+    store, queries = make_store(n, D, Q, dtype, seed=D + Q)
+    store[12345] = 0  # a zero row scores 0 under unit norms
+    qd = unit_queries(queries, dtype).to(dtype)
+    ref = oscan.scorer_score({"m": store}, {"m": qd}, ["m"], dtype=torch.float32, unit_normalize=True).T  # [Q, n]
+    dev_store, dev_q = store.to(device), qd.to(device)
+    res = ops.scan(dev_store, dev_q, unit_norm=True, k=k, want_row_max=True, want_row_mean=True, want_scores=True,
+                   want_sumsq=True)
+    torch.cuda.synchronize()
+    assert (res.scores.cpu().T - ref).abs().max().item() <= COS_TOL
+    assert res.scores[12345].abs().max().item() == 0
+    assert (res.row_mean.cpu() - ref.mean(0)).abs().max().item() <= COS_TOL
+    assert torch.allclose(res.sumsq.cpu(), store.float().pow(2).sum(1), rtol=1e-4)
+    assert (res.row_max.cpu() - ref.max(0).values).abs().max().item() <= COS_TOL
+    check_topk(res.topk_values.cpu(), res.topk_indices.cpu(), ref, k)
+    # the tile kernel on the same inputs (passes too short for the streaming kernel) selects the same rows
+    tiled = ops.scan(dev_store, dev_q, unit_norm=True, k=k, want_row_mean=True, chunk_rows=65536 - 256)
+    torch.cuda.synchronize()
+    check_topk(tiled.topk_values.cpu(), tiled.topk_indices.cpu(), ref, k)
+    same = (tiled.topk_indices == res.topk_indices)
+    assert (tiled.topk_values[same] - res.topk_values[same]).abs().max().item() <= 1e-5
+    assert (tiled.row_mean - res.row_mean).abs().max().item() <= 1e-5
+
+
+def test_scan_streamed_passes_and_short_tail(device):
+    """Passes of exactly one tile per compute unit, then a tail too short for the streaming kernel."""
+    from bergson_amd import ops
+
+    n, D, Q, k = 2 * 65536 + 100, 128, 12, 300
+    store, queries = make_store(n, D, Q, torch.float16, seed=3)
+    store[-50:] *= 3.0
+    ref = queries.to(torch.float16).float() @ store.float().T  # raw inner products
+    res = ops.scan(store.to(device), queries.to(torch.float16).to(device), unit_norm=False, k=k, chunk_rows=65536,
+                   want_row_mean=True)
+    torch.cuda.synchronize()
+    rv, ri = torch.topk(ref, k, dim=1)
+    scale = ref.abs().max().item()
+    assert (res.topk_values.cpu() - rv).abs().max().item() <= 2e-3 * scale
+    agree = (res.topk_indices.cpu() == ri).float().mean().item()
+    assert agree > 0.99  # rows may swap only where scores agree to rounding
+    assert (res.row_mean.cpu() - ref.mean(0)).abs().max().item() <= 2e-3 * scale
+
+
+def test_scan_streamed_without_topk(device):
+    from bergson_amd import ops
+
+    n, D, Q = STREAM_ROWS, 64, 9
+    store, queries = make_store(n, D, Q, torch.bfloat16, seed=21)
+    qd = unit_queries(queries, torch.bfloat16).to(torch.bfloat16)
+    ref = oscan.scorer_score({"m": store}, {"m": qd}, ["m"], dtype=torch.float32, unit_normalize=True)  # [n, Q]
+    res = ops.scan(store.to(device), qd.to(device), unit_norm=True, want_row_mean=True, want_row_max=True)
+    torch.cuda.synchronize()
+    assert res.topk_values is None
+    assert (res.row_mean.cpu() - ref.mean(1)).abs().max().item() <= COS_TOL
+    assert (res.row_max.cpu() - ref.max(1).values).abs().max().item() <= COS_TOL
+
+
+def test_scan_streamed_ties_pick_lowest_rows(device):
+    """Every row the same: every candidate of the first pass survives the sample bound's score, and the order
+    among equal scores is by row number."""
+    from bergson_amd import ops
+
+    row = torch.randn(64, generator=torch.Generator().manual_seed(2))
+    store = row.repeat(STREAM_ROWS, 1).to(torch.float16)
+    res = ops.scan(store.to(device), row[None].to(torch.float16).to(device), unit_norm=True, k=150)
+    torch.cuda.synchronize()
+    assert res.topk_indices.cpu()[0].tolist() == list(range(150))
+
+
+def test_scan_streamed_best_rows_last(device):
+    """Scores that grow with the row number: the threshold of each pass is met by every later row."""
+    from bergson_amd import ops
+
+    n, D, k = STREAM_ROWS, 64, 64
+    gen = torch.Generator().manual_seed(8)
+    q = torch.randn(D, generator=gen)
+    q = q / q.norm()
+    ramp = torch.linspace(0.1, 4.0, n)[:, None]
+    store = (q[None] * ramp + 0.01 * torch.randn(n, D, generator=gen)).to(torch.float16)
+    qd = q[None].to(torch.float16)
+    ref = qd.float() @ store.float().T
+    res = ops.scan(store.to(device), qd.to(device), unit_norm=False, k=k)
+    torch.cuda.synchronize()
+    rv, ri = torch.topk(ref, k, dim=1)
+    assert torch.allclose(res.topk_values.cpu(), rv, rtol=1e-3, atol=1e-3)
+    assert len(set(res.topk_indices.cpu()[0].tolist()) & set(ri[0].tolist())) >= k - 2
