@@ -74,6 +74,8 @@ struct ScanArgs {
   uint64_t* cand;        // [Q][cand_cap]
   int64_t cand_cap;
   int first_pass;        // streaming kernel, no thresholds yet: row r of the pass is entry r of every query's list
+  int units_per_wave;    // streaming kernel: 16-row units per wave of the grid, the first units_rem waves one more
+  int units_rem;
 };
 
 // Workgroup tile BM x BN, WM x WN waves, each wave (BM/WM) x (BN/WN) as 32x32 MFMA blocks.
@@ -327,45 +329,66 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void scan_stream_kernel(ScanArg
 
   const T* store = (const T*)args.store + args.row0 * args.store_stride;
   const int nkp = (int)(args.D / (2 * M::KS));
-  const int64_t n_tiles = (args.rows + SS_TILE_ROWS - 1) / SS_TILE_ROWS;
-  const int64_t t_first = n_tiles * blockIdx.x / gridDim.x;
-  const int64_t t_last = n_tiles * (blockIdx.x + 1) / gridDim.x;
+  // Rows are dealt to the waves of the grid in units of 16, as evenly as those allow; a wave walks its
+  // stretch 64 rows at a time and its last step may be shorter.
+  const int gw = blockIdx.x * 4 + wave;
+  const int64_t r_first = ((int64_t)gw * args.units_per_wave + min(gw, args.units_rem)) * 16;
+  const int64_t r_last =
+      min(args.rows, r_first + ((int64_t)args.units_per_wave + (gw < args.units_rem ? 1 : 0)) * 16);
+  const int n_steps = (int)((r_last - r_first + SS_WAVE_ROWS - 1) / SS_WAVE_ROWS);
 
   if (args.first_pass && blockIdx.x == 0 && tid < args.Q) args.cand_count[tid] = (uint32_t)args.rows;
 
+  // Every wave walks D from its own starting k-pair (a multiple of the queue length) and wraps around: at any
+  // moment the waves of the chip then read different parts of the query table, whose 4 KB stretches would
+  // otherwise each be wanted by every wave at once.  A step is two segments, [rot, nkp) and [0, rot).
+  const int nblk = nkp / STREAM_Q;
+  const int rot = nblk >= 2 ? (int)(((unsigned)gw * 7u) % (unsigned)nblk) * STREAM_Q : 0;
+  const int nseg = rot > 0 ? 2 : 1;
+  constexpr int KP = 2 * M::KS;        // elements of a k-pair
+  constexpr int FP = 2 * QB * WAVE;    // table entries of a k-pair
+
   uint4 v[STREAM_Q][RG];
   uint4 rq[STREAM_Q][2 * QB];
+  f32x4 acc[SS_MTW * QB];
+  float ssq[RG];
   bool primed = false;
-  for (int64_t tile = t_first; tile < t_last; ++tile) {
-    const int64_t prow0 = tile * SS_TILE_ROWS + wave * SS_WAVE_ROWS;  // pass-local first row of this wave
-    const int rows_valid = (int)min((int64_t)SS_WAVE_ROWS, args.rows - prow0);
-    if (rows_valid <= 0) {
-      primed = false;
-      continue;
-    }
+  for (int item = 0; item < n_steps * nseg; ++item) {
+    const int step = item / nseg;
+    const int sg = item - step * nseg;
+    const int64_t prow0 = r_first + (int64_t)step * SS_WAVE_ROWS;  // pass-local first row of this step
+    const int rows_valid = (int)min((int64_t)SS_WAVE_ROWS, r_last - prow0);
+    const int k0 = sg == 0 ? rot : 0;
+    const int len = nseg == 1 ? nkp : (sg == 0 ? nkp - rot : rot);
     const T* ur[RG];
     const T* un[RG];
-    stream_rows<T, SS_MTW>(store + prow0 * args.store_stride, args.store_stride, rows_valid, lane, ur);
-    if (!primed) stream_prime<T, SS_MTW, true, QB>(ur, nkp, qfrag, lane, v, rq);
-    int nkp_next = 0;
+    stream_rows<T, SS_MTW>(store + prow0 * args.store_stride + k0 * KP, args.store_stride, rows_valid, lane, ur);
+    if (!primed) stream_prime<T, SS_MTW, true, QB>(ur, len, qfrag + k0 * FP, lane, v, rq);
+    int len_next = 0;
+    int k1 = 0;
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg) un[rg] = ur[rg];
-    if (tile + 1 < t_last) {
-      const int64_t prow1 = prow0 + SS_TILE_ROWS;
-      const int rows1 = (int)min((int64_t)SS_WAVE_ROWS, args.rows - prow1);
-      if (rows1 > 0) {
-        stream_rows<T, SS_MTW>(store + prow1 * args.store_stride, args.store_stride, rows1, lane, un);
-        nkp_next = nkp;
-      }
+    if (sg + 1 < nseg) {
+      // the same rows from k-pair 0
+      stream_rows<T, SS_MTW>(store + prow0 * args.store_stride, args.store_stride, rows_valid, lane, un);
+      len_next = rot;
+    } else if (step + 1 < n_steps) {
+      const int64_t prow1 = prow0 + SS_WAVE_ROWS;
+      const int rows1 = (int)min((int64_t)SS_WAVE_ROWS, r_last - prow1);
+      k1 = rot;
+      stream_rows<T, SS_MTW>(store + prow1 * args.store_stride + k1 * KP, args.store_stride, rows1, lane, un);
+      len_next = nkp - rot;
     }
-    f32x4 acc[SS_MTW * QB];
+    if (sg == 0) {
 #pragma unroll
-    for (int i = 0; i < SS_MTW * QB; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float ssq[RG];
+      for (int i = 0; i < SS_MTW * QB; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int rg = 0; rg < RG; ++rg) ssq[rg] = 0.f;
-    stream_segment<T, SS_MTW, true, QB, true>(ur, nkp, un, nkp_next, qfrag, qfrag, stage, lane, v, rq, acc, ssq);
-    primed = nkp_next > 0;
+      for (int rg = 0; rg < RG; ++rg) ssq[rg] = 0.f;
+    }
+    stream_segment<T, SS_MTW, true, QB, true>(ur, len, un, len_next, qfrag + k0 * FP, qfrag + k1 * FP, stage, lane, v, rq,
+                                              acc, ssq);
+    primed = len_next > 0;
+    if (sg + 1 < nseg) continue;
 
     // ---- row norms: lane (rho, sig) carried slot sig of row rg * 8 + rho; a row's 8 lanes add up ----
     __builtin_amdgcn_wave_barrier();
@@ -817,6 +840,8 @@ int gemm_scores(const void* rows, int64_t n_rows, int64_t D, int64_t stride, int
   a.cand = nullptr;
   a.cand_cap = 0;
   a.first_pass = 0;
+  a.units_per_wave = 0;
+  a.units_rem = 0;
   const int epl = dtype == BGX_F32 ? 4 : 8;
   const bool aligned = ((uintptr_t)rows % 16 == 0) && ((uintptr_t)queries % 16 == 0) && (D % epl == 0) &&
                        (stride % epl == 0);
@@ -931,6 +956,8 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
     a.cand = cand;
     a.cand_cap = chunk;
     a.first_pass = 0;
+    a.units_per_wave = 0;
+    a.units_rem = 0;
     int rc;
     if (stream_scan && rows >= 16 * SS_TILE_ROWS) {
       a.first_pass = want_topk && done == 0;
@@ -945,6 +972,9 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
       a.q_tiles = 1;
       a.n_parts = 1;
       const int wgs = (int)std::min<int64_t>(std::max(cus, 1), a.row_tiles);
+      const int64_t units = (rows + 15) / 16;
+      a.units_per_wave = (int)(units / (4 * wgs));
+      a.units_rem = (int)(units % (4 * wgs));
       const int blocks = (Q + 15) / 16;
       rc = dtype == BGX_F16    ? launch_stream<f16_t>(a, blocks, qtable, wgs, st)
            : dtype == BGX_BF16 ? launch_stream<bf16_t>(a, blocks, qtable, wgs, st)
