@@ -39,7 +39,7 @@ HBM_PEAK_GBS = 8000.0
 COLLECT_TRAFFIC_RATIO = 1.036
 # the same for the store scan: 1024 queries (four query tiles re-read each row tile, half from L2), at most 32 queries
 SCAN_TRAFFIC_RATIO_Q1024 = 1.51
-SCAN_TRAFFIC_RATIO_FEW = 1.005
+SCAN_TRAFFIC_RATIO_FEW = 1.0016
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
