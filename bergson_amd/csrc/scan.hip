@@ -78,6 +78,65 @@ struct ScanArgs {
   int units_rem;
 };
 
+// Epilogue of a workgroup tile whose waves hold (TM x TN) blocks of 32 x 32 scores in MFMA layout: scale by the
+// row multipliers s_inv, then dense scores, row maxima, row-sum partials and the threshold filter.
+template <int TM, int TN, int WTM, int WTN, int WN>
+__device__ inline void scan_tile_epilogue(const ScanArgs& args, f32x16 (&acc)[TM][TN], const float* s_inv, int wm,
+                                          int wn, int fr, int fh, int64_t g_row0, int64_t q_row0, int qt,
+                                          int block_rot = 0) {
+  float thr[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int64_t q = q_row0 + wn * WTN + j * 32 + fr;
+    thr[j] = (args.thr != nullptr && q < args.Q) ? args.thr[q] : INFINITY;
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      // acc[i] is the wave's 32-row block (i + block_rot) mod TM
+      const int row = wm * WTM + ((i + block_rot) & (TM - 1)) * 32 + (e >> 2) * 8 + fh * 4 + (e & 3);
+      const int64_t prow = g_row0 + row;  // pass-local row
+      const bool row_ok = prow < args.rows;
+      const int64_t grow = args.row0 + prow;
+      const float w = s_inv[row];
+      float rmax = -INFINITY;
+      float rsum = 0.f;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int64_t q = q_row0 + wn * WTN + j * 32 + fr;
+        const float v = acc[i][j][e] * w;
+        if (row_ok && q < args.Q) {
+          rmax = fmaxf(rmax, v);
+          rsum += v;
+          if (args.scores != nullptr) args.scores[grow * args.Q + q] = v;
+          if (v > thr[j]) {
+            const uint32_t pos = atomicAdd(&args.cand_count[q], 1u);
+            if ((int64_t)pos < args.cand_cap) args.cand[q * args.cand_cap + pos] = make_key(v, (uint32_t)grow);
+          }
+        }
+      }
+      if (args.row_max_enc != nullptr) {
+        rmax = fmaxf(rmax, __shfl_xor(rmax, 1));
+        rmax = fmaxf(rmax, __shfl_xor(rmax, 2));
+        rmax = fmaxf(rmax, __shfl_xor(rmax, 4));
+        rmax = fmaxf(rmax, __shfl_xor(rmax, 8));
+        rmax = fmaxf(rmax, __shfl_xor(rmax, 16));
+        if (fr == 0 && row_ok) atomicMax(&args.row_max_enc[grow], f32_ordered(rmax));
+      }
+      if (args.row_sum_part != nullptr) {
+        // fixed-order butterfly over the 32 lanes that hold this row's scores; one writer per (row, part)
+        rsum += __shfl_xor(rsum, 1);
+        rsum += __shfl_xor(rsum, 2);
+        rsum += __shfl_xor(rsum, 4);
+        rsum += __shfl_xor(rsum, 8);
+        rsum += __shfl_xor(rsum, 16);
+        if (fr == 0 && row_ok) args.row_sum_part[prow * args.n_parts + qt * WN + wn] = rsum;
+      }
+    }
+  }
+}
+
 // Workgroup tile BM x BN, WM x WN waves, each wave (BM/WM) x (BN/WN) as 32x32 MFMA blocks.
 // PF = how many K tiles the global loads run ahead of the LDS stores (one register set per tile in flight);
 // STREAM = non-temporal loads of the store rows, for launches with one query tile, where every store line
@@ -231,57 +290,222 @@ __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
   }
   __syncthreads();
 
-  // ---- epilogue -----------------------------------------------------------------------
-  float thr[TN];
+  scan_tile_epilogue<TM, TN, WTM, WTN, WN>(args, acc, s_inv, wm, wn, fr, fh, g_row0, q_row0, qt);
+}
+
+// ---- many queries, 16-bit stores: tiles loaded straight into LDS ---------------------------------------
+// The 256 x 256 tile of the kernel above with 8 waves as 2 x 4, for aligned fp16 / bf16 operands whose D is a
+// multiple of 64.  What differs is how the tiles reach LDS and how the fragments leave it:
+//  * global_load_lds (16 bytes per lane, 1 KB per wave instruction) writes the K tiles into LDS without passing
+//    through registers: no staging registers, no ds_write, and the row sums of squares come from the A fragments
+//    each wave reads anyway (the four waves that share 128 rows take a 32-row block each);
+//  * rows are 128 bytes, unpadded; chunk c of row r sits at position c ^ (r & 7) ^ ((r >> 3) & 1), which the
+//    loader produces by permuting which global chunk each lane fetches: fragment reads are conflict-free;
+//  * three A buffers and two B buffers (160 KB): the store rows are fetched two K tiles ahead, the queries
+//    (L2-resident) one ahead; the per-tile wait is a vmcnt that leaves the youngest A tile in flight, and the
+//    barrier is the bare s_barrier -- __syncthreads would wait for every outstanding load;
+//  * the fragments are double-buffered in registers and the pipeline runs across the barrier: the reads of
+//    step 0 of the next tile are issued right after it, before the MFMAs of the last step of this tile.
+constexpr int SD_BM = 256, SD_BN = 256, SD_ROW = 128;
+constexpr int SD_A_BYTES = SD_BM * SD_ROW, SD_B_BYTES = SD_BN * SD_ROW;
+constexpr int SD_LDS_BYTES = 3 * SD_A_BYTES + 2 * SD_B_BYTES;
+constexpr int SD_THREADS = 512;
+
+__device__ inline int sd_key(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+// 16 bytes from LDS byte address `addr`; the caller waits (lgkmcnt) before it uses the value
+__device__ inline uint4 sd_lds_read16(uint32_t addr) {
+  uint4 v;
+  asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+  return v;
+}
+
+template <typename T>
+__global__ __launch_bounds__(SD_THREADS) void scan_direct_kernel(ScanArgs args) {
+  using M = Mma32<T>;
+  typedef __attribute__((address_space(1))) const void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
+  constexpr int BK = 64;  // elements of K per tile
+  constexpr int TM = 4, TN = 2, WTM = 128, WTN = 64, WN = 4;
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* s_inv = reinterpret_cast<float*>(smem);  // after the main loop: [SD_BM] row multipliers
+
+  const int b = blockIdx.x;
+  const int xcd = b & 7;
+  const int slot = b >> 3;
+  const int rt_local = slot / args.q_tiles;
+  const int qt = slot - rt_local * args.q_tiles;
+  const int rt = rt_local * 8 + xcd;
+  if (rt >= args.row_tiles) return;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 2, wn = wave & 3;
+  const int64_t g_row0 = (int64_t)rt * SD_BM;  // pass-local first row
+  const int64_t q_row0 = (int64_t)qt * SD_BN;
+  const int KT = (int)(args.D / BK);
+
+  // loader: instruction i of a wave fills rows i * 64 + wave * 8 .. + 7 of a tile; lane l is position l & 7 of
+  // row l >> 3 and fetches the chunk that belongs there.  Rows past the end repeat the last one (their scores
+  // are never written).
+  const T* aptr[4];
+  const T* bptr[4];
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int64_t q = q_row0 + wn * WTN + j * 32 + fr;
-    thr[j] = (args.thr != nullptr && q < args.Q) ? args.thr[q] : INFINITY;
+  for (int i = 0; i < 4; ++i) {
+    const int r = i * 64 + wave * 8 + (lane >> 3);
+    const int ch = (lane & 7) ^ sd_key(r);
+    const int64_t grow = min(g_row0 + r, args.rows - 1);
+    const int64_t qrow = min(q_row0 + r, (int64_t)args.Q - 1);
+    aptr[i] = (const T*)args.store + (args.row0 + grow) * args.store_stride + ch * 8;
+    bptr[i] = (const T*)args.queries + qrow * args.D + ch * 8;
   }
+  auto load_a = [&](int kt) {
+    unsigned char* dst = smem + (kt % 3) * SD_A_BYTES + wave * 1024;
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_global_load_lds((gptr_t)(aptr[i] + (int64_t)kt * BK), (lptr_t)(dst + i * 8192), 16, 0, 0);
+  };
+  auto load_b = [&](int kt) {
+    unsigned char* dst = smem + 3 * SD_A_BYTES + (kt & 1) * SD_B_BYTES + wave * 1024;
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int row = wm * WTM + i * 32 + (e >> 2) * 8 + fh * 4 + (e & 3);
-      const int64_t prow = g_row0 + row;  // pass-local row
-      const bool row_ok = prow < args.rows;
-      const int64_t grow = args.row0 + prow;
-      const float w = s_inv[row];
-      float rmax = -INFINITY;
-      float rsum = 0.f;
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_global_load_lds((gptr_t)(bptr[i] + (int64_t)kt * BK), (lptr_t)(dst + i * 8192), 16, 0, 0);
+  };
+
+  f32x16 acc[TM][TN];
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int64_t q = q_row0 + wn * WTN + j * 32 + fr;
-        const float v = acc[i][j][e] * w;
-        if (row_ok && q < args.Q) {
-          rmax = fmaxf(rmax, v);
-          rsum += v;
-          if (args.scores != nullptr) args.scores[grow * args.Q + q] = v;
-          if (v > thr[j]) {
-            const uint32_t pos = atomicAdd(&args.cand_count[q], 1u);
-            if ((int64_t)pos < args.cand_cap) args.cand[q * args.cand_cap + pos] = make_key(v, (uint32_t)grow);
-          }
-        }
-      }
-      if (args.row_max_enc != nullptr) {
-        rmax = fmaxf(rmax, __shfl_xor(rmax, 1));
-        rmax = fmaxf(rmax, __shfl_xor(rmax, 2));
-        rmax = fmaxf(rmax, __shfl_xor(rmax, 4));
-        rmax = fmaxf(rmax, __shfl_xor(rmax, 8));
-        rmax = fmaxf(rmax, __shfl_xor(rmax, 16));
-        if (fr == 0 && row_ok) atomicMax(&args.row_max_enc[grow], f32_ordered(rmax));
-      }
-      if (args.row_sum_part != nullptr) {
-        // fixed-order butterfly over the 32 lanes that hold this row's scores; one writer per (row, part)
-        rsum += __shfl_xor(rsum, 1);
-        rsum += __shfl_xor(rsum, 2);
-        rsum += __shfl_xor(rsum, 4);
-        rsum += __shfl_xor(rsum, 8);
-        rsum += __shfl_xor(rsum, 16);
-        if (fr == 0 && row_ok) args.row_sum_part[prow * args.n_parts + qt * WN + wn] = rsum;
-      }
-    }
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  // one partial per 16-byte chunk position of the K tile, as the tile kernel's loader threads keep them: the
+  // row norms then come out bit-identical, whichever of the two kernels scores a row
+  float ss[4] = {0.f, 0.f, 0.f, 0.f};
+
+  const int fr = lane & 31;
+  const int fh = lane >> 5;
+  int aoff[TM], boff[TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) aoff[i] = (wm * WTM + ((i + wn) & 3) * 32 + fr) * SD_ROW;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) boff[j] = 3 * SD_A_BYTES + (wn * WTN + j * 32 + fr) * SD_ROW;
+  const int key = sd_key(fr);  // rows advance in steps of 32: the key depends on fr alone
+  // The four waves that share 128 rows number their 32-row blocks from different starts (block (i + wn) & 3 is
+  // wave wn's i-th): each wave's first block is then a different one, and summing its squares is that wave's
+  // share of the row norms -- no choice of fragment at run time.
+
+  // The fragment reads are spelled as instructions: the compiler makes an LDS read it can see wait for every
+  // outstanding direct-to-LDS load (it cannot tell the buffers apart), which would undo the prefetch.  The
+  // waits are explicit too: LDS reads return in order, so "at most 6 outstanding" means that the step issued
+  // before the latest six reads has arrived.  (No other LDS or scalar-memory traffic inside the loop.)
+  uint4 af[2][TM], bf[2][TN];
+  uint32_t chk[4];  // byte offset of this lane's chunk in its row, per k-step of the tile
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) chk[kk] = (uint32_t)(((kk * 2 + fh) ^ key) * 16);
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+  auto rd = [&](int kt, auto kk_tag, auto set_tag) {
+    constexpr int SET = decltype(set_tag)::value;
+    constexpr int KK = decltype(kk_tag)::value;
+    const uint32_t ab = lds0 + (uint32_t)(kt % 3) * SD_A_BYTES + chk[KK];
+    const uint32_t bb = lds0 + (uint32_t)(kt & 1) * SD_B_BYTES + chk[KK];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      af[SET][i] = sd_lds_read16(ab + (uint32_t)aoff[i]);
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      bf[SET][j] = sd_lds_read16(bb + (uint32_t)boff[j]);
+  };
+  auto mm = [&](auto set_tag, auto kk_tag) {
+    constexpr int SET = decltype(set_tag)::value;
+    constexpr int KK = decltype(kk_tag)::value;
+    ss[KK] = M::sumsq(af[SET][0], ss[KK]);  // this wave's share of the row norms: its first 32-row block
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) M::mma(af[SET][i], bf[SET][j], acc[i][j]);
+  };
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+
+  // prologue: A(0), B(0), then A(1) stays in flight over the first barrier
+  load_a(0);
+  load_b(0);
+  if (KT > 1) {
+    load_a(1);
+    __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4)
+  } else {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   }
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  using K0 = std::integral_constant<int, 0>;
+  using K1 = std::integral_constant<int, 1>;
+  using K2 = std::integral_constant<int, 2>;
+  using K3 = std::integral_constant<int, 3>;
+  constexpr int WAIT_LDS_6 = 0xC67F;  // lgkmcnt(6), nothing else
+  constexpr int WAIT_LDS_0 = 0xC07F;  // lgkmcnt(0), nothing else
+  __builtin_amdgcn_sched_barrier(0);
+  rd(0, K0{}, S0{});
+  __builtin_amdgcn_sched_barrier(0);
+  if (1 < KT) load_b(1);
+  if (2 < KT) load_a(2);
+  for (int kt = 0; kt < KT; ++kt) {
+    __builtin_amdgcn_sched_barrier(0);
+    rd(kt, K1{}, S1{});
+    __builtin_amdgcn_s_waitcnt(WAIT_LDS_6);
+    __builtin_amdgcn_sched_barrier(0);
+    mm(S0{}, K0{});
+    __builtin_amdgcn_sched_barrier(0);
+    rd(kt, K2{}, S0{});
+    __builtin_amdgcn_s_waitcnt(WAIT_LDS_6);
+    __builtin_amdgcn_sched_barrier(0);
+    mm(S1{}, K1{});
+    __builtin_amdgcn_sched_barrier(0);
+    rd(kt, K3{}, S1{});
+    __builtin_amdgcn_s_waitcnt(WAIT_LDS_6);
+    __builtin_amdgcn_sched_barrier(0);
+    mm(S0{}, K2{});
+    __builtin_amdgcn_sched_barrier(0);
+    // In flight, oldest first: A(kt + 1), then B(kt + 1) and A(kt + 2).  Tile kt + 1 must have landed (this
+    // wave's part; the barrier makes that all of it), A(kt + 2) may still fly; the fragment reads above have
+    // completed, so after the barrier tile kt's buffers take B(kt + 2) and A(kt + 3).
+    if (kt + 2 < KT)
+      __builtin_amdgcn_s_waitcnt(0x0074);  // vmcnt(4) lgkmcnt(0)
+    else
+      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    if (kt + 1 < KT) rd(kt + 1, K0{}, S0{});
+    __builtin_amdgcn_sched_barrier(0);
+    mm(S1{}, K3{});  // its fragments arrived before the barrier
+    __builtin_amdgcn_sched_barrier(0);
+    // the loads go out behind the first MFMAs after the barrier, so that those are not held up by their issue
+    if (kt + 2 < KT) load_b(kt + 2);
+    if (kt + 3 < KT) load_a(kt + 3);
+  }
+  __builtin_amdgcn_s_waitcnt(WAIT_LDS_0);
+
+  // ---- row sum of squares -> per-row multiplier (the tile buffers are free now) ----------------------------
+  // chunk positions 2 kk (lanes fh = 0) and 2 kk + 1 (fh = 1), added up in the order of the tile kernel's butterfly
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) ss[kk] += __shfl_xor(ss[kk], 32);
+  const float ssq = (ss[0] + ss[1]) + (ss[2] + ss[3]);
+  __builtin_amdgcn_s_waitcnt(0x0070);
+  __builtin_amdgcn_s_barrier();  // every wave is past its last fragment read
+  __builtin_amdgcn_sched_barrier(0);
+  if (fh == 0) {
+    const int row = wm * WTM + wn * 32 + fr;
+    float w = args.query_scale;
+    if (args.unit_norm) w = ssq > 0.f ? args.query_scale / sqrtf(ssq) : 0.f;
+    s_inv[row] = w;
+    const int64_t grow = g_row0 + row;
+    if (qt == 0 && args.sumsq != nullptr && grow < args.rows) args.sumsq[args.row0 + grow] = ssq;
+  }
+  __syncthreads();
+
+  scan_tile_epilogue<TM, TN, WTM, WTN, WN>(args, acc, s_inv, wm, wn, fr, fh, g_row0, q_row0, qt, wn);
 }
 
 // ---- few queries: the store streamed once, no tiles in LDS ---------------------------------------
@@ -342,8 +566,7 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void scan_stream_kernel(ScanArg
   // Every wave walks D from its own starting k-pair (a multiple of the queue length) and wraps around: at any
   // moment the waves of the chip then read different parts of the query table, whose 4 KB stretches would
   // otherwise each be wanted by every wave at once.  A step is two segments, [rot, nkp) and [0, rot).
-  const int nblk = nkp / STREAM_Q;
-  const int rot = nblk >= 2 ? (int)(((unsigned)gw * 7u) % (unsigned)nblk) * STREAM_Q : 0;
+  const int rot = stream_rotation(nkp, gw);
   const int nseg = rot > 0 ? 2 : 1;
   constexpr int KP = 2 * M::KS;        // elements of a k-pair
   constexpr int FP = 2 * QB * WAVE;    // table entries of a k-pair
@@ -799,6 +1022,17 @@ static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
     a.row_tiles = (int)((a.rows + BM - 1) / BM);
     a.q_tiles = (a.Q + BN - 1) / BN;
     a.n_parts = a.q_tiles * 4;
+    if constexpr (sizeof(T) == 2) {
+      // aligned 16-bit operands, D a multiple of the K tile: tiles loaded straight into LDS
+      if (aligned && a.D % 64 == 0 && getenv("BGX_SCAN_DIRECT_OFF") == nullptr) {
+        const int row_tiles_pad = (a.row_tiles + 7) / 8 * 8;
+        auto kern = scan_direct_kernel<T>;
+        BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SD_LDS_BYTES));
+        hipLaunchKernelGGL(kern, dim3((unsigned)(row_tiles_pad * a.q_tiles)), dim3(SD_THREADS), SD_LDS_BYTES, st, a);
+        BGX_HIP(hipGetLastError());
+        return 0;
+      }
+    }
     return launch_gemm<T, BM, BN, 2, 4>(a, aligned, st);
   } else if (a.Q > 32) {
     constexpr int BM = 128, BN = 64;

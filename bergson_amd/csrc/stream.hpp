@@ -110,6 +110,15 @@ __device__ inline void stream_rows(const T* base, int64_t tok_stride, int rows_v
     urow[rg] = base + (int64_t)min(rg * 8 + rho, rows_valid - 1) * tok_stride + (sig ^ rho ^ (rg & 1)) * Mma<T>::EPL;
 }
 
+// The k-pair at which wave `gw` of the grid starts a segment of nkp k-pairs whose fragments come from a table in
+// global memory (it then wraps around): a multiple of the queue length, 0 where the segment is too short.  Every
+// wave of a launch reads the same table; walking it in step, all of them ask for the same 4 KB stretch at once
+// and those requests queue at the one L2 channel that holds it.
+__device__ inline int stream_rotation(int nkp, int gw) {
+  const int nblk = nkp / STREAM_Q;
+  return nblk >= 2 ? (int)(((unsigned)gw * 7u) % (unsigned)nblk) * STREAM_Q : 0;
+}
+
 // Every block issues exactly STREAM_Q * RG loads, in k-pair order, whatever its length: a k-pair that does
 // not exist is replaced by a repeat of the block's first one, which is never used.  With that the number of
 // loads between the issue of a k-pair and its use is the same on every path through the code, so the

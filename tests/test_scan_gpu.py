@@ -277,3 +277,35 @@ def test_scan_streamed_best_rows_last(device):
     rv, ri = torch.topk(ref, k, dim=1)
     assert torch.allclose(res.topk_values.cpu(), rv, rtol=1e-3, atol=1e-3)
     assert len(set(res.topk_indices.cpu()[0].tolist()) & set(ri[0].tolist())) >= k - 2
+
+
+# ---- many queries over a long 16-bit store: the tile kernel that loads straight into LDS ----------------
+# At least 256 tiles of 256 rows x 256 queries, aligned fp16 / bf16 operands and D a multiple of 64 take the
+# variant whose K tiles travel global -> LDS without registers (three row buffers, two query buffers); D of
+# 64 to 320 covers its pipeline with one to five K tiles, rows and queries that do not fill the last tiles.
+@pytest.mark.parametrize("dtype,D,Q", [(torch.float16, 64, 300), (torch.float16, 128, 257), (torch.bfloat16, 192, 300),
+                                       (torch.float16, 256, 512), (torch.bfloat16, 320, 70)])
+def test_scan_many_queries_direct_tiles(device, dtype, D, Q):
+    from bergson_amd import ops
+
+    n, k = 66_000 if Q > 256 else 131_000, 50
+    store, queries = make_store(n, D, Q, dtype, seed=D + Q)
+    store[777] = 0
+    qd = unit_queries(queries, dtype).to(dtype)
+    ref = oscan.scorer_score({"m": store}, {"m": qd}, ["m"], dtype=torch.float32, unit_normalize=True).T  # [Q, n]
+    dev_store, dev_q = store.to(device), qd.to(device)
+    res = ops.scan(dev_store, dev_q, unit_norm=True, k=k, want_row_max=True, want_row_mean=True, want_scores=True,
+                   want_sumsq=True, chunk_rows=n)
+    torch.cuda.synchronize()
+    assert (res.scores.cpu().T - ref).abs().max().item() <= COS_TOL
+    assert res.scores[777].abs().max().item() == 0
+    assert (res.row_mean.cpu() - ref.mean(0)).abs().max().item() <= COS_TOL
+    assert torch.allclose(res.sumsq.cpu(), store.float().pow(2).sum(1), rtol=1e-4)
+    assert (res.row_max.cpu() - ref.max(0).values).abs().max().item() <= COS_TOL
+    check_topk(res.topk_values.cpu(), res.topk_indices.cpu(), ref, k)
+    # the same through passes too short for the large tiles (the 128-row tile kernel)
+    small = ops.scan(dev_store, dev_q, unit_norm=True, k=k, chunk_rows=4096)
+    torch.cuda.synchronize()
+    same = small.topk_indices == res.topk_indices
+    assert same.float().mean().item() > 0.99
+    assert (small.topk_values[same] - res.topk_values[same]).abs().max().item() <= 1e-5
