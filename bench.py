@@ -38,7 +38,7 @@ HBM_PEAK_GBS = 8000.0
 # WRITE_SIZE hardware counters (profiles/collect_and_scan_kernels_pmc_hbm_traffic.txt)
 COLLECT_TRAFFIC_RATIO = 1.036
 # the same for the store scan: 1024 queries (four query tiles re-read each row tile, half from L2), at most 32 queries
-SCAN_TRAFFIC_RATIO_Q1024 = 1.51
+SCAN_TRAFFIC_RATIO_Q1024 = 1.50
 SCAN_TRAFFIC_RATIO_FEW = 1.0016
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
@@ -52,6 +52,8 @@ def parse_args():
     ap.add_argument("--token-batch-size", type=int, default=4096)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-scan", action="store_true")
+    ap.add_argument("--scan-only", action="store_true",
+                    help="run the store-scan leg alone and print its entry (for counter runs on the scan kernels)")
     ap.add_argument("--scan-rows", type=int, default=1_000_000)
     ap.add_argument("--scan-queries", type=int, default=1024)
     ap.add_argument("--cpu-sample-tokens", type=int, default=32768)
@@ -245,6 +247,9 @@ def main():
         torch.cuda.synchronize()
         del src, dst
         torch.cuda.empty_cache()
+    if args.scan_only:
+        print(json.dumps({"store_scan": scan_leg(args, torch, device)}))
+        return
     coll, docs, lengths = collection_leg(args, torch, device)
     scan = None if args.no_scan else scan_leg(args, torch, device)
     cpu = None if args.no_cpu_baseline else cpu_baseline_leg(args, torch, docs, lengths)
