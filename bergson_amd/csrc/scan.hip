@@ -306,10 +306,12 @@ __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
 //    barrier is the bare s_barrier -- __syncthreads would wait for every outstanding load;
 //  * the fragments are double-buffered in registers and the pipeline runs across the barrier: the reads of
 //    step 0 of the next tile are issued right after it, before the MFMAs of the last step of this tile.
-constexpr int SD_BM = 256, SD_BN = 256, SD_ROW = 128;
-constexpr int SD_A_BYTES = SD_BM * SD_ROW, SD_B_BYTES = SD_BN * SD_ROW;
-constexpr int SD_LDS_BYTES = 3 * SD_A_BYTES + 2 * SD_B_BYTES;
+constexpr int SD_BM = 256, SD_ROW = 128;
+constexpr int SD_A_BYTES = SD_BM * SD_ROW;
 constexpr int SD_THREADS = 512;
+// BN = 256, or 128 for at most 128 queries (one query tile: half the MFMA work of a 256-wide tile that would be
+// half empty)
+constexpr int sd_lds_bytes(int bn) { return 3 * SD_A_BYTES + 2 * bn * SD_ROW; }
 
 __device__ inline int sd_key(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
@@ -320,13 +322,16 @@ __device__ inline uint4 sd_lds_read16(uint32_t addr) {
   return v;
 }
 
-template <typename T>
+template <typename T, int BN>
 __global__ __launch_bounds__(SD_THREADS) void scan_direct_kernel(ScanArgs args) {
   using M = Mma32<T>;
   typedef __attribute__((address_space(1))) const void* gptr_t;
   typedef __attribute__((address_space(3))) void* lptr_t;
   constexpr int BK = 64;  // elements of K per tile
-  constexpr int TM = 4, TN = 2, WTM = 128, WTN = 64, WN = 4;
+  constexpr int WN = 4, WTM = 128, WTN = BN / WN, TM = 4, TN = WTN / 32;
+  constexpr int NB = BN / 64;  // query-tile load instructions per wave
+  constexpr int SD_B_BYTES = BN * SD_ROW;
+  static_assert(BN == 256 || BN == 128, "query tile");
   extern __shared__ __align__(16) unsigned char smem[];
   float* s_inv = reinterpret_cast<float*>(smem);  // after the main loop: [SD_BM] row multipliers
 
@@ -343,33 +348,36 @@ __global__ __launch_bounds__(SD_THREADS) void scan_direct_kernel(ScanArgs args) 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 2, wn = wave & 3;
   const int64_t g_row0 = (int64_t)rt * SD_BM;  // pass-local first row
-  const int64_t q_row0 = (int64_t)qt * SD_BN;
+  const int64_t q_row0 = (int64_t)qt * BN;
   const int KT = (int)(args.D / BK);
 
   // loader: instruction i of a wave fills rows i * 64 + wave * 8 .. + 7 of a tile; lane l is position l & 7 of
   // row l >> 3 and fetches the chunk that belongs there.  Rows past the end repeat the last one (their scores
   // are never written).
   const T* aptr[4];
-  const T* bptr[4];
+  const T* bptr[NB];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = i * 64 + wave * 8 + (lane >> 3);
     const int ch = (lane & 7) ^ sd_key(r);
     const int64_t grow = min(g_row0 + r, args.rows - 1);
-    const int64_t qrow = min(q_row0 + r, (int64_t)args.Q - 1);
     aptr[i] = (const T*)args.store + (args.row0 + grow) * args.store_stride + ch * 8;
-    bptr[i] = (const T*)args.queries + qrow * args.D + ch * 8;
+    if (i < NB) {
+      const int64_t qrow = min(q_row0 + r, (int64_t)args.Q - 1);
+      bptr[i] = (const T*)args.queries + qrow * args.D + ch * 8;
+    }
   }
   auto load_a = [&](int kt) {
     unsigned char* dst = smem + (kt % 3) * SD_A_BYTES + wave * 1024;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      __builtin_amdgcn_global_load_lds((gptr_t)(aptr[i] + (int64_t)kt * BK), (lptr_t)(dst + i * 8192), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)(aptr[i] + (int64_t)kt * BK), (lptr_t)(dst + i * 8192), 16, 0,
+                                       BN == 128 ? 2 : 0);  // one query tile: every store line is wanted once (nt)
   };
   auto load_b = [&](int kt) {
     unsigned char* dst = smem + 3 * SD_A_BYTES + (kt & 1) * SD_B_BYTES + wave * 1024;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < NB; ++i)
       __builtin_amdgcn_global_load_lds((gptr_t)(bptr[i] + (int64_t)kt * BK), (lptr_t)(dst + i * 8192), 16, 0, 0);
   };
 
@@ -398,8 +406,8 @@ __global__ __launch_bounds__(SD_THREADS) void scan_direct_kernel(ScanArgs args) 
 
   // The fragment reads are spelled as instructions: the compiler makes an LDS read it can see wait for every
   // outstanding direct-to-LDS load (it cannot tell the buffers apart), which would undo the prefetch.  The
-  // waits are explicit too: LDS reads return in order, so "at most 6 outstanding" means that the step issued
-  // before the latest six reads has arrived.  (No other LDS or scalar-memory traffic inside the loop.)
+  // waits are explicit too: LDS reads return in order, so "at most TM + TN outstanding" means that the step
+  // issued before the latest TM + TN reads has arrived.  (No other LDS or scalar-memory traffic inside the loop.)
   uint4 af[2][TM], bf[2][TN];
   uint32_t chk[4];  // byte offset of this lane's chunk in its row, per k-step of the tile
 #pragma unroll
@@ -444,7 +452,7 @@ __global__ __launch_bounds__(SD_THREADS) void scan_direct_kernel(ScanArgs args) 
   using K1 = std::integral_constant<int, 1>;
   using K2 = std::integral_constant<int, 2>;
   using K3 = std::integral_constant<int, 3>;
-  constexpr int WAIT_LDS_6 = 0xC67F;  // lgkmcnt(6), nothing else
+  constexpr int WAIT_LDS_STEP = 0xC07F | ((TM + TN) << 8);  // lgkmcnt(TM + TN), nothing else
   constexpr int WAIT_LDS_0 = 0xC07F;  // lgkmcnt(0), nothing else
   __builtin_amdgcn_sched_barrier(0);
   rd(0, K0{}, S0{});
@@ -454,17 +462,17 @@ __global__ __launch_bounds__(SD_THREADS) void scan_direct_kernel(ScanArgs args) 
   for (int kt = 0; kt < KT; ++kt) {
     __builtin_amdgcn_sched_barrier(0);
     rd(kt, K1{}, S1{});
-    __builtin_amdgcn_s_waitcnt(WAIT_LDS_6);
+    __builtin_amdgcn_s_waitcnt(WAIT_LDS_STEP);
     __builtin_amdgcn_sched_barrier(0);
     mm(S0{}, K0{});
     __builtin_amdgcn_sched_barrier(0);
     rd(kt, K2{}, S0{});
-    __builtin_amdgcn_s_waitcnt(WAIT_LDS_6);
+    __builtin_amdgcn_s_waitcnt(WAIT_LDS_STEP);
     __builtin_amdgcn_sched_barrier(0);
     mm(S1{}, K1{});
     __builtin_amdgcn_sched_barrier(0);
     rd(kt, K3{}, S1{});
-    __builtin_amdgcn_s_waitcnt(WAIT_LDS_6);
+    __builtin_amdgcn_s_waitcnt(WAIT_LDS_STEP);
     __builtin_amdgcn_sched_barrier(0);
     mm(S0{}, K2{});
     __builtin_amdgcn_sched_barrier(0);
@@ -1026,9 +1034,18 @@ static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
       // aligned 16-bit operands, D a multiple of the K tile: tiles loaded straight into LDS
       if (aligned && a.D % 64 == 0 && getenv("BGX_SCAN_DIRECT_OFF") == nullptr) {
         const int row_tiles_pad = (a.row_tiles + 7) / 8 * 8;
-        auto kern = scan_direct_kernel<T>;
-        BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SD_LDS_BYTES));
-        hipLaunchKernelGGL(kern, dim3((unsigned)(row_tiles_pad * a.q_tiles)), dim3(SD_THREADS), SD_LDS_BYTES, st, a);
+        if (a.Q <= 128) {
+          a.q_tiles = 1;
+          a.n_parts = 4;
+          auto kern = scan_direct_kernel<T, 128>;
+          BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, sd_lds_bytes(128)));
+          hipLaunchKernelGGL(kern, dim3((unsigned)row_tiles_pad), dim3(SD_THREADS), sd_lds_bytes(128), st, a);
+        } else {
+          auto kern = scan_direct_kernel<T, 256>;
+          BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, sd_lds_bytes(256)));
+          hipLaunchKernelGGL(kern, dim3((unsigned)(row_tiles_pad * a.q_tiles)), dim3(SD_THREADS), sd_lds_bytes(256), st,
+                             a);
+        }
         BGX_HIP(hipGetLastError());
         return 0;
       }

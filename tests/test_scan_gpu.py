@@ -282,9 +282,11 @@ def test_scan_streamed_best_rows_last(device):
 # ---- many queries over a long 16-bit store: the tile kernel that loads straight into LDS ----------------
 # At least 256 tiles of 256 rows x 256 queries, aligned fp16 / bf16 operands and D a multiple of 64 take the
 # variant whose K tiles travel global -> LDS without registers (three row buffers, two query buffers); D of
-# 64 to 320 covers its pipeline with one to five K tiles, rows and queries that do not fill the last tiles.
+# 64 to 320 covers its pipeline with one to five K tiles, rows and queries that do not fill the last tiles; at most
+# 128 queries take its 128-query-wide form.
 @pytest.mark.parametrize("dtype,D,Q", [(torch.float16, 64, 300), (torch.float16, 128, 257), (torch.bfloat16, 192, 300),
-                                       (torch.float16, 256, 512), (torch.bfloat16, 320, 70)])
+                                       (torch.float16, 256, 512), (torch.bfloat16, 320, 70), (torch.float16, 128, 128),
+                                       (torch.float16, 64, 97)])
 def test_scan_many_queries_direct_tiles(device, dtype, D, Q):
     from bergson_amd import ops
 
