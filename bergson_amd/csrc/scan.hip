@@ -7,9 +7,17 @@
 //                      dense score write, per-row max over queries, and a
 //                      per-query threshold filter that appends the few scores
 //                      that can still enter the top-k to a candidate list.
+//   scan_direct_kernel the same 256 x 256 (or 256 x 128) tile for aligned 16-bit
+//                      operands: K tiles loaded straight into LDS, fragment
+//                      pipeline across the barrier; the kernel of scans with more
+//                      than 64 queries.
+//   scan_stream_kernel at most 32 queries over a long store: no tiles, every wave
+//                      streams its own rows through a register queue and takes the
+//                      queries as MFMA fragments from a table in L2.
 //   scan_select_kernel per query: exact top-k of (running top-k U candidates) by
 //                      radix select on unique 64-bit keys, sorted; raises the
-//                      query's threshold for the next pass.
+//                      query's threshold for the next pass.  Long candidate lists
+//                      are first cut down by the k-th largest of a sample.
 //   scan_finish_kernel decodes keys into (value, row) and the row maxima.
 //
 // The store is processed in passes of at most `chunk_rows` rows so that the
