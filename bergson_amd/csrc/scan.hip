@@ -311,7 +311,7 @@ __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
 //    loader produces by permuting which global chunk each lane fetches: fragment reads are conflict-free;
 //  * three A buffers and two B buffers (160 KB): the store rows are fetched two K tiles ahead, the queries
 //    (L2-resident) one ahead; the per-tile wait is a vmcnt that leaves the youngest A tile in flight, and the
-//    barrier is the bare s_barrier -- __syncthreads would wait for every outstanding load;
+//    barrier is the bare s_barrier (wg_barrier_lds) -- __syncthreads would wait for every outstanding load;
 //  * the fragments are double-buffered in registers and the pipeline runs across the barrier: the reads of
 //    step 0 of the next tile are issued right after it, before the MFMAs of the last step of this tile.
 constexpr int SD_BM = 256, SD_ROW = 128;
@@ -322,6 +322,18 @@ constexpr int SD_THREADS = 512;
 constexpr int sd_lds_bytes(int bn) { return 3 * SD_A_BYTES + 2 * bn * SD_ROW; }
 
 __device__ inline int sd_key(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+// Workgroup barrier without a fence (a fence would wait for every load in flight): waits for this wave's LDS
+// traffic, and for all but the youngest VM_LEFT of its vector-memory operations, then s_barrier.  The memory
+// clobber keeps the compiler from moving memory accesses across it.
+template <int VM_LEFT>
+__device__ inline void wg_barrier_lds() {
+  static_assert(VM_LEFT == 0 || VM_LEFT == 4, "spelled-out wait counts");
+  if constexpr (VM_LEFT == 0)
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  else
+    asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
 
 // 16 bytes from LDS byte address `addr`; the caller waits (lgkmcnt) before it uses the value
 __device__ inline uint4 sd_lds_read16(uint32_t addr) {
@@ -450,11 +462,10 @@ __global__ __launch_bounds__(SD_THREADS) void scan_direct_kernel(ScanArgs args) 
   load_b(0);
   if (KT > 1) {
     load_a(1);
-    __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4)
+    wg_barrier_lds<4>();
   } else {
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    wg_barrier_lds<0>();
   }
-  __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
   using K0 = std::integral_constant<int, 0>;
   using K1 = std::integral_constant<int, 1>;
@@ -488,10 +499,9 @@ __global__ __launch_bounds__(SD_THREADS) void scan_direct_kernel(ScanArgs args) 
     // wave's part; the barrier makes that all of it), A(kt + 2) may still fly; the fragment reads above have
     // completed, so after the barrier tile kt's buffers take B(kt + 2) and A(kt + 3).
     if (kt + 2 < KT)
-      __builtin_amdgcn_s_waitcnt(0x0074);  // vmcnt(4) lgkmcnt(0)
+      wg_barrier_lds<4>();
     else
-      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
-    __builtin_amdgcn_s_barrier();
+      wg_barrier_lds<0>();
     __builtin_amdgcn_sched_barrier(0);
     if (kt + 1 < KT) rd(kt + 1, K0{}, S0{});
     __builtin_amdgcn_sched_barrier(0);
@@ -508,8 +518,7 @@ __global__ __launch_bounds__(SD_THREADS) void scan_direct_kernel(ScanArgs args) 
 #pragma unroll
   for (int kk = 0; kk < 4; ++kk) ss[kk] += __shfl_xor(ss[kk], 32);
   const float ssq = (ss[0] + ss[1]) + (ss[2] + ss[3]);
-  __builtin_amdgcn_s_waitcnt(0x0070);
-  __builtin_amdgcn_s_barrier();  // every wave is past its last fragment read
+  wg_barrier_lds<0>();  // every wave is past its last fragment read
   __builtin_amdgcn_sched_barrier(0);
   if (fh == 0) {
     const int row = wm * WTM + wn * 32 + fr;
