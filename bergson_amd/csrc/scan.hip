@@ -342,7 +342,7 @@ __device__ inline uint4 sd_lds_read16(uint32_t addr) {
   return v;
 }
 
-template <typename T, int BN>
+template <typename T, int BN, bool ONE_QT>
 __global__ __launch_bounds__(SD_THREADS) void scan_direct_kernel(ScanArgs args) {
   using M = Mma32<T>;
   typedef __attribute__((address_space(1))) const void* gptr_t;
@@ -392,7 +392,7 @@ __global__ __launch_bounds__(SD_THREADS) void scan_direct_kernel(ScanArgs args) 
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       __builtin_amdgcn_global_load_lds((gptr_t)(aptr[i] + (int64_t)kt * BK), (lptr_t)(dst + i * 8192), 16, 0,
-                                       BN == 128 ? 2 : 0);  // one query tile: every store line is wanted once (nt)
+                                       ONE_QT ? 2 : 0);  // one query tile: every store line is wanted once (nt)
   };
   auto load_b = [&](int kt) {
     unsigned char* dst = smem + 3 * SD_A_BYTES + (kt & 1) * SD_B_BYTES + wave * 1024;
@@ -1051,18 +1051,22 @@ static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
       // aligned 16-bit operands, D a multiple of the K tile: tiles loaded straight into LDS
       if (aligned && a.D % 64 == 0 && getenv("BGX_SCAN_DIRECT_OFF") == nullptr) {
         const int row_tiles_pad = (a.row_tiles + 7) / 8 * 8;
+        auto launch = [&](auto kern, int bn, unsigned wgs) -> int {
+          BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, sd_lds_bytes(bn)));
+          hipLaunchKernelGGL(kern, dim3(wgs), dim3(SD_THREADS), sd_lds_bytes(bn), st, a);
+          return 0;
+        };
+        int rc;
         if (a.Q <= 128) {
           a.q_tiles = 1;
           a.n_parts = 4;
-          auto kern = scan_direct_kernel<T, 128>;
-          BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, sd_lds_bytes(128)));
-          hipLaunchKernelGGL(kern, dim3((unsigned)row_tiles_pad), dim3(SD_THREADS), sd_lds_bytes(128), st, a);
+          rc = launch(scan_direct_kernel<T, 128, true>, 128, (unsigned)row_tiles_pad);
+        } else if (a.q_tiles == 1) {
+          rc = launch(scan_direct_kernel<T, 256, true>, 256, (unsigned)row_tiles_pad);
         } else {
-          auto kern = scan_direct_kernel<T, 256>;
-          BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, sd_lds_bytes(256)));
-          hipLaunchKernelGGL(kern, dim3((unsigned)(row_tiles_pad * a.q_tiles)), dim3(SD_THREADS), sd_lds_bytes(256), st,
-                             a);
+          rc = launch(scan_direct_kernel<T, 256, false>, 256, (unsigned)(row_tiles_pad * a.q_tiles));
         }
+        if (rc != 0) return rc;
         BGX_HIP(hipGetLastError());
         return 0;
       }
