@@ -26,6 +26,7 @@
 #include <algorithm>
 #include <atomic>
 #include <type_traits>
+#include <queue>
 #include <vector>
 
 #include "common.hpp"
@@ -344,6 +345,7 @@ struct PersistArgs {
   int out_vec8;             // per-token rows: every p x p block starts 16-byte aligned and p is 8 or 16
   const uint4* frag;        // RFG: scaled projection fragments of every module in global memory
   const int64_t* frag_off;  // RFG: [n_modules] first k-step of a module's fragments (r_in's, then r_out's)
+  const int32_t* order;     // RFG: the items in the order the workgroups take them (wg_first indexes this list), or null
 };
 
 // x' = x @ R'^T for this wave's 16*MTW tokens over all of K, R' fragments read from LDS.
@@ -446,7 +448,13 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
   uint4 v[STAGED ? STREAM_Q : 1][2 * MTW];
   uint4 rq[RFG ? STREAM_Q : 1][2];  // RFG: the fragments that go with v
   bool primed = false;
-  for (int item = item0; item < item1; ++item) {
+  for (int idx = item0; idx < item1; ++idx) {
+    // With the fragments in a global table nothing ties a workgroup to consecutive items (no projections staged
+    // per module), so the host deals the items out one by one for even loads and passes the resulting list.
+    int item = idx;
+    if constexpr (RFG) {
+      if (pa.order != nullptr) item = load_uniform(pa.order + idx);
+    }
     const int m = item / pa.tiles_pm;
     const int tile = item - m * pa.tiles_pm;
     const int n = tile / args.tiles_per_seq;
@@ -508,9 +516,13 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
         const uint4* rfN = rfG;  // RFG: the next tile's r_in fragments (any readable address when none follows)
 #pragma unroll
         for (int rg = 0; rg < RG; ++rg) un[rg] = ug[rg];
-        if (item + 1 < item1) {
-          const int m2 = (item + 1) / pa.tiles_pm;
-          const int tile2 = item + 1 - m2 * pa.tiles_pm;
+        if (idx + 1 < item1) {
+          int item2 = idx + 1;
+          if constexpr (RFG) {
+            if (pa.order != nullptr) item2 = load_uniform(pa.order + idx + 1);
+          }
+          const int m2 = item2 / pa.tiles_pm;
+          const int tile2 = item2 - m2 * pa.tiles_pm;
           const int n2 = tile2 / args.tiles_per_seq;
           const int s02 = (tile2 - n2 * args.tiles_per_seq) * TILE_T;
           const int rows2 = min(WAVE_T, seq_token_limit_uniform(args.lengths, n2, args.S) - s02 - wave * WAVE_T);
@@ -768,10 +780,18 @@ static size_t fragment_table_bytes(const bgx_module_desc* mods, int n_modules, i
 }
 
 // The workspace that also holds the fragment table, for launches whose modules are too wide for LDS.
+static size_t item_list_bytes(int n_modules, int N, int S) {
+  return (size_t)n_modules * (size_t)N * (size_t)((S + 63) / 64) * sizeof(int32_t);
+}
+
 size_t collect_workspace_bytes_for(const bgx_module_desc* mods, int n_modules, int N, int S, int p, int in_dtype) {
   const size_t base = collect_workspace_bytes(n_modules, N, S, p);
   if (base == 0 || mods == nullptr) return base;
-  return align_up(base, 256) + fragment_table_bytes(mods, n_modules, p, in_dtype);
+  const size_t table = fragment_table_bytes(mods, n_modules, p, in_dtype);
+  if (table == 0) return align_up(base, 256);
+  // behind the table: the list of (module, tile) items in the order the workgroups take them, at most one per 64
+  // tokens of a sequence and module
+  return align_up(align_up(base, 256) + table, 256) + item_list_bytes(n_modules, N, S);
 }
 
 template <typename T, int PB, bool ALIGNED, int MT, int U>
@@ -969,6 +989,11 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
 
   std::vector<unsigned char> head((size_t)n_modules * sizeof(bgx_module_desc));
   memcpy(head.data(), sorted.data(), head.size());
+  // table variant: room behind the table for the item list that lets the workgroups take items out of order
+  const size_t order_ws_off = align_up(frag_ws_off + frag_bytes, 256);
+  const bool rfg_order = rfg && ws_bytes >= order_ws_off + (size_t)tiles * n_modules * sizeof(int32_t) &&
+                         getenv("BGX_COLLECT_LPT_OFF") == nullptr;
+  std::vector<int32_t> order;
   int wgs = 0;
   if (persist) {
     int cus = 0;
@@ -1023,6 +1048,26 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     first[0] = 0;
     fill(hi_l, first.data());
     first[wgs] = (int32_t)items;
+    if (rfg_order) {
+      // Longest item first to the least loaded workgroup: the modules are sorted by width, so the items come in that
+      // order already.  A workgroup's items stay in ascending order (tiles of one module one after the other).
+      std::vector<int32_t> owner((size_t)items);
+      std::vector<int32_t> count((size_t)wgs, 0);
+      typedef std::pair<double, int> Load;
+      std::priority_queue<Load, std::vector<Load>, std::greater<Load>> heap;
+      for (int g = 0; g < wgs; ++g) heap.push(Load(0.0, g));
+      for (int64_t it = 0; it < items; ++it) {
+        const Load l = heap.top();
+        heap.pop();
+        owner[(size_t)it] = l.second;
+        ++count[(size_t)l.second];
+        heap.push(Load(l.first + w[(size_t)(it / tiles)], l.second));
+      }
+      for (int g = 0; g < wgs; ++g) first[(size_t)g + 1] = first[(size_t)g] + count[(size_t)g];
+      order.resize((size_t)items);
+      std::vector<int32_t> next(first.begin(), first.end() - 1);
+      for (int64_t it = 0; it < items; ++it) order[(size_t)next[(size_t)owner[(size_t)it]]++] = (int32_t)it;
+    }
     head.resize(desc_bytes(n_modules), 0);
     memcpy(head.data() + ranges_offset(n_modules), first.data(), first.size() * sizeof(int32_t));
     if (rfg) {  // where each module's fragments start, in k-steps
@@ -1036,6 +1081,9 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     }
   }
   BGX_HIP(hipMemcpyAsync(mods_dev, head.data(), head.size(), hipMemcpyHostToDevice, st));
+  if (!order.empty())
+    BGX_HIP(hipMemcpyAsync((char*)ws + order_ws_off, order.data(), order.size() * sizeof(int32_t), hipMemcpyHostToDevice,
+                           st));
   uint4* frag_dev = (uint4*)((char*)ws + frag_ws_off);
   const int64_t* frag_off_dev = (const int64_t*)((const char*)ws + frag_off_offset(n_modules));
   if (rfg) {
@@ -1067,6 +1115,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     pa.wg_first = (const int32_t*)((const char*)ws + ranges_offset(n_modules));
     pa.frag = frag_dev;
     pa.frag_off = frag_off_dev;
+    pa.order = order.empty() ? nullptr : (const int32_t*)((const char*)ws + order_ws_off);
     pa.tiles_pm = (int)tiles;
     pa.r_steps = r_steps;
     pa.scratch_bytes = (int)scratch_bytes;

@@ -97,7 +97,8 @@ int bgx_adafactor_scales(const float* row_dev, int32_t O, const float* col_dev,
  * bgx_collect_workspace_bytes is the minimum for any modules of that count.
  * bgx_collect_workspace_bytes_for looks at the modules (only I, O and bias_col
  * of each descriptor are read) and adds room for a table of pre-scaled
- * projection fragments, 32 bytes per input and output feature: with it,
+ * projection fragments, 32 bytes per input and output feature, and for the
+ * list of work items behind it (4 bytes per module and 64 tokens): with it,
  * modules too wide for their projections to be kept on chip (Llama-3-8B's
  * 4096 x 14336) still run through the streamed persistent kernel; without it
  * such launches use the one-workgroup-per-tile kernel.  Both sizes are

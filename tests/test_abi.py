@@ -71,7 +71,9 @@ def test_workspace_sizes():
     for d, (I, O) in zip(descs, [(4096, 14336), (4096, 1024)]):
         d.I, d.O = I, O
     base = lib.bgx_collect_workspace_bytes(2, 2, 2048, 16)
-    assert lib.bgx_collect_workspace_bytes_for(descs, 2, 2, 2048, 16, 2) == -(-base // 256) * 256 + (4096 + 14336 + 4096 + 1024) * 32
+    # the table (32 bytes per column of a and g) and, behind it, the list of items: one per 64 tokens and module
+    assert (lib.bgx_collect_workspace_bytes_for(descs, 2, 2, 2048, 16, 2)
+            == -(-base // 256) * 256 + (4096 + 14336 + 4096 + 1024) * 32 + 2 * 2 * (2048 // 64) * 4)
     descs[1].O = 1000   # a width the streamed kernel cannot take: no table
     assert lib.bgx_collect_workspace_bytes_for(descs, 2, 2, 2048, 16, 2) == -(-base // 256) * 256
     small = lib.bgx_scan_workspace_bytes(8, 10, 1024)
