@@ -57,6 +57,9 @@ def parse_args():
     ap.add_argument("--scan-rows", type=int, default=1_000_000)
     ap.add_argument("--scan-queries", type=int, default=1024)
     ap.add_argument("--cpu-sample-tokens", type=int, default=32768)
+    ap.add_argument("--plain-loop", action="store_true",
+                    help="time the reference's loop shape (forward, backward, hooks, one batch at a time) instead "
+                         "of the overlapped loop that CollectorComputer runs by default")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy (reads 1 GiB, writes 1 GiB): the known-size "
                          "kernel that hardware byte counters are scaled by")
@@ -66,6 +69,7 @@ def parse_args():
 def collection_leg(args, torch, device):
     import bergson_amd as B
     from bergson_amd import ops
+    from bergson_amd.collector import OverlappedSteps
     from bergson_amd.synthetic import ListDataset, adafactor_moments, lognormal_lengths, make_gpt_neox, random_docs
 
     lengths = lognormal_lengths(args.docs, seed=0)
@@ -93,23 +97,36 @@ def collection_leg(args, torch, device):
         staged.append((indices, b, x, y, mask))
     torch.cuda.synchronize()
 
+    # the loop body of CollectorComputer.run_with_collector_hooks: by default each batch's backward pass
+    # runs beside the next batch's forward pass; --plain-loop times one batch at a time
+    overlapped = None if args.plain_loop else OverlappedSteps(model, collector, cfg)
+
     def step(item):
         indices, b, x, y, mask = item
+        if overlapped is not None:
+            overlapped.step(indices, b, x, y, mask)
+            return
         with collector.with_batch(mask):
             losses = fwd_bwd(model, x, y, b)
         collector.process_batch(indices, losses=losses)
 
     for item in staged[:args.warmup]:
         step(item)
+    if overlapped is not None:
+        overlapped.drain()
     torch.cuda.synchronize()
     ops.collect_timer = []
     ops.collect_timing_start(args.steps + 8)
     t0 = time.perf_counter()
     for item in staged[args.warmup:need]:
         step(item)
+    if overlapped is not None:
+        overlapped.drain()
     collector.builder.flush()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
+    if overlapped is not None:
+        overlapped.close()
     timer, ops.collect_timer = ops.collect_timer, None
     kernel_only_ms = ops.collect_timing_stop()
 
@@ -277,6 +294,8 @@ def main():
             "tokens_timed": coll["tokens"],
             "padded_tokens_timed": coll["padded_tokens"],
             "batches_total": coll["n_batches_total"],
+            "loop": "plain (one batch at a time)" if args.plain_loop
+                    else "overlapped (backward of batch i beside forward of batch i+1, one stream)",
         },
         "roofline": {
             "bound": "hbm",

@@ -106,6 +106,7 @@ class HookCollectorBase(ContextDecorator, ABC):
         self._deferred_full: list = []  # unprojected / global-projection modules: (FullGradModule, name, a, g)
         self._full_prepared: dict = {}
         self._active = False
+        self._recording: BatchRecord | None = None
         self._scale_cache: dict[str, tuple[Tensor | None, Tensor | None]] = {}
         self.target_info = self.discover_targets(self.model, self.target_modules, self.processor.include_bias,
                                                  self.filter_modules)
@@ -281,7 +282,14 @@ class HookCollectorBase(ContextDecorator, ABC):
         assert x.ndim == 3, f"Expected input of shape [N, S, I], got {x.shape}"
         self.forward_hook(module, x)
         if isinstance(out, Tensor) and out.requires_grad:
-            out.register_hook(functools.partial(self._on_output_grad, module))
+            rec = self._recording
+            if rec is not None:
+                # the gradient of `out` is asked of autograd by whoever runs the backward pass
+                # (`replay_backward`); no Python runs during that pass
+                rec.entries.append((module, getattr(module, "_inputs", None), out))
+                rec.versions.append(out._version)
+            else:
+                out.register_hook(functools.partial(self._on_output_grad, module))
 
     def _on_output_grad(self, module: nn.Module, grad: Tensor) -> None:
         if self._active:
@@ -294,6 +302,31 @@ class HookCollectorBase(ContextDecorator, ABC):
         self.backward_hook(module, g)
         if hasattr(module, "_inputs"):
             del module._inputs
+
+    # ---- recorded batches: the backward pass without Python hooks ---------------------------------
+    def begin_recording(self, collection_mask: Tensor | None = None) -> "BatchRecord":
+        """Until `end_recording`, forward hooks list (module, kept input, module output) in the returned
+        record instead of attaching tensor hooks.  The caller obtains the gradients of
+        `record.outputs()` from autograd (e.g. `torch.autograd.grad`, possibly on another thread while the
+        next batch's forward pass runs here) and hands them to `replay_backward`."""
+        self._recording = BatchRecord(collection_mask)
+        return self._recording
+
+    def end_recording(self) -> None:
+        self._recording = None
+
+    def replay_backward(self, record: "BatchRecord", grads) -> None:
+        """Calls `backward_hook(module, g)` for every module call of `record`, last call first -- the
+        order and arguments a backward pass with tensor hooks would have produced (collector.py:435-472)."""
+        assert len(grads) == len(record.entries), (len(grads), len(record.entries))
+        self._current_collection_mask = record.mask
+        for (module, kept, _out), g in zip(reversed(record.entries), reversed(grads)):
+            if g is None:  # the loss does not depend on this call's output
+                continue
+            if kept is not None:
+                module._inputs = kept
+            self._process_grad(module, None, (g,))
+        record.entries.clear()
 
     def invalidate_prepared(self) -> None:
         """Forget everything derived from the processor's normalizers (folded factor vectors, Adam tables):
@@ -633,16 +666,47 @@ class HookCollectorBase(ContextDecorator, ABC):
     def process_batch(self, indices: list[int], **kwargs) -> None: ...
 
 
+class BatchRecord:
+    """What the forward hooks saw during one recorded batch: `entries` = (module, kept input, output) per
+    call of a target module, in call order; `mask` = the batch's collection mask."""
+
+    __slots__ = ("mask", "entries", "versions")
+
+    def __init__(self, mask: Tensor | None):
+        self.mask = mask
+        self.entries: list[tuple[nn.Module, Tensor | None, Tensor]] = []
+        self.versions: list[int] = []
+
+    def outputs(self) -> list[Tensor]:
+        """The recorded module outputs, for `torch.autograd.grad(loss, record.outputs())`.  A tensor hook is
+        tied to the value a module returned; `autograd.grad` is tied to the tensor object, so a model that
+        overwrites a module's output in place afterwards would be given the gradient of the overwritten
+        value: refused here."""
+        for (module, _kept, out), version in zip(self.entries, self.versions):
+            if out._version != version:
+                raise RuntimeError(
+                    f"the output of {getattr(module, '_name', module)} was modified in place after the module "
+                    "returned it; the overlapped loop cannot collect from such a model: construct "
+                    "CollectorComputer with overlap_backward=False (or set BGX_OVERLAP_BACKWARD=0)")
+        return [e[2] for e in self.entries]
+
+
 class CollectorComputer:
     """Runs forward/backward over the batches and feeds the collector (collector.py:771-923)."""
 
     def __init__(self, model, data, *, collector: HookCollectorBase, batches: list[list[int]] | None = None,
-                 cfg: IndexConfig):
+                 cfg: IndexConfig, overlap_backward: bool | None = None):
+        """`overlap_backward`: run each batch's backward pass beside the next batch's forward pass
+        (`OverlappedSteps`); None = on for models on a GPU unless the environment has
+        `BGX_OVERLAP_BACKWARD=0`.  Off gives the reference's plain loop, one batch at a time."""
         self.model = model
         self.device = torch.device(model.device)
         self.data = data
         self.batches = batches if batches is not None else [[idx] for idx in range(len(data))]
         self.forward_backward = fwd_bwd_factory(cfg)
+        if overlap_backward is None:
+            overlap_backward = self.device.type == "cuda" and os.environ.get("BGX_OVERLAP_BACKWARD", "1") != "0"
+        self.overlap_backward = overlap_backward
         self.collector = collector
         self.cfg = cfg
         self.rank = dist.get_rank() if dist.is_initialized() else 0
@@ -652,14 +716,28 @@ class CollectorComputer:
         """For each batch: pad, forward, loss, backward (hooks fire), `collector.process_batch`; then
         `collector.teardown()`.  No host synchronisation happens inside the loop."""
         total_processed = torch.tensor(0, device=self.device)
-        for indices in self.batches:
-            batch = self.data[indices]
-            x, y, _, collection_mask = pad_and_tensor(batch["input_ids"], labels=batch.get("labels"),
-                                                      device=self.device, sync_max_len=False)
-            total_processed += collection_mask.sum()
-            with self.collector.with_batch(collection_mask):
-                losses = self.forward_backward(self.model, x, y, batch)
-            self.collector.process_batch(indices, losses=losses)
+        overlapped = OverlappedSteps(self.model, self.collector, self.cfg) if self.overlap_backward else None
+        try:
+            for indices in self.batches:
+                batch = self.data[indices]
+                x, y, _, collection_mask = pad_and_tensor(batch["input_ids"], labels=batch.get("labels"),
+                                                          device=self.device, sync_max_len=False)
+                total_processed += collection_mask.sum()
+                if overlapped is not None:
+                    overlapped.step(indices, batch, x, y, collection_mask)
+                    continue
+                with self.collector.with_batch(collection_mask):
+                    losses = self.forward_backward(self.model, x, y, batch)
+                self.collector.process_batch(indices, losses=losses)
+            if overlapped is not None:
+                overlapped.drain()
+        except BaseException:
+            if overlapped is not None:
+                overlapped.close(failed=True)
+                overlapped = None
+            raise
+        if overlapped is not None:
+            overlapped.close()
         self.collector.teardown()
         self.collector.remove_hooks()
         if dist.is_initialized():
@@ -670,14 +748,13 @@ class CollectorComputer:
         self.total_processed = total_processed
 
 
-def fwd_bwd_factory(cfg: IndexConfig) -> Callable:
-    """fwd_bwd(model, x, y, batch) -> per-sample losses [N] (collector.py:926-985, cross-entropy branch)."""
+def forward_loss_factory(cfg: IndexConfig) -> Callable:
+    """forward_loss(model, x, y, batch) -> per-sample losses [N] with their autograd graph: the forward half
+    of collector.py:926-985 (cross-entropy branch)."""
     if cfg.loss_fn != "ce":
         raise NotImplementedError("only the cross-entropy loss is supported (loss_fn='kl' needs PEFT)")
 
-    trainable: dict[int, list] = {}
-
-    def fwd_bwd(model, x: Tensor, y: Tensor, batch: dict):
+    def forward_loss(model, x: Tensor, y: Tensor, batch: dict):
         logits = model(x).logits[:, :-1]
         masks = y[:, 1:] != -100
         denoms = masks.sum(dim=1, dtype=model.dtype) if cfg.loss_reduction == "mean" else 1.0
@@ -686,6 +763,18 @@ def fwd_bwd_factory(cfg: IndexConfig) -> Callable:
         losses = losses.sum(1) / denoms
         if "advantage" in batch:
             losses *= torch.tensor(batch["advantage"], device=losses.device)
+        return losses
+
+    return forward_loss
+
+
+def fwd_bwd_factory(cfg: IndexConfig) -> Callable:
+    """fwd_bwd(model, x, y, batch) -> per-sample losses [N] (collector.py:926-985, cross-entropy branch)."""
+    forward_loss = forward_loss_factory(cfg)
+    trainable: dict[int, list] = {}
+
+    def fwd_bwd(model, x: Tensor, y: Tensor, batch: dict):
+        losses = forward_loss(model, x, y, batch)
         losses.sum().backward()
         # model.zero_grad(): only parameters that require grad can hold one; the list is built once
         params = trainable.get(id(model))
@@ -696,3 +785,83 @@ def fwd_bwd_factory(cfg: IndexConfig) -> Callable:
         return losses
 
     return fwd_bwd
+
+
+class OverlappedSteps:
+    """The loop body of `run_with_collector_hooks` with the backward pass of a batch running beside the
+    forward pass of the next one.
+
+    A step of a small model is bound by the host: the forward pass is Python issuing a few hundred small
+    kernels, the backward pass is the autograd engine's own thread issuing as many, and each waits for the
+    other.  Here the forward hooks only record (module, input, output); the gradients of the recorded
+    outputs are asked of `torch.autograd.grad` on a helper thread, which holds no interpreter lock while
+    the engine runs, and the caller goes on to the next batch's forward pass.  When a batch's gradients
+    are there, `backward_hook` is called per module as a backward pass would have (`replay_backward`)
+    and `process_batch` launches the batch's kernels.  Every launch goes to the caller's current
+    stream, so kernels of neighbouring batches interleave in one queue and their order within a batch is
+    unchanged; the rows are the same as those of the plain loop.  Parameter gradients are computed as in
+    the plain loop and dropped instead of being accumulated and zeroed, so nothing is left in `.grad`.
+    """
+
+    def __init__(self, model, collector: HookCollectorBase, cfg: IndexConfig):
+        from concurrent.futures import ThreadPoolExecutor
+
+        self.model = model
+        self.collector = collector
+        self.forward_loss = forward_loss_factory(cfg)
+        self._pool = ThreadPoolExecutor(max_workers=1, thread_name_prefix="bgx-backward")
+        self._pending = None
+        self._entered = False
+        self._trainable = [q for q in model.parameters() if q.requires_grad]
+
+    @staticmethod
+    def _gradients(total: Tensor, outputs: list[Tensor], stream, n_recorded: int):
+        if stream is None:  # host tensors (the loop logic is testable without a GPU; the kernels are not)
+            return torch.autograd.grad(total, outputs, allow_unused=True)[:n_recorded]
+        with torch.cuda.device(total.device), torch.cuda.stream(stream):
+            return torch.autograd.grad(total, outputs, allow_unused=True)[:n_recorded]
+
+    def step(self, indices: list[int], batch: dict, x: Tensor, y: Tensor, collection_mask: Tensor) -> None:
+        col = self.collector
+        if not self._entered:
+            col.__enter__()
+            self._entered = True
+        record = col.begin_recording(collection_mask)
+        try:
+            losses = self.forward_loss(self.model, x, y, batch)
+        finally:
+            col.end_recording()
+        # The trainable parameters are asked for too (and their gradients dropped, as the plain loop drops
+        # them with zero_grad): the engine then runs the same nodes as `backward()` would, so hooks that
+        # others have put on the model still fire.
+        outputs = record.outputs() + self._trainable
+        stream = torch.cuda.current_stream(x.device) if x.is_cuda else None
+        future = self._pool.submit(self._gradients, losses.sum(), outputs, stream, len(record.entries))
+        del outputs
+        self._finish()
+        self._pending = (indices, record, losses.detach(), future)
+
+    def _finish(self) -> None:
+        if self._pending is None:
+            return
+        (indices, record, losses, future), self._pending = self._pending, None
+        grads = future.result()
+        self.collector.replay_backward(record, grads)
+        self.collector.process_batch(indices, losses=losses)
+
+    def drain(self) -> None:
+        """Finish the batch whose backward pass is still out."""
+        self._finish()
+
+    def close(self, failed: bool = False) -> None:
+        if self._pending is not None:
+            future = self._pending[3]
+            self._pending = None
+            try:
+                future.result()
+            except Exception:
+                pass
+        self._pool.shutdown(wait=True)
+        if self._entered:
+            self.collector.__exit__(RuntimeError if failed else None, None, None)
+            self._entered = False

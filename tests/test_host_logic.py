@@ -174,3 +174,120 @@ def test_product_does_not_import_the_oracle():
     root = pathlib.Path(__file__).resolve().parent.parent / "bergson_amd"
     for f in root.rglob("*.py"):
         assert not re.search(r"^\s*(from|import)\s+oracle\b", f.read_text(), re.M), f
+
+
+class _ToyLM(nn.Module):
+    """Two target layers in sequence behind an embedding, shaped [N, S, *] like a language model."""
+
+    def __init__(self, inplace: bool = False):
+        super().__init__()
+        self.emb = nn.Embedding(11, 8)
+        self.fc1 = nn.Linear(8, 16)
+        self.fc2 = nn.Linear(16, 8, bias=False)
+        self.inplace = inplace
+        self.device = torch.device("cpu")
+
+    def forward(self, x):
+        h = self.fc1(self.emb(x))
+        if self.inplace:
+            h.mul_(2.0)
+        return self.fc2(torch.tanh(h))
+
+
+def _logging_stub(model):
+    from bergson_amd import GradientProcessor, HookCollectorBase
+
+    class Log(HookCollectorBase):
+        def setup(self):
+            self.seen = []
+            self.batches = []
+
+        def teardown(self): ...
+
+        def backward_hook(self, module, g):
+            self.seen.append((module._name, module._inputs.clone(), g.clone(), self._current_collection_mask))
+
+        def process_batch(self, indices, **k):
+            self.batches.append((list(indices), k["losses"].clone(), len(self.seen)))
+
+    return Log(model=model, processor=GradientProcessor(projection_dim=4, projection_type="normal"))
+
+
+def test_recorded_backward_matches_tensor_hooks():
+    """`begin_recording` + `torch.autograd.grad` + `replay_backward` hands `backward_hook` the same modules,
+    inputs and output gradients, in the same order, as the tensor hooks of a plain backward pass."""
+    torch.manual_seed(0)
+    m = _ToyLM()
+    x = torch.randint(0, 11, (3, 5))
+    mask = torch.ones(3, 5, dtype=torch.bool)
+    c = _logging_stub(m)
+    with c.with_batch(mask):
+        m(x).square().sum().backward()
+    plain, c.seen = c.seen, []
+    assert [n for n, *_ in plain] == ["fc2", "fc1"]
+    m.zero_grad()
+
+    with c:
+        rec = c.begin_recording(mask)
+        loss = m(x).square().sum()
+        c.end_recording()
+        assert len(rec.entries) == 2 and not c.seen
+        grads = torch.autograd.grad(loss, rec.outputs(), allow_unused=True)
+        c.replay_backward(rec, grads)
+    assert [n for n, *_ in c.seen] == [n for n, *_ in plain]
+    for (_, a0, g0, m0), (_, a1, g1, m1) in zip(plain, c.seen):
+        assert torch.equal(a0, a1) and torch.equal(g0, g1) and m1 is mask
+    assert not hasattr(m.fc1, "_inputs") and not rec.entries
+    assert all(p.grad is None for p in m.fc1.parameters())  # autograd.grad accumulates nothing
+
+
+def test_recorded_backward_refuses_outputs_modified_in_place():
+    m = _ToyLM(inplace=True)
+    c = _logging_stub(m)
+    with c:
+        rec = c.begin_recording(None)
+        m(torch.randint(0, 11, (2, 4))).sum()
+        c.end_recording()
+        with pytest.raises(RuntimeError, match="modified in place"):
+            rec.outputs()
+
+
+def test_overlapped_steps_equal_the_plain_loop():
+    """`OverlappedSteps` (backward pass of batch i on a helper thread beside the forward pass of batch i+1)
+    gives every batch the hook calls and losses of the plain loop, batch by batch, in order."""
+    from bergson_amd import IndexConfig
+    from bergson_amd.collector import CollectorComputer
+
+    class LM(_ToyLM):
+        def forward(self, x):
+            out = super().forward(x)
+            logits = torch.cat([out, out.flip(-1)[..., :3]], -1)  # 11 "vocabulary" entries
+            return type("O", (), {"logits": logits})()
+
+    class Data:
+        docs = [[1, 2, 3, 4], [5, 6, 7], [8, 9, 10, 1, 2], [3, 4], [6, 5, 4, 3, 2, 1]]
+
+        def __len__(self):
+            return len(self.docs)
+
+        def __getitem__(self, idx):
+            return {"input_ids": [self.docs[i] for i in idx]}
+
+    torch.manual_seed(1)
+    m = LM()
+    m.dtype = torch.float32
+    batches = [[0, 1], [2], [3, 4]]
+    cfg = IndexConfig(run_path="", projection_dim=4, projection_type="normal")
+    logs = []
+    for overlap in (False, True):
+        c = _logging_stub(m)
+        CollectorComputer(model=m, data=Data(), collector=c, batches=batches, cfg=cfg,
+                          overlap_backward=overlap).run_with_collector_hooks()
+        logs.append(c)
+    plain, over = logs
+    assert [b[0] for b in over.batches] == batches and [b[2] for b in over.batches] == [b[2] for b in plain.batches]
+    for (_, l0, _), (_, l1, _) in zip(plain.batches, over.batches):
+        assert torch.equal(l0, l1)
+    assert len(plain.seen) == len(over.seen) == 6
+    for (n0, a0, g0, m0), (n1, a1, g1, m1) in zip(plain.seen, over.seen):
+        assert n0 == n1 and torch.equal(a0, a1) and torch.equal(g0, g1) and torch.equal(m0, m1)
