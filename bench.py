@@ -150,6 +150,9 @@ def collection_leg(args, torch, device):
         "n_batches_total": len(batches),
         "store_rows_nonzero": int((abs(store[:, :256].astype("float32")).sum(axis=1) > 0).sum()),
         "total_tokens_all_docs": int(sum(lengths)),
+        "loop": "plain (one batch at a time)" if overlapped is None else
+                f"overlapped (backward pass of batch i beside the forward pass of batch i+1, batches alternating "
+                f"between {overlapped._n_streams} streams, the collection launch alone on the GPU)",
     }
     del collector, model
     torch.cuda.empty_cache()
@@ -294,8 +297,7 @@ def main():
             "tokens_timed": coll["tokens"],
             "padded_tokens_timed": coll["padded_tokens"],
             "batches_total": coll["n_batches_total"],
-            "loop": "plain (one batch at a time)" if args.plain_loop
-                    else "overlapped (backward of batch i beside forward of batch i+1, one stream)",
+            "loop": coll["loop"],
         },
         "roofline": {
             "bound": "hbm",

@@ -803,7 +803,7 @@ class OverlappedSteps:
     the plain loop and dropped instead of being accumulated and zeroed, so nothing is left in `.grad`.
     """
 
-    def __init__(self, model, collector: HookCollectorBase, cfg: IndexConfig):
+    def __init__(self, model, collector: HookCollectorBase, cfg: IndexConfig, *, streams: int | None = None):
         from concurrent.futures import ThreadPoolExecutor
 
         self.model = model
@@ -813,6 +813,13 @@ class OverlappedSteps:
         self._pending = None
         self._entered = False
         self._trainable = [q for q in model.parameters() if q.requires_grad]
+        # With two streams, batches alternate between them: the kernels of one batch's backward pass and of
+        # the next batch's forward pass then sit in different queues and the many small ones among them run
+        # side by side.  A batch's own launches (which share the collector's workspace and store with every
+        # other batch's) wait for both streams and hold both, see `step`.
+        self._streams: list = []
+        self._n_streams = min(2, streams if streams is not None else int(os.environ.get("BGX_OVERLAP_STREAMS", "2")))
+        self._step_no = 0
 
     @staticmethod
     def _gradients(total: Tensor, outputs: list[Tensor], stream, n_recorded: int):
@@ -826,32 +833,66 @@ class OverlappedSteps:
         if not self._entered:
             col.__enter__()
             self._entered = True
+        stream = None
+        if x.is_cuda:
+            stream = caller = torch.cuda.current_stream(x.device)
+            if self._n_streams > 1:
+                if not self._streams:
+                    self._streams = [torch.cuda.Stream(x.device) for _ in range(self._n_streams)]
+                stream = self._streams[self._step_no % self._n_streams]
+                stream.wait_stream(caller)  # the batch's tensors were made on the caller's stream
+                for t in (x, y, collection_mask):
+                    t.record_stream(stream)
+            self._step_no += 1
         record = col.begin_recording(collection_mask)
         try:
-            losses = self.forward_loss(self.model, x, y, batch)
+            with torch.cuda.stream(stream) if stream is not None else nullcontext():
+                losses = self.forward_loss(self.model, x, y, batch)
+                total = losses.sum()
         finally:
             col.end_recording()
         # The trainable parameters are asked for too (and their gradients dropped, as the plain loop drops
         # them with zero_grad): the engine then runs the same nodes as `backward()` would, so hooks that
         # others have put on the model still fire.
         outputs = record.outputs() + self._trainable
-        stream = torch.cuda.current_stream(x.device) if x.is_cuda else None
-        future = self._pool.submit(self._gradients, losses.sum(), outputs, stream, len(record.entries))
-        del outputs
-        self._finish()
-        self._pending = (indices, record, losses.detach(), future)
+        if self._n_streams > 1 and stream is not None:
+            # the previous batch's launch gets the GPU to itself: it starts when this forward pass has
+            # finished too, and this batch's backward pass waits for it (an HBM-bound kernel sharing the
+            # chip with the other queue's kernels takes half as long again, and slows them in turn)
+            self._finish(before=stream)
+            future = self._pool.submit(self._gradients, total, outputs, stream, len(record.entries))
+        else:
+            future = self._pool.submit(self._gradients, total, outputs, stream, len(record.entries))
+            self._finish()
+        del outputs, total
+        self._pending = (indices, record, losses.detach(), future, stream)
 
-    def _finish(self) -> None:
+    def _finish(self, before=None) -> None:
+        """Hooks and `process_batch` of the batch whose backward pass is out, on that batch's stream;
+        `before` = the stream of the batch that follows (its work so far precedes the launch, its later
+        work follows it)."""
         if self._pending is None:
             return
-        (indices, record, losses, future), self._pending = self._pending, None
+        (indices, record, losses, future, stream), self._pending = self._pending, None
         grads = future.result()
-        self.collector.replay_backward(record, grads)
-        self.collector.process_batch(indices, losses=losses)
+        if stream is None or self._n_streams <= 1:
+            self.collector.replay_backward(record, grads)
+            self.collector.process_batch(indices, losses=losses)
+            return
+        with torch.cuda.stream(stream):
+            if before is not None:
+                stream.wait_stream(before)
+            self.collector.replay_backward(record, grads)
+            self.collector.process_batch(indices, losses=losses)
+        if before is not None:
+            before.wait_stream(stream)
 
     def drain(self) -> None:
-        """Finish the batch whose backward pass is still out."""
+        """Finish the batch whose backward pass is still out; the caller's stream then waits for the
+        streams the batches ran on."""
         self._finish()
+        for s in self._streams:
+            torch.cuda.current_stream(s.device).wait_stream(s)
 
     def close(self, failed: bool = False) -> None:
         if self._pending is not None:
