@@ -238,3 +238,52 @@ def test_global_projection_matches_cpu_loop(device, tmp_path, attribute_tokens):
         got = torch.from_numpy(np.array(load_gradients(part)))
     assert got.shape == want.shape
     assert rel_l2(got, want) <= 1e-3
+
+
+@pytest.mark.parametrize("attribute_tokens", [False, True])
+def test_overlapped_loop_equals_plain_loop_bitwise(device, attribute_tokens):
+    """The loop with two batches in flight (backward pass of one beside the forward pass of the next, on one
+    stream and on two) writes the same store and the same losses as the loop that handles one batch at a
+    time, bit for bit: same kernels on the same operands, only their place in the queues differs.  Many
+    batches of different shapes, so that a launch that overtook its operands, or two launches sharing the
+    workspace at once, would show."""
+    from bergson_amd import AdafactorNormalizer, GradientCollector, IndexConfig, allocate_batches
+    from bergson_amd.collector import CollectorComputer, OverlappedSteps
+    from bergson_amd.synthetic import ListDataset, adafactor_moments, lognormal_lengths, make_gpt_neox, random_docs
+
+    lengths = lognormal_lengths(40, mu=4.0, sigma=0.8, lo=2, hi=256, seed=11)
+    docs = random_docs(lengths, seed=11)
+    batches = allocate_batches(lengths, 256)
+    assert len(batches) >= 8
+    model = make_gpt_neox("pythia-160m", torch.bfloat16, device, seed=0, layers=2)
+    moments = adafactor_moments(model.base_model, seed=0)
+    normalizers = {n: AdafactorNormalizer(row=r.to(device), col=c.to(device)) for n, (r, c) in moments.items()}
+    cfg = IndexConfig(run_path="", projection_dim=16, projection_type="normal", attribute_tokens=attribute_tokens)
+
+    def run(overlap, streams, monkeypatch_streams):
+        col = GradientCollector(model=model.base_model, cfg=cfg, data=ListDataset(docs),
+                                processor=_processor(16, normalizers), store_dtype=torch.float16)
+        monkeypatch_streams(streams)
+        CollectorComputer(model=model, data=ListDataset(docs), collector=col, batches=batches, cfg=cfg,
+                          overlap_backward=overlap).run_with_collector_hooks()
+        torch.cuda.synchronize()
+        return np.array(col.builder.grad_buffer).copy(), col.per_doc_losses.cpu().clone()
+
+    init = OverlappedSteps.__init__
+
+    def set_streams(n):
+        def patched(self, *a, **k):
+            k["streams"] = n
+            init(self, *a, **k)
+        OverlappedSteps.__init__ = patched
+
+    try:
+        plain, plain_losses = run(False, 1, set_streams)
+        for streams in (1, 2):
+            got, losses = run(True, streams, set_streams)
+            assert np.array_equal(got.view(np.uint16), plain.view(np.uint16)), streams
+            assert torch.equal(losses, plain_losses), streams
+    finally:
+        OverlappedSteps.__init__ = init
+    assert np.abs(plain.astype(np.float32)).sum() > 0
+    assert all(p.grad is None for p in model.parameters())
