@@ -787,6 +787,19 @@ def fwd_bwd_factory(cfg: IndexConfig) -> Callable:
     return fwd_bwd
 
 
+_SECOND_STREAMS: dict = {}
+
+
+def _second_stream(device: torch.device):
+    """The one extra stream per device that `OverlappedSteps` alternates with the caller's.  Made once per
+    process: which hardware queue a stream lands on depends on how many were made before it, and two
+    streams that share a queue run nothing side by side."""
+    key = torch.device(device)
+    if key not in _SECOND_STREAMS:
+        _SECOND_STREAMS[key] = torch.cuda.Stream(key)
+    return _SECOND_STREAMS[key]
+
+
 class OverlappedSteps:
     """The loop body of `run_with_collector_hooks` with the backward pass of a batch running beside the
     forward pass of the next one.
@@ -823,10 +836,15 @@ class OverlappedSteps:
 
     @staticmethod
     def _gradients(total: Tensor, outputs: list[Tensor], stream, n_recorded: int):
+        # retain_graph: the engine then frees no saved tensor while it runs.  Almost every one of them has
+        # been seen by Python, and releasing such a tensor from the engine's thread takes the interpreter
+        # lock -- hundreds of times per pass, each time against the thread that is issuing the next forward
+        # pass.  The graph is dropped by the caller's thread instead (`_finish`), which holds the lock anyway.
+        retain = os.environ.get("BGX_OVERLAP_RETAIN", "1") != "0"
         if stream is None:  # host tensors (the loop logic is testable without a GPU; the kernels are not)
-            return torch.autograd.grad(total, outputs, allow_unused=True)[:n_recorded]
+            return torch.autograd.grad(total, outputs, allow_unused=True, retain_graph=retain)[:n_recorded]
         with torch.cuda.device(total.device), torch.cuda.stream(stream):
-            return torch.autograd.grad(total, outputs, allow_unused=True)[:n_recorded]
+            return torch.autograd.grad(total, outputs, allow_unused=True, retain_graph=retain)[:n_recorded]
 
     def step(self, indices: list[int], batch: dict, x: Tensor, y: Tensor, collection_mask: Tensor) -> None:
         col = self.collector
@@ -838,11 +856,12 @@ class OverlappedSteps:
             stream = caller = torch.cuda.current_stream(x.device)
             if self._n_streams > 1:
                 if not self._streams:
-                    self._streams = [torch.cuda.Stream(x.device) for _ in range(self._n_streams)]
-                stream = self._streams[self._step_no % self._n_streams]
-                stream.wait_stream(caller)  # the batch's tensors were made on the caller's stream
-                for t in (x, y, collection_mask):
-                    t.record_stream(stream)
+                    self._streams = [caller, _second_stream(x.device)]
+                stream = self._streams[self._step_no % 2]
+                if stream is not caller:
+                    stream.wait_stream(caller)  # the batch's tensors were made on the caller's stream
+                    for t in (x, y, collection_mask):
+                        t.record_stream(stream)
             self._step_no += 1
         record = col.begin_recording(collection_mask)
         try:
@@ -864,8 +883,8 @@ class OverlappedSteps:
         else:
             future = self._pool.submit(self._gradients, total, outputs, stream, len(record.entries))
             self._finish()
-        del outputs, total
-        self._pending = (indices, record, losses.detach(), future, stream)
+        del outputs
+        self._pending = (indices, record, losses.detach(), future, stream, total)
 
     def _finish(self, before=None) -> None:
         """Hooks and `process_batch` of the batch whose backward pass is out, on that batch's stream;
@@ -873,8 +892,9 @@ class OverlappedSteps:
         work follows it)."""
         if self._pending is None:
             return
-        (indices, record, losses, future, stream), self._pending = self._pending, None
+        (indices, record, losses, future, stream, total), self._pending = self._pending, None
         grads = future.result()
+        del total, future  # with the record's outputs (cleared by replay_backward), the last owners of the graph
         if stream is None or self._n_streams <= 1:
             self.collector.replay_backward(record, grads)
             self.collector.process_batch(indices, losses=losses)
@@ -891,8 +911,8 @@ class OverlappedSteps:
         """Finish the batch whose backward pass is still out; the caller's stream then waits for the
         streams the batches ran on."""
         self._finish()
-        for s in self._streams:
-            torch.cuda.current_stream(s.device).wait_stream(s)
+        for s in self._streams[1:]:
+            self._streams[0].wait_stream(s)
 
     def close(self, failed: bool = False) -> None:
         if self._pending is not None:
