@@ -296,27 +296,59 @@ struct FusedArgs {
   float* ptok;  // [tokens][p * p]
 };
 
+// two fp32 values rounded to nearest-even in T, packed low | high << 16 (the hardware's packed conversion
+// for bf16: the software rounding of f32_to_bf16_bits costs six vector instructions per value, and a
+// workgroup converts 65 536 values per chunk of output features)
+template <typename T>
+__device__ inline uint32_t pack2_bits(float lo, float hi) {
+  if constexpr (Elem<T>::code == BGX_F16) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    const h2 r = {(_Float16)lo, (_Float16)hi};
+    return __builtin_bit_cast(uint32_t, r);
+  } else {
+    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    const f2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, b2));
+  }
+}
+
 constexpr int FUSED_TILE = 256;
-constexpr int FUSED_ZROW = FUSED_TILE * 2 + 16;  // bytes per token row of the staged tile (padded)
+
+// (x0 * g.lo, x1 * g.hi) rounded to T, packed like `g2` (two T values).  fp16 rounds x to T first: the packed
+// half multiply then gives the once-rounded exact product in one instruction; bf16 multiplies in fp32.
+template <typename T>
+__device__ inline uint32_t scaled_pair_bits(float x0, float x1, uint32_t g2) {
+  if constexpr (Elem<T>::code == BGX_F16) {
+    typedef _Float16 hv __attribute__((ext_vector_type(2)));
+    const uint32_t h2 = pack2_bits<T>(x0, x1);
+    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(hv, h2) * __builtin_bit_cast(hv, g2));
+  } else {
+    const float b0 = __uint_as_float(g2 << 16), b1 = __uint_as_float(g2 & 0xffff0000u);
+    return pack2_bits<T>(x0 * b0, x1 * b1);
+  }
+}
 
 template <typename T>
 __global__ __launch_bounds__(512) void adam_fused_kernel(FusedArgs a) {
   using M = Mma32<T>;
   static_assert(sizeof(T) == 2, "the fused Adam kernel is for 16-bit model dtypes");
-  constexpr int BM = FUSED_TILE, BN = FUSED_TILE, WN = 4, NT = 512;
+  constexpr int BM = FUSED_TILE, BN = FUSED_TILE, NT = 512;
   constexpr int EPL = M::EPL;
   constexpr int BK = TILE_CHUNKS * EPL;
-  constexpr int WTM = 128, WTN = 64, TM = 4, TN = 2;
+  // 8 waves as 4 (tokens) x 2 (output features), 64 x 128 per wave: two 32-token blocks per wave keep the
+  // second pass's accumulators at 32 registers
+  constexpr int WNW = 2, WTM = 64, WTN = 128, TM = 2, TN = 4;
   constexpr int GCH = BM * TILE_CHUNKS / NT, QCH = BN * TILE_CHUNKS / NT;
   constexpr int ROWS_PER_PASS = NT / TILE_CHUNKS;
   constexpr int BUF_BYTES = (BM + BN) * LDS_ROW_BYTES;
-  static_assert(BM * FUSED_ZROW <= 2 * BUF_BYTES, "the staged tile reuses the GEMM's LDS buffers");
+  static_assert((NT / 64 / WNW) * TM * 16 * 64 * 4 <= 2 * BUF_BYTES, "the final reduction reuses the GEMM's LDS buffers");
   extern __shared__ __align__(16) unsigned char smem[];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave / WN, wn = wave % WN;
+  const int wm = wave / WNW, wn = wave % WNW;
   const int fr = lane & 31;
   const int fh = lane >> 5;
   const int lrow = tid / TILE_CHUNKS;
@@ -328,125 +360,162 @@ __global__ __launch_bounds__(512) void adam_fused_kernel(FusedArgs a) {
   const int rows_here = a.tokens - t_row0;  // valid tokens of this tile (may exceed BM)
 
   const T* act = (const T*)a.a + (int64_t)t_row0 * a.a_tok_stride;
-  const T* Lmat = (const T*)a.r_out;
 
-  // this lane's token in the second pass and its g row
-  const int my_tl = t_row0 + wave * 32 + fr;
-  const int64_t my_t = a.t0 + (my_tl < a.tokens ? my_tl : a.tokens - 1);
-  const int my_n = (int)(my_t / a.S);
-  const int my_s = (int)(my_t - (int64_t)my_n * a.S);
-  const T* my_g = (const T*)a.g + (int64_t)my_n * a.g_seq_stride + (int64_t)my_s * a.g_tok_stride + fh * EPL;
-  const T* my_l = Lmat + (int64_t)min(fr, p - 1) * O + fh * EPL;
-
-  f32x16 pacc;
+  // Second pass, straight from the accumulators.  The GEMM blocks are accumulated transposed (the table's
+  // fragment as the A operand): lane (fr, fh) then holds token fr of a block, and its 16 accumulators are rows
+  // q*8 + fh*4 + c (q, c = 0..3) of the 32 table rows of the block.  The loader puts table row
+  // fh*16 + q*4 + c at that place of the LDS tile, so those 16 accumulators are 16 consecutive output features,
+  // fh*16 + e: a k-step of the second pass takes e = 8s .. 8s+7, one 16-byte piece of the token's g row and of
+  // a row of L per lane (the order of k inside an MFMA is free as long as both operands use the same one).
+  // H never leaves the registers: no staged tile in LDS, no barrier around the second pass, and the K-tile
+  // pipeline runs on across the chunks of output features.
+  const T* g_row[TM];
 #pragma unroll
-  for (int e = 0; e < 16; ++e) pacc[e] = 0.f;
+  for (int i = 0; i < TM; ++i) {
+    const int tl = t_row0 + wm * WTM + i * 32 + fr;
+    const int64_t t = a.t0 + (tl < a.tokens ? tl : a.tokens - 1);
+    const int n = (int)(t / a.S);
+    const int sp = (int)(t - (int64_t)n * a.S);
+    g_row[i] = (const T*)a.g + (int64_t)n * a.g_seq_stride + (int64_t)sp * a.g_tok_stride + wn * WTN + fh * 16;
+  }
+  const T* l_row = (const T*)a.r_out + (int64_t)min(fr, p - 1) * O + wn * WTN + fh * 16;
+
+  f32x16 pacc[TM];
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) pacc[i][e] = 0.f;
+#pragma unroll
+    for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][jj][e] = 0.f;
+  }
 
   const int KT = (int)(I / BK);
-  for (int oc = 0; oc < O; oc += BN) {
-    const T* tab = (const T*)a.table + ((int64_t)j * O + oc) * I;
-    f32x16 acc[TM][TN];
+  const int total = KT * (O / BN);  // K tiles of all chunks, one pipeline
+
+  // the loader runs two tiles ahead of the MFMAs and has its own position
+  int ld_kt = 0;
+  const T* ld_tab = (const T*)a.table + (int64_t)j * O * I;
+  uint4 gr[GCH], qr[QCH];
+  // table row that goes to LDS row lrow (+ multiples of 64): bits (q1 q0 h c1 c0) -> (h q1 q0 c1 c0)
+  const int prow = (lrow & ~31) | ((lrow & 4) << 2) | ((lrow & 24) >> 1) | (lrow & 3);
+  auto gload = [&]() {
+    const int64_t k = (int64_t)ld_kt * BK + lcol * EPL;
+#pragma unroll
+    for (int i = 0; i < GCH; ++i)
+      gr[i] = load_chunk<T, true>(act, lrow + i * ROWS_PER_PASS, rows_here, a.a_tok_stride, k, I);
+#pragma unroll
+    for (int i = 0; i < QCH; ++i) qr[i] = load_chunk<T, true>(ld_tab, prow + i * ROWS_PER_PASS, BN, I, k, I);
+    if (++ld_kt == KT) {
+      ld_kt = 0;
+      ld_tab += (int64_t)BN * I;
+    }
+  };
+  auto lstore = [&](int buf) {
+    unsigned char* base = smem + buf * BUF_BYTES;
+#pragma unroll
+    for (int i = 0; i < GCH; ++i)
+      *reinterpret_cast<uint4*>(base + (lrow + i * ROWS_PER_PASS) * LDS_ROW_BYTES + lcol * 16) = gr[i];
+#pragma unroll
+    for (int i = 0; i < QCH; ++i)
+      *reinterpret_cast<uint4*>(base + (BM + lrow + i * ROWS_PER_PASS) * LDS_ROW_BYTES + lcol * 16) = qr[i];
+  };
+  auto mma_step = [&](const unsigned char* gb, const unsigned char* qb, int kk) {
+    uint4 af[TM], bf[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const uint4*>(gb + i * 32 * LDS_ROW_BYTES + kk * 32);
+#pragma unroll
+    for (int jj = 0; jj < TN; ++jj) bf[jj] = *reinterpret_cast<const uint4*>(qb + jj * 32 * LDS_ROW_BYTES + kk * 32);
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int jj = 0; jj < TN; ++jj)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][jj][e] = 0.f;
+      for (int jj = 0; jj < TN; ++jj) M::mma(bf[jj], af[i], acc[i][jj]);  // transposed block: rows = o
+  };
 
-    uint4 gr[GCH], qr[QCH];
-    auto gload = [&](int kt) {
-      const int64_t k = (int64_t)kt * BK + lcol * EPL;
+  // same pipeline as the store scan: MFMAs of tile t from buffer t&1 while tile t+1 goes to the other
+  // buffer and the loads of tile t+2 are in flight; one barrier per tile
+  gload();
+  lstore(0);
+  if (total > 1) gload();
+  __syncthreads();
+  int kt = 0, oc = 0;
+  for (int t = 0; t < total; ++t) {
+    const int buf = t & 1;
+    const unsigned char* gb = smem + buf * BUF_BYTES + (wm * WTM + fr) * LDS_ROW_BYTES + fh * 16;
+    const unsigned char* qb = smem + buf * BUF_BYTES + (BM + wn * WTN + fr) * LDS_ROW_BYTES + fh * 16;
+    mma_step(gb, qb, 0);
+    if (t + 1 < total) lstore(buf ^ 1);
+    if (t + 2 < total) gload();
 #pragma unroll
-      for (int i = 0; i < GCH; ++i)
-        gr[i] = load_chunk<T, true>(act, lrow + i * ROWS_PER_PASS, rows_here, a.a_tok_stride, k, I);
+    for (int kk = 1; kk < TILE_CHUNKS / 2; ++kk) mma_step(gb, qb, kk);
+    if (++kt == KT) {
+      // the chunk's H is complete: pacc[t, i] += sum_o (H[t, o] * g[t, o]) * L[i, o] over this wave's 128 o
+      kt = 0;
+      // group = (jj, s): 16 output features per lane pair; the operands of group n + 1 are asked for before
+      // the MFMAs of group n, so one round trip to L2 is exposed per chunk, not one per group
+      uint4 lq[2], gq[2][TM];
+      auto ask = [&](int grp, int slot) {
+        const int off = oc + (grp >> 1) * 32 + (grp & 1) * 8;
+        lq[slot] = load16_global(l_row + off);
 #pragma unroll
-      for (int i = 0; i < QCH; ++i) qr[i] = load_chunk<T, true>(tab, lrow + i * ROWS_PER_PASS, BN, I, k, I);
-    };
-    auto lstore = [&](int buf) {
-      unsigned char* base = smem + buf * BUF_BYTES;
+        for (int i = 0; i < TM; ++i) gq[slot][i] = load16_global(g_row[i] + off);
+      };
+      ask(0, 0);
 #pragma unroll
-      for (int i = 0; i < GCH; ++i)
-        *reinterpret_cast<uint4*>(base + (lrow + i * ROWS_PER_PASS) * LDS_ROW_BYTES + lcol * 16) = gr[i];
+      for (int grp = 0; grp < 2 * TN; ++grp) {
+        const int slot = grp & 1, jj = grp >> 1, s = grp & 1;
+        if (grp + 1 < 2 * TN) ask(grp + 1, slot ^ 1);
 #pragma unroll
-      for (int i = 0; i < QCH; ++i)
-        *reinterpret_cast<uint4*>(base + (BM + lrow + i * ROWS_PER_PASS) * LDS_ROW_BYTES + lcol * 16) = qr[i];
-    };
-    auto mma_step = [&](const unsigned char* gb, const unsigned char* qb, int kk) {
-      uint4 af[TM], bf[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const uint4*>(gb + i * 32 * LDS_ROW_BYTES + kk * 32);
-#pragma unroll
-      for (int jj = 0; jj < TN; ++jj) bf[jj] = *reinterpret_cast<const uint4*>(qb + jj * 32 * LDS_ROW_BYTES + kk * 32);
+        for (int i = 0; i < TM; ++i) {
+          const f32x16& h = acc[i][jj];
+          uint4 af;
+          af.x = scaled_pair_bits<T>(h[8 * s + 0], h[8 * s + 1], gq[slot][i].x);
+          af.y = scaled_pair_bits<T>(h[8 * s + 2], h[8 * s + 3], gq[slot][i].y);
+          af.z = scaled_pair_bits<T>(h[8 * s + 4], h[8 * s + 5], gq[slot][i].z);
+          af.w = scaled_pair_bits<T>(h[8 * s + 6], h[8 * s + 7], gq[slot][i].w);
+          M::mma(af, lq[slot], pacc[i]);
+        }
+      }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int jj = 0; jj < TN; ++jj) M::mma(af[i], bf[jj], acc[i][jj]);
-    };
-
-    // same pipeline as the store scan: MFMAs of tile kt from buffer kt&1 while tile kt+1 goes to the
-    // other buffer and the loads of tile kt+2 are in flight; one barrier per tile
-    gload(0);
-    lstore(0);
-    if (KT > 1) gload(1);
-    __syncthreads();
-    for (int kt = 0; kt < KT; ++kt) {
-      const int buf = kt & 1;
-      const unsigned char* gb = smem + buf * BUF_BYTES + (wm * WTM + fr) * LDS_ROW_BYTES + fh * 16;
-      const unsigned char* qb = smem + buf * BUF_BYTES + (BM + wn * WTN + fr) * LDS_ROW_BYTES + fh * 16;
-      mma_step(gb, qb, 0);
-      if (kt + 1 < KT) lstore(buf ^ 1);
-      if (kt + 2 < KT) gload(kt + 2);
+        for (int jj = 0; jj < TN; ++jj)
 #pragma unroll
-      for (int kk = 1; kk < TILE_CHUNKS / 2; ++kk) mma_step(gb, qb, kk);
-      __syncthreads();
+          for (int e = 0; e < 16; ++e) acc[i][jj][e] = 0.f;
+      oc += BN;
     }
+    __syncthreads();
+  }
 
-    // acc -> LDS as [token][o] in the model dtype
+  // the two waves that share 64 tokens add their halves of the sum over o, in a fixed order
+  float* red = reinterpret_cast<float*>(smem);
+  if (wn == 1) {
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int jj = 0; jj < TN; ++jj)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int row = wm * WTM + i * 32 + (e >> 2) * 8 + fh * 4 + (e & 3);
-          const int col = wn * WTN + jj * 32 + fr;
-          uint16_t bits;
-          if constexpr (Elem<T>::code == BGX_F16)
-            bits = (uint16_t)f32_to_f16_bits(acc[i][jj][e]);
-          else
-            bits = (uint16_t)f32_to_bf16_bits(acc[i][jj][e]);
-          *reinterpret_cast<uint16_t*>(smem + row * FUSED_ZROW + col * 2) = bits;
-        }
-    __syncthreads();
-
-    // second pass: this wave's 32 tokens x 32 rows of L, K = the chunk's 256 output features
-    const unsigned char* zrow = smem + (wave * 32 + fr) * FUSED_ZROW + fh * 16;
-#pragma unroll 4
-    for (int ks = 0; ks < BN / 16; ++ks) {
-      const uint4 zf = *reinterpret_cast<const uint4*>(zrow + ks * 32);
-      const uint4 gf = load16_global(my_g + oc + ks * 16);
-      const uint4 lf = load16_global(my_l + oc + ks * 16);
-      uint4 af = make_uint4(0u, 0u, 0u, 0u);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) Mma<T>::set(af, e, Mma<T>::get(zf, e) * Mma<T>::get(gf, e));
-      M::mma(af, lf, pacc);
-    }
-    __syncthreads();  // the next chunk's tiles overwrite the staged tile
+      for (int e = 0; e < 16; ++e) red[((wm * TM + i) * 16 + e) * 64 + lane] = pacc[i][e];
   }
-
-  // pacc[e] = P[token (e>>2)*8 + fh*4 + (e&3) of this wave][i = fr], column j
+  __syncthreads();
+  if (wn == 0) {
+    // pacc[i][e] = P[token (e>>2)*8 + fh*4 + (e&3) of block i of this wave][row fr], column j
 #pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const int tl = t_row0 + wave * 32 + (e >> 2) * 8 + fh * 4 + (e & 3);
-    if (tl < a.tokens && fr < p) {
-      bool valid = true;
-      if (a.lengths != nullptr) {
-        const int64_t t = a.t0 + tl;
-        const int n = (int)(t / a.S);
-        valid = (int)(t - (int64_t)n * a.S) < a.lengths[n] - 1;
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int tl = t_row0 + wm * WTM + i * 32 + (e >> 2) * 8 + fh * 4 + (e & 3);
+        if (tl < a.tokens && fr < p) {
+          bool valid = true;
+          if (a.lengths != nullptr) {
+            const int64_t t = a.t0 + tl;
+            const int n = (int)(t / a.S);
+            valid = (int)(t - (int64_t)n * a.S) < a.lengths[n] - 1;
+          }
+          const float v = pacc[i][e] + red[((wm * TM + i) * 16 + e) * 64 + lane];
+          a.ptok[(int64_t)tl * pp + fr * p + j] = valid ? v : 0.f;
+        }
       }
-      a.ptok[(int64_t)tl * pp + fr * p + j] = valid ? pacc[e] : 0.f;
-    }
   }
 }
 
