@@ -51,12 +51,14 @@ def parse_args():
     ap.add_argument("--docs", type=int, default=2048)
     ap.add_argument("--token-batch-size", type=int, default=4096)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-scan", action="store_true")
+    ap.add_argument("--no-scan", action="store_true", help="skip the store-scan and per-token Adam legs")
     ap.add_argument("--scan-only", action="store_true",
                     help="run the store-scan leg alone and print its entry (for counter runs on the scan kernels)")
     ap.add_argument("--scan-rows", type=int, default=1_000_000)
     ap.add_argument("--scan-queries", type=int, default=1024)
     ap.add_argument("--cpu-sample-tokens", type=int, default=32768)
+    ap.add_argument("--adam-only", action="store_true",
+                    help="run the per-token Adam leg alone and print its entry (for counter runs on that kernel)")
     ap.add_argument("--plain-loop", action="store_true",
                     help="time the reference's loop shape (forward, backward, hooks, one batch at a time) instead "
                          "of the overlapped loop that CollectorComputer runs by default")
@@ -219,6 +221,48 @@ def scan_leg(args, torch, device):
     return out
 
 
+def adam_leg(args, torch, device):
+    """Per-token gradients under an Adam normalizer at p = 32 (configs[3]: Pythia-410m shape): the four Linear
+    modules of one layer on one 4096-token batch, i.e. the fused kernel that dominates that configuration."""
+    from bergson_amd import ops
+
+    N, S, p, d = 4, 1024, 32, 1024
+    gen = torch.Generator(device=device).manual_seed(2)
+    rnd = lambda *shape: torch.randn(*shape, generator=gen, device=device)
+    lengths = torch.full((N,), S, dtype=torch.int32, device=device)
+    offsets = torch.arange(N, device=device, dtype=torch.int64) * (S - 1)
+    out = torch.zeros(N * (S - 1), p * p, device=device, dtype=torch.bfloat16)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    reps, total_ms, total_flops, modules = 5, 0.0, 0.0, {}
+    for name, (I, O) in (("query_key_value", (d, 3 * d)), ("dense", (d, d)), ("dense_h_to_4h", (d, 4 * d)),
+                         ("dense_4h_to_h", (4 * d, d))):
+        a = rnd(N, S, I).to(torch.bfloat16)
+        g = (rnd(N, S, O) * 0.01).to(torch.bfloat16)
+        v = torch.rand(O, I, generator=gen, device=device) * 1e-5 + 1e-10
+        prep = ops.AdamPrepared(rnd(p, I).to(torch.bfloat16), rnd(p, O).to(torch.bfloat16), v, 0)
+        run = lambda: ops.collect_adam(prep, a, g, out, per_token=True, lengths=lengths, rows=offsets, lo=-3e38,
+                                       hi=3e38)
+        run()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        flops = 2.0 * N * S * I * O * p
+        modules[name] = {"I": I, "O": O, "ms": ms, "tflops": flops / (ms * 1e-3) / 1e12}
+        total_ms += ms
+        total_flops += flops
+        del a, g, v, prep
+    tf = total_flops / (total_ms * 1e-3) / 1e12
+    return {"workload": "configs[3]: one Pythia-410m layer, 4 x 1024 tokens, p=32, Adam, per-token rows (bf16)",
+            "ms_per_layer": total_ms, "tokens_per_s_24_layers_hooks_only": N * S / (total_ms * 24e-3),
+            "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": tf / MFMA_F16_PEAK_TFLOPS, "traffic": None},
+            "modules": modules}
+
+
 def cpu_baseline_leg(args, torch, docs, lengths):
     """The CPU oracle on the first documents of the same workload, about `cpu_sample_tokens` tokens."""
     from bergson_amd.synthetic import adafactor_moments, make_gpt_neox
@@ -270,8 +314,12 @@ def main():
     if args.scan_only:
         print(json.dumps({"store_scan": scan_leg(args, torch, device)}))
         return
+    if args.adam_only:
+        print(json.dumps({"adam_per_token": adam_leg(args, torch, device)}))
+        return
     coll, docs, lengths = collection_leg(args, torch, device)
     scan = None if args.no_scan else scan_leg(args, torch, device)
+    adam = None if args.no_scan else adam_leg(args, torch, device)
     cpu = None if args.no_cpu_baseline else cpu_baseline_leg(args, torch, docs, lengths)
 
     value = coll["tokens"] / coll["seconds"]
@@ -315,6 +363,7 @@ def main():
         },
         "cpu_baseline": cpu,
         "store_scan": scan,
+        "adam_per_token": adam,
     }
     print(json.dumps(line))
 
