@@ -755,11 +755,22 @@ def forward_loss_factory(cfg: IndexConfig) -> Callable:
         raise NotImplementedError("only the cross-entropy loss is supported (loss_fn='kl' needs PEFT)")
 
     def forward_loss(model, x: Tensor, y: Tensor, batch: dict):
-        logits = model(x).logits[:, :-1]
+        # The reference slices `logits[:, :-1]` and reshapes, which copies the [N, S-1, V] logits (400 MB for a
+        # 4096-token batch of a 50k vocabulary) and, in the backward pass, zero-fills and copies them again.
+        # The same losses come from the whole [N, S, V] tensor as a view, with the labels shifted left and the
+        # last position ignored (-100 is cross_entropy's ignore_index: loss 0, gradient 0 -- what the slice's
+        # backward pass fills in).
+        logits = model(x).logits
+        targets = F.pad(y[:, 1:], (0, 1), value=-100)
         masks = y[:, 1:] != -100
         denoms = masks.sum(dim=1, dtype=model.dtype) if cfg.loss_reduction == "mean" else 1.0
-        losses = F.cross_entropy(logits.reshape(-1, logits.size(-1)), y[:, 1:].flatten(), reduction="none",
-                                 label_smoothing=cfg.label_smoothing).reshape_as(y[:, 1:])
+        if logits.is_contiguous():
+            losses = F.cross_entropy(logits.view(-1, logits.size(-1)), targets.flatten(), reduction="none",
+                                     label_smoothing=cfg.label_smoothing).view_as(targets)
+        else:
+            logits = logits[:, :-1]
+            losses = F.cross_entropy(logits.reshape(-1, logits.size(-1)), y[:, 1:].flatten(), reduction="none",
+                                     label_smoothing=cfg.label_smoothing).reshape_as(y[:, 1:])
         losses = losses.sum(1) / denoms
         if "advantage" in batch:
             losses *= torch.tensor(batch["advantage"], device=losses.device)
