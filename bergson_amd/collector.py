@@ -815,16 +815,25 @@ class OverlappedSteps:
     """The loop body of `run_with_collector_hooks` with the backward pass of a batch running beside the
     forward pass of the next one.
 
-    A step of a small model is bound by the host: the forward pass is Python issuing a few hundred small
-    kernels, the backward pass is the autograd engine's own thread issuing as many, and each waits for the
-    other.  Here the forward hooks only record (module, input, output); the gradients of the recorded
-    outputs are asked of `torch.autograd.grad` on a helper thread, which holds no interpreter lock while
-    the engine runs, and the caller goes on to the next batch's forward pass.  When a batch's gradients
-    are there, `backward_hook` is called per module as a backward pass would have (`replay_backward`)
-    and `process_batch` launches the batch's kernels.  Every launch goes to the caller's current
-    stream, so kernels of neighbouring batches interleave in one queue and their order within a batch is
-    unchanged; the rows are the same as those of the plain loop.  Parameter gradients are computed as in
-    the plain loop and dropped instead of being accumulated and zeroed, so nothing is left in `.grad`.
+    Issued one batch at a time, a step of a small model leaves both sides idle in turn: the forward pass is
+    Python issuing a few hundred small kernels, the backward pass is the autograd engine's own thread
+    issuing as many, and most of the kernels are too small to fill the GPU.  Here the forward hooks only
+    record (module, input, output); the gradients of the recorded outputs are asked of
+    `torch.autograd.grad` on a helper thread, which holds no interpreter lock while the engine runs, and
+    the caller goes on to the next batch's forward pass.  When a batch's gradients are there,
+    `backward_hook` is called per module as a backward pass would have (`replay_backward`) and
+    `process_batch` launches the batch's kernels.
+
+    `streams=2` (the default; `BGX_OVERLAP_STREAMS=1` for one): batches alternate between the caller's
+    stream and one extra stream of the same priority, so the two passes that overlap on the host also sit
+    in different queues on the GPU.  A batch's hooks and launches go to its own stream, after the other
+    stream's work so far, and the other stream's later work waits for them: the collector's kernels have
+    the GPU to themselves, and its workspace and store are never touched by two launches at once.  With
+    one stream the kernels of neighbouring batches interleave in the caller's queue.
+
+    The rows and losses are those of the plain loop, bit for bit.  Parameter gradients are computed as
+    in the plain loop and dropped instead of being accumulated and zeroed, so nothing is left in `.grad`.
+    Two batches' activations are alive at a time.
     """
 
     def __init__(self, model, collector: HookCollectorBase, cfg: IndexConfig, *, streams: int | None = None):
@@ -844,6 +853,12 @@ class OverlappedSteps:
         self._streams: list = []
         self._n_streams = min(2, streams if streams is not None else int(os.environ.get("BGX_OVERLAP_STREAMS", "2")))
         self._step_no = 0
+        if self._n_streams > 1:
+            # every other batch's graph ends at parameters whose gradient accumulators sit on the caller's
+            # stream; the engine orders the two streams itself, and says so once per process unless told not to
+            quiet = getattr(torch.autograd.graph, "set_warn_on_accumulate_grad_stream_mismatch", None)
+            if quiet is not None:
+                quiet(False)
 
     @staticmethod
     def _gradients(total: Tensor, outputs: list[Tensor], stream, n_recorded: int):
