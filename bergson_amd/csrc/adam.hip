@@ -455,28 +455,27 @@ __global__ __launch_bounds__(512) void adam_fused_kernel(FusedArgs a) {
       kt = 0;
       // group = (jj, s): 16 output features per lane pair; the operands of group n + 1 are asked for before
       // the MFMAs of group n, so one round trip to L2 is exposed per chunk, not one per group
-      uint4 lq[2], gq[2][TM];
-      auto ask = [&](int grp, int slot) {
+      // one 32-token block after the other: the eight pieces of a token's g row (two 128-byte lines) are then
+      // asked for back to back, while the lines are still in the L1
+      uint4 lq[2], gq[2];
+      auto ask = [&](int n, int slot) {  // n = i * 8 + group
+        const int grp = n & 7;
         const int off = oc + (grp >> 1) * 32 + (grp & 1) * 8;
         lq[slot] = load16_global(l_row + off);
-#pragma unroll
-        for (int i = 0; i < TM; ++i) gq[slot][i] = load16_global(g_row[i] + off);
+        gq[slot] = load16_global(g_row[n >> 3] + off);
       };
       ask(0, 0);
 #pragma unroll
-      for (int grp = 0; grp < 2 * TN; ++grp) {
-        const int slot = grp & 1, jj = grp >> 1, s = grp & 1;
-        if (grp + 1 < 2 * TN) ask(grp + 1, slot ^ 1);
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          const f32x16& h = acc[i][jj];
-          uint4 af;
-          af.x = scaled_pair_bits<T>(h[8 * s + 0], h[8 * s + 1], gq[slot][i].x);
-          af.y = scaled_pair_bits<T>(h[8 * s + 2], h[8 * s + 3], gq[slot][i].y);
-          af.z = scaled_pair_bits<T>(h[8 * s + 4], h[8 * s + 5], gq[slot][i].z);
-          af.w = scaled_pair_bits<T>(h[8 * s + 6], h[8 * s + 7], gq[slot][i].w);
-          M::mma(af, lq[slot], pacc[i]);
-        }
+      for (int n = 0; n < TM * 2 * TN; ++n) {
+        const int slot = n & 1, i = n >> 3, grp = n & 7, jj = grp >> 1, s = grp & 1;
+        if (n + 1 < TM * 2 * TN) ask(n + 1, slot ^ 1);
+        const f32x16& h = acc[i][jj];
+        uint4 af;
+        af.x = scaled_pair_bits<T>(h[8 * s + 0], h[8 * s + 1], gq[slot].x);
+        af.y = scaled_pair_bits<T>(h[8 * s + 2], h[8 * s + 3], gq[slot].y);
+        af.z = scaled_pair_bits<T>(h[8 * s + 4], h[8 * s + 5], gq[slot].z);
+        af.w = scaled_pair_bits<T>(h[8 * s + 6], h[8 * s + 7], gq[slot].w);
+        M::mma(af, lq[slot], pacc[i]);
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
