@@ -40,6 +40,9 @@ COLLECT_TRAFFIC_RATIO = 1.036
 # the same for the store scan: 1024 queries (four query tiles re-read each row tile, half from L2), at most 32 queries
 SCAN_TRAFFIC_RATIO_Q1024 = 1.50
 SCAN_TRAFFIC_RATIO_FEW = 1.0016
+# bytes the four fused Adam launches of one layer fetch through the L2s and write, from the same counters
+# (profiles/adam_fused_pythia410m_layer_p32.txt): 5.16 GB + 0.07 GB, against 0.94 GB read once each
+ADAM_TRAFFIC_BYTES_PER_LAYER = 5.22e9
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
@@ -259,7 +262,7 @@ def adam_leg(args, torch, device):
     return {"workload": "configs[3]: one Pythia-410m layer, 4 x 1024 tokens, p=32, Adam, per-token rows (bf16)",
             "ms_per_layer": total_ms, "tokens_per_s_24_layers_hooks_only": N * S / (total_ms * 24e-3),
             "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                         "frac": tf / MFMA_F16_PEAK_TFLOPS, "traffic": None},
+                         "frac": tf / MFMA_F16_PEAK_TFLOPS, "traffic": ADAM_TRAFFIC_BYTES_PER_LAYER},
             "modules": modules}
 
 

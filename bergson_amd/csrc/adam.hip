@@ -294,6 +294,7 @@ struct FusedArgs {
   int S, I, O, p;
   const int32_t* lengths;
   float* ptok;  // [tokens][p * p]
+  int ttx;      // token tiles per group of 32 workgroups that share an XCD; 0 = plain workgroup order
 };
 
 // two fp32 values rounded to nearest-even in T, packed low | high << 16 (the hardware's packed conversion
@@ -353,8 +354,19 @@ __global__ __launch_bounds__(512) void adam_fused_kernel(FusedArgs a) {
   const int fh = lane >> 5;
   const int lrow = tid / TILE_CHUNKS;
   const int lcol = tid % TILE_CHUNKS;
-  const int t_row0 = blockIdx.x * BM;  // chunk-local first token of the tile
-  const int j = blockIdx.y;
+  // Which (token tile, column j) this workgroup takes.  Workgroup b runs on XCD b % 8, and the 32 that an XCD
+  // runs at a time share operands through its L2: `ttx` token tiles x 32 / ttx columns (chosen by the host).
+  // In the plain order every XCD walks the whole table; here it reads only its own columns' share.
+  int tt = blockIdx.x, j = blockIdx.y;
+  if (a.ttx > 0) {
+    const int b = blockIdx.x + gridDim.x * blockIdx.y;
+    const int xcd = b & 7, slot = b >> 3;
+    const int jx = 32 / a.ttx, n_super_tt = gridDim.x / a.ttx;
+    const int super = (slot >> 5) * 8 + xcd, within = slot & 31;
+    tt = (super % n_super_tt) * a.ttx + within % a.ttx;
+    j = (super / n_super_tt) * jx + within / a.ttx;
+  }
+  const int t_row0 = tt * BM;  // chunk-local first token of the tile
   const int p = a.p, O = a.O, pp = p * p;
   const int64_t I = a.I;
   const int rows_here = a.tokens - t_row0;  // valid tokens of this tile (may exceed BM)
@@ -696,6 +708,23 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
       f.lengths = lengths;
       f.ptok = ptok_f;
       const dim3 grid((unsigned)((rows_c + FUSED_TILE - 1) / FUSED_TILE), (unsigned)p);
+      // 4 token tiles x 8 columns per XCD at a time fetched least through the L2s on every module shape of
+      // the benchmark layer (1.3 GB against 1.9 for the plain order on 1024 x 3072; 16 x 2 fetched 2.2: the
+      // token tiles' activations then no longer stay in a 4 MB L2); 8 x 4 is next
+      int ttx = 0;
+      if ((grid.x * grid.y) % 256 == 0) {
+        const int prefer[3] = {4, 8, 2};
+        for (int c : prefer)
+          if (grid.x % c == 0 && p % (32 / c) == 0) {
+            ttx = c;
+            break;
+          }
+        if (const char* e = getenv("BGX_ADAM_TTX")) {
+          const int v = atoi(e);
+          if (v == 0 || ((v == 2 || v == 4 || v == 8 || v == 16) && grid.x % v == 0 && p % (32 / v) == 0)) ttx = v;
+        }
+      }
+      f.ttx = ttx;
       if (dtype == BGX_F16) {
         auto kern = adam_fused_kernel<f16_t>;
         BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));

@@ -597,6 +597,33 @@ def test_adam_fused_path(device, dtype, p, per_token, monkeypatch):
     assert rel_l2(got, other) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("ttx", [None, 2, 8])
+def test_adam_fused_xcd_order(device, ttx, monkeypatch):
+    """A grid of 256 workgroups (8 token tiles x 32 columns): the fused kernel then deals (token tile, column)
+    pairs to the workgroups so that those sharing an XCD share operands.  Every pair must still be taken exactly
+    once: the rows equal those of the plain order bit for bit, and the oracle's within tolerance."""
+    N, S, I, O, p = 2, 1024, 64, 256, 32
+    case = _adam_case(N, S, I, O, p, torch.bfloat16, seed=61)
+    a, g, left, right, norm = case
+    lengths = [1024, 700]
+    g = g.clone()
+    for n, l in enumerate(lengths):
+        g[n, l - 1:] = 0
+    case = (a, g, left, right, norm)
+    counts = [l - 1 for l in lengths]
+    offs = [0, counts[0]]
+    kw = dict(per_token=True, lengths=lengths, row_offsets=offs, n_rows=sum(counts))
+    if ttx is not None:
+        monkeypatch.setenv("BGX_ADAM_TTX", str(ttx))
+    got = _run_adam(device, case, p, torch.bfloat16, **kw)
+    monkeypatch.setenv("BGX_ADAM_TTX", "0")
+    plain = _run_adam(device, case, p, torch.bfloat16, **kw)
+    assert torch.equal(got, plain)
+    mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+    want = ohooks.module_gradient(a, g, norm, left, right, attribute_tokens=True, collection_mask=mask)
+    assert rel_l2(got, want) <= TOL[torch.bfloat16]
+
+
 def test_adam_seq_many_short_sequences(device):
     """Many short sequences of a fused-eligible shape: the per-sequence rows come from the per-token kernel."""
     N, S, I, O, p = 40, 24, 128, 256, 16
