@@ -866,11 +866,10 @@ class OverlappedSteps:
         # been seen by Python, and releasing such a tensor from the engine's thread takes the interpreter
         # lock -- hundreds of times per pass, each time against the thread that is issuing the next forward
         # pass.  The graph is dropped by the caller's thread instead (`_finish`), which holds the lock anyway.
-        retain = os.environ.get("BGX_OVERLAP_RETAIN", "1") != "0"
         if stream is None:  # host tensors (the loop logic is testable without a GPU; the kernels are not)
-            return torch.autograd.grad(total, outputs, allow_unused=True, retain_graph=retain)[:n_recorded]
+            return torch.autograd.grad(total, outputs, allow_unused=True, retain_graph=True)[:n_recorded]
         with torch.cuda.device(total.device), torch.cuda.stream(stream):
-            return torch.autograd.grad(total, outputs, allow_unused=True, retain_graph=retain)[:n_recorded]
+            return torch.autograd.grad(total, outputs, allow_unused=True, retain_graph=True)[:n_recorded]
 
     def step(self, indices: list[int], batch: dict, x: Tensor, y: Tensor, collection_mask: Tensor) -> None:
         col = self.collector
@@ -945,9 +944,9 @@ class OverlappedSteps:
             future = self._pending[3]
             self._pending = None
             try:
-                future.result()
+                future.result()  # let the backward pass that is still out finish before the hooks go away
             except Exception:
-                pass
+                pass  # close() runs after a failure too; the first error is the one the caller sees
         self._pool.shutdown(wait=True)
         if self._entered:
             self.collector.__exit__(RuntimeError if failed else None, None, None)
