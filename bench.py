@@ -49,8 +49,13 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=40)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=260,
+                    help="timed batches (default: 260 of the workload's 323, so that the store flush at the end and the "
+                         "pipeline's first and last half-steps weigh about what they weigh in a whole run)")
+    ap.add_argument("--warmup", type=int, default=60,
+                    help="untimed batches first (default 60: in a fresh process the first ~50 batches of new shapes run "
+                         "at 12 ms instead of 8.8: the libraries under the model load kernels and pick GEMM variants "
+                         "on first use)")
     ap.add_argument("--docs", type=int, default=2048)
     ap.add_argument("--token-batch-size", type=int, default=4096)
     ap.add_argument("--no-cpu-baseline", action="store_true")
