@@ -831,8 +831,7 @@ class OverlappedSteps:
     the GPU to themselves, and its workspace and store are never touched by two launches at once.  With
     one stream the kernels of neighbouring batches interleave in the caller's queue.
 
-    The rows and losses are those of the plain loop, bit for bit.  Parameter gradients are computed as
-    in the plain loop and dropped instead of being accumulated and zeroed, so nothing is left in `.grad`.
+    The rows and losses are those of the plain loop, bit for bit.  Nothing is accumulated into `.grad`.
     Two batches' activations are alive at a time.
     """
 
@@ -846,6 +845,17 @@ class OverlappedSteps:
         self._pending = None
         self._entered = False
         self._trainable = [q for q in model.parameters() if q.requires_grad]
+        # The backward pass is asked to go down to the output of the input embedding (every layer's nodes run,
+        # so hooks that others have put on the layers still fire) rather than to the parameters: a parameter's
+        # gradient accumulator belongs to one stream, and the engine makes that stream wait for the end of
+        # every backward pass on the other one -- in the middle of the next batch's forward pass, whenever the
+        # host happens to be that far.  Models without `get_input_embeddings` are asked for the parameters.
+        self._embedding_output: Tensor | None = None
+        self._embedding_hook = None
+        embedding = getattr(model, "get_input_embeddings", None)
+        embedding = embedding() if callable(embedding) and os.environ.get("BGX_OVERLAP_ROOT") != "parameters" else None
+        if isinstance(embedding, nn.Module):
+            self._embedding_hook = embedding.register_forward_hook(self._keep_embedding_output)
         # With two streams, batches alternate between them: the kernels of one batch's backward pass and of
         # the next batch's forward pass then sit in different queues and the many small ones among them run
         # side by side.  A batch's own launches (which share the collector's workspace and store with every
@@ -859,6 +869,10 @@ class OverlappedSteps:
             quiet = getattr(torch.autograd.graph, "set_warn_on_accumulate_grad_stream_mismatch", None)
             if quiet is not None:
                 quiet(False)
+
+    def _keep_embedding_output(self, _module, _inp, out):
+        if self.collector._recording is not None and isinstance(out, Tensor) and out.requires_grad:
+            self._embedding_output = out
 
     @staticmethod
     def _gradients(total: Tensor, outputs: list[Tensor], stream, n_recorded: int):
@@ -895,10 +909,11 @@ class OverlappedSteps:
                 total = losses.sum()
         finally:
             col.end_recording()
-        # The trainable parameters are asked for too (and their gradients dropped, as the plain loop drops
-        # them with zero_grad): the engine then runs the same nodes as `backward()` would, so hooks that
-        # others have put on the model still fire.
-        outputs = record.outputs() + self._trainable
+        # besides the recorded outputs: the embedding's output (see __init__), or the trainable parameters,
+        # whose gradients are dropped as the plain loop drops them with zero_grad
+        root, self._embedding_output = self._embedding_output, None
+        outputs = record.outputs() + ([root] if root is not None else self._trainable)
+        del root
         if self._n_streams > 1 and stream is not None:
             # the previous batch's launch gets the GPU to itself: it starts when this forward pass has
             # finished too, and this batch's backward pass waits for it (an HBM-bound kernel sharing the
@@ -948,6 +963,9 @@ class OverlappedSteps:
             except Exception:
                 pass  # close() runs after a failure too; the first error is the one the caller sees
         self._pool.shutdown(wait=True)
+        if self._embedding_hook is not None:
+            self._embedding_hook.remove()
+            self._embedding_hook = None
         if self._entered:
             self.collector.__exit__(RuntimeError if failed else None, None, None)
             self._entered = False
