@@ -252,7 +252,8 @@ def test_recorded_backward_refuses_outputs_modified_in_place():
             rec.outputs()
 
 
-def test_overlapped_steps_equal_the_plain_loop():
+@pytest.mark.parametrize("embedding_root", [False, True])
+def test_overlapped_steps_equal_the_plain_loop(embedding_root):
     """`OverlappedSteps` (backward pass of batch i on a helper thread beside the forward pass of batch i+1)
     gives every batch the hook calls and losses of the plain loop, batch by batch, in order."""
     from bergson_amd import IndexConfig
@@ -263,6 +264,9 @@ def test_overlapped_steps_equal_the_plain_loop():
             out = super().forward(x)
             logits = torch.cat([out, out.flip(-1)[..., :3]], -1)  # 11 "vocabulary" entries
             return type("O", (), {"logits": logits})()
+
+    if embedding_root:  # the backward pass then stops at the embedding's output instead of the parameters
+        LM.get_input_embeddings = lambda self: self.emb
 
     class Data:
         docs = [[1, 2, 3, 4], [5, 6, 7], [8, 9, 10, 1, 2], [3, 4], [6, 5, 4, 3, 2, 1]]
@@ -289,5 +293,11 @@ def test_overlapped_steps_equal_the_plain_loop():
     for (_, l0, _), (_, l1, _) in zip(plain.batches, over.batches):
         assert torch.equal(l0, l1)
     assert len(plain.seen) == len(over.seen) == 6
+    m.zero_grad()
+    c = _logging_stub(m)
+    CollectorComputer(model=m, data=Data(), collector=c, batches=batches, cfg=cfg,
+                      overlap_backward=True).run_with_collector_hooks()
+    assert all(q.grad is None for q in m.parameters())  # the overlapped loop leaves nothing in .grad
+    assert not m.emb._forward_hooks  # and no hook behind on the embedding
     for (n0, a0, g0, m0), (n1, a1, g1, m1) in zip(plain.seen, over.seen):
         assert n0 == n1 and torch.equal(a0, a1) and torch.equal(g0, g1) and torch.equal(m0, m1)
