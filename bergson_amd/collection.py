@@ -10,10 +10,12 @@ from .gradients import GradientProcessor
 def collect_gradients(model, data, processor: GradientProcessor, cfg: IndexConfig, *,
                       batches: list[list[int]] | None = None, target_modules: set[str] | None = None,
                       attention_cfgs: dict[str, AttentionConfig] | None = None, scorer=None,
-                      preprocess_cfg: PreprocessConfig | None = None, **collector_kwargs):
+                      preprocess_cfg: PreprocessConfig | None = None, overlap_backward: bool | None = None,
+                      **collector_kwargs):
     """Hooks `model.base_model`, runs every batch and writes the store at `cfg.partial_run_path`.
 
     Returns the collector (the reference returns None; callers that ignore the result are unaffected).
+    `overlap_backward` is handed to `CollectorComputer`; other extra keywords go to `GradientCollector`.
     """
     collector = GradientCollector(
         model=model.base_model,
@@ -27,7 +29,8 @@ def collect_gradients(model, data, processor: GradientProcessor, cfg: IndexConfi
         filter_modules=cfg.filter_modules,
         **collector_kwargs,
     )
-    computer = CollectorComputer(model=model, data=data, collector=collector, batches=batches, cfg=cfg)
+    computer = CollectorComputer(model=model, data=data, collector=collector, batches=batches, cfg=cfg,
+                                 overlap_backward=overlap_backward)
     computer.run_with_collector_hooks(desc="New worker - Collecting gradients")
     collector.total_processed = computer.total_processed
     return collector

@@ -64,25 +64,28 @@ def random_docs(lengths: list[int], vocab: int = 50304, seed: int = 0) -> list[l
 
 
 class ListDataset:
-    """Minimal stand-in for a `datasets.Dataset` of token ids: `len`, `column_names`, `ds[list_of_indices]`."""
+    """Minimal stand-in for a `datasets.Dataset` of token ids: `len`, `column_names`, `ds[list_of_indices]`.
+    Optional per-document columns: `labels` (token labels, -100 = not supervised) and `advantage`."""
 
-    def __init__(self, docs: list[list[int]]):
+    def __init__(self, docs: list[list[int]], *, labels: list[list[int]] | None = None,
+                 advantage: list[float] | None = None):
         self.docs = docs
-        self.column_names = ["input_ids", "length"]
+        self.columns = {"input_ids": docs, "length": [len(d) for d in docs]}
+        if labels is not None:
+            self.columns["labels"] = labels
+        if advantage is not None:
+            self.columns["advantage"] = advantage
+        self.column_names = list(self.columns)
 
     def __len__(self) -> int:
         return len(self.docs)
 
     def __getitem__(self, key):
         if isinstance(key, str):
-            if key == "input_ids":
-                return self.docs
-            if key == "length":
-                return [len(d) for d in self.docs]
-            raise KeyError(key)
+            return self.columns[key]
         if isinstance(key, (list, tuple)):
-            return {"input_ids": [self.docs[i] for i in key], "length": [len(self.docs[i]) for i in key]}
-        return {"input_ids": self.docs[key], "length": len(self.docs[key])}
+            return {name: [col[i] for i in key] for name, col in self.columns.items()}
+        return {name: col[key] for name, col in self.columns.items()}
 
 
 def adafactor_moments(base_model, *, scale: float = 1e-4, seed: int = 0) -> dict[str, tuple[torch.Tensor, torch.Tensor]]:

@@ -57,15 +57,18 @@ def pad_and_tensor(sequences: list[list[int]], labels: list[list[int]] | None = 
     return x, y, mask
 
 
-def losses_and_backward(model, x: Tensor, y: Tensor, loss_reduction: str = "sum", label_smoothing: float = 0.0
-                        ) -> Tensor:
-    """collector.py:948-983 (cross-entropy branch)."""
+def losses_and_backward(model, x: Tensor, y: Tensor, loss_reduction: str = "sum", label_smoothing: float = 0.0,
+                        advantage: list[float] | None = None) -> Tensor:
+    """collector.py:948-983 (cross-entropy branch; `advantage` is the batch's optional "advantage" column,
+    :975-976)."""
     logits = model(x).logits[:, :-1]
     masks = y[:, 1:] != -100
     denoms = masks.sum(dim=1, dtype=logits.dtype) if loss_reduction == "mean" else 1.0
     losses = F.cross_entropy(logits.reshape(-1, logits.size(-1)), y[:, 1:].flatten(), reduction="none",
                              label_smoothing=label_smoothing).reshape_as(y[:, 1:])
     losses = losses.sum(1) / denoms
+    if advantage is not None:
+        losses = losses * torch.tensor(advantage, dtype=losses.dtype)
     losses.sum().backward()
     model.zero_grad()
     return losses
@@ -79,8 +82,13 @@ def target_linears(base_model: nn.Module) -> dict[str, nn.Linear]:
 def collect(model, base_model: nn.Module, docs: list[list[int]], batches: list[list[int]], *, p: int | None,
             normalizers: dict | None = None, projection_type: str = "normal", attribute_tokens: bool = False,
             include_bias: bool = False, save_dtype: torch.dtype | None = None, loss_reduction: str = "sum",
-            unit_normalize: bool = False, global_dim: int | None = None) -> tuple[Tensor, Tensor]:
+            unit_normalize: bool = False, global_dim: int | None = None, label_smoothing: float = 0.0,
+            labels: list[list[int]] | None = None, advantages: list[float] | None = None
+            ) -> tuple[Tensor, Tensor]:
     """The whole reference loop on CPU: returns (rows, losses).
+
+    `labels` (per document, -100 = not supervised) and `advantages` (one factor per document) are the
+    dataset's optional "labels" and "advantage" columns (collector.py:877-886, :975-976).
 
     rows is [num_docs, D] (per sequence) or [sum(max(len-1, 0)), D] (per token), in save_dtype.
     global_dim (with p=None) is projection_target="global": every module's unprojected gradient goes through
@@ -141,9 +149,11 @@ def collect(model, base_model: nn.Module, docs: list[list[int]], batches: list[l
     losses_out = torch.zeros(len(docs), dtype=torch.float32)
     try:
         for indices in batches:
-            x, y, mask = pad_and_tensor([docs[i] for i in indices])
+            x, y, mask = pad_and_tensor([docs[i] for i in indices],
+                                        None if labels is None else [labels[i] for i in indices])
             state["mask"] = mask
-            losses = losses_and_backward(model, x, y, loss_reduction)
+            losses = losses_and_backward(model, x, y, loss_reduction, label_smoothing,
+                                         None if advantages is None else [advantages[i] for i in indices])
             if global_dim is not None:  # finalize_global_projection, collector.py:392-402
                 mod_grads["gradients"] = mod_grads["gradients"].to(save_dtype)
                 grad_sizes = {"gradients": global_dim}

@@ -34,7 +34,10 @@ def scorer_score(index_grads: dict[str, Tensor], query_grads: dict[str, Tensor],
 def normalize_and_aggregate_queries(query_grads: dict[str, Tensor], modules: list[str], *, unit_normalize: bool,
                                     aggregation: str = "none", normalize_aggregated: bool = False
                                     ) -> dict[str, Tensor]:
-    """process_grads.py:139-182: fp32 per-query unit norm over all modules, then mean / sum over queries."""
+    """process_grads.py:139-182: fp32 per-query unit norm over all modules, then mean / sum over queries, then
+    (optionally) one norm over everything that is left; nothing to do = inputs returned in their dtype."""
+    if aggregation == "none" and not unit_normalize:
+        return {m: query_grads[m] for m in modules}
     q = {m: query_grads[m].to(torch.float32) for m in modules}
     if unit_normalize:
         norms = torch.cat([q[m] for m in modules], dim=1).norm(dim=1, keepdim=True)
@@ -43,8 +46,8 @@ def normalize_and_aggregate_queries(query_grads: dict[str, Tensor], modules: lis
         q = {m: q[m].mean(dim=0, keepdim=True) for m in modules}
     elif aggregation == "sum":
         q = {m: q[m].sum(dim=0, keepdim=True) for m in modules}
-    if aggregation != "none" and normalize_aggregated:
-        norm = torch.cat([q[m] for m in modules], dim=1).norm(dim=1, keepdim=True)
+    if normalize_aggregated:
+        norm = torch.cat([q[m].flatten() for m in modules], dim=0).norm()
         q = {m: q[m] / norm for m in modules}
     return q
 

@@ -287,3 +287,39 @@ def test_overlapped_loop_equals_plain_loop_bitwise(device, attribute_tokens):
         OverlappedSteps.__init__ = init
     assert np.abs(plain.astype(np.float32)).sum() > 0
     assert all(p.grad is None for p in model.parameters())
+
+
+@pytest.mark.parametrize("overlap", [True, False])
+@pytest.mark.parametrize("reduction,smoothing,use_labels,use_advantage", [
+    ("mean", 0.0, False, False),
+    ("sum", 0.1, False, False),
+    ("mean", 0.1, True, False),
+    ("sum", 0.0, True, True),
+    ("mean", 0.1, False, True),
+])
+def test_loss_options_match_cpu_loop(device, reduction, smoothing, use_labels, use_advantage, overlap):
+    """`loss_reduction="mean"`, `label_smoothing`, prompt-masked labels and the advantage column
+    (bergson/collector/collector.py:948-983): the product loop, plain and overlapped, against the oracle's
+    loop, whose loss arithmetic is pinned against autograd on the CPU."""
+    from bergson_amd import IndexConfig, allocate_batches, collect_gradients
+    from bergson_amd.synthetic import ListDataset, make_gpt_neox, random_docs
+
+    lengths = [31, 18, 2, 25, 9, 40]
+    docs = random_docs(lengths, seed=13)
+    labels = [[-100] * (len(d) // 3) + d[len(d) // 3:] for d in docs] if use_labels else None
+    advantage = [0.5, -1.5, 2.0, 1.0, 0.25, -0.75] if use_advantage else None
+    batches = allocate_batches(lengths, 80)
+    model_cpu = make_gpt_neox("pythia-14m", torch.float32, "cpu", seed=0, layers=2)
+    want, want_losses = oloop.collect(model_cpu, model_cpu.base_model, docs, batches, p=16, loss_reduction=reduction,
+                                      label_smoothing=smoothing, labels=labels, advantages=advantage)
+    model = make_gpt_neox("pythia-14m", torch.float32, device, seed=0, layers=2)
+    cfg = IndexConfig(run_path="", projection_dim=16, projection_type="normal", loss_reduction=reduction,
+                      label_smoothing=smoothing)
+    data = ListDataset(docs, labels=labels, advantage=advantage)
+    col = collect_gradients(model, data, _processor(16), cfg, batches=batches, overlap_backward=overlap)
+    torch.cuda.synchronize()
+    got = torch.from_numpy(np.array(col.builder.grad_buffer))
+    assert rel_l2(got, want) <= 1e-3
+    assert torch.allclose(col.per_doc_losses.cpu(), want_losses, rtol=1e-4, atol=1e-4)
+    for i in range(len(docs)):  # row by row: a short document must not hide behind a long one
+        assert rel_l2(got[i], want[i]) <= 2e-3, i

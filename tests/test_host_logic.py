@@ -301,3 +301,42 @@ def test_overlapped_steps_equal_the_plain_loop(embedding_root):
     assert not m.emb._forward_hooks  # and no hook behind on the embedding
     for (n0, a0, g0, m0), (n1, a1, g1, m1) in zip(plain.seen, over.seen):
         assert n0 == n1 and torch.equal(a0, a1) and torch.equal(g0, g1) and torch.equal(m0, m1)
+
+
+@pytest.mark.parametrize("unit", [False, True])
+@pytest.mark.parametrize("agg", ["none", "mean", "sum"])
+@pytest.mark.parametrize("norm_agg", [False, True])
+def test_query_normalisation_and_aggregation(unit, agg, norm_agg):
+    """`normalize_and_aggregate_grads` against the oracle's restatement and against the formulas in float64."""
+    import numpy as np
+    from bergson_amd import normalize_and_aggregate_grads, normalize_flat_grad
+    from oracle import scan as oscan
+
+    gen = torch.Generator().manual_seed(4)
+    grads = {"b": torch.randn(5, 7, generator=gen).to(torch.float16), "a": torch.randn(5, 3, generator=gen).to(torch.float16)}
+    names = ["a", "b"]
+    got = normalize_and_aggregate_grads(grads, names, unit, torch.device("cpu"), agg, norm_agg)
+    want = oscan.normalize_and_aggregate_queries(grads, names, unit_normalize=unit, aggregation=agg,
+                                                 normalize_aggregated=norm_agg)
+    assert list(got) == names
+    for n in names:
+        assert got[n].shape == want[n].shape and got[n].dtype == want[n].dtype
+        assert torch.allclose(got[n].float(), want[n].float(), rtol=1e-6, atol=1e-7)
+    m = np.concatenate([grads["a"].double().numpy(), grads["b"].double().numpy()], axis=1)
+    if unit or agg != "none":
+        if unit:
+            m = m / np.sqrt((m ** 2).sum(1, keepdims=True))
+        if agg == "mean":
+            m = m.mean(0, keepdims=True)
+        elif agg == "sum":
+            m = m.sum(0, keepdims=True)
+        if norm_agg:
+            m = m / np.sqrt((m ** 2).sum())
+    flat = torch.cat([got["a"], got["b"]], dim=1).double().numpy()
+    assert np.allclose(flat, m, rtol=1e-5, atol=1e-7)
+    v = normalize_flat_grad(grads["b"], torch.device("cpu"))
+    assert v.dtype == torch.float16 and abs(float(v.float().norm()) - 1.0) < 1e-3
+    with pytest.warns(UserWarning):
+        assert not normalize_flat_grad(torch.zeros(4), torch.device("cpu")).any()
+    with pytest.raises(ValueError):
+        normalize_and_aggregate_grads(grads, names, True, torch.device("cpu"), "median")
