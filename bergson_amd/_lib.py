@@ -11,7 +11,7 @@ from pathlib import Path
 LIB_PATH = Path(__file__).resolve().parent / "libbergson_amd.so"
 
 BGX_F32, BGX_F16, BGX_BF16 = 0, 1, 2
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 
 class ModuleDesc(C.Structure):
@@ -51,6 +51,7 @@ class BlockDesc(C.Structure):
 SIGNATURES: dict[str, tuple] = {
     "bgx_abi_version": (C.c_int, []),
     "bgx_last_error": (C.c_char_p, []),
+    "bgx_reload_switches": (C.c_int, []),
     "bgx_adafactor_scales": (
         C.c_int,
         [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p],
@@ -143,6 +144,11 @@ def load() -> C.CDLL:
         raise ImportError(f"{LIB_PATH}: ABI version {got}, expected {ABI_VERSION}")
     _lib = lib
     return lib
+
+
+def reload_switches() -> None:
+    """Make the library read its BGX_* environment switches again (they are read once otherwise)."""
+    load().bgx_reload_switches()
 
 
 def check(rc: int, what: str) -> None:

@@ -532,9 +532,11 @@ class HookCollectorBase(ContextDecorator, ABC):
             prep = ops.AdamPrepared(right[:, :i].contiguous(), r_out, normalizer.weight_avg_sq, out_col,
                                     bias_col=right[:, i], bias_avg_sq=normalizer.bias_avg_sq)
         else:
-            parent = self.split_head_name(name)
-            right_name = parent[0] if parent is not None and parent[0] in self.attention_cfgs else name
-            r_in = self.projection(right_name, p, i, "right", g.device, g.dtype)
+            # the Adam branch projects in the backward hook, under the name the module carries there: for a
+            # split attention module every head has a right projection of its own, "<module>.head_h/right"
+            # (collector.py:545-550, :626-644), unlike the other branches, whose input side is projected in
+            # the forward hook under the parent's name
+            r_in = self.projection(name, p, i, "right", g.device, g.dtype)
             prep = ops.AdamPrepared(r_in, r_out, normalizer.weight_avg_sq, out_col)
         self._adam_prepared[key] = prep
         return prep
@@ -854,7 +856,7 @@ class OverlappedSteps:
         self._embedding_hook = None
         embedding = getattr(model, "get_input_embeddings", None)
         embedding = embedding() if callable(embedding) and os.environ.get("BGX_OVERLAP_ROOT") != "parameters" else None
-        if isinstance(embedding, nn.Module):
+        if isinstance(embedding, nn.Module) and not self._has_foreign_hooks(embedding):
             self._embedding_hook = embedding.register_forward_hook(self._keep_embedding_output)
         # With two streams, batches alternate between them: the kernels of one batch's backward pass and of
         # the next batch's forward pass then sit in different queues and the many small ones among them run
@@ -869,6 +871,21 @@ class OverlappedSteps:
             quiet = getattr(torch.autograd.graph, "set_warn_on_accumulate_grad_stream_mismatch", None)
             if quiet is not None:
                 quiet(False)
+
+    @staticmethod
+    def _has_foreign_hooks(embedding: nn.Module) -> bool:
+        """Whether someone else watches the input embedding: hooks on the module, or on its parameters'
+        gradients.  Stopping the backward pass at the embedding's output leaves the embedding's own backward
+        node out (the reference runs it: the embedding is the one trainable module,
+        bergson/utils/worker_utils.py:224-225), so such hooks would not fire; with them present the backward
+        pass goes down to the parameters as `backward()` does."""
+        module_hooks = ("_forward_hooks", "_forward_pre_hooks", "_backward_hooks", "_backward_pre_hooks")
+        if any(len(getattr(embedding, attr, None) or ()) for attr in module_hooks):
+            return True
+        for q in embedding.parameters(recurse=False):
+            if getattr(q, "_backward_hooks", None) or getattr(q, "_post_accumulate_grad_hooks", None):
+                return True
+        return False
 
     def _keep_embedding_output(self, _module, _inp, out):
         if self.collector._recording is not None and isinstance(out, Tensor) and out.requires_grad:

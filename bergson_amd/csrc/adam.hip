@@ -681,12 +681,14 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
   const bool fused = dtype != BGX_F32 && O % FUSED_TILE == 0 && I % 64 == 0 && p <= 32 && bias_col == nullptr &&
                      (uintptr_t)a % 16 == 0 && (uintptr_t)g % 16 == 0 && (uintptr_t)r_out % 16 == 0 &&
                      (uintptr_t)table % 16 == 0 && a_tok_stride % 8 == 0 && g_seq_stride % 8 == 0 &&
-                     g_tok_stride % 8 == 0 && getenv("BGX_ADAM_FUSED_OFF") == nullptr;
+                     g_tok_stride % 8 == 0 && !switches().adam_fused_off;
   if (fused) {
     // no H: the region reserved for it holds the per-token fp32 results, so a chunk can be much larger
-    int64_t fc = (int64_t)((size_t)tc * O * p * 4 / ((size_t)pp * 4));
-    fc = fc / FUSED_TILE * FUSED_TILE;
-    if (fc > T) fc = T;
+    // (tc * O / p tokens; O >= 256 and p <= 32 make that at least 8 tc, so a batch smaller than one tile is
+    // a single pass of T tokens -- the kernel bounds partial tiles by `tokens`)
+    const int64_t cap = (int64_t)((size_t)tc * O * p * 4 / ((size_t)pp * 4));
+    int64_t fc = cap >= T ? T : cap / FUSED_TILE * FUSED_TILE;
+    if (fc <= 0) fc = cap;
     float* ptok_f = (float*)w;
     constexpr size_t smem = 2 * (size_t)(2 * FUSED_TILE) * LDS_ROW_BYTES;
     for (int64_t t0 = 0; t0 < T; t0 += fc) {
@@ -719,8 +721,8 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
             ttx = c;
             break;
           }
-        if (const char* e = getenv("BGX_ADAM_TTX")) {
-          const int v = atoi(e);
+        if (switches().adam_ttx >= 0) {
+          const int v = switches().adam_ttx;
           if (v == 0 || ((v == 2 || v == 4 || v == 8 || v == 16) && grid.x % v == 0 && p % (32 / v) == 0)) ttx = v;
         }
       }

@@ -1,6 +1,9 @@
 // extern "C" entry points of libbergson_amd.so (declared in include/bergson_amd.h).
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
+
+#include <atomic>
 
 #include "common.hpp"
 
@@ -20,11 +23,47 @@ int hip_fail(hipError_t e, const char* what) {
   return (int)e;
 }
 
+static const Switches* read_switches() {
+  Switches* s = new Switches;
+  auto off = [](const char* name) {
+    const char* e = getenv(name);
+    return e != nullptr && e[0] == '0';
+  };
+  s->adam_fused_off = getenv("BGX_ADAM_FUSED_OFF") != nullptr;
+  if (const char* e = getenv("BGX_ADAM_TTX")) s->adam_ttx = atoi(e);
+  s->collect_staged = !off("BGX_COLLECT_STAGED");
+  s->collect_persist = !off("BGX_COLLECT_PERSIST");
+  s->collect_lpt_off = getenv("BGX_COLLECT_LPT_OFF") != nullptr;
+  s->scan_direct_off = getenv("BGX_SCAN_DIRECT_OFF") != nullptr;
+  s->scan_stream_off = getenv("BGX_SCAN_STREAM_OFF") != nullptr;
+  s->scan_wide_off = getenv("BGX_SCAN_WIDE_OFF") != nullptr;
+  return s;
+}
+
+// The current record.  A superseded record is never freed (a launch on another thread may still be reading
+// it; a record is a few bytes and reloading is something only tests do).
+static std::atomic<const Switches*> g_switches{nullptr};
+
+const Switches& switches() {
+  const Switches* s = g_switches.load(std::memory_order_acquire);
+  if (s == nullptr) {
+    const Switches* fresh = read_switches();
+    if (g_switches.compare_exchange_strong(s, fresh, std::memory_order_acq_rel))
+      s = fresh;
+    else
+      delete fresh;
+  }
+  return *s;
+}
+
+void reload_switches() { g_switches.store(read_switches(), std::memory_order_release); }
+
 size_t collect_workspace_bytes(int n_modules, int N, int S, int p);
 size_t collect_workspace_bytes_for(const bgx_module_desc* mods, int n_modules, int N, int S, int p, int in_dtype);
 int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules, int N, int S, int p, int in_dtype,
                  const int32_t* lengths, const int64_t* rows_or_offsets, void* out, int64_t out_row_stride,
-                 int out_dtype, float lo, float hi, void* ws, size_t ws_bytes, void* stream);
+                 int out_dtype, float lo, float hi, void* ws, size_t ws_bytes, void* stream,
+                 bool tables_by_kernel = false);
 int adafactor_scales_impl(const float* row, int O, const float* col, int I, int dtype, float* row_scale,
                           float* col_scale, void* stream);
 size_t adam_table_bytes(int O, int I, int p, int dtype);
@@ -84,6 +123,11 @@ int bgx_gram_accumulate(const void* rows_dev, int32_t dtype, int64_t row_stride,
 }
 
 int bgx_abi_version(void) { return BGX_ABI_VERSION; }
+
+int bgx_reload_switches(void) {
+  bgx::reload_switches();
+  return 0;
+}
 
 const char* bgx_last_error(void) { return bgx::g_err; }
 

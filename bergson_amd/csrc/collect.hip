@@ -25,6 +25,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <mutex>
 #include <type_traits>
 #include <queue>
 #include <vector>
@@ -714,11 +715,15 @@ __global__ __launch_bounds__(256) void unit_normalize_kernel(T* rows, int64_t n_
 }
 
 // ---- host side ------------------------------------------------------------------------
-// Optional event pairs around collect_kernel (benchmark support).
+// Optional event pairs around collect_kernel (benchmark support).  Launches may come from several host
+// threads and streams at once (each pair is recorded on its own launch's stream); a launch claims its pair
+// under the lock.  Enabling and reading are for the thread that owns the measurement, between launches.
+static std::mutex g_timing_lock;
 static std::vector<hipEvent_t> g_timing_events;  // start0, stop0, start1, stop1, ...
 static int g_timing_used = 0;
 
 int collect_timing_enable(int max_launches) {
+  std::lock_guard<std::mutex> hold(g_timing_lock);
   for (hipEvent_t e : g_timing_events) (void)hipEventDestroy(e);
   g_timing_events.clear();
   g_timing_used = 0;
@@ -733,12 +738,53 @@ int collect_timing_enable(int max_launches) {
 
 int collect_timing_read(float* ms_out, int capacity, int* count_out) {
   BGX_REQUIRE(ms_out && count_out && capacity >= 0, BGX_E_ARG, "collect_timing_read: null output");
+  std::lock_guard<std::mutex> hold(g_timing_lock);
   const int n = g_timing_used < capacity ? g_timing_used : capacity;
   for (int i = 0; i < n; ++i) {
     BGX_HIP(hipEventSynchronize(g_timing_events[2 * i + 1]));
     BGX_HIP(hipEventElapsedTime(&ms_out[i], g_timing_events[2 * i], g_timing_events[2 * i + 1]));
   }
   *count_out = n;
+  return 0;
+}
+
+// The event pair of the next timed launch, or false when timing is off or the pairs are used up.
+static bool claim_timing_pair(hipEvent_t* start, hipEvent_t* stop) {
+  std::lock_guard<std::mutex> hold(g_timing_lock);
+  if (2 * (g_timing_used + 1) > (int)g_timing_events.size()) return false;
+  *start = g_timing_events[2 * g_timing_used];
+  *stop = g_timing_events[2 * g_timing_used + 1];
+  ++g_timing_used;
+  return true;
+}
+
+// ---- host words into device memory without a copy engine ------------------------------------------------
+// A launch's descriptor table normally reaches the workspace by hipMemcpyAsync from pageable memory.  For the
+// entry point that must not allocate or stage anything, the same bytes travel as kernel arguments instead:
+// 3584 bytes per launch, written by the kernel itself.
+constexpr int POKE_WORDS = 896;
+struct PokeArgs {
+  uint32_t words[POKE_WORDS];
+};
+__global__ void __launch_bounds__(256) poke_kernel(uint32_t* __restrict__ dst, int n, const PokeArgs a) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) dst[i] = a.words[i];
+}
+
+static int upload(void* dst, const void* src, size_t bytes, hipStream_t st, bool by_kernel) {
+  if (!by_kernel) {
+    BGX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, st));
+    return 0;
+  }
+  BGX_REQUIRE(bytes % 4 == 0, BGX_E_ARG, "collect: table of %zu bytes is not a whole number of words", bytes);
+  const size_t words = bytes / 4;
+  for (size_t w0 = 0; w0 < words; w0 += POKE_WORDS) {
+    PokeArgs a;
+    const int n = (int)std::min<size_t>(POKE_WORDS, words - w0);
+    memcpy(a.words, (const char*)src + w0 * 4, (size_t)n * 4);
+    hipLaunchKernelGGL(poke_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (uint32_t*)dst + w0, n, a);
+    BGX_HIP(hipGetLastError());
+  }
   return 0;
 }
 
@@ -893,7 +939,7 @@ static size_t persist_scratch_bytes(int tile_tokens) {
 int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules, int N, int S,
                  int p, int in_dtype, const int32_t* lengths, const int64_t* rows_or_offsets,
                  void* out, int64_t out_row_stride, int out_dtype, float lo, float hi, void* ws,
-                 size_t ws_bytes, void* stream) {
+                 size_t ws_bytes, void* stream, bool tables_by_kernel) {
   BGX_REQUIRE(mods_host && out && ws, BGX_E_ARG, "collect: null mods/out/workspace");
   BGX_REQUIRE(n_modules > 0 && N > 0 && S > 0, BGX_E_ARG, "collect: n_modules=%d N=%d S=%d", n_modules, N, S);
   BGX_REQUIRE(n_modules <= 65535, BGX_E_SHAPE, "collect: n_modules=%d exceeds 65535", n_modules);
@@ -967,7 +1013,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   bool staged = persist && persist_lds + stage_bytes <= LDS_PER_WG;
   for (int m = 0; m < n_modules && staged; ++m)
     staged = sorted[m].I % (2 * kstep) == 0 && sorted[m].O % (2 * kstep) == 0;
-  if (const char* e = getenv("BGX_COLLECT_STAGED")) staged = staged && e[0] != '0';
+  staged = staged && switches().collect_staged;
   if (staged) persist_lds += stage_bytes;
   // Modules too wide for LDS: the streamed kernel with the fragments in a global table, when the caller's
   // workspace has room for it (bgx_collect_workspace_bytes_for) -- else the tile kernel.
@@ -975,24 +1021,22 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   const size_t frag_ws_off = align_up(need, 256);
   bool rfg = !persist && pb == 1 && aligned && !any_bias && tiles * n_modules <= 0x7fffffffLL && frag_bytes > 0 &&
              ws_bytes >= frag_ws_off + frag_bytes;
-  if (const char* e = getenv("BGX_COLLECT_STAGED")) rfg = rfg && e[0] != '0';
+  rfg = rfg && switches().collect_staged;
   if (rfg) {
     persist = staged = true;
     r_steps = 0;
     persist_lds = scratch_bytes + stage_bytes;
   }
   // BGX_COLLECT_PERSIST=0 in the environment forces the one-workgroup-per-tile kernel (tests, comparisons)
-  if (const char* e = getenv("BGX_COLLECT_PERSIST")) {
-    persist = persist && e[0] != '0';
-    rfg = rfg && persist;
-  }
+  persist = persist && switches().collect_persist;
+  rfg = rfg && persist;
 
   std::vector<unsigned char> head((size_t)n_modules * sizeof(bgx_module_desc));
   memcpy(head.data(), sorted.data(), head.size());
   // table variant: room behind the table for the item list that lets the workgroups take items out of order
   const size_t order_ws_off = align_up(frag_ws_off + frag_bytes, 256);
   const bool rfg_order = rfg && ws_bytes >= order_ws_off + (size_t)tiles * n_modules * sizeof(int32_t) &&
-                         getenv("BGX_COLLECT_LPT_OFF") == nullptr;
+                         !switches().collect_lpt_off;
   std::vector<int32_t> order;
   int wgs = 0;
   if (persist) {
@@ -1080,10 +1124,11 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
       memcpy(head.data() + frag_off_offset(n_modules), foff.data(), foff.size() * sizeof(int64_t));
     }
   }
-  BGX_HIP(hipMemcpyAsync(mods_dev, head.data(), head.size(), hipMemcpyHostToDevice, st));
+  if (const int rc = upload(mods_dev, head.data(), head.size(), st, tables_by_kernel)) return rc;
   if (!order.empty())
-    BGX_HIP(hipMemcpyAsync((char*)ws + order_ws_off, order.data(), order.size() * sizeof(int32_t), hipMemcpyHostToDevice,
-                           st));
+    if (const int rc = upload((char*)ws + order_ws_off, order.data(), order.size() * sizeof(int32_t), st,
+                              tables_by_kernel))
+      return rc;
   uint4* frag_dev = (uint4*)((char*)ws + frag_ws_off);
   const int64_t* frag_off_dev = (const int64_t*)((const char*)ws + frag_off_offset(n_modules));
   if (rfg) {
@@ -1107,8 +1152,9 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   args.hi = hi;
 
   const dim3 grid((unsigned)tiles, (unsigned)n_modules);
-  const bool timed = 2 * (g_timing_used + 1) <= (int)g_timing_events.size();
-  if (timed) BGX_HIP(hipEventRecord(g_timing_events[2 * g_timing_used], st));
+  hipEvent_t ev_start, ev_stop;
+  const bool timed = claim_timing_pair(&ev_start, &ev_stop);
+  if (timed) BGX_HIP(hipEventRecord(ev_start, st));
   if (persist) {
     PersistArgs pa;
     pa.c = args;
@@ -1139,10 +1185,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     launch_collect_pb<bf16_t>(pb, aligned, per_token, any_bias, tile_tokens, grid, st, args);
   }
   BGX_HIP(hipGetLastError());
-  if (timed) {
-    BGX_HIP(hipEventRecord(g_timing_events[2 * g_timing_used + 1], st));
-    ++g_timing_used;
-  }
+  if (timed) BGX_HIP(hipEventRecord(ev_stop, st));
 
   if (!per_token) {
     hipLaunchKernelGGL(collect_finalize_kernel, dim3((unsigned)N, (unsigned)n_modules), dim3(256), 0, st,

@@ -27,6 +27,21 @@ int hip_fail(hipError_t e, const char* what);
     }                                \
   } while (0)
 
+// ---- diagnostic switches (defined in capi.hip) --------------------------------
+// BGX_* environment variables that force a kernel variant, for tests and comparisons.  They are read once,
+// on first use, into an immutable record; bgx_reload_switches() publishes a fresh one.
+struct Switches {
+  bool adam_fused_off = false;    // BGX_ADAM_FUSED_OFF set
+  int adam_ttx = -1;              // BGX_ADAM_TTX (token tiles per XCD group), -1 = unset
+  bool collect_staged = true;     // BGX_COLLECT_STAGED != "0"
+  bool collect_persist = true;    // BGX_COLLECT_PERSIST != "0"
+  bool collect_lpt_off = false;   // BGX_COLLECT_LPT_OFF set
+  bool scan_direct_off = false;   // BGX_SCAN_DIRECT_OFF set
+  bool scan_stream_off = false;   // BGX_SCAN_STREAM_OFF set
+  bool scan_wide_off = false;     // BGX_SCAN_WIDE_OFF set
+};
+const Switches& switches();
+
 // ---- vector types for the MFMA builtins -----------------------------------
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;

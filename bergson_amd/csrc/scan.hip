@@ -1049,7 +1049,7 @@ static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
     a.n_parts = a.q_tiles * 4;
     if constexpr (sizeof(T) == 2) {
       // aligned 16-bit operands, D a multiple of the K tile: tiles loaded straight into LDS
-      if (aligned && a.D % 64 == 0 && getenv("BGX_SCAN_DIRECT_OFF") == nullptr) {
+      if (aligned && a.D % 64 == 0 && !switches().scan_direct_off) {
         const int row_tiles_pad = (a.row_tiles + 7) / 8 * 8;
         auto launch = [&](auto kern, int bn, unsigned wgs) -> int {
           BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, sd_lds_bytes(bn)));
@@ -1184,7 +1184,7 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
     BGX_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
   }
   const bool stream_ok = table_bytes > 0 && aligned && ws != nullptr && ((uintptr_t)ws & 255) == 0 &&
-                         ws_bytes >= table_off + table_bytes && getenv("BGX_SCAN_STREAM_OFF") == nullptr;
+                         ws_bytes >= table_off + table_bytes && !switches().scan_stream_off;
   // With top-k the streaming scan opens with one tile per workgroup and no thresholds (the select kernel
   // cuts that pass's one-entry-per-row lists down); every later pass is as long as the workspace allows.
   const int64_t stream_first = (int64_t)std::max(cus, 1) * SS_TILE_ROWS;

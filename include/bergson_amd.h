@@ -13,9 +13,10 @@
  *     before anything was enqueued.  bgx_last_error() gives the message of
  *     the last failure on the calling thread.
  *   - all pointers named *_dev are device pointers owned by the caller; the
- *     library allocates nothing and never synchronises the host: all work is
- *     enqueued on `stream` (a hipStream_t passed as void*; NULL = the null
- *     stream).
+ *     library allocates no device memory and never synchronises the host: all
+ *     work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the
+ *     null stream).  Entry points that take a host table (mods_host,
+ *     blocks_host) copy it to the workspace with hipMemcpyAsync.
  *   - "rows" are store rows; "tokens" are (sequence, position) pairs.
  *   - dtypes are BGX_F32 / BGX_F16 / BGX_BF16.
  */
@@ -29,7 +30,7 @@
 extern "C" {
 #endif
 
-#define BGX_ABI_VERSION 5
+#define BGX_ABI_VERSION 6
 
 enum bgx_dtype { BGX_F32 = 0, BGX_F16 = 1, BGX_BF16 = 2 };
 
@@ -81,6 +82,15 @@ typedef struct bgx_module_desc {
 
 int bgx_abi_version(void);
 const char* bgx_last_error(void);
+
+/* Diagnostics (no counterpart in the reference).  A handful of BGX_*
+ * environment variables force a kernel variant, so that tests can compare the
+ * variants (BGX_COLLECT_PERSIST=0, BGX_COLLECT_STAGED=0, BGX_COLLECT_LPT_OFF,
+ * BGX_ADAM_FUSED_OFF, BGX_ADAM_TTX=n, BGX_SCAN_DIRECT_OFF, BGX_SCAN_STREAM_OFF,
+ * BGX_SCAN_WIDE_OFF).  The library reads them once, on its first launch;
+ * bgx_reload_switches() reads them again.  Launches that are being issued from
+ * other threads at that moment see either the old or the new settings. */
+int bgx_reload_switches(void);
 
 /* Adafactor factors of one module, computed once per module.
  * Replaces collector.py:532-535 and :655-658 (closed form in
@@ -236,7 +246,10 @@ int bgx_fullgrad_tok(const void* a_dev, const void* g_dev,
  *   bgx_collect_timing_enable(n)  n > 0: start recording, at most n launches;
  *                                 n = 0: stop and release the events
  *   bgx_collect_timing_read(ms, capacity, &count): waits for the recorded
- *       events and writes each launch's kernel time in milliseconds. */
+ *       events and writes each launch's kernel time in milliseconds.
+ * Launches from several threads and streams may be in flight while recording is
+ * on (each claims its pair under a lock and records it on its own stream);
+ * enable and read belong to one thread, between launches. */
 int bgx_collect_timing_enable(int32_t max_launches);
 int bgx_collect_timing_read(float* ms_out, int32_t capacity, int32_t* count_out);
 

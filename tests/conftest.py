@@ -23,3 +23,28 @@ def device():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     return torch.device("cuda:0")
+
+
+@pytest.fixture
+def bgx_env():
+    """bgx_env(name, value) sets one of the library's BGX_* switches for the running test (None removes it)
+    and makes the library read its switches again; everything is put back afterwards."""
+    from bergson_amd import _lib
+
+    saved: dict[str, str | None] = {}
+
+    def set_switch(name: str, value):
+        saved.setdefault(name, os.environ.get(name))
+        if value is None:
+            os.environ.pop(name, None)
+        else:
+            os.environ[name] = str(value)
+        _lib.reload_switches()
+
+    yield set_switch
+    for name, old in saved.items():
+        if old is None:
+            os.environ.pop(name, None)
+        else:
+            os.environ[name] = old
+    _lib.reload_switches()

@@ -103,6 +103,46 @@ def test_attention_head_split(device):
         assert rel_l2(got[:, h * 256:(h + 1) * 256], want) <= 1e-4
 
 
+@pytest.mark.parametrize("attribute_tokens", [False, True])
+def test_attention_head_split_adam(device, attribute_tokens):
+    """With an Adam normalizer a head is projected on BOTH sides under its own name (the reference's Adam
+    branch calls double_sided_projection with the head's name, bergson/collector/collector.py:545-550,
+    :626-644), and its second moments are the head's rows of the module's."""
+    from bergson_amd import AdamNormalizer, AttentionConfig, GradientCollector, IndexConfig
+    from bergson_amd.collector import CollectorComputer
+
+    lengths = [30, 21]
+    docs, data, batches, cpu, gpu = _setup(device, lengths, layers=1)
+    name = "layers.0.attention.dense"
+    heads, hs = 4, 32
+    gen = torch.Generator().manual_seed(1)
+    v = torch.rand(128, 128, generator=gen) * 1e-4 + 1e-8
+    cap = {}
+    mod = gpu.base_model.get_submodule(name)
+    h1 = mod.register_forward_hook(lambda m, i, o: cap.__setitem__("a", i[0].detach().cpu()))
+    h2 = mod.register_full_backward_hook(lambda m, gi, go: cap.__setitem__("g", go[0].detach().cpu()))
+    cfg = IndexConfig(projection_dim=16, projection_type="normal", attribute_tokens=attribute_tokens)
+    col = GradientCollector(model=gpu.base_model, cfg=cfg, data=data, target_modules={name},
+                            processor=_proc(16, {name: AdamNormalizer(v.to(device))}),
+                            attention_cfgs={name: AttentionConfig(heads, hs, 2)})
+    CollectorComputer(model=gpu, data=data, collector=col, batches=[[0, 1]], cfg=cfg).run_with_collector_hooks()
+    h1.remove(), h2.remove()
+    got = torch.from_numpy(np.array(col.builder.grad_buffer))
+    a, g = cap["a"], cap["g"]
+    mask = (torch.arange(30).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+    assert got.shape == (int(mask.sum()) if attribute_tokens else 2, heads * 256)
+    for h in range(heads):
+        left = projection_matrix(f"{name}.head_{h}/left", 16, hs, torch.float32)
+        right = projection_matrix(f"{name}.head_{h}/right", 16, 128, torch.float32)
+        want = ohooks.module_gradient(a, g[:, :, h * hs:(h + 1) * hs], ohooks.Adam(v[h * hs:(h + 1) * hs]), left,
+                                      right, attribute_tokens=attribute_tokens,
+                                      collection_mask=mask if attribute_tokens else None)
+        assert rel_l2(got[:, h * 256:(h + 1) * 256], want) <= 1e-4, h
+    # the parent's matrix is another one: sharing it would not pass
+    assert not torch.equal(projection_matrix(f"{name}/right", 16, 128, torch.float32),
+                           projection_matrix(f"{name}.head_0/right", 16, 128, torch.float32))
+
+
 def test_scorer_on_the_fly_matches_oracle(device, tmp_path):
     from bergson_amd import IndexConfig, Scorer, collect_gradients
     from bergson_amd.data import load_scores

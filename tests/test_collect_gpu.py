@@ -13,16 +13,12 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.fixture(params=["streamed", "persistent", "grid"], autouse=True)
-def kernel_variant(request, monkeypatch):
+def kernel_variant(request, bgx_env):
     """Every case runs three times: with the persistent collection kernel and its streamed loads where they
     apply (the default), with the persistent kernel's direct fragment loads, and with the
     one-workgroup-per-tile kernel, the latter two forced through the library's environment switches."""
-    monkeypatch.delenv("BGX_COLLECT_PERSIST", raising=False)
-    monkeypatch.delenv("BGX_COLLECT_STAGED", raising=False)
-    if request.param == "grid":
-        monkeypatch.setenv("BGX_COLLECT_PERSIST", "0")
-    elif request.param == "persistent":
-        monkeypatch.setenv("BGX_COLLECT_STAGED", "0")
+    bgx_env("BGX_COLLECT_PERSIST", "0" if request.param == "grid" else None)
+    bgx_env("BGX_COLLECT_STAGED", "0" if request.param == "persistent" else None)
     return request.param
 
 
@@ -570,7 +566,7 @@ def test_adam_seq_with_lengths_and_rows(device):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("p", [16, 32])
 @pytest.mark.parametrize("per_token", [False, True])
-def test_adam_fused_path(device, dtype, p, per_token, monkeypatch):
+def test_adam_fused_path(device, dtype, p, per_token, bgx_env):
     """Shapes the fused Adam kernel takes (16-bit, O % 256 == 0, I % 64 == 0, p <= 32): several token tiles,
     two chunks of output features, ragged lengths; against the oracle and against the two-kernel path."""
     N, S, I, O = 3, 200, 128, 512
@@ -592,13 +588,13 @@ def test_adam_fused_path(device, dtype, p, per_token, monkeypatch):
         kw = dict(chunk_tokens=256)  # the per-token formulation, summed per sequence
     got = _run_adam(device, case, p, dtype, **kw)
     assert rel_l2(got, want) <= TOL[dtype]
-    monkeypatch.setenv("BGX_ADAM_FUSED_OFF", "1")
+    bgx_env("BGX_ADAM_FUSED_OFF", "1")
     other = _run_adam(device, case, p, dtype, **kw)
     assert rel_l2(got, other) <= TOL[dtype]
 
 
 @pytest.mark.parametrize("ttx", [None, 2, 8])
-def test_adam_fused_xcd_order(device, ttx, monkeypatch):
+def test_adam_fused_xcd_order(device, ttx, bgx_env):
     """A grid of 256 workgroups (8 token tiles x 32 columns): the fused kernel then deals (token tile, column)
     pairs to the workgroups so that those sharing an XCD share operands.  Every pair must still be taken exactly
     once: the rows equal those of the plain order bit for bit, and the oracle's within tolerance."""
@@ -614,9 +610,9 @@ def test_adam_fused_xcd_order(device, ttx, monkeypatch):
     offs = [0, counts[0]]
     kw = dict(per_token=True, lengths=lengths, row_offsets=offs, n_rows=sum(counts))
     if ttx is not None:
-        monkeypatch.setenv("BGX_ADAM_TTX", str(ttx))
+        bgx_env("BGX_ADAM_TTX", str(ttx))
     got = _run_adam(device, case, p, torch.bfloat16, **kw)
-    monkeypatch.setenv("BGX_ADAM_TTX", "0")
+    bgx_env("BGX_ADAM_TTX", "0")
     plain = _run_adam(device, case, p, torch.bfloat16, **kw)
     assert torch.equal(got, plain)
     mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
@@ -631,3 +627,28 @@ def test_adam_seq_many_short_sequences(device):
     a, g, left, right, norm = case
     got = _run_adam(device, case, p, torch.bfloat16)
     assert rel_l2(got, ohooks.module_gradient(a, g, norm, left, right)) <= TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("per_token", [False, True])
+@pytest.mark.parametrize("shape", [(1, 4, 768, 768, 16), (1, 2, 64, 256, 32), (2, 3, 128, 512, 8)])
+def test_adam_fused_shapes_with_fewer_tokens_than_a_tile(device, per_token, shape):
+    """A batch of a few tokens on a shape the fused Adam kernel takes: one pass of T tokens (a chunk size
+    rounded down to whole 256-token tiles would be zero here)."""
+    N, S, I, O, p = shape
+    case = _adam_case(N, S, I, O, p, torch.bfloat16, seed=70)
+    a, g, left, right, norm = case
+    lengths = [S] * N
+    g = g.clone()
+    g[:, S - 1:] = 0
+    case = (a, g, left, right, norm)
+    if per_token:
+        mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+        offs = [n * (S - 1) for n in range(N)]
+        want = ohooks.module_gradient(a, g, norm, left, right, attribute_tokens=True, collection_mask=mask)
+        got = _run_adam(device, case, p, torch.bfloat16, per_token=True, lengths=lengths, row_offsets=offs,
+                        n_rows=N * (S - 1))
+    else:
+        want = ohooks.module_gradient(a, g, norm, left, right)
+        got = _run_adam(device, case, p, torch.bfloat16)
+    assert got.shape == want.shape
+    assert rel_l2(got, want) <= TOL[torch.bfloat16]

@@ -340,3 +340,47 @@ def test_query_normalisation_and_aggregation(unit, agg, norm_agg):
         assert not normalize_flat_grad(torch.zeros(4), torch.device("cpu")).any()
     with pytest.raises(ValueError):
         normalize_and_aggregate_grads(grads, names, True, torch.device("cpu"), "median")
+
+
+def test_overlapped_steps_keep_foreign_hooks_on_the_embedding_firing():
+    """Someone else's hook on the input embedding's weight gradient (or on the module): the overlapped loop then
+    runs the backward pass down to the parameters, as `backward()` does, so the hook fires once per batch
+    with the gradient the plain loop gives it."""
+    from bergson_amd import IndexConfig
+    from bergson_amd.collector import CollectorComputer, OverlappedSteps
+
+    class LM(_ToyLM):
+        def forward(self, x):
+            out = super().forward(x)
+            return type("O", (), {"logits": torch.cat([out, out.flip(-1)[..., :3]], -1)})()
+
+        def get_input_embeddings(self):
+            return self.emb
+
+    class Data:
+        docs = [[1, 2, 3, 4], [5, 6, 7], [8, 9, 10, 1, 2]]
+
+        def __len__(self):
+            return len(self.docs)
+
+        def __getitem__(self, idx):
+            return {"input_ids": [self.docs[i] for i in idx]}
+
+    torch.manual_seed(2)
+    m = LM()
+    m.dtype = torch.float32
+    cfg = IndexConfig(run_path="", projection_dim=4, projection_type="normal")
+    assert not OverlappedSteps._has_foreign_hooks(m.emb)
+    seen = {False: [], True: []}
+    for overlap in (False, True):
+        handle = m.emb.weight.register_hook(lambda g, overlap=overlap: seen[overlap].append(g.clone()))
+        assert OverlappedSteps._has_foreign_hooks(m.emb)
+        CollectorComputer(model=m, data=Data(), collector=_logging_stub(m), batches=[[0, 1], [2]], cfg=cfg,
+                          overlap_backward=overlap).run_with_collector_hooks()
+        handle.remove()
+    assert len(seen[False]) == len(seen[True]) == 2
+    for g0, g1 in zip(seen[False], seen[True]):
+        assert torch.equal(g0, g1)
+    handle = m.emb.register_full_backward_hook(lambda mod, gi, go: None)
+    assert OverlappedSteps._has_foreign_hooks(m.emb)
+    handle.remove()
