@@ -200,3 +200,114 @@ def test_store_scan_full_size_properties(device):
     # selection is exact on (score, row) keys and a row's score does not depend on the pass it is in
     assert torch.equal(res2.topk_values, vals[:256])
     assert torch.equal(res2.topk_indices, idx[:256])
+
+
+# ---- configuration 1 at its stated size: Pythia-14m fp32, 64 x 256 tokens, 2048-token batches ------------------
+def test_pythia14m_config1_full_size_against_cpu_loop(device):
+    """The reference's own CPU-runnable case in full: 64 documents of 256 uniform token ids, batches of 8
+    (token_batch_size 2048), p = 16, no normalizer, per sequence, sum reduction -- the product loop on the GPU
+    against the oracle's loop on the CPU (rel-L2 <= 1e-3: the model's own fp32 forward/backward differs
+    between the devices at rounding level)."""
+    import numpy as np
+    from bergson_amd import GradientProcessor, IndexConfig, allocate_batches, collect_gradients
+    from bergson_amd.synthetic import ListDataset, make_gpt_neox, random_docs
+    from oracle import loop as oloop
+
+    lengths = [256] * 64
+    docs = random_docs(lengths, seed=0)
+    batches = allocate_batches(lengths, 2048)
+    assert len(batches) == 8 and all(len(b) == 8 for b in batches)
+    cpu = make_gpt_neox("pythia-14m", torch.float32, "cpu", seed=0)
+    want, want_losses = oloop.collect(cpu, cpu.base_model, docs, batches, p=16)
+    gpu = make_gpt_neox("pythia-14m", torch.float32, device, seed=0)
+    cfg = IndexConfig(run_path="", projection_dim=16, projection_type="normal")
+    col = collect_gradients(gpu, ListDataset(docs), GradientProcessor(projection_dim=16, projection_type="normal"),
+                            cfg, batches=batches)
+    torch.cuda.synchronize()
+    got = torch.from_numpy(np.array(col.builder.grad_buffer))
+    assert got.shape == want.shape == (64, 24 * 256)
+    assert rel_l2(got, want) <= 1e-3
+    for m in range(24):  # every module on its own
+        assert rel_l2(got[:, m * 256:(m + 1) * 256], want[:, m * 256:(m + 1) * 256]) <= 2e-3, m
+    assert torch.allclose(col.per_doc_losses.cpu(), want_losses, rtol=1e-4)
+    assert int(col.total_processed) == 64 * 255
+
+
+# ---- configuration 5 through a model: Llama-3-8B-shaped decoder, bf16, Adafactor, fp16 store -----------------
+def _run_llama(device, layers, lengths, vocab, capture):
+    """Collects from a Llama-shaped model; returns (store rows, {name: (a, g)} for the modules in `capture`
+    -- a predicate on the module name --, moments, names)."""
+    import numpy as np
+    from bergson_amd import AdafactorNormalizer, GradientCollector, GradientProcessor, IndexConfig
+    from bergson_amd.collector import CollectorComputer
+    from bergson_amd.synthetic import ListDataset, adafactor_moments, make_llama, random_docs
+
+    docs = random_docs(lengths, vocab=vocab, seed=21)
+    model = make_llama(torch.bfloat16, device, layers=layers, vocab=vocab, seed=0)
+    moments = adafactor_moments(model.base_model, seed=0)
+    names = list(moments)
+    normalizers = {n: AdafactorNormalizer(row=r.to(device), col=c.to(device)) for n, (r, c) in moments.items()}
+    captured, handles = {}, []
+    for name, mod in model.base_model.named_modules():
+        if isinstance(mod, torch.nn.Linear) and capture(name):
+            handles.append(mod.register_forward_hook(
+                lambda m, inp, out, name=name: captured.setdefault(name, {}).__setitem__("a", inp[0].detach().cpu())))
+            handles.append(mod.register_full_backward_hook(
+                lambda m, gin, gout, name=name: captured[name].__setitem__("g", gout[0].detach().cpu())))
+    cfg = IndexConfig(run_path="", projection_dim=16, projection_type="normal")
+    col = GradientCollector(model=model.base_model, cfg=cfg, data=ListDataset(docs), store_dtype=torch.float16,
+                            processor=GradientProcessor(normalizers=normalizers, projection_dim=16,
+                                                        projection_type="normal"))
+    assert list(col.shapes()) == names
+    CollectorComputer(model=model, data=ListDataset(docs), collector=col, batches=[list(range(len(docs)))], cfg=cfg
+                      ).run_with_collector_hooks()
+    torch.cuda.synchronize()
+    for h in handles:
+        h.remove()
+    assert col.builder.base_dtype == "float16"
+    got = torch.from_numpy(np.array(col.builder.grad_buffer).astype(np.float32))
+    return got, captured, moments, names
+
+
+def _check_llama_blocks(got, captured, moments, names):
+    assert torch.isfinite(got).all()
+    for name, ag in captured.items():
+        a, g = ag["a"], ag["g"]
+        row, col = moments[name]
+        left, right = module_projections(name, 16, g.shape[-1], a.shape[-1], torch.bfloat16)
+        want = ohooks.module_gradient(a, g, ohooks.Adafactor(row=row, col=col), left, right).float().clamp(-65504, 65504)
+        b = names.index(name)
+        block = got[:, b * 256:(b + 1) * 256]
+        assert want.abs().max() > 0
+        assert rel_l2(block, want) <= TOL[torch.bfloat16], name
+
+
+def test_llama8b_two_layers_through_the_model(device):
+    """Two layers at the full Llama-3-8B widths (4096 / 14336, 32 query and 8 key-value heads): target discovery
+    on a Llama model, bias-less modules, q/k/v and gate/up sharing one input tensor, the grouped-query widths
+    (k_proj, v_proj 4096 -> 1024), ragged documents, modules too wide for their projections to stay on chip --
+    every module's block against the oracle on the (a, g) the hooks saw."""
+    lengths = [150, 97]
+    got, captured, moments, names = _run_llama(device, 2, lengths, 32000, lambda name: True)
+    assert len(names) == 14 and got.shape == (2, 14 * 256)
+    assert [n.split(".", 2)[2] for n in names[:7]] == ["self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj",
+                                                       "self_attn.o_proj", "mlp.gate_proj", "mlp.up_proj",
+                                                       "mlp.down_proj"]
+    assert captured["layers.0.self_attn.k_proj"]["g"].shape[-1] == 1024
+    assert captured["layers.1.mlp.down_proj"]["a"].shape[-1] == 14336
+    _check_llama_blocks(got, captured, moments, names)
+
+
+def test_llama8b_full_depth_224_modules(device):
+    """The whole configuration-5 model shape (32 layers, 224 hooked modules, rows of 57 344 values) in one
+    launch per batch; three layers' modules are checked against the oracle on the (a, g) the hooks saw."""
+    free, _ = torch.cuda.mem_get_info()
+    if free < 60 * 2**30:
+        pytest.skip("needs 60 GB of free HBM")
+    lengths = [96, 61]
+    picked = ("layers.0.", "layers.17.", "layers.31.")
+    got, captured, moments, names = _run_llama(device, 32, lengths, 128256, lambda name: name.startswith(picked))
+    assert len(names) == 224 and got.shape == (2, 57344) and len(captured) == 21
+    _check_llama_blocks(got, captured, moments, names)
+    norms = got.view(2, 224, 256).norm(dim=2)
+    assert (norms > 0).all()  # every module wrote its block
