@@ -64,6 +64,9 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
                  const int32_t* lengths, const int64_t* rows_or_offsets, void* out, int64_t out_row_stride,
                  int out_dtype, float lo, float hi, void* ws, size_t ws_bytes, void* stream,
                  bool tables_by_kernel = false);
+int collect_seq_static_impl(const bgx_module_desc* mods_host, int n_modules, int N, int S, int p, int in_dtype,
+                            const int32_t* lengths, const int64_t* out_rows, void* out, int64_t out_row_stride,
+                            int out_dtype, float lo, float hi, void* stream);
 int adafactor_scales_impl(const float* row, int O, const float* col, int I, int dtype, float* row_scale,
                           float* col_scale, void* stream);
 size_t adam_table_bytes(int O, int I, int p, int dtype);
@@ -159,6 +162,13 @@ int bgx_collect_tok(const bgx_module_desc* mods_host, int32_t n_modules, int32_t
                     size_t workspace_bytes, void* stream) {
   return bgx::collect_impl(true, mods_host, n_modules, N, S, p, in_dtype, lengths_dev, row_offsets_dev, out_dev,
                            out_row_stride, out_dtype, clamp_lo, clamp_hi, workspace_dev, workspace_bytes, stream);
+}
+
+int bgx_collect_seq_static(const bgx_module_desc* mods_host, int32_t n_modules, int32_t N, int32_t S, int32_t p,
+                           int32_t in_dtype, const int32_t* lengths_dev, const int64_t* out_rows_dev, void* out_dev,
+                           int64_t out_row_stride, int32_t out_dtype, float clamp_lo, float clamp_hi, void* stream) {
+  return bgx::collect_seq_static_impl(mods_host, n_modules, N, S, p, in_dtype, lengths_dev, out_rows_dev, out_dev,
+                                      out_row_stride, out_dtype, clamp_lo, clamp_hi, stream);
 }
 
 size_t bgx_adam_table_bytes(int32_t O, int32_t I, int32_t p, int32_t dtype) {

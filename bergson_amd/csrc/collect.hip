@@ -1196,6 +1196,49 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   return 0;
 }
 
+// ---- the entry point that allocates nothing ------------------------------------------------------------
+// Its workspace is this array: one copy per GPU, held from the moment the library is loaded on that GPU until
+// the process ends.  `scratch` itself is a host-side stand-in, not a device address: host code only ever uses
+// the address hipGetSymbolAddress returns for the device that is current, looked up once per device.
+static __device__ __align__(256) unsigned char scratch[BGX_STATIC_SCRATCH_BYTES];
+static std::mutex g_scratch_lock;
+static void* g_scratch_ptr[MAX_DEVICES];  // per device, nullptr until the first call on it
+
+static int static_scratch(void** out) {
+  int dev = 0;
+  BGX_HIP(hipGetDevice(&dev));
+  BGX_REQUIRE(dev >= 0 && dev < MAX_DEVICES, BGX_E_ARG, "collect_seq_static: device %d outside 0..%d", dev,
+              MAX_DEVICES - 1);
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    BGX_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    BGX_REQUIRE(ptr != nullptr && ((uintptr_t)ptr & 255) == 0, BGX_E_ALIGN,
+                "collect_seq_static: the scratch array's device address %p is unusable", ptr);
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+int collect_seq_static_impl(const bgx_module_desc* mods_host, int n_modules, int N, int S, int p, int in_dtype,
+                            const int32_t* lengths, const int64_t* out_rows, void* out, int64_t out_row_stride,
+                            int out_dtype, float lo, float hi, void* stream) {
+  BGX_REQUIRE(mods_host != nullptr && n_modules > 0 && N > 0 && S > 0 && p >= 1 && p <= 64, BGX_E_ARG,
+              "collect_seq_static: n_modules=%d N=%d S=%d p=%d", n_modules, N, S, p);
+  const size_t need = collect_workspace_bytes(n_modules, N, S, p);
+  BGX_REQUIRE(need <= (size_t)BGX_STATIC_SCRATCH_BYTES, BGX_E_WORKSPACE,
+              "collect_seq_static: %d modules x %d sequences x %d tokens at p=%d need %zu bytes of scratch, the "
+              "static array holds %zu; use bgx_collect_seq with a workspace of the caller's",
+              n_modules, N, S, p, need, (size_t)BGX_STATIC_SCRATCH_BYTES);
+  void* ptr = nullptr;
+  if (const int rc = static_scratch(&ptr)) return rc;
+  // Every word of the workspace that a launch reads, the same launch has written before (descriptors and item
+  // ranges by the table upload, partials by the collection kernel), so nothing needs clearing between calls.
+  return collect_impl(false, mods_host, n_modules, N, S, p, in_dtype, lengths, out_rows, out, out_row_stride,
+                      out_dtype, lo, hi, ptr, (size_t)BGX_STATIC_SCRATCH_BYTES, stream, /*tables_by_kernel=*/true);
+}
+
 int adafactor_scales_impl(const float* row, int O, const float* col, int I, int dtype, float* row_scale,
                           float* col_scale, void* stream) {
   BGX_REQUIRE(dtype >= BGX_F32 && dtype <= BGX_BF16, BGX_E_DTYPE, "adafactor_scales: dtype=%d", dtype);

@@ -113,7 +113,7 @@ def _rows_view(t: Tensor, name: str) -> Tensor:
 
 
 def _collect(per_token: bool, modules: list[ModuleInput], p: int, out: Tensor, lengths: Tensor | None,
-             rows: Tensor | None, lo: float, hi: float) -> None:
+             rows: Tensor | None, lo: float, hi: float, static_scratch: bool = False) -> None:
     lib = _lib.load()
     if not modules:
         raise ValueError("no modules to collect")
@@ -164,6 +164,11 @@ def _collect(per_token: bool, modules: list[ModuleInput], p: int, out: Tensor, l
         if rows.dtype != torch.int64 or rows.numel() != N or not rows.is_contiguous():
             raise ValueError("row indices / offsets must be a contiguous int64 vector of N elements")
         _need_gpu(rows, "rows")
+    if static_scratch:
+        rc = lib.bgx_collect_seq_static(descs, len(modules), N, S, p, dtype_code(in_dtype), _ptr(lengths), _ptr(rows),
+                                        _ptr(out), out.stride(0), dtype_code(out.dtype), lo, hi, _stream())
+        _lib.check(rc, "bgx_collect_seq_static")
+        return
     nbytes = lib.bgx_collect_workspace_bytes_for(descs, len(modules), N, S, p, dtype_code(in_dtype))
     ws = _workspace(out.device, nbytes, "collect")
     fn = lib.bgx_collect_tok if per_token else lib.bgx_collect_seq
@@ -457,6 +462,14 @@ def collect_seq(modules: list[ModuleInput], p: int, out: Tensor, *, lengths: Ten
                 out_rows: Tensor | None = None, lo: float = float("-inf"), hi: float = float("inf")) -> None:
     """out[row(n), m.out_col : m.out_col + p*p] = clamp(sum_s g'[n,s] (x) a'[n,s]) for every module m."""
     _collect(False, modules, p, out, lengths, out_rows, lo, hi)
+
+
+def collect_seq_static(modules: list[ModuleInput], p: int, out: Tensor, *, lengths: Tensor | None = None,
+                       out_rows: Tensor | None = None, lo: float = float("-inf"), hi: float = float("inf")) -> None:
+    """`collect_seq` through the entry point that allocates nothing: no workspace tensor, the library's own
+    static scratch array instead (16 MiB per GPU; larger launches are refused).  Calls that could overlap on
+    one GPU must not use it at the same time."""
+    _collect(False, modules, p, out, lengths, out_rows, lo, hi, static_scratch=True)
 
 
 def collect_tok(modules: list[ModuleInput], p: int, out: Tensor, *, lengths: Tensor, row_offsets: Tensor,

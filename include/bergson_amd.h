@@ -16,7 +16,8 @@
  *     library allocates no device memory and never synchronises the host: all
  *     work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the
  *     null stream).  Entry points that take a host table (mods_host,
- *     blocks_host) copy it to the workspace with hipMemcpyAsync.
+ *     blocks_host) copy it to the workspace with hipMemcpyAsync;
+ *     bgx_collect_seq_static does not even do that.
  *   - "rows" are store rows; "tokens" are (sequence, position) pairs.
  *   - dtypes are BGX_F32 / BGX_F16 / BGX_BF16.
  */
@@ -30,7 +31,7 @@
 extern "C" {
 #endif
 
-#define BGX_ABI_VERSION 6
+#define BGX_ABI_VERSION 7
 
 enum bgx_dtype { BGX_F32 = 0, BGX_F16 = 1, BGX_BF16 = 2 };
 
@@ -142,6 +143,29 @@ int bgx_collect_seq(const bgx_module_desc* mods_host, int32_t n_modules,
                     void* out_dev, int64_t out_row_stride, int32_t out_dtype,
                     float clamp_lo, float clamp_hi, void* workspace_dev,
                     size_t workspace_bytes, void* stream);
+
+/* bgx_collect_seq for callers that cannot allocate device memory or hand over a
+ * workspace (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc).  No counterpart in the reference.  Same arguments and
+ * results as bgx_collect_seq, minus the workspace: the descriptor table, the
+ * work-item ranges and the per-tile partial sums live in an array of
+ * BGX_STATIC_SCRATCH_BYTES that is part of the library's device image (one copy
+ * per GPU, held until the process ends), and the tables reach it as kernel
+ * arguments rather than through a host-to-device copy.  The call allocates
+ * nothing and frees nothing.  A launch whose bgx_collect_workspace_bytes() is
+ * larger than the array is rejected with BGX_E_WORKSPACE before anything is
+ * enqueued (16 MiB holds 48 modules x 4096 tokens at p = 16 five times over;
+ * modules too wide for on-chip projections run through the per-tile kernel
+ * unless their fragment table fits as well).  All calls on one GPU share the
+ * array: calls that may overlap on a GPU (different streams, different
+ * threads) race; calls on one stream are ordered by the stream. */
+#define BGX_STATIC_SCRATCH_BYTES (16u << 20)
+int bgx_collect_seq_static(const bgx_module_desc* mods_host, int32_t n_modules,
+                           int32_t N, int32_t S, int32_t p, int32_t in_dtype,
+                           const int32_t* lengths_dev,
+                           const int64_t* out_rows_dev, void* out_dev,
+                           int64_t out_row_stride, int32_t out_dtype,
+                           float clamp_lo, float clamp_hi, void* stream);
 
 /* Per-token variant (attribute_tokens): no token reduction; row
  * row_offsets_dev[n] + s of `out` receives flatten(g'[n,s] (x) a'[n,s]) for
