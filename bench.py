@@ -8,17 +8,26 @@ lognormal(6, 1) clipped to [16, 2048], bin-packed into 4096-token batches, unifo
 projection_dim 16 Gaussian projections on all 48 Linear modules; Adafactor normalizer with second
 moments |N(0,1)| * 1e-4; per-sequence gradients written to an fp16 store.
 
-A step is one batch through the whole path: forward, loss, backward (hooks queue the modules), one
-fused collection launch into the device-resident fp16 store.  The store is copied to its memory-mapped
-file once after the last timed step, inside the timed region.  Padded batches are staged in HBM
-before the timed region starts.  value = documents' tokens / wall seconds.
+A step is one batch through the whole path: padding and upload of the token ids, forward, loss, backward
+(hooks queue the modules), one fused collection launch into the device-resident fp16 store.  The timed
+region is `CollectorComputer.run_with_collector_hooks` over the K timed batches as a whole -- the reference's
+own definition (benchmarks/benchmark_bergson.py:355-358: tokens / seconds of the build loop) -- so it also
+holds the store flush to its memory-mapped file, the loss column and the processor files written by
+`teardown()`.  value = documents' tokens / wall seconds.  `prestaged` is the same K batches once more with the
+padded batches already in HBM and only the store flush behind the loop (what earlier records called value).
 
 One JSON line is printed.  It also carries
   roofline      the fused collection kernel: algorithmic bytes (a and g read once) per launch over its
                 duration measured with events on the launch stream, against 8 TB/s;
   cpu_baseline  the CPU oracle (the reference's op sequence on PyTorch CPU) on a bounded sample;
+  gpu_torch_baseline  the same op sequence as cpu_baseline issued as stock PyTorch-ROCm ops on this GPU (module
+                hooks, elementwise scale, skinny GEMMs, bmm, clamp, cat): what the fused launch replaces;
   store_scan    the second half of the metric: 10^6 fp16 rows of 12288 scanned against 1024 queries
-                with unit-norm cosine, top-100 per query and the per-row max.
+                with unit-norm cosine, top-100 per query and the per-row max; its own cpu_baseline is the
+                reference's search on a slice of the store;
+  per_token     configs[1]'s modules with one row per token (attribute_tokens), kernel only;
+  llama8b_layers  configs[4]'s module shapes through a 4-layer Llama-3-8B-shaped model;
+  adam_per_token  configs[3]'s hot kernel.
 """
 from __future__ import annotations
 
@@ -59,12 +68,19 @@ def parse_args():
     ap.add_argument("--docs", type=int, default=2048)
     ap.add_argument("--token-batch-size", type=int, default=4096)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-scan", action="store_true", help="skip the store-scan and per-token Adam legs")
+    ap.add_argument("--no-scan", action="store_true",
+                    help="skip every leg but the headline one (store scan, per-token, Llama shapes, Adam)")
     ap.add_argument("--scan-only", action="store_true",
                     help="run the store-scan leg alone and print its entry (for counter runs on the scan kernels)")
     ap.add_argument("--scan-rows", type=int, default=1_000_000)
     ap.add_argument("--scan-queries", type=int, default=1024)
     ap.add_argument("--cpu-sample-tokens", type=int, default=32768)
+    ap.add_argument("--scan-cpu-rows", type=int, default=20000,
+                    help="rows of the store the CPU baseline of the scan searches (all queries)")
+    ap.add_argument("--torch-baseline-steps", type=int, default=40,
+                    help="batches the stock-PyTorch op sequence is timed on, on this GPU")
+    ap.add_argument("--llama-only", action="store_true", help="run the Llama-shaped leg alone and print its entry")
+    ap.add_argument("--per-token-only", action="store_true", help="run the per-token collection leg alone")
     ap.add_argument("--adam-only", action="store_true",
                     help="run the per-token Adam leg alone and print its entry (for counter runs on that kernel)")
     ap.add_argument("--plain-loop", action="store_true",
@@ -79,7 +95,7 @@ def parse_args():
 def collection_leg(args, torch, device):
     import bergson_amd as B
     from bergson_amd import ops
-    from bergson_amd.collector import OverlappedSteps
+    from bergson_amd.collector import CollectorComputer, OverlappedSteps
     from bergson_amd.synthetic import ListDataset, adafactor_moments, lognormal_lengths, make_gpt_neox, random_docs
 
     lengths = lognormal_lengths(args.docs, seed=0)
@@ -94,79 +110,120 @@ def collection_leg(args, torch, device):
     normalizers = {n: B.AdafactorNormalizer(row=r.to(device), col=c.to(device)) for n, (r, c) in moments.items()}
     processor = B.GradientProcessor(normalizers=normalizers, projection_dim=16, projection_type="normal")
     run_dir = tempfile.mkdtemp(prefix="bgx_bench_")
-    cfg = B.IndexConfig(run_path=os.path.join(run_dir, "store"), projection_dim=16, projection_type="normal",
-                        token_batch_size=args.token_batch_size)
-    collector = B.GradientCollector(model=model.base_model, cfg=cfg, data=data, processor=processor,
-                                    store_dtype=torch.float16)
-    fwd_bwd = B.fwd_bwd_factory(cfg)
+    overlap = not args.plain_loop
 
-    staged = []
-    for indices in batches[:need]:
-        b = data[indices]
-        x, y, _, mask = B.pad_and_tensor(b["input_ids"], device=device, sync_max_len=False)
-        staged.append((indices, b, x, y, mask))
-    torch.cuda.synchronize()
+    def make_collector(tag):
+        cfg = B.IndexConfig(run_path=os.path.join(run_dir, tag), projection_dim=16, projection_type="normal",
+                            token_batch_size=args.token_batch_size)
+        return cfg, B.GradientCollector(model=model.base_model, cfg=cfg, data=data, processor=processor,
+                                        store_dtype=torch.float16)
 
-    # the loop body of CollectorComputer.run_with_collector_hooks: by default each batch's backward pass
-    # runs beside the next batch's forward pass; --plain-loop times one batch at a time
-    overlapped = None if args.plain_loop else OverlappedSteps(model, collector, cfg)
+    # untimed: the first W batches through the same entry point
+    if args.warmup:
+        cfg, collector = make_collector("warmup")
+        CollectorComputer(model=model, data=data, collector=collector, batches=batches[:args.warmup], cfg=cfg,
+                          overlap_backward=overlap).run_with_collector_hooks()
+        del collector
+    timed_batches = batches[args.warmup:need]
+    tokens = sum(lengths[i] for indices in timed_batches for i in indices)
 
-    def step(item):
-        indices, b, x, y, mask = item
-        if overlapped is not None:
-            overlapped.step(indices, b, x, y, mask)
-            return
-        with collector.with_batch(mask):
-            losses = fwd_bwd(model, x, y, b)
-        collector.process_batch(indices, losses=losses)
-
-    for item in staged[:args.warmup]:
-        step(item)
-    if overlapped is not None:
-        overlapped.drain()
+    # timed: run_with_collector_hooks over the K batches, padding / upload / flush / teardown included
+    cfg, collector = make_collector("store")
+    computer = CollectorComputer(model=model, data=data, collector=collector, batches=timed_batches, cfg=cfg,
+                                 overlap_backward=overlap)
     torch.cuda.synchronize()
     ops.collect_timer = []
     ops.collect_timing_start(args.steps + 8)
     t0 = time.perf_counter()
-    for item in staged[args.warmup:need]:
-        step(item)
+    computer.run_with_collector_hooks()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    timer, ops.collect_timer = ops.collect_timer, None
+    kernel_only_ms = ops.collect_timing_stop()
+    store = collector.builder.grad_buffer
+    nonzero = int((abs(store[:, :256].astype("float32")).sum(axis=1) > 0).sum())
+    total_processed = int(computer.total_processed)
+    del collector, computer
+
+    # the same batches once more, padded and uploaded beforehand
+    cfg, collector = make_collector("prestaged")
+    fwd_bwd = B.fwd_bwd_factory(cfg)
+    staged = []
+    for indices in timed_batches:
+        b = data[indices]
+        x, y, _, mask = B.pad_and_tensor(b["input_ids"], device=device, sync_max_len=False)
+        staged.append((indices, b, x, y, mask))
+    padded = sum(int(item[2].numel()) for item in staged)
+    overlapped = OverlappedSteps(model, collector, cfg) if overlap else None
+    torch.cuda.synchronize()
+    p0 = time.perf_counter()
+    for indices, b, x, y, mask in staged:
+        if overlapped is not None:
+            overlapped.step(indices, b, x, y, mask)
+            continue
+        with collector.with_batch(mask):
+            losses = fwd_bwd(model, x, y, b)
+        collector.process_batch(indices, losses=losses)
     if overlapped is not None:
         overlapped.drain()
     collector.builder.flush()
     torch.cuda.synchronize()
-    t1 = time.perf_counter()
+    p1 = time.perf_counter()
     if overlapped is not None:
+        n_streams = overlapped._n_streams
         overlapped.close()
-    timer, ops.collect_timer = ops.collect_timer, None
-    kernel_only_ms = ops.collect_timing_stop()
+    collector.remove_hooks()
 
-    tokens = sum(lengths[i] for item in staged[args.warmup:need] for i in item[0])
-    padded = sum(int(item[2].numel()) for item in staged[args.warmup:need])
     bracket_ms = sum(e0.elapsed_time(e1) for e0, e1, _ in timer)
     kernel_ms = sum(kernel_only_ms)
-    assert len(kernel_only_ms) == len(timer), (len(kernel_only_ms), len(timer))
+    assert len(kernel_only_ms) == len(timer) == len(timed_batches), (len(kernel_only_ms), len(timer))
     kernel_bytes = sum(nb for _, _, nb in timer)
     achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9 if kernel_ms > 0 else 0.0
-    store = collector.builder.grad_buffer
     out = {
         "seconds": t1 - t0,
         "tokens": tokens,
         "padded_tokens": padded,
+        "total_processed": total_processed,
+        "prestaged_seconds": p1 - p0,
         "launches": len(timer),
         "kernel_ms_per_launch": kernel_ms / max(1, len(timer)),
         "bracket_ms_per_launch": bracket_ms / max(1, len(timer)),
         "kernel_bytes_per_launch": kernel_bytes / max(1, len(timer)),
         "achieved_gbs": achieved,
         "n_batches_total": len(batches),
-        "store_rows_nonzero": int((abs(store[:, :256].astype("float32")).sum(axis=1) > 0).sum()),
+        "store_rows_nonzero": nonzero,
         "total_tokens_all_docs": int(sum(lengths)),
-        "loop": "plain (one batch at a time)" if overlapped is None else
+        "loop": "plain (one batch at a time)" if not overlap else
                 f"overlapped (backward pass of batch i beside the forward pass of batch i+1, batches alternating "
-                f"between {overlapped._n_streams} streams, the collection launch alone on the GPU)",
+                f"between {n_streams} streams, the collection launch alone on the GPU)",
     }
-    del collector, model
-    torch.cuda.empty_cache()
-    return out, docs, lengths
+    extra = {"model": model, "moments": moments, "batches": batches, "data": data}
+    del collector
+    return out, docs, lengths, extra
+
+
+def gpu_torch_baseline_leg(args, torch, device, docs, lengths, extra):
+    """The reference's hook sequence issued as stock PyTorch ops on this GPU, on the first batches after the
+    warm-up ones of the same workload: what the fused launch replaces (module forward and full-backward hooks,
+    a * rsqrt(col), a @ R^T, g * factor, g @ L^T, g^T a, clamp, cat, scatter into the store)."""
+    from oracle import hooks as ohooks
+    from oracle import loop as oloop
+
+    model, batches = extra["model"], extra["batches"]
+    norms = {n: ohooks.Adafactor(row=r.to(device), col=c.to(device)) for n, (r, c) in extra["moments"].items()}
+    warm = batches[:3]
+    timed = batches[args.warmup:args.warmup + args.torch_baseline_steps]
+    oloop.collect(model, model.base_model, docs, warm, p=16, normalizers=norms, save_dtype=torch.float16, device=device)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    oloop.collect(model, model.base_model, docs, timed, p=16, normalizers=norms, save_dtype=torch.float16,
+                  device=device)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    tok = sum(lengths[i] for b in timed for i in b)
+    return {"value": tok / dt, "unit": "tokens/s", "ms_per_step": dt / len(timed) * 1e3, "steps": len(timed),
+            "what": "reference op sequence (PyTorch-ROCm ops from module hooks, one batch at a time, rows kept on the "
+                    "device) on the same model, batches and GPU"}
 
 
 def scan_leg(args, torch, device):
@@ -224,7 +281,121 @@ def scan_leg(args, torch, device):
         out[f"q{nq}"] = {"ms": ms_few, "rows_per_s": n / (ms_few * 1e-3),
                          "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                       "frac": gbs / HBM_PEAK_GBS, "traffic": n * D * 2 * SCAN_TRAFFIC_RATIO_FEW}}
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = scan_cpu_baseline(args, torch, store, qd, k)
     del store
+    torch.cuda.empty_cache()
+    return out
+
+
+def scan_cpu_baseline(args, torch, store, qd, k):
+    """The reference's search (bergson/query/attributor.py:169-235: index and queries to fp32, unit norms,
+    Q x N score matrix, torch.topk) on the host cores, on the first rows of the same store."""
+    from oracle import scan as oscan
+
+    n = min(args.scan_cpu_rows, store.shape[0])
+    rows = store[:n].cpu()
+    q = qd.cpu()
+    t0 = time.perf_counter()
+    vals, idx = oscan.attributor_search({"g": rows}, {"g": q}, ["g"], k, unit_norm=True)
+    dt = time.perf_counter() - t0
+    return {"value": n / dt, "unit": "rows/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"the first {n} of {store.shape[0]} rows against all {q.shape[0]} queries, top-{k}, in {dt:.2f} s; the "
+                      f"scan is linear in the rows, so the whole store would take {store.shape[0] / n:.0f} x as long"}
+
+
+def per_token_leg(args, torch, device):
+    """configs[1]'s 48 modules with one row per token (attribute_tokens) at p = 16: the persistent collection kernel
+    writing every valid token's p x p blocks, 2 x 2048 tokens per launch, bf16 rows.  Kernel only, synthetic a / g."""
+    from bergson_amd import ops
+
+    N, S, p, d = 2, 2048, 16, 768
+    gen = torch.Generator(device=device).manual_seed(3)
+    rnd = lambda *shape: torch.randn(*shape, generator=gen, device=device)
+    mods, col = [], 0
+    for layer in range(12):
+        for I, O in ((d, 3 * d), (d, d), (d, 4 * d), (4 * d, d)):
+            rs, cs = ops.adafactor_scales(rnd(O).abs() * 1e-4 + 1e-12, rnd(I).abs() * 1e-4 + 1e-12, torch.bfloat16)
+            mods.append(ops.ModuleInput(a=rnd(N, S, I).to(torch.bfloat16), g=(rnd(N, S, O) * 0.01).to(torch.bfloat16),
+                                        r_in=(rnd(p, I) / 4).to(torch.bfloat16), r_out=(rnd(p, O) / 4).to(torch.bfloat16),
+                                        out_col=col, col_scale=cs, row_scale=rs))
+            col += p * p
+    lengths = torch.full((N,), S, dtype=torch.int32, device=device)
+    offsets = torch.arange(N, device=device, dtype=torch.int64) * (S - 1)
+    out = torch.zeros(N * (S - 1), col, device=device, dtype=torch.bfloat16)
+    reps = 10
+    ops.collect_tok(mods, p, out, lengths=lengths, row_offsets=offsets, lo=-3e38, hi=3e38)
+    torch.cuda.synchronize()
+    ops.collect_timing_start(reps)
+    for _ in range(reps):
+        ops.collect_tok(mods, p, out, lengths=lengths, row_offsets=offsets, lo=-3e38, hi=3e38)
+    torch.cuda.synchronize()
+    ms = ops.collect_timing_stop()
+    ms = sum(ms) / len(ms)
+    read = N * S * sum(m.a.shape[2] + m.g.shape[2] for m in mods) * 2
+    written = out.numel() * 2
+    gbs = (read + written) / (ms * 1e-3) / 1e9
+    return {"workload": "configs[1] modules, per-token rows: 48 Pythia-160m modules, 2 x 2048 tokens, p=16, Adafactor, "
+                        "bf16 rows of 12288",
+            "ms_per_launch": ms, "tokens_per_s_hooks_only": N * S / (ms * 1e-3),
+            "roofline": {"bound": "hbm", "kernel": "bgx::collect_persist_kernel<bf16_t, true, 2, 4, true, false>",
+                         "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                         "bytes_read": read, "bytes_written": written, "traffic": None}}
+
+
+def llama_leg(args, torch, device):
+    """configs[4]'s module shapes through a model: four layers of a Llama-3-8B-shaped decoder (28 hooked modules
+    of 4096 x {4096, 1024, 14336}), batches of 2 x 2048 tokens, p = 16, Adafactor, fp16 store.  The roofline entry
+    is the collection kernel of those launches (the streamed kernel with its projection fragments in a global
+    table, since 4096 x 14336 does not fit on chip), timed by event pairs on its stream."""
+    import bergson_amd as B
+    from bergson_amd import ops
+    from bergson_amd.collector import CollectorComputer
+    from bergson_amd.synthetic import ListDataset, adafactor_moments, make_llama, random_docs
+
+    layers, n_batches, warm = 4, 6, 2
+    lengths = [2048] * (2 * (n_batches + warm))
+    docs = random_docs(lengths, vocab=128256, seed=5)
+    data = ListDataset(docs)
+    batches = [[2 * i, 2 * i + 1] for i in range(n_batches + warm)]
+    model = make_llama(torch.bfloat16, device, layers=layers, seed=0)
+    moments = adafactor_moments(model.base_model, seed=0)
+    normalizers = {n: B.AdafactorNormalizer(row=r.to(device), col=c.to(device)) for n, (r, c) in moments.items()}
+    processor = B.GradientProcessor(normalizers=normalizers, projection_dim=16, projection_type="normal")
+    cfg = B.IndexConfig(run_path="", projection_dim=16, projection_type="normal", token_batch_size=4096)
+
+    def run(which):
+        col = B.GradientCollector(model=model.base_model, cfg=cfg, data=data, processor=processor,
+                                  store_dtype=torch.float16)
+        CollectorComputer(model=model, data=data, collector=col, batches=which, cfg=cfg).run_with_collector_hooks()
+        torch.cuda.synchronize()
+        return col
+
+    run(batches[:warm])
+    ops.collect_timer = []
+    ops.collect_timing_start(n_batches + 2)
+    t0 = time.perf_counter()
+    col = run(batches[warm:])
+    dt = time.perf_counter() - t0
+    timer, ops.collect_timer = ops.collect_timer, None
+    ms = ops.collect_timing_stop()
+    assert len(ms) == n_batches, len(ms)
+    nbytes = sum(nb for _, _, nb in timer) / len(timer)
+    ms_launch = sum(ms) / len(ms)
+    gbs = nbytes / (ms_launch * 1e-3) / 1e9
+    rows = col.builder.grad_buffer
+    assert rows.shape[1] == 7 * layers * 256
+    out = {"workload": f"configs[4] shapes: {layers} layers of a Llama-3-8B-shaped decoder (28 modules), 2 x 2048-token "
+                       "batches, p=16, Adafactor, fp16 store",
+           "tokens_per_s_this_4_layer_model": 4096 * n_batches / dt, "ms_per_step": dt / n_batches * 1e3,
+           "roofline": {"bound": "hbm", "kernel": "bgx::collect_persist_kernel<bf16_t, false, 2, 4, true, true> "
+                                                  "(streamed loads, projection fragments from a global table)",
+                        "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                        "bytes_per_launch": nbytes, "ms_per_launch": ms_launch, "launches": len(ms),
+                        "ms_per_launch_with_table_build_and_finalize":
+                            sum(e0.elapsed_time(e1) for e0, e1, _ in timer) / len(timer),
+                        "traffic": None}}
+    del col, model
     torch.cuda.empty_cache()
     return out
 
@@ -325,8 +496,19 @@ def main():
     if args.adam_only:
         print(json.dumps({"adam_per_token": adam_leg(args, torch, device)}))
         return
-    coll, docs, lengths = collection_leg(args, torch, device)
+    if args.llama_only:
+        print(json.dumps({"llama8b_layers": llama_leg(args, torch, device)}))
+        return
+    if args.per_token_only:
+        print(json.dumps({"per_token": per_token_leg(args, torch, device)}))
+        return
+    coll, docs, lengths, extra = collection_leg(args, torch, device)
+    gpu_torch = None if args.no_scan else gpu_torch_baseline_leg(args, torch, device, docs, lengths, extra)
+    del extra
+    torch.cuda.empty_cache()
     scan = None if args.no_scan else scan_leg(args, torch, device)
+    per_token = None if args.no_scan else per_token_leg(args, torch, device)
+    llama = None if args.no_scan else llama_leg(args, torch, device)
     adam = None if args.no_scan else adam_leg(args, torch, device)
     cpu = None if args.no_cpu_baseline else cpu_baseline_leg(args, torch, docs, lengths)
 
@@ -352,9 +534,16 @@ def main():
             "token_batch_size": args.token_batch_size,
             "tokens_timed": coll["tokens"],
             "padded_tokens_timed": coll["padded_tokens"],
+            "total_processed": coll["total_processed"],
             "batches_total": coll["n_batches_total"],
             "loop": coll["loop"],
+            "timed_region": "CollectorComputer.run_with_collector_hooks over the timed batches: padding, upload of the "
+                            "token ids, forward, backward, fused launch, store flush, teardown artefacts",
         },
+        "prestaged": {"value": coll["tokens"] / coll["prestaged_seconds"], "unit": "tokens/s",
+                      "ms_per_step": coll["prestaged_seconds"] / args.steps * 1e3,
+                      "what": "the same batches once more, padded and uploaded before the clock starts; loop body and "
+                              "store flush only"},
         "roofline": {
             "bound": "hbm",
             "kernel": "bgx::collect_persist_kernel<bf16_t, false, 2, 4, true, false> and <bf16_t, false, 1, 8, true, false> (128- and 64-token tiles, streamed loads, projections in LDS)",
@@ -370,7 +559,10 @@ def main():
             "launches": coll["launches"],
         },
         "cpu_baseline": cpu,
+        "gpu_torch_baseline": gpu_torch,
         "store_scan": scan,
+        "per_token": per_token,
+        "llama8b_layers": llama,
         "adam_per_token": adam,
     }
     print(json.dumps(line))

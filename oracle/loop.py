@@ -68,7 +68,7 @@ def losses_and_backward(model, x: Tensor, y: Tensor, loss_reduction: str = "sum"
                              label_smoothing=label_smoothing).reshape_as(y[:, 1:])
     losses = losses.sum(1) / denoms
     if advantage is not None:
-        losses = losses * torch.tensor(advantage, dtype=losses.dtype)
+        losses = losses * torch.tensor(advantage, dtype=losses.dtype, device=losses.device)
     losses.sum().backward()
     model.zero_grad()
     return losses
@@ -83,10 +83,13 @@ def collect(model, base_model: nn.Module, docs: list[list[int]], batches: list[l
             normalizers: dict | None = None, projection_type: str = "normal", attribute_tokens: bool = False,
             include_bias: bool = False, save_dtype: torch.dtype | None = None, loss_reduction: str = "sum",
             unit_normalize: bool = False, global_dim: int | None = None, label_smoothing: float = 0.0,
-            labels: list[list[int]] | None = None, advantages: list[float] | None = None
-            ) -> tuple[Tensor, Tensor]:
+            labels: list[list[int]] | None = None, advantages: list[float] | None = None,
+            device: str | torch.device = "cpu") -> tuple[Tensor, Tensor]:
     """The whole reference loop on CPU: returns (rows, losses).
 
+    `device`: where the model lives and the hooks' tensor arithmetic runs.  "cpu" is the checker and the
+    timed CPU baseline; with the model on a GPU the very same op sequence runs as stock PyTorch device ops --
+    what the benchmark times beside the fused kernels as the sequence they replace.
     `labels` (per document, -100 = not supervised) and `advantages` (one factor per document) are the
     dataset's optional "labels" and "advantage" columns (collector.py:877-886, :975-976).
 
@@ -112,8 +115,8 @@ def collect(model, base_model: nn.Module, docs: list[list[int]], batches: list[l
             return None, None
         if name not in proj:
             bias = include_bias and mod.bias is not None
-            proj[name] = module_projections(name, p, mod.out_features, mod.in_features, dtype, projection_type,
-                                            "jl", bias)
+            proj[name] = tuple(t.to(device) for t in module_projections(
+                name, p, mod.out_features, mod.in_features, dtype, projection_type, "jl", bias))
         return proj[name]
 
     def fwd(name):
@@ -132,7 +135,8 @@ def collect(model, base_model: nn.Module, docs: list[list[int]], batches: list[l
             P = hooks.backward_hook(stash.pop(name), g, normalizers.get(name), left, right, collect_bias=bias,
                                     attribute_tokens=attribute_tokens, collection_mask=state["mask"], lo=lo, hi=hi)
             if global_dim is not None:
-                R = projection_matrix(f"{name}/single", global_dim, P.shape[1], P.dtype, projection_type, "jl")
+                R = projection_matrix(f"{name}/single", global_dim, P.shape[1], P.dtype, projection_type, "jl"
+                                      ).to(device)
                 mod_grads["gradients"] = hooks.accumulate_global_projection(mod_grads.get("gradients"), P, R)
             else:
                 mod_grads[name] = P.to(save_dtype)
@@ -151,6 +155,7 @@ def collect(model, base_model: nn.Module, docs: list[list[int]], batches: list[l
         for indices in batches:
             x, y, mask = pad_and_tensor([docs[i] for i in indices],
                                         None if labels is None else [labels[i] for i in indices])
+            x, y, mask = x.to(device), y.to(device), mask.to(device)
             state["mask"] = mask
             losses = losses_and_backward(model, x, y, loss_reduction, label_smoothing,
                                          None if advantages is None else [advantages[i] for i in indices])
@@ -163,7 +168,7 @@ def collect(model, base_model: nn.Module, docs: list[list[int]], batches: list[l
             mod_grads.clear()
             if rows is None:
                 n_rows = int(offsets[-1]) if attribute_tokens else len(docs)
-                rows = torch.zeros(n_rows, g.shape[1], dtype=save_dtype)
+                rows = torch.zeros(n_rows, g.shape[1], dtype=save_dtype, device=device)
             if attribute_tokens:
                 r = 0
                 for idx in indices:
@@ -172,7 +177,7 @@ def collect(model, base_model: nn.Module, docs: list[list[int]], batches: list[l
                     r += n
             else:
                 rows[indices] = g
-            losses_out[indices] = losses.detach().float()
+            losses_out[indices] = losses.detach().float().cpu()
     finally:
         for h in handles:
             h.remove()
