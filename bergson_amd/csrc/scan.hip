@@ -29,6 +29,9 @@
 // bergson/query/attributor.py:137-167, :229-235 (row normalisation, GEMM,
 // torch.topk).
 
+#include <type_traits>
+#include <utility>
+
 #include "common.hpp"
 #include "mma32.hpp"
 #include "stream.hpp"
@@ -88,61 +91,79 @@ struct ScanArgs {
 
 // Epilogue of a workgroup tile whose waves hold (TM x TN) blocks of 32 x 32 scores in MFMA layout: scale by the
 // row multipliers s_inv, then dense scores, row maxima, row-sum partials and the threshold filter.
+// One row block (acc_row = the wave's TN blocks of 32 rows x 32 queries; `blk` = which 32 rows of the wave's):
+template <int TN, int WTM, int WTN, int WN>
+__device__ __forceinline__ void scan_block_epilogue(const ScanArgs& args, f32x16 (&acc_row)[TN], const float (&thr)[TN],
+                                                    const float* s_inv, int blk, int wm, int wn, int fr, int fh,
+                                                    int64_t g_row0, int64_t q_row0, int qt) {
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const int row = wm * WTM + blk * 32 + (e >> 2) * 8 + fh * 4 + (e & 3);
+    const int64_t prow = g_row0 + row;  // pass-local row
+    const bool row_ok = prow < args.rows;
+    const int64_t grow = args.row0 + prow;
+    const float w = s_inv[row];
+    float rmax = -INFINITY;
+    float rsum = 0.f;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int64_t q = q_row0 + wn * WTN + j * 32 + fr;
+      const float v = acc_row[j][e] * w;
+      if (row_ok && q < args.Q) {
+        rmax = fmaxf(rmax, v);
+        rsum += v;
+        if (args.scores != nullptr) args.scores[grow * args.Q + q] = v;
+        if (v > thr[j]) {
+          const uint32_t pos = atomicAdd(&args.cand_count[q], 1u);
+          if ((int64_t)pos < args.cand_cap) args.cand[q * args.cand_cap + pos] = make_key(v, (uint32_t)grow);
+        }
+      }
+    }
+    if (args.row_max_enc != nullptr) {
+      rmax = fmaxf(rmax, __shfl_xor(rmax, 1));
+      rmax = fmaxf(rmax, __shfl_xor(rmax, 2));
+      rmax = fmaxf(rmax, __shfl_xor(rmax, 4));
+      rmax = fmaxf(rmax, __shfl_xor(rmax, 8));
+      rmax = fmaxf(rmax, __shfl_xor(rmax, 16));
+      if (fr == 0 && row_ok) atomicMax(&args.row_max_enc[grow], f32_ordered(rmax));
+    }
+    if (args.row_sum_part != nullptr) {
+      // fixed-order butterfly over the 32 lanes that hold this row's scores; one writer per (row, part)
+      rsum += __shfl_xor(rsum, 1);
+      rsum += __shfl_xor(rsum, 2);
+      rsum += __shfl_xor(rsum, 4);
+      rsum += __shfl_xor(rsum, 8);
+      rsum += __shfl_xor(rsum, 16);
+      if (fr == 0 && row_ok) args.row_sum_part[prow * args.n_parts + qt * WN + wn] = rsum;
+    }
+  }
+}
+
+// The row blocks are taken by a pack expansion, not a loop: their indices are then constants whatever the
+// unroller decides, and the accumulators never need an address.  acc[i] is the wave's 32-row block
+// (i + block_rot) mod TM.
+template <int TM, int TN, int WTM, int WTN, int WN, int... Is>
+__device__ __forceinline__ void scan_tile_epilogue_blocks(const ScanArgs& args, f32x16 (&acc)[TM][TN],
+                                                          const float (&thr)[TN], const float* s_inv, int wm, int wn,
+                                                          int fr, int fh, int64_t g_row0, int64_t q_row0, int qt,
+                                                          int block_rot, std::integer_sequence<int, Is...>) {
+  (scan_block_epilogue<TN, WTM, WTN, WN>(args, acc[Is], thr, s_inv, (Is + block_rot) % TM, wm, wn, fr, fh, g_row0,
+                                         q_row0, qt),
+   ...);
+}
+
 template <int TM, int TN, int WTM, int WTN, int WN>
-__device__ inline void scan_tile_epilogue(const ScanArgs& args, f32x16 (&acc)[TM][TN], const float* s_inv, int wm,
-                                          int wn, int fr, int fh, int64_t g_row0, int64_t q_row0, int qt,
-                                          int block_rot = 0) {
+__device__ __forceinline__ void scan_tile_epilogue(const ScanArgs& args, f32x16 (&acc)[TM][TN], const float* s_inv,
+                                                   int wm, int wn, int fr, int fh, int64_t g_row0, int64_t q_row0,
+                                                   int qt, int block_rot = 0) {
   float thr[TN];
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int64_t q = q_row0 + wn * WTN + j * 32 + fr;
     thr[j] = (args.thr != nullptr && q < args.Q) ? args.thr[q] : INFINITY;
   }
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      // acc[i] is the wave's 32-row block (i + block_rot) mod TM
-      const int row = wm * WTM + ((i + block_rot) & (TM - 1)) * 32 + (e >> 2) * 8 + fh * 4 + (e & 3);
-      const int64_t prow = g_row0 + row;  // pass-local row
-      const bool row_ok = prow < args.rows;
-      const int64_t grow = args.row0 + prow;
-      const float w = s_inv[row];
-      float rmax = -INFINITY;
-      float rsum = 0.f;
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int64_t q = q_row0 + wn * WTN + j * 32 + fr;
-        const float v = acc[i][j][e] * w;
-        if (row_ok && q < args.Q) {
-          rmax = fmaxf(rmax, v);
-          rsum += v;
-          if (args.scores != nullptr) args.scores[grow * args.Q + q] = v;
-          if (v > thr[j]) {
-            const uint32_t pos = atomicAdd(&args.cand_count[q], 1u);
-            if ((int64_t)pos < args.cand_cap) args.cand[q * args.cand_cap + pos] = make_key(v, (uint32_t)grow);
-          }
-        }
-      }
-      if (args.row_max_enc != nullptr) {
-        rmax = fmaxf(rmax, __shfl_xor(rmax, 1));
-        rmax = fmaxf(rmax, __shfl_xor(rmax, 2));
-        rmax = fmaxf(rmax, __shfl_xor(rmax, 4));
-        rmax = fmaxf(rmax, __shfl_xor(rmax, 8));
-        rmax = fmaxf(rmax, __shfl_xor(rmax, 16));
-        if (fr == 0 && row_ok) atomicMax(&args.row_max_enc[grow], f32_ordered(rmax));
-      }
-      if (args.row_sum_part != nullptr) {
-        // fixed-order butterfly over the 32 lanes that hold this row's scores; one writer per (row, part)
-        rsum += __shfl_xor(rsum, 1);
-        rsum += __shfl_xor(rsum, 2);
-        rsum += __shfl_xor(rsum, 4);
-        rsum += __shfl_xor(rsum, 8);
-        rsum += __shfl_xor(rsum, 16);
-        if (fr == 0 && row_ok) args.row_sum_part[prow * args.n_parts + qt * WN + wn] = rsum;
-      }
-    }
-  }
+  scan_tile_epilogue_blocks<TM, TN, WTM, WTN, WN>(args, acc, thr, s_inv, wm, wn, fr, fh, g_row0, q_row0, qt, block_rot,
+                                                  std::make_integer_sequence<int, TM>{});
 }
 
 // Workgroup tile BM x BN, WM x WN waves, each wave (BM/WM) x (BN/WN) as 32x32 MFMA blocks.
@@ -531,6 +552,318 @@ __global__ __launch_bounds__(SD_THREADS) void scan_direct_kernel(ScanArgs args) 
   __syncthreads();
 
   scan_tile_epilogue<TM, TN, WTM, WTN, WN>(args, acc, s_inv, wm, wn, fr, fh, g_row0, q_row0, qt, wn);
+}
+
+// ---- many queries, many rows: 384 x 256 tiles on four waves ---------------------------------------------------
+// What bounds the 256 x 256 kernel above is the path from L2 into a compute unit: a CU keeps about 50-60 cache
+// lines in flight whatever is asked of it, i.e. ~16 B per cycle at the ~430 cycles an L2 request takes, and a
+// 256 x 256 tile needs 1/128 byte per flop.  The only lever left is fewer bytes per flop, and that is bounded by
+// the accumulators the register file can hold: this kernel gives one wave per SIMD all 512 registers (the
+// accumulators overflow into the AccVGPRs) -- four waves as 2 x 2, each 192 rows x 128 queries = 6 x 4 blocks of
+// 32 x 32 = 384 accumulator registers -- for a 384 x 256 tile: 1/153.6 byte per flop, 17 % less.  The tile's two
+// K tiles (2 x 80 KB) fill the LDS; with one wave per SIMD nothing else hides a stall, so every global load and
+// every fragment read is placed by hand between two MFMAs of the step before the one that needs it
+// (sched_barrier after each: the order below is the order that is executed).
+//   LDS layout, swizzle, direct-to-LDS loads, explicit waits, row norms from the fragments: as in
+//   scan_direct_kernel, and the scores are the same bits (each is the same sequence of MFMAs over K).
+//   The launch covers whole tiles only: rows a multiple of 384 (the host cuts its passes accordingly; what is left
+//   goes to the kernel above).
+constexpr int SW_BM = 384, SW_BN = 256, SW_THREADS = 256;
+constexpr int SW_A_BYTES = SW_BM * SD_ROW, SW_B_BYTES = SW_BN * SD_ROW, SW_STAGE = SW_A_BYTES + SW_B_BYTES;
+constexpr int SW_LDS_BYTES = 2 * SW_STAGE;
+constexpr int64_t SW_ROUND_ROWS = 64 * SW_BM;  // rows of one round of the chip: 64 row tiles x 4 query tiles = 256 tiles
+
+template <int OFF>
+__device__ inline uint4 sw_lds_read16(uint32_t addr) {
+  uint4 v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+  return v;
+}
+
+// One 32 x 32 x 16 MFMA with the accumulator block pinned to the AccVGPRs (IN_ACC) or to the ordinary VGPRs.
+// Written as instructions: 384 accumulator registers beside 60 of fragments leave the register allocator no
+// slack, and left to itself it shuffles blocks between the two files and spills.  (Volatile: the statements
+// execute in the order they are written, which is the hand-made schedule.)
+template <typename T, bool IN_ACC>
+__device__ inline void sw_mfma(const uint4& a, const uint4& b, f32x16& c) {
+  typedef uint32_t raw4 __attribute__((ext_vector_type(4)));
+  const raw4 av = {a.x, a.y, a.z, a.w}, bv = {b.x, b.y, b.z, b.w};
+  if constexpr (std::is_same<T, f16_t>::value) {
+    if constexpr (IN_ACC)
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(av), "v"(bv));
+    else
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "v"(bv));
+  } else {
+    if constexpr (IN_ACC)
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(av), "v"(bv));
+    else
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "v"(bv));
+  }
+}
+
+template <int N>
+__device__ inline void sw_wait_lds() {  // s_waitcnt lgkmcnt(N), nothing else
+  __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8));
+}
+
+// 16 bytes per lane from global memory (uniform 64-bit base + one 32-bit offset per lane) straight to LDS at
+// byte address `lds` + 16 * lane.  Spelled out so that a load is four instructions (M0, the wait state it needs,
+// the load, and at most one add for the offset) -- the builtin went through 64-bit vector address arithmetic.
+__device__ inline void sw_load_lds16(uint64_t base, uint32_t voff, uint32_t lds) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(voff), "s"(base), "s"(lds)
+               : "memory", "m0");
+}
+
+template <typename T>
+__global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
+  using M = Mma32<T>;
+  constexpr int BK = 64;
+  constexpr int TM = 6, TN = 4, WTM = 192, WTN = 128, WN = 2;
+  constexpr int NA = SW_BM / 32, NB = SW_BN / 32;  // load instructions per wave and K tile: 12 + 8
+  constexpr int ACC_TM = 4;                        // row blocks 0 .. 3 accumulate in AccVGPRs (256), 4 and 5 in VGPRs
+  extern __shared__ __align__(128) unsigned char smem[];
+  float* s_inv = reinterpret_cast<float*>(smem);  // after the main loop: [SW_BM] row multipliers
+
+  const int b = blockIdx.x;
+  const int xcd = b & 7;
+  const int slot = b >> 3;
+  const int rt_local = slot / args.q_tiles;
+  const int qt = slot - rt_local * args.q_tiles;
+  const int rt = rt_local * 8 + xcd;
+  if (rt >= args.row_tiles) return;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int64_t g_row0 = (int64_t)rt * SW_BM;  // pass-local first row
+  const int64_t q_row0 = (int64_t)qt * SW_BN;
+  const int KT = (int)(args.D / BK);
+  const int fr = lane & 31;
+  const int fh = lane >> 5;
+
+  // ---- loader: instruction i of wave w fills rows i * 32 + w * 8 .. + 7 of a tile (1 KB of LDS); lane l is
+  // position l & 7 of row l >> 3 and fetches the chunk that belongs there: chunk c of row r sits at position
+  // c ^ (r & 7) ^ ((r >> 3) & 1), and (r >> 3) & 1 = w & 1 for every i.  Addresses are a uniform base (the tile,
+  // advanced by one K tile per iteration) plus one 32-bit offset per lane and instruction.
+  const int lrow = wave * 8 + (lane >> 3);
+  const int lch = (lane & 7) ^ (lane >> 3) ^ (wave & 1);
+  const uint32_t row_bytes = (uint32_t)(args.store_stride * sizeof(T));
+  const uint32_t q_bytes = (uint32_t)(args.D * sizeof(T));
+  const uint64_t a_base = (uint64_t)(uintptr_t)args.store + (uint64_t)((args.row0 + g_row0) * args.store_stride) * sizeof(T);
+  const uint64_t b_base = (uint64_t)(uintptr_t)args.queries + (uint64_t)(q_row0 * args.D) * sizeof(T);
+  const uint32_t a_voff = (uint32_t)lrow * row_bytes + (uint32_t)lch * 16u;
+  const int q_last = args.Q - 1 - (int)q_row0;  // last valid query row of this tile (rows past it repeat it)
+  uint32_t b_voff[NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) b_voff[i] = (uint32_t)min(i * 32 + lrow, q_last) * q_bytes + (uint32_t)lch * 16u;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+  const uint32_t lds_wave = lds0 + (uint32_t)wave * 1024u;
+  // instruction idx (0 .. NA-1: rows of the store; NA .. NA+NB-1: queries) of K tile kt, into stage `stg`
+  auto load_one_to = [&](int kt, int stg, int idx) {
+    const uint32_t stage = lds_wave + (uint32_t)stg * SW_STAGE;
+    const uint64_t koff = (uint64_t)kt * (BK * sizeof(T));
+    if (idx < NA)
+      sw_load_lds16(a_base + koff, a_voff + (uint32_t)idx * 32u * row_bytes, stage + (uint32_t)idx * 4096u);
+    else
+      sw_load_lds16(b_base + koff, b_voff[idx - NA], stage + (uint32_t)(SW_A_BYTES + (idx - NA) * 4096));
+  };
+  auto load_one = [&](int kt, int idx) { load_one_to(kt, kt & 1, idx); };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  // Row norms: the two waves that share 192 rows take three 32-row blocks each.  Wave wn numbers its blocks from
+  // 3 wn (its block i is rows (i + 3 wn) mod 6), so that "the first three" is the same code in both; one partial
+  // per 16-byte chunk position of the K tile, as in the other tile kernels: identical bits.
+  float ss[3][4];
+#pragma unroll
+  for (int i = 0; i < 3; ++i)
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) ss[i][kk] = 0.f;
+
+  // fragment addresses: row (wm * 192 + blk * 32 + fr), position ((2 kk + fh) ^ key) with key = sd_key(fr) for
+  // every block; (2 kk + fh) ^ key = (2 kk) ^ (fh ^ key), so a k-step is an XOR on the (128-byte aligned) address.
+  // The wave's blocks 0 .. 2 start at row block 3 wn, its blocks 3 .. 5 at row block 3 (1 - wn).
+  const uint32_t c0 = (uint32_t)((fh ^ sd_key(fr)) * 16);
+  const uint32_t a_frag_lo = lds0 + (uint32_t)((wm * WTM + 96 * wn + fr) * SD_ROW) + c0;
+  const uint32_t a_frag_hi = lds0 + (uint32_t)((wm * WTM + 96 * (1 - wn) + fr) * SD_ROW) + c0;
+  const uint32_t b_frag = lds0 + (uint32_t)(SW_A_BYTES + (wn * WTN + fr) * SD_ROW) + c0;
+  // Row fragments have one register set: block i's four MFMAs come one after the other, and the read of the next
+  // step's block i goes out right behind them.  Query fragments are used by all six blocks and have two sets.
+  uint4 af[TM], bf[2][TN];
+  uint32_t ra_lo, ra_hi, rb;  // read addresses of the step that is being read
+  auto rd_base = [&](int stage, auto kk_tag) {
+    constexpr int KK = decltype(kk_tag)::value;
+    const uint32_t st = (uint32_t)stage * SW_STAGE;
+    ra_lo = (a_frag_lo + st) ^ (uint32_t)(KK * 32);
+    ra_hi = (a_frag_hi + st) ^ (uint32_t)(KK * 32);
+    rb = (b_frag + st) ^ (uint32_t)(KK * 32);
+  };
+  auto rd_a = [&](auto i_tag) {
+    constexpr int I = decltype(i_tag)::value;
+    af[I] = sw_lds_read16<(I % 3) * 32 * SD_ROW>(I < 3 ? ra_lo : ra_hi);
+  };
+  auto rd_b = [&](auto set_tag, auto j_tag) {
+    constexpr int SET = decltype(set_tag)::value;
+    constexpr int J = decltype(j_tag)::value;
+    bf[SET][J] = sw_lds_read16<J * 32 * SD_ROW>(rb);
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
+  using I4 = std::integral_constant<int, 4>;
+  using I5 = std::integral_constant<int, 5>;
+
+  // One k-step: the 24 MFMAs of step KK from query set SET; behind them, one at a time, the reads of the step
+  // that follows (k-step NKK of stage `nstage`, query set 1 - SET) and whatever `side(n)` adds behind MFMA n.
+  // LDS reads return in order, so "at most N outstanding" names the read that has arrived.  Issue order within a
+  // step: A0 B0 B1 B2 A1 B3 A2 A3 A4 A5 (behind MFMAs 3 4 5 6 7 8 11 15 19 23).
+  //   before MFMA 0:  A0, B0..B3, A1 of this step, i.e. all but the last four reads of the step before   -> 4
+  //   before MFMA 8:  A2; younger: A3 A4 A5 and this step's A0 B0 B1 B2 A1                                  -> 8
+  //   before MFMA 12: A3; younger: A4 A5, A0 B0 B1 B2 A1 B3 A2                                              -> 9
+  //   before MFMA 16: A4; younger: A5, A0 B0 B1 B2 A1 B3 A2 A3                                              -> 9
+  //   before MFMA 20: A5; younger: A0 B0 B1 B2 A1 B3 A2 A3 A4                                               -> 9
+  // `mid()` runs before the read behind MFMA 3 (the tile change puts its barrier there).  Every step is the same
+  // code: the very last one reads a step that does not exist (whatever the other stage holds; never used).
+  auto step = [&](auto set_tag, auto kk_tag, auto nkk_tag, int nstage, auto&& mid, auto&& side) {
+    constexpr int SET = decltype(set_tag)::value;
+    constexpr int KK = decltype(kk_tag)::value;
+    using NK = decltype(nkk_tag);
+    using NS = std::integral_constant<int, 1 - SET>;
+    sw_wait_lds<4>();
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      if (i == 2) { sw_wait_lds<8>(); __builtin_amdgcn_sched_barrier(0); }
+      if (i >= 3) { sw_wait_lds<9>(); __builtin_amdgcn_sched_barrier(0); }
+      if (i < 3) ss[i][KK] = M::sumsq(af[i], ss[i][KK]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int n = i * TN + j;
+        if (i < ACC_TM)
+          sw_mfma<T, true>(af[i], bf[SET][j], acc[i][j]);
+        else
+          sw_mfma<T, false>(af[i], bf[SET][j], acc[i][j]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (n == 3) mid();
+        if (n == 3) { rd_base(nstage, NK{}); rd_a(I0{}); }
+        if (n == 4) rd_b(NS{}, I0{});
+        if (n == 5) rd_b(NS{}, I1{});
+        if (n == 6) rd_b(NS{}, I2{});
+        if (n == 7) rd_a(I1{});
+        if (n == 8) rd_b(NS{}, I3{});
+        if (n == 11) rd_a(I2{});
+        if (n == 15) rd_a(I3{});
+        if (n == 19) rd_a(I4{});
+        if (n == 23) rd_a(I5{});
+        side(n);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+  using K0 = std::integral_constant<int, 0>;
+  using K1 = std::integral_constant<int, 1>;
+  using K2 = std::integral_constant<int, 2>;
+  using K3 = std::integral_constant<int, 3>;
+  auto nothing = [] {};
+  auto tile_change = [] {
+    wg_barrier_lds<0>();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // The 20 loads of a tile are spread over a whole tile period, one behind every fourth MFMA: a compute unit takes
+  // its lines from L2 at a fixed pace, and a wave that asks faster than that is held at the load instruction --
+  // with one wave per SIMD, the MFMAs behind it wait too.  Tile t + 2's first five loads go out behind the barrier
+  // that gives up tile t's stage (last step of tile t), the other fifteen during the first three steps of tile
+  // t + 1; the last of them is 14 MFMAs ahead of the barrier that needs it.
+  // There is ONE copy of the tile code and no branch in it: past the end of the row the loads fetch the last K
+  // tile again (into a stage nobody reads any more; a few loads per 192 tiles) and the reads take whatever the
+  // other stage holds.  One copy on purpose: in every copy the compiler has to find registers for the whole tile
+  // without spilling, and a spilled fragment would be stored before its read has arrived -- the first version,
+  // with the first and last tiles peeled off, failed exactly so.
+
+  // prologue: tile 0 lands, its step 0 is read, tile 1 begins
+#pragma unroll
+  for (int idx = 0; idx < NA + NB; ++idx) load_one(0, idx);
+  wg_barrier_lds<0>();
+  __builtin_amdgcn_sched_barrier(0);
+  rd_base(0, K0{});
+  rd_a(I0{});
+  rd_b(S0{}, I0{});
+  rd_b(S0{}, I1{});
+  rd_b(S0{}, I2{});
+  rd_a(I1{});
+  rd_b(S0{}, I3{});
+  rd_a(I2{});
+  rd_a(I3{});
+  rd_a(I4{});
+  rd_a(I5{});
+  {
+    const int k1 = min(1, KT - 1);
+#pragma unroll
+    for (int idx = 0; idx < 5; ++idx) load_one(k1, idx);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  for (int kt = 0; kt < KT; ++kt) {
+    const int st = kt & 1;
+    const int k1 = min(kt + 1, KT - 1);  // the tile whose loads are finished during this one ...
+    const int k2 = min(kt + 2, KT - 1);  // ... and the one whose loads begin behind this tile's barrier
+    // (a clamped tile number only changes where the data comes from: the stage is the one tile kt + 1 / kt + 2 would use)
+    step(S0{}, K0{}, K1{}, st, nothing, [&](int n) {
+      if ((n & 3) == 1 && n <= 21) load_one_to(k1, st ^ 1, 5 + (n >> 2));
+    });
+    step(S1{}, K1{}, K2{}, st, nothing, [&](int n) {
+      if ((n & 3) == 1 && n <= 17) load_one_to(k1, st ^ 1, 11 + (n >> 2));
+    });
+    step(S0{}, K2{}, K3{}, st, nothing, [&](int n) {
+      if ((n & 3) == 1 && n <= 13) load_one_to(k1, st ^ 1, 16 + (n >> 2));
+    });
+    // Last step of the tile.  Its fragments were asked for during the step before; behind its first four MFMAs
+    // every read of this stage has to be back (the stage is given up) and tile kt + 1 has to have landed in the
+    // other stage: all of this wave's loads and reads done, then the barrier makes that all waves'.  Behind the
+    // barrier: step 0 of tile kt + 1 is read, and tile kt + 2 begins to load into the stage just given up.
+    step(S1{}, K3{}, K0{}, st ^ 1, tile_change, [&](int n) {
+      if ((n & 3) == 1 && n >= 5) load_one_to(k2, st, (n >> 2) - 1);
+    });
+    // The MFMAs are opaque to the compiler, which therefore adds no wait states before code of its own that reads
+    // an accumulator (it may place such code right behind the loop): the last results are given their 20 states
+    // here, where it cannot get in between.
+    asm volatile("s_nop 15\n\ts_nop 4" ::: "memory");
+  }
+  sw_wait_lds<0>();
+
+  // ---- row sum of squares -> per-row multiplier (the tile buffers are free now) ----------------------------
+  wg_barrier_lds<0>();  // every wave is past its last fragment read
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) ss[i][kk] += __shfl_xor(ss[i][kk], 32);
+    const float ssq = (ss[i][0] + ss[i][1]) + (ss[i][2] + ss[i][3]);
+    if (fh == 0) {
+      const int row = wm * WTM + (wn * 3 + i) * 32 + fr;
+      float w = args.query_scale;
+      if (args.unit_norm) w = ssq > 0.f ? args.query_scale / sqrtf(ssq) : 0.f;
+      s_inv[row] = w;
+      const int64_t grow = g_row0 + row;
+      if (qt == 0 && args.sumsq != nullptr && grow < args.rows) args.sumsq[args.row0 + grow] = ssq;
+    }
+  }
+  __syncthreads();
+
+  scan_tile_epilogue<TM, TN, WTM, WTN, WN>(args, acc, s_inv, wm, wn, fr, fh, g_row0, q_row0, qt, 3 * wn);
 }
 
 // ---- few queries: the store streamed once, no tiles in LDS ---------------------------------------
@@ -960,6 +1293,12 @@ static ScanLayout scan_layout(int Q, int k, int64_t chunk_rows) {
 // default keeps Q * chunk near 64 Mi entries (512 MB) -- 65536 rows at 1024 queries, more for fewer.
 static int64_t effective_chunk(int64_t chunk_rows, int Q) {
   if (chunk_rows > 0) return chunk_rows;
+  if (Q > SW_BN) {
+    // many queries: whole rounds of the 384 x 256 tile kernel (24 576 rows each), Q * chunk near 96 Mi entries --
+    // 98 304 rows at 1024 queries
+    const int64_t c = ((int64_t)96 << 20) / Q / SW_ROUND_ROWS * SW_ROUND_ROWS;
+    if (c >= SW_ROUND_ROWS) return c;
+  }
   int64_t c = ((int64_t)64 << 20) / (Q > 0 ? Q : 1);
   if (c > ((int64_t)1 << 20)) c = (int64_t)1 << 20;
   if (c < SCAN_DEFAULT_CHUNK) c = SCAN_DEFAULT_CHUNK;
@@ -1037,6 +1376,12 @@ static int launch_gemm(const ScanArgs& a, bool aligned, hipStream_t st) {
   return launch_gemm_v<T, BM, BN, WM, WN, true, PF, false>(a, st);
 }
 
+// Whether passes of this scan can run on the 384 x 256 tile kernel (whole rounds of it; see scan_wide_kernel).
+static bool wide_scan_ok(int dtype, bool aligned, int64_t D, int64_t stride, int Q) {
+  return dtype != BGX_F32 && aligned && D % 64 == 0 && Q > SW_BN && !switches().scan_wide_off &&
+         stride * 2 * (SW_BM + 8) < ((int64_t)1 << 32) && D * 2 * (SW_BN + 8) < ((int64_t)1 << 32);
+}
+
 template <typename T>
 static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
   // large tiles when there is enough work to fill the chip with them
@@ -1048,6 +1393,16 @@ static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
     a.q_tiles = (a.Q + BN - 1) / BN;
     a.n_parts = a.q_tiles * 4;
     if constexpr (sizeof(T) == 2) {
+      if (wide_scan_ok(Elem<T>::code, aligned, a.D, a.store_stride, a.Q) && a.rows % SW_ROUND_ROWS == 0) {
+        a.row_tiles = (int)(a.rows / SW_BM);
+        a.q_tiles = (a.Q + SW_BN - 1) / SW_BN;
+        a.n_parts = a.q_tiles * 2;
+        auto kern = scan_wide_kernel<T>;
+        BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SW_LDS_BYTES));
+        hipLaunchKernelGGL(kern, dim3((unsigned)(a.row_tiles * a.q_tiles)), dim3(SW_THREADS), SW_LDS_BYTES, st, a);
+        BGX_HIP(hipGetLastError());
+        return 0;
+      }
       // aligned 16-bit operands, D a multiple of the K tile: tiles loaded straight into LDS
       if (aligned && a.D % 64 == 0 && !switches().scan_direct_off) {
         const int row_tiles_pad = (a.row_tiles + 7) / 8 * 8;
@@ -1206,6 +1561,9 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
       if (rows > lim) rows = lim;
     }
     if (row_part != nullptr && rows > chunk) rows = chunk;  // the partial sums of one pass fit the workspace
+    // many queries: passes of whole rounds of the 384 x 256 tile kernel; what is left over at the end of the store
+    // (and the short opening passes) go to the 256 x 256 kernels, whose scores are the same bits
+    if (rows >= SW_ROUND_ROWS && wide_scan_ok(dtype, aligned, D, stride, Q)) rows = rows / SW_ROUND_ROWS * SW_ROUND_ROWS;
     ScanArgs a;
     a.store = store;
     a.queries = queries;

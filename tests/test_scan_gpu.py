@@ -311,3 +311,38 @@ def test_scan_many_queries_direct_tiles(device, dtype, D, Q):
     same = small.topk_indices == res.topk_indices
     assert same.float().mean().item() > 0.99
     assert (small.topk_values[same] - res.topk_values[same]).abs().max().item() <= 1e-5
+
+
+@pytest.mark.parametrize("dtype,D,Q", [(torch.float16, 192, 300), (torch.bfloat16, 128, 520), (torch.float16, 64, 1024)])
+def test_scan_wide_tiles_equal_the_256_tiles_bitwise(device, dtype, D, Q, bgx_env):
+    """More than 256 queries over many rows: whole rounds of 24 576 rows run on the 384 x 256 tile kernel (one
+    wave per SIMD, accumulators in both register files), the rest on the 256 x 256 kernels.  Every score is the
+    same sequence of matrix instructions over D in both, and the row norms are summed in the same order: scores,
+    norms, row maxima and the top-k must be the same bits with the wide kernel switched off; the row means add
+    their per-wave partial sums in another order and agree to rounding.  Scores are also held to the oracle."""
+    from bergson_amd import ops
+
+    n, k = 4096 + 16384 + 2 * 24576 + 1500, 40
+    store, queries = make_store(n, D, Q, dtype, seed=3 * D + Q)
+    store[30_000] = 0
+    qd = unit_queries(queries, dtype).to(dtype)
+    dev_store, dev_q = store.to(device), qd.to(device)
+
+    def run():
+        r = ops.scan(dev_store, dev_q, unit_norm=True, k=k, want_row_max=True, want_row_mean=True, want_scores=True,
+                     want_sumsq=True)
+        torch.cuda.synchronize()
+        return r
+
+    wide = run()
+    bgx_env("BGX_SCAN_WIDE_OFF", "1")
+    narrow = run()
+    assert torch.equal(wide.scores, narrow.scores)
+    assert torch.equal(wide.sumsq, narrow.sumsq)
+    assert torch.equal(wide.row_max, narrow.row_max)
+    assert torch.equal(wide.topk_values, narrow.topk_values) and torch.equal(wide.topk_indices, narrow.topk_indices)
+    assert (wide.row_mean - narrow.row_mean).abs().max().item() <= 1e-6
+    ref = oscan.scorer_score({"m": store}, {"m": qd}, ["m"], dtype=torch.float32, unit_normalize=True)  # [n, Q]
+    assert (wide.scores.cpu() - ref).abs().max().item() <= COS_TOL
+    assert wide.scores[30_000].abs().max().item() == 0
+    check_topk(wide.topk_values.cpu(), wide.topk_indices.cpu(), ref.T, k)
