@@ -572,6 +572,7 @@ constexpr int SW_BM = 384, SW_BN = 256, SW_THREADS = 256;
 constexpr int SW_A_BYTES = SW_BM * SD_ROW, SW_B_BYTES = SW_BN * SD_ROW, SW_STAGE = SW_A_BYTES + SW_B_BYTES;
 constexpr int SW_LDS_BYTES = 2 * SW_STAGE;
 constexpr int64_t SW_ROUND_ROWS = 64 * SW_BM;  // rows of one round of the chip: 64 row tiles x 4 query tiles = 256 tiles
+constexpr int64_t SW_MIN_ROWS = 8192;          // shorter passes leave most of the chip idle whatever the tile
 
 template <int OFF>
 __device__ inline uint4 sw_lds_read16(uint32_t addr) {
@@ -654,8 +655,11 @@ __global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
   const uint32_t q_bytes = (uint32_t)(args.D * sizeof(T));
   const uint64_t a_base = (uint64_t)(uintptr_t)args.store + (uint64_t)((args.row0 + g_row0) * args.store_stride) * sizeof(T);
   const uint64_t b_base = (uint64_t)(uintptr_t)args.queries + (uint64_t)(q_row0 * args.D) * sizeof(T);
-  const uint32_t a_voff = (uint32_t)lrow * row_bytes + (uint32_t)lch * 16u;
+  const int r_last = (int)min((int64_t)SW_BM, args.rows - g_row0) - 1;  // last valid row of this tile, likewise
   const int q_last = args.Q - 1 - (int)q_row0;  // last valid query row of this tile (rows past it repeat it)
+  uint32_t a_voff[NA];
+#pragma unroll
+  for (int i = 0; i < NA; ++i) a_voff[i] = (uint32_t)min(i * 32 + lrow, r_last) * row_bytes + (uint32_t)lch * 16u;
   uint32_t b_voff[NB];
 #pragma unroll
   for (int i = 0; i < NB; ++i) b_voff[i] = (uint32_t)min(i * 32 + lrow, q_last) * q_bytes + (uint32_t)lch * 16u;
@@ -666,7 +670,7 @@ __global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
     const uint32_t stage = lds_wave + (uint32_t)stg * SW_STAGE;
     const uint64_t koff = (uint64_t)kt * (BK * sizeof(T));
     if (idx < NA)
-      sw_load_lds16(a_base + koff, a_voff + (uint32_t)idx * 32u * row_bytes, stage + (uint32_t)idx * 4096u);
+      sw_load_lds16(a_base + koff, a_voff[idx], stage + (uint32_t)idx * 4096u);
     else
       sw_load_lds16(b_base + koff, b_voff[idx - NA], stage + (uint32_t)(SW_A_BYTES + (idx - NA) * 4096));
   };
@@ -812,7 +816,7 @@ __global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
   {
     const int k1 = min(1, KT - 1);
 #pragma unroll
-    for (int idx = 0; idx < 5; ++idx) load_one(k1, idx);
+    for (int idx = 0; idx < 5; ++idx) load_one_to(k1, 1, idx);  // what the last step of a tile issues for the next but one
   }
   __builtin_amdgcn_sched_barrier(0);
 
@@ -1393,13 +1397,14 @@ static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
     a.q_tiles = (a.Q + BN - 1) / BN;
     a.n_parts = a.q_tiles * 4;
     if constexpr (sizeof(T) == 2) {
-      if (wide_scan_ok(Elem<T>::code, aligned, a.D, a.store_stride, a.Q) && a.rows % SW_ROUND_ROWS == 0) {
-        a.row_tiles = (int)(a.rows / SW_BM);
+      if (wide_scan_ok(Elem<T>::code, aligned, a.D, a.store_stride, a.Q) && a.rows >= SW_MIN_ROWS) {
+        a.row_tiles = (int)((a.rows + SW_BM - 1) / SW_BM);
+        const int row_tiles_pad = (a.row_tiles + 7) / 8 * 8;
         a.q_tiles = (a.Q + SW_BN - 1) / SW_BN;
         a.n_parts = a.q_tiles * 2;
         auto kern = scan_wide_kernel<T>;
         BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SW_LDS_BYTES));
-        hipLaunchKernelGGL(kern, dim3((unsigned)(a.row_tiles * a.q_tiles)), dim3(SW_THREADS), SW_LDS_BYTES, st, a);
+        hipLaunchKernelGGL(kern, dim3((unsigned)(row_tiles_pad * a.q_tiles)), dim3(SW_THREADS), SW_LDS_BYTES, st, a);
         BGX_HIP(hipGetLastError());
         return 0;
       }
@@ -1555,14 +1560,17 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
       // the first pass has no threshold yet and appends every score: each query's list grows by one
       // serialised atomic per row, so that pass stays small and later passes grow fourfold
       int64_t lim = done == 0 ? SCAN_FIRST_CHUNK : done * 4;
+      // with the wide tile kernel the second pass is a whole round already (thresholds from 4096 rows let
+      // through k / 4096 of the scores: a few hundred candidates per query)
+      if (done > 0 && lim < SW_ROUND_ROWS && wide_scan_ok(dtype, aligned, D, stride, Q)) lim = SW_ROUND_ROWS;
       if (stream_scan) lim = done == 0 ? stream_first : chunk;
       if (lim < k) lim = k;
       if (lim > chunk) lim = chunk;
       if (rows > lim) rows = lim;
     }
     if (row_part != nullptr && rows > chunk) rows = chunk;  // the partial sums of one pass fit the workspace
-    // many queries: passes of whole rounds of the 384 x 256 tile kernel; what is left over at the end of the store
-    // (and the short opening passes) go to the 256 x 256 kernels, whose scores are the same bits
+    // many queries: long passes are cut to whole rounds of the 384 x 256 tile kernel (the end of the store makes
+    // one last, shorter pass)
     if (rows >= SW_ROUND_ROWS && wide_scan_ok(dtype, aligned, D, stride, Q)) rows = rows / SW_ROUND_ROWS * SW_ROUND_ROWS;
     ScanArgs a;
     a.store = store;
