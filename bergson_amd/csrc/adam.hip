@@ -17,7 +17,10 @@
 
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "common.hpp"
+#include "direct.hpp"
 #include "mma16.hpp"
 #include "mma32.hpp"
 
@@ -530,6 +533,301 @@ __global__ __launch_bounds__(512) void adam_fused_kernel(FusedArgs a) {
   }
 }
 
+// ---- fused path, tiles loaded straight into LDS ------------------------------------------------------------
+// The same computation as adam_fused_kernel with the store scan's direct-to-LDS pipeline (direct.hpp) and the
+// second pass fed from LDS as well:
+//  * eight waves as 8 x 1: a wave owns 32 tokens against all 256 table rows of the chunk (8 blocks of 32 x 32,
+//    128 accumulators); its half of nothing is added to another wave's, so there is no exchange at the end;
+//  * one ring of tiles -- three row buffers, two operand buffers, 160 KB -- carries two kinds of tile: the K tiles
+//    of a chunk (256 tokens x 64 of I against 256 table rows x 64), and behind them four slices of the chunk's g
+//    values (256 tokens x 64 output features, whole 128-byte lines, in a row buffer) with the matching slice of L
+//    (p rows x 64 features, in the operand buffer, which a g slice does not otherwise need).  The g values used to
+//    be fetched by the lanes that needed them, 32 bytes of 32 different lines per load instruction, and came
+//    through the L1 up to four times: with the path from L2 into the CU as the bound, a quarter of the kernel;
+//  * a g slice is four MFMAs per wave (H of two 32-feature blocks, scaled by g in registers, against L), its
+//    operands read from LDS with the K tiles' swizzle; nothing of the second pass touches global memory, and its
+//    loads travel two tiles ahead like all others;
+//  * loads are uniform base + 32-bit lane offset (sw_load_lds16), fragment reads and waits are spelled out as in
+//    scan_direct_kernel.
+// Token tile x column mapping to workgroups (ttx), validity masking and the ptok layout are the old kernel's.
+constexpr int FD_A_BYTES = FUSED_TILE * SD_ROW, FD_B_BYTES = FUSED_TILE * SD_ROW;
+constexpr int FD_LDS_BYTES = 3 * FD_A_BYTES + 2 * FD_B_BYTES;
+constexpr int FD_GSLICES = 4;  // slices of 64 output features per chunk of 256
+
+template <typename T>
+__global__ __launch_bounds__(512) void adam_fused_direct_kernel(FusedArgs a) {
+  using M = Mma32<T>;
+  static_assert(sizeof(T) == 2, "the fused Adam kernel is for 16-bit model dtypes");
+  constexpr int BM = FUSED_TILE, BN = FUSED_TILE, BK = 64;
+  constexpr int TN = BN / 32;  // 8 table-row blocks per wave; one token block
+  extern __shared__ __align__(128) unsigned char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int fr = lane & 31;
+  const int fh = lane >> 5;
+  int tt = blockIdx.x, j = blockIdx.y;
+  if (a.ttx > 0) {
+    const int b = blockIdx.x + gridDim.x * blockIdx.y;
+    const int xcd = b & 7, slot = b >> 3;
+    const int jx = 32 / a.ttx, n_super_tt = gridDim.x / a.ttx;
+    const int super = (slot >> 5) * 8 + xcd, within = slot & 31;
+    tt = (super % n_super_tt) * a.ttx + within % a.ttx;
+    j = (super / n_super_tt) * jx + within / a.ttx;
+  }
+  const int t_row0 = tt * BM;  // chunk-local first token of the tile
+  const int p = a.p, O = a.O, pp = p * p;
+  const int rows_here = a.tokens - t_row0;  // valid tokens of this tile (may exceed BM)
+  const int KT = a.I / BK;
+  const int n_chunks = O / BN;
+  const int per_chunk = KT + FD_GSLICES;
+  const int total = per_chunk * n_chunks;
+
+  // ---- loader: instruction i of wave w fills rows i * 64 + w * 8 .. + 7 of a 256-row tile; lane l is position
+  // l & 7 of row l >> 3 and fetches chunk (l & 7) ^ sd_key(row).  Rows past the end repeat the last one.
+  const uint32_t a_row_bytes = (uint32_t)(a.a_tok_stride * sizeof(T));
+  const uint32_t g_row_bytes = (uint32_t)(a.g_tok_stride * sizeof(T));
+  const uint32_t t_row_bytes = (uint32_t)(a.I * sizeof(T));
+  const uint32_t l_row_bytes = (uint32_t)(O * sizeof(T));
+  uint32_t voff_a[4], voff_g[4], voff_t[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = i * 64 + wave * 8 + (lane >> 3);
+    const uint32_t ch = (uint32_t)((lane & 7) ^ sd_key(r)) * 16u;
+    const uint32_t rc = (uint32_t)min(r, rows_here - 1);
+    voff_a[i] = rc * a_row_bytes + ch;
+    voff_g[i] = rc * g_row_bytes + ch;
+    // table row that goes to LDS row r: bits (q1 q0 h c1 c0) -> (h q1 q0 c1 c0) within each block of 32, so that a
+    // lane's 16 accumulators of a block are 16 consecutive output features (see adam_fused_kernel)
+    const int pr = (r & ~31) | ((r & 4) << 2) | ((r & 24) >> 1) | (r & 3);
+    voff_t[i] = (uint32_t)pr * t_row_bytes + ch;
+  }
+  // L slice: rows 0 .. 31 of the operand buffer, loaded by waves 0 .. 3 (8 rows each); rows past p repeat row p - 1
+  const uint32_t voff_l = (uint32_t)min((wave & 3) * 8 + (lane >> 3), p - 1) * l_row_bytes +
+                          (uint32_t)((lane & 7) ^ sd_key(wave * 8 + (lane >> 3))) * 16u;
+  const uint64_t act_base = (uint64_t)(uintptr_t)a.a + (uint64_t)t_row0 * a_row_bytes;
+  const uint64_t g_base = (uint64_t)(uintptr_t)a.g + (uint64_t)(a.t0 + t_row0) * g_row_bytes;
+  const uint64_t tab_base = (uint64_t)(uintptr_t)a.table + (uint64_t)j * O * t_row_bytes;
+  const uint64_t l_base = (uint64_t)(uintptr_t)a.r_out;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+  const uint32_t lds_wave = lds0 + (uint32_t)wave * 1024u;
+  // tile t of the sequence: chunk t / per_chunk, position t % per_chunk (< KT: K tile, else g slice)
+  int ld_a_pos = 0, ld_a_chunk = 0, ld_b_pos = 0, ld_b_chunk = 0;  // the two loaders' own places in the sequence
+  auto load_a = [&](int t) {
+    const uint32_t dst = lds_wave + (uint32_t)(t % 3) * FD_A_BYTES;
+    if (ld_a_pos < KT) {
+      const uint64_t base = act_base + (uint64_t)ld_a_pos * (BK * sizeof(T));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sw_load_lds16(base, voff_a[i], dst + (uint32_t)i * 8192u);
+    } else {
+      const uint64_t base = g_base + ((uint64_t)ld_a_chunk * BN + (uint64_t)(ld_a_pos - KT) * 64) * sizeof(T);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sw_load_lds16(base, voff_g[i], dst + (uint32_t)i * 8192u);
+    }
+    if (++ld_a_pos == per_chunk) {
+      ld_a_pos = 0;
+      ++ld_a_chunk;
+    }
+  };
+  auto load_b = [&](int t) {
+    const uint32_t dst = lds_wave + (uint32_t)(3 * FD_A_BYTES) + (uint32_t)(t & 1) * FD_B_BYTES;
+    const bool is_k = ld_b_pos < KT;
+    const uint64_t base =
+        is_k ? tab_base + (uint64_t)ld_b_chunk * BN * t_row_bytes + (uint64_t)ld_b_pos * (BK * sizeof(T))
+             : l_base + ((uint64_t)ld_b_chunk * BN + (uint64_t)(ld_b_pos - KT) * 64) * sizeof(T);
+    // an L slice is 32 rows: instruction 0 of waves 0 .. 3 (the other waves fetch the same rows again into rows
+    // 32 .. 63 of the buffer, which nothing reads: every wave then issues the same number of loads, and
+    // "all but the youngest four" means the same thing to all of them)
+    if (is_k) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sw_load_lds16(base, voff_t[i], dst + (uint32_t)i * 8192u);
+    } else {
+      sw_load_lds16(base, voff_l, dst);
+    }
+    if (++ld_b_pos == per_chunk) {
+      ld_b_pos = 0;
+      ++ld_b_chunk;
+    }
+  };
+
+  f32x16 pacc;
+  f32x16 acc[TN];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) pacc[e] = 0.f;
+#pragma unroll
+  for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[jj][e] = 0.f;
+
+  // fragment reads: the wave's 32 token rows (one fragment per k-step) and all 256 table rows (eight)
+  const uint32_t key = (uint32_t)sd_key(fr);  // rows advance in steps of 32: the key depends on fr alone
+  const uint32_t a_frag = lds0 + (uint32_t)((wave * 32 + fr) * SD_ROW);
+  const uint32_t b_frag = lds0 + (uint32_t)(3 * FD_A_BYTES + fr * SD_ROW);
+  uint4 af[2], bf[2][TN];
+  auto rd = [&](int t, auto kk_tag, auto set_tag) {
+    constexpr int SET = decltype(set_tag)::value;
+    constexpr int KK = decltype(kk_tag)::value;
+    const uint32_t chk = (((uint32_t)(KK * 2 + fh)) ^ key) * 16u;
+    const uint32_t ab = a_frag + (uint32_t)(t % 3) * FD_A_BYTES + chk;
+    const uint32_t bb = b_frag + (uint32_t)(t & 1) * FD_B_BYTES + chk;
+    af[SET] = sd_lds_read16(ab);
+    bf[SET][0] = sw_lds_read16<0 * 32 * SD_ROW>(bb);
+    bf[SET][1] = sw_lds_read16<1 * 32 * SD_ROW>(bb);
+    bf[SET][2] = sw_lds_read16<2 * 32 * SD_ROW>(bb);
+    bf[SET][3] = sw_lds_read16<3 * 32 * SD_ROW>(bb);
+    bf[SET][4] = sw_lds_read16<4 * 32 * SD_ROW>(bb);
+    bf[SET][5] = sw_lds_read16<5 * 32 * SD_ROW>(bb);
+    bf[SET][6] = sw_lds_read16<6 * 32 * SD_ROW>(bb);
+    bf[SET][7] = sw_lds_read16<7 * 32 * SD_ROW>(bb);
+  };
+  auto mm = [&](auto set_tag) {
+    constexpr int SET = decltype(set_tag)::value;
+#pragma unroll
+    for (int jj = 0; jj < TN; ++jj) M::mma(bf[SET][jj], af[SET], acc[jj]);  // transposed block: rows = output features
+  };
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+  using K0 = std::integral_constant<int, 0>;
+  using K1 = std::integral_constant<int, 1>;
+  using K2 = std::integral_constant<int, 2>;
+  using K3 = std::integral_constant<int, 3>;
+  constexpr int WAIT_LDS_STEP = 0xC07F | ((1 + TN) << 8);  // lgkmcnt(9): the step issued before the latest nine reads
+  constexpr int WAIT_LDS_0 = 0xC07F;
+
+  // prologue: tile 0 lands, its step 0 is read; tile 1's operands and tile 2's rows are under way
+  load_a(0);
+  load_b(0);
+  if (total > 1) {
+    load_a(1);
+    wg_barrier_lds<4>();
+  } else {
+    wg_barrier_lds<0>();
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  rd(0, K0{}, S0{});
+  __builtin_amdgcn_sched_barrier(0);
+  if (1 < total) load_b(1);
+  if (2 < total) load_a(2);
+
+  auto tile_end_barrier = [&](int t) {
+    // In flight, oldest first: rows(t + 1), then operands(t + 1) and rows(t + 2).  Tile t + 1 must have landed
+    // (this wave's part; the barrier makes that all of it), rows(t + 2) -- always the youngest four loads of a
+    // wave -- may still fly; this tile's reads have completed, so its buffers can take operands(t + 2) and
+    // rows(t + 3) behind the barrier.
+    if (t + 2 < total)
+      wg_barrier_lds<4>();
+    else
+      wg_barrier_lds<0>();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // one g slice: pacc[t, i] += sum over its 64 features of (H[t, o] * g[t, o]) * L[i, o].  H of slice S is
+  // accumulator blocks 2 S and 2 S + 1; lane (fr, fh) holds token fr and features fh * 16 + e of a block, and takes
+  // them eight at a time (sp = 0, 1): 16-byte chunk 4 b + 2 fh + sp of the token's 128 bytes of g, and the same
+  // chunk of row fr of L.
+  auto g_slice = [&](int t, auto s_tag) {
+    constexpr int S = decltype(s_tag)::value;
+    const uint32_t gb = a_frag + (uint32_t)(t % 3) * FD_A_BYTES;
+    const uint32_t lb = b_frag + (uint32_t)(t & 1) * FD_B_BYTES;
+    uint4 gq[4], lq[4];
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      const uint32_t chk = (((uint32_t)((n >> 1) * 4 + fh * 2 + (n & 1))) ^ key) * 16u;
+      gq[n] = sd_lds_read16(gb + chk);
+      lq[n] = sd_lds_read16(lb + chk);
+    }
+    __builtin_amdgcn_s_waitcnt(WAIT_LDS_0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      const int sp = n & 1;
+      const f32x16& h = acc[2 * S + (n >> 1)];
+      uint4 zf;
+      zf.x = scaled_pair_bits<T>(h[8 * sp + 0], h[8 * sp + 1], gq[n].x);
+      zf.y = scaled_pair_bits<T>(h[8 * sp + 2], h[8 * sp + 3], gq[n].y);
+      zf.z = scaled_pair_bits<T>(h[8 * sp + 4], h[8 * sp + 5], gq[n].z);
+      zf.w = scaled_pair_bits<T>(h[8 * sp + 6], h[8 * sp + 7], gq[n].w);
+      M::mma(zf, lq[n], pacc);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  int t = 0;
+  for (int c = 0; c < n_chunks; ++c) {
+    // ---- the chunk's K tiles: four k-steps each, fragments double-buffered, the pipeline runs across the barrier
+    for (int kt = 0; kt < KT; ++kt, ++t) {
+      __builtin_amdgcn_sched_barrier(0);
+      rd(t, K1{}, S1{});
+      __builtin_amdgcn_s_waitcnt(WAIT_LDS_STEP);
+      __builtin_amdgcn_sched_barrier(0);
+      mm(S0{});
+      __builtin_amdgcn_sched_barrier(0);
+      rd(t, K2{}, S0{});
+      __builtin_amdgcn_s_waitcnt(WAIT_LDS_STEP);
+      __builtin_amdgcn_sched_barrier(0);
+      mm(S1{});
+      __builtin_amdgcn_sched_barrier(0);
+      rd(t, K3{}, S1{});
+      __builtin_amdgcn_s_waitcnt(WAIT_LDS_STEP);
+      __builtin_amdgcn_sched_barrier(0);
+      mm(S0{});
+      __builtin_amdgcn_sched_barrier(0);
+      tile_end_barrier(t);
+      if (kt + 1 < KT) rd(t + 1, K0{}, S0{});
+      __builtin_amdgcn_sched_barrier(0);
+      mm(S1{});  // its fragments arrived before the barrier
+      __builtin_amdgcn_sched_barrier(0);
+      // the loads go out behind the first MFMAs after the barrier, so that those are not held up by their issue
+      if (t + 2 < total) load_b(t + 2);
+      if (t + 3 < total) load_a(t + 3);
+    }
+    // ---- the chunk's four g slices
+    g_slice(t, std::integral_constant<int, 0>{});
+    tile_end_barrier(t);
+    load_b(t + 2);
+    load_a(t + 3);
+    ++t;
+    g_slice(t, std::integral_constant<int, 1>{});
+    tile_end_barrier(t);
+    if (t + 2 < total) load_b(t + 2);
+    if (t + 3 < total) load_a(t + 3);
+    ++t;
+    g_slice(t, std::integral_constant<int, 2>{});
+    tile_end_barrier(t);
+    if (t + 2 < total) load_b(t + 2);
+    if (t + 3 < total) load_a(t + 3);
+    ++t;
+    g_slice(t, std::integral_constant<int, 3>{});
+#pragma unroll
+    for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[jj][e] = 0.f;
+    __builtin_amdgcn_sched_barrier(0);
+    tile_end_barrier(t);
+    if (c + 1 < n_chunks) rd(t + 1, K0{}, S0{});
+    __builtin_amdgcn_sched_barrier(0);
+    if (t + 2 < total) load_b(t + 2);
+    if (t + 3 < total) load_a(t + 3);
+    ++t;
+  }
+  __builtin_amdgcn_s_waitcnt(WAIT_LDS_0);
+
+  // pacc[e] = P[token (e>>2)*8 + fh*4 + (e&3) of this wave's 32][row fr], column j
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const int tl = t_row0 + wave * 32 + (e >> 2) * 8 + fh * 4 + (e & 3);
+    if (tl < a.tokens && fr < p) {
+      bool valid = true;
+      if (a.lengths != nullptr) {
+        const int64_t t = a.t0 + tl;
+        const int n = (int)(t / a.S);
+        valid = (int)(t - (int64_t)n * a.S) < a.lengths[n] - 1;
+      }
+      a.ptok[(int64_t)tl * pp + fr * p + j] = valid ? pacc[e] : 0.f;
+    }
+  }
+}
+
 // per-token rows from ptok: clamp, cast, scatter to the rows of the valid tokens
 __global__ __launch_bounds__(256) void adam_tok_finalize_kernel(const float* __restrict__ ptok, int64_t t0, int tokens,
                                                                 int S, int pp, const int32_t* __restrict__ lengths,
@@ -727,7 +1025,23 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
         }
       }
       f.ttx = ttx;
-      if (dtype == BGX_F16) {
+      // tiles straight into LDS, the second pass fed from LDS: needs g uniformly strided over the flattened tokens
+      // and 32-bit byte offsets within a tile
+      const bool direct = !switches().adam_direct_off && (N == 1 || g_seq_stride == (int64_t)S * g_tok_stride) &&
+                          (int64_t)FUSED_TILE * a_tok_stride * 2 < ((int64_t)1 << 32) &&
+                          (int64_t)FUSED_TILE * g_tok_stride * 2 < ((int64_t)1 << 32) &&
+                          (int64_t)FUSED_TILE * I * 2 < ((int64_t)1 << 32) && (int64_t)p * O * 2 < ((int64_t)1 << 32);
+      if (direct) {
+        if (dtype == BGX_F16) {
+          auto kern = adam_fused_direct_kernel<f16_t>;
+          BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, FD_LDS_BYTES));
+          hipLaunchKernelGGL(kern, grid, dim3(512), FD_LDS_BYTES, st, f);
+        } else {
+          auto kern = adam_fused_direct_kernel<bf16_t>;
+          BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, FD_LDS_BYTES));
+          hipLaunchKernelGGL(kern, grid, dim3(512), FD_LDS_BYTES, st, f);
+        }
+      } else if (dtype == BGX_F16) {
         auto kern = adam_fused_kernel<f16_t>;
         BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         hipLaunchKernelGGL(kern, grid, dim3(512), smem, st, f);

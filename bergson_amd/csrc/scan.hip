@@ -33,6 +33,7 @@
 #include <utility>
 
 #include "common.hpp"
+#include "direct.hpp"
 #include "mma32.hpp"
 #include "stream.hpp"
 
@@ -335,33 +336,12 @@ __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
 //    barrier is the bare s_barrier (wg_barrier_lds) -- __syncthreads would wait for every outstanding load;
 //  * the fragments are double-buffered in registers and the pipeline runs across the barrier: the reads of
 //    step 0 of the next tile are issued right after it, before the MFMAs of the last step of this tile.
-constexpr int SD_BM = 256, SD_ROW = 128;
+constexpr int SD_BM = 256;
 constexpr int SD_A_BYTES = SD_BM * SD_ROW;
 constexpr int SD_THREADS = 512;
 // BN = 256, or 128 for at most 128 queries (one query tile: half the MFMA work of a 256-wide tile that would be
 // half empty)
 constexpr int sd_lds_bytes(int bn) { return 3 * SD_A_BYTES + 2 * bn * SD_ROW; }
-
-__device__ inline int sd_key(int row) { return (row & 7) ^ ((row >> 3) & 1); }
-
-// Workgroup barrier without a fence (a fence would wait for every load in flight): waits for this wave's LDS
-// traffic, and for all but the youngest VM_LEFT of its vector-memory operations, then s_barrier.  The memory
-// clobber keeps the compiler from moving memory accesses across it.
-template <int VM_LEFT>
-__device__ inline void wg_barrier_lds() {
-  static_assert(VM_LEFT == 0 || VM_LEFT == 4, "spelled-out wait counts");
-  if constexpr (VM_LEFT == 0)
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  else
-    asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
-// 16 bytes from LDS byte address `addr`; the caller waits (lgkmcnt) before it uses the value
-__device__ inline uint4 sd_lds_read16(uint32_t addr) {
-  uint4 v;
-  asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr) : "memory");
-  return v;
-}
 
 template <typename T, int BN, bool ONE_QT>
 __global__ __launch_bounds__(SD_THREADS) void scan_direct_kernel(ScanArgs args) {
@@ -574,13 +554,6 @@ constexpr int SW_LDS_BYTES = 2 * SW_STAGE;
 constexpr int64_t SW_ROUND_ROWS = 64 * SW_BM;  // rows of one round of the chip: 64 row tiles x 4 query tiles = 256 tiles
 constexpr int64_t SW_MIN_ROWS = 8192;          // shorter passes leave most of the chip idle whatever the tile
 
-template <int OFF>
-__device__ inline uint4 sw_lds_read16(uint32_t addr) {
-  uint4 v;
-  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
-  return v;
-}
-
 // One 32 x 32 x 16 MFMA with the accumulator block pinned to the AccVGPRs (IN_ACC) or to the ordinary VGPRs.
 // Written as instructions: 384 accumulator registers beside 60 of fragments leave the register allocator no
 // slack, and left to itself it shuffles blocks between the two files and spills.  (Volatile: the statements
@@ -605,16 +578,6 @@ __device__ inline void sw_mfma(const uint4& a, const uint4& b, f32x16& c) {
 template <int N>
 __device__ inline void sw_wait_lds() {  // s_waitcnt lgkmcnt(N), nothing else
   __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8));
-}
-
-// 16 bytes per lane from global memory (uniform 64-bit base + one 32-bit offset per lane) straight to LDS at
-// byte address `lds` + 16 * lane.  Spelled out so that a load is four instructions (M0, the wait state it needs,
-// the load, and at most one add for the offset) -- the builtin went through 64-bit vector address arithmetic.
-__device__ inline void sw_load_lds16(uint64_t base, uint32_t voff, uint32_t lds) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               :
-               : "v"(voff), "s"(base), "s"(lds)
-               : "memory", "m0");
 }
 
 template <typename T>

@@ -39,7 +39,7 @@ def _ptr(t: Tensor | None) -> C.c_void_p | None:
     return None if t is None else C.c_void_p(t.data_ptr())
 
 
-_workspaces: dict[tuple[int, str], Tensor] = {}
+_workspaces: dict[tuple[int, int, str], Tensor] = {}
 
 # When set to a list, every collection launch appends (start_event, stop_event, algorithmic_bytes): the
 # events bracket the launch on the stream it runs on.  Used by the benchmark; None costs nothing.
@@ -47,8 +47,11 @@ collect_timer: list | None = None
 
 
 def _workspace(device: torch.device, nbytes: int, tag: str) -> Tensor:
-    """Per-device scratch buffer, grown on demand and reused between calls (stream-ordered)."""
-    key = (device.index if device.index is not None else torch.cuda.current_device(), tag)
+    """Scratch buffer per (device, stream, purpose), grown on demand and reused between calls.  One per stream:
+    launches on different streams may overlap, and a buffer that is replaced by a larger one goes back to the
+    allocator, which only orders its reuse against the stream it was allocated on."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    key = (index, torch.cuda.current_stream(device).cuda_stream, tag)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
@@ -272,6 +275,36 @@ def collect_prepared(per_token: bool, items: list, p: int, out: Tensor, lengths:
     del keep
 
 
+adam_table_budget_bytes: int | None = None
+"""Device memory the Adam tables of all modules may hold together; None = a quarter of the device's memory."""
+_tables_in_use: dict = {}  # id(prep) -> weak reference to it; insertion order = least recently used first
+
+
+def _touch_table(prep: "AdamPrepared") -> None:
+    """Marks `prep`'s table as just used and drops the least recently used tables beyond the budget."""
+    import weakref
+
+    _tables_in_use.pop(id(prep), None)
+    _tables_in_use[id(prep)] = weakref.ref(prep)
+    budget = adam_table_budget_bytes
+    if budget is None:
+        budget = torch.cuda.get_device_properties(prep.r_in.device).total_memory // 4
+    live = {}
+    for key, ref in list(_tables_in_use.items()):
+        q = ref()
+        if q is None or q._table is None:
+            del _tables_in_use[key]  # the module's state is gone, or its table was dropped
+        else:
+            live[key] = q
+    held = sum(q._table.numel() * q._table.element_size() for q in live.values())
+    for key, q in live.items():
+        if held <= budget or key == id(prep):
+            break
+        held -= q._table.numel() * q._table.element_size()
+        q._table = None
+        del _tables_in_use[key]
+
+
 class AdamPrepared:
     """Per-module state of the Adam path: the [(O*p), I] table built from the right projection and the
     second moments, and the left projection."""
@@ -303,7 +336,10 @@ class AdamPrepared:
 
     @property
     def table(self) -> Tensor:
-        """[(O*p), I] table of the per-token path, built on first use."""
+        """[(O*p), I] table of the per-token path: p times the bytes of the weight matrix, so the tables of all
+        modules of a large model do not fit beside it.  Built on first use and kept while the tables of the
+        process stay within `adam_table_budget_bytes` (least recently used go first, rebuilt when needed again:
+        one pass over the second moments)."""
         if self._table is None:
             lib = _lib.load()
             nbytes = lib.bgx_adam_table_bytes(self.O, self.I, self.p, dtype_code(self.dtype))
@@ -311,6 +347,9 @@ class AdamPrepared:
             rc = lib.bgx_adam_prepare(_ptr(self.r_in), _ptr(self.v), self.O, self.I, self.p, dtype_code(self.dtype),
                                       _ptr(self._table), _stream())
             _lib.check(rc, "bgx_adam_prepare")
+        _touch_table(self)
+        # the table may be dropped and its memory handed out again while this stream still reads it
+        self._table.record_stream(torch.cuda.current_stream(self._table.device))
         return self._table
 
     def seq_state(self):

@@ -652,3 +652,26 @@ def test_adam_fused_shapes_with_fewer_tokens_than_a_tile(device, per_token, shap
         got = _run_adam(device, case, p, torch.bfloat16)
     assert got.shape == want.shape
     assert rel_l2(got, want) <= TOL[torch.bfloat16]
+
+
+def test_adam_tables_stay_within_their_budget(device, monkeypatch):
+    """The per-module Adam tables (p times the weight bytes each) are dropped least recently used first once
+    together they exceed the budget, and rebuilt on demand with the same contents."""
+    from bergson_amd import ops
+
+    gen = torch.Generator().manual_seed(3)
+    p, I, O = 16, 64, 256
+    preps = []
+    for k in range(3):
+        left, right = module_projections(f"layers.{k}.mlp.dense_h_to_4h", p, O, I, torch.bfloat16)
+        v = torch.rand(O, I, generator=gen) * 1e-5 + 1e-9
+        preps.append(ops.AdamPrepared(right.to(device), left.to(device), v.to(device), 0))
+    one = O * p * I * 2
+    monkeypatch.setattr(ops, "adam_table_budget_bytes", 2 * one)
+    first = preps[0].table.clone()
+    assert preps[1].table is not None and preps[0]._table is not None
+    preps[2].table  # the third table does not fit: the least recently used one goes
+    torch.cuda.synchronize()
+    assert preps[0]._table is None and preps[1]._table is not None and preps[2]._table is not None
+    assert torch.equal(preps[0].table, first)  # rebuilt
+    assert preps[1]._table is None
