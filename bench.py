@@ -46,11 +46,14 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes moved per algorithmic byte by collect_kernel on this workload, from the FETCH_SIZE and
 # WRITE_SIZE hardware counters (profiles/collect_and_scan_kernels_pmc_hbm_traffic.txt)
 COLLECT_TRAFFIC_RATIO = 1.036
-# the same for the store scan: 1024 queries (four query tiles re-read each row tile, half from L2), at most 32 queries
-SCAN_TRAFFIC_RATIO_Q1024 = 1.50
+# the same for the store scan: 1024 queries (four query tiles of 256 re-read each 384-row tile, most of it from the
+# L2 they share), at most 32 queries; and for per-token collection and the Llama-3-8B-shaped layers
+SCAN_TRAFFIC_RATIO_Q1024 = 1.39
 SCAN_TRAFFIC_RATIO_FEW = 1.0016
+PER_TOKEN_TRAFFIC_RATIO = 1.030
+LLAMA_TRAFFIC_RATIO = 1.007
 # bytes the four fused Adam launches of one layer fetch through the L2s and write, from the same counters
-# (profiles/adam_fused_pythia410m_layer_p32.txt): 5.16 GB + 0.07 GB, against 0.94 GB read once each
+# (profiles/adam_fused_pythia410m_layer_p32.txt): 5.14 GB + 0.08 GB, against 0.94 GB read once each
 ADAM_TRAFFIC_BYTES_PER_LAYER = 5.22e9
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
@@ -262,7 +265,8 @@ def scan_leg(args, torch, device):
         "rows": n, "dim": D, "queries": Q, "k": k, "ms": ms, "rows_per_s": n / (ms * 1e-3),
         "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": MFMA_F16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": flops / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
-                     "traffic": n * D * 2 * SCAN_TRAFFIC_RATIO_Q1024},
+                     "traffic": n * D * 2 * SCAN_TRAFFIC_RATIO_Q1024,
+                     "kernel": "bgx::scan_wide_kernel<f16_t> (384 x 256 tiles, operands loaded straight into LDS)"},
         "hbm_gbs": n * D * 2 / (ms * 1e-3) / 1e9,
         "top1_mean": float(res.topk_values[:Q, 0].mean().item()),
     }
@@ -340,7 +344,8 @@ def per_token_leg(args, torch, device):
             "ms_per_launch": ms, "tokens_per_s_hooks_only": N * S / (ms * 1e-3),
             "roofline": {"bound": "hbm", "kernel": "bgx::collect_persist_kernel<bf16_t, true, 2, 4, true, false>",
                          "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-                         "bytes_read": read, "bytes_written": written, "traffic": None}}
+                         "bytes_read": read, "bytes_written": written,
+                         "traffic": (read + written) * PER_TOKEN_TRAFFIC_RATIO}}
 
 
 def llama_leg(args, torch, device):
@@ -394,7 +399,7 @@ def llama_leg(args, torch, device):
                         "bytes_per_launch": nbytes, "ms_per_launch": ms_launch, "launches": len(ms),
                         "ms_per_launch_with_table_build_and_finalize":
                             sum(e0.elapsed_time(e1) for e0, e1, _ in timer) / len(timer),
-                        "traffic": None}}
+                        "traffic": nbytes * LLAMA_TRAFFIC_RATIO}}
     del col, model
     torch.cuda.empty_cache()
     return out
@@ -438,7 +443,8 @@ def adam_leg(args, torch, device):
     return {"workload": "configs[3]: one Pythia-410m layer, 4 x 1024 tokens, p=32, Adam, per-token rows (bf16)",
             "ms_per_layer": total_ms, "tokens_per_s_24_layers_hooks_only": N * S / (total_ms * 24e-3),
             "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                         "frac": tf / MFMA_F16_PEAK_TFLOPS, "traffic": ADAM_TRAFFIC_BYTES_PER_LAYER},
+                         "frac": tf / MFMA_F16_PEAK_TFLOPS, "traffic": ADAM_TRAFFIC_BYTES_PER_LAYER,
+                         "kernel": "bgx::adam_fused_direct_kernel<bf16_t>"},
             "modules": modules}
 
 
@@ -482,6 +488,9 @@ def main():
         sys.exit(1)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    import datasets
+
+    datasets.disable_progress_bars()  # the loop's teardown saves a dataset; keep stderr to what this script says
 
     if args.copy_calibration:
         src = torch.ones(1 << 28, dtype=torch.float32, device=device)

@@ -620,6 +620,36 @@ def test_adam_fused_xcd_order(device, ttx, bgx_env):
     assert rel_l2(got, want) <= TOL[torch.bfloat16]
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(2, 700, 256, 512, 32), (1, 1024, 1024, 1024, 32), (3, 300, 192, 768, 16)])
+def test_adam_direct_tiles_against_register_staged_kernel(device, dtype, shape, bgx_env):
+    """The fused Adam kernel whose operands all travel through LDS tiles loaded directly from global memory, on
+    shapes with several K tiles, several chunks of output features and ragged lengths: per-token rows against
+    the oracle where it is quick, and against the register-staged fused kernel (BGX_ADAM_DIRECT_OFF) everywhere."""
+    N, S, I, O, p = shape
+    case = _adam_case(N, S, I, O, p, dtype, seed=83)
+    a, g, left, right, norm = case
+    # second moments bounded away from zero: the table entries R / sqrt(v) stay inside fp16's range
+    norm = ohooks.Adam(weight_avg_sq=norm.weight_avg_sq * 100 + 1e-6)
+    lengths = [S, max(2, S // 3), max(2, S - 41)][:N]
+    g = g.clone()
+    for n, l in enumerate(lengths):
+        g[n, l - 1:] = 0
+    case = (a, g, left, right, norm)
+    counts = [l - 1 for l in lengths]
+    offs = [sum(counts[:n]) for n in range(N)]
+    kw = dict(per_token=True, lengths=lengths, row_offsets=offs, n_rows=sum(counts))
+    got = _run_adam(device, case, p, dtype, **kw)
+    bgx_env("BGX_ADAM_DIRECT_OFF", "1")
+    staged = _run_adam(device, case, p, dtype, **kw)
+    assert rel_l2(got, staged) <= TOL[dtype]
+    assert bool(torch.isfinite(got.float()).all())
+    if I * O <= 256 * 768:
+        mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+        want = ohooks.module_gradient(a, g, norm, left, right, attribute_tokens=True, collection_mask=mask)
+        assert rel_l2(got, want) <= TOL[dtype]
+
+
 def test_adam_seq_many_short_sequences(device):
     """Many short sequences of a fused-eligible shape: the per-sequence rows come from the per-token kernel."""
     N, S, I, O, p = 40, 24, 128, 256, 16
