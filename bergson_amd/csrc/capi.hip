@@ -90,6 +90,11 @@ int fullgrad_tok_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
                       const float* col_scale, const float* adam_v, int collect_bias, const float* bias_scale,
                       const int32_t* lengths, const int64_t* row_offsets, void* out, int64_t out_row_stride,
                       int64_t out_col, int out_dtype, float lo, float hi, void* stream);
+int fullgrad_seq_gemm_impl(const void* a, const void* g, int64_t a_seq_stride, int64_t a_tok_stride,
+                           int64_t g_seq_stride, int64_t g_tok_stride, int N, int S, int I, int O, int dtype,
+                           const float* row_scale, const float* col_scale, const float* adam_v, int collect_bias,
+                           const float* bias_scale, const int32_t* lengths, const int64_t* out_rows, void* out,
+                           int64_t out_row_stride, int64_t out_col, int out_dtype, float lo, float hi, void* stream);
 int collect_timing_enable(int max_launches);
 int collect_timing_read(float* ms_out, int capacity, int* count_out);
 int unit_normalize_impl(void* rows, int64_t n_rows, int64_t D, int64_t stride, int dtype, void* stream);
@@ -223,6 +228,19 @@ int bgx_fullgrad_tok(const void* a_dev, const void* g_dev, int64_t a_seq_stride,
                                 row_scale_dev, col_scale_dev, adam_v_dev, collect_bias, bias_scale_dev, lengths_dev,
                                 row_offsets_dev, out_dev, out_row_stride, out_col, out_dtype, clamp_lo, clamp_hi,
                                 stream);
+}
+
+int bgx_fullgrad_seq_gemm(const void* a_dev, const void* g_dev, int64_t a_seq_stride, int64_t a_tok_stride,
+                          int64_t g_seq_stride, int64_t g_tok_stride, int32_t N, int32_t S, int32_t I, int32_t O,
+                          int32_t dtype, const float* row_scale_dev, const float* col_scale_dev,
+                          const float* adam_v_dev, int32_t collect_bias, const float* bias_scale_dev,
+                          const int32_t* lengths_dev, const int64_t* out_rows_dev, void* out_dev,
+                          int64_t out_row_stride, int64_t out_col, int32_t out_dtype, float clamp_lo, float clamp_hi,
+                          void* stream) {
+  return bgx::fullgrad_seq_gemm_impl(a_dev, g_dev, a_seq_stride, a_tok_stride, g_seq_stride, g_tok_stride, N, S, I, O,
+                                     dtype, row_scale_dev, col_scale_dev, adam_v_dev, collect_bias, bias_scale_dev,
+                                     lengths_dev, out_rows_dev, out_dev, out_row_stride, out_col, out_dtype, clamp_lo,
+                                     clamp_hi, stream);
 }
 
 int bgx_collect_timing_enable(int32_t max_launches) { return bgx::collect_timing_enable(max_launches); }

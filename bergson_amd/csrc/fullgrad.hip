@@ -12,6 +12,7 @@
 #include <algorithm>
 
 #include "common.hpp"
+#include "mma32.hpp"
 
 namespace bgx {
 
@@ -122,6 +123,243 @@ __global__ __launch_bounds__(256) void fullgrad_tok_kernel(FullArgs a, const voi
   }
 }
 
+// ---- per-sequence gradient with the GEMM over tokens fused ---------------------------------------------------
+// out[row(n), out_col + o * Iw + i] = clamp(normalise(sum_s g[n, s, o] * a[n, s, i])) in one kernel: the
+// reference's `g.mT @ a` (collector.py:623, :684, :735) and everything after it.  Both operands are stored token
+// by token, i.e. with the contraction index as the slow one, which is the wrong way round for the MFMA operands (a
+// lane wants 8 consecutive tokens of one feature).  Tiles of BK tokens x 64 features go to LDS as they are; for
+// 16-bit types the fragments come out of LDS through the transposing read ds_read_b64_tr_b16: within each group of
+// 16 lanes, lane 4 q + c receives, as element e, element c of what lane q + 4 e of the group read.  A lane that
+// reads 4 consecutive features at (token k0 + s / 4, feature m0 + 4 (s % 4)), s = its place in the group, therefore
+// ends up with 4 consecutive tokens of feature m0 + s; two such reads are a K = 8 half of a 32 x 32 x 16 operand.
+// fp32 operands use the 32 x 32 x 2 MFMA, whose operands are one value per lane and need no transposition.
+// A workgroup of four waves (2 x 2 blocks of 32 x 32) owns 64 x 64 of one sequence's [O, I] -- small tiles, so that
+// the few-sequence batches of small modules still spread over the chip and several workgroups share a CU; the K
+// loop runs over the sequence's tokens (those below lengths[n] - 1 when lengths are given), two LDS stages, global
+// loads of the next stage in flight during the MFMAs.  The results leave through LDS so that a lane stores 8
+// consecutive values.  Rounding points are those of the two-step path: the sum is rounded to the model dtype (the
+// GEMM's output), normalised, rounded again, clamped, cast.
+struct WgradIn {
+  const void* act;
+  const void* g;
+  int64_t a_seq_stride, a_tok_stride, g_seq_stride, g_tok_stride;
+  int S;
+  const int32_t* lengths;   // NULL: all S tokens
+  const int64_t* out_rows;  // NULL: row n
+  int aligned;              // whole 16-byte pieces of both operands can be loaded at once
+  int tiles_i;
+};
+
+constexpr int WG_BT = 64;            // tile edge
+constexpr int WG_OUT_PITCH = 68;     // floats per row of the staged result tile
+
+template <typename T>
+struct WgradTile {
+  static constexpr bool F32 = sizeof(T) == 4;
+  static constexpr int BK = F32 ? 32 : 64;               // tokens per stage
+  static constexpr int VEC = 16 / (int)sizeof(T);        // elements per 16-byte piece
+  static constexpr int PITCH = WG_BT * (int)sizeof(T);   // bytes per token row of a tile
+  static constexpr int OPERAND = BK * PITCH;             // 8 KB
+  static constexpr int STAGE = 2 * OPERAND;              // g tile, then a tile
+  static constexpr int NCH = BK * (WG_BT / VEC) / 256;   // 16-byte pieces per thread, operand and stage
+  // byte offset of element (token k, feature c) inside an operand tile.  16-bit: the two 64-byte halves of a row
+  // swap on every second pair of token rows, so that the four rows a transposing read touches fall into different
+  // banks; fp32: odd token rows are shifted by half the banks, for the two rows a K = 2 operand reads.
+  __device__ static int off(int k, int c) {
+    if constexpr (F32) {
+      return k * PITCH + ((c ^ ((k & 1) << 5)) << 2);
+    } else {
+      const int b = c * 2;
+      return k * PITCH + (((b >> 6) ^ ((k >> 1) & 1)) << 6) + (b & 63);
+    }
+  }
+};
+
+typedef short s16x4 __attribute__((__vector_size__(4 * sizeof(short))));
+
+__device__ inline uint2 lds_read_tr16(const unsigned char* p) {
+  typedef __attribute__((address_space(3))) s16x4* lds_ptr;
+  const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(uintptr_t)(uint32_t)(uintptr_t)p);
+  return __builtin_bit_cast(uint2, v);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void wgrad_seq_kernel(FullArgs a, WgradIn in) {
+  using L = WgradTile<T>;
+  constexpr int BT = WG_BT, BK = L::BK, VEC = L::VEC, NCH = L::NCH;
+  constexpr int CPR = BT / VEC;  // 16-byte pieces per tile row
+  static_assert(2 * L::STAGE >= BT * WG_OUT_PITCH * 4, "the staged result tile reuses the operand stages");
+  __shared__ __align__(16) unsigned char smem[2 * L::STAGE];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int fr = lane & 31, fh = lane >> 5;
+  const int n = blockIdx.y;
+  const int o0 = (blockIdx.x / in.tiles_i) * BT, i0 = (blockIdx.x % in.tiles_i) * BT;
+  int Sn = in.S;
+  if (in.lengths != nullptr) Sn = max(0, min(in.S, in.lengths[n] - 1));
+  const int KT = (Sn + BK - 1) / BK;
+  const bool with_bias = a.Iw > a.I && i0 == 0;
+
+  const T* gp = (const T*)in.g + (int64_t)n * in.g_seq_stride;
+  const T* ap = (const T*)in.act + (int64_t)n * in.a_seq_stride;
+
+  // ---- loader: piece c of a stage is 16 bytes of token row c / CPR
+  uint4 gv[NCH], av[NCH];
+  auto fetch = [&](const T* base, int64_t tok_stride, int width, int col0, int kt, int j) -> uint4 {
+    const int c = tid + 256 * j;
+    const int k = c / CPR, col = col0 + (c % CPR) * VEC;
+    const int s = kt * BK + k;
+    uint4 v = make_uint4(0u, 0u, 0u, 0u);
+    if (s < Sn && col < width) {
+      const T* src = base + (int64_t)s * tok_stride + col;
+      if (in.aligned && col + VEC <= width) {
+        v = load16_global(src);
+      } else {
+        struct {
+          T e[VEC];
+        } tmp;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) tmp.e[e] = col + e < width ? src[e] : T{};
+        v = __builtin_bit_cast(uint4, tmp);
+      }
+    }
+    return v;
+  };
+  auto load_stage = [&](int kt) {
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      gv[j] = fetch(gp, in.g_tok_stride, a.O, o0, kt, j);
+      av[j] = fetch(ap, in.a_tok_stride, a.I, i0, kt, j);
+    }
+  };
+  auto store_stage = [&](int st) {
+    unsigned char* base = smem + st * L::STAGE;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const int c = tid + 256 * j;
+      const int off = L::off(c / CPR, (c % CPR) * VEC);
+      *reinterpret_cast<uint4*>(base + off) = gv[j];
+      *reinterpret_cast<uint4*>(base + L::OPERAND + off) = av[j];
+    }
+  };
+
+  f32x16 acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+  float bias_part = 0.f;
+  constexpr int PARTS = 256 / BT;  // threads per output feature for the bias sum
+  const int b_col = tid % BT, b_part = tid / BT;
+
+  auto compute = [&](int st) {
+    const unsigned char* gt = smem + st * L::STAGE;
+    const unsigned char* at = gt + L::OPERAND;
+    if constexpr (L::F32) {
+#pragma unroll
+      for (int kk = 0; kk < BK; kk += 2) {
+        const float af = *reinterpret_cast<const float*>(gt + L::off(kk + fh, wm * 32 + fr));
+        const float bf = *reinterpret_cast<const float*>(at + L::off(kk + fh, wn * 32 + fr));
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af, bf, acc, 0, 0, 0);
+      }
+    } else {
+      // place of this lane's read: token (lane % 16) / 4 of its K = 4 group, features 4 (lane % 4) .. + 3 of the 16
+      // its group of lanes covers
+      const int rk = 8 * fh + ((lane & 15) >> 2);
+      const int rc = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+#pragma unroll
+      for (int ks = 0; ks < BK; ks += 16) {
+        const uint2 g0 = lds_read_tr16(gt + L::off(ks + rk, wm * 32 + rc));
+        const uint2 g1 = lds_read_tr16(gt + L::off(ks + rk + 4, wm * 32 + rc));
+        const uint2 a0 = lds_read_tr16(at + L::off(ks + rk, wn * 32 + rc));
+        const uint2 a1 = lds_read_tr16(at + L::off(ks + rk + 4, wn * 32 + rc));
+        Mma32<T>::mma(make_uint4(g0.x, g0.y, g1.x, g1.y), make_uint4(a0.x, a0.y, a1.x, a1.y), acc);
+      }
+    }
+    if (with_bias) {
+      for (int k = b_part; k < BK; k += PARTS)
+        bias_part += Elem<T>::load(reinterpret_cast<const T*>(gt + L::off(k, b_col)));
+    }
+  };
+
+  if (KT > 0) {
+    load_stage(0);
+    store_stage(0);
+  }
+  __syncthreads();
+  for (int kt = 0; kt < KT; ++kt) {
+    if (kt + 1 < KT) load_stage(kt + 1);
+    compute(kt & 1);
+    if (kt + 1 < KT) store_stage((kt + 1) & 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: normalise in place, stage the tile in LDS (the operand stages are done with: the loop ends on a
+  // barrier), then every lane stores 8 consecutive values of a row
+  const int64_t row = in.out_rows ? in.out_rows[n] : (int64_t)n;
+  const int64_t dst0 = row * a.out_row_stride + a.out_col;
+  float* tile = reinterpret_cast<float*>(smem);
+  {
+    // acc[e] = sum for output feature o0 + 32 wm + 8 (e / 4) + 4 fh + e % 4, input feature i0 + 32 wn + fr
+    const int il = wn * 32 + fr, i = i0 + il;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int ol = wm * 32 + 8 * (e >> 2) + 4 * fh + (e & 3), o = o0 + ol;
+      float v = 0.f;
+      if (o < a.O && i < a.I) {
+        v = round_to_dtype(acc[e], a.dtype);
+        v = clampf(round_to_dtype(normalise_weight(a, v, o, i), a.dtype), a.lo, a.hi);
+      }
+      tile[ol * WG_OUT_PITCH + il] = v;
+    }
+  }
+  float bias_total = 0.f;
+  if (with_bias) {
+    // the bias sums take the rows of the tile array behind the tile itself
+    float* red = tile + BT * WG_OUT_PITCH;
+    static_assert(2 * L::STAGE >= (BT * WG_OUT_PITCH + 256) * 4, "room for the bias partial sums");
+    red[b_part * BT + b_col] = bias_part;
+  }
+  __syncthreads();
+  const int es = (int)dtype_size(a.out_dtype);
+  // rows of the tile start on 16-byte boundaries of the output when the row pitch and the tile's first element do
+  const bool rows_aligned = ((uintptr_t)a.out + (uintptr_t)(dst0 + (int64_t)o0 * a.Iw + i0) * es) % 16 == 0 &&
+                            ((int64_t)a.Iw * es) % 16 == 0;
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int piece = tid + 256 * q;
+    const int ol = piece >> 3, il = (piece & 7) * 8;
+    const int o = o0 + ol, i = i0 + il;
+    if (o >= a.O || i >= a.I) continue;
+    float v[8];
+    const f32x4 lo4 = *reinterpret_cast<const f32x4*>(tile + ol * WG_OUT_PITCH + il);
+    const f32x4 hi4 = *reinterpret_cast<const f32x4*>(tile + ol * WG_OUT_PITCH + il + 4);
+    v[0] = lo4[0], v[1] = lo4[1], v[2] = lo4[2], v[3] = lo4[3];
+    v[4] = hi4[0], v[5] = hi4[1], v[6] = hi4[2], v[7] = hi4[3];
+    const int64_t dst = dst0 + (int64_t)o * a.Iw + i;
+    if (rows_aligned && i + 8 <= a.I) {
+      if (a.out_dtype == BGX_F32)
+        store8_as<BGX_F32>(a.out, dst, v);
+      else if (a.out_dtype == BGX_F16)
+        store8_as<BGX_F16>(a.out, dst, v);
+      else
+        store8_as<BGX_BF16>(a.out, dst, v);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (i + e < a.I) store_as(a.out, dst + e, v[e], a.out_dtype);
+    }
+  }
+  if (with_bias && b_part == 0 && o0 + b_col < a.O) {
+    const float* red = tile + BT * WG_OUT_PITCH;
+#pragma unroll
+    for (int q = 0; q < PARTS; ++q) bias_total += red[q * BT + b_col];
+    const int o = o0 + b_col;
+    if (a.bias_scale != nullptr) bias_total *= a.bias_scale[o];
+    bias_total = round_to_dtype(bias_total, a.dtype);
+    store_as(a.out, dst0 + (int64_t)o * a.Iw + a.I, clampf(bias_total, a.lo, a.hi), a.out_dtype);
+  }
+}
+
 static bool dtype_ok(int dt) { return dt >= BGX_F32 && dt <= BGX_BF16; }
 
 int token_sum_impl(const void* g, int64_t g_seq_stride, int64_t g_tok_stride, int N, int S, int O, int dtype,
@@ -177,6 +415,56 @@ int fullgrad_seq_impl(const void* P, int N, int O, int I, int dtype, const float
   const unsigned gx = (unsigned)std::min<int64_t>((per_seq + 1023) / 1024, 4096);
   hipLaunchKernelGGL(fullgrad_seq_kernel, dim3(gx, (unsigned)N), dim3(256), 0, (hipStream_t)stream, fa, P, bias_sum,
                      out_rows);
+  BGX_HIP(hipGetLastError());
+  return 0;
+}
+
+template <typename T>
+static void launch_wgrad(const FullArgs& fa, WgradIn in, int N, hipStream_t st) {
+  in.tiles_i = (fa.I + WG_BT - 1) / WG_BT;
+  const unsigned tiles = (unsigned)(((fa.O + WG_BT - 1) / WG_BT) * in.tiles_i);
+  hipLaunchKernelGGL(wgrad_seq_kernel<T>, dim3(tiles, (unsigned)N), dim3(256), 0, st, fa, in);
+}
+
+int fullgrad_seq_gemm_impl(const void* a, const void* g, int64_t a_seq_stride, int64_t a_tok_stride,
+                           int64_t g_seq_stride, int64_t g_tok_stride, int N, int S, int I, int O, int dtype,
+                           const float* row_scale, const float* col_scale, const float* adam_v, int collect_bias,
+                           const float* bias_scale, const int32_t* lengths, const int64_t* out_rows, void* out,
+                           int64_t out_row_stride, int64_t out_col, int out_dtype, float lo, float hi, void* stream) {
+  BGX_REQUIRE(a && g, BGX_E_ARG, "fullgrad_seq_gemm: null pointer");
+  BGX_REQUIRE(N > 0 && S > 0 && N <= 65535, BGX_E_SHAPE, "fullgrad_seq_gemm: N=%d S=%d", N, S);
+  BGX_REQUIRE(a_tok_stride >= I && g_tok_stride >= O && a_seq_stride >= 0 && g_seq_stride >= 0, BGX_E_ARG,
+              "fullgrad_seq_gemm: strides a (%lld, %lld) g (%lld, %lld)", (long long)a_seq_stride,
+              (long long)a_tok_stride, (long long)g_seq_stride, (long long)g_tok_stride);
+  FullArgs fa;
+  const int rc = fill_args(fa, "fullgrad_seq_gemm", O, I, dtype, row_scale, col_scale, adam_v, collect_bias,
+                           bias_scale, out, out_row_stride, out_col, out_dtype, lo, hi);
+  if (rc != 0) return rc;
+  BGX_REQUIRE(((int64_t)((O + 63) / 64)) * ((I + 63) / 64) <= 0x7fffffff, BGX_E_SHAPE,
+              "fullgrad_seq_gemm: O=%d I=%d", O, I);
+  WgradIn in;
+  in.act = a;
+  in.g = g;
+  in.a_seq_stride = a_seq_stride;
+  in.a_tok_stride = a_tok_stride;
+  in.g_seq_stride = g_seq_stride;
+  in.g_tok_stride = g_tok_stride;
+  in.S = S;
+  in.lengths = lengths;
+  in.out_rows = out_rows;
+  const int64_t es = (int64_t)dtype_size(dtype);
+  auto whole = [&](const void* p, int64_t s0, int64_t s1) {
+    return ((uintptr_t)p % 16 == 0) && (s0 * es) % 16 == 0 && (s1 * es) % 16 == 0;
+  };
+  in.aligned = whole(a, a_seq_stride, a_tok_stride) && whole(g, g_seq_stride, g_tok_stride);
+  in.tiles_i = 0;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == BGX_F32)
+    launch_wgrad<float>(fa, in, N, st);
+  else if (dtype == BGX_F16)
+    launch_wgrad<f16_t>(fa, in, N, st);
+  else
+    launch_wgrad<bf16_t>(fa, in, N, st);
   BGX_HIP(hipGetLastError());
   return 0;
 }

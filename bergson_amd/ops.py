@@ -433,8 +433,9 @@ def full_gradient(mod: FullGradModule, a: Tensor, g: Tensor, out: Tensor, *, per
                   lengths: Tensor | None, rows: Tensor | None, lo: float, hi: float) -> None:
     """Weight-shaped gradient of one module written to its columns of `out` (see bgx_fullgrad_seq / _tok).
 
-    per_token=False: out[rows[n] (or n)] gets flatten(normalise(g[n]^T a[n])) -- the batched GEMM runs on
-    the BLAS, as the reference's `g.mT @ a` does; per_token=True: out[rows[n] + s] gets
+    per_token=False: out[rows[n] (or n)] gets flatten(normalise(g[n]^T a[n])), the sum running over the
+    tokens s < lengths[n] - 1 when lengths are given (all of them otherwise) -- one kernel, GEMM on the matrix
+    cores with the normalisation behind it; per_token=True: out[rows[n] + s] gets
     flatten(normalise(g[n, s] (x) a[n, s])) for s < lengths[n] - 1.
     """
     lib = _lib.load()
@@ -462,35 +463,27 @@ def full_gradient(mod: FullGradModule, a: Tensor, g: Tensor, out: Tensor, *, per
                                   mod.out_col, dtype_code(out.dtype), lo, hi, _stream())
         _lib.check(rc, "bgx_fullgrad_tok")
         return
-    P = torch.bmm(g.transpose(1, 2), a)  # [N, O, I], the plain library GEMM of the path
-    bias_sum = None
-    if mod.collect_bias:
-        bias_sum = torch.empty((N, O), dtype=torch.float32, device=g.device)
-        rc = lib.bgx_token_sum(_ptr(g), g.stride(0), g.stride(1), N, S, O, code, _ptr(bias_sum), _stream())
-        _lib.check(rc, "bgx_token_sum")
-    rc = lib.bgx_fullgrad_seq(_ptr(P), N, O, I, code, _ptr(mod.row_scale), _ptr(mod.col_scale), _ptr(mod.adam_v),
-                              _ptr(bias_sum), _ptr(mod.bias_scale), _ptr(rows), _ptr(out), out.stride(0), mod.out_col,
-                              dtype_code(out.dtype), lo, hi, _stream())
-    _lib.check(rc, "bgx_fullgrad_seq")
+    rc = lib.bgx_fullgrad_seq_gemm(_ptr(a), _ptr(g), a.stride(0), a.stride(1), g.stride(0), g.stride(1), N, S, I, O,
+                                   code, _ptr(mod.row_scale), _ptr(mod.col_scale), _ptr(mod.adam_v),
+                                   int(mod.collect_bias), _ptr(mod.bias_scale), _ptr(lengths), _ptr(rows), _ptr(out),
+                                   out.stride(0), mod.out_col, dtype_code(out.dtype), lo, hi, _stream())
+    _lib.check(rc, "bgx_fullgrad_seq_gemm")
 
 
 def _collect_adam_seq(prep: AdamPrepared, a: Tensor, g: Tensor, out: Tensor, lengths: Tensor | None,
                       rows: Tensor | None, lo: float, hi: float) -> None:
     """Per-sequence Adam without anything per token: the normalisation is applied to the summed gradient, as
     the reference does (collector.py:634-644):
-        Q[n] = (g[n]^T a[n]) / (sqrt(v) + 1e-8)  [| bias column]     batched GEMM + bgx_fullgrad_seq
+        Q[n] = (g[n]^T a[n]) / (sqrt(v) + 1e-8)  [| bias column]     bgx_fullgrad_seq_gemm
         P[n] = L Q[n] R^T                                            bgx_collect_seq with the output features
     in the role of tokens: "a" = Q[n] ([O, I(+1)] rows), projected by R; "g" = L^T ([O, p], shared by all n,
     sequence stride 0) with an identity projection; the token reduction is the sum over output features.
     """
     N, S, _ = a.shape
     full, r_in, lt, eye = prep.seq_state()
-    if lengths is not None:
-        # positions from len-1 on carry no label; zero them instead of relying on the model's zeros
-        keep = (torch.arange(S, device=g.device).unsqueeze(0) + 1 < lengths.unsqueeze(1)).unsqueeze(-1)
-        g = g * keep
     q = torch.empty((N, full.width), dtype=prep.dtype, device=a.device)
-    full_gradient(full, a, g, q, per_token=False, lengths=None, rows=None, lo=float("-inf"), hi=float("inf"))
+    # positions from len-1 on carry no label: the kernel leaves them out of the sum
+    full_gradient(full, a, g, q, per_token=False, lengths=lengths, rows=None, lo=float("-inf"), hi=float("inf"))
     Iw = full.width // prep.O
     m = ModuleInput(a=q.view(N, prep.O, Iw), g=lt.unsqueeze(0).expand(N, prep.O, prep.p), r_in=r_in, r_out=eye,
                     out_col=prep.out_col)

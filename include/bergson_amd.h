@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define BGX_ABI_VERSION 7
+#define BGX_ABI_VERSION 8
 
 enum bgx_dtype { BGX_F32 = 0, BGX_F16 = 1, BGX_BF16 = 2 };
 
@@ -236,6 +236,14 @@ int bgx_collect_adam(const void* a_dev, const void* g_dev,
  *   :684, :735).  Writes out[row(n), out_col + o*(I+b) + i] =
  *   cast(clamp(normalise(P[n, o, i]))), row(n) = out_rows[n] (n when NULL);
  *   bias_sum_dev [N, O] non-NULL adds the bias column (b = 1).
+ * bgx_fullgrad_seq_gemm: the same rows straight from a [N, S, I] and
+ *   g [N, S, O] (strides in elements, innermost contiguous): the GEMM over the
+ *   tokens of a sequence (`g.mT @ a`, collector.py:623, :684, :735; only
+ *   tokens s < lengths[n] - 1 when lengths_dev is given) on the matrix cores
+ *   with normalisation, bias column (collect_bias != 0: sum_s g[n, s, o] *
+ *   bias_scale[o]), clamp, cast and scatter fused behind it, so the [N, O, I]
+ *   product never reaches memory.  Same rounding points as BLAS GEMM +
+ *   bgx_fullgrad_seq: the sum is rounded to `dtype` before it is normalised.
  * bgx_fullgrad_tok: per token s < lengths[n] - 1 writes row
  *   row_offsets[n] + s with out_col + o*(I+b) + i = normalise(g[o] * a[i])
  *   (collector.py:620-632, :668-683, :730-734), bias column g[o] *
@@ -251,6 +259,18 @@ int bgx_fullgrad_seq(const void* P_dev, int32_t N, int32_t O, int32_t I,
                      int64_t out_row_stride, int64_t out_col,
                      int32_t out_dtype, float clamp_lo, float clamp_hi,
                      void* stream);
+int bgx_fullgrad_seq_gemm(const void* a_dev, const void* g_dev,
+                          int64_t a_seq_stride, int64_t a_tok_stride,
+                          int64_t g_seq_stride, int64_t g_tok_stride,
+                          int32_t N, int32_t S, int32_t I, int32_t O,
+                          int32_t dtype, const float* row_scale_dev,
+                          const float* col_scale_dev, const float* adam_v_dev,
+                          int32_t collect_bias, const float* bias_scale_dev,
+                          const int32_t* lengths_dev,
+                          const int64_t* out_rows_dev, void* out_dev,
+                          int64_t out_row_stride, int64_t out_col,
+                          int32_t out_dtype, float clamp_lo, float clamp_hi,
+                          void* stream);
 int bgx_fullgrad_tok(const void* a_dev, const void* g_dev,
                      int64_t a_seq_stride, int64_t a_tok_stride,
                      int64_t g_seq_stride, int64_t g_tok_stride, int32_t N,

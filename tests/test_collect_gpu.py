@@ -524,6 +524,94 @@ def test_fullgrad_seq(device, dtype, kind, bias):
     assert got[:, :7].abs().sum() == 0 and got[[1, 3]].abs().sum() == 0
 
 
+def _wgrad_reference(a, g, lengths):
+    """sum_s g[n, s, :] (x) a[n, s, :] over the tokens s < lengths[n] - 1, in float64."""
+    a64, g64 = a.double(), g.double().clone()
+    if lengths is not None:
+        for n, l in enumerate(lengths):
+            g64[n, max(l - 1, 0):] = 0
+    return torch.einsum("nso,nsi->noi", g64, a64)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [
+    (3, 37, 24, 40),       # one ragged 64-wide tile, tokens not a multiple of a stage
+    (2, 130, 200, 136),    # several 64-wide tiles with ragged edges
+    (3, 96, 1024, 1024),   # 128-wide tiles (64 tiles x 3 sequences)
+    (1, 70, 70, 61),       # odd widths: pieces of 16 bytes cannot be loaded whole
+    (4, 1, 64, 64),        # a single token
+])
+def test_fullgrad_seq_gemm_against_float64(device, dtype, shape):
+    """The fused GEMM-over-tokens kernel alone (no normaliser): every tile variant and edge against the float64
+    contraction, with lengths that cut sequences short (one of them to nothing) and scattered output rows."""
+    from bergson_amd import ops
+
+    N, S, I, O = shape
+    gen = torch.Generator().manual_seed(91)
+    a = torch.randn(N, S, I, generator=gen).to(dtype)
+    g = (torch.randn(N, S, O, generator=gen) * 0.1).to(dtype)
+    lengths = [S + 1, max(1, S // 2), 1, S][:N]
+    want = _wgrad_reference(a, g, lengths).reshape(N, O * I)
+    out = torch.full((N + 1, 3 + O * I), 7.0, dtype=torch.float32, device=device)
+    rows = torch.tensor(list(range(N, 0, -1)), dtype=torch.int64, device=device)
+    mod = ops.FullGradModule(O=O, I=I, out_col=3)
+    ops.full_gradient(mod, a.to(device), g.to(device), out, per_token=False,
+                      lengths=torch.tensor(lengths, dtype=torch.int32, device=device), rows=rows, lo=-3e38, hi=3e38)
+    torch.cuda.synchronize()
+    got = out.cpu()
+    assert bool((got[0] == 7).all()) and bool((got[:, :3] == 7).all())
+    assert rel_l2(got[list(range(N, 0, -1)), 3:].double(), want) <= TOL[dtype]
+    if N >= 3:
+        assert got[N - 2, 3:].abs().sum() == 0  # the sequence of length 1 has no labelled token
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_fullgrad_seq_gemm_strided_operands(device, dtype):
+    """Operands that are views: token rows wider than the features used, sequences far apart, and a g whose first
+    element is not 16-byte aligned (the element-wise loader)."""
+    from bergson_amd import ops
+
+    N, S, I, O = 2, 45, 72, 88
+    gen = torch.Generator().manual_seed(92)
+    a_big = torch.randn(N, S + 3, I + 24, generator=gen).to(dtype).to(device)
+    g_big = (torch.randn(N, S, O + 9, generator=gen) * 0.1).to(dtype).to(device)
+    a = a_big[:, 1:S + 1, 8:8 + I]
+    g = g_big[:, :, 3:3 + O]
+    want = _wgrad_reference(a.cpu(), g.cpu(), None).reshape(N, O * I)
+    out = torch.zeros(N, O * I, dtype=torch.float32, device=device)
+    ops.full_gradient(ops.FullGradModule(O=O, I=I, out_col=0), a, g, out, per_token=False, lengths=None, rows=None,
+                      lo=-3e38, hi=3e38)
+    torch.cuda.synchronize()
+    assert rel_l2(out.cpu().double(), want) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("kind", [None, "adafactor", "adam"])
+def test_fullgrad_two_step_entries_agree_with_fused(device, kind):
+    """bgx_token_sum + bgx_fullgrad_seq behind a caller's own GEMM (the entries a C caller with its own BLAS uses)
+    give the rows of the fused entry: same rounding points, sums in another order."""
+    from bergson_amd import _lib, ops
+    from bergson_amd.ops import _ptr, _stream, dtype_code
+
+    N, S, I, O = 3, 64, 96, 80
+    dtype = torch.bfloat16
+    a, g, norm = _full_case(N, S, I, O, dtype, kind, True, seed=93)
+    mod = _full_module(device, a, g, norm, True, 0)
+    a, g = a.to(device), g.to(device)
+    fused = torch.zeros(N, mod.width, dtype=dtype, device=device)
+    ops.full_gradient(mod, a, g, fused, per_token=False, lengths=None, rows=None, lo=-3e38, hi=3e38)
+    lib = _lib.load()
+    P = torch.einsum("nso,nsi->noi", g.float(), a.float()).to(dtype).contiguous()
+    bias_sum = torch.empty(N, O, dtype=torch.float32, device=device)
+    code = dtype_code(dtype)
+    _lib.check(lib.bgx_token_sum(_ptr(g), g.stride(0), g.stride(1), N, S, O, code, _ptr(bias_sum), _stream()), "sum")
+    two = torch.zeros_like(fused)
+    _lib.check(lib.bgx_fullgrad_seq(_ptr(P), N, O, I, code, _ptr(mod.row_scale), _ptr(mod.col_scale),
+                                    _ptr(mod.adam_v), _ptr(bias_sum), _ptr(mod.bias_scale), None, _ptr(two),
+                                    two.stride(0), 0, code, -3e38, 3e38, _stream()), "fullgrad_seq")
+    torch.cuda.synchronize()
+    assert rel_l2(fused.cpu(), two.cpu()) <= 4e-3
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("kind", [None, "adafactor", "adam"])
 @pytest.mark.parametrize("bias", [False, True])
