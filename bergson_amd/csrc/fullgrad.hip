@@ -3,9 +3,10 @@
 // Reference: bergson/collector/collector.py:609-644 (Adam), :646-700 (Adafactor), :701-742 (no
 // normaliser) with p = None; bergson/gradients.py:300-349, :380-400 (normalisers).
 //
-// Per sequence the gradient g^T a [O, I] is a plain batched GEMM that the caller runs with its BLAS
-// (the reference's `g.mT @ a`); fullgrad_seq_kernel is everything after it: normalisation, the bias
-// column, clamp to the store dtype's range, cast, and the scatter into the rows of the store.
+// Per sequence the gradient is g^T a [O, I] (the reference's `g.mT @ a`): wgrad_seq_kernel runs that GEMM
+// over the tokens and everything after it -- normalisation, the bias column, clamp to the store dtype's
+// range, cast, and the scatter into the rows of the store.  fullgrad_seq_kernel is the second half alone,
+// for a caller that has formed the product with a GEMM of its own.
 // Per token the gradient is the outer product g_t (x) a_t; fullgrad_tok_kernel forms it, normalises it
 // and writes it straight to the token's row.  Both are bound by the bytes they write.
 
