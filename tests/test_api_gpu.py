@@ -316,6 +316,47 @@ def test_attributor_full_ranking_beyond_the_fused_top_k(device, tmp_path):
     assert all(sorted(r.tolist()) == list(range(n)) for r in idx.cpu())
 
 
+@pytest.mark.parametrize("store_dtype", ["bfloat16", "float16"])
+def test_attributor_on_16_bit_stores_against_fp32_search(device, tmp_path, store_dtype):
+    """The reference scores a 16-bit store in fp32 against fp32 queries (attributor.py:137-167, dtype default);
+    here the scan multiplies the store by queries rounded to the store dtype, so a score can be off by
+    2^-9 |g||q| (bf16) or 2^-12 |g||q| (fp16) in the worst case and by 1 / sqrt(D) of that typically.
+    Pinned with an explicit tolerance: values within 2e-3 / 1e-3 of the fp32 search over the same stored
+    values, planted self-matches first, and every reported row scoring within that tolerance of the k-th
+    best fp32 score."""
+    from bergson_amd import Attributor, GradientProcessor
+    from bergson_amd.data import create_index
+    from bergson_amd.utils import tensor_to_numpy
+
+    n, sizes, k = 3000, {"a": 96, "b": 160}, 50
+    tdt = torch.bfloat16 if store_dtype == "bfloat16" else torch.float16
+    tol = 2e-3 if store_dtype == "bfloat16" else 1e-3
+    gen = torch.Generator().manual_seed(21)
+    rows = torch.randn(n, 256, generator=gen).to(tdt)
+    path = tmp_path / store_dtype
+    mm = create_index(path, n, sizes, store_dtype)
+    mm[:] = tensor_to_numpy(rows)
+    mm.flush()
+    GradientProcessor(projection_dim=None).save(path)
+    attr = Attributor(path, device="cuda:0", unit_norm=True)
+    q = torch.randn(6, 256, generator=gen)
+    q[:2] = rows[[11, 2222]].float() + 0.01 * torch.randn(2, 256, generator=gen)
+    vals, idx = attr.search({"a": q[:, :96].to(device), "b": q[:, 96:].to(device)}, k=k)
+    stored = rows.float()
+    index = {"a": stored[:, :96], "b": stored[:, 96:]}
+    ref_v, ref_i = oscan.attributor_search(index, {"a": q[:, :96], "b": q[:, 96:]}, ["a", "b"], k, unit_norm=True)
+    assert idx[:2, 0].tolist() == [11, 2222]
+    assert (vals.cpu() - ref_v).abs().max().item() <= tol
+    # the fp32 score of every reported row reaches the k-th best fp32 score up to the tolerance
+    full_v, _ = oscan.attributor_search(index, {"a": q[:, :96], "b": q[:, 96:]}, ["a", "b"], n, unit_norm=True)
+    _, order = oscan.attributor_search(index, {"a": q[:, :96], "b": q[:, 96:]}, ["a", "b"], n, unit_norm=True)
+    score_of = torch.empty(6, n)
+    score_of.scatter_(1, order, full_v)
+    reported = score_of.gather(1, idx.cpu())
+    assert bool((reported >= ref_v[:, -1:] - tol).all())
+    assert (idx.cpu() == ref_i).float().mean().item() > 0.9
+
+
 @pytest.mark.parametrize("attribute_tokens", [False, True])
 def test_builder_flushes_only_changed_rows(device, tmp_path, attribute_tokens):
     """Device-resident store: rows reach the file at flush(), run by run of changed rows; a second flush after
