@@ -99,6 +99,12 @@ SIGNATURES: dict[str, tuple] = {
          C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p,
          C.c_void_p, C.c_int64, C.c_int64, C.c_int32, C.c_float, C.c_float, C.c_void_p],
     ),
+    "bgx_project_rows_workspace_bytes": (C.c_size_t, [C.c_int64, C.c_int64, C.c_int32, C.c_int32]),
+    "bgx_project_rows": (
+        C.c_int,
+        [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_int64,
+         C.c_void_p, C.c_size_t, C.c_void_p],
+    ),
     "bgx_fullgrad_tok": (
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32,

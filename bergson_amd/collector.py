@@ -495,7 +495,7 @@ class HookCollectorBase(ContextDecorator, ABC):
             ops.full_gradient(prep, a, g, tmp, per_token=self.attribute_tokens, lengths=lens,
                               rows=local if self.attribute_tokens else None, lo=self.lo, hi=self.hi)
             R = self.projection(name, pd, prep.width, "single", g.device, g.dtype)
-            acc += (tmp @ R.T).float()
+            ops.project_rows(tmp, R, acc)
         res = acc.to(out.dtype)
         if self.attribute_tokens:
             assert row_offsets is not None and counts is not None and local is not None

@@ -95,6 +95,9 @@ int fullgrad_seq_gemm_impl(const void* a, const void* g, int64_t a_seq_stride, i
                            const float* row_scale, const float* col_scale, const float* adam_v, int collect_bias,
                            const float* bias_scale, const int32_t* lengths, const int64_t* out_rows, void* out,
                            int64_t out_row_stride, int64_t out_col, int out_dtype, float lo, float hi, void* stream);
+size_t project_rows_workspace_bytes(int64_t M, int64_t W, int P, int dtype);
+int project_rows_impl(const void* rows, int64_t M, int64_t W, int64_t row_stride, int dtype, const void* proj, int P,
+                      float* acc, int64_t acc_stride, void* ws, size_t ws_bytes, void* stream);
 int collect_timing_enable(int max_launches);
 int collect_timing_read(float* ms_out, int capacity, int* count_out);
 int unit_normalize_impl(void* rows, int64_t n_rows, int64_t D, int64_t stride, int dtype, void* stream);
@@ -241,6 +244,17 @@ int bgx_fullgrad_seq_gemm(const void* a_dev, const void* g_dev, int64_t a_seq_st
                                      dtype, row_scale_dev, col_scale_dev, adam_v_dev, collect_bias, bias_scale_dev,
                                      lengths_dev, out_rows_dev, out_dev, out_row_stride, out_col, out_dtype, clamp_lo,
                                      clamp_hi, stream);
+}
+
+size_t bgx_project_rows_workspace_bytes(int64_t n_rows, int64_t width, int32_t P, int32_t dtype) {
+  return bgx::project_rows_workspace_bytes(n_rows, width, P, dtype);
+}
+
+int bgx_project_rows(const void* rows_dev, int64_t n_rows, int64_t width, int64_t row_stride, int32_t dtype,
+                     const void* proj_dev, int32_t P, float* acc_dev, int64_t acc_stride, void* workspace_dev,
+                     size_t workspace_bytes, void* stream) {
+  return bgx::project_rows_impl(rows_dev, n_rows, width, row_stride, dtype, proj_dev, P, acc_dev, acc_stride,
+                                workspace_dev, workspace_bytes, stream);
 }
 
 int bgx_collect_timing_enable(int32_t max_launches) { return bgx::collect_timing_enable(max_launches); }

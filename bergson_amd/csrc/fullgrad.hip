@@ -361,6 +361,129 @@ __global__ __launch_bounds__(256) void wgrad_seq_kernel(FullArgs a, WgradIn in) 
   }
 }
 
+// ---- the global projection: acc[m, j] += sum_k rows[m, k] * proj[j, k] ---------------------------------------
+// projection_target = "global" (collector.py:364-390): every module's flattened gradient [rows, W] times its
+// block [P, W] of the one projection matrix, summed into a [rows, P] fp32 accumulator.  Both operands have few
+// rows and a very long contraction (W = O * I: 10^5 .. 10^7), so the work is split along k: a workgroup takes 32
+// rows, up to 64 columns of the result and one slab of k; its four waves take every fourth k-step of the slab, so
+// that together they read whole 128-byte lines, with fragments loaded straight from global memory (both operands
+// have the contraction index as the fast one, which is what the MFMA operands want).  The waves' sums are added in
+// a fixed order through LDS and written to partial[slab][m][j]; project_reduce_kernel adds the slabs in order, so
+// the result does not depend on which workgroup finishes first.
+struct ProjArgs {
+  const void* rows;
+  const void* proj;
+  int64_t M, W, row_stride;
+  int P;
+  int64_t slab_len;  // elements of k per workgroup, a multiple of four k-steps
+  int n_slabs;
+  float* partial;    // [n_slabs, M, P]
+};
+
+constexpr int PROJ_PB = 2;  // 32-column blocks of the result per workgroup
+
+template <typename T, bool ALIGNED>
+__global__ __launch_bounds__(256) void project_rows_kernel(ProjArgs a) {
+  using M32 = Mma32<T>;
+  constexpr int EPL = M32::EPL, KS = 2 * EPL;
+  __shared__ float red[3][PROJ_PB][16][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int fr = lane & 31, fh = lane >> 5;
+  const int slab = blockIdx.x;
+  const int64_t m0 = (int64_t)blockIdx.y * 32;
+  const int j0 = blockIdx.z * (32 * PROJ_PB);
+  const int64_t k_begin = (int64_t)slab * a.slab_len;
+  const int64_t k_end = min(a.W, k_begin + a.slab_len);
+
+  const T* arow = (const T*)a.rows + min(m0 + fr, a.M - 1) * a.row_stride;
+  const T* prow[PROJ_PB];
+#pragma unroll
+  for (int b = 0; b < PROJ_PB; ++b) prow[b] = (const T*)a.proj + (int64_t)min(j0 + b * 32 + fr, a.P - 1) * a.W;
+
+  auto frag = [&](const T* row, int64_t k) -> uint4 {
+    if (ALIGNED) return k < k_end ? load16_global(row + k) : make_uint4(0u, 0u, 0u, 0u);
+    struct {
+      T e[EPL];
+    } tmp;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) tmp.e[e] = k + e < k_end ? row[k + e] : T{};
+    return __builtin_bit_cast(uint4, tmp);
+  };
+
+  f32x16 acc[PROJ_PB];
+#pragma unroll
+  for (int b = 0; b < PROJ_PB; ++b)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[b][e] = 0.f;
+  const bool second = j0 + 32 < a.P;  // the second block of columns exists
+  // four k-steps of this wave per round, their loads issued together
+  constexpr int UN = 4;
+  for (int64_t k = k_begin + wave * KS; k < k_end; k += UN * 4 * KS) {
+    uint4 af[UN], b0[UN], b1[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int64_t ka = k + (int64_t)u * 4 * KS + EPL * fh;
+      af[u] = frag(arow, ka);
+      b0[u] = frag(prow[0], ka);
+      b1[u] = second ? frag(prow[1], ka) : make_uint4(0u, 0u, 0u, 0u);
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      M32::mma(af[u], b0[u], acc[0]);
+      if (second) M32::mma(af[u], b1[u], acc[1]);
+    }
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int b = 0; b < PROJ_PB; ++b)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) red[wave - 1][b][e][lane] = acc[b][e];
+  }
+  __syncthreads();
+  if (wave == 0) {
+    // acc[b][e] = row m0 + 8 (e / 4) + 4 fh + e % 4, column j0 + 32 b + fr
+#pragma unroll
+    for (int b = 0; b < PROJ_PB; ++b) {
+      const int j = j0 + b * 32 + fr;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int64_t m = m0 + 8 * (e >> 2) + 4 * fh + (e & 3);
+        if (m < a.M && j < a.P)
+          a.partial[((int64_t)slab * a.M + m) * a.P + j] =
+              ((acc[b][e] + red[0][b][e][lane]) + red[1][b][e][lane]) + red[2][b][e][lane];
+      }
+    }
+  }
+}
+
+// acc[m, j] += sum over the slabs, in an order that depends on the shape alone.  Few results: one wave per
+// result, lane l adds slabs l, l + 64, ... and the lanes' sums meet in a butterfly; many results: one thread each.
+__global__ __launch_bounds__(256) void project_reduce_kernel(const float* __restrict__ partial, int n_slabs, int64_t M,
+                                                             int P, float* __restrict__ acc, int64_t acc_stride,
+                                                             int by_wave) {
+  const int64_t total = M * P;
+  if (by_wave) {
+    const int64_t e = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (e >= total) return;
+    const int lane = threadIdx.x & 63;
+    float s = 0.f;
+    for (int t = lane; t < n_slabs; t += 64) s += partial[(int64_t)t * total + e];
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) s += __shfl_xor(s, d);
+    if (lane == 0) {
+      const int64_t m = e / P;
+      acc[m * acc_stride + (e - m * P)] += s;
+    }
+  } else {
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= total) return;
+    float s = 0.f;
+    for (int t = 0; t < n_slabs; ++t) s += partial[(int64_t)t * total + e];
+    const int64_t m = e / P;
+    acc[m * acc_stride + (e - m * P)] += s;
+  }
+}
+
 static bool dtype_ok(int dt) { return dt >= BGX_F32 && dt <= BGX_BF16; }
 
 int token_sum_impl(const void* g, int64_t g_seq_stride, int64_t g_tok_stride, int N, int S, int O, int dtype,
@@ -466,6 +589,77 @@ int fullgrad_seq_gemm_impl(const void* a, const void* g, int64_t a_seq_stride, i
     launch_wgrad<f16_t>(fa, in, N, st);
   else
     launch_wgrad<bf16_t>(fa, in, N, st);
+  BGX_HIP(hipGetLastError());
+  return 0;
+}
+
+// how the contraction is cut: enough workgroups to fill the chip, slabs of whole groups of four k-steps
+static void project_plan(int64_t M, int64_t W, int P, int dtype, int64_t* slab_len, int* n_slabs) {
+  const int64_t ks4 = 4 * (dtype == BGX_F32 ? 8 : 16);
+  const int64_t tiles = ((M + 31) / 32) * ((P + 32 * PROJ_PB - 1) / (32 * PROJ_PB));
+  int64_t want = std::max<int64_t>(1, 1024 / tiles);
+  const int64_t max_slabs = std::max<int64_t>(1, W / (16 * ks4));
+  want = std::min(std::min(want, max_slabs), (int64_t)4096);
+  int64_t len = (W + want - 1) / want;
+  len = (len + ks4 - 1) / ks4 * ks4;
+  *slab_len = len;
+  *n_slabs = (int)((W + len - 1) / len);
+}
+
+size_t project_rows_workspace_bytes(int64_t M, int64_t W, int P, int dtype) {
+  if (M <= 0 || W <= 0 || P <= 0) return 0;
+  int64_t len;
+  int n;
+  project_plan(M, W, P, dtype, &len, &n);
+  return (size_t)n * (size_t)M * (size_t)P * sizeof(float);
+}
+
+int project_rows_impl(const void* rows, int64_t M, int64_t W, int64_t row_stride, int dtype, const void* proj, int P,
+                      float* acc, int64_t acc_stride, void* ws, size_t ws_bytes, void* stream) {
+  BGX_REQUIRE(rows && proj && acc, BGX_E_ARG, "project_rows: null pointer");
+  BGX_REQUIRE(M > 0 && W > 0 && P > 0 && row_stride >= W && acc_stride >= P, BGX_E_SHAPE,
+              "project_rows: M=%lld W=%lld P=%d strides %lld %lld", (long long)M, (long long)W, P,
+              (long long)row_stride, (long long)acc_stride);
+  BGX_REQUIRE(dtype_ok(dtype), BGX_E_DTYPE, "project_rows: dtype=%d", dtype);
+  BGX_REQUIRE((M + 31) / 32 <= 65535 && (P + 32 * PROJ_PB - 1) / (32 * PROJ_PB) <= 65535, BGX_E_SHAPE,
+              "project_rows: M=%lld P=%d", (long long)M, P);
+  ProjArgs pa;
+  project_plan(M, W, P, dtype, &pa.slab_len, &pa.n_slabs);
+  const size_t need = (size_t)pa.n_slabs * (size_t)M * (size_t)P * sizeof(float);
+  BGX_REQUIRE(ws != nullptr && ws_bytes >= need, BGX_E_WORKSPACE, "project_rows: workspace of %zu bytes, need %zu",
+              ws_bytes, need);
+  pa.rows = rows;
+  pa.proj = proj;
+  pa.M = M;
+  pa.W = W;
+  pa.row_stride = row_stride;
+  pa.P = P;
+  pa.partial = (float*)ws;
+  const int64_t es = (int64_t)dtype_size(dtype);
+  const bool aligned = (uintptr_t)rows % 16 == 0 && (uintptr_t)proj % 16 == 0 && (row_stride * es) % 16 == 0 &&
+                       (W * es) % 16 == 0;
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid((unsigned)pa.n_slabs, (unsigned)((M + 31) / 32), (unsigned)((P + 32 * PROJ_PB - 1) / (32 * PROJ_PB)));
+#define BGX_PROJ_LAUNCH(T)                                                                         \
+  do {                                                                                             \
+    if (aligned)                                                                                   \
+      hipLaunchKernelGGL((project_rows_kernel<T, true>), grid, dim3(256), 0, st, pa);              \
+    else                                                                                           \
+      hipLaunchKernelGGL((project_rows_kernel<T, false>), grid, dim3(256), 0, st, pa);             \
+  } while (0)
+  if (dtype == BGX_F32)
+    BGX_PROJ_LAUNCH(float);
+  else if (dtype == BGX_F16)
+    BGX_PROJ_LAUNCH(f16_t);
+  else
+    BGX_PROJ_LAUNCH(bf16_t);
+#undef BGX_PROJ_LAUNCH
+  BGX_HIP(hipGetLastError());
+  const int64_t total = M * P;
+  const int by_wave = total < 16384 ? 1 : 0;
+  const int64_t blocks = by_wave ? (total + 3) / 4 : (total + 255) / 256;
+  hipLaunchKernelGGL(project_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, st, pa.partial, pa.n_slabs, M, P, acc,
+                     acc_stride, by_wave);
   BGX_HIP(hipGetLastError());
   return 0;
 }

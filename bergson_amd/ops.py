@@ -470,6 +470,30 @@ def full_gradient(mod: FullGradModule, a: Tensor, g: Tensor, out: Tensor, *, per
     _lib.check(rc, "bgx_fullgrad_seq_gemm")
 
 
+def project_rows(rows: Tensor, proj: Tensor, acc: Tensor) -> None:
+    """acc[m, j] += sum_k rows[m, k] * proj[j, k]: one module's share of the global projection
+    (collector.py:364-390).  rows [M, W] and proj [P, W] in the model dtype, acc [M, P] fp32, added to."""
+    lib = _lib.load()
+    for t, name in ((rows, "rows"), (proj, "proj"), (acc, "acc")):
+        _need_gpu(t, name)
+    if rows.dim() != 2 or proj.dim() != 2 or rows.shape[1] != proj.shape[1] or rows.dtype != proj.dtype:
+        raise ValueError(f"rows {tuple(rows.shape)} {rows.dtype} / proj {tuple(proj.shape)} {proj.dtype} do not match")
+    if acc.dtype != torch.float32 or acc.shape != (rows.shape[0], proj.shape[0]) or acc.stride(1) != 1:
+        raise ValueError("acc must be fp32 [rows, P] with contiguous rows")
+    if rows.stride(1) != 1:
+        rows = rows.contiguous()
+    proj = proj.contiguous()
+    M, W = rows.shape
+    P = proj.shape[0]
+    if M == 0:
+        return
+    code = dtype_code(rows.dtype)
+    ws = _workspace(rows.device, lib.bgx_project_rows_workspace_bytes(M, W, P, code), "project")
+    rc = lib.bgx_project_rows(_ptr(rows), M, W, rows.stride(0), code, _ptr(proj), P, _ptr(acc), acc.stride(0),
+                              _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "bgx_project_rows")
+
+
 def _collect_adam_seq(prep: AdamPrepared, a: Tensor, g: Tensor, out: Tensor, lengths: Tensor | None,
                       rows: Tensor | None, lo: float, hi: float) -> None:
     """Per-sequence Adam without anything per token: the normalisation is applied to the summed gradient, as

@@ -271,6 +271,21 @@ int bgx_fullgrad_seq_gemm(const void* a_dev, const void* g_dev,
                           int64_t out_row_stride, int64_t out_col,
                           int32_t out_dtype, float clamp_lo, float clamp_hi,
                           void* stream);
+/* The global projection (projection_target = "global",
+ * collector.py:364-390: `grad.flatten(1) @ proj.T` per module, summed over
+ * the modules): acc_dev[m, j] += sum_k rows_dev[m, k] * proj_dev[j, k] for
+ * m < n_rows, j < P, k < width.  rows_dev [n_rows, width] (row stride in
+ * elements) is what bgx_fullgrad_seq_gemm / bgx_fullgrad_tok wrote for one
+ * module, proj_dev [P, width] (contiguous) the module's block of the projection
+ * matrix, both in `dtype`; acc_dev is fp32 and is added to, so a caller zeroes
+ * it once and calls this per module.  The contraction is split into slabs
+ * whose sums are added in a fixed order (workspace: partial sums). */
+size_t bgx_project_rows_workspace_bytes(int64_t n_rows, int64_t width,
+                                        int32_t P, int32_t dtype);
+int bgx_project_rows(const void* rows_dev, int64_t n_rows, int64_t width,
+                     int64_t row_stride, int32_t dtype, const void* proj_dev,
+                     int32_t P, float* acc_dev, int64_t acc_stride,
+                     void* workspace_dev, size_t workspace_bytes, void* stream);
 int bgx_fullgrad_tok(const void* a_dev, const void* g_dev,
                      int64_t a_seq_stride, int64_t a_tok_stride,
                      int64_t g_seq_stride, int64_t g_tok_stride, int32_t N,

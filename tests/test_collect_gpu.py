@@ -612,6 +612,47 @@ def test_fullgrad_two_step_entries_agree_with_fused(device, kind):
     assert rel_l2(fused.cpu(), two.cpu()) <= 4e-3
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(3, 40 * 24, 16), (70, 5000, 40), (2, 393216, 32), (33, 1001, 100), (1, 7, 1)])
+def test_project_rows_against_float64(device, dtype, shape):
+    """The global projection's contraction (rows [M, W] times a [P, W] block, added to an fp32 accumulator):
+    few and many rows, widths that are no multiple of a k-step (and of nothing: the element-wise loader), more
+    columns than one workgroup takes, a second call adding to the first, and the same bits on a repeat."""
+    from bergson_amd import ops
+
+    M, W, P = shape
+    gen = torch.Generator().manual_seed(95)
+    rows = (torch.randn(M, W, generator=gen) * 0.1).to(dtype)
+    proj = (torch.randn(P, W, generator=gen) / W ** 0.5).to(dtype)
+    want = rows.double() @ proj.double().T
+    acc = torch.zeros(M, P, dtype=torch.float32, device=device)
+    ops.project_rows(rows.to(device), proj.to(device), acc)
+    torch.cuda.synchronize()
+    first = acc.clone()
+    assert rel_l2(first.cpu().double(), want) <= (1e-5 if dtype == torch.float32 else 1e-4)  # exact products, fp32 sums
+    ops.project_rows(rows.to(device), proj.to(device), acc)
+    again = torch.zeros_like(first)
+    ops.project_rows(rows.to(device), proj.to(device), again)
+    torch.cuda.synchronize()
+    assert torch.equal(again, first)
+    assert rel_l2(acc.cpu().double(), 2 * want) <= (1e-5 if dtype == torch.float32 else 1e-4)
+
+
+def test_project_rows_strided_rows(device):
+    """Rows that are a column slice of a wider buffer (row stride above the width, first element off a 16-byte
+    boundary)."""
+    from bergson_amd import ops
+
+    gen = torch.Generator().manual_seed(96)
+    big = (torch.randn(9, 700, generator=gen) * 0.1).to(torch.bfloat16).to(device)
+    rows = big[:, 3:3 + 640]
+    proj = (torch.randn(24, 640, generator=gen) / 25).to(torch.bfloat16).to(device)
+    acc = torch.zeros(9, 24, dtype=torch.float32, device=device)
+    ops.project_rows(rows, proj, acc)
+    torch.cuda.synchronize()
+    assert rel_l2(acc.cpu().double(), rows.cpu().double() @ proj.cpu().double().T) <= 1e-4
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("kind", [None, "adafactor", "adam"])
 @pytest.mark.parametrize("bias", [False, True])
