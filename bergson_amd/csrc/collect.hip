@@ -591,11 +591,15 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
         const int lt = p == 16 ? 5 : 3;       // log2 of the p * jg lane tasks per token
         auto write_rows = [&](auto dt_tag) {  // one copy of the loop per output dtype, chosen outside it
           constexpr int DT = decltype(dt_tag)::value;
-          for (int x = lane; x < (rows_valid << lt); x += WAVE) {
-            const int t = x >> lt;
-            const int rem = x & ((1 << lt) - 1);
-            const int i = rem >> (jg - 1);
-            const int j0 = (rem & (jg - 1)) << 3;
+          // a lane keeps its place (i, j0) in the block and walks the tokens in steps of 64 >> lt, so that
+          // nothing but two additions depends on the token
+          const int rem = lane & ((1 << lt) - 1);
+          const int i = rem >> (jg - 1);
+          const int j0 = (rem & (jg - 1)) << 3;
+          const int step_t = WAVE >> lt;
+          int64_t dst = (row0 + (lane >> lt)) * args.out_row_stride + d.out_col + i * p + j0;
+          const int64_t dst_step = (int64_t)step_t * args.out_row_stride;
+          for (int t = lane >> lt; t < rows_valid; t += step_t, dst += dst_step) {
             const float gv = tok[wave][1][t][i];
             const float4 a_lo = *reinterpret_cast<const float4*>(&tok[wave][0][t][j0]);
             const float4 a_hi = *reinterpret_cast<const float4*>(&tok[wave][0][t][j0 + 4]);
@@ -603,7 +607,7 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
                                 clampf(gv * a_lo.z, args.lo, args.hi), clampf(gv * a_lo.w, args.lo, args.hi),
                                 clampf(gv * a_hi.x, args.lo, args.hi), clampf(gv * a_hi.y, args.lo, args.hi),
                                 clampf(gv * a_hi.z, args.lo, args.hi), clampf(gv * a_hi.w, args.lo, args.hi)};
-            store8_as<DT>(args.out, (row0 + t) * args.out_row_stride + d.out_col + i * p + j0, o);
+            store8_as<DT>(args.out, dst, o);
           }
         };
         if (args.out_dtype == BGX_F32)

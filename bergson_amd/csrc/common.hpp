@@ -89,12 +89,21 @@ __host__ __device__ inline size_t dtype_size(int dt) {
 __device__ inline float bf16_bits_to_f32(uint32_t b) {
   return __uint_as_float(b << 16);
 }
-// round-to-nearest-even, NaN kept quiet
+// round-to-nearest-even, NaN kept quiet: the hardware conversion (v_cvt_pk_bf16_f32)
 __device__ inline uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0u;
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return u >> 16;
+  return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
+}
+// two values at once, the first in the low half
+__device__ inline uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
+  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  const f2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, b2));
+}
+__device__ inline uint32_t f32x2_to_f16x2_bits(float lo, float hi) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  const h2 r = {(_Float16)lo, (_Float16)hi};
+  return __builtin_bit_cast(uint32_t, r);
 }
 __device__ inline float f16_bits_to_f32(uint32_t b) {
   union {
@@ -163,11 +172,8 @@ __device__ inline void store8_as(void* base, int64_t idx, const float (&v)[8]) {
   } else {
     uint32_t w[4];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const uint32_t lo = DT == BGX_F16 ? f32_to_f16_bits(v[2 * k]) : f32_to_bf16_bits(v[2 * k]);
-      const uint32_t hi = DT == BGX_F16 ? f32_to_f16_bits(v[2 * k + 1]) : f32_to_bf16_bits(v[2 * k + 1]);
-      w[k] = (lo & 0xffffu) | (hi << 16);
-    }
+    for (int k = 0; k < 4; ++k)
+      w[k] = DT == BGX_F16 ? f32x2_to_f16x2_bits(v[2 * k], v[2 * k + 1]) : f32x2_to_bf16x2_bits(v[2 * k], v[2 * k + 1]);
     typedef uint32_t raw4 __attribute__((ext_vector_type(4)));
     __builtin_nontemporal_store(raw4{w[0], w[1], w[2], w[3]}, reinterpret_cast<raw4*>((uint16_t*)base + idx));
   }
@@ -180,8 +186,10 @@ __device__ inline float load_as(const void* base, int64_t idx, int dt) {
 }
 
 __device__ inline float clampf(float v, float lo, float hi) {
-  // NaN propagates like torch.clamp
-  return v < lo ? lo : (v > hi ? hi : v);
+  // lo <= hi; the median of the three is the clamped value (one instruction), and NaN propagates like
+  // torch.clamp (the median instruction alone would turn it into lo)
+  const float r = __builtin_amdgcn_fmed3f(v, lo, hi);
+  return v != v ? v : r;
 }
 
 }  // namespace bgx
