@@ -1,4 +1,4 @@
-"""A build-time property of `scan_wide_kernel` that no numerical test can be relied on to catch.
+"""Build-time properties of the hand-scheduled kernels that no numerical test can be relied on to catch.
 
 The kernel issues its LDS fragment reads and its matrix instructions as inline assembly and waits for the reads
 itself; to the compiler the value of a read is there as soon as the statement is.  Should the register allocator
@@ -6,7 +6,9 @@ run out of registers inside the tile loop (the kernel uses all 512 of a wave), i
 scratch memory before the read has arrived, or reuse a register that a read in flight is still going to write
 -- wrong rows in the first case, a wild address in the second.  So the compiled code is inspected: from the first
 fragment read to the end of the tile loop there must be no scratch instruction, and the loop must be one copy
-(one loop header).  hipcc cross-compiles without a GPU; the test takes about a minute.
+(one loop header).  The other kernels that read their fragments this way (`scan_direct_kernel`,
+`adam_fused_direct_kernel`) have registers to spare; for them the check is that they use no scratch memory at all.
+hipcc cross-compiles without a GPU; the two compilations run side by side and take about a minute.
 """
 import re
 import subprocess
@@ -18,14 +20,29 @@ ROOT = Path(__file__).resolve().parent.parent
 
 
 @pytest.fixture(scope="module")
-def scan_isa(tmp_path_factory):
+def isa(tmp_path_factory):
+    """{source name: compiled device code as text} for scan.hip and adam.hip."""
+    from concurrent.futures import ThreadPoolExecutor
+
     from bergson_amd import build_ext
 
-    out = tmp_path_factory.mktemp("isa") / "scan.s"
-    cmd = [build_ext.HIPCC, *build_ext.FLAGS, "--cuda-device-only", "-S", str(build_ext.CSRC / "scan.hip"), "-o", str(out)]
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    assert res.returncode == 0, res.stderr[-2000:]
-    return out.read_text()
+    tmp = tmp_path_factory.mktemp("isa")
+
+    def compile_one(src):
+        out = tmp / (src + ".s")
+        cmd = [build_ext.HIPCC, *build_ext.FLAGS, "--cuda-device-only", "-S", str(build_ext.CSRC / src), "-o", str(out)]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        assert res.returncode == 0, res.stderr[-2000:]
+        return out.read_text()
+
+    with ThreadPoolExecutor(max_workers=2) as ex:
+        texts = list(ex.map(compile_one, ["scan.hip", "adam.hip"]))
+    return {"scan.hip": texts[0], "adam.hip": texts[1]}
+
+
+@pytest.fixture(scope="module")
+def scan_isa(isa):
+    return isa["scan.hip"]
 
 
 @pytest.mark.parametrize("elem", ["5f16_t", "6bf16_t"])
@@ -45,3 +62,20 @@ def test_wide_scan_kernel_keeps_its_fragments_in_registers(scan_isa, elem):
     assert not scratch, f"scratch traffic between the first fragment read and the end of the tile loop: {scratch[:4]}"
     assert not any(re.search(r"\bs_load|s_buffer_load", l) for l in lines[headers[0]:loop_end]), \
         "scalar loads inside the loop share the counter the fragment waits count on"
+
+
+@pytest.mark.parametrize("source,pattern", [
+    ("scan.hip", r"_ZN3bgx18scan_direct_kernelI\S*"),
+    ("adam.hip", r"_ZN3bgx24adam_fused_direct_kernelI\S*"),
+])
+def test_direct_to_lds_kernels_use_no_scratch(isa, source, pattern):
+    """Every instantiation: no scratch instruction anywhere and a private segment of zero bytes."""
+    text = isa[source]
+    names = sorted(set(re.findall(rf"^({pattern}):", text, re.M)))
+    assert names, f"no kernel matching {pattern} in {source}"
+    for name in names:
+        m = re.search(rf"^{re.escape(name)}:[^\n]*\n(.*?)\n\s*s_endpgm", text, re.S | re.M)
+        assert m, name
+        assert "scratch_" not in m.group(1), f"{name} spills"
+        meta = re.search(rf"\.amdhsa_kernel {re.escape(name)}\n(.*?)\.end_amdhsa_kernel", text, re.S)
+        assert meta and re.search(r"\.amdhsa_private_segment_fixed_size 0\b", meta.group(1)), name
