@@ -90,52 +90,89 @@ struct ScanArgs {
   int units_rem;
 };
 
+// Reduction over the 32 lanes of a half wave with data-parallel-primitive moves (no LDS round trips): a running
+// combination over shifts of 1, 2, 4 and 8 lanes inside each row of 16, then the first row's total handed to the
+// second.  The total of lanes 0 .. 31 ends up in lane 31, that of lanes 32 .. 63 in lane 63; the other lanes hold
+// partial results.  `identity` is what a lane without a source contributes.
+template <bool IS_MAX>
+__device__ __forceinline__ float reduce_half_wave(float v, float identity) {
+  auto op = [](float x, float y) { return IS_MAX ? fmaxf(x, y) : x + y; };
+  const int id = __float_as_int(identity);
+  v = op(v, __int_as_float(__builtin_amdgcn_update_dpp(id, __float_as_int(v), 0x111, 0xf, 0xf, false)));  // row_shr:1
+  v = op(v, __int_as_float(__builtin_amdgcn_update_dpp(id, __float_as_int(v), 0x112, 0xf, 0xf, false)));  // row_shr:2
+  v = op(v, __int_as_float(__builtin_amdgcn_update_dpp(id, __float_as_int(v), 0x114, 0xf, 0xf, false)));  // row_shr:4
+  v = op(v, __int_as_float(__builtin_amdgcn_update_dpp(id, __float_as_int(v), 0x118, 0xf, 0xf, false)));  // row_shr:8
+  v = op(v, __int_as_float(__builtin_amdgcn_update_dpp(id, __float_as_int(v), 0x142, 0xa, 0xf, false)));  // row_bcast:15
+  return v;
+}
+
 // Epilogue of a workgroup tile whose waves hold (TM x TN) blocks of 32 x 32 scores in MFMA layout: scale by the
 // row multipliers s_inv, then dense scores, row maxima, row-sum partials and the threshold filter.
-// One row block (acc_row = the wave's TN blocks of 32 rows x 32 queries; `blk` = which 32 rows of the wave's):
+// One row block (acc_row = the wave's TN blocks of 32 rows x 32 queries; `blk` = which 32 rows of the wave's).
+// A lane holds, for 16 rows (e), one score per query block: the products and their maximum / sum over the query
+// blocks are a handful of instructions per row, the reductions over the 32 lanes use no LDS, only the lane that
+// ends up with a row's result touches memory, all addresses are a per-lane base plus constants, and the
+// candidate path (scores above a query's current k-th best: rare once the thresholds have settled) is entered
+// only by rows that have one.  thr[j] is +inf for queries past Q.
 template <int TN, int WTM, int WTN, int WN>
 __device__ __forceinline__ void scan_block_epilogue(const ScanArgs& args, f32x16 (&acc_row)[TN], const float (&thr)[TN],
                                                     const float* s_inv, int blk, int wm, int wn, int fr, int fh,
                                                     int64_t g_row0, int64_t q_row0, int qt) {
+  const int row_b = wm * WTM + blk * 32 + fh * 4;  // tile row of e = 0; e adds (e >> 2) * 8 + (e & 3)
+  const int64_t prow_b = g_row0 + row_b;           // pass-local
+  const int64_t grow_b = args.row0 + prow_b;
+  const int64_t q_b = q_row0 + wn * WTN + fr;      // query of j = 0; j adds 32
+  bool q_ok[TN];
 #pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const int row = wm * WTM + blk * 32 + (e >> 2) * 8 + fh * 4 + (e & 3);
-    const int64_t prow = g_row0 + row;  // pass-local row
-    const bool row_ok = prow < args.rows;
-    const int64_t grow = args.row0 + prow;
-    const float w = s_inv[row];
-    float rmax = -INFINITY;
-    float rsum = 0.f;
+  for (int j = 0; j < TN; ++j) q_ok[j] = q_b + j * 32 < args.Q;
+  // how many of the 16 rows exist: rows_here <= 0 none, >= 28 all
+  const int64_t rows_here = args.rows - prow_b;
+  uint32_t* const rmax_p = args.row_max_enc != nullptr ? args.row_max_enc + grow_b : nullptr;
+  float* const rsum_p =
+      args.row_sum_part != nullptr ? args.row_sum_part + prow_b * args.n_parts + (qt * WN + wn) : nullptr;
+  const bool writer = fr == 31;
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int64_t q = q_row0 + wn * WTN + j * 32 + fr;
-      const float v = acc_row[j][e] * w;
-      if (row_ok && q < args.Q) {
-        rmax = fmaxf(rmax, v);
-        rsum += v;
-        if (args.scores != nullptr) args.scores[grow * args.Q + q] = v;
-        if (v > thr[j]) {
-          const uint32_t pos = atomicAdd(&args.cand_count[q], 1u);
-          if ((int64_t)pos < args.cand_cap) args.cand[q * args.cand_cap + pos] = make_key(v, (uint32_t)grow);
+  for (int g = 0; g < 4; ++g) {
+    const f32x4 w4 = *reinterpret_cast<const f32x4*>(s_inv + row_b + g * 8);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int e = g * 4 + c;
+      const int dr = g * 8 + c;  // row offset of this e
+      const bool row_ok = dr < rows_here;
+      float v[TN];
+      float rmax = -INFINITY, rsum = 0.f;
+      bool any = false;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        v[j] = acc_row[j][e] * w4[c];
+        if (q_ok[j]) {
+          rmax = fmaxf(rmax, v[j]);
+          rsum += v[j];
         }
+        any |= v[j] > thr[j];
       }
-    }
-    if (args.row_max_enc != nullptr) {
-      rmax = fmaxf(rmax, __shfl_xor(rmax, 1));
-      rmax = fmaxf(rmax, __shfl_xor(rmax, 2));
-      rmax = fmaxf(rmax, __shfl_xor(rmax, 4));
-      rmax = fmaxf(rmax, __shfl_xor(rmax, 8));
-      rmax = fmaxf(rmax, __shfl_xor(rmax, 16));
-      if (fr == 0 && row_ok) atomicMax(&args.row_max_enc[grow], f32_ordered(rmax));
-    }
-    if (args.row_sum_part != nullptr) {
-      // fixed-order butterfly over the 32 lanes that hold this row's scores; one writer per (row, part)
-      rsum += __shfl_xor(rsum, 1);
-      rsum += __shfl_xor(rsum, 2);
-      rsum += __shfl_xor(rsum, 4);
-      rsum += __shfl_xor(rsum, 8);
-      rsum += __shfl_xor(rsum, 16);
-      if (fr == 0 && row_ok) args.row_sum_part[prow * args.n_parts + qt * WN + wn] = rsum;
+      if (args.scores != nullptr && row_ok) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          if (q_ok[j]) args.scores[(grow_b + dr) * args.Q + q_b + j * 32] = v[j];
+      }
+      if (any && row_ok) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          if (v[j] > thr[j]) {
+            const int64_t q = q_b + j * 32;
+            const uint32_t pos = atomicAdd(&args.cand_count[q], 1u);
+            if ((int64_t)pos < args.cand_cap) args.cand[q * args.cand_cap + pos] = make_key(v[j], (uint32_t)(grow_b + dr));
+          }
+      }
+      if (rmax_p != nullptr) {
+        rmax = reduce_half_wave<true>(rmax, -INFINITY);
+        if (writer && row_ok) atomicMax(rmax_p + dr, f32_ordered(rmax));
+      }
+      if (rsum_p != nullptr) {
+        rsum = reduce_half_wave<false>(rsum, 0.f);
+        if (writer && row_ok) rsum_p[(int64_t)dr * args.n_parts] = rsum;
+      }
     }
   }
 }
@@ -188,7 +225,7 @@ __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
   extern __shared__ __align__(16) unsigned char smem[];
   // [buf][BM + BN rows][LDS_ROW_BYTES]
   constexpr int BUF_BYTES = (BM + BN) * LDS_ROW_BYTES;
-  __shared__ float s_inv[BM];
+  __shared__ __align__(16) float s_inv[BM];
 
   // XCD-aware tile order: workgroup b runs on XCD b % 8; the q_tiles
   // workgroups of one row tile share that XCD's L2.
@@ -749,11 +786,13 @@ __global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  // The 20 loads of a tile are spread over a whole tile period, one behind every fourth MFMA: a compute unit takes
-  // its lines from L2 at a fixed pace, and a wave that asks faster than that is held at the load instruction --
-  // with one wave per SIMD, the MFMAs behind it wait too.  Tile t + 2's first five loads go out behind the barrier
-  // that gives up tile t's stage (last step of tile t), the other fifteen during the first three steps of tile
-  // t + 1; the last of them is 14 MFMAs ahead of the barrier that needs it.
+  // The 20 loads of a tile go out one behind every third MFMA, starting right behind the barrier that gives up the
+  // stage they fill: seven in what is left of the last step of tile t, eight and five in the first two steps of tile
+  // t + 1, for tile t + 2.  The barrier that needs them waits for all of this wave's loads, the youngest included, so
+  // what counts is how long before it the last one is issued: 58 MFMAs here (it was 14 with one load per four
+  // MFMAs spread over the whole period, and the wait for that load showed in every tile).  Issued faster than
+  // one per two or three MFMAs the loads hold up the wave at the load instruction -- with one wave per SIMD the
+  // MFMAs behind it wait too.
   // There is ONE copy of the tile code and no branch in it: past the end of the row the loads fetch the last K
   // tile again (into a stage nobody reads any more; a few loads per 192 tiles) and the reads take whatever the
   // other stage holds.  One copy on purpose: in every copy the compiler has to find registers for the whole tile
@@ -779,7 +818,7 @@ __global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
   {
     const int k1 = min(1, KT - 1);
 #pragma unroll
-    for (int idx = 0; idx < 5; ++idx) load_one_to(k1, 1, idx);  // what the last step of a tile issues for the next but one
+    for (int idx = 0; idx < 7; ++idx) load_one_to(k1, 1, idx);  // what the last step of a tile issues for the next but one
   }
   __builtin_amdgcn_sched_barrier(0);
 
@@ -789,20 +828,18 @@ __global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
     const int k2 = min(kt + 2, KT - 1);  // ... and the one whose loads begin behind this tile's barrier
     // (a clamped tile number only changes where the data comes from: the stage is the one tile kt + 1 / kt + 2 would use)
     step(S0{}, K0{}, K1{}, st, nothing, [&](int n) {
-      if ((n & 3) == 1 && n <= 21) load_one_to(k1, st ^ 1, 5 + (n >> 2));
+      if (n % 3 == 1 && n <= 22) load_one_to(k1, st ^ 1, 7 + n / 3);
     });
     step(S1{}, K1{}, K2{}, st, nothing, [&](int n) {
-      if ((n & 3) == 1 && n <= 17) load_one_to(k1, st ^ 1, 11 + (n >> 2));
+      if (n % 3 == 1 && n <= 13) load_one_to(k1, st ^ 1, 15 + n / 3);
     });
-    step(S0{}, K2{}, K3{}, st, nothing, [&](int n) {
-      if ((n & 3) == 1 && n <= 13) load_one_to(k1, st ^ 1, 16 + (n >> 2));
-    });
+    step(S0{}, K2{}, K3{}, st, nothing, [](int) {});
     // Last step of the tile.  Its fragments were asked for during the step before; behind its first four MFMAs
     // every read of this stage has to be back (the stage is given up) and tile kt + 1 has to have landed in the
     // other stage: all of this wave's loads and reads done, then the barrier makes that all waves'.  Behind the
     // barrier: step 0 of tile kt + 1 is read, and tile kt + 2 begins to load into the stage just given up.
     step(S1{}, K3{}, K0{}, st ^ 1, tile_change, [&](int n) {
-      if ((n & 3) == 1 && n >= 5) load_one_to(k2, st, (n >> 2) - 1);
+      if (n % 3 == 1 && n >= 4) load_one_to(k2, st, n / 3 - 1);
     });
     // The MFMAs are opaque to the compiler, which therefore adds no wait states before code of its own that reads
     // an accumulator (it may place such code right behind the loop): the last results are given their 20 states
