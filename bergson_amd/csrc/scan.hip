@@ -177,6 +177,118 @@ __device__ __forceinline__ void scan_block_epilogue(const ScanArgs& args, f32x16
   }
 }
 
+// Sixteen values per lane reduced over the 32 lanes of a half wave at once: at each of four exchanges a lane
+// keeps one half of its values and hands the other half to a partner that keeps the opposite half (partners: lane
+// ^ 16 through a swizzle, then the mirror images within 16 and within 8 lanes, then lane ^ 2), so the values
+// halve while the lanes combined double; a last exchange with lane ^ 1 completes it.  Lane fr ends up with the
+// result for value (fr >> 1) & 15 (lanes fr and fr ^ 1 hold the same).  62 instructions for 16 reductions; the
+// order of the additions is fixed by the lane numbers.
+template <bool IS_MAX>
+__device__ __forceinline__ float reduce16_half_wave(const float (&x)[16], int fr) {
+  auto op = [](float p, float q) { return IS_MAX ? fmaxf(p, q) : p + q; };
+  auto dpp = [](float v, auto ctrl_tag) {
+    constexpr int CTRL = decltype(ctrl_tag)::value;
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+  };
+  const bool b4 = (fr & 16) != 0, b3 = (fr & 8) != 0, b2 = (fr & 4) != 0, b1 = (fr & 2) != 0;
+  float a8[8], a4[4], a2[2];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float keep = b4 ? x[8 + i] : x[i], send = b4 ? x[i] : x[8 + i];
+    a8[i] = op(keep, __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(send), 0x401F)));  // lane ^ 16
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float keep = b3 ? a8[4 + i] : a8[i], send = b3 ? a8[i] : a8[4 + i];
+    a4[i] = op(keep, dpp(send, std::integral_constant<int, 0x140>{}));  // row_mirror: lane <-> 15 - lane
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const float keep = b2 ? a4[2 + i] : a4[i], send = b2 ? a4[i] : a4[2 + i];
+    a2[i] = op(keep, dpp(send, std::integral_constant<int, 0x141>{}));  // row_half_mirror: lane <-> 7 - lane
+  }
+  const float keep = b1 ? a2[1] : a2[0], send = b1 ? a2[0] : a2[1];
+  float r = op(keep, dpp(send, std::integral_constant<int, 0x4E>{}));  // quad_perm [2, 3, 0, 1]: lane ^ 2
+  r = op(r, dpp(r, std::integral_constant<int, 0xB1>{}));                // quad_perm [1, 0, 3, 2]: lane ^ 1
+  return r;
+}
+
+// The same for a block whose 32 rows and TN * 32 queries all exist (every block of a scan whose row and query
+// counts are multiples of the tile, and all but the edge blocks otherwise): straight-line code -- the products and
+// each row's maximum / sum over the lane's query blocks, the sixteen rows reduced over the lanes together, one
+// atomic / store instruction in which sixteen lanes write a row each.
+// Candidates (scores above their query's current k-th best; a few per thousand scores once the thresholds have
+// settled): a lane looks at the sixteen scores of a query block one by one only when the largest of them is above
+// the query's threshold, and that code is marked unlikely so that it is laid out behind the function -- stepping
+// over it, block after block, otherwise costs more in instruction fetch than the rest of the epilogue.
+template <int TN, int WTM, int WTN, int WN>
+__device__ __forceinline__ void scan_block_epilogue_full(const ScanArgs& args, f32x16 (&acc_row)[TN],
+                                                         const float (&thr)[TN],
+                                                         const float* s_inv, int blk, int wm, int wn, int fr, int fh,
+                                                         int64_t g_row0, int64_t q_row0, int qt) {
+  const int row_b = wm * WTM + blk * 32 + fh * 4;
+  const int64_t prow_b = g_row0 + row_b;
+  const int64_t grow_b = args.row0 + prow_b;
+  const int64_t q_b = q_row0 + wn * WTN + fr;
+  float rmax[16], rsum[16];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const f32x4 w4 = *reinterpret_cast<const f32x4*>(s_inv + row_b + g * 8);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int e = g * 4 + c;
+      float m = -INFINITY, t = 0.f;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const float v = acc_row[j][e] * w4[c];
+        acc_row[j][e] = v;  // kept for the dense scores and the candidate path
+        m = fmaxf(m, v);
+        t += v;
+      }
+      rmax[e] = m;
+      rsum[e] = t;
+    }
+  }
+  if (args.scores != nullptr) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        args.scores[(grow_b + (e >> 2) * 8 + (e & 3)) * args.Q + q_b + j * 32] = acc_row[j][e];
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    float cmax = acc_row[j][0];
+#pragma unroll
+    for (int e = 1; e < 16; ++e) cmax = fmaxf(cmax, acc_row[j][e]);
+    if (__builtin_expect(cmax > thr[j], 0)) {
+      const int64_t q = q_b + j * 32;
+      uint32_t* const cnt = args.cand_count + q;
+      uint64_t* const list = args.cand + q * args.cand_cap;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float v = acc_row[j][e];
+        if (v > thr[j]) {
+          const uint32_t pos = atomicAdd(cnt, 1u);
+          if ((int64_t)pos < args.cand_cap) list[pos] = make_key(v, (uint32_t)(grow_b + (e >> 2) * 8 + (e & 3)));
+        }
+      }
+    }
+  }
+  // this lane's row after the reductions: value (fr >> 1) & 15
+  const int e_mine = (fr >> 1) & 15;
+  const int dr_mine = (e_mine >> 2) * 8 + (e_mine & 3);
+  const bool writer = (fr & 1) == 0;
+  if (args.row_max_enc != nullptr) {
+    const float row_max = reduce16_half_wave<true>(rmax, fr);
+    if (writer) atomicMax(args.row_max_enc + grow_b + dr_mine, f32_ordered(row_max));
+  }
+  if (args.row_sum_part != nullptr) {
+    const float row_sum = reduce16_half_wave<false>(rsum, fr);
+    if (writer) args.row_sum_part[(prow_b + dr_mine) * args.n_parts + (qt * WN + wn)] = row_sum;
+  }
+}
+
 // The row blocks are taken by a pack expansion, not a loop: their indices are then constants whatever the
 // unroller decides, and the accumulators never need an address.  acc[i] is the wave's 32-row block
 // (i + block_rot) mod TM.
@@ -185,9 +297,17 @@ __device__ __forceinline__ void scan_tile_epilogue_blocks(const ScanArgs& args, 
                                                           const float (&thr)[TN], const float* s_inv, int wm, int wn,
                                                           int fr, int fh, int64_t g_row0, int64_t q_row0, int qt,
                                                           int block_rot, std::integer_sequence<int, Is...>) {
-  (scan_block_epilogue<TN, WTM, WTN, WN>(args, acc[Is], thr, s_inv, (Is + block_rot) % TM, wm, wn, fr, fh, g_row0,
-                                         q_row0, qt),
-   ...);
+  // whether every row and query of this wave's sub-tile exists (the same for all lanes of the wave)
+  const bool full = g_row0 + (wm + 1) * WTM <= args.rows && q_row0 + (wn + 1) * WTN <= args.Q;
+  if (full) {
+    (scan_block_epilogue_full<TN, WTM, WTN, WN>(args, acc[Is], thr, s_inv, (Is + block_rot) % TM, wm, wn, fr, fh,
+                                                g_row0, q_row0, qt),
+     ...);
+  } else {
+    (scan_block_epilogue<TN, WTM, WTN, WN>(args, acc[Is], thr, s_inv, (Is + block_rot) % TM, wm, wn, fr, fh, g_row0,
+                                           q_row0, qt),
+     ...);
+  }
 }
 
 template <int TM, int TN, int WTM, int WTN, int WN>
