@@ -11,7 +11,7 @@ from pathlib import Path
 LIB_PATH = Path(__file__).resolve().parent / "libbergson_amd.so"
 
 BGX_F32, BGX_F16, BGX_BF16 = 0, 1, 2
-ABI_VERSION = 8
+ABI_VERSION = 9
 STATIC_SCRATCH_BYTES = 16 << 20
 
 
@@ -128,6 +128,12 @@ SIGNATURES: dict[str, tuple] = {
     "bgx_scan_workspace_bytes": (C.c_size_t, [C.c_int32, C.c_int32, C.c_int64]),
     "bgx_scan_workspace_bytes_for": (C.c_size_t, [C.c_int32, C.c_int32, C.c_int64, C.c_int64, C.c_int32]),
     "bgx_scan": (
+        C.c_int,
+        [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_int32, C.c_float, C.c_int32,
+         C.c_int32, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+         C.c_size_t, C.c_int64, C.c_void_p],
+    ),
+    "bgx_scan_known_norms": (
         C.c_int,
         [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_int32, C.c_float, C.c_int32,
          C.c_int32, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,

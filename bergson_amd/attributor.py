@@ -99,6 +99,9 @@ class Attributor:
             free, _ = torch.cuda.mem_get_info(self.device)
             out_dtype = torch.float32 if self.store.numel() * 4 <= free // 2 else self.store.dtype
             self.store = self.preconditioner.apply_rows(self.store, self.grad_sizes, out_dtype=out_dtype)
+        # sums of squares of the store's rows, kept from the first unit-norm scan on: the reference normalises the
+        # index once at load time (attributor.py:137-167); here later scans take their row multipliers from this
+        self._row_sumsq: Tensor | None = None
 
     @property
     def grads(self) -> dict[str, Tensor]:
@@ -126,7 +129,11 @@ class Attributor:
         shift = 0 if qmax == 0 or not math.isfinite(qmax) else -math.frexp(qmax)[1]
         qd = (q * (2.0 ** shift)).to(self.store.dtype)
         if k <= ops.SCAN_KMAX:
-            res = ops.scan(self.store, qd, unit_norm=self.unit_norm, k=k, query_scale=2.0 ** (-shift))
+            first = self.unit_norm and self._row_sumsq is None
+            res = ops.scan(self.store, qd, unit_norm=self.unit_norm, k=k, query_scale=2.0 ** (-shift),
+                           want_sumsq=first, row_sumsq=self._row_sumsq)
+            if first:
+                self._row_sumsq = res.sumsq
             values, indices = res.topk_values, res.topk_indices
         else:
             # beyond the fused selection's capacity (k = None asks for a full ranking of the store): the

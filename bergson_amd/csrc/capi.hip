@@ -105,8 +105,8 @@ size_t scan_workspace_bytes(int Q, int k, int64_t chunk_rows);
 size_t scan_workspace_bytes_for(int Q, int k, int64_t chunk_rows, int64_t D, int dtype);
 int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int dtype, const void* queries, int Q,
               float query_scale, int unit_norm, int k, int64_t row_base, float* topk_val, int64_t* topk_idx,
-              float* row_max, float* row_mean, float* scores, float* sumsq, void* ws, size_t ws_bytes,
-              int64_t chunk_rows, void* stream);
+              float* row_max, float* row_mean, float* scores, float* sumsq, const float* sumsq_in, void* ws,
+              size_t ws_bytes, int64_t chunk_rows, void* stream);
 size_t precond_workspace_bytes(int n_blocks);
 int block_gemm_impl(const void* in, int in_dtype, int64_t in_stride, void* out, int out_dtype, int64_t out_stride,
                     int64_t rows, const bgx_block_desc* blocks, int n_blocks, void* ws, size_t ws_bytes,
@@ -281,8 +281,22 @@ int bgx_scan(const void* store_dev, int64_t n_rows, int64_t D, int64_t store_row
              float* topk_val_dev, int64_t* topk_idx_dev, float* row_max_dev, float* row_mean_dev, float* scores_dev,
              float* sumsq_dev, void* workspace_dev, size_t workspace_bytes, int64_t chunk_rows, void* stream) {
   return bgx::scan_impl(store_dev, n_rows, D, store_row_stride, dtype, queries_dev, Q, query_scale, unit_norm, k,
-                        row_base, topk_val_dev, topk_idx_dev, row_max_dev, row_mean_dev, scores_dev, sumsq_dev,
+                        row_base, topk_val_dev, topk_idx_dev, row_max_dev, row_mean_dev, scores_dev, sumsq_dev, nullptr,
                         workspace_dev, workspace_bytes, chunk_rows, stream);
+}
+
+int bgx_scan_known_norms(const void* store_dev, int64_t n_rows, int64_t D, int64_t store_row_stride, int32_t dtype,
+                         const void* queries_dev, int32_t Q, float query_scale, int32_t unit_norm, int32_t k,
+                         int64_t row_base, const float* row_sumsq_dev, float* topk_val_dev, int64_t* topk_idx_dev,
+                         float* row_max_dev, float* row_mean_dev, float* scores_dev, void* workspace_dev,
+                         size_t workspace_bytes, int64_t chunk_rows, void* stream) {
+  if (row_sumsq_dev == nullptr) {
+    bgx::set_error("scan_known_norms: null row_sumsq");
+    return BGX_E_ARG;
+  }
+  return bgx::scan_impl(store_dev, n_rows, D, store_row_stride, dtype, queries_dev, Q, query_scale, unit_norm, k,
+                        row_base, topk_val_dev, topk_idx_dev, row_max_dev, row_mean_dev, scores_dev, nullptr,
+                        row_sumsq_dev, workspace_dev, workspace_bytes, chunk_rows, stream);
 }
 
 }  // extern "C"

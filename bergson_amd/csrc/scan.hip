@@ -78,6 +78,7 @@ struct ScanArgs {
   // outputs / state (may be null)
   float* scores;         // [n_rows, Q]
   float* sumsq;          // [n_rows]
+  const float* sumsq_in; // [n_rows] row sums of squares from an earlier scan of the same store, or null
   uint32_t* row_max_enc; // [n_rows] ordered-uint encoding
   float* row_sum_part;   // [rows of this pass][n_parts] sum over each wave column's queries, or null
   int n_parts;           // q_tiles * (waves along the queries)
@@ -737,7 +738,7 @@ __device__ inline void sw_wait_lds() {  // s_waitcnt lgkmcnt(N), nothing else
   __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8));
 }
 
-template <typename T>
+template <typename T, bool NORMS_GIVEN>
 __global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
   using M = Mma32<T>;
   constexpr int BK = 64;
@@ -868,7 +869,7 @@ __global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
     for (int i = 0; i < TM; ++i) {
       if (i == 2) { sw_wait_lds<8>(); __builtin_amdgcn_sched_barrier(0); }
       if (i >= 3) { sw_wait_lds<9>(); __builtin_amdgcn_sched_barrier(0); }
-      if (i < 3) ss[i][KK] = M::sumsq(af[i], ss[i][KK]);
+      if (!NORMS_GIVEN && i < 3) ss[i][KK] = M::sumsq(af[i], ss[i][KK]);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
@@ -975,9 +976,10 @@ __global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
   for (int i = 0; i < 3; ++i) {
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) ss[i][kk] += __shfl_xor(ss[i][kk], 32);
-    const float ssq = (ss[i][0] + ss[i][1]) + (ss[i][2] + ss[i][3]);
+    float ssq = (ss[i][0] + ss[i][1]) + (ss[i][2] + ss[i][3]);
     if (fh == 0) {
       const int row = wm * WTM + (wn * 3 + i) * 32 + fr;
+      if (NORMS_GIVEN) ssq = g_row0 + row < args.rows ? args.sumsq_in[args.row0 + g_row0 + row] : 0.f;
       float w = args.query_scale;
       if (args.unit_norm) w = ssq > 0.f ? args.query_scale / sqrtf(ssq) : 0.f;
       s_inv[row] = w;
@@ -1522,7 +1524,7 @@ static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
         const int row_tiles_pad = (a.row_tiles + 7) / 8 * 8;
         a.q_tiles = (a.Q + SW_BN - 1) / SW_BN;
         a.n_parts = a.q_tiles * 2;
-        auto kern = scan_wide_kernel<T>;
+        auto kern = a.sumsq_in != nullptr ? scan_wide_kernel<T, true> : scan_wide_kernel<T, false>;
         BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SW_LDS_BYTES));
         hipLaunchKernelGGL(kern, dim3((unsigned)(row_tiles_pad * a.q_tiles)), dim3(SW_THREADS), SW_LDS_BYTES, st, a);
         BGX_HIP(hipGetLastError());
@@ -1584,6 +1586,7 @@ int gemm_scores(const void* rows, int64_t n_rows, int64_t D, int64_t stride, int
   a.unit_norm = 0;
   a.scores = scores;
   a.sumsq = nullptr;
+  a.sumsq_in = nullptr;
   a.row_max_enc = nullptr;
   a.row_sum_part = nullptr;
   a.n_parts = 0;
@@ -1604,8 +1607,8 @@ int gemm_scores(const void* rows, int64_t n_rows, int64_t D, int64_t stride, int
 
 int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int dtype, const void* queries, int Q,
               float query_scale, int unit_norm, int k, int64_t row_base, float* topk_val, int64_t* topk_idx,
-              float* row_max, float* row_mean, float* scores, float* sumsq, void* ws, size_t ws_bytes,
-              int64_t chunk_rows, void* stream) {
+              float* row_max, float* row_mean, float* scores, float* sumsq, const float* sumsq_in, void* ws,
+              size_t ws_bytes, int64_t chunk_rows, void* stream) {
   BGX_REQUIRE(store && queries, BGX_E_ARG, "scan: null store/queries");
   BGX_REQUIRE(n_rows > 0 && D > 0 && Q > 0 && stride >= D, BGX_E_ARG, "scan: n_rows=%lld D=%lld Q=%d stride=%lld",
               (long long)n_rows, (long long)D, Q, (long long)stride);
@@ -1706,6 +1709,7 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
     a.unit_norm = unit_norm;
     a.scores = scores;
     a.sumsq = sumsq;
+    a.sumsq_in = sumsq_in;
     a.row_max_enc = row_max_enc;
     a.row_sum_part = row_part;
     a.n_parts = 0;

@@ -615,8 +615,10 @@ class ScanResult:
 
 def scan(store: Tensor, queries: Tensor, *, unit_norm: bool, k: int = 0, query_scale: float = 1.0, row_base: int = 0,
          want_row_max: bool = False, want_row_mean: bool = False, want_scores: bool = False,
-         want_sumsq: bool = False, chunk_rows: int = 0) -> ScanResult:
-    """Score store rows [n, D] against queries [Q, D] (same dtype); see bgx_scan in include/bergson_amd.h."""
+         want_sumsq: bool = False, chunk_rows: int = 0, row_sumsq: Tensor | None = None) -> ScanResult:
+    """Score store rows [n, D] against queries [Q, D] (same dtype); see bgx_scan in include/bergson_amd.h.
+    `row_sumsq` [n] fp32: the `sumsq` of an earlier scan of the same rows (bgx_scan_known_norms): kernels then
+    leave the row norms out of their inner loops."""
     lib = _lib.load()
     _need_gpu(store, "store")
     _need_gpu(queries, "queries")
@@ -640,11 +642,24 @@ def scan(store: Tensor, queries: Tensor, *, unit_norm: bool, k: int = 0, query_s
         res.row_mean = torch.empty((n,), dtype=torch.float32, device=dev)
     if want_scores:
         res.scores = torch.empty((n, Q), dtype=torch.float32, device=dev)
-    if want_sumsq:
+    if want_sumsq and row_sumsq is None:
         res.sumsq = torch.empty((n,), dtype=torch.float32, device=dev)
     ws = None
     if k or want_row_mean or Q <= 32:  # few queries: the streaming kernel keeps its query fragments there
         ws = _workspace(dev, lib.bgx_scan_workspace_bytes_for(Q, k, chunk_rows, D, dtype_code(store.dtype)), "scan")
+    if row_sumsq is not None:
+        _need_gpu(row_sumsq, "row_sumsq")
+        if row_sumsq.dtype != torch.float32 or row_sumsq.shape != (n,) or not row_sumsq.is_contiguous():
+            raise ValueError("row_sumsq must be a contiguous fp32 vector with one entry per store row")
+        if want_sumsq:
+            res.sumsq = row_sumsq
+        rc = lib.bgx_scan_known_norms(_ptr(store), n, D, store.stride(0), dtype_code(store.dtype), _ptr(queries), Q,
+                                      query_scale, int(unit_norm), k, row_base, _ptr(row_sumsq),
+                                      _ptr(res.topk_values), _ptr(res.topk_indices), _ptr(res.row_max),
+                                      _ptr(res.row_mean), _ptr(res.scores), _ptr(ws), 0 if ws is None else ws.numel(),
+                                      chunk_rows, _stream())
+        _lib.check(rc, "bgx_scan_known_norms")
+        return res
     rc = lib.bgx_scan(_ptr(store), n, D, store.stride(0), dtype_code(store.dtype), _ptr(queries), Q, query_scale,
                       int(unit_norm), k, row_base, _ptr(res.topk_values), _ptr(res.topk_indices), _ptr(res.row_max),
                       _ptr(res.row_mean), _ptr(res.scores), _ptr(res.sumsq), _ptr(ws), 0 if ws is None else ws.numel(), chunk_rows,

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define BGX_ABI_VERSION 8
+#define BGX_ABI_VERSION 9
 
 enum bgx_dtype { BGX_F32 = 0, BGX_F16 = 1, BGX_BF16 = 2 };
 
@@ -363,6 +363,25 @@ int bgx_scan(const void* store_dev, int64_t n_rows, int64_t D,
              float* row_max_dev, float* row_mean_dev, float* scores_dev,
              float* sumsq_dev, void* workspace_dev, size_t workspace_bytes,
              int64_t chunk_rows, void* stream);
+
+/* bgx_scan for a store whose row sums of squares are known: row_sumsq_dev
+ * [n_rows] is the sumsq_dev output of an earlier bgx_scan of the same rows.
+ * The reference normalises an index once, when it loads it
+ * (query/attributor.py:137-167), and scores it many times; this is the same
+ * economy -- kernels that would otherwise sum the squares of every row in
+ * their inner loop leave that out and take the multiplier from the array
+ * (the 384 x 256 tile kernel for more than 256 queries; the other kernels
+ * compute the sums as before, which gives the same values).  Everything else
+ * as bgx_scan; there is no sumsq output. */
+int bgx_scan_known_norms(const void* store_dev, int64_t n_rows, int64_t D,
+                         int64_t store_row_stride, int32_t dtype,
+                         const void* queries_dev, int32_t Q, float query_scale,
+                         int32_t unit_norm, int32_t k, int64_t row_base,
+                         const float* row_sumsq_dev, float* topk_val_dev,
+                         int64_t* topk_idx_dev, float* row_max_dev,
+                         float* row_mean_dev, float* scores_dev,
+                         void* workspace_dev, size_t workspace_bytes,
+                         int64_t chunk_rows, void* stream);
 
 /* ---- dense per-module preconditioner --------------------------------------
  * One fp32 matrix h_dev [dim, dim] (row-major) per module; the module's values

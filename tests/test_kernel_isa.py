@@ -45,9 +45,10 @@ def scan_isa(isa):
     return isa["scan.hip"]
 
 
+@pytest.mark.parametrize("norms_given", [0, 1])
 @pytest.mark.parametrize("elem", ["5f16_t", "6bf16_t"])
-def test_wide_scan_kernel_keeps_its_fragments_in_registers(scan_isa, elem):
-    name = f"_ZN3bgx16scan_wide_kernelINS_{elem}EEEvNS_8ScanArgsE"
+def test_wide_scan_kernel_keeps_its_fragments_in_registers(scan_isa, elem, norms_given):
+    name = f"_ZN3bgx16scan_wide_kernelINS_{elem}ELb{norms_given}EEEvNS_8ScanArgsE"
     m = re.search(rf"^{name}:[^\n]*\n(.*?)\n\s*s_endpgm", scan_isa, re.S | re.M)
     assert m, f"{name} not found in the compiled code"
     lines = m.group(1).splitlines()

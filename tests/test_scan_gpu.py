@@ -346,3 +346,26 @@ def test_scan_wide_tiles_equal_the_256_tiles_bitwise(device, dtype, D, Q, bgx_en
     assert (wide.scores.cpu() - ref).abs().max().item() <= COS_TOL
     assert wide.scores[30_000].abs().max().item() == 0
     check_topk(wide.topk_values.cpu(), wide.topk_indices.cpu(), ref.T, k)
+
+
+def test_scan_with_known_row_norms_equals_the_plain_scan_bitwise(device):
+    """bgx_scan_known_norms: the row sums of squares of one scan handed to the next.  With more than 256 queries the
+    wide-tile kernel then leaves the norms out of its K loop; everything it reports is the same bits, and so it is
+    for query counts whose kernels ignore the array."""
+    from bergson_amd import ops
+
+    gen = torch.Generator().manual_seed(77)
+    n, D = 24576 + 8192 + 300, 256
+    store = torch.randn(n, D, generator=gen).to(torch.float16).to(device)
+    for Q in (1024, 300, 40):
+        q = torch.randn(Q, D, generator=gen).to(torch.float16).to(device)
+        plain = ops.scan(store, q, unit_norm=True, k=10, want_row_max=True, want_row_mean=True, want_sumsq=True)
+        known = ops.scan(store, q, unit_norm=True, k=10, want_row_max=True, want_row_mean=True,
+                         row_sumsq=plain.sumsq)
+        torch.cuda.synchronize()
+        assert torch.equal(plain.topk_values, known.topk_values)
+        assert torch.equal(plain.topk_indices, known.topk_indices)
+        assert torch.equal(plain.row_max, known.row_max)
+        assert torch.equal(plain.row_mean, known.row_mean)
+    with pytest.raises(ValueError):
+        ops.scan(store, q, unit_norm=True, k=10, row_sumsq=plain.sumsq[:-1])
