@@ -536,17 +536,20 @@ __global__ __launch_bounds__(512) void adam_fused_kernel(FusedArgs a) {
 // ---- fused path, tiles loaded straight into LDS ------------------------------------------------------------
 // The same computation as adam_fused_kernel with the store scan's direct-to-LDS pipeline (direct.hpp) and the
 // second pass fed from LDS as well:
-//  * eight waves as 8 x 1: a wave owns 32 tokens against all 256 table rows of the chunk (8 blocks of 32 x 32,
-//    128 accumulators); its half of nothing is added to another wave's, so there is no exchange at the end;
+//  * eight waves as 4 x 2: a wave owns 64 tokens against 128 table rows of the chunk (2 x 4 blocks of 32 x 32,
+//    128 accumulators), so that a K tile costs the workgroup 192 KB of fragment reads -- with 8 x 1 (every wave
+//    reading all 256 table rows) it was 288 KB, and together with the 64 KB the loads write that is more LDS time
+//    than the tile has MFMA time; the two waves that share tokens add their sums once, at the end;
 //  * one ring of tiles -- three row buffers, two operand buffers, 160 KB -- carries two kinds of tile: the K tiles
 //    of a chunk (256 tokens x 64 of I against 256 table rows x 64), and behind them four slices of the chunk's g
-//    values (256 tokens x 64 output features, whole 128-byte lines, in a row buffer) with the matching slice of L
+//    values (256 tokens x 2 x 32 output features: 32 from each half of the chunk, so that every wave has work on
+//    every slice; in a row buffer) with the matching slice of L
 //    (p rows x 64 features, in the operand buffer, which a g slice does not otherwise need).  The g values used to
 //    be fetched by the lanes that needed them, 32 bytes of 32 different lines per load instruction, and came
 //    through the L1 up to four times: with the path from L2 into the CU as the bound, a quarter of the kernel;
-//  * a g slice is four MFMAs per wave (H of two 32-feature blocks, scaled by g in registers, against L), its
-//    operands read from LDS with the K tiles' swizzle; nothing of the second pass touches global memory, and its
-//    loads travel two tiles ahead like all others;
+//  * a g slice is four MFMAs per wave (H of one 32-feature block for two token blocks, scaled by g in registers,
+//    against L), its operands read from LDS with the K tiles' swizzle; nothing of the second pass touches global
+//    memory, and its loads travel two tiles ahead like all others;
 //  * loads are uniform base + 32-bit lane offset (sw_load_lds16), fragment reads and waits are spelled out as in
 //    scan_direct_kernel.
 // Token tile x column mapping to workgroups (ttx), validity masking and the ptok layout are the old kernel's.
@@ -559,12 +562,13 @@ __global__ __launch_bounds__(512) void adam_fused_direct_kernel(FusedArgs a) {
   using M = Mma32<T>;
   static_assert(sizeof(T) == 2, "the fused Adam kernel is for 16-bit model dtypes");
   constexpr int BM = FUSED_TILE, BN = FUSED_TILE, BK = 64;
-  constexpr int TN = BN / 32;  // 8 table-row blocks per wave; one token block
+  constexpr int TM = 2, TN = 4;  // eight waves as 4 x 2: 64 tokens (two blocks) x 128 table rows (four blocks) per wave
   extern __shared__ __align__(128) unsigned char smem[];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
   const int fr = lane & 31;
   const int fh = lane >> 5;
   int tt = blockIdx.x, j = blockIdx.y;
@@ -597,15 +601,18 @@ __global__ __launch_bounds__(512) void adam_fused_direct_kernel(FusedArgs a) {
     const uint32_t ch = (uint32_t)((lane & 7) ^ sd_key(r)) * 16u;
     const uint32_t rc = (uint32_t)min(r, rows_here - 1);
     voff_a[i] = rc * a_row_bytes + ch;
-    voff_g[i] = rc * g_row_bytes + ch;
+    // a g slice takes 32 features from each half of the chunk (see g_slice): chunks 0 .. 3 of an LDS row are
+    // features 32 s .. of the chunk, chunks 4 .. 7 features 128 + 32 s ..
+    voff_g[i] = rc * g_row_bytes + (ch < 64u ? ch : ch + 192u);
     // table row that goes to LDS row r: bits (q1 q0 h c1 c0) -> (h q1 q0 c1 c0) within each block of 32, so that a
     // lane's 16 accumulators of a block are 16 consecutive output features (see adam_fused_kernel)
     const int pr = (r & ~31) | ((r & 4) << 2) | ((r & 24) >> 1) | (r & 3);
     voff_t[i] = (uint32_t)pr * t_row_bytes + ch;
   }
   // L slice: rows 0 .. 31 of the operand buffer, loaded by waves 0 .. 3 (8 rows each); rows past p repeat row p - 1
-  const uint32_t voff_l = (uint32_t)min((wave & 3) * 8 + (lane >> 3), p - 1) * l_row_bytes +
-                          (uint32_t)((lane & 7) ^ sd_key(wave * 8 + (lane >> 3))) * 16u;
+  const uint32_t ch_l = (uint32_t)((lane & 7) ^ sd_key(wave * 8 + (lane >> 3))) * 16u;
+  const uint32_t voff_l =
+      (uint32_t)min((wave & 3) * 8 + (lane >> 3), p - 1) * l_row_bytes + (ch_l < 64u ? ch_l : ch_l + 192u);
   const uint64_t act_base = (uint64_t)(uintptr_t)a.a + (uint64_t)t_row0 * a_row_bytes;
   const uint64_t g_base = (uint64_t)(uintptr_t)a.g + (uint64_t)(a.t0 + t_row0) * g_row_bytes;
   const uint64_t tab_base = (uint64_t)(uintptr_t)a.table + (uint64_t)j * O * t_row_bytes;
@@ -621,7 +628,7 @@ __global__ __launch_bounds__(512) void adam_fused_direct_kernel(FusedArgs a) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) sw_load_lds16(base, voff_a[i], dst + (uint32_t)i * 8192u);
     } else {
-      const uint64_t base = g_base + ((uint64_t)ld_a_chunk * BN + (uint64_t)(ld_a_pos - KT) * 64) * sizeof(T);
+      const uint64_t base = g_base + ((uint64_t)ld_a_chunk * BN + (uint64_t)(ld_a_pos - KT) * 32) * sizeof(T);
 #pragma unroll
       for (int i = 0; i < 4; ++i) sw_load_lds16(base, voff_g[i], dst + (uint32_t)i * 8192u);
     }
@@ -635,7 +642,7 @@ __global__ __launch_bounds__(512) void adam_fused_direct_kernel(FusedArgs a) {
     const bool is_k = ld_b_pos < KT;
     const uint64_t base =
         is_k ? tab_base + (uint64_t)ld_b_chunk * BN * t_row_bytes + (uint64_t)ld_b_pos * (BK * sizeof(T))
-             : l_base + ((uint64_t)ld_b_chunk * BN + (uint64_t)(ld_b_pos - KT) * 64) * sizeof(T);
+             : l_base + ((uint64_t)ld_b_chunk * BN + (uint64_t)(ld_b_pos - KT) * 32) * sizeof(T);
     // an L slice is 32 rows: instruction 0 of waves 0 .. 3 (the other waves fetch the same rows again into rows
     // 32 .. 63 of the buffer, which nothing reads: every wave then issues the same number of loads, and
     // "all but the youngest four" means the same thing to all of them)
@@ -651,40 +658,43 @@ __global__ __launch_bounds__(512) void adam_fused_direct_kernel(FusedArgs a) {
     }
   };
 
-  f32x16 pacc;
-  f32x16 acc[TN];
+  f32x16 pacc[TM];
+  f32x16 acc[TM][TN];
 #pragma unroll
-  for (int e = 0; e < 16; ++e) pacc[e] = 0.f;
+  for (int i = 0; i < TM; ++i) {
 #pragma unroll
-  for (int jj = 0; jj < TN; ++jj)
+    for (int e = 0; e < 16; ++e) pacc[i][e] = 0.f;
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[jj][e] = 0.f;
+    for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][jj][e] = 0.f;
+  }
 
-  // fragment reads: the wave's 32 token rows (one fragment per k-step) and all 256 table rows (eight)
+  // fragment reads per k-step: the wave's 64 token rows (two fragments) and its 128 table rows (four)
   const uint32_t key = (uint32_t)sd_key(fr);  // rows advance in steps of 32: the key depends on fr alone
-  const uint32_t a_frag = lds0 + (uint32_t)((wave * 32 + fr) * SD_ROW);
-  const uint32_t b_frag = lds0 + (uint32_t)(3 * FD_A_BYTES + fr * SD_ROW);
-  uint4 af[2], bf[2][TN];
+  const uint32_t a_frag = lds0 + (uint32_t)((wm * 64 + fr) * SD_ROW);
+  const uint32_t b_frag = lds0 + (uint32_t)(3 * FD_A_BYTES + (wn * 128 + fr) * SD_ROW);
+  uint4 af[2][TM], bf[2][TN];
   auto rd = [&](int t, auto kk_tag, auto set_tag) {
     constexpr int SET = decltype(set_tag)::value;
     constexpr int KK = decltype(kk_tag)::value;
     const uint32_t chk = (((uint32_t)(KK * 2 + fh)) ^ key) * 16u;
     const uint32_t ab = a_frag + (uint32_t)(t % 3) * FD_A_BYTES + chk;
     const uint32_t bb = b_frag + (uint32_t)(t & 1) * FD_B_BYTES + chk;
-    af[SET] = sd_lds_read16(ab);
+    af[SET][0] = sw_lds_read16<0 * 32 * SD_ROW>(ab);
+    af[SET][1] = sw_lds_read16<1 * 32 * SD_ROW>(ab);
     bf[SET][0] = sw_lds_read16<0 * 32 * SD_ROW>(bb);
     bf[SET][1] = sw_lds_read16<1 * 32 * SD_ROW>(bb);
     bf[SET][2] = sw_lds_read16<2 * 32 * SD_ROW>(bb);
     bf[SET][3] = sw_lds_read16<3 * 32 * SD_ROW>(bb);
-    bf[SET][4] = sw_lds_read16<4 * 32 * SD_ROW>(bb);
-    bf[SET][5] = sw_lds_read16<5 * 32 * SD_ROW>(bb);
-    bf[SET][6] = sw_lds_read16<6 * 32 * SD_ROW>(bb);
-    bf[SET][7] = sw_lds_read16<7 * 32 * SD_ROW>(bb);
   };
   auto mm = [&](auto set_tag) {
     constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
-    for (int jj = 0; jj < TN; ++jj) M::mma(bf[SET][jj], af[SET], acc[jj]);  // transposed block: rows = output features
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int jj = 0; jj < TN; ++jj)
+        M::mma(bf[SET][jj], af[SET][i], acc[i][jj]);  // transposed block: rows = output features
   };
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1>;
@@ -692,7 +702,7 @@ __global__ __launch_bounds__(512) void adam_fused_direct_kernel(FusedArgs a) {
   using K1 = std::integral_constant<int, 1>;
   using K2 = std::integral_constant<int, 2>;
   using K3 = std::integral_constant<int, 3>;
-  constexpr int WAIT_LDS_STEP = 0xC07F | ((1 + TN) << 8);  // lgkmcnt(9): the step issued before the latest nine reads
+  constexpr int WAIT_LDS_STEP = 0xC07F | ((TM + TN) << 8);  // lgkmcnt(6): the step issued before the latest six reads
   constexpr int WAIT_LDS_0 = 0xC07F;
 
   // prologue: tile 0 lands, its step 0 is read; tile 1's operands and tile 2's rows are under way
@@ -721,34 +731,37 @@ __global__ __launch_bounds__(512) void adam_fused_direct_kernel(FusedArgs a) {
       wg_barrier_lds<0>();
     __builtin_amdgcn_sched_barrier(0);
   };
-  // one g slice: pacc[t, i] += sum over its 64 features of (H[t, o] * g[t, o]) * L[i, o].  H of slice S is
-  // accumulator blocks 2 S and 2 S + 1; lane (fr, fh) holds token fr and features fh * 16 + e of a block, and takes
-  // them eight at a time (sp = 0, 1): 16-byte chunk 4 b + 2 fh + sp of the token's 128 bytes of g, and the same
-  // chunk of row fr of L.
+  // one g slice: pacc[t, i] += sum over its features of (H[t, o] * g[t, o]) * L[i, o].  Slice S is features
+  // 32 S .. 32 S + 31 of both halves of the chunk, i.e. accumulator block S of every wave, so that all eight waves
+  // work on every slice; the half of wave column wn sits in chunks 4 wn .. 4 wn + 3 of the LDS rows.  Lane (fr, fh)
+  // holds token fr and features fh * 16 + e of the block, and takes them eight at a time (sp = 0, 1): chunk
+  // 4 wn + 2 fh + sp of the token's row of g, and the same chunk of row fr of L.
   auto g_slice = [&](int t, auto s_tag) {
     constexpr int S = decltype(s_tag)::value;
     const uint32_t gb = a_frag + (uint32_t)(t % 3) * FD_A_BYTES;
-    const uint32_t lb = b_frag + (uint32_t)(t & 1) * FD_B_BYTES;
-    uint4 gq[4], lq[4];
+    const uint32_t lb = lds0 + (uint32_t)(3 * FD_A_BYTES + fr * SD_ROW) + (uint32_t)(t & 1) * FD_B_BYTES;
+    uint4 gq[TM][2], lq[2];
 #pragma unroll
-    for (int n = 0; n < 4; ++n) {
-      const uint32_t chk = (((uint32_t)((n >> 1) * 4 + fh * 2 + (n & 1))) ^ key) * 16u;
-      gq[n] = sd_lds_read16(gb + chk);
-      lq[n] = sd_lds_read16(lb + chk);
+    for (int sp = 0; sp < 2; ++sp) {
+      const uint32_t chk = (((uint32_t)(4 * wn + fh * 2 + sp)) ^ key) * 16u;
+      lq[sp] = sd_lds_read16(lb + chk);
+      gq[0][sp] = sw_lds_read16<0 * 32 * SD_ROW>(gb + chk);
+      gq[1][sp] = sw_lds_read16<1 * 32 * SD_ROW>(gb + chk);
     }
     __builtin_amdgcn_s_waitcnt(WAIT_LDS_0);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int n = 0; n < 4; ++n) {
-      const int sp = n & 1;
-      const f32x16& h = acc[2 * S + (n >> 1)];
-      uint4 zf;
-      zf.x = scaled_pair_bits<T>(h[8 * sp + 0], h[8 * sp + 1], gq[n].x);
-      zf.y = scaled_pair_bits<T>(h[8 * sp + 2], h[8 * sp + 3], gq[n].y);
-      zf.z = scaled_pair_bits<T>(h[8 * sp + 4], h[8 * sp + 5], gq[n].z);
-      zf.w = scaled_pair_bits<T>(h[8 * sp + 6], h[8 * sp + 7], gq[n].w);
-      M::mma(zf, lq[n], pacc);
-    }
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int sp = 0; sp < 2; ++sp) {
+        const f32x16& h = acc[i][S];
+        uint4 zf;
+        zf.x = scaled_pair_bits<T>(h[8 * sp + 0], h[8 * sp + 1], gq[i][sp].x);
+        zf.y = scaled_pair_bits<T>(h[8 * sp + 2], h[8 * sp + 3], gq[i][sp].y);
+        zf.z = scaled_pair_bits<T>(h[8 * sp + 4], h[8 * sp + 5], gq[i][sp].z);
+        zf.w = scaled_pair_bits<T>(h[8 * sp + 6], h[8 * sp + 7], gq[i][sp].w);
+        M::mma(zf, lq[sp], pacc[i]);
+      }
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -799,9 +812,11 @@ __global__ __launch_bounds__(512) void adam_fused_direct_kernel(FusedArgs a) {
     ++t;
     g_slice(t, std::integral_constant<int, 3>{});
 #pragma unroll
-    for (int jj = 0; jj < TN; ++jj)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) acc[jj][e] = 0.f;
+      for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][jj][e] = 0.f;
     __builtin_amdgcn_sched_barrier(0);
     tile_end_barrier(t);
     if (c + 1 < n_chunks) rd(t + 1, K0{}, S0{});
@@ -812,19 +827,36 @@ __global__ __launch_bounds__(512) void adam_fused_direct_kernel(FusedArgs a) {
   }
   __builtin_amdgcn_s_waitcnt(WAIT_LDS_0);
 
-  // pacc[e] = P[token (e>>2)*8 + fh*4 + (e&3) of this wave's 32][row fr], column j
+  // the two waves that share 64 tokens add their halves of the sum over the output features, in a fixed order,
+  // through the tile buffers (every wave is past its last fragment read behind the barrier)
+  float* red = reinterpret_cast<float*>(smem);
+  wg_barrier_lds<0>();
+  __builtin_amdgcn_sched_barrier(0);
+  if (wn == 1) {
 #pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const int tl = t_row0 + wave * 32 + (e >> 2) * 8 + fh * 4 + (e & 3);
-    if (tl < a.tokens && fr < p) {
-      bool valid = true;
-      if (a.lengths != nullptr) {
-        const int64_t t = a.t0 + tl;
-        const int n = (int)(t / a.S);
-        valid = (int)(t - (int64_t)n * a.S) < a.lengths[n] - 1;
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) red[((wm * TM + i) * 16 + e) * 64 + lane] = pacc[i][e];
+  }
+  __syncthreads();
+  if (wn == 0) {
+    // pacc[i][e] = P[token (e>>2)*8 + fh*4 + (e&3) of block i of this wave's 64][row fr], column j
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int tl = t_row0 + wm * 64 + i * 32 + (e >> 2) * 8 + fh * 4 + (e & 3);
+        if (tl < a.tokens && fr < p) {
+          bool valid = true;
+          if (a.lengths != nullptr) {
+            const int64_t t = a.t0 + tl;
+            const int n = (int)(t / a.S);
+            valid = (int)(t - (int64_t)n * a.S) < a.lengths[n] - 1;
+          }
+          const float v = pacc[i][e] + red[((wm * TM + i) * 16 + e) * 64 + lane];
+          a.ptok[(int64_t)tl * pp + fr * p + j] = valid ? v : 0.f;
+        }
       }
-      a.ptok[(int64_t)tl * pp + fr * p + j] = valid ? pacc[e] : 0.f;
-    }
   }
 }
 
