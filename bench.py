@@ -46,9 +46,9 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes moved per algorithmic byte by collect_kernel on this workload, from the FETCH_SIZE and
 # WRITE_SIZE hardware counters (profiles/collect_and_scan_kernels_pmc_hbm_traffic.txt)
 COLLECT_TRAFFIC_RATIO = 1.036
-# the same for the store scan: 1024 queries (four query tiles of 256 re-read each 384-row tile, most of it from the
-# L2 they share), at most 32 queries; and for per-token collection and the Llama-3-8B-shaped layers
-SCAN_TRAFFIC_RATIO_Q1024 = 1.39
+# the same for the store scan: 1024 queries (rows once; the 25 MB of queries once per round of 24 576 rows and XCD),
+# at most 32 queries; and for per-token collection and the Llama-3-8B-shaped layers
+SCAN_TRAFFIC_RATIO_Q1024 = 1.38
 SCAN_TRAFFIC_RATIO_FEW = 1.0016
 PER_TOKEN_TRAFFIC_RATIO = 1.030
 LLAMA_TRAFFIC_RATIO = 1.007
