@@ -693,15 +693,16 @@ __global__ __launch_bounds__(SD_THREADS) void scan_direct_kernel(ScanArgs args) 
 }
 
 // ---- many queries, many rows: 384 x 256 tiles on four waves ---------------------------------------------------
-// What bounds the 256 x 256 kernel above is the path from L2 into a compute unit: a CU keeps about 50-60 cache
-// lines in flight whatever is asked of it, i.e. ~16 B per cycle at the ~430 cycles an L2 request takes, and a
-// 256 x 256 tile needs 1/128 byte per flop.  The only lever left is fewer bytes per flop, and that is bounded by
-// the accumulators the register file can hold: this kernel gives one wave per SIMD all 512 registers (the
-// accumulators overflow into the AccVGPRs) -- four waves as 2 x 2, each 192 rows x 128 queries = 6 x 4 blocks of
-// 32 x 32 = 384 accumulator registers -- for a 384 x 256 tile: 1/153.6 byte per flop, 17 % less.  The tile's two
-// K tiles (2 x 80 KB) fill the LDS; with one wave per SIMD nothing else hides a stall, so every global load and
-// every fragment read is placed by hand between two MFMAs of the step before the one that needs it
-// (sched_barrier after each: the order below is the order that is executed).
+// With eight waves on a 256 x 256 tile a wave issues 32 MFMAs per K tile, and what it pays per tile beside them --
+// 24 fragment reads, the barrier, its share of the loads, the loop -- leaves the matrix pipes half idle.  This
+// kernel gives one wave per SIMD all 512 registers (the accumulators overflow into the AccVGPRs) -- four waves as
+// 2 x 2, each 192 rows x 128 queries = 6 x 4 blocks of 32 x 32 = 384 accumulator registers -- for a 384 x 256
+// tile: 96 MFMAs per wave and K tile against 40 fragment reads, and 1/153.6 byte per flop from L2 instead of
+// 1/128.  The tile's two K tiles (2 x 80 KB) fill the LDS; with one wave per SIMD nothing else hides a stall (a
+// vector-ALU instruction between two MFMAs costs its whole latency), so every global load and every fragment read
+// is placed by hand between two MFMAs of the step before the one that needs it (sched_barrier after each: the
+// order below is the order that is executed), and the loads of a tile go out right behind the barrier that
+// frees their stage, so that the youngest has most of a tile's time before the wait at the next barrier.
 //   LDS layout, swizzle, direct-to-LDS loads, explicit waits, row norms from the fragments: as in
 //   scan_direct_kernel, and the scores are the same bits (each is the same sequence of MFMAs over K).
 //   The launch covers whole tiles only: rows a multiple of 384 (the host cuts its passes accordingly; what is left
