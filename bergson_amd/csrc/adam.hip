@@ -860,6 +860,412 @@ __global__ __launch_bounds__(512) void adam_fused_direct_kernel(FusedArgs a) {
   }
 }
 
+// ---- fused path, one wave per SIMD ----------------------------------------------------------------------------
+// adam_fused_direct_kernel's computation and tile ring on four waves instead of eight.  With eight waves on a
+// 256 x 256 tile every wave reads 2 + 4 fragments per k-step, 192 KB per K tile and workgroup, and the loads
+// write another 64 KB: 2048 cycles of LDS time beside the 2048 cycles the tile's MFMAs take.  Four waves as 2 x 2
+// own 128 tokens x 128 table rows each (4 x 4 blocks of 32 x 32) and read 4 + 4 fragments per k-step, 128 KB per
+// tile.  The 256 accumulators of a wave are the AccVGPRs (MFMAs written as instructions, as in the store scan's
+// wide-tile kernel), pacc and everything else the ordinary registers; one wave per SIMD means nothing hides a
+// stall, so fragment reads and loads are placed by hand between the MFMAs:
+//  * a K tile is four k-steps of 16 MFMAs; the 8 fragment reads of the next step follow MFMAs 0 .. 7 of a step
+//    (into the other register set), and every step ends with a wait for them -- no read is in flight across a
+//    step boundary;
+//  * tile t's part of the load stream is "stage t": the 8 loads of operands(t + 2) and the 8 of rows(t + 3).
+//    Four of them go out behind the barrier of tile t, which sits after the fourth MFMA of its last k-step and
+//    frees the buffers they write; the other twelve are spread over tile t + 1, before its barrier.  That barrier
+//    waits for all but the youngest eight loads (rows(t + 3)), so operands(t + 2) and rows(t + 2) have landed;
+//  * every load instruction is a uniform 64-bit base + one per-lane offset that is the same for all eight
+//    instructions of a tile (instruction i fetches rows 32 i + 8 wave + lane / 8, and 32 rows on, the swizzle key
+//    and the permuted table row repeat): the kernel takes whole token tiles only;
+//  * past the end of the sequence the stream goes on fetching the last tile into the buffers whose turn it is
+//    (which nothing reads any more), so that the wait counts mean the same in every tile;
+//  * the first k-step of a chunk's first tile accumulates onto a literal zero, which saves clearing 256
+//    accumulators per chunk.
+// Token tile x column mapping (ttx), the second pass's operand layout and the ptok layout are the direct kernel's.
+constexpr int FW_THREADS = 256;
+
+template <typename T>
+__device__ inline void fw_mfma_zero(const uint4& a, const uint4& b, f32x16& c) {
+  typedef uint32_t raw4 __attribute__((ext_vector_type(4)));
+  const raw4 av = {a.x, a.y, a.z, a.w}, bv = {b.x, b.y, b.z, b.w};
+  if constexpr (std::is_same<T, f16_t>::value)
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=a"(c) : "v"(av), "v"(bv));
+  else
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(av), "v"(bv));
+}
+
+template <typename T>
+__device__ inline void fw_mfma_after_valu(const uint4& a, const uint4& b, f32x16& c) {
+  typedef uint32_t raw4 __attribute__((ext_vector_type(4)));
+  const raw4 av = {a.x, a.y, a.z, a.w}, bv = {b.x, b.y, b.z, b.w};
+  if constexpr (std::is_same<T, f16_t>::value)
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "v"(bv));
+  else
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "v"(bv));
+}
+
+template <int... Is, typename F>
+__device__ inline void fw_static_for(std::integer_sequence<int, Is...>, F&& f) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+
+template <typename T>
+__global__ __launch_bounds__(FW_THREADS) void adam_fused_wide_kernel(FusedArgs a) {
+  using M = Mma32<T>;
+  static_assert(sizeof(T) == 2, "the fused Adam kernel is for 16-bit model dtypes");
+  constexpr int BM = FUSED_TILE, BN = FUSED_TILE, BK = 64;
+  constexpr int TM = 4, TN = 4;
+  extern __shared__ __align__(128) unsigned char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int fr = lane & 31;
+  const int fh = lane >> 5;
+  int tt = blockIdx.x, j = blockIdx.y;
+  if (a.ttx > 0) {
+    const int b = blockIdx.x + gridDim.x * blockIdx.y;
+    const int xcd = b & 7, slot = b >> 3;
+    const int jx = 32 / a.ttx, n_super_tt = gridDim.x / a.ttx;
+    const int super = (slot >> 5) * 8 + xcd, within = slot & 31;
+    tt = (super % n_super_tt) * a.ttx + within % a.ttx;
+    j = (super / n_super_tt) * jx + within / a.ttx;
+  }
+  const int t_row0 = tt * BM;
+  const int p = a.p, O = a.O, pp = p * p;
+  const int KT = a.I / BK;  // at least 4 (host)
+  const int n_chunks = O / BN;
+  const int per_chunk = KT + FD_GSLICES;
+  const int total = per_chunk * n_chunks;
+
+  // ---- the load stream
+  const uint32_t a_row_bytes = (uint32_t)(a.a_tok_stride * sizeof(T));
+  const uint32_t g_row_bytes = (uint32_t)(a.g_tok_stride * sizeof(T));
+  const uint32_t t_row_bytes = (uint32_t)(a.I * sizeof(T));
+  const uint32_t l_row_bytes = (uint32_t)(O * sizeof(T));
+  const int rbase = wave * 8 + (lane >> 3);  // row of the first of a tile's eight load instructions
+  const uint32_t ch = (uint32_t)((lane & 7) ^ sd_key(rbase)) * 16u;
+  const uint32_t gch = ch < 64u ? ch : ch + 192u;  // a g / L slice is 32 features from each half of the chunk
+  const uint32_t v_act = (uint32_t)rbase * a_row_bytes + ch;
+  const uint32_t v_g = (uint32_t)rbase * g_row_bytes + gch;
+  // table row that goes to LDS row r: bits (q1 q0 h c1 c0) -> (h q1 q0 c1 c0) within each block of 32
+  const uint32_t v_tab = (uint32_t)(((rbase & 4) << 2) | ((rbase & 24) >> 1) | (rbase & 3)) * t_row_bytes + ch;
+  const uint32_t v_l = (uint32_t)min(rbase, p - 1) * l_row_bytes + gch;
+  const uint64_t act_base = (uint64_t)(uintptr_t)a.a + (uint64_t)t_row0 * a_row_bytes;
+  const uint64_t g_base = (uint64_t)(uintptr_t)a.g + (uint64_t)(a.t0 + t_row0) * g_row_bytes;
+  const uint64_t tab_base = (uint64_t)(uintptr_t)a.table + (uint64_t)j * O * t_row_bytes;
+  const uint64_t l_base = (uint64_t)(uintptr_t)a.r_out;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+  const uint32_t lds_wave = lds0 + (uint32_t)wave * 1024u;
+
+  // one tile's eight loads: base + i * step for the lanes' common offset, to dst + i * 4096.  Which tile a stage
+  // fetches follows from the place in the chunk, which is fixed where the stage is set up (set_* below), so a
+  // descriptor is a handful of scalar additions.
+  struct Desc {
+    uint64_t base;
+    uint32_t step, dst, voff;
+  };
+  Desc db, da;  // the stage under way: operands, then rows
+  uint32_t a_off = 0, b_off = 0;  // byte offsets of the current tile's buffers within their rings; the stage set up in
+                                  // tile t writes the buffers tile t has just left
+  const uint32_t k_step_tab = 32u * t_row_bytes, k_step_act = 32u * a_row_bytes, k_step_g = 32u * g_row_bytes;
+  auto set_b_k = [&](int chunk, int pos) {  // K tile `pos` of the table rows of `chunk`
+    db.base = tab_base + (uint64_t)chunk * BN * t_row_bytes + (uint64_t)pos * (BK * sizeof(T));
+    db.step = k_step_tab;
+    db.voff = v_tab;
+    db.dst = lds_wave + (uint32_t)(3 * FD_A_BYTES) + b_off;
+  };
+  auto set_b_l = [&](int chunk, int sl) {  // slice `sl` of L: 32 rows, fetched by all eight instructions (rows 32 .. of the buffer are never read)
+    db.base = l_base + ((uint64_t)chunk * BN + (uint64_t)sl * 32) * sizeof(T);
+    db.step = 0u;
+    db.voff = v_l;
+    db.dst = lds_wave + (uint32_t)(3 * FD_A_BYTES) + b_off;
+  };
+  auto set_a_k = [&](int pos) {
+    da.base = act_base + (uint64_t)pos * (BK * sizeof(T));
+    da.step = k_step_act;
+    da.voff = v_act;
+    da.dst = lds_wave + a_off;
+  };
+  auto set_a_g = [&](int chunk, int sl) {
+    da.base = g_base + ((uint64_t)chunk * BN + (uint64_t)sl * 32) * sizeof(T);
+    da.step = k_step_g;
+    da.voff = v_g;
+    da.dst = lds_wave + a_off;
+  };
+  auto issue = [&](auto n_tag) {  // load n of the stage: 0 .. 7 operands, 8 .. 15 rows
+    constexpr int N = decltype(n_tag)::value;
+    if constexpr (N < 8)
+      sw_load_lds16(db.base + (uint64_t)N * db.step, db.voff, db.dst + (uint32_t)N * 4096u);
+    else
+      sw_load_lds16(da.base + (uint64_t)(N - 8) * da.step, da.voff, da.dst + (uint32_t)(N - 8) * 4096u);
+  };
+
+  f32x16 pacc[TM];
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) pacc[i][e] = 0.f;
+
+  // ---- fragment reads: the wave's 128 token rows and its 128 table rows, four fragments each per k-step
+  const uint32_t key = (uint32_t)sd_key(fr);
+  const uint32_t a_frag = lds0 + (uint32_t)((wm * 128 + fr) * SD_ROW);
+  const uint32_t b_frag = lds0 + (uint32_t)(3 * FD_A_BYTES + (wn * 128 + fr) * SD_ROW);
+  uint32_t chk[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) chk[kk] = (((uint32_t)(kk * 2 + fh)) ^ key) * 16u;
+  uint4 af[2][TM], bf[2][TN];
+  // read n of a k-step's eight, in the order the MFMAs want them
+  auto rd_one = [&](uint32_t ab, uint32_t bb, auto set_tag, auto n_tag) {
+    constexpr int SET = decltype(set_tag)::value;
+    constexpr int N = decltype(n_tag)::value;
+    if constexpr (N == 0) bf[SET][0] = sw_lds_read16<0 * 32 * SD_ROW>(bb);
+    if constexpr (N == 1) af[SET][0] = sw_lds_read16<0 * 32 * SD_ROW>(ab);
+    if constexpr (N == 2) bf[SET][1] = sw_lds_read16<1 * 32 * SD_ROW>(bb);
+    if constexpr (N == 3) bf[SET][2] = sw_lds_read16<2 * 32 * SD_ROW>(bb);
+    if constexpr (N == 4) bf[SET][3] = sw_lds_read16<3 * 32 * SD_ROW>(bb);
+    if constexpr (N == 5) af[SET][1] = sw_lds_read16<1 * 32 * SD_ROW>(ab);
+    if constexpr (N == 6) af[SET][2] = sw_lds_read16<2 * 32 * SD_ROW>(ab);
+    if constexpr (N == 7) af[SET][3] = sw_lds_read16<3 * 32 * SD_ROW>(ab);
+  };
+  // MFMA n of a k-step: token block n / 4 against table block n % 4, transposed (rows = output features)
+  auto mfma_one = [&](auto set_tag, auto n_tag, auto zero_tag) {
+    constexpr int SET = decltype(set_tag)::value;
+    constexpr int N = decltype(n_tag)::value;
+    if constexpr (decltype(zero_tag)::value)
+      fw_mfma_zero<T>(bf[SET][N % 4], af[SET][N / 4], acc[N / 4][N % 4]);
+    else
+      sw_mfma<T, true>(bf[SET][N % 4], af[SET][N / 4], acc[N / 4][N % 4]);
+  };
+  using I16 = std::make_integer_sequence<int, 16>;
+  using I8 = std::make_integer_sequence<int, 8>;
+  using I4 = std::make_integer_sequence<int, 4>;
+  using TrueT = std::true_type;
+  using FalseT = std::false_type;
+  constexpr int WAIT_LDS_0 = 0xC07F;
+  auto next_offsets = [&](uint32_t& an, uint32_t& bn) {
+    an = a_off + FD_A_BYTES;
+    if (an == 3u * FD_A_BYTES) an = 0;
+    bn = b_off ^ (uint32_t)FD_B_BYTES;
+  };
+  // the tile's barrier: everything but the youngest eight loads (rows of the tile after next) has landed, for every
+  // wave; behind it this tile's buffers take the first loads of the next stage
+  auto tile_barrier = [&](auto&& set_stage) {
+    asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    set_stage();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // ---- one K tile.  FIRST: the chunk's first (accumulate onto zero); LAST: the chunk's last (a g slice follows, which
+  // reads its own operands)
+  auto k_tile = [&](auto first_tag, auto last_tag, auto&& set_stage) {
+    constexpr bool FIRST = decltype(first_tag)::value, LAST = decltype(last_tag)::value;
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    // k-steps 0 .. 2: MFMAs of the step, reads of the next one behind MFMAs 0 .. 7, four loads behind 8, 10, 12, 14
+    auto step = [&](auto cur_tag, auto nxt_tag, auto kk_tag, auto zero_tag) {
+      constexpr int KK = decltype(kk_tag)::value;  // the step that is read
+      const uint32_t ab = a_frag + a_off + chk[KK], bb = b_frag + b_off + chk[KK];
+      __builtin_amdgcn_sched_barrier(0);
+      fw_static_for(I16{}, [&](auto n) {
+        constexpr int N = decltype(n)::value;
+        mfma_one(cur_tag, n, zero_tag);
+        if constexpr (N < 8) rd_one(ab, bb, nxt_tag, n);
+        if constexpr (N >= 8 && N % 2 == 0) issue(std::integral_constant<int, 4 * KK + (N - 8) / 2>{});
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      __builtin_amdgcn_s_waitcnt(WAIT_LDS_0);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    step(S0{}, S1{}, std::integral_constant<int, 1>{}, std::integral_constant<bool, FIRST>{});
+    step(S1{}, S0{}, std::integral_constant<int, 2>{}, FalseT{});
+    step(S0{}, S1{}, std::integral_constant<int, 3>{}, FalseT{});
+    // k-step 3: the barrier behind the fourth MFMA, then the next tile's first reads and the next stage's first loads
+    uint32_t an, bn;
+    next_offsets(an, bn);
+    const uint32_t ab = a_frag + an + chk[0], bb = b_frag + bn + chk[0];
+    __builtin_amdgcn_sched_barrier(0);
+    fw_static_for(I16{}, [&](auto n) {
+      constexpr int N = decltype(n)::value;
+      mfma_one(S1{}, n, FalseT{});
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (N == 3) tile_barrier(set_stage);
+      if constexpr (!LAST && N >= 4 && N < 12) rd_one(ab, bb, S0{}, std::integral_constant<int, N - 4>{});
+      if constexpr (N >= 12) issue(std::integral_constant<int, N - 12>{});
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    __builtin_amdgcn_s_waitcnt(WAIT_LDS_0);
+    a_off = an;
+    b_off = bn;
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // ---- one g slice: pacc[t, i] += sum over its features of (H[t, o] * g[t, o]) * L[i, o].  Slice S is features
+  // 32 S .. 32 S + 31 of both halves of the chunk, i.e. accumulator block S of every wave; the half of wave column wn
+  // sits in chunks 4 wn .. 4 wn + 3 of the LDS rows.  Lane (fr, fh) holds token fr and features fh * 16 + e of the block
+  // and takes them eight at a time (sp = 0, 1): chunk 4 wn + 2 fh + sp of the token's row of g and of row fr of L.
+  auto g_slice = [&](auto s_tag, auto&& set_stage) {
+    constexpr int S = decltype(s_tag)::value;
+    const uint32_t gb = a_frag + a_off;
+    const uint32_t lb = lds0 + (uint32_t)(3 * FD_A_BYTES + fr * SD_ROW) + b_off;
+    uint4 gq[TM][2], lq[2];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int sp = 0; sp < 2; ++sp) {
+      const uint32_t c16 = (((uint32_t)(4 * wn + fh * 2 + sp)) ^ key) * 16u;
+      lq[sp] = sd_lds_read16(lb + c16);
+      gq[0][sp] = sw_lds_read16<0 * 32 * SD_ROW>(gb + c16);
+      gq[1][sp] = sw_lds_read16<1 * 32 * SD_ROW>(gb + c16);
+      gq[2][sp] = sw_lds_read16<2 * 32 * SD_ROW>(gb + c16);
+      gq[3][sp] = sw_lds_read16<3 * 32 * SD_ROW>(gb + c16);
+    }
+    issue(std::integral_constant<int, 4>{});
+    issue(std::integral_constant<int, 5>{});
+    __builtin_amdgcn_s_waitcnt(WAIT_LDS_0);
+    __builtin_amdgcn_sched_barrier(0);
+    fw_static_for(I8{}, [&](auto n) {
+      constexpr int N = decltype(n)::value;
+      constexpr int sp = N / 4, i = N % 4;
+      const f32x16& h = acc[i][S];
+      uint4 zf;
+      zf.x = scaled_pair_bits<T>(h[8 * sp + 0], h[8 * sp + 1], gq[i][sp].x);
+      zf.y = scaled_pair_bits<T>(h[8 * sp + 2], h[8 * sp + 3], gq[i][sp].y);
+      zf.z = scaled_pair_bits<T>(h[8 * sp + 4], h[8 * sp + 5], gq[i][sp].z);
+      zf.w = scaled_pair_bits<T>(h[8 * sp + 6], h[8 * sp + 7], gq[i][sp].w);
+      // pacc stays in the ordinary registers (left to the compiler it wanders between the two files, 16 moves a
+      // time), so this MFMA is an instruction too -- and it reads what vector instructions have just written, which
+      // the hardware does not interlock: two wait states in front of it (the compiler puts as many before its own)
+      fw_mfma_after_valu<T>(zf, lq[sp], pacc[i]);
+      if constexpr (N < 5) {
+        issue(std::integral_constant<int, 6 + 2 * N>{});
+        issue(std::integral_constant<int, 7 + 2 * N>{});
+      }
+    });
+    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");  // pacc's last MFMA has left the pipe before anything the compiler places reads it
+    __builtin_amdgcn_sched_barrier(0);
+    tile_barrier(set_stage);
+    fw_static_for(I4{}, [&](auto n) { issue(n); });
+    uint32_t an, bn;
+    next_offsets(an, bn);
+    a_off = an;
+    b_off = bn;
+    if constexpr (S == 3) {  // a K tile follows (after the last chunk: buffers that hold nothing anyone uses)
+      const uint32_t ab = a_frag + a_off + chk[0], bb = b_frag + b_off + chk[0];
+      fw_static_for(I8{}, [&](auto n) { rd_one(ab, bb, std::integral_constant<int, 0>{}, n); });
+      __builtin_amdgcn_s_waitcnt(WAIT_LDS_0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // ---- prologue: rows(0), operands(0), rows(1), then the first four loads of stage -1 = operands(1), rows(2)
+  set_a_k(0);
+  fw_static_for(I8{}, [&](auto n) { issue(std::integral_constant<int, 8 + decltype(n)::value>{}); });
+  set_b_k(0, 0);
+  fw_static_for(I8{}, [&](auto n) { issue(n); });
+  a_off = FD_A_BYTES;
+  set_a_k(1);
+  fw_static_for(I8{}, [&](auto n) { issue(std::integral_constant<int, 8 + decltype(n)::value>{}); });
+  a_off = 2 * FD_A_BYTES;
+  b_off = FD_B_BYTES;
+  set_b_k(0, 1);
+  set_a_k(2);
+  fw_static_for(I4{}, [&](auto n) { issue(n); });
+  a_off = 0;
+  b_off = 0;
+  asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");  // tile 0 has landed
+  __builtin_amdgcn_sched_barrier(0);
+  {
+    const uint32_t ab = a_frag + chk[0], bb = b_frag + chk[0];
+    fw_static_for(I8{}, [&](auto n) { rd_one(ab, bb, std::integral_constant<int, 0>{}, n); });
+    __builtin_amdgcn_s_waitcnt(WAIT_LDS_0);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  // A chunk is KT >= 4 K tiles and four g slices; the stage set up in the tile at place q fetches operands(q + 2) and
+  // rows(q + 3), and after the last chunk the stream fetches the last chunk's first tiles again, into buffers that
+  // nothing reads any more.
+  for (int c = 0; c < n_chunks; ++c) {
+    const int cn = c + 1 < n_chunks ? c + 1 : c;
+    k_tile(TrueT{}, FalseT{}, [&]() {
+      set_b_k(c, 2);
+      set_a_k(3);
+    });
+    for (int q = 1; q <= KT - 4; ++q)
+      k_tile(FalseT{}, FalseT{}, [&]() {
+        set_b_k(c, q + 2);
+        set_a_k(q + 3);
+      });
+    k_tile(FalseT{}, FalseT{}, [&]() {
+      set_b_k(c, KT - 1);
+      set_a_g(c, 0);
+    });
+    k_tile(FalseT{}, FalseT{}, [&]() {
+      set_b_l(c, 0);
+      set_a_g(c, 1);
+    });
+    k_tile(FalseT{}, TrueT{}, [&]() {
+      set_b_l(c, 1);
+      set_a_g(c, 2);
+    });
+    // the MFMAs above are instructions the compiler does not see through: their results are read (by instructions
+    // it places) no sooner than the last one has left the pipe
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    g_slice(std::integral_constant<int, 0>{}, [&]() {
+      set_b_l(c, 2);
+      set_a_g(c, 3);
+    });
+    g_slice(std::integral_constant<int, 1>{}, [&]() {
+      set_b_l(c, 3);
+      set_a_k(0);
+    });
+    g_slice(std::integral_constant<int, 2>{}, [&]() {
+      set_b_k(cn, 0);
+      set_a_k(1);
+    });
+    g_slice(std::integral_constant<int, 3>{}, [&]() {
+      set_b_k(cn, 1);
+      set_a_k(2);
+    });
+  }
+
+  // the two waves that share 128 tokens add their halves of the sum over the output features, in a fixed order,
+  // through the tile buffers (behind the barrier every load has landed and every wave is past its last read)
+  float* red = reinterpret_cast<float*>(smem);
+  wg_barrier_lds<0>();
+  __builtin_amdgcn_sched_barrier(0);
+  if (wn == 1) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) red[((wm * TM + i) * 16 + e) * 64 + lane] = pacc[i][e];
+  }
+  __syncthreads();
+  if (wn == 0) {
+    // pacc[i][e] = P[token (e>>2)*8 + fh*4 + (e&3) of block i of this wave's 128][row fr], column j
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int tl = t_row0 + wm * 128 + i * 32 + (e >> 2) * 8 + fh * 4 + (e & 3);
+        if (tl < a.tokens && fr < p) {
+          bool valid = true;
+          if (a.lengths != nullptr) {
+            const int64_t t = a.t0 + tl;
+            const int n = (int)(t / a.S);
+            valid = (int)(t - (int64_t)n * a.S) < a.lengths[n] - 1;
+          }
+          const float v = pacc[i][e] + red[((wm * TM + i) * 16 + e) * 64 + lane];
+          a.ptok[(int64_t)tl * pp + fr * p + j] = valid ? v : 0.f;
+        }
+      }
+  }
+}
+
 // per-token rows from ptok: clamp, cast, scatter to the rows of the valid tokens
 __global__ __launch_bounds__(256) void adam_tok_finalize_kernel(const float* __restrict__ ptok, int64_t t0, int tokens,
                                                                 int S, int pp, const int32_t* __restrict__ lengths,
@@ -1063,7 +1469,19 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
                           (int64_t)FUSED_TILE * a_tok_stride * 2 < ((int64_t)1 << 32) &&
                           (int64_t)FUSED_TILE * g_tok_stride * 2 < ((int64_t)1 << 32) &&
                           (int64_t)FUSED_TILE * I * 2 < ((int64_t)1 << 32) && (int64_t)p * O * 2 < ((int64_t)1 << 32);
-      if (direct) {
+      // one wave per SIMD: whole token tiles, at least four K tiles per chunk
+      const bool wide = direct && switches().adam_wide && rows_c % FUSED_TILE == 0 && I >= 256;
+      if (wide) {
+        if (dtype == BGX_F16) {
+          auto kern = adam_fused_wide_kernel<f16_t>;
+          BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, FD_LDS_BYTES));
+          hipLaunchKernelGGL(kern, grid, dim3(FW_THREADS), FD_LDS_BYTES, st, f);
+        } else {
+          auto kern = adam_fused_wide_kernel<bf16_t>;
+          BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, FD_LDS_BYTES));
+          hipLaunchKernelGGL(kern, grid, dim3(FW_THREADS), FD_LDS_BYTES, st, f);
+        }
+      } else if (direct) {
         if (dtype == BGX_F16) {
           auto kern = adam_fused_direct_kernel<f16_t>;
           BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, FD_LDS_BYTES));

@@ -7,6 +7,8 @@
 // consecutive rows conflict-free.
 #pragma once
 
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace bgx {
@@ -20,11 +22,13 @@ __device__ inline int sd_key(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 // clobber keeps the compiler from moving memory accesses across it.
 template <int VM_LEFT>
 __device__ inline void wg_barrier_lds() {
-  static_assert(VM_LEFT == 0 || VM_LEFT == 4, "spelled-out wait counts");
+  static_assert(VM_LEFT == 0 || VM_LEFT == 4 || VM_LEFT == 8, "spelled-out wait counts");
   if constexpr (VM_LEFT == 0)
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  else
+  else if constexpr (VM_LEFT == 4)
     asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  else
+    asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
 // 16 bytes from LDS byte address `addr`; the caller waits (lgkmcnt) before it uses the value
@@ -49,6 +53,27 @@ __device__ inline void sw_load_lds16(uint64_t base, uint32_t voff, uint32_t lds)
                :
                : "v"(voff), "s"(base), "s"(lds)
                : "memory", "m0");
+}
+
+// One 32 x 32 x 16 MFMA with the accumulator block pinned to the AccVGPRs (IN_ACC) or to the ordinary VGPRs.
+// Written as instructions: in kernels whose accumulators fill most of the register file (one wave per SIMD) the
+// register allocator has no slack, and left to itself it shuffles blocks between the two files and spills.  (Volatile: the statements
+// execute in the order they are written, which is the hand-made schedule.)
+template <typename T, bool IN_ACC>
+__device__ inline void sw_mfma(const uint4& a, const uint4& b, f32x16& c) {
+  typedef uint32_t raw4 __attribute__((ext_vector_type(4)));
+  const raw4 av = {a.x, a.y, a.z, a.w}, bv = {b.x, b.y, b.z, b.w};
+  if constexpr (std::is_same<T, f16_t>::value) {
+    if constexpr (IN_ACC)
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(av), "v"(bv));
+    else
+      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "v"(bv));
+  } else {
+    if constexpr (IN_ACC)
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(av), "v"(bv));
+    else
+      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "v"(bv));
+  }
 }
 
 }  // namespace bgx

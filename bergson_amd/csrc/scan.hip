@@ -713,27 +713,6 @@ constexpr int SW_LDS_BYTES = 2 * SW_STAGE;
 constexpr int64_t SW_ROUND_ROWS = 64 * SW_BM;  // rows of one round of the chip: 64 row tiles x 4 query tiles = 256 tiles
 constexpr int64_t SW_MIN_ROWS = 8192;          // shorter passes leave most of the chip idle whatever the tile
 
-// One 32 x 32 x 16 MFMA with the accumulator block pinned to the AccVGPRs (IN_ACC) or to the ordinary VGPRs.
-// Written as instructions: 384 accumulator registers beside 60 of fragments leave the register allocator no
-// slack, and left to itself it shuffles blocks between the two files and spills.  (Volatile: the statements
-// execute in the order they are written, which is the hand-made schedule.)
-template <typename T, bool IN_ACC>
-__device__ inline void sw_mfma(const uint4& a, const uint4& b, f32x16& c) {
-  typedef uint32_t raw4 __attribute__((ext_vector_type(4)));
-  const raw4 av = {a.x, a.y, a.z, a.w}, bv = {b.x, b.y, b.z, b.w};
-  if constexpr (std::is_same<T, f16_t>::value) {
-    if constexpr (IN_ACC)
-      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(av), "v"(bv));
-    else
-      asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "v"(bv));
-  } else {
-    if constexpr (IN_ACC)
-      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(av), "v"(bv));
-    else
-      asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(av), "v"(bv));
-  }
-}
-
 template <int N>
 __device__ inline void sw_wait_lds() {  // s_waitcnt lgkmcnt(N), nothing else
   __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8));
