@@ -470,7 +470,7 @@ def adam_leg(args, torch, device):
             "ms_per_layer": total_ms, "tokens_per_s_24_layers_hooks_only": N * S / (total_ms * 24e-3),
             "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": tf / MFMA_F16_PEAK_TFLOPS, "traffic": ADAM_TRAFFIC_BYTES_PER_LAYER,
-                         "kernel": "bgx::adam_fused_direct_kernel<bf16_t>"},
+                         "kernel": "bgx::adam_fused_wide_kernel<bf16_t>"},
             "modules": modules}
 
 

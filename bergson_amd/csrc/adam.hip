@@ -977,7 +977,7 @@ __global__ __launch_bounds__(FW_THREADS) void adam_fused_wide_kernel(FusedArgs a
     db.voff = v_tab;
     db.dst = lds_wave + (uint32_t)(3 * FD_A_BYTES) + b_off;
   };
-  auto set_b_l = [&](int chunk, int sl) {  // slice `sl` of L: 32 rows, fetched by all eight instructions (rows 32 .. of the buffer are never read)
+  auto set_b_l = [&](int chunk, int sl) {  // slice `sl` of L: 32 rows, one load instruction (issue() skips the other seven)
     db.base = l_base + ((uint64_t)chunk * BN + (uint64_t)sl * 32) * sizeof(T);
     db.step = 0u;
     db.voff = v_l;
@@ -995,11 +995,14 @@ __global__ __launch_bounds__(FW_THREADS) void adam_fused_wide_kernel(FusedArgs a
     da.voff = v_g;
     da.dst = lds_wave + a_off;
   };
-  auto issue = [&](auto n_tag) {  // load n of the stage: 0 .. 7 operands, 8 .. 15 rows
+  // load n of the stage: 0 .. 7 operands (an L slice has load 0 only: B_IS_L), 8 .. 15 rows
+  auto issue = [&](auto n_tag, auto b_is_l_tag) {
     constexpr int N = decltype(n_tag)::value;
-    if constexpr (N < 8)
-      sw_load_lds16(db.base + (uint64_t)N * db.step, db.voff, db.dst + (uint32_t)N * 4096u);
-    else
+    constexpr bool B_IS_L = decltype(b_is_l_tag)::value;
+    if constexpr (N < 8) {
+      if constexpr (!B_IS_L || N == 0)
+        sw_load_lds16(db.base + (uint64_t)N * db.step, db.voff, db.dst + (uint32_t)N * 4096u);
+    } else
       sw_load_lds16(da.base + (uint64_t)(N - 8) * da.step, da.voff, da.dst + (uint32_t)(N - 8) * 4096u);
   };
 
@@ -1061,8 +1064,8 @@ __global__ __launch_bounds__(FW_THREADS) void adam_fused_wide_kernel(FusedArgs a
   };
 
   // ---- one K tile.  FIRST: the chunk's first (accumulate onto zero); LAST: the chunk's last (a g slice follows, which
-  // reads its own operands)
-  auto k_tile = [&](auto first_tag, auto last_tag, auto&& set_stage) {
+  // reads its own operands); prevl / newl: the operands of the stage under way / of the stage set up here are a slice of L
+  auto k_tile = [&](auto first_tag, auto last_tag, auto prevl, auto newl, auto&& set_stage) {
     constexpr bool FIRST = decltype(first_tag)::value, LAST = decltype(last_tag)::value;
     using S0 = std::integral_constant<int, 0>;
     using S1 = std::integral_constant<int, 1>;
@@ -1075,7 +1078,7 @@ __global__ __launch_bounds__(FW_THREADS) void adam_fused_wide_kernel(FusedArgs a
         constexpr int N = decltype(n)::value;
         mfma_one(cur_tag, n, zero_tag);
         if constexpr (N < 8) rd_one(ab, bb, nxt_tag, n);
-        if constexpr (N >= 8 && N % 2 == 0) issue(std::integral_constant<int, 4 * KK + (N - 8) / 2>{});
+        if constexpr (N >= 8 && N % 2 == 0) issue(std::integral_constant<int, 4 * KK + (N - 8) / 2>{}, prevl);
         __builtin_amdgcn_sched_barrier(0);
       });
       __builtin_amdgcn_s_waitcnt(WAIT_LDS_0);
@@ -1095,7 +1098,7 @@ __global__ __launch_bounds__(FW_THREADS) void adam_fused_wide_kernel(FusedArgs a
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (N == 3) tile_barrier(set_stage);
       if constexpr (!LAST && N >= 4 && N < 12) rd_one(ab, bb, S0{}, std::integral_constant<int, N - 4>{});
-      if constexpr (N >= 12) issue(std::integral_constant<int, N - 12>{});
+      if constexpr (N >= 12) issue(std::integral_constant<int, N - 12>{}, newl);
       __builtin_amdgcn_sched_barrier(0);
     });
     __builtin_amdgcn_s_waitcnt(WAIT_LDS_0);
@@ -1108,7 +1111,7 @@ __global__ __launch_bounds__(FW_THREADS) void adam_fused_wide_kernel(FusedArgs a
   // 32 S .. 32 S + 31 of both halves of the chunk, i.e. accumulator block S of every wave; the half of wave column wn
   // sits in chunks 4 wn .. 4 wn + 3 of the LDS rows.  Lane (fr, fh) holds token fr and features fh * 16 + e of the block
   // and takes them eight at a time (sp = 0, 1): chunk 4 wn + 2 fh + sp of the token's row of g and of row fr of L.
-  auto g_slice = [&](auto s_tag, auto&& set_stage) {
+  auto g_slice = [&](auto s_tag, auto prevl, auto newl, auto&& set_stage) {
     constexpr int S = decltype(s_tag)::value;
     const uint32_t gb = a_frag + a_off;
     const uint32_t lb = lds0 + (uint32_t)(3 * FD_A_BYTES + fr * SD_ROW) + b_off;
@@ -1123,9 +1126,12 @@ __global__ __launch_bounds__(FW_THREADS) void adam_fused_wide_kernel(FusedArgs a
       gq[2][sp] = sw_lds_read16<2 * 32 * SD_ROW>(gb + c16);
       gq[3][sp] = sw_lds_read16<3 * 32 * SD_ROW>(gb + c16);
     }
-    issue(std::integral_constant<int, 4>{});
-    issue(std::integral_constant<int, 5>{});
+    issue(std::integral_constant<int, 4>{}, prevl);
+    issue(std::integral_constant<int, 5>{}, prevl);
     __builtin_amdgcn_s_waitcnt(WAIT_LDS_0);
+    uint32_t an, bn;
+    next_offsets(an, bn);
+    const uint32_t ab = a_frag + an + chk[0], bb = b_frag + bn + chk[0];  // the K tile behind slice 3
     __builtin_amdgcn_sched_barrier(0);
     fw_static_for(I8{}, [&](auto n) {
       constexpr int N = decltype(n)::value;
@@ -1140,40 +1146,43 @@ __global__ __launch_bounds__(FW_THREADS) void adam_fused_wide_kernel(FusedArgs a
       // time), so this MFMA is an instruction too -- and it reads what vector instructions have just written, which
       // the hardware does not interlock: two wait states in front of it (the compiler puts as many before its own)
       fw_mfma_after_valu<T>(zf, lq[sp], pacc[i]);
-      if constexpr (N < 5) {
-        issue(std::integral_constant<int, 6 + 2 * N>{});
-        issue(std::integral_constant<int, 7 + 2 * N>{});
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (N < 5) {  // the rest of the stage under way goes out before the barrier ...
+        issue(std::integral_constant<int, 6 + 2 * N>{}, prevl);
+        issue(std::integral_constant<int, 7 + 2 * N>{}, prevl);
       }
+      if constexpr (N == 5) {
+        // ... which sits here: the slice's operands were read at its start, the rest of it works from registers.  Behind
+        // it the first reads of the K tile that follows slice 3 (after the last chunk: of buffers that hold nothing
+        // anyone uses) and the next stage's first loads
+        tile_barrier(set_stage);
+        if constexpr (S == 3) fw_static_for(I8{}, [&](auto r) { rd_one(ab, bb, std::integral_constant<int, 0>{}, r); });
+      }
+      if constexpr (N >= 6) {
+        issue(std::integral_constant<int, 2 * (N - 6)>{}, newl);
+        issue(std::integral_constant<int, 2 * (N - 6) + 1>{}, newl);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     });
-    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");  // pacc's last MFMA has left the pipe before anything the compiler places reads it
-    __builtin_amdgcn_sched_barrier(0);
-    tile_barrier(set_stage);
-    fw_static_for(I4{}, [&](auto n) { issue(n); });
-    uint32_t an, bn;
-    next_offsets(an, bn);
     a_off = an;
     b_off = bn;
-    if constexpr (S == 3) {  // a K tile follows (after the last chunk: buffers that hold nothing anyone uses)
-      const uint32_t ab = a_frag + a_off + chk[0], bb = b_frag + b_off + chk[0];
-      fw_static_for(I8{}, [&](auto n) { rd_one(ab, bb, std::integral_constant<int, 0>{}, n); });
-      __builtin_amdgcn_s_waitcnt(WAIT_LDS_0);
-    }
+    __builtin_amdgcn_s_waitcnt(WAIT_LDS_0);
     __builtin_amdgcn_sched_barrier(0);
   };
 
   // ---- prologue: rows(0), operands(0), rows(1), then the first four loads of stage -1 = operands(1), rows(2)
   set_a_k(0);
-  fw_static_for(I8{}, [&](auto n) { issue(std::integral_constant<int, 8 + decltype(n)::value>{}); });
+  fw_static_for(I8{}, [&](auto n) { issue(std::integral_constant<int, 8 + decltype(n)::value>{}, FalseT{}); });
   set_b_k(0, 0);
-  fw_static_for(I8{}, [&](auto n) { issue(n); });
+  fw_static_for(I8{}, [&](auto n) { issue(n, FalseT{}); });
   a_off = FD_A_BYTES;
   set_a_k(1);
-  fw_static_for(I8{}, [&](auto n) { issue(std::integral_constant<int, 8 + decltype(n)::value>{}); });
+  fw_static_for(I8{}, [&](auto n) { issue(std::integral_constant<int, 8 + decltype(n)::value>{}, FalseT{}); });
   a_off = 2 * FD_A_BYTES;
   b_off = FD_B_BYTES;
   set_b_k(0, 1);
   set_a_k(2);
-  fw_static_for(I4{}, [&](auto n) { issue(n); });
+  fw_static_for(I4{}, [&](auto n) { issue(n, FalseT{}); });
   a_off = 0;
   b_off = 0;
   asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");  // tile 0 has landed
@@ -1190,24 +1199,24 @@ __global__ __launch_bounds__(FW_THREADS) void adam_fused_wide_kernel(FusedArgs a
   // nothing reads any more.
   for (int c = 0; c < n_chunks; ++c) {
     const int cn = c + 1 < n_chunks ? c + 1 : c;
-    k_tile(TrueT{}, FalseT{}, [&]() {
+    k_tile(TrueT{}, FalseT{}, FalseT{}, FalseT{}, [&]() {
       set_b_k(c, 2);
       set_a_k(3);
     });
     for (int q = 1; q <= KT - 4; ++q)
-      k_tile(FalseT{}, FalseT{}, [&]() {
+      k_tile(FalseT{}, FalseT{}, FalseT{}, FalseT{}, [&]() {
         set_b_k(c, q + 2);
         set_a_k(q + 3);
       });
-    k_tile(FalseT{}, FalseT{}, [&]() {
+    k_tile(FalseT{}, FalseT{}, FalseT{}, FalseT{}, [&]() {
       set_b_k(c, KT - 1);
       set_a_g(c, 0);
     });
-    k_tile(FalseT{}, FalseT{}, [&]() {
+    k_tile(FalseT{}, FalseT{}, FalseT{}, TrueT{}, [&]() {
       set_b_l(c, 0);
       set_a_g(c, 1);
     });
-    k_tile(FalseT{}, TrueT{}, [&]() {
+    k_tile(FalseT{}, TrueT{}, TrueT{}, TrueT{}, [&]() {
       set_b_l(c, 1);
       set_a_g(c, 2);
     });
@@ -1215,19 +1224,19 @@ __global__ __launch_bounds__(FW_THREADS) void adam_fused_wide_kernel(FusedArgs a
     // it places) no sooner than the last one has left the pipe
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
-    g_slice(std::integral_constant<int, 0>{}, [&]() {
+    g_slice(std::integral_constant<int, 0>{}, TrueT{}, TrueT{}, [&]() {
       set_b_l(c, 2);
       set_a_g(c, 3);
     });
-    g_slice(std::integral_constant<int, 1>{}, [&]() {
+    g_slice(std::integral_constant<int, 1>{}, TrueT{}, TrueT{}, [&]() {
       set_b_l(c, 3);
       set_a_k(0);
     });
-    g_slice(std::integral_constant<int, 2>{}, [&]() {
+    g_slice(std::integral_constant<int, 2>{}, TrueT{}, FalseT{}, [&]() {
       set_b_k(cn, 0);
       set_a_k(1);
     });
-    g_slice(std::integral_constant<int, 3>{}, [&]() {
+    g_slice(std::integral_constant<int, 3>{}, FalseT{}, FalseT{}, [&]() {
       set_b_k(cn, 1);
       set_a_k(2);
     });
@@ -1236,6 +1245,7 @@ __global__ __launch_bounds__(FW_THREADS) void adam_fused_wide_kernel(FusedArgs a
   // the two waves that share 128 tokens add their halves of the sum over the output features, in a fixed order,
   // through the tile buffers (behind the barrier every load has landed and every wave is past its last read)
   float* red = reinterpret_cast<float*>(smem);
+  asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");  // pacc's last MFMA has left the pipe before anything the compiler places reads it
   wg_barrier_lds<0>();
   __builtin_amdgcn_sched_barrier(0);
   if (wn == 1) {
@@ -1470,7 +1480,7 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
                           (int64_t)FUSED_TILE * g_tok_stride * 2 < ((int64_t)1 << 32) &&
                           (int64_t)FUSED_TILE * I * 2 < ((int64_t)1 << 32) && (int64_t)p * O * 2 < ((int64_t)1 << 32);
       // one wave per SIMD: whole token tiles, at least four K tiles per chunk
-      const bool wide = direct && switches().adam_wide && rows_c % FUSED_TILE == 0 && I >= 256;
+      const bool wide = direct && !switches().adam_wide_off && rows_c % FUSED_TILE == 0 && I >= 256;
       if (wide) {
         if (dtype == BGX_F16) {
           auto kern = adam_fused_wide_kernel<f16_t>;

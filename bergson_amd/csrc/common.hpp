@@ -33,7 +33,7 @@ int hip_fail(hipError_t e, const char* what);
 struct Switches {
   bool adam_fused_off = false;    // BGX_ADAM_FUSED_OFF set
   bool adam_direct_off = false;   // BGX_ADAM_DIRECT_OFF set
-  bool adam_wide = false;         // BGX_ADAM_WIDE set: four waves of 128 x 128 instead of eight of 64 x 128
+  bool adam_wide_off = false;     // BGX_ADAM_WIDE_OFF set: eight waves of 64 x 128 where four of 128 x 128 would run
   int adam_ttx = -1;              // BGX_ADAM_TTX (token tiles per XCD group), -1 = unset
   bool collect_staged = true;     // BGX_COLLECT_STAGED != "0"
   bool collect_persist = true;    // BGX_COLLECT_PERSIST != "0"

@@ -750,6 +750,41 @@ def test_adam_fused_xcd_order(device, ttx, bgx_env):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(1, 256, 256, 256, 32), (2, 512, 320, 512, 32), (1, 768, 1024, 768, 16),
+                                   (3, 256, 512, 1024, 8)])
+def test_adam_wide_tiles_equal_the_eight_wave_kernel_bitwise(device, dtype, shape, bgx_env):
+    """Whole 256-token tiles with I >= 256 run on four waves per workgroup (one per SIMD, 128 x 128 per wave); the
+    sums are formed in the same order as on eight waves, so the rows are the same bits.  Shapes: the smallest the
+    kernel takes (four K tiles, one chunk), a K count that is not a power of two, several chunks, p below 32,
+    ragged lengths; and against the oracle where that is quick."""
+    N, S, I, O, p = shape
+    case = _adam_case(N, S, I, O, p, dtype, seed=97)
+    a, g, left, right, norm = case
+    norm = ohooks.Adam(weight_avg_sq=norm.weight_avg_sq * 100 + 1e-6)
+    lengths = [S, max(2, S // 3), max(2, S - 41)][:N]
+    g = g.clone()
+    for n, l in enumerate(lengths):
+        g[n, l - 1:] = 0
+    case = (a, g, left, right, norm)
+    counts = [l - 1 for l in lengths]
+    offs = [sum(counts[:n]) for n in range(N)]
+    kw = dict(per_token=True, lengths=lengths, row_offsets=offs, n_rows=sum(counts))
+    got = _run_adam(device, case, p, dtype, **kw)
+    bgx_env("BGX_ADAM_WIDE_OFF", "1")
+    eight = _run_adam(device, case, p, dtype, **kw)
+    assert torch.equal(got, eight)
+    assert bool(torch.isfinite(got.float()).all())
+    if I * O * N * S <= 256 * 256 * 512:
+        mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+        want = ohooks.module_gradient(a, g, norm, left, right, attribute_tokens=True, collection_mask=mask)
+        assert rel_l2(got, want) <= TOL[dtype]
+    # per-sequence rows are sums of the same per-token results
+    seq = _run_adam(device, case, p, dtype)
+    bgx_env("BGX_ADAM_WIDE_OFF", None)
+    assert torch.equal(_run_adam(device, case, p, dtype), seq)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("shape", [(2, 700, 256, 512, 32), (1, 1024, 1024, 1024, 32), (3, 300, 192, 768, 16)])
 def test_adam_direct_tiles_against_register_staged_kernel(device, dtype, shape, bgx_env):
     """The fused Adam kernel whose operands all travel through LDS tiles loaded directly from global memory, on

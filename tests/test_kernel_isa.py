@@ -8,6 +8,12 @@ scratch memory before the read has arrived, or reuse a register that a read in f
 fragment read to the end of the tile loop there must be no scratch instruction, and the loop must be one copy
 (one loop header).  The other kernels that read their fragments this way (`scan_direct_kernel`,
 `adam_fused_direct_kernel`) have registers to spare; for them the check is that they use no scratch memory at all.
+`adam_fused_wide_kernel` runs one wave per SIMD like the wide scan kernel, with several copies of its tile code;
+it ends every k-step with a wait for its reads, so that no read is in flight where the copies meet, and the checks
+are: no scratch memory, no wait for all vector-memory loads between the first and the last matrix instruction (a
+scratch access or a table the compiler keeps in memory would bring one, and it would drain the load pipeline
+every tile), the accumulators never moved between the register files, and two wait states in front of every
+matrix instruction that reads what vector instructions have just written.
 hipcc cross-compiles without a GPU; the two compilations run side by side and take about a minute.
 """
 import re
@@ -80,3 +86,31 @@ def test_direct_to_lds_kernels_use_no_scratch(isa, source, pattern):
         assert "scratch_" not in m.group(1), f"{name} spills"
         meta = re.search(rf"\.amdhsa_kernel {re.escape(name)}\n(.*?)\.end_amdhsa_kernel", text, re.S)
         assert meta and re.search(r"\.amdhsa_private_segment_fixed_size 0\b", meta.group(1)), name
+
+
+@pytest.mark.parametrize("elem", ["5f16_t", "6bf16_t"])
+def test_wide_adam_kernel_keeps_its_pipeline(isa, elem):
+    name = f"_ZN3bgx22adam_fused_wide_kernelINS_{elem}EEEvNS_9FusedArgsE"
+    text = isa["adam.hip"]
+    m = re.search(rf"^{name}:[^\n]*\n(.*?)\n\s*s_endpgm", text, re.S | re.M)
+    assert m, f"{name} not found in the compiled code"
+    meta = re.search(rf"\.amdhsa_kernel {re.escape(name)}\n(.*?)\.end_amdhsa_kernel", text, re.S)
+    assert meta and re.search(r"\.amdhsa_private_segment_fixed_size 0\b", meta.group(1))
+    lines = [l.strip() for l in m.group(1).splitlines()]
+    lines = [l for l in lines if l and not l.startswith(";")]
+    assert not any("scratch_" in l for l in lines), "spills"
+    mfma = [i for i, l in enumerate(lines) if l.startswith("v_mfma_f32_32x32x16")]
+    body = lines[mfma[0]:mfma[-1] + 1]
+    # five copies of the K tile (64 each) and four g slices (8 each)
+    assert len(mfma) == 5 * 64 + 4 * 8
+    assert not any(re.match(r"s_waitcnt.*vmcnt\(0\)", l) for l in body), "a wait for every load inside the pipeline"
+    assert not any(re.search(r"\bs_load|s_buffer_load|flat_load|global_load_dword", l) for l in body), \
+        "memory reads other than the direct-to-LDS loads inside the pipeline"
+    assert not any(l.startswith(("v_accvgpr_write", "v_accvgpr_mov")) for l in body), "accumulators moved between the files"
+    # 256 accumulators are read once per chunk, 64 per slice
+    assert sum(l.startswith("v_accvgpr_read") for l in body) == 256
+    # the second pass's MFMAs (ordinary registers as destination) follow an s_nop 1
+    second = [i for i in mfma if re.match(r"v_mfma\S+ v\[", lines[i])]
+    assert len(second) == 32
+    for i in second:
+        assert lines[i - 1] == "s_nop 1", (lines[i - 2:i + 1])
