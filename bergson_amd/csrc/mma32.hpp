@@ -26,6 +26,13 @@ struct Mma32<f16_t> {
     s = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, v.w), __builtin_bit_cast(h2, v.w), s, false);
     return s;
   }
+  // the E-th of sumsq's four steps (the four in order give the same bits)
+  template <int E>
+  __device__ static float sumsq_part(const uint4& v, float s) {
+    typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+    const uint32_t w = E == 0 ? v.x : E == 1 ? v.y : E == 2 ? v.z : v.w;
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, w), __builtin_bit_cast(h2, w), s, false);
+  }
 };
 
 template <>
@@ -45,6 +52,14 @@ struct Mma32<bf16_t> {
       s = fmaf(hi, hi, s);
     }
     return s;
+  }
+  template <int E>
+  __device__ static float sumsq_part(const uint4& v, float s) {
+    const uint32_t w = E == 0 ? v.x : E == 1 ? v.y : E == 2 ? v.z : v.w;
+    const float lo = __uint_as_float(w << 16);
+    const float hi = __uint_as_float(w & 0xffff0000u);
+    s = fmaf(lo, lo, s);
+    return fmaf(hi, hi, s);
   }
 };
 

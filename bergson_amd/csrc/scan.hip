@@ -830,12 +830,18 @@ __global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
   // One k-step: the 24 MFMAs of step KK from query set SET; behind them, one at a time, the reads of the step
   // that follows (k-step NKK of stage `nstage`, query set 1 - SET) and whatever `side(n)` adds behind MFMA n.
   // LDS reads return in order, so "at most N outstanding" names the read that has arrived.  Issue order within a
-  // step: A0 B0 B1 B2 A1 B3 A2 A3 A4 A5 (behind MFMAs 3 4 5 6 7 8 11 15 19 23).
-  //   before MFMA 0:  A0, B0..B3, A1 of this step, i.e. all but the last four reads of the step before   -> 4
-  //   before MFMA 8:  A2; younger: A3 A4 A5 and this step's A0 B0 B1 B2 A1                                  -> 8
-  //   before MFMA 12: A3; younger: A4 A5, A0 B0 B1 B2 A1 B3 A2                                              -> 9
-  //   before MFMA 16: A4; younger: A5, A0 B0 B1 B2 A1 B3 A2 A3                                              -> 9
-  //   before MFMA 20: A5; younger: A0 B0 B1 B2 A1 B3 A2 A3 A4                                               -> 9
+  // step: B0 B1 B2 B3 A0 A1 A2 A3 A4 A5 (behind MFMAs 3 4 5 6 8 9 11 15 19 23).
+  //   before MFMA 0:  B0..B3, A0 of this step, i.e. all but the last five reads of the step before            -> 5
+  //   before MFMA 4:  A1; younger: A2 A3 A4 A5 and this step's B0                                            -> 5
+  //   before MFMA 8:  A2; younger: A3 A4 A5 and this step's B0 B1 B2 B3                                      -> 7
+  //   before MFMA 12: A3; younger: A4 A5, B0 B1 B2 B3 A0 A1 A2                                              -> 9
+  //   before MFMA 16: A4; younger: A5, B0 B1 B2 B3 A0 A1 A2 A3                                              -> 9
+  //   before MFMA 20: A5; younger: B0 B1 B2 B3 A0 A1 A2 A3 A4                                               -> 9
+  // Row blocks 0 and 1 are refilled only behind MFMAs 8 and 9 so that, just before MFMA 8, the fragments of the
+  // three blocks whose norms this wave sums are all in their registers: the twelve steps of the three sums of
+  // squares then run as four rounds of three independent instructions.  (Four dependent ones in front of each
+  // block's MFMAs wait for one another, and one behind each MFMA costs more still: with one wave per SIMD every
+  // switch from the matrix pipe to the vector pipe and back is paid for.)
   // `mid()` runs before the read behind MFMA 3 (the tile change puts its barrier there).  Every step is the same
   // code: the very last one reads a step that does not exist (whatever the other stage holds; never used).
   auto step = [&](auto set_tag, auto kk_tag, auto nkk_tag, int nstage, auto&& mid, auto&& side) {
@@ -843,13 +849,27 @@ __global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
     constexpr int KK = decltype(kk_tag)::value;
     using NK = decltype(nkk_tag);
     using NS = std::integral_constant<int, 1 - SET>;
-    sw_wait_lds<4>();
+    sw_wait_lds<5>();
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      if (i == 2) { sw_wait_lds<8>(); __builtin_amdgcn_sched_barrier(0); }
+      if (i == 1) { sw_wait_lds<5>(); __builtin_amdgcn_sched_barrier(0); }
+      if (i == 2) { sw_wait_lds<7>(); __builtin_amdgcn_sched_barrier(0); }
       if (i >= 3) { sw_wait_lds<9>(); __builtin_amdgcn_sched_barrier(0); }
-      if (!NORMS_GIVEN && i < 3) ss[i][KK] = M::sumsq(af[i], ss[i][KK]);
+      if (!NORMS_GIVEN && i == 2) {
+        ss[0][KK] = M::template sumsq_part<0>(af[0], ss[0][KK]);
+        ss[1][KK] = M::template sumsq_part<0>(af[1], ss[1][KK]);
+        ss[2][KK] = M::template sumsq_part<0>(af[2], ss[2][KK]);
+        ss[0][KK] = M::template sumsq_part<1>(af[0], ss[0][KK]);
+        ss[1][KK] = M::template sumsq_part<1>(af[1], ss[1][KK]);
+        ss[2][KK] = M::template sumsq_part<1>(af[2], ss[2][KK]);
+        ss[0][KK] = M::template sumsq_part<2>(af[0], ss[0][KK]);
+        ss[1][KK] = M::template sumsq_part<2>(af[1], ss[1][KK]);
+        ss[2][KK] = M::template sumsq_part<2>(af[2], ss[2][KK]);
+        ss[0][KK] = M::template sumsq_part<3>(af[0], ss[0][KK]);
+        ss[1][KK] = M::template sumsq_part<3>(af[1], ss[1][KK]);
+        ss[2][KK] = M::template sumsq_part<3>(af[2], ss[2][KK]);
+      }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
@@ -860,12 +880,12 @@ __global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
           sw_mfma<T, false>(af[i], bf[SET][j], acc[i][j]);
         __builtin_amdgcn_sched_barrier(0);
         if (n == 3) mid();
-        if (n == 3) { rd_base(nstage, NK{}); rd_a(I0{}); }
-        if (n == 4) rd_b(NS{}, I0{});
-        if (n == 5) rd_b(NS{}, I1{});
-        if (n == 6) rd_b(NS{}, I2{});
-        if (n == 7) rd_a(I1{});
-        if (n == 8) rd_b(NS{}, I3{});
+        if (n == 3) { rd_base(nstage, NK{}); rd_b(NS{}, I0{}); }
+        if (n == 4) rd_b(NS{}, I1{});
+        if (n == 5) rd_b(NS{}, I2{});
+        if (n == 6) rd_b(NS{}, I3{});
+        if (n == 8) rd_a(I0{});
+        if (n == 9) rd_a(I1{});
         if (n == 11) rd_a(I2{});
         if (n == 15) rd_a(I3{});
         if (n == 19) rd_a(I4{});
@@ -906,12 +926,12 @@ __global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
   wg_barrier_lds<0>();
   __builtin_amdgcn_sched_barrier(0);
   rd_base(0, K0{});
-  rd_a(I0{});
   rd_b(S0{}, I0{});
   rd_b(S0{}, I1{});
   rd_b(S0{}, I2{});
-  rd_a(I1{});
   rd_b(S0{}, I3{});
+  rd_a(I0{});
+  rd_a(I1{});
   rd_a(I2{});
   rd_a(I3{});
   rd_a(I4{});
