@@ -711,7 +711,7 @@ constexpr int SW_BM = 384, SW_BN = 256, SW_THREADS = 256;
 constexpr int SW_A_BYTES = SW_BM * SD_ROW, SW_B_BYTES = SW_BN * SD_ROW, SW_STAGE = SW_A_BYTES + SW_B_BYTES;
 constexpr int SW_LDS_BYTES = 2 * SW_STAGE;
 constexpr int64_t SW_ROUND_ROWS = 64 * SW_BM;  // rows of one round of the chip: 64 row tiles x 4 query tiles = 256 tiles
-constexpr int64_t SW_MIN_ROWS = 8192;          // shorter passes leave most of the chip idle whatever the tile
+constexpr int64_t SW_MIN_ROWS = 10240;         // shorter passes leave most of the chip idle whatever the tile
 
 template <int N>
 __device__ inline void sw_wait_lds() {  // s_waitcnt lgkmcnt(N), nothing else
@@ -1512,14 +1512,19 @@ template <typename T>
 static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
   // large tiles when there is enough work to fill the chip with them
   const int64_t big_tiles = ((a.rows + 255) / 256) * ((a.Q + 255) / 256);
-  if (a.Q > 64 && a.rows >= 256 && big_tiles >= 256) {
+  // (a pass the 384 x 256 tiles take is theirs even when it is less than a round of the chip: the last 12 864 rows
+  // of a million, 136 workgroups, take 0.62 ms there and 0.77 ms on the 128 x 64 tiles)
+  bool wide_pass = false;
+  if constexpr (sizeof(T) == 2)
+    wide_pass = wide_scan_ok(Elem<T>::code, aligned, a.D, a.store_stride, a.Q) && a.rows >= SW_MIN_ROWS;
+  if (a.Q > 64 && a.rows >= 256 && (big_tiles >= 256 || wide_pass)) {
     // 8 waves, each 128 x 64: two waves per SIMD hide each other's LDS and barrier stalls
     constexpr int BM = 256, BN = 256;
     a.row_tiles = (int)((a.rows + BM - 1) / BM);
     a.q_tiles = (a.Q + BN - 1) / BN;
     a.n_parts = a.q_tiles * 4;
     if constexpr (sizeof(T) == 2) {
-      if (wide_scan_ok(Elem<T>::code, aligned, a.D, a.store_stride, a.Q) && a.rows >= SW_MIN_ROWS) {
+      if (wide_pass) {
         a.row_tiles = (int)((a.rows + SW_BM - 1) / SW_BM);
         const int row_tiles_pad = (a.row_tiles + 7) / 8 * 8;
         a.q_tiles = (a.Q + SW_BN - 1) / SW_BN;
