@@ -48,7 +48,7 @@ HBM_PEAK_GBS = 8000.0
 COLLECT_TRAFFIC_RATIO = 1.036
 # the same for the store scan: 1024 queries (rows once; the 25 MB of queries once per round of 24 576 rows and XCD),
 # at most 32 queries; and for per-token collection and the Llama-3-8B-shaped layers
-SCAN_TRAFFIC_RATIO_Q1024 = 1.38
+SCAN_TRAFFIC_RATIO_Q1024 = 1.345
 SCAN_TRAFFIC_RATIO_FEW = 1.0016
 PER_TOKEN_TRAFFIC_RATIO = 1.030
 LLAMA_TRAFFIC_RATIO = 1.007
