@@ -751,12 +751,12 @@ def test_adam_fused_xcd_order(device, ttx, bgx_env):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("shape", [(1, 256, 256, 256, 32), (2, 512, 320, 512, 32), (1, 768, 1024, 768, 16),
-                                   (3, 256, 512, 1024, 8)])
+                                   (3, 256, 512, 1024, 8), (1, 256, 1024, 4096, 32), (1, 512, 4096, 1024, 32)])
 def test_adam_wide_tiles_equal_the_eight_wave_kernel_bitwise(device, dtype, shape, bgx_env):
     """Whole 256-token tiles with I >= 256 run on four waves per workgroup (one per SIMD, 128 x 128 per wave); the
     sums are formed in the same order as on eight waves, so the rows are the same bits.  Shapes: the smallest the
     kernel takes (four K tiles, one chunk), a K count that is not a power of two, several chunks, p below 32,
-    ragged lengths; and against the oracle where that is quick."""
+    ragged lengths, the widest modules of a Pythia-410m layer; and against the oracle where that is quick."""
     N, S, I, O, p = shape
     case = _adam_case(N, S, I, O, p, dtype, seed=97)
     a, g, left, right, norm = case
