@@ -53,7 +53,7 @@ SCAN_TRAFFIC_RATIO_FEW = 1.0016
 PER_TOKEN_TRAFFIC_RATIO = 1.030
 LLAMA_TRAFFIC_RATIO = 1.007
 # bytes the four fused Adam launches of one layer fetch through the L2s and write, from the same counters
-# (profiles/adam_fused_pythia410m_layer_p32.txt): 5.14 GB + 0.08 GB, against 0.94 GB read once each
+# (profiles/adam_fused_pythia410m_layer_p32.txt): 5.19 GB + 0.07 GB, against 0.94 GB read once each
 ADAM_TRAFFIC_BYTES_PER_LAYER = 5.26e9
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
