@@ -86,7 +86,7 @@ struct ScanArgs {
   uint32_t* cand_count;  // [Q]
   uint64_t* cand;        // [Q][cand_cap]
   int64_t cand_cap;
-  int first_pass;        // streaming kernel, no thresholds yet: row r of the pass is entry r of every query's list
+  int first_pass;        // no thresholds yet: row r of the pass is entry r of every query's list (streaming kernel, scan_gemm_kernel)
   int units_per_wave;    // streaming kernel: 16-row units per wave of the grid, the first units_rem waves one more
   int units_rem;
 };
@@ -115,7 +115,7 @@ __device__ __forceinline__ float reduce_half_wave(float v, float identity) {
 // ends up with a row's result touches memory, all addresses are a per-lane base plus constants, and the
 // candidate path (scores above a query's current k-th best: rare once the thresholds have settled) is entered
 // only by rows that have one.  thr[j] is +inf for queries past Q.
-template <int TN, int WTM, int WTN, int WN>
+template <int TN, int WTM, int WTN, int WN, bool FIRST_OK>
 __device__ __forceinline__ void scan_block_epilogue(const ScanArgs& args, f32x16 (&acc_row)[TN], const float (&thr)[TN],
                                                     const float* s_inv, int blk, int wm, int wn, int fr, int fh,
                                                     int64_t g_row0, int64_t q_row0, int qt) {
@@ -157,7 +157,16 @@ __device__ __forceinline__ void scan_block_epilogue(const ScanArgs& args, f32x16
         for (int j = 0; j < TN; ++j)
           if (q_ok[j]) args.scores[(grow_b + dr) * args.Q + q_b + j * 32] = v[j];
       }
-      if (any && row_ok) {
+      if (FIRST_OK && args.first_pass) {
+        // no thresholds yet: every score is a candidate, and row r of the pass is entry r of each query's list
+        // (one serialised atomic per score otherwise)
+        if (row_ok) {
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            if (q_ok[j])
+              args.cand[(q_b + j * 32) * args.cand_cap + prow_b + dr] = make_key(v[j], (uint32_t)(grow_b + dr));
+        }
+      } else if (any && row_ok) {
 #pragma unroll
         for (int j = 0; j < TN; ++j)
           if (v[j] > thr[j]) {
@@ -293,25 +302,27 @@ __device__ __forceinline__ void scan_block_epilogue_full(const ScanArgs& args, f
 // The row blocks are taken by a pack expansion, not a loop: their indices are then constants whatever the
 // unroller decides, and the accumulators never need an address.  acc[i] is the wave's 32-row block
 // (i + block_rot) mod TM.
-template <int TM, int TN, int WTM, int WTN, int WN, int... Is>
+template <int TM, int TN, int WTM, int WTN, int WN, bool FIRST_OK, int... Is>
 __device__ __forceinline__ void scan_tile_epilogue_blocks(const ScanArgs& args, f32x16 (&acc)[TM][TN],
                                                           const float (&thr)[TN], const float* s_inv, int wm, int wn,
                                                           int fr, int fh, int64_t g_row0, int64_t q_row0, int qt,
                                                           int block_rot, std::integer_sequence<int, Is...>) {
   // whether every row and query of this wave's sub-tile exists (the same for all lanes of the wave)
-  const bool full = g_row0 + (wm + 1) * WTM <= args.rows && q_row0 + (wn + 1) * WTN <= args.Q;
+  // (a first pass that writes its candidates by row number takes the general path: it is a few thousand rows)
+  const bool full = g_row0 + (wm + 1) * WTM <= args.rows && q_row0 + (wn + 1) * WTN <= args.Q &&
+                    !(FIRST_OK && args.first_pass);
   if (full) {
     (scan_block_epilogue_full<TN, WTM, WTN, WN>(args, acc[Is], thr, s_inv, (Is + block_rot) % TM, wm, wn, fr, fh,
                                                 g_row0, q_row0, qt),
      ...);
   } else {
-    (scan_block_epilogue<TN, WTM, WTN, WN>(args, acc[Is], thr, s_inv, (Is + block_rot) % TM, wm, wn, fr, fh, g_row0,
-                                           q_row0, qt),
+    (scan_block_epilogue<TN, WTM, WTN, WN, FIRST_OK>(args, acc[Is], thr, s_inv, (Is + block_rot) % TM, wm, wn, fr, fh,
+                                                     g_row0, q_row0, qt),
      ...);
   }
 }
 
-template <int TM, int TN, int WTM, int WTN, int WN>
+template <int TM, int TN, int WTM, int WTN, int WN, bool FIRST_OK = false>
 __device__ __forceinline__ void scan_tile_epilogue(const ScanArgs& args, f32x16 (&acc)[TM][TN], const float* s_inv,
                                                    int wm, int wn, int fr, int fh, int64_t g_row0, int64_t q_row0,
                                                    int qt, int block_rot = 0) {
@@ -321,8 +332,8 @@ __device__ __forceinline__ void scan_tile_epilogue(const ScanArgs& args, f32x16 
     const int64_t q = q_row0 + wn * WTN + j * 32 + fr;
     thr[j] = (args.thr != nullptr && q < args.Q) ? args.thr[q] : INFINITY;
   }
-  scan_tile_epilogue_blocks<TM, TN, WTM, WTN, WN>(args, acc, thr, s_inv, wm, wn, fr, fh, g_row0, q_row0, qt, block_rot,
-                                                  std::make_integer_sequence<int, TM>{});
+  scan_tile_epilogue_blocks<TM, TN, WTM, WTN, WN, FIRST_OK>(args, acc, thr, s_inv, wm, wn, fr, fh, g_row0, q_row0, qt,
+                                                            block_rot, std::make_integer_sequence<int, TM>{});
 }
 
 // Workgroup tile BM x BN, WM x WN waves, each wave (BM/WM) x (BN/WN) as 32x32 MFMA blocks.
@@ -478,7 +489,9 @@ __global__ __launch_bounds__(WM* WN * 64) void scan_gemm_kernel(ScanArgs args) {
   }
   __syncthreads();
 
-  scan_tile_epilogue<TM, TN, WTM, WTN, WN>(args, acc, s_inv, wm, wn, fr, fh, g_row0, q_row0, qt);
+  if (args.first_pass && blockIdx.x == 0)
+    for (int q = tid; q < args.Q; q += NT) args.cand_count[q] = (uint32_t)args.rows;
+  scan_tile_epilogue<TM, TN, WTM, WTN, WN, true>(args, acc, s_inv, wm, wn, fr, fh, g_row0, q_row0, qt);
 }
 
 // ---- many queries, 16-bit stores: tiles loaded straight into LDS ---------------------------------------
@@ -1746,12 +1759,14 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
       rc = dtype == BGX_F16    ? launch_stream<f16_t>(a, blocks, qtable, wgs, st)
            : dtype == BGX_BF16 ? launch_stream<bf16_t>(a, blocks, qtable, wgs, st)
                                : launch_stream<float>(a, blocks, qtable, wgs, st);
-    } else if (dtype == BGX_F16)
-      rc = launch_gemm_t<f16_t>(a, aligned, st);
-    else if (dtype == BGX_BF16)
-      rc = launch_gemm_t<bf16_t>(a, aligned, st);
-    else
-      rc = launch_gemm_t<float>(a, aligned, st);
+    } else {
+      // (honoured by scan_gemm_kernel, which takes the short first pass; the other tile kernels let every score of
+      // a pass without thresholds through their candidate filter instead, with the same result)
+      a.first_pass = want_topk && done == 0;
+      rc = dtype == BGX_F16    ? launch_gemm_t<f16_t>(a, aligned, st)
+           : dtype == BGX_BF16 ? launch_gemm_t<bf16_t>(a, aligned, st)
+                               : launch_gemm_t<float>(a, aligned, st);
+    }
     if (rc != 0) return rc;
     if (row_part != nullptr) {
       hipLaunchKernelGGL(scan_row_mean_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, row_part,
