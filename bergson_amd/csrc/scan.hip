@@ -1179,15 +1179,17 @@ struct SelectArgs {
   int k;
 };
 
-constexpr int SELECT_THREADS = 1024;
+// Threads per query: 1024 behind a pass without thresholds (one candidate per row), 256 behind the others, whose
+// lists are a few hundred entries -- the selection is some fifty workgroup barriers, and those cost by the wave.
+constexpr int SELECT_THREADS_LONG = 1024, SELECT_THREADS_SHORT = 256;
 constexpr uint32_t SELECT_SAMPLE = 4096;                     // > SCAN_KMAX
 constexpr uint32_t SELECT_PRESELECT_MIN = 4 * SELECT_SAMPLE;  // shorter lists go to the exact selection directly
-constexpr int SELECT_COMPACT_U = 4;                           // keys per thread and compaction step
+constexpr int SELECT_COMPACT_KEYS = 4096;                     // keys per compaction step: 64 (sub-block, wave) pairs
 
 struct SelectShared {
   uint64_t keys[SCAN_KMAX];
   uint32_t hist[256];
-  uint32_t part[SELECT_COMPACT_U * SELECT_THREADS / 64 + 1];  // compaction: per (sub-block, wave) counts, then offsets
+  uint32_t part[SELECT_COMPACT_KEYS / 64 + 1];  // compaction: per (sub-block, wave) counts, then offsets
   uint64_t prefix;
   uint32_t rank;
   uint32_t fill;
@@ -1195,7 +1197,7 @@ struct SelectShared {
 
 // The rank-th largest (rank from 1, rank <= n) of the n keys elem(0..n-1): radix select, 8 bits per pass from
 // the top.  Every thread of the workgroup calls it.
-template <typename F>
+template <int THREADS, typename F>
 __device__ uint64_t radix_kth(F elem, uint32_t n, uint32_t rank, SelectShared& sh) {
   const int tid = threadIdx.x;
   if (tid == 0) {
@@ -1208,7 +1210,7 @@ __device__ uint64_t radix_kth(F elem, uint32_t n, uint32_t rank, SelectShared& s
     __syncthreads();
     const uint64_t prefix = sh.prefix;
     const uint64_t mask = shift == 56 ? 0ull : (~0ull << (shift + 8));
-    for (uint32_t i = tid; i < n; i += SELECT_THREADS) {
+    for (uint32_t i = tid; i < n; i += THREADS) {
       const uint64_t key = elem(i);
       if ((key & mask) == prefix) atomicAdd(&sh.hist[(uint32_t)(key >> shift) & 255u], 1u);
     }
@@ -1255,7 +1257,10 @@ __device__ uint64_t radix_kth(F elem, uint32_t n, uint32_t rank, SelectShared& s
 // Merges each query's candidate list into its running top-k.  A long list (a pass without a threshold
 // leaves one entry per row) is first cut down in place: the k-th largest of a strided sample of it is a
 // lower bound of the k-th largest overall, and only entries at or above that bound stay.
-__global__ __launch_bounds__(SELECT_THREADS) void scan_select_kernel(SelectArgs a) {
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void scan_select_kernel(SelectArgs a) {
+  constexpr int SELECT_THREADS = THREADS;
+  constexpr int SELECT_COMPACT_U = SELECT_COMPACT_KEYS / THREADS;
   __shared__ SelectShared sh;
 
   const int q = blockIdx.x;
@@ -1273,7 +1278,7 @@ __global__ __launch_bounds__(SELECT_THREADS) void scan_select_kernel(SelectArgs 
   if (ncand >= SELECT_PRESELECT_MIN) {
     const uint32_t step = ncand / SELECT_SAMPLE;
     const uint64_t bound =
-        radix_kth([&](uint32_t i) -> uint64_t { return cand[(uint64_t)i * step]; }, SELECT_SAMPLE, (uint32_t)k, sh);
+        radix_kth<THREADS>([&](uint32_t i) -> uint64_t { return cand[(uint64_t)i * step]; }, SELECT_SAMPLE, (uint32_t)k, sh);
     // order-preserving compaction in place: a step reads SELECT_COMPACT_U * SELECT_THREADS entries, and writes
     // its survivors only after every thread has read, at positions no later step reads from
     constexpr int NW = SELECT_THREADS / 64;
@@ -1320,13 +1325,13 @@ __global__ __launch_bounds__(SELECT_THREADS) void scan_select_kernel(SelectArgs 
     __syncthreads();
     ncand = w_base;
   }
-  static_assert(SELECT_COMPACT_U * SELECT_THREADS / 64 == 64, "the compaction's offsets are one wave's prefix sum");
+  static_assert(SELECT_COMPACT_U * SELECT_THREADS / 64 == 64 && THREADS >= 256, "the compaction's offsets are one wave's prefix sum");
 
   const uint32_t total = ntop + ncand;
   auto elem = [&](uint32_t i) -> uint64_t { return i < ntop ? top[i] : cand[i - ntop]; };
 
   uint64_t kth = 0;  // keep keys >= kth
-  if (total > (uint32_t)k) kth = radix_kth(elem, total, (uint32_t)k, sh);
+  if (total > (uint32_t)k) kth = radix_kth<THREADS>(elem, total, (uint32_t)k, sh);
 
   if (tid == 0) sh.fill = 0;
   __syncthreads();
@@ -1782,7 +1787,10 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
       s.thr = thr;
       s.cand_cap = chunk;
       s.k = k;
-      hipLaunchKernelGGL(scan_select_kernel, dim3((unsigned)Q), dim3(SELECT_THREADS), 0, st, s);
+      if (a.first_pass)
+        hipLaunchKernelGGL(scan_select_kernel<SELECT_THREADS_LONG>, dim3((unsigned)Q), dim3(SELECT_THREADS_LONG), 0, st, s);
+      else
+        hipLaunchKernelGGL(scan_select_kernel<SELECT_THREADS_SHORT>, dim3((unsigned)Q), dim3(SELECT_THREADS_SHORT), 0, st, s);
       BGX_HIP(hipGetLastError());
     }
     done += rows;
