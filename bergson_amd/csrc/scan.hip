@@ -723,7 +723,13 @@ __global__ __launch_bounds__(SD_THREADS) void scan_direct_kernel(ScanArgs args) 
 constexpr int SW_BM = 384, SW_BN = 256, SW_THREADS = 256;
 constexpr int SW_A_BYTES = SW_BM * SD_ROW, SW_B_BYTES = SW_BN * SD_ROW, SW_STAGE = SW_A_BYTES + SW_B_BYTES;
 constexpr int SW_LDS_BYTES = 2 * SW_STAGE;
-constexpr int64_t SW_ROUND_ROWS = 64 * SW_BM;  // rows of one round of the chip: 64 row tiles x 4 query tiles = 256 tiles
+// Rows of one round of the chip -- 256 workgroups, one per compute unit: 256 / (query tiles) row tiles.  24 576 rows
+// at 1024 queries (64 row tiles x 4 query tiles), 98 304 with one query tile.
+static int64_t sw_round_rows(int Q) {
+  const int q_tiles = (Q + SW_BN - 1) / SW_BN;
+  const int row_tiles = 256 / q_tiles;
+  return (int64_t)(row_tiles > 0 ? row_tiles : 1) * SW_BM;
+}
 constexpr int64_t SW_MIN_ROWS = 10240;         // shorter passes leave most of the chip idle whatever the tile
 
 template <int N>
@@ -1437,11 +1443,12 @@ static ScanLayout scan_layout(int Q, int k, int64_t chunk_rows) {
 // default keeps Q * chunk near 64 Mi entries (512 MB) -- 65536 rows at 1024 queries, more for fewer.
 static int64_t effective_chunk(int64_t chunk_rows, int Q) {
   if (chunk_rows > 0) return chunk_rows;
-  if (Q > SW_BN) {
-    // many queries: whole rounds of the 384 x 256 tile kernel (24 576 rows each), Q * chunk near 96 Mi entries --
-    // 98 304 rows at 1024 queries
-    const int64_t c = ((int64_t)96 << 20) / Q / SW_ROUND_ROWS * SW_ROUND_ROWS;
-    if (c >= SW_ROUND_ROWS) return c;
+  if (Q > SW_BN / 2) {
+    // many queries: whole rounds of the 384 x 256 tile kernel, Q * chunk near 96 Mi entries -- 98 304 rows (four
+    // rounds) at 1024 queries, 393 216 (four rounds) at 256
+    const int64_t round = sw_round_rows(Q);
+    const int64_t c = ((int64_t)96 << 20) / Q / round * round;
+    if (c >= round) return c;
   }
   int64_t c = ((int64_t)64 << 20) / (Q > 0 ? Q : 1);
   if (c > ((int64_t)1 << 20)) c = (int64_t)1 << 20;
@@ -1522,7 +1529,7 @@ static int launch_gemm(const ScanArgs& a, bool aligned, hipStream_t st) {
 
 // Whether passes of this scan can run on the 384 x 256 tile kernel (whole rounds of it; see scan_wide_kernel).
 static bool wide_scan_ok(int dtype, bool aligned, int64_t D, int64_t stride, int Q) {
-  return dtype != BGX_F32 && aligned && D % 64 == 0 && Q > SW_BN && !switches().scan_wide_off &&
+  return dtype != BGX_F32 && aligned && D % 64 == 0 && Q > SW_BN / 2 && !switches().scan_wide_off &&
          stride * 2 * (SW_BM + 8) < ((int64_t)1 << 32) && D * 2 * (SW_BN + 8) < ((int64_t)1 << 32);
 }
 
@@ -1703,12 +1710,12 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
   while (done < n_rows) {
     int64_t rows = n_rows - done;
     if (want_topk) {
-      // the first pass has no threshold yet and appends every score: each query's list grows by one
-      // serialised atomic per row, so that pass stays small and later passes grow fourfold
+      // the first pass has no threshold yet and keeps every score (the selection behind it then sorts one entry per
+      // row and query), so that pass stays small and later passes grow fourfold
       int64_t lim = done == 0 ? SCAN_FIRST_CHUNK : done * 4;
       // with the wide tile kernel the second pass is a whole round already (thresholds from 4096 rows let
       // through k / 4096 of the scores: a few hundred candidates per query)
-      if (done > 0 && lim < SW_ROUND_ROWS && wide_scan_ok(dtype, aligned, D, stride, Q)) lim = SW_ROUND_ROWS;
+      if (done > 0 && lim < sw_round_rows(Q) && wide_scan_ok(dtype, aligned, D, stride, Q)) lim = sw_round_rows(Q);
       if (stream_scan) lim = done == 0 ? stream_first : chunk;
       if (lim < k) lim = k;
       if (lim > chunk) lim = chunk;
@@ -1717,7 +1724,7 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
     if (row_part != nullptr && rows > chunk) rows = chunk;  // the partial sums of one pass fit the workspace
     // many queries: long passes are cut to whole rounds of the 384 x 256 tile kernel (the end of the store makes
     // one last, shorter pass)
-    if (rows >= SW_ROUND_ROWS && wide_scan_ok(dtype, aligned, D, stride, Q)) rows = rows / SW_ROUND_ROWS * SW_ROUND_ROWS;
+    if (rows >= sw_round_rows(Q) && wide_scan_ok(dtype, aligned, D, stride, Q)) rows = rows / sw_round_rows(Q) * sw_round_rows(Q);
     ScanArgs a;
     a.store = store;
     a.queries = queries;

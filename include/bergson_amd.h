@@ -370,7 +370,7 @@ int bgx_scan(const void* store_dev, int64_t n_rows, int64_t D,
  * (query/attributor.py:137-167), and scores it many times; this is the same
  * economy -- kernels that would otherwise sum the squares of every row in
  * their inner loop leave that out and take the multiplier from the array
- * (the 384 x 256 tile kernel for more than 256 queries; the other kernels
+ * (the 384 x 256 tile kernel for more than 128 queries; the other kernels
  * compute the sums as before, which gives the same values).  Everything else
  * as bgx_scan; there is no sumsq output. */
 int bgx_scan_known_norms(const void* store_dev, int64_t n_rows, int64_t D,
