@@ -313,16 +313,18 @@ def test_scan_many_queries_direct_tiles(device, dtype, D, Q):
     assert (small.topk_values[same] - res.topk_values[same]).abs().max().item() <= 1e-5
 
 
-@pytest.mark.parametrize("dtype,D,Q", [(torch.float16, 192, 300), (torch.bfloat16, 128, 520), (torch.float16, 64, 1024)])
+@pytest.mark.parametrize("dtype,D,Q", [(torch.float16, 192, 300), (torch.bfloat16, 128, 520), (torch.float16, 64, 1024),
+                                       (torch.float16, 128, 200), (torch.bfloat16, 64, 129)])
 def test_scan_wide_tiles_equal_the_256_tiles_bitwise(device, dtype, D, Q, bgx_env):
-    """More than 256 queries over many rows: whole rounds of 24 576 rows run on the 384 x 256 tile kernel (one
-    wave per SIMD, accumulators in both register files), the rest on the 256 x 256 kernels.  Every score is the
+    """More than 128 queries over many rows: whole rounds of the chip (256 workgroups: 24 576 rows with four query
+    tiles, 98 304 with one) run on the 384 x 256 tile kernel (one wave per SIMD, accumulators in both register
+    files), the rest on the 256 x 256 kernels.  Every score is the
     same sequence of matrix instructions over D in both, and the row norms are summed in the same order: scores,
     norms, row maxima and the top-k must be the same bits with the wide kernel switched off; the row means add
     their per-wave partial sums in another order and agree to rounding.  Scores are also held to the oracle."""
     from bergson_amd import ops
 
-    n, k = 4096 + 16384 + 2 * 24576 + 1500, 40
+    n, k = (4096 + 16384 + 2 * 24576 + 1500, 40) if Q > 256 else (4096 + 98304 + 11000, 40)
     store, queries = make_store(n, D, Q, dtype, seed=3 * D + Q)
     store[30_000] = 0
     qd = unit_queries(queries, dtype).to(dtype)
