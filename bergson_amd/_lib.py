@@ -11,7 +11,7 @@ from pathlib import Path
 LIB_PATH = Path(__file__).resolve().parent / "libbergson_amd.so"
 
 BGX_F32, BGX_F16, BGX_BF16 = 0, 1, 2
-ABI_VERSION = 9
+ABI_VERSION = 10
 STATIC_SCRATCH_BYTES = 16 << 20
 
 
@@ -53,6 +53,7 @@ SIGNATURES: dict[str, tuple] = {
     "bgx_abi_version": (C.c_int, []),
     "bgx_last_error": (C.c_char_p, []),
     "bgx_reload_switches": (C.c_int, []),
+    "bgx_last_kernel": (C.c_char_p, [C.c_int32]),
     "bgx_adafactor_scales": (
         C.c_int,
         [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p],
@@ -173,6 +174,14 @@ def load() -> C.CDLL:
 def reload_switches() -> None:
     """Make the library read its BGX_* environment switches again (they are read once otherwise)."""
     load().bgx_reload_switches()
+
+
+FAMILY_COLLECT, FAMILY_ADAM, FAMILY_SCAN, FAMILY_FULLGRAD = 0, 1, 2, 3
+
+
+def last_kernel(family: int) -> str:
+    """Name of the main kernel this thread's last launch of a family enqueued ("" before the first)."""
+    return load().bgx_last_kernel(family).decode()
 
 
 def check(rc: int, what: str) -> None:

@@ -1511,6 +1511,7 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
         hipLaunchKernelGGL(kern, grid, dim3(512), smem, st, f);
       }
       BGX_HIP(hipGetLastError());
+      note_kernel(FAMILY_ADAM, wide ? "adam_fused_wide" : direct ? "adam_fused_direct" : "adam_fused_staged");
       if (per_token) {
         hipLaunchKernelGGL(adam_tok_finalize_kernel, dim3((unsigned)rows_c), dim3(256), 0, st, ptok_f, t0, (int)rows_c,
                            S, pp, lengths, rows, out, out_row_stride, out_col, out_dtype, lo, hi);
@@ -1532,6 +1533,7 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
     return 0;
   }
 
+  note_kernel(FAMILY_ADAM, "adam_two_kernel");
   for (int64_t t0 = 0; t0 < T; t0 += tc) {
     const int64_t rows_c = T - t0 < tc ? T - t0 : tc;
     const char* a_chunk = (const char*)a + (size_t)t0 * a_tok_stride * esz;

@@ -23,6 +23,16 @@ int hip_fail(hipError_t e, const char* what) {
   return (int)e;
 }
 
+static thread_local const char* g_last_kernel[FAMILY_COUNT] = {"", "", "", ""};
+
+void note_kernel(int family, const char* name) {
+  if (family >= 0 && family < FAMILY_COUNT) g_last_kernel[family] = name;
+}
+
+const char* noted_kernel(int family) {
+  return family >= 0 && family < FAMILY_COUNT ? g_last_kernel[family] : "";
+}
+
 static const Switches* read_switches() {
   Switches* s = new Switches;
   auto off = [](const char* name) {
@@ -143,6 +153,10 @@ int bgx_reload_switches(void) {
 }
 
 const char* bgx_last_error(void) { return bgx::g_err; }
+
+const char* bgx_last_kernel(int32_t family) {
+  return bgx::noted_kernel(family);
+}
 
 int bgx_adafactor_scales(const float* row_dev, int32_t O, const float* col_dev, int32_t I, int32_t dtype,
                          float* row_scale_dev, float* col_scale_dev, void* stream) {

@@ -1181,6 +1181,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     else
       rc = launch_persist<bf16_t>(staged, rfg, per_token, tile_tokens, wgs, persist_lds, st, pa);
     if (rc != 0) return rc;
+    note_kernel(FAMILY_COLLECT, rfg ? "collect_persist_table" : staged ? "collect_persist_lds" : "collect_persist_direct");
   } else if (in_dtype == BGX_F32) {
     launch_collect_pb<float>(pb, aligned, per_token, any_bias, tile_tokens, grid, st, args);
   } else if (in_dtype == BGX_F16) {
@@ -1189,6 +1190,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     launch_collect_pb<bf16_t>(pb, aligned, per_token, any_bias, tile_tokens, grid, st, args);
   }
   BGX_HIP(hipGetLastError());
+  if (!persist) note_kernel(FAMILY_COLLECT, "collect_tile");
   if (timed) BGX_HIP(hipEventRecord(ev_stop, st));
 
   if (!per_token) {

@@ -44,6 +44,14 @@ struct Switches {
 };
 const Switches& switches();
 
+// ---- which kernel ran (defined in capi.hip) -------------------------------------
+// Every entry point with more than one kernel behind it notes the name of the main kernel it enqueued, per
+// calling thread and family; bgx_last_kernel() reads it back.  Tests use it to assert a route without
+// forcing one through the switches above.
+enum KernelFamily { FAMILY_COLLECT = 0, FAMILY_ADAM = 1, FAMILY_SCAN = 2, FAMILY_FULLGRAD = 3, FAMILY_COUNT = 4 };
+void note_kernel(int family, const char* name);
+const char* noted_kernel(int family);
+
 // ---- vector types for the MFMA builtins -----------------------------------
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;

@@ -1558,6 +1558,7 @@ static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
         BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SW_LDS_BYTES));
         hipLaunchKernelGGL(kern, dim3((unsigned)(row_tiles_pad * a.q_tiles)), dim3(SW_THREADS), SW_LDS_BYTES, st, a);
         BGX_HIP(hipGetLastError());
+        note_kernel(FAMILY_SCAN, a.sumsq_in != nullptr ? "scan_wide_known_norms" : "scan_wide");
         return 0;
       }
       // aligned 16-bit operands, D a multiple of the K tile: tiles loaded straight into LDS
@@ -1580,17 +1581,21 @@ static int launch_gemm_t(ScanArgs& a, bool aligned, hipStream_t st) {
         }
         if (rc != 0) return rc;
         BGX_HIP(hipGetLastError());
+        note_kernel(FAMILY_SCAN, "scan_direct");
         return 0;
       }
     }
+    note_kernel(FAMILY_SCAN, "scan_gemm");
     return launch_gemm<T, BM, BN, 2, 4>(a, aligned, st);
   } else if (a.Q > 32) {
+    note_kernel(FAMILY_SCAN, "scan_gemm");
     constexpr int BM = 128, BN = 64;
     a.row_tiles = (int)((a.rows + BM - 1) / BM);
     a.q_tiles = (a.Q + BN - 1) / BN;
     a.n_parts = a.q_tiles;
     return launch_gemm<T, BM, BN, 4, 1, 2>(a, aligned, st);
   } else {
+    note_kernel(FAMILY_SCAN, "scan_gemm");
     constexpr int BM = 128, BN = 32;
     a.row_tiles = (int)((a.rows + BM - 1) / BM);
     a.q_tiles = (a.Q + BN - 1) / BN;
@@ -1707,6 +1712,8 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
   bool table_built = false;
 
   int64_t done = 0;
+  int64_t longest_pass = 0;
+  const char* main_kernel = "";
   while (done < n_rows) {
     int64_t rows = n_rows - done;
     if (want_topk) {
@@ -1771,6 +1778,7 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
       rc = dtype == BGX_F16    ? launch_stream<f16_t>(a, blocks, qtable, wgs, st)
            : dtype == BGX_BF16 ? launch_stream<bf16_t>(a, blocks, qtable, wgs, st)
                                : launch_stream<float>(a, blocks, qtable, wgs, st);
+      note_kernel(FAMILY_SCAN, "scan_stream");
     } else {
       // (honoured by scan_gemm_kernel, which takes the short first pass; the other tile kernels let every score of
       // a pass without thresholds through their candidate filter instead, with the same result)
@@ -1780,6 +1788,10 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
                                : launch_gemm_t<float>(a, aligned, st);
     }
     if (rc != 0) return rc;
+    if (rows > longest_pass) {  // the scan is named after the kernel of its longest pass
+      longest_pass = rows;
+      main_kernel = noted_kernel(FAMILY_SCAN);
+    }
     if (row_part != nullptr) {
       hipLaunchKernelGGL(scan_row_mean_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, row_part,
                          a.n_parts, rows, done, 1.0f / (float)Q, row_mean);
@@ -1802,6 +1814,7 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
     }
     done += rows;
   }
+  note_kernel(FAMILY_SCAN, main_kernel);
 
   if (need_init) {
     const int64_t n_fin = ((int64_t)Q * k > (row_max ? n_rows : 0)) ? (int64_t)Q * k : n_rows;

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define BGX_ABI_VERSION 9
+#define BGX_ABI_VERSION 10
 
 enum bgx_dtype { BGX_F32 = 0, BGX_F16 = 1, BGX_BF16 = 2 };
 
@@ -92,6 +92,17 @@ const char* bgx_last_error(void);
  * bgx_reload_switches() reads them again.  Launches that are being issued from
  * other threads at that moment see either the old or the new settings. */
 int bgx_reload_switches(void);
+
+/* Diagnostics (no counterpart in the reference).  Name of the main kernel the
+ * calling thread's last launch of a family enqueued ("" before the first):
+ * family 0 = bgx_collect_seq/_tok/_static ("collect_persist_lds",
+ * "collect_persist_table", "collect_persist_direct", "collect_tile"),
+ * 1 = bgx_collect_adam ("adam_fused_wide", "adam_fused_direct",
+ * "adam_fused_staged", "adam_two_kernel"), 2 = bgx_scan* (the kernel of the
+ * longest pass: "scan_wide", "scan_wide_known_norms", "scan_direct", "scan_stream",
+ * "scan_gemm"), 3 = bgx_fullgrad_* / bgx_project_rows.  The pointer is to a
+ * string literal. */
+const char* bgx_last_kernel(int32_t family);
 
 /* Adafactor factors of one module, computed once per module.
  * Replaces collector.py:532-535 and :655-658 (closed form in

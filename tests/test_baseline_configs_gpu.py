@@ -86,6 +86,120 @@ def test_pythia410m_adam_per_token_against_oracle(device, shape):
     assert rel_l2(out.cpu(), want) <= TOL[torch.bfloat16]
 
 
+def _adam_closed_form_fp64(a_t, g_t, v, left, right):
+    """P_t = L (g_t a_t^T / (sqrt(v) + 1e-8)) R^T for one token in float64, from the formula
+    (bergson/gradients.py:380-388 applied to the outer product of collector.py:611-612)."""
+    full = torch.outer(g_t.double(), a_t.double()) / (v.double().sqrt() + 1e-8)
+    return (left.double() @ full @ right.double().T).flatten()
+
+
+@pytest.mark.parametrize("shape", [(1024, 3072), (1024, 1024), (1024, 4096), (4096, 1024)])
+def test_pythia410m_adam_per_token_whole_tiles_sampled_against_oracle(device, shape):
+    """The configuration's production route -- whole 256-token tiles on the four-wave fused kernel -- held to the
+    oracle directly: per-token rows do not depend on each other, so the oracle and the float64 closed form are
+    evaluated on a sample of the tokens of a full launch (first and last token of every tile, the last valid
+    token of each sequence, random interior ones).  Two sequences of 512, the second ragged."""
+    from bergson_amd import _lib, ops
+
+    I, O = shape
+    N, S, p = 2, 512, 32
+    lengths = [512, 389]
+    a, g, left, right, norm = _case(N, S, I, O, p, torch.bfloat16, 72, "adam", "layers.5.mlp.dense_4h_to_h")
+    for n, l in enumerate(lengths):
+        g[n, l - 1:] = 0
+    prep = ops.AdamPrepared(right.to(device), left.to(device), norm.weight_avg_sq.to(device), 0)
+    counts = [l - 1 for l in lengths]
+    offs = [0, counts[0]]
+
+    def run(out_dtype, per_token=True):
+        out = torch.zeros(sum(counts) if per_token else N, p * p, dtype=out_dtype, device=device)
+        ops.collect_adam(prep, a.to(device), g.to(device), out, per_token=per_token,
+                         lengths=torch.tensor(lengths, dtype=torch.int32, device=device),
+                         rows=torch.tensor(offs if per_token else [0, 1], dtype=torch.int64, device=device),
+                         lo=torch.finfo(out_dtype).min, hi=torch.finfo(out_dtype).max)
+        torch.cuda.synchronize()
+        return out.cpu()
+
+    got = run(torch.bfloat16)
+    assert _lib.last_kernel(_lib.FAMILY_ADAM) == "adam_fused_wide"   # no switch set: this is the default route
+    got32 = run(torch.float32)
+    assert torch.isfinite(got32).all()
+    gen = torch.Generator().manual_seed(5)
+    for n in range(N):
+        last = counts[n] - 1
+        idx = {0, 255, 256, last, last - 1, 1, 254, 257}
+        idx |= {t for t in (511, 510) if t <= last}
+        idx |= set(torch.randint(2, last, (12,), generator=gen).tolist())
+        idx = sorted(idx)
+        ones = torch.ones(1, len(idx), dtype=torch.bool)
+        want = ohooks.module_gradient(a[n:n + 1, idx], g[n:n + 1, idx], norm, left, right, attribute_tokens=True,
+                                      collection_mask=ones)
+        rows = torch.tensor(idx) + offs[n]
+        assert rel_l2(got[rows], want) <= TOL[torch.bfloat16]
+        for j, t in enumerate(idx):   # each sampled token on its own, so one wrong row cannot hide in the norm
+            assert rel_l2(got[rows[j]], want[j]) <= 2 * TOL[torch.bfloat16], (n, t)
+        for t in idx[:6] + idx[-3:]:
+            exact = _adam_closed_form_fp64(a[n, t], g[n, t], norm.weight_avg_sq, left, right)
+            assert rel_l2(got32[offs[n] + t], exact) <= TOL[torch.bfloat16], (n, t)
+    # the per-sequence rows of the same inputs against the sum of the per-token rows
+    seq = run(torch.float32, per_token=False)
+    for n in range(N):
+        assert rel_l2(seq[n], got32[offs[n]:offs[n] + counts[n]].sum(0)) <= TOL[torch.bfloat16]
+
+
+def test_pythia410m_width_two_layers_adam_per_token_through_the_model(device):
+    """Two layers at the Pythia-410m widths (1024 / 4096, 16 heads), bf16, Adam second moments, p = 32, per-token
+    rows, two documents of 512 and 389 tokens in one batch through the product loop; every module's block of
+    sampled tokens against the oracle on the (a, g) the hooks saw."""
+    import numpy as np
+    from bergson_amd import AdamNormalizer, GradientCollector, GradientProcessor, IndexConfig
+    from bergson_amd.collector import CollectorComputer
+    from bergson_amd.synthetic import ListDataset, make_gpt_neox, random_docs
+
+    lengths = [512, 389]
+    p = 32
+    docs = random_docs(lengths, seed=23)
+    model = make_gpt_neox("pythia-410m", torch.bfloat16, device, seed=0, layers=2)
+    gen = torch.Generator().manual_seed(9)
+    moments, captured, handles = {}, {}, []
+    for name, mod in model.base_model.named_modules():
+        if isinstance(mod, torch.nn.Linear):
+            moments[name] = torch.randn(mod.weight.shape, generator=gen).abs() * 1e-5 + 1e-12
+            handles.append(mod.register_forward_hook(
+                lambda m, inp, out, name=name: captured.setdefault(name, {}).__setitem__("a", inp[0].detach().cpu())))
+            handles.append(mod.register_full_backward_hook(
+                lambda m, gin, gout, name=name: captured[name].__setitem__("g", gout[0].detach().cpu())))
+    names = list(moments)
+    assert len(names) == 8
+    normalizers = {n: AdamNormalizer(weight_avg_sq=v.to(device)) for n, v in moments.items()}
+    cfg = IndexConfig(run_path="", projection_dim=p, projection_type="normal", attribute_tokens=True)
+    col = GradientCollector(model=model.base_model, cfg=cfg, data=ListDataset(docs),
+                            processor=GradientProcessor(normalizers=normalizers, projection_dim=p,
+                                                        projection_type="normal"))
+    CollectorComputer(model=model, data=ListDataset(docs), collector=col, batches=[[0, 1]], cfg=cfg
+                      ).run_with_collector_hooks()
+    torch.cuda.synchronize()
+    for h in handles:
+        h.remove()
+    assert col.builder.base_dtype == "bfloat16"   # the model's gradient dtype; numpy maps it as uint16 bit patterns
+    got = torch.from_numpy(np.array(col.builder.grad_buffer).view(np.int16)).view(torch.bfloat16).float()
+    counts = [l - 1 for l in lengths]
+    assert got.shape == (sum(counts), 8 * p * p) and torch.isfinite(got).all()
+    sample = {0: [0, 1, 255, 256, 300, 509, 510], 1: [0, 17, 255, 256, 386, 387]}
+    for name in names:
+        a, g = captured[name]["a"], captured[name]["g"]
+        left, right = module_projections(name, p, g.shape[-1], a.shape[-1], torch.bfloat16)
+        b = names.index(name)
+        for n, idx in sample.items():
+            ones = torch.ones(1, len(idx), dtype=torch.bool)
+            want = ohooks.module_gradient(a[n:n + 1, idx], g[n:n + 1, idx], ohooks.Adam(moments[name]), left, right,
+                                          attribute_tokens=True, collection_mask=ones).float()
+            rows = torch.tensor(idx) + (0 if n == 0 else counts[0])
+            block = got[rows, b * p * p:(b + 1) * p * p]
+            assert want.abs().max() > 0
+            assert rel_l2(block, want) <= TOL[torch.bfloat16], (name, n)
+
+
 # ---- configuration 2 at full size: 4096-token batch, all 48 Pythia-160m modules ----------------------------
 def _pythia160m_modules(N, S, seed):
     d = 768
