@@ -23,7 +23,7 @@ import math
 import os
 from abc import ABC, abstractmethod
 from contextlib import ContextDecorator, nullcontext
-from dataclasses import astuple, dataclass, field
+from dataclasses import dataclass, field
 from fnmatch import fnmatchcase
 from typing import Callable, Literal, Mapping, Optional
 
@@ -70,6 +70,49 @@ def create_projection_matrix(identifier: str, m: int, n: int, dtype: torch.dtype
     return A.to(device)
 
 
+@dataclass(frozen=True)
+class GradBlock:
+    """One block of store columns: the gradient of a whole module, or of one attention head of it."""
+
+    name: str  # key in shapes(), in the normalizers of a head-wise processor and in the projection cache
+    module: str  # the hooked module the block belongs to
+    head: int | None  # None for a whole module
+    first: int  # first output feature of the block
+    width: int  # number of output features
+    axis: int  # dimension of g the output features lie on (heads only)
+    weight_shape: torch.Size  # [O, I (+1)] of the block when nothing is projected
+
+
+class HeadView:
+    """Stands in for a hooked module while one of its attention heads is processed: `_name` is the head's
+    name, the module's output-feature attribute reads as the head's width, everything else (the kept input,
+    the bias flag, the input width, the module's type for isinstance checks) is the module's own."""
+
+    __slots__ = ("_hv_module", "_hv_block", "_hv_width_attr")
+
+    def __init__(self, module: nn.Module, block: GradBlock):
+        object.__setattr__(self, "_hv_module", module)
+        object.__setattr__(self, "_hv_block", block)
+        object.__setattr__(self, "_hv_width_attr", LayerAdapter.out_attr(module))
+
+    @property
+    def __class__(self):  # isinstance(view, nn.Linear) answers for the module
+        return type(self._hv_module)
+
+    def __getattr__(self, key):
+        if key == "_name":
+            return self._hv_block.name
+        if key == self._hv_width_attr:
+            return self._hv_block.width
+        return getattr(self._hv_module, key)
+
+    def __setattr__(self, key, value):
+        setattr(self._hv_module, key, value)
+
+    def __delattr__(self, key):
+        delattr(self._hv_module, key)
+
+
 @dataclass
 class HookCollectorBase(ContextDecorator, ABC):
     """Attaches forward and backward hooks to the supported layers of `model`.
@@ -99,6 +142,7 @@ class HookCollectorBase(ContextDecorator, ABC):
         self._fwd_hooks: list[RemovableHandle] = []
         self._bwd_hooks: list[RemovableHandle] = []
         self._current_collection_mask: Tensor | None = None
+        self._current_doc_lengths: list[int] | None = None
         self._deferred: list = []
         self._prepared: dict[str, ops.PreparedModule] = {}
         self._adam_prepared: dict[str, ops.AdamPrepared] = {}
@@ -134,72 +178,97 @@ class HookCollectorBase(ContextDecorator, ABC):
             target_info[name] = (layer.weight.device, torch.Size([o, i]), collect_bias)
         return target_info
 
+    # ---- column blocks: whole modules and attention heads (collector.py:185-334) --------------------------
     @staticmethod
     def get_head_name(name: str, head_idx: int) -> str:
         return f"{name}.head_{head_idx}"
 
     @staticmethod
     def split_head_name(name: str) -> tuple[str, int] | None:
+        """("<module>", h) for "<module>.head_<h>", None for any other name."""
         base, sep, suffix = name.rpartition(".head_")
-        if not sep or not suffix.isdigit():
-            return None
-        return base, int(suffix)
+        return (base, int(suffix)) if sep and suffix.isdigit() else None
+
+    def _plan_blocks(self) -> dict[str, tuple["GradBlock", ...]]:
+        """module name -> the column blocks its gradient is stored as, in store order: one block for an
+        ordinary module; for a module listed in `attention_cfgs`, one per head, each covering `head_size`
+        consecutive output features along dimension `head_dim` of g.  Every block becomes one descriptor
+        of the batch's fused launch: a head's descriptor points `first` features into the rows of g and
+        carries its own output column, so splitting costs no copy and no extra launch."""
+        plan: dict[str, tuple[GradBlock, ...]] = {}
+        for name, (_, weight_shape, with_bias) in self.target_info.items():
+            dims = [int(d) for d in weight_shape]
+            cfg = self.attention_cfgs.get(name)
+            if cfg is None:
+                heads: list[tuple[int | None, int, int]] = [(None, 0, dims[0])]
+                axis = -1
+            else:
+                heads = [(h, h * cfg.head_size, cfg.head_size) for h in range(cfg.num_heads)]
+                axis = cfg.head_dim
+                dims[axis - 2] = cfg.head_size  # g is [N, S, ...]: its dimension `axis` is dimension `axis - 2` of the weight
+            if with_bias:
+                dims[-1] += 1
+            plan[name] = tuple(GradBlock(name if h is None else self.get_head_name(name, h), name, h, first, width,
+                                         axis, torch.Size(dims)) for h, first, width in heads)
+        return plan
+
+    def blocks_of(self, module_name: str) -> tuple["GradBlock", ...]:
+        plan = self.__dict__.get("_blocks")
+        if plan is None or module_name not in plan:
+            plan = self._blocks = self._plan_blocks()
+        return plan[module_name]
 
     @staticmethod
     def split_attention_heads(fn):
-        """Decorator: calls `fn(self, module, g_head)` once per head for modules in `attention_cfgs`
-        (collector.py:191-233).  The head's slice of g is a strided view; nothing is copied."""
+        """Decorator for `backward_hook(self, module, g)`: a module listed in `attention_cfgs` is handed to
+        `fn` once per head (collector.py:191-233), as a `HeadView` of the module -- an object that answers
+        `_name` with the head's name and the output-feature count with the head's width and passes every
+        other attribute through -- together with the head's columns of g (a strided view).  The module
+        itself is never modified, so an exception inside `fn` leaves nothing to restore."""
 
         @functools.wraps(fn)
-        def wrapper(self, module, g):
-            name = module._name
-            if name not in self.attention_cfgs:
+        def per_block(self, module, g):
+            blocks = self.blocks_of(module._name)
+            if blocks[0].head is None:
                 return fn(self, module, g)
-            num_heads, head_size, head_dim = astuple(self.attention_cfgs[name])
-            orig_out = getattr(module, LayerAdapter.out_attr(module))
-            assert num_heads * head_size == orig_out, (
-                f"{name}: num_heads * head_size = {num_heads * head_size} does not cover the module's "
-                f"{orig_out} output features")
-            setattr(module, LayerAdapter.out_attr(module), head_size)
-            try:
-                for h in range(num_heads):
-                    module._name = self.get_head_name(name, h)
-                    try:
-                        head_g = torch.narrow(g, head_dim, h * head_size, head_size)
-                    except Exception:
-                        print(f"Error processing gradient of shape {g.shape} for head {h} in module {name}. "
-                              f"Provided head config may be incorrect. Head config: head dim {head_dim}, "
-                              f"head size {head_size}, num heads {num_heads}.")
-                        raise
-                    fn(self, module, head_g)
-            finally:
-                module._name = name
-                setattr(module, LayerAdapter.out_attr(module), orig_out)
+            covered = sum(b.width for b in blocks)
+            features = getattr(module, LayerAdapter.out_attr(module))
+            if covered != features:
+                raise AssertionError(f"{module._name}: {len(blocks)} heads of {blocks[0].width} features make "
+                                     f"{covered}, the module has {features} output features")
+            for block in blocks:
+                try:
+                    g_head = g.narrow(block.axis, block.first, block.width)
+                except Exception:
+                    cfg = self.attention_cfgs[module._name]
+                    print(f"{module._name}: cannot take head {block.head} out of a gradient of shape "
+                          f"{tuple(g.shape)} with {cfg}; the head configuration may be wrong.")
+                    raise
+                fn(self, HeadView(module, block), g_head)
 
-        return wrapper
+        return per_block
 
     def normalizer_for(self, name: str):
-        """Normalizer of module `name`; a split head takes its rows of the parent's (collector.py:243-279)."""
-        normalizer = self.processor.normalizers.get(name)
-        if normalizer is not None:
-            return normalizer
-        split = self.split_head_name(name)
-        if split is None:
+        """The normalizer registered under `name`; for an attention head, its rows of the normalizer that is
+        registered under the module's name (collector.py:243-279)."""
+        registered = self.processor.normalizers
+        own = registered.get(name)
+        if own is not None:
+            return own
+        parsed = self.split_head_name(name)
+        if parsed is None:
             return None
-        base, head_idx = split
-        normalizer = self.processor.normalizers.get(base)
-        if normalizer is None or base not in self.attention_cfgs:
-            return normalizer
-        head_size = self.attention_cfgs[base].head_size
-        lo, hi = head_idx * head_size, (head_idx + 1) * head_size
-        if isinstance(normalizer, AdamNormalizer):
-            bias = normalizer.bias_avg_sq
-            return AdamNormalizer(normalizer.weight_avg_sq[lo:hi], bias[lo:hi] if bias is not None else None)
-        if isinstance(normalizer, AdafactorNormalizer):
-            bias = normalizer.bias_avg_sq
-            return AdafactorNormalizer(normalizer.row[lo:hi], normalizer.col,
-                                       bias[lo:hi] if bias is not None else None)
-        return normalizer
+        whole = registered.get(parsed[0])
+        cfg = self.attention_cfgs.get(parsed[0])
+        if whole is None or cfg is None:
+            return whole
+        rows = slice(parsed[1] * cfg.head_size, (parsed[1] + 1) * cfg.head_size)
+        cut = lambda t: None if t is None else t[rows]  # noqa: E731
+        if isinstance(whole, AdafactorNormalizer):  # the column moments belong to the shared input side
+            return AdafactorNormalizer(cut(whole.row), whole.col, cut(whole.bias_avg_sq))
+        if isinstance(whole, AdamNormalizer):
+            return AdamNormalizer(cut(whole.weight_avg_sq), cut(whole.bias_avg_sq))
+        return whole
 
     @property
     def per_module_projection_dim(self) -> int | None:
@@ -208,34 +277,15 @@ class HookCollectorBase(ContextDecorator, ABC):
         return self.processor.projection_dim or None
 
     def shapes(self) -> Mapping[str, torch.Size]:
-        """Shapes of the collected gradients; their order is the column order of the store
-        (collector.py:288-334)."""
+        """Shape of every stored block, in the column order of the store (collector.py:288-334): one
+        "gradients" vector in global mode, [p, p] per block when projecting per module, else the block's
+        [O, I (+1)] weight shape."""
         if self.processor.projection_target == "global":
             assert self.processor.projection_dim is not None
             return {"gradients": torch.Size((self.processor.projection_dim,))}
-        p_dim = self.per_module_projection_dim
-        proj_shape = torch.Size((p_dim, p_dim)) if p_dim is not None else None
-        shapes = {}
-        for name, (_, target_shape, collect_bias) in self.target_info.items():
-            if name in self.attention_cfgs:
-                cfg = self.attention_cfgs[name]
-                if proj_shape:
-                    head_shape = proj_shape
-                else:
-                    attention_shape = list(target_shape)
-                    attention_shape[cfg.head_dim - 2] = cfg.head_size
-                    if collect_bias:
-                        attention_shape[-1] += 1
-                    head_shape = torch.Size(attention_shape)
-                shapes.update({self.get_head_name(name, h): head_shape for h in range(cfg.num_heads)})
-            elif proj_shape:
-                shapes[name] = proj_shape
-            else:
-                grad_shape = list(target_shape)
-                if collect_bias:
-                    grad_shape[-1] += 1
-                shapes[name] = torch.Size(grad_shape)
-        return shapes
+        p = self.per_module_projection_dim
+        return {block.name: block.weight_shape if p is None else torch.Size((p, p))
+                for blocks in self._plan_blocks().values() for block in blocks}
 
     def projection(self, name: str, m: int, n: int, role: Literal["left", "right", "single"],
                    device: torch.device, dtype: torch.dtype) -> Tensor:
@@ -255,9 +305,13 @@ class HookCollectorBase(ContextDecorator, ABC):
         return len(data)
 
     # ---- batch protocol (collector.py:413-491) -------------------------------------------
-    def with_batch(self, collection_mask: Tensor | None = None) -> "HookCollectorBase":
-        """Sets the [N, S] mask of collected positions (every real position but each sequence's last)."""
+    def with_batch(self, collection_mask: Tensor | None = None, doc_lengths: list[int] | None = None
+                   ) -> "HookCollectorBase":
+        """Sets the [N, S] mask of collected positions (every real position but each sequence's last).
+        `doc_lengths`: the documents' lengths as the host knows them; with them the number of per-token rows
+        of the batch needs no read-back from the device."""
         self._current_collection_mask = collection_mask
+        self._current_doc_lengths = doc_lengths
         return self
 
     def __enter__(self):
@@ -304,12 +358,13 @@ class HookCollectorBase(ContextDecorator, ABC):
             del module._inputs
 
     # ---- recorded batches: the backward pass without Python hooks ---------------------------------
-    def begin_recording(self, collection_mask: Tensor | None = None) -> "BatchRecord":
+    def begin_recording(self, collection_mask: Tensor | None = None, doc_lengths: list[int] | None = None
+                        ) -> "BatchRecord":
         """Until `end_recording`, forward hooks list (module, kept input, module output) in the returned
         record instead of attaching tensor hooks.  The caller obtains the gradients of
         `record.outputs()` from autograd (e.g. `torch.autograd.grad`, possibly on another thread while the
         next batch's forward pass runs here) and hands them to `replay_backward`."""
-        self._recording = BatchRecord(collection_mask)
+        self._recording = BatchRecord(collection_mask, doc_lengths)
         return self._recording
 
     def end_recording(self) -> None:
@@ -320,6 +375,7 @@ class HookCollectorBase(ContextDecorator, ABC):
         order and arguments a backward pass with tensor hooks would have produced (collector.py:435-472)."""
         assert len(grads) == len(record.entries), (len(grads), len(record.entries))
         self._current_collection_mask = record.mask
+        self._current_doc_lengths = record.doc_lengths
         for (module, kept, _out), g in zip(reversed(record.entries), reversed(grads)):
             if g is None:  # the loss does not depend on this call's output
                 continue
@@ -470,7 +526,15 @@ class HookCollectorBase(ContextDecorator, ABC):
         assert lengths is not None, "attribute_tokens needs a collection mask (with_batch)"
         counts = (lengths.to(torch.int64) - 1).clamp_min_(0)
         offsets = torch.cumsum(counts, 0) - counts
-        return lengths, counts, offsets, int(counts.sum().item())
+        return lengths, counts, offsets, self._token_total(counts)
+
+    def _token_total(self, counts: Tensor) -> int:
+        """Per-token rows of the current batch: from the host's document lengths when the loop supplied them
+        (`with_batch(mask, doc_lengths)`), else read back from the device (one synchronisation)."""
+        host = self._current_doc_lengths
+        if host is not None and len(host) == counts.numel():
+            return sum(max(int(n) - 1, 0) for n in host)
+        return int(counts.sum().item())
 
     def _global_projection(self, items: list, out: Tensor, lengths: Tensor | None, out_rows: Tensor | None,
                            row_offsets: Tensor | None) -> None:
@@ -569,7 +633,7 @@ class HookCollectorBase(ContextDecorator, ABC):
                 assert lengths is not None, "attribute_tokens needs a collection mask (with_batch)"
                 counts = (lengths.to(torch.int64) - 1).clamp_min_(0)
                 offsets = torch.cumsum(counts, 0) - counts
-                out = torch.empty((int(counts.sum().item()), p * p), dtype=g.dtype, device=g.device)
+                out = torch.empty((self._token_total(counts), p * p), dtype=g.dtype, device=g.device)
                 if out.shape[0]:
                     ops.collect_adam(prep, a, g, out, per_token=True, lengths=lengths, rows=offsets, lo=self.lo,
                                      hi=self.hi)
@@ -584,7 +648,7 @@ class HookCollectorBase(ContextDecorator, ABC):
             assert lengths is not None, "attribute_tokens needs a collection mask (with_batch)"
             counts = (lengths.to(torch.int64) - 1).clamp_min_(0)
             offsets = torch.cumsum(counts, 0) - counts
-            total = int(counts.sum().item())
+            total = self._token_total(counts)
             out = torch.empty((total, p * p), dtype=g.dtype, device=g.device)
             if total:
                 ops.collect_tok([mi], p, out, lengths=lengths, row_offsets=offsets, lo=self.lo, hi=self.hi)
@@ -672,10 +736,11 @@ class BatchRecord:
     """What the forward hooks saw during one recorded batch: `entries` = (module, kept input, output) per
     call of a target module, in call order; `mask` = the batch's collection mask."""
 
-    __slots__ = ("mask", "entries", "versions")
+    __slots__ = ("mask", "doc_lengths", "entries", "versions")
 
-    def __init__(self, mask: Tensor | None):
+    def __init__(self, mask: Tensor | None, doc_lengths: list[int] | None = None):
         self.mask = mask
+        self.doc_lengths = doc_lengths
         self.entries: list[tuple[nn.Module, Tensor | None, Tensor]] = []
         self.versions: list[int] = []
 
@@ -728,7 +793,7 @@ class CollectorComputer:
                 if overlapped is not None:
                     overlapped.step(indices, batch, x, y, collection_mask)
                     continue
-                with self.collector.with_batch(collection_mask):
+                with self.collector.with_batch(collection_mask, [len(seq) for seq in batch["input_ids"]]):
                     losses = self.forward_backward(self.model, x, y, batch)
                 self.collector.process_batch(indices, losses=losses)
             if overlapped is not None:
@@ -919,7 +984,8 @@ class OverlappedSteps:
                     for t in (x, y, collection_mask):
                         t.record_stream(stream)
             self._step_no += 1
-        record = col.begin_recording(collection_mask)
+        record = col.begin_recording(collection_mask, [len(seq) for seq in batch["input_ids"]]
+                                     if isinstance(batch, dict) and "input_ids" in batch else None)
         try:
             with torch.cuda.stream(stream) if stream is not None else nullcontext():
                 losses = self.forward_loss(self.model, x, y, batch)

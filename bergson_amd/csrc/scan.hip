@@ -61,6 +61,13 @@ __device__ inline uint64_t make_key(float score, uint32_t row) {
   return ((uint64_t)f32_ordered(score) << 32) | (uint64_t)(0xffffffffu - row);
 }
 
+// Entry of a by-row candidate list (a pass without thresholds writes row r's score to entry r): the key, or 0 --
+// below every key of a real score, and dropped by the selection -- for a score no later pass would admit either
+// (NaN and -inf fail every `score > threshold` test).  A row's fate then does not depend on the pass it falls in.
+__device__ inline uint64_t make_key_or_empty(float score, uint32_t row) {
+  return score > -INFINITY ? make_key(score, row) : 0ull;
+}
+
 constexpr int SCAN_KMAX = 2048;
 
 struct ScanArgs {
@@ -164,7 +171,7 @@ __device__ __forceinline__ void scan_block_epilogue(const ScanArgs& args, f32x16
 #pragma unroll
           for (int j = 0; j < TN; ++j)
             if (q_ok[j])
-              args.cand[(q_b + j * 32) * args.cand_cap + prow_b + dr] = make_key(v[j], (uint32_t)(grow_b + dr));
+              args.cand[(q_b + j * 32) * args.cand_cap + prow_b + dr] = make_key_or_empty(v[j], (uint32_t)(grow_b + dr));
         }
       } else if (any && row_ok) {
 #pragma unroll
@@ -1158,7 +1165,7 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void scan_stream_kernel(ScanArg
           rsum += val;  // queries in ascending order: a fixed sum
           if (args.scores != nullptr) args.scores[grow * args.Q + qi] = val;
           if (args.first_pass) {
-            args.cand[qi * args.cand_cap + prow] = make_key(val, (uint32_t)grow);
+            args.cand[qi * args.cand_cap + prow] = make_key_or_empty(val, (uint32_t)grow);
           } else if (val > thr) {
             const uint32_t pos = atomicAdd(&args.cand_count[qi], 1u);
             if ((int64_t)pos < args.cand_cap) args.cand[qi * args.cand_cap + pos] = make_key(val, (uint32_t)grow);
@@ -1343,7 +1350,7 @@ __global__ __launch_bounds__(THREADS) void scan_select_kernel(SelectArgs a) {
   __syncthreads();
   for (uint32_t i = tid; i < total; i += SELECT_THREADS) {
     const uint64_t key = elem(i);
-    if (key >= kth) {
+    if (key >= kth && key != 0) {  // 0 = an empty entry of a by-row list
       const uint32_t pos = atomicAdd(&sh.fill, 1u);
       if (pos < SCAN_KMAX) sh.keys[pos] = key;
     }
@@ -1389,13 +1396,16 @@ __global__ void scan_init_kernel(uint32_t* top_count, uint32_t* cand_count, floa
   if (row_max_enc && i < n_rows) row_max_enc[i] = 0;  // below every encoded float
 }
 
-__global__ void scan_finish_kernel(const uint64_t* top, int Q, int k, int64_t row_base, float* topk_val,
-                                   int64_t* topk_idx, const uint32_t* row_max_enc, float* row_max, int64_t n_rows) {
+// A query with fewer than k selectable scores (NaN and -inf are never selected) gets (-inf, -1) in the rest.
+__global__ void scan_finish_kernel(const uint64_t* top, const uint32_t* top_count, int Q, int k, int64_t row_base,
+                                   float* topk_val, int64_t* topk_idx, const uint32_t* row_max_enc, float* row_max,
+                                   int64_t n_rows) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (top != nullptr && i < (int64_t)Q * k) {
-    const uint64_t key = top[i];
-    topk_val[i] = ordered_f32((uint32_t)(key >> 32));
-    topk_idx[i] = (int64_t)(0xffffffffu - (uint32_t)key) + row_base;
+    const bool filled = (uint32_t)(i % k) < top_count[i / k];
+    const uint64_t key = filled ? top[i] : 0ull;
+    topk_val[i] = filled ? ordered_f32((uint32_t)(key >> 32)) : -INFINITY;
+    topk_idx[i] = filled ? (int64_t)(0xffffffffu - (uint32_t)key) + row_base : (int64_t)-1;
   }
   if (row_max != nullptr && i < n_rows) row_max[i] = ordered_f32(row_max_enc[i]);
 }
@@ -1448,7 +1458,7 @@ static int64_t effective_chunk(int64_t chunk_rows, int Q) {
     // rounds) at 1024 queries, 393 216 (four rounds) at 256
     const int64_t round = sw_round_rows(Q);
     const int64_t c = ((int64_t)96 << 20) / Q / round * round;
-    if (c >= round) return c;
+    if (c >= round && c >= SCAN_KMAX) return c;  // (a pass is never shorter than the largest k by default)
   }
   int64_t c = ((int64_t)64 << 20) / (Q > 0 ? Q : 1);
   if (c > ((int64_t)1 << 20)) c = (int64_t)1 << 20;
@@ -1819,8 +1829,8 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
   if (need_init) {
     const int64_t n_fin = ((int64_t)Q * k > (row_max ? n_rows : 0)) ? (int64_t)Q * k : n_rows;
     hipLaunchKernelGGL(scan_finish_kernel, dim3((unsigned)((n_fin + 255) / 256)), dim3(256), 0, st,
-                       (const uint64_t*)top, Q, k, row_base, topk_val, topk_idx, (const uint32_t*)row_max_enc, row_max,
-                       row_max ? n_rows : 0);
+                       (const uint64_t*)top, (const uint32_t*)top_count, Q, k, row_base, topk_val, topk_idx,
+                       (const uint32_t*)row_max_enc, row_max, row_max ? n_rows : 0);
     BGX_HIP(hipGetLastError());
   }
   return 0;

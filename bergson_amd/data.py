@@ -253,81 +253,86 @@ def allocate_batches(doc_lengths: list[int], N: int, seed: int = 42, max_batch_s
     return batches
 
 
+def pack_by_padded_cost(doc_lengths: list[int], budget: int, max_batch_size: int | None = None) -> list[list[int]]:
+    """Batches of document indices under `longest document * documents <= budget` (bergson/data.py:290-322).
+
+    Documents are taken longest first (equal lengths in index order), and a batch is filled until the next
+    document would break the budget or the size limit.  Since the first document of a batch is its longest,
+    a batch headed by a document of length L holds exactly min(budget // L, max_batch_size) documents
+    (fewer only at the end of the data), so the batches are consecutive runs of the sorted order and no
+    per-document test is needed.  Documents with fewer than two tokens have no next-token label and are left
+    out (their rows of the store stay zero)."""
+    lengths = np.asarray(doc_lengths, dtype=np.int64)
+    order = np.argsort(-lengths, kind="stable")
+    order = order[lengths[order] >= 2]
+    if order.size and lengths[order[0]] > budget:
+        raise RuntimeError(f"At least one document is too long for the token batch size {budget}.")
+    batches, at = [], 0
+    while at < order.size:
+        room = int(budget // lengths[order[at]])
+        if max_batch_size is not None:
+            room = min(room, max_batch_size)
+        batches.append(order[at:at + max(room, 1)].tolist())
+        at += max(room, 1)
+    return batches
+
+
+def spread_over_ranks(batches: list[list[int]], world_size: int) -> list[list[list[int]]]:
+    """Makes the number of batches a multiple of `world_size` by peeling single documents off existing
+    batches, and deals them out round-robin: result[r] = batches r, r + world_size, ... (bergson/data.py:
+    324-369).  With fewer batches than ranks, documents are first split off the currently largest batch
+    (the earliest such batch on ties) until every rank has one; the batch order after that step is the
+    array order of Python's binary heap under the keys (-size, insertion number), as in the reference."""
+    if world_size == 1:
+        return [batches]
+    if len(batches) < world_size:
+        ticket = len(batches)
+        heap: list[tuple[int, int, list[int]]] = []
+        for t, b in enumerate(batches):
+            heapq.heappush(heap, (-len(b), t, b))
+        while len(heap) < world_size:
+            _, _, largest = heapq.heappop(heap)
+            if len(largest) < 2:
+                raise RuntimeError("Not enough documents to give each worker at least one batch.")
+            peeled = [largest.pop()]
+            heapq.heappush(heap, (-len(largest), ticket, largest))
+            heapq.heappush(heap, (-1, ticket + 1, peeled))
+            ticket += 2
+        batches = [entry[2] for entry in heap]
+    missing = -len(batches) % world_size
+    visit = 0
+    while missing and visit < len(batches):
+        donor = batches[visit % len(batches)]
+        visit += 1
+        if len(donor) > 1:
+            batches.append([donor.pop()])
+            missing -= 1
+    if missing:
+        raise AssertionError("Could not construct a number of batches divisible by the world size. If variability "
+                             "of item lengths in your dataset is low consider using a different dataset size or "
+                             "token batch size.")
+    return [batches[r::world_size] for r in range(world_size)]
+
+
 def _allocate_batches_world(doc_lengths: list[int], N: int, world_size: int, seed: int = 42,
                             ranks: list[int] | None = None, max_batch_size: int | None = None
                             ) -> list[list[list[int]]]:
-    """Greedy length-sorted bin packing, split to a multiple of the world size, dealt round-robin,
-    shuffled per rank with `random.seed(seed)` (bergson/data.py:239-377).  Documents shorter than two
-    tokens are left out (their store rows stay zero)."""
+    """The batches of the given ranks (all when None): `pack_by_padded_cost`, `spread_over_ranks`, then each
+    rank's list shuffled by `random.seed(seed); random.shuffle` (bergson/data.py:239-377)."""
     doc_lengths = list(doc_lengths)
-    if ranks is None:
-        ranks = list(range(world_size))
-    docs_sorted = sorted(((i, l) for i, l in enumerate(doc_lengths) if l >= 2), key=lambda x: x[1], reverse=True)
-    n_skipped = len(doc_lengths) - len(docs_sorted)
-    if n_skipped > 0 and _rank() == 0:
-        print(f"Skipping {n_skipped} documents with fewer than 2 tokens (no valid next-token labels).")
-    if len(docs_sorted) < world_size:
+    usable = sum(1 for n in doc_lengths if n >= 2)
+    if usable < len(doc_lengths) and _rank() == 0:
+        print(f"Skipping {len(doc_lengths) - usable} documents with fewer than 2 tokens (no valid next-token labels).")
+    if usable < world_size:
         raise RuntimeError("Not enough documents (with 2+ tokens) to distribute across workers.")
-    if docs_sorted[0][1] > N:
-        raise RuntimeError(f"At least one document is too long for the token batch size {N}.")
-
-    batches: list[list[int]] = []
-    cur: list[int] = []
-    for idx, length in docs_sorted:
-        if not cur:
-            cur.append(idx)
-            continue
-        new_cost = max(length, doc_lengths[cur[0]]) * (len(cur) + 1)
-        within_count = max_batch_size is None or len(cur) + 1 <= max_batch_size
-        if new_cost <= N and within_count:
-            cur.append(idx)
-        else:
-            batches.append(cur)
-            cur = [idx]
-    if cur:
-        batches.append(cur)
-
-    if len(batches) < world_size:  # every worker needs at least one batch
-        counter = 0
-        heap: list[tuple[int, int, list[int]]] = []
-        for batch in batches:
-            heapq.heappush(heap, (-len(batch), counter, batch))
-            counter += 1
-        while len(heap) < world_size:
-            _, _, big = heapq.heappop(heap)
-            if len(big) == 1:
-                raise RuntimeError("Not enough documents to give each worker at least one batch.")
-            singleton = [big.pop()]
-            heapq.heappush(heap, (-len(big), counter, big))
-            counter += 1
-            heapq.heappush(heap, (-1, counter, singleton))
-            counter += 1
-        batches = [b for _, _, b in heap]
-
-    k = -(-len(batches) // world_size)
-    target_batches = world_size * k
-    i = 0
-    while len(batches) < target_batches and i < len(batches):
-        batch = batches[i % len(batches)]
-        if len(batch) == 1:
-            i += 1
-            continue
-        batches.append([batch.pop()])
-        i += 1
-    assert len(batches) == target_batches, (
-        "Could not construct a number of batches divisible by the world size."
-        " If variability of item lengths in your dataset is low "
-        "consider using a different dataset size or token batch size.")
-    assert all(max(doc_lengths[i] for i in batch) * len(batch) <= N for batch in batches)
-
-    allocation: list[list[list[int]]] = [[] for _ in range(world_size)]
-    for b_idx, batch in enumerate(batches):
-        allocation[b_idx % world_size].append(batch)
-    assert len({len(b) for b in allocation}) == 1
-    for rank in ranks:
+    per_rank = spread_over_ranks(pack_by_padded_cost(doc_lengths, N, max_batch_size), world_size)
+    assert all(max(doc_lengths[i] for i in b) * len(b) <= N for share in per_rank for b in share)
+    picked = []
+    for r in (range(world_size) if ranks is None else ranks):
         random.seed(seed)
-        random.shuffle(allocation[rank])
-    return [allocation[rank] for rank in ranks]
+        random.shuffle(per_rank[r])
+        picked.append(per_rank[r])
+    return picked
 
 
 def pad_and_tensor(sequences: list[list[int]], labels: list[list[int]] | None = None, *, padding_value: int = 0,

@@ -77,7 +77,7 @@ class _DeferredBatchMixin:
                 return block
             counts = (lengths.to(torch.int64) - 1).clamp_min_(0)
             offsets = torch.cumsum(counts, 0) - counts
-            total = int(counts.sum().item())
+            total = self._token_total(counts)
             rows = torch.zeros((total, self._row_width), dtype=self.save_dtype, device=dev)
             if total:
                 self.launch_deferred(rows, lengths=lengths, row_offsets=offsets)

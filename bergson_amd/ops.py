@@ -109,6 +109,21 @@ class ModuleInput:
     bias_scale: Tensor | None = None  # [O] fp32: factor of g for the bias column (None = 1)
 
 
+def _check_batch_vectors(lengths: Tensor | None, rows: Tensor | None, N: int, device: torch.device) -> None:
+    """`lengths` (int32 [N]) and `rows` (int64 [N]: store rows or first-row offsets) as every kernel reads them.
+    A wrong dtype would make a kernel read garbage lengths, a wrong size an out-of-range scatter: both are
+    refused before anything is launched."""
+    for t, name, dt in ((lengths, "lengths", torch.int32), (rows, "row indices / offsets", torch.int64)):
+        if t is None:
+            continue
+        if t.dtype != dt or t.dim() != 1 or t.numel() != N or not t.is_contiguous():
+            raise ValueError(f"{name} must be a contiguous {str(dt).removeprefix('torch.')} vector of N={N} elements, "
+                             f"got {str(t.dtype).removeprefix('torch.')} {tuple(t.shape)}")
+        _need_gpu(t, name)
+        if t.device != device:
+            raise ValueError(f"{name} live on {t.device}, the output on {device}")
+
+
 def _rows_view(t: Tensor, name: str) -> Tensor:
     if t.dim() != 3:
         raise ValueError(f"{name} must be [N, S, features], got {tuple(t.shape)}")
@@ -159,14 +174,7 @@ def _collect(per_token: bool, modules: list[ModuleInput], p: int, out: Tensor, l
         d.g_seq_stride, d.g_tok_stride = g.stride(0), g.stride(1)
         d.out_col = m.out_col
         d.I, d.O = I, O
-    if lengths is not None:
-        if lengths.dtype != torch.int32 or lengths.numel() != N or not lengths.is_contiguous():
-            raise ValueError("lengths must be a contiguous int32 vector of N elements")
-        _need_gpu(lengths, "lengths")
-    if rows is not None:
-        if rows.dtype != torch.int64 or rows.numel() != N or not rows.is_contiguous():
-            raise ValueError("row indices / offsets must be a contiguous int64 vector of N elements")
-        _need_gpu(rows, "rows")
+    _check_batch_vectors(lengths, rows, N, out.device)
     if static_scratch:
         rc = lib.bgx_collect_seq_static(descs, len(modules), N, S, p, dtype_code(in_dtype), _ptr(lengths), _ptr(rows),
                                         _ptr(out), out.stride(0), dtype_code(out.dtype), lo, hi, _stream())
@@ -257,9 +265,7 @@ def collect_prepared(per_token: bool, items: list, p: int, out: Tensor, lengths:
         d.a_seq_stride, d.a_tok_stride = a.stride(0), a.stride(1)
         d.g_seq_stride, d.g_tok_stride = g.stride(0), g.stride(1)
         nbytes_alg += pm.I + pm.O
-    for t, name, dt in ((lengths, "lengths", torch.int32), (rows, "rows", torch.int64)):
-        if t is not None and (t.dtype != dt or t.numel() != N or not t.is_contiguous() or not t.is_cuda):
-            raise ValueError(f"{name} must be a contiguous {dt} GPU vector of N={N} elements")
+    _check_batch_vectors(lengths, rows, N, out.device)
     ws = _workspace(out.device, lib.bgx_collect_workspace_bytes_for(descs, n, N, S, p, dtype_code(in_dtype)), "collect")
     fn = lib.bgx_collect_tok if per_token else lib.bgx_collect_seq
     timer = collect_timer
@@ -390,6 +396,7 @@ def collect_adam(prep: AdamPrepared, a: Tensor, g: Tensor, out: Tensor, *, per_t
         raise ValueError("out must be a 2-D tensor with contiguous rows")
     if per_token and (lengths is None or rows is None):
         raise ValueError("per-token collection needs lengths and row offsets")
+    _check_batch_vectors(lengths, rows, N, out.device)
     if not per_token and chunk_tokens == 0:
         # Two ways to the per-sequence rows.  Normalising the summed gradient costs ~ N * O * I (bound by the
         # bytes of the [N, O, I] gradient); summing per-token results costs ~ N * S * p * O * I flops on the
@@ -454,9 +461,10 @@ def full_gradient(mod: FullGradModule, a: Tensor, g: Tensor, out: Tensor, *, per
     if g.stride(2) != 1:
         g = g.contiguous()
     code = dtype_code(a.dtype)
+    if per_token and (lengths is None or rows is None):
+        raise ValueError("per-token collection needs lengths and row offsets")
+    _check_batch_vectors(lengths, rows, N, out.device)
     if per_token:
-        if lengths is None or rows is None:
-            raise ValueError("per-token collection needs lengths and row offsets")
         rc = lib.bgx_fullgrad_tok(_ptr(a), _ptr(g), a.stride(0), a.stride(1), g.stride(0), g.stride(1), N, S, I, O, code,
                                   _ptr(mod.row_scale), _ptr(mod.col_scale), _ptr(mod.adam_v), int(mod.collect_bias),
                                   _ptr(mod.bias_scale), _ptr(lengths), _ptr(rows), _ptr(out), out.stride(0),

@@ -169,7 +169,12 @@ int bgx_collect_seq(const bgx_module_desc* mods_host, int32_t n_modules,
  * modules too wide for on-chip projections run through the per-tile kernel
  * unless their fragment table fits as well).  All calls on one GPU share the
  * array: calls that may overlap on a GPU (different streams, different
- * threads) race; calls on one stream are ordered by the stream. */
+ * threads) race; calls on one stream are ordered by the stream.
+ * `stream` must belong to the device that is current in the calling thread
+ * (the array's address is taken for the current device).  The first call on a
+ * device looks that address up, reads the device's compute-unit count and
+ * opts the kernels into their LDS size; a caller that records the call into
+ * a HIP graph makes one call outside the capture first. */
 #define BGX_STATIC_SCRATCH_BYTES (16u << 20)
 int bgx_collect_seq_static(const bgx_module_desc* mods_host, int32_t n_modules,
                            int32_t N, int32_t S, int32_t p, int32_t in_dtype,
@@ -356,7 +361,10 @@ size_t bgx_scan_workspace_bytes_for(int32_t Q, int32_t k, int64_t chunk_rows,
  * Outputs, each optional (NULL to skip):
  *   topk_val_dev [Q, k] fp32, topk_idx_dev [Q, k] int64: per query the k
  *     largest scores in descending order, ties broken by lower row index
- *     (torch.topk, attributor.py:229-235); requires k <= n_rows, k <= 2048
+ *     (torch.topk, attributor.py:229-235); requires k <= n_rows, k <= 2048.
+ *     Scores that are NaN or -inf are never selected, whichever pass or
+ *     kernel meets them (torch.topk would rank NaN first); a query with
+ *     fewer than k selectable scores gets (-inf, -1) in its last entries
  *   row_max_dev [n_rows] fp32: max over queries (score_mode "nearest",
  *     scorer.py:111-113)
  *   row_mean_dev [n_rows] fp32: mean over queries, summed in a fixed order.

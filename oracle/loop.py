@@ -68,7 +68,8 @@ def losses_and_backward(model, x: Tensor, y: Tensor, loss_reduction: str = "sum"
                              label_smoothing=label_smoothing).reshape_as(y[:, 1:])
     losses = losses.sum(1) / denoms
     if advantage is not None:
-        losses = losses * torch.tensor(advantage, dtype=losses.dtype, device=losses.device)
+        # in place by an fp32 tensor: the product is formed in fp32 and rounded once to the dtype of the losses
+        losses *= torch.tensor(advantage, device=losses.device)
     losses.sum().backward()
     model.zero_grad()
     return losses

@@ -869,3 +869,27 @@ def test_adam_tables_stay_within_their_budget(device, monkeypatch):
     assert preps[0]._table is None and preps[1]._table is not None and preps[2]._table is not None
     assert torch.equal(preps[0].table, first)  # rebuilt
     assert preps[1]._table is None
+
+
+def test_full_gradient_refuses_malformed_lengths_and_rows(device):
+    """Both branches of the unprojected path check lengths (int32 [N]) and rows (int64 [N]) before launching."""
+    from bergson_amd import ops
+
+    N, S, I, O = 2, 8, 16, 32
+    a = torch.randn(N, S, I, device=device)
+    g = torch.randn(N, S, O, device=device)
+    mod = ops.FullGradModule(O=O, I=I, out_col=0)
+    out = torch.zeros(N * S, O * I, device=device)
+    good_l = torch.tensor([8, 5], dtype=torch.int32, device=device)
+    good_r = torch.tensor([0, 7], dtype=torch.int64, device=device)
+    for per_token in (False, True):
+        for lengths, rows in ((good_l.long(), good_r), (good_l, good_r.int()), (good_l[:1], good_r), (good_l, good_r[:1]),
+                              (good_l.cpu(), good_r)):
+            with pytest.raises((ValueError, RuntimeError)):
+                ops.full_gradient(mod, a, g, out, per_token=per_token, lengths=lengths, rows=rows, lo=-1e30, hi=1e30)
+    ops.full_gradient(mod, a, g, out, per_token=True, lengths=good_l, rows=good_r, lo=-1e30, hi=1e30)
+    ops.full_gradient(mod, a, g, out, per_token=False, lengths=good_l, rows=torch.tensor([0, 1], device=device),
+                      lo=-1e30, hi=1e30)
+    torch.cuda.synchronize()
+    want = torch.einsum("so,si->oi", g[1, :4], a[1, :4]).flatten()
+    assert torch.allclose(out[1], want, rtol=1e-4, atol=1e-4)

@@ -31,6 +31,42 @@ def test_allocate_batches_budget_order_and_oracle():
     assert max(len(b) for b in allocate_batches(lengths, 4096, max_batch_size=3)) <= 3
 
 
+def test_allocate_batches_hand_worked_answers():
+    """Known answers worked out by hand from the specification (bergson/data.py:239-377), for the product and
+    for the oracle's single-worker version.
+
+    lengths [5, 3, 9, 2, 9, 1, 4], budget 18: document 5 has one token and is left out; longest first with
+    ties in index order gives 2, 4, 0, 6, 1, 3 (lengths 9 9 5 4 3 2).  A batch headed by length 9 holds
+    18 // 9 = 2 documents, the next is headed by 5 and holds 18 // 5 = 3, the last takes what is left:
+    [[2, 4], [0, 6, 1], [3]].  random.seed(42); random.shuffle of three items puts them in the order 1, 0, 2.
+    """
+    from bergson_amd import allocate_batches
+    from bergson_amd.data import _allocate_batches_world, pack_by_padded_cost, spread_over_ranks
+
+    lengths = [5, 3, 9, 2, 9, 1, 4]
+    assert pack_by_padded_cost(lengths, 18) == [[2, 4], [0, 6, 1], [3]]
+    assert allocate_batches(lengths, 18) == [[0, 6, 1], [2, 4], [3]]
+    assert oloop.allocate_batches(lengths, 18) == [[0, 6, 1], [2, 4], [3]]
+    # at most two documents per batch: [2, 4], [0, 6], [1, 3]; a shuffle of three again
+    assert allocate_batches(lengths, 18, max_batch_size=2) == [[0, 6], [2, 4], [1, 3]]
+    assert oloop.allocate_batches(lengths, 18, max_batch_size=2) == [[0, 6], [2, 4], [1, 3]]
+    # another seed: random.seed(7) orders three items 2, 0, 1
+    assert allocate_batches(lengths, 18, seed=7) == [[3], [2, 4], [0, 6, 1]]
+    # two workers: three batches become four by peeling document 4 off the first batch that has two or more,
+    # [[2], [0, 6, 1], [3], [4]]; dealt in turn, worker 0 has [[2], [3]] and worker 1 [[0, 6, 1], [4]]; each list is
+    # shuffled with seed 42, which swaps a pair
+    assert _allocate_batches_world(lengths, 18, 2) == [[[3], [2]], [[4], [0, 6, 1]]]
+    assert _allocate_batches_world(lengths, 18, 2, ranks=[1]) == [[[4], [0, 6, 1]]]
+    # fewer batches than workers: documents are split off the largest batch until there are four,
+    # [0,1,2,3,4] -> [0,1,2,3] + [4] -> [0,1,2] + [3] -> [0,1] + [2], kept in the order of the binary heap
+    # on (-size, insertion number): [[0, 1], [3], [4], [2]]
+    assert spread_over_ranks([[0, 1, 2, 3, 4]], 4) == [[[0, 1]], [[3]], [[4]], [[2]]]
+    with pytest.raises(RuntimeError, match="at least one batch"):
+        spread_over_ranks([[0], [1]], 3)
+    with pytest.raises(RuntimeError, match="Not enough documents"):
+        _allocate_batches_world([1, 0, 5], 16, 2)
+
+
 def test_pad_and_tensor_masks():
     from bergson_amd import pad_and_tensor
 
@@ -103,6 +139,53 @@ def test_shapes_and_head_normalizers():
     assert h2.weight_avg_sq.shape == (4, 8) and h2.bias_avg_sq.tolist() == [8.0, 9.0, 10.0, 11.0]
 
 
+def test_heads_are_views_of_an_untouched_module():
+    """A split module reaches the backward hook once per head as a view that answers with the head's name and
+    width; the module keeps its own name and width throughout, also when the hook raises."""
+    from bergson_amd import AttentionConfig, GradientProcessor, HookCollectorBase
+    from bergson_amd.collector import HeadView
+
+    m = _Toy()
+    seen = []
+
+    class Probe(HookCollectorBase):
+        def setup(self): ...
+        def teardown(self): ...
+        def process_batch(self, indices, **k): ...
+
+        @HookCollectorBase.split_attention_heads
+        def backward_hook(self, module, g):
+            assert isinstance(module, nn.Linear)
+            seen.append((module._name, module.out_features, module.in_features, tuple(g.shape), g.data_ptr(),
+                         m.attn._name, m.attn.out_features, type(module) is HeadView or module is m.attn or module is m.mlp[0]))
+            if module._name.endswith("head_1") and getattr(self, "fail", False):
+                raise RuntimeError("boom")
+
+    c = Probe(model=m, processor=GradientProcessor(projection_dim=4), attention_cfgs={"attn": AttentionConfig(3, 4, 2)})
+    m.attn._name, m.mlp[0]._name = "attn", "mlp.0"
+    g = torch.zeros(2, 5, 12)
+    c.backward_hook(m.attn, g)
+    assert [(s[0], s[1], s[2], s[3]) for s in seen] == [(f"attn.head_{h}", 4, 8, (2, 5, 4)) for h in range(3)]
+    assert [s[4] for s in seen] == [g.data_ptr() + 16 * h for h in range(3)]  # views into g, nothing copied
+    assert all(s[5] == "attn" and s[6] == 12 and s[7] for s in seen)
+    seen.clear()
+    c.backward_hook(m.mlp[0], torch.zeros(2, 5, 16))  # an ordinary module goes through as itself
+    assert seen[0][:4] == ("mlp.0", 16, 8, (2, 5, 16))
+    c.fail = True
+    with pytest.raises(RuntimeError, match="boom"):
+        c.backward_hook(m.attn, g)
+    assert m.attn._name == "attn" and m.attn.out_features == 12
+    with pytest.raises(AssertionError, match="output features"):
+        Probe(model=m, processor=GradientProcessor(projection_dim=4),
+              attention_cfgs={"attn": AttentionConfig(2, 4, 2)}).backward_hook(m.attn, g)
+    # attributes set through a view land on the module (the kept input, for one)
+    view = HeadView(m.attn, c.blocks_of("attn")[2])
+    view._inputs = g
+    assert m.attn._inputs is g
+    del view._inputs
+    assert not hasattr(m.attn, "_inputs")
+
+
 def test_projection_cache_and_roles():
     from bergson_amd import GradientProcessor
 
@@ -165,6 +248,28 @@ def test_no_cpu_fallback():
         mod._inputs = torch.randn(1, 3, 8)
         with pytest.raises(RuntimeError, match="no CPU path"):
             c._compute_gradient(mod, torch.randn(1, 3, 12))
+
+
+def test_batch_vectors_are_checked_before_any_launch():
+    """lengths / rows of a wrong dtype, size or layout are refused on the host (a kernel would read garbage
+    lengths or scatter out of range); the check comes before the one for the device, so it runs here."""
+    from bergson_amd import ops
+
+    dev = torch.device("cpu")
+    ok_l, ok_r = torch.zeros(3, dtype=torch.int32), torch.zeros(3, dtype=torch.int64)
+    with pytest.raises(ValueError, match="lengths must be a contiguous int32"):
+        ops._check_batch_vectors(ok_r, None, 3, dev)
+    with pytest.raises(ValueError, match="offsets must be a contiguous int64"):
+        ops._check_batch_vectors(None, ok_l, 3, dev)
+    with pytest.raises(ValueError, match="N=4"):
+        ops._check_batch_vectors(ok_l, None, 4, dev)
+    with pytest.raises(ValueError, match="contiguous"):
+        ops._check_batch_vectors(torch.zeros(6, dtype=torch.int32)[::2], None, 3, dev)
+    with pytest.raises(ValueError, match="vector"):
+        ops._check_batch_vectors(torch.zeros(3, 1, dtype=torch.int32), None, 3, dev)
+    with pytest.raises(RuntimeError, match="no CPU path"):   # well-formed vectors: only then the device matters
+        ops._check_batch_vectors(ok_l, ok_r, 3, dev)
+    ops._check_batch_vectors(None, None, 3, dev)
 
 
 def test_product_does_not_import_the_oracle():

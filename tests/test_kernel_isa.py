@@ -1,5 +1,8 @@
 """Build-time properties of the hand-scheduled kernels that no numerical test can be relied on to catch.
 
+The rules themselves live in bergson_amd/isa_checks.py, and `build_ext.build()` applies them to every library it
+links; this file runs them on a fresh compilation and checks that they do report violations.
+
 The kernel issues its LDS fragment reads and its matrix instructions as inline assembly and waits for the reads
 itself; to the compiler the value of a read is there as soon as the statement is.  Should the register allocator
 run out of registers inside the tile loop (the kernel uses all 512 of a wave), it would store such a value to
@@ -46,29 +49,12 @@ def isa(tmp_path_factory):
     return {"scan.hip": texts[0], "adam.hip": texts[1]}
 
 
-@pytest.fixture(scope="module")
-def scan_isa(isa):
-    return isa["scan.hip"]
-
-
 @pytest.mark.parametrize("norms_given", [0, 1])
 @pytest.mark.parametrize("elem", ["5f16_t", "6bf16_t"])
-def test_wide_scan_kernel_keeps_its_fragments_in_registers(scan_isa, elem, norms_given):
-    name = f"_ZN3bgx16scan_wide_kernelINS_{elem}ELb{norms_given}EEEvNS_8ScanArgsE"
-    m = re.search(rf"^{name}:[^\n]*\n(.*?)\n\s*s_endpgm", scan_isa, re.S | re.M)
-    assert m, f"{name} not found in the compiled code"
-    lines = m.group(1).splitlines()
-    reads = [i for i, l in enumerate(lines) if "ds_read_b128" in l]
-    headers = [i for i, l in enumerate(lines) if "Loop Header" in l and i > reads[0]]
-    back = [i for i, l in enumerate(lines) if re.search(r"s_cbranch_scc\d\s+\.LBB", l) and i > headers[0]]
-    assert reads and headers and back
-    loop_end = back[0]
-    body = lines[reads[0]:loop_end + 1]
-    assert sum("v_mfma_f32_32x32x16" in l for l in lines[headers[0]:loop_end]) == 96, "one copy of the tile code"
-    scratch = [l.strip() for l in body if "scratch_" in l]
-    assert not scratch, f"scratch traffic between the first fragment read and the end of the tile loop: {scratch[:4]}"
-    assert not any(re.search(r"\bs_load|s_buffer_load", l) for l in lines[headers[0]:loop_end]), \
-        "scalar loads inside the loop share the counter the fragment waits count on"
+def test_wide_scan_kernel_keeps_its_fragments_in_registers(isa, elem, norms_given):
+    from bergson_amd import isa_checks
+
+    assert isa_checks.wide_scan_kernel(isa["scan.hip"], elem, norms_given) == []
 
 
 @pytest.mark.parametrize("source,pattern", [
@@ -77,40 +63,42 @@ def test_wide_scan_kernel_keeps_its_fragments_in_registers(scan_isa, elem, norms
 ])
 def test_direct_to_lds_kernels_use_no_scratch(isa, source, pattern):
     """Every instantiation: no scratch instruction anywhere and a private segment of zero bytes."""
-    text = isa[source]
-    names = sorted(set(re.findall(rf"^({pattern}):", text, re.M)))
-    assert names, f"no kernel matching {pattern} in {source}"
-    for name in names:
-        m = re.search(rf"^{re.escape(name)}:[^\n]*\n(.*?)\n\s*s_endpgm", text, re.S | re.M)
-        assert m, name
-        assert "scratch_" not in m.group(1), f"{name} spills"
-        meta = re.search(rf"\.amdhsa_kernel {re.escape(name)}\n(.*?)\.end_amdhsa_kernel", text, re.S)
-        assert meta and re.search(r"\.amdhsa_private_segment_fixed_size 0\b", meta.group(1)), name
+    from bergson_amd import isa_checks
+
+    assert isa_checks.no_scratch(isa[source], pattern) == []
 
 
 @pytest.mark.parametrize("elem", ["5f16_t", "6bf16_t"])
 def test_wide_adam_kernel_keeps_its_pipeline(isa, elem):
-    name = f"_ZN3bgx22adam_fused_wide_kernelINS_{elem}EEEvNS_9FusedArgsE"
-    text = isa["adam.hip"]
-    m = re.search(rf"^{name}:[^\n]*\n(.*?)\n\s*s_endpgm", text, re.S | re.M)
-    assert m, f"{name} not found in the compiled code"
-    meta = re.search(rf"\.amdhsa_kernel {re.escape(name)}\n(.*?)\.end_amdhsa_kernel", text, re.S)
-    assert meta and re.search(r"\.amdhsa_private_segment_fixed_size 0\b", meta.group(1))
-    lines = [l.strip() for l in m.group(1).splitlines()]
-    lines = [l for l in lines if l and not l.startswith(";")]
-    assert not any("scratch_" in l for l in lines), "spills"
-    mfma = [i for i, l in enumerate(lines) if l.startswith("v_mfma_f32_32x32x16")]
-    body = lines[mfma[0]:mfma[-1] + 1]
-    # five copies of the K tile (64 each) and four g slices (8 each)
-    assert len(mfma) == 5 * 64 + 4 * 8
-    assert not any(re.match(r"s_waitcnt.*vmcnt\(0\)", l) for l in body), "a wait for every load inside the pipeline"
-    assert not any(re.search(r"\bs_load|s_buffer_load|flat_load|global_load_dword", l) for l in body), \
-        "memory reads other than the direct-to-LDS loads inside the pipeline"
-    assert not any(l.startswith(("v_accvgpr_write", "v_accvgpr_mov")) for l in body), "accumulators moved between the files"
-    # 256 accumulators are read once per chunk, 64 per slice
-    assert sum(l.startswith("v_accvgpr_read") for l in body) == 256
-    # the second pass's MFMAs (ordinary registers as destination) follow an s_nop 1
-    second = [i for i in mfma if re.match(r"v_mfma\S+ v\[", lines[i])]
-    assert len(second) == 32
-    for i in second:
-        assert lines[i - 1] == "s_nop 1", (lines[i - 2:i + 1])
+    from bergson_amd import isa_checks
+
+    assert isa_checks.wide_adam_kernel(isa["adam.hip"], elem) == []
+
+
+def test_the_checks_see_a_violation(isa):
+    """The inspection is not vacuous: a scratch store planted in the tile loop, a dropped wait state and a
+    missing kernel are each reported."""
+    from bergson_amd import isa_checks
+
+    text = isa["scan.hip"]
+    name = "_ZN3bgx16scan_wide_kernelINS_5f16_tELb0EEEvNS_8ScanArgsE"
+    start = text.index(f"\n{name}:")
+    at = text.index("v_mfma_f32_32x32x16", text.index("Loop Header", text.index("ds_read_b128", start)))
+    planted = text[:at] + "scratch_store_dword off, v0, off\n\t" + text[at:]
+    assert any("scratch" in v for v in isa_checks.wide_scan_kernel(planted, "5f16_t", 0))
+    adam = isa["adam.hip"].replace("s_nop 1", "s_nop 0")
+    assert any("s_nop" in v for v in isa_checks.wide_adam_kernel(adam, "6bf16_t"))
+    assert isa_checks.wide_scan_kernel("", "5f16_t", 0) and isa_checks.no_scratch("", "_ZN3bgx18scan_direct_kernelI\\S*")
+
+
+def test_build_refuses_a_library_that_breaks_the_rules(monkeypatch):
+    """build() runs the same inspection before it links (here with the inspection made to fail, and the
+    compile and link steps left out)."""
+    from bergson_amd import build_ext, isa_checks
+
+    monkeypatch.setattr(build_ext, "_compile", lambda src, verbose, temps=None: build_ext.CSRC / "x.o")
+    monkeypatch.setattr(build_ext, "device_assembly", lambda temps, src: "")
+    monkeypatch.setattr(build_ext.Path, "unlink", lambda self, missing_ok=False: None)
+    with pytest.raises(RuntimeError, match="scheduling rules"):
+        build_ext.build(verbose=False)
+    assert isa_checks.all_violations({"scan.hip": "", "adam.hip": ""})

@@ -371,3 +371,69 @@ def test_scan_with_known_row_norms_equals_the_plain_scan_bitwise(device):
         assert torch.equal(plain.row_mean, known.row_mean)
     with pytest.raises(ValueError):
         ops.scan(store, q, unit_norm=True, k=10, row_sumsq=plain.sumsq[:-1])
+
+
+@pytest.mark.parametrize("n,D,Q", [(9000, 128, 5), (9000, 128, 48), (12000, 128, 300), (140000, 64, 8)])
+def test_scan_rows_with_nan_scores_are_never_selected(device, n, D, Q):
+    """A row whose score is NaN (a NaN or infinite element) is left out of the top-k whichever pass and kernel
+    meets it -- inside the first, threshold-free pass (rows 7, 4000 of the tile scans' 4096; any row of the
+    streaming scan's first 65 536) or beyond it -- so the result is the oracle's on the store without those
+    rows.  The last shape runs the few-queries streaming kernel."""
+    from bergson_amd import ops
+
+    store, queries = make_store(n, D, Q, torch.float16, seed=n + Q, outliers=False)
+    bad = [7, 4000, 4100, n - 3]
+    store[bad[0], 3] = float("nan")
+    store[bad[1], 5] = float("inf")
+    store[bad[2], 0] = float("nan")
+    store[bad[3], 9] = float("-inf")
+    qd = unit_queries(queries, torch.float16).to(torch.float16)
+    clean = store.clone()
+    clean[bad] = 0
+    ref = oscan.scorer_score({"m": clean}, {"m": qd}, ["m"], dtype=torch.float32, unit_normalize=True).T
+    ref[:, bad] = float("-inf")
+    for known in (False, True):
+        res = ops.scan(store.to(device), qd.to(device), unit_norm=True, k=50, want_sumsq=True)
+        if known:
+            res = ops.scan(store.to(device), qd.to(device), unit_norm=True, k=50, row_sumsq=res.sumsq)
+        torch.cuda.synchronize()
+        idx = res.topk_indices.cpu()
+        assert not set(idx.flatten().tolist()) & set(bad)
+        assert torch.isfinite(res.topk_values).all()
+        check_topk(res.topk_values.cpu(), idx, ref, 50)
+
+
+def test_scan_fewer_selectable_rows_than_k(device):
+    """Twenty rows of which fifteen score NaN, k = 10: the five real scores in order, then (-inf, -1)."""
+    from bergson_amd import ops
+
+    store, queries = make_store(20, 64, 3, torch.float32, seed=2, outliers=False)
+    good = [1, 4, 9, 10, 17]
+    for r in range(20):
+        if r not in good:
+            store[r, r % 64] = float("nan")
+    res = ops.scan(store.to(device), queries.to(device), unit_norm=False, k=10)
+    torch.cuda.synchronize()
+    ref = queries @ store[good].T
+    rv, ri = torch.topk(ref, 5, dim=1)
+    assert torch.allclose(res.topk_values.cpu()[:, :5], rv, rtol=1e-5, atol=1e-5)
+    assert torch.equal(res.topk_indices.cpu()[:, :5], torch.tensor(good)[ri])
+    assert (res.topk_values.cpu()[:, 5:] == float("-inf")).all() and (res.topk_indices.cpu()[:, 5:] == -1).all()
+
+
+@pytest.mark.parametrize("Q", [6, 70, 200])
+def test_scan_passes_shorter_than_k(device, Q):
+    """An explicit chunk_rows below k: the early passes hold fewer than k rows, no threshold exists until k
+    scores have been seen, and the result is still the oracle's."""
+    from bergson_amd import ops
+
+    n, D, k = 3000, 256, 500
+    store, queries = make_store(n, D, Q, torch.float16, seed=77)
+    qd = unit_queries(queries, torch.float16).to(torch.float16)
+    ref = oscan.scorer_score({"m": store}, {"m": qd}, ["m"], dtype=torch.float32, unit_normalize=True).T
+    res = ops.scan(store.to(device), qd.to(device), unit_norm=True, k=k, chunk_rows=256)
+    torch.cuda.synchronize()
+    check_topk(res.topk_values.cpu(), res.topk_indices.cpu(), ref, k)
+    whole = ops.scan(store.to(device), qd.to(device), unit_norm=True, k=k)
+    torch.cuda.synchronize()
+    assert torch.equal(whole.topk_indices, res.topk_indices) and torch.equal(whole.topk_values, res.topk_values)

@@ -71,6 +71,30 @@ def test_static_scratch_entry_equals_the_workspace_entry(device, dtype, out_dtyp
         assert got[untouched].abs().sum() == 0
 
 
+def test_static_scratch_entry_allocates_no_device_memory(device):
+    """The property the entry point is named for: a call (after the first on the device, which looks up the
+    array's address) leaves the device's free memory and torch's allocator exactly where they were."""
+    from bergson_amd import ops
+
+    p, N, S, lengths = 16, 2, 200, [200, 77]
+    mods = _case(N, S, [(128, 256), (256, 128)], p, torch.bfloat16, 90, lengths)
+    inputs = [ops.ModuleInput(a=a.to(device), g=g.to(device), r_in=right.to(device), r_out=left.to(device),
+                              out_col=k * p * p) for k, (a, g, left, right, _norm) in enumerate(mods)]
+    out = torch.zeros(N, len(mods) * p * p, dtype=torch.float16, device=device)
+    ldev = torch.tensor(lengths, dtype=torch.int32, device=device)
+    ops.collect_seq_static(inputs, p, out, lengths=ldev)   # warm-up: first use on this device
+    torch.cuda.synchronize()
+    first = out.clone()
+    free0, _ = torch.cuda.mem_get_info()
+    held0, reserved0 = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    for _ in range(3):
+        ops.collect_seq_static(inputs, p, out, lengths=ldev)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == held0 and torch.cuda.memory_reserved() == reserved0
+    assert torch.cuda.mem_get_info()[0] == free0
+    assert torch.equal(out, first)
+
+
 def test_static_scratch_entry_refuses_what_does_not_fit(device):
     from bergson_amd import _lib
 
