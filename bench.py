@@ -27,7 +27,10 @@ One JSON line is printed.  It also carries
                 reference's search on a slice of the store;
   per_token     configs[1]'s modules with one row per token (attribute_tokens), kernel only;
   llama8b_layers  configs[4]'s module shapes through a 4-layer Llama-3-8B-shaped model;
-  adam_per_token  configs[3]'s hot kernel.
+  adam_per_token  configs[3]'s hot kernel, and `end_to_end`: the product loop on a Pythia-410m-shaped model over a
+                slice of that configuration, into the real 98 304-wide per-token store;
+  config1       configs[0], the one configuration the reference's CPU path runs, in full on both sides: the product
+                loop on the GPU and the oracle loop on the host cores.
 """
 from __future__ import annotations
 
@@ -84,6 +87,7 @@ def parse_args():
                     help="batches the stock-PyTorch op sequence is timed on, on this GPU")
     ap.add_argument("--llama-only", action="store_true", help="run the Llama-shaped leg alone and print its entry")
     ap.add_argument("--per-token-only", action="store_true", help="run the per-token collection leg alone")
+    ap.add_argument("--config1-only", action="store_true", help="run configs[0] (GPU and CPU in full) alone")
     ap.add_argument("--adam-only", action="store_true",
                     help="run the per-token Adam leg alone and print its entry (for counter runs on that kernel)")
     ap.add_argument("--plain-loop", action="store_true",
@@ -295,7 +299,21 @@ def scan_leg(args, torch, device):
         "what": "bgx_scan_known_norms: row sums of squares taken from an earlier scan of the store instead of "
                 "being summed again in the K loop",
     }
-    del sumsq, res_known
+    # the one pass that forms those sums when an index is loaded (Attributor: the reference normalises the index
+    # at load time), bit-equal to the sums the scan hands out
+    loaded = ops.row_sumsq(store)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        ops.row_sumsq(store)
+    e1.record()
+    torch.cuda.synchronize()
+    ms_norms = e0.elapsed_time(e1) / reps
+    out["row_norms_at_load"] = {
+        "ms": ms_norms, "equal_to_the_scans_own_sums": bool(torch.equal(loaded, sumsq)),
+        "roofline": {"bound": "hbm", "achieved": n * D * 2 / (ms_norms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": n * D * 2 / (ms_norms * 1e-3) / 1e9 / HBM_PEAK_GBS, "kernel": "bgx::row_sumsq_kernel<f16_t, true>"}}
+    del sumsq, res_known, loaded
     # the HBM-bound regime: few queries per pass (the streaming kernel, one block of 16 queries or two)
     for nq in (32, 8):
         qs = qd[:nq].contiguous()
@@ -441,17 +459,20 @@ def adam_leg(args, torch, device):
     rnd = lambda *shape: torch.randn(*shape, generator=gen, device=device)
     lengths = torch.full((N,), S, dtype=torch.int32, device=device)
     offsets = torch.arange(N, device=device, dtype=torch.int64) * (S - 1)
-    out = torch.zeros(N * (S - 1), p * p, device=device, dtype=torch.bfloat16)
+    # the configuration's store layout: rows of 96 modules x p x p values, a module's block 196 608 bytes further on
+    # in every row (the four modules timed here write blocks 40..43)
+    n_blocks = 96
+    out = torch.zeros(N * (S - 1), n_blocks * p * p, device=device, dtype=torch.bfloat16)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     # 30 timed launches behind 5 untimed ones per module: the first launches of a burst run at lower clocks (5 timed
     # launches read 7 % slower than 60), and the configuration this stands for issues 96 of them per batch
     reps, total_ms, total_flops, modules = 30, 0.0, 0.0, {}
-    for name, (I, O) in (("query_key_value", (d, 3 * d)), ("dense", (d, d)), ("dense_h_to_4h", (d, 4 * d)),
-                         ("dense_4h_to_h", (4 * d, d))):
+    for block, (name, (I, O)) in enumerate((("query_key_value", (d, 3 * d)), ("dense", (d, d)),
+                                            ("dense_h_to_4h", (d, 4 * d)), ("dense_4h_to_h", (4 * d, d)))):
         a = rnd(N, S, I).to(torch.bfloat16)
         g = (rnd(N, S, O) * 0.01).to(torch.bfloat16)
         v = torch.rand(O, I, generator=gen, device=device) * 1e-5 + 1e-10
-        prep = ops.AdamPrepared(rnd(p, I).to(torch.bfloat16), rnd(p, O).to(torch.bfloat16), v, 0)
+        prep = ops.AdamPrepared(rnd(p, I).to(torch.bfloat16), rnd(p, O).to(torch.bfloat16), v, (40 + block) * p * p)
         run = lambda: ops.collect_adam(prep, a, g, out, per_token=True, lengths=lengths, rows=offsets, lo=-3e38,
                                        hi=3e38)
         for _ in range(5):
@@ -469,12 +490,134 @@ def adam_leg(args, torch, device):
         total_flops += flops
         del a, g, v, prep
     tf = total_flops / (total_ms * 1e-3) / 1e12
-    return {"workload": "configs[3]: one Pythia-410m layer, 4 x 1024 tokens, p=32, Adam, per-token rows (bf16)",
+    del out
+    torch.cuda.empty_cache()
+    return {"workload": "configs[3]: one Pythia-410m layer, 4 x 1024 tokens, p=32, Adam, per-token rows (bf16) "
+                        "written as blocks of the configuration's 98 304-wide store rows",
+            "end_to_end": adam_end_to_end(torch, device),
             "ms_per_layer": total_ms, "tokens_per_s_24_layers_hooks_only": N * S / (total_ms * 24e-3),
             "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": tf / MFMA_F16_PEAK_TFLOPS, "traffic": ADAM_TRAFFIC_BYTES_PER_LAYER,
                          "kernel": "bgx::adam_fused_wide_kernel<bf16_t>"},
             "modules": modules}
+
+
+def adam_end_to_end(torch, device, n_batches=8, warm=2):
+    """configs[3] through the product loop on a slice: a Pythia-410m-shaped model (24 layers, 96 hooked modules),
+    documents of 1024 tokens in batches of 4, p = 32, Adam second moments |N(0,1)| * 1e-5 for every module, per-token
+    rows of 98 304 bf16 values written into the device-resident store (`warm` untimed batches first, in which the
+    Adam tables are built)."""
+    import bergson_amd as B
+    from bergson_amd.collector import CollectorComputer
+    from bergson_amd.synthetic import ListDataset, make_gpt_neox, random_docs
+
+    p, per_batch, S = 32, 4, 1024
+    lengths = [S] * (per_batch * (n_batches + warm))
+    data = ListDataset(random_docs(lengths, seed=4))
+    batches = [list(range(per_batch * i, per_batch * (i + 1))) for i in range(n_batches + warm)]
+    model = make_gpt_neox("pythia-410m", torch.bfloat16, device, seed=0)
+    gen = torch.Generator(device=device).manual_seed(3)
+    normalizers = {}
+    for name, mod in model.base_model.named_modules():
+        if isinstance(mod, torch.nn.Linear):
+            v = torch.randn(mod.out_features, mod.in_features, generator=gen, device=device).abs_() * 1e-5
+            normalizers[name] = B.AdamNormalizer(weight_avg_sq=v)
+    processor = B.GradientProcessor(normalizers=normalizers, projection_dim=p, projection_type="normal")
+    cfg = B.IndexConfig(run_path="", projection_dim=p, projection_type="normal", token_batch_size=per_batch * S,
+                        attribute_tokens=True)
+
+    from bergson_amd.collector import OverlappedSteps
+
+    staged = []
+    for indices in batches:
+        b = data[indices]
+        x, y, _, mask = B.pad_and_tensor(b["input_ids"], device=device, sync_max_len=False)
+        staged.append((indices, b, x, y, mask))
+    col = B.GradientCollector(model=model.base_model, cfg=cfg, data=data, processor=processor)
+    steps = OverlappedSteps(model, col, cfg)
+    for item in staged[:warm]:
+        steps.step(*item)
+    steps.drain()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for item in staged[warm:]:
+        steps.step(*item)
+    steps.drain()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    steps.close()
+    device_resident = bool(col.builder.direct)
+    f0 = time.perf_counter()
+    col.builder.flush()
+    torch.cuda.synchronize()
+    flush_s = time.perf_counter() - f0
+    col.remove_hooks()
+    rows, width = col.builder.grad_buffer.shape
+    filled = int((col.builder.grad_buffer[:, 40 * p * p] != 0).sum())
+    modules = len(col.target_info)
+    del col, steps, model, normalizers, processor, staged
+    torch.cuda.empty_cache()
+    tokens = n_batches * per_batch * S
+    return {"workload": f"configs[3] on a slice: Pythia-410m-shaped GPT-NeoX bf16 ({modules} hooked modules), {n_batches} "
+                        f"batches of {per_batch} x {S} tokens after {warm} untimed ones (in which the Adam tables are "
+                        f"built), p={p}, Adam normalizer on every module, per-token rows of {width} bf16 values",
+            "value": tokens / dt, "unit": "tokens/s", "ms_per_batch": dt / n_batches * 1e3, "batches": n_batches,
+            "store_rows": rows, "store_row_width": width, "store_device_resident": device_resident,
+            "rows_written": filled,
+            "timed_region": "the product loop (OverlappedSteps: forward, backward, 96 fused launches per batch) over the "
+                            "timed batches, token ids already on the device, rows landing in the device-resident store",
+            "flush_seconds": flush_s,
+            "flush": f"copying the {rows * width * 2 / 1e9:.1f} GB store to host memory afterwards (once per job)"}
+
+
+def config1_leg(args, torch, device):
+    """configs[0] in full, the one configuration the reference's CPU path runs: Pythia-14m-shaped fp32 model, 64
+    documents of 256 uniform-random tokens, 2048-token batches, p = 16 on the 24 Linear modules, no normalizer,
+    per-sequence rows -- the product loop on the GPU (second pass over the data in this process) beside the
+    oracle's loop on the host cores, both over all 16 384 tokens, and their rows compared."""
+    import numpy as np
+
+    import bergson_amd as B
+    from bergson_amd.collector import CollectorComputer
+    from bergson_amd.synthetic import ListDataset, make_gpt_neox, random_docs
+    from oracle import loop as oloop
+
+    lengths = [256] * 64
+    docs = random_docs(lengths, seed=0)
+    data = ListDataset(docs)
+    batches = B.allocate_batches(lengths, 2048)
+    tokens = sum(lengths)
+    gpu = make_gpt_neox("pythia-14m", torch.float32, device, seed=0)
+    cfg = B.IndexConfig(run_path="", projection_dim=16, projection_type="normal", token_batch_size=2048)
+    processor = B.GradientProcessor(projection_dim=16, projection_type="normal")
+
+    def run():
+        col = B.GradientCollector(model=gpu.base_model, cfg=cfg, data=data, processor=processor)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        CollectorComputer(model=gpu, data=data, collector=col, batches=batches, cfg=cfg).run_with_collector_hooks()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, col
+
+    run()
+    dt, col = run()
+    got = torch.from_numpy(np.array(col.builder.grad_buffer))
+    out = {"workload": "configs[0]: Pythia-14m-shaped GPT-NeoX fp32, 64 x 256 tokens, 2048-token batches, p=16 normal "
+                       "projections on 24 modules, no normalizer, per-sequence rows",
+           "value": tokens / dt, "unit": "tokens/s", "seconds": dt, "tokens": tokens, "batches": len(batches),
+           "dtype": "f32"}
+    if not args.no_cpu_baseline:
+        cpu = make_gpt_neox("pythia-14m", torch.float32, "cpu", seed=0)
+        t0 = time.perf_counter()
+        want, _ = oloop.collect(cpu, cpu.base_model, docs, batches, p=16)
+        cdt = time.perf_counter() - t0
+        err = ((got.double() - want.double()).norm() / want.double().norm()).item()
+        out["cpu_baseline"] = {"value": tokens / cdt, "unit": "tokens/s", "cores": torch.get_num_threads(),
+                               "kind": "port", "seconds": cdt,
+                               "sample": f"the whole configuration: {tokens} tokens in {cdt:.1f} s (reference op "
+                                         "sequence on PyTorch CPU, fp32)"}
+        out["rel_l2_gpu_vs_cpu_rows"] = err
+    return out
 
 
 def cpu_baseline_leg(args, torch, docs, lengths):
@@ -502,6 +645,25 @@ def cpu_baseline_leg(args, torch, docs, lengths):
     return {"value": tok / dt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"{len(picked)} documents / {tok} tokens of the same workload in {dt:.1f} s "
                       f"(reference op sequence on PyTorch CPU, bf16 model, fp16 rows)"}
+
+
+def end_child_processes() -> list[str]:
+    """Names of the child processes this script still had when it was done (worker pools of the libraries it
+    used); they are ended, so that nothing outlives the benchmark."""
+    import multiprocessing
+
+    import psutil
+
+    names = []
+    for child in multiprocessing.active_children():
+        child.terminate()
+    for child in psutil.Process().children(recursive=True):
+        try:
+            names.append(" ".join(child.cmdline()[:3]) or child.name())
+            child.terminate()
+        except psutil.Error:
+            pass
+    return names
 
 
 def main():
@@ -537,6 +699,9 @@ def main():
     if args.llama_only:
         print(json.dumps({"llama8b_layers": llama_leg(args, torch, device)}))
         return
+    if args.config1_only:
+        print(json.dumps({"config1": config1_leg(args, torch, device)}))
+        return
     if args.per_token_only:
         print(json.dumps({"per_token": per_token_leg(args, torch, device)}))
         return
@@ -548,6 +713,7 @@ def main():
     per_token = None if args.no_scan else per_token_leg(args, torch, device)
     llama = None if args.no_scan else llama_leg(args, torch, device)
     adam = None if args.no_scan else adam_leg(args, torch, device)
+    config1 = None if args.no_scan else config1_leg(args, torch, device)
     cpu = None if args.no_cpu_baseline else cpu_baseline_leg(args, torch, docs, lengths)
 
     value = coll["tokens"] / coll["seconds"]
@@ -577,6 +743,9 @@ def main():
             "loop": coll["loop"],
             "timed_region": "CollectorComputer.run_with_collector_hooks over the timed batches: padding, upload of the "
                             "token ids, forward, backward, fused launch, store flush, teardown artefacts",
+            "warm_up_caveat": "in a fresh process the first ~50 batches of new shapes run at ~12 ms instead of ~8.8 (the "
+                              "libraries under the model load kernels and pick GEMM variants on first use): with fewer "
+                              "than ~50 untimed batches part of that falls into the timed steps and lowers `value`",
         },
         "prestaged": {"value": coll["tokens"] / coll["prestaged_seconds"], "unit": "tokens/s",
                       "ms_per_step": coll["prestaged_seconds"] / args.steps * 1e3,
@@ -602,7 +771,9 @@ def main():
         "per_token": per_token,
         "llama8b_layers": llama,
         "adam_per_token": adam,
+        "config1": config1,
     }
+    line["child_processes_at_exit"] = end_child_processes()
     print(json.dumps(line))
 
 

@@ -134,6 +134,7 @@ SIGNATURES: dict[str, tuple] = {
          C.c_int32, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
          C.c_size_t, C.c_int64, C.c_void_p],
     ),
+    "bgx_row_sumsq": (C.c_int, [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]),
     "bgx_scan_known_norms": (
         C.c_int,
         [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_int32, C.c_float, C.c_int32,

@@ -90,6 +90,8 @@ class Attributor:
         base = store_base_dtype(info)
         if base == "float64":
             raise TypeError("float64 stores are not supported by the scan kernels")
+        self._row_sumsq: Tensor | None = None
+        self._row_sumsq_of: tuple | None = None
         self.store = upload_store(load_gradients(index_path), base, self.device)
         self.N = self.store.shape[0]
         if self.preconditioner is not None and unit_norm:
@@ -99,9 +101,20 @@ class Attributor:
             free, _ = torch.cuda.mem_get_info(self.device)
             out_dtype = torch.float32 if self.store.numel() * 4 <= free // 2 else self.store.dtype
             self.store = self.preconditioner.apply_rows(self.store, self.grad_sizes, out_dtype=out_dtype)
-        # sums of squares of the store's rows, kept from the first unit-norm scan on: the reference normalises the
-        # index once at load time (attributor.py:137-167); here later scans take their row multipliers from this
-        self._row_sumsq: Tensor | None = None
+        if unit_norm:
+            self.row_sumsq()  # the reference normalises the index when it loads it (attributor.py:137-167)
+
+    def row_sumsq(self) -> Tensor:
+        """Sums of squares of the store's rows (one HBM-bound pass), kept for every search: the index-side
+        normalisation the reference applies once at load time (attributor.py:137-167), here as the row
+        multipliers the scan takes instead of summing the squares of every row again.  Recomputed when `store`
+        has been replaced or written to since (its storage, shape or version counter changed)."""
+        store = self.store
+        state = (store.data_ptr(), tuple(store.shape), store.dtype, store._version)
+        if self._row_sumsq is None or self._row_sumsq_of != state:
+            self._row_sumsq = ops.row_sumsq(store)
+            self._row_sumsq_of = state
+        return self._row_sumsq
 
     @property
     def grads(self) -> dict[str, Tensor]:
@@ -128,12 +141,9 @@ class Attributor:
         qmax = float(q.abs().max().item())
         shift = 0 if qmax == 0 or not math.isfinite(qmax) else -math.frexp(qmax)[1]
         qd = (q * (2.0 ** shift)).to(self.store.dtype)
+        norms = self.row_sumsq() if self.unit_norm else None
         if k <= ops.SCAN_KMAX:
-            first = self.unit_norm and self._row_sumsq is None
-            res = ops.scan(self.store, qd, unit_norm=self.unit_norm, k=k, query_scale=2.0 ** (-shift),
-                           want_sumsq=first, row_sumsq=self._row_sumsq)
-            if first:
-                self._row_sumsq = res.sumsq
+            res = ops.scan(self.store, qd, unit_norm=self.unit_norm, k=k, query_scale=2.0 ** (-shift), row_sumsq=norms)
             values, indices = res.topk_values, res.topk_indices
         else:
             # beyond the fused selection's capacity (k = None asks for a full ranking of the store): the
@@ -143,7 +153,7 @@ class Attributor:
             vals, idxs = [], []
             for lo in range(0, qd.shape[0], step):
                 res = ops.scan(self.store, qd[lo:lo + step].contiguous(), unit_norm=self.unit_norm,
-                               query_scale=2.0 ** (-shift), want_scores=True)
+                               query_scale=2.0 ** (-shift), want_scores=True, row_sumsq=norms)
                 v, i = torch.topk(res.scores.T, k, dim=1)
                 vals.append(v)
                 idxs.append(i)

@@ -118,6 +118,7 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
               float query_scale, int unit_norm, int k, int64_t row_base, float* topk_val, int64_t* topk_idx,
               float* row_max, float* row_mean, float* scores, float* sumsq, const float* sumsq_in, void* ws,
               size_t ws_bytes, int64_t chunk_rows, void* stream);
+int row_sumsq_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int dtype, float* sumsq, void* stream);
 size_t precond_workspace_bytes(int n_blocks);
 int block_gemm_impl(const void* in, int in_dtype, int64_t in_stride, void* out, int out_dtype, int64_t out_stride,
                     int64_t rows, const bgx_block_desc* blocks, int n_blocks, void* ws, size_t ws_bytes,
@@ -298,6 +299,11 @@ int bgx_scan(const void* store_dev, int64_t n_rows, int64_t D, int64_t store_row
   return bgx::scan_impl(store_dev, n_rows, D, store_row_stride, dtype, queries_dev, Q, query_scale, unit_norm, k,
                         row_base, topk_val_dev, topk_idx_dev, row_max_dev, row_mean_dev, scores_dev, sumsq_dev, nullptr,
                         workspace_dev, workspace_bytes, chunk_rows, stream);
+}
+
+int bgx_row_sumsq(const void* store_dev, int64_t n_rows, int64_t D, int64_t store_row_stride, int32_t dtype,
+                  float* row_sumsq_dev, void* stream) {
+  return bgx::row_sumsq_impl(store_dev, n_rows, D, store_row_stride, dtype, row_sumsq_dev, stream);
 }
 
 int bgx_scan_known_norms(const void* store_dev, int64_t n_rows, int64_t D, int64_t store_row_stride, int32_t dtype,

@@ -1420,6 +1420,39 @@ __global__ void scan_row_mean_kernel(const float* __restrict__ part, int n_parts
   row_mean[row0 + r] = s * inv_q;
 }
 
+// ---- row sums of squares on their own ---------------------------------------------------------------------
+// sumsq[n] = sum_k store[n, k]^2 in exactly the order the tile kernels form it inside a scan: one partial per
+// 16-byte position c of a 128-byte K tile, each running over the K tiles in ascending order, the eight partials
+// combined as ((c0 + c1) + (c2 + c3)) + ((c4 + c5) + (c6 + c7)).  The values are therefore the bits a scan's own
+// `sumsq` output holds (scan_gemm_kernel without its rotated start, scan_direct_kernel, scan_wide_kernel), and a
+// scan that is given them (bgx_scan_known_norms) returns the bits of a scan that computed them.
+// Eight lanes per row (lane c owns position c: a load instruction reads whole 128-byte lines of eight rows),
+// eight K tiles in flight per lane, every row read once with the non-temporal hint: bound by HBM.
+template <typename T, bool ALIGNED>
+__global__ __launch_bounds__(256) void row_sumsq_kernel(const T* __restrict__ store, int64_t n_rows, int64_t D,
+                                                        int64_t stride, float* __restrict__ sumsq) {
+  using M = Mma32<T>;
+  constexpr int EPL = M::EPL;
+  constexpr int BK = TILE_CHUNKS * EPL;  // elements per 128-byte K tile
+  constexpr int U = 8;
+  const int c = threadIdx.x & 7;
+  const int64_t row = (int64_t)blockIdx.x * 32 + (threadIdx.x >> 3);
+  const int64_t KT = (D + BK - 1) / BK;
+  float s = 0.f;
+  for (int64_t kt0 = 0; kt0 < KT; kt0 += U) {
+    uint4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      v[u] = load_chunk<T, ALIGNED, ALIGNED>(store, row, n_rows, stride, (kt0 + u) * BK + c * EPL, D);
+#pragma unroll
+    for (int u = 0; u < U; ++u) s = M::sumsq(v[u], s);  // a chunk past the end is zero and adds nothing
+  }
+  s += __shfl_xor(s, 1);
+  s += __shfl_xor(s, 2);
+  s += __shfl_xor(s, 4);
+  if (c == 0 && row < n_rows) sumsq[row] = s;
+}
+
 // ---- host side --------------------------------------------------------------------------------
 constexpr int64_t SCAN_DEFAULT_CHUNK = 65536;
 constexpr int64_t SCAN_FIRST_CHUNK = 4096;
@@ -1833,6 +1866,33 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
                        (const uint32_t*)row_max_enc, row_max, row_max ? n_rows : 0);
     BGX_HIP(hipGetLastError());
   }
+  return 0;
+}
+
+int row_sumsq_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int dtype, float* sumsq, void* stream) {
+  BGX_REQUIRE(store && sumsq, BGX_E_ARG, "row_sumsq: null store/sumsq");
+  BGX_REQUIRE(n_rows > 0 && D > 0 && stride >= D, BGX_E_ARG, "row_sumsq: n_rows=%lld D=%lld stride=%lld",
+              (long long)n_rows, (long long)D, (long long)stride);
+  BGX_REQUIRE(dtype >= BGX_F32 && dtype <= BGX_BF16, BGX_E_DTYPE, "row_sumsq: dtype=%d", dtype);
+  BGX_REQUIRE((n_rows + 31) / 32 <= 0x7fffffffLL, BGX_E_SHAPE, "row_sumsq: too many rows");
+  const int epl = dtype == BGX_F32 ? 4 : 8;
+  const bool aligned = ((uintptr_t)store % 16 == 0) && (D % epl == 0) && (stride % epl == 0);
+  const dim3 grid((unsigned)((n_rows + 31) / 32)), block(256);
+  hipStream_t st = (hipStream_t)stream;
+#define BGX_ROW_SUMSQ(T_)                                                                                        \
+  if (aligned)                                                                                                   \
+    hipLaunchKernelGGL((row_sumsq_kernel<T_, true>), grid, block, 0, st, (const T_*)store, n_rows, D, stride, sumsq); \
+  else                                                                                                           \
+    hipLaunchKernelGGL((row_sumsq_kernel<T_, false>), grid, block, 0, st, (const T_*)store, n_rows, D, stride, sumsq);
+  if (dtype == BGX_F16) {
+    BGX_ROW_SUMSQ(f16_t)
+  } else if (dtype == BGX_BF16) {
+    BGX_ROW_SUMSQ(bf16_t)
+  } else {
+    BGX_ROW_SUMSQ(float)
+  }
+#undef BGX_ROW_SUMSQ
+  BGX_HIP(hipGetLastError());
   return 0;
 }
 

@@ -611,6 +611,21 @@ def gram_accumulate(rows: Tensor, blocks: list[tuple[Tensor, int]]) -> None:
     _lib.check(rc, "bgx_gram_accumulate")
 
 
+def row_sumsq(store: Tensor) -> Tensor:
+    """fp32 [n] sums of squares of the rows of `store` in one HBM-bound pass: the values a scan's own `sumsq`
+    holds, bit for bit (see bgx_row_sumsq), so `scan(..., row_sumsq=row_sumsq(store))` equals a plain scan."""
+    lib = _lib.load()
+    _need_gpu(store, "store")
+    if store.dim() != 2 or store.stride(1) != 1:
+        raise ValueError("store must be 2-D with contiguous rows")
+    out = torch.empty((store.shape[0],), dtype=torch.float32, device=store.device)
+    if store.shape[0]:
+        rc = lib.bgx_row_sumsq(_ptr(store), store.shape[0], store.shape[1], store.stride(0), dtype_code(store.dtype),
+                               _ptr(out), _stream())
+        _lib.check(rc, "bgx_row_sumsq")
+    return out
+
+
 @dataclass
 class ScanResult:
     topk_values: Tensor | None = None  # [Q, k] fp32

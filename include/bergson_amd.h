@@ -383,8 +383,18 @@ int bgx_scan(const void* store_dev, int64_t n_rows, int64_t D,
              float* sumsq_dev, void* workspace_dev, size_t workspace_bytes,
              int64_t chunk_rows, void* stream);
 
+/* Sums of squares of the rows of a store, in one pass over it (bound by HBM):
+ * the index-side half of bergson/query/attributor.py:137-167, which
+ * normalises an index once when it is loaded.  row_sumsq_dev [n_rows] fp32
+ * receives exactly the values a bgx_scan of the same rows writes to its
+ * sumsq_dev (same order of additions), so a scan given them
+ * (bgx_scan_known_norms) returns the bits of a scan that formed them. */
+int bgx_row_sumsq(const void* store_dev, int64_t n_rows, int64_t D,
+                  int64_t store_row_stride, int32_t dtype, float* row_sumsq_dev,
+                  void* stream);
+
 /* bgx_scan for a store whose row sums of squares are known: row_sumsq_dev
- * [n_rows] is the sumsq_dev output of an earlier bgx_scan of the same rows.
+ * [n_rows] is the sumsq_dev output of an earlier bgx_scan of the same rows, or of bgx_row_sumsq.
  * The reference normalises an index once, when it loads it
  * (query/attributor.py:137-167), and scores it many times; this is the same
  * economy -- kernels that would otherwise sum the squares of every row in

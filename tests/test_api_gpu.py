@@ -219,6 +219,48 @@ def test_attributor_search_and_trace(device, tmp_path):
     assert result.indices[0, 0].item() == 3 and result.scores[0, 0].item() > 0.99
 
 
+def test_attributor_searches_again_and_notices_a_changed_store(device, tmp_path):
+    """The row norms are formed once when the index is loaded and serve every search: a search with 4 queries
+    and one with 300 (another kernel) against the oracle's search, and -- the norms being a cache of `store` --
+    rows edited in place or a replaced store are seen by the next search."""
+    from bergson_amd import Attributor, ops
+    from bergson_amd.data import create_index
+    from bergson_amd.gradients import GradientProcessor
+
+    gen = torch.Generator().manual_seed(11)
+    n, sizes = 6000, {"a": 256, "b": 128, "c": 128}
+    rows = torch.randn(n, 512, generator=gen) * (torch.rand(n, 1, generator=gen) * 3 + 0.1)
+    path = tmp_path / "idx"
+    mm = create_index(path, num_grads=n, grad_sizes=sizes, dtype="float16")
+    mm[:] = rows.to(torch.float16).numpy()
+    mm.flush()
+    GradientProcessor(projection_dim=16).save(path)
+    stored = torch.from_numpy(np.array(mm)).float()
+    index = {"a": stored[:, :256], "b": stored[:, 256:384], "c": stored[:, 384:]}
+    attr = Attributor(path, device="cuda:0", unit_norm=True)
+    assert attr._row_sumsq is not None   # formed at load time, before any search
+    assert torch.equal(attr._row_sumsq, ops.row_sumsq(attr.store))
+    for Q in (4, 300, 4):
+        picks = torch.randint(0, n, (Q,), generator=gen)
+        noisy = stored[picks] + 0.3 * torch.randn(Q, 512, generator=gen) * stored[picks].norm(dim=1, keepdim=True) / 512 ** 0.5
+        queries = {"a": noisy[:, :256], "b": noisy[:, 256:384], "c": noisy[:, 384:]}
+        vals, idx = attr.search({m: q.to(device) for m, q in queries.items()}, k=5)
+        ref_v, ref_i = oscan.attributor_search(index, queries, ["a", "b", "c"], 5, unit_norm=True)
+        assert (idx[:, 0].cpu() == picks).all()
+        assert (vals.cpu() - ref_v).abs().max().item() <= 1e-3
+        assert (idx.cpu() == ref_i).float().mean().item() >= 0.98   # neighbours within the tolerance may swap
+    # an in-place edit: row 17 becomes a scaled copy of the first query, and must now be its best match
+    first = torch.cat([queries[m][0] for m in ("a", "b", "c")])
+    attr.store[17] = (first * 100).to(torch.float16).to(device)
+    vals, idx = attr.search({m: q.to(device) for m, q in queries.items()}, k=2)
+    assert idx[0, 0].item() == 17 and abs(vals[0, 0].item() - 1.0) <= 1e-3
+    # a replaced store
+    attr.store = attr.store[:100].clone()
+    attr.N = 100
+    vals, idx = attr.search({m: q.to(device) for m, q in queries.items()}, k=2)
+    assert attr._row_sumsq.shape == (100,) and idx[0, 0].item() == 17
+
+
 def test_include_bias_end_to_end(device):
     """include_bias=True through the collector: every module's block against the oracle on captured (a, g)."""
     from bergson_amd import GradientCollector, GradientProcessor, IndexConfig

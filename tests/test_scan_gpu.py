@@ -437,3 +437,35 @@ def test_scan_passes_shorter_than_k(device, Q):
     whole = ops.scan(store.to(device), qd.to(device), unit_norm=True, k=k)
     torch.cuda.synchronize()
     assert torch.equal(whole.topk_indices, res.topk_indices) and torch.equal(whole.topk_values, res.topk_values)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("n,D", [(4096 + 24576 + 300, 256), (5000, 192), (1000, 12288), (777, 100)])
+def test_row_sumsq_equals_the_sums_a_scan_forms(device, dtype, n, D):
+    """bgx_row_sumsq, the one pass that stands for the reference's normalisation of an index at load time: against
+    float64, and bit for bit against the `sumsq` output of scans on the tile kernels (256 x 256 register-staged,
+    direct-to-LDS, 384 x 256 wide), whose order of additions it follows -- so a scan given these sums returns
+    exactly what a scan that forms them returns."""
+    from bergson_amd import ops
+
+    gen = torch.Generator().manual_seed(n + D)
+    store = (torch.randn(n, D, generator=gen) * torch.rand(n, 1, generator=gen) * 4).to(dtype)
+    store[5] = 0
+    dev_store = store.to(device)
+    got = ops.row_sumsq(dev_store)
+    torch.cuda.synchronize()
+    want = store.double().pow(2).sum(1)
+    assert torch.allclose(got.cpu().double(), want, rtol=2e-5, atol=0)  # fp32 running sums over up to 1536 K tiles
+    assert got[5].item() == 0.0
+    for Q in (300, 100):
+        q = torch.randn(Q, D, generator=gen).to(dtype).to(device)
+        plain = ops.scan(dev_store, q, unit_norm=True, k=10, want_sumsq=True, want_row_max=True)
+        given = ops.scan(dev_store, q, unit_norm=True, k=10, row_sumsq=got, want_row_max=True)
+        torch.cuda.synchronize()
+        assert torch.equal(plain.sumsq, got), Q
+        assert torch.equal(plain.topk_values, given.topk_values) and torch.equal(plain.topk_indices, given.topk_indices)
+        assert torch.equal(plain.row_max, given.row_max)
+    # a strided view (rows of a wider matrix) gives the same sums
+    wide = torch.zeros(n, D + 24, dtype=dtype, device=device)
+    wide[:, :D] = dev_store
+    assert torch.equal(ops.row_sumsq(wide[:, :D]), got)
