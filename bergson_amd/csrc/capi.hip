@@ -46,6 +46,7 @@ static const Switches* read_switches() {
   s->collect_staged = !off("BGX_COLLECT_STAGED");
   s->collect_persist = !off("BGX_COLLECT_PERSIST");
   s->collect_lpt_off = getenv("BGX_COLLECT_LPT_OFF") != nullptr;
+  s->collect_two_step_off = getenv("BGX_COLLECT_TWO_STEP_OFF") != nullptr;
   s->scan_direct_off = getenv("BGX_SCAN_DIRECT_OFF") != nullptr;
   s->scan_stream_off = getenv("BGX_SCAN_STREAM_OFF") != nullptr;
   s->scan_wide_off = getenv("BGX_SCAN_WIDE_OFF") != nullptr;

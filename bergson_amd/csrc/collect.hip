@@ -347,6 +347,7 @@ struct PersistArgs {
   const uint4* frag;        // RFG: scaled projection fragments of every module in global memory
   const int64_t* frag_off;  // RFG: [n_modules] first k-step of a module's fragments (r_in's, then r_out's)
   const int32_t* order;     // RFG: the items in the order the workgroups take them (wg_first indexes this list), or null
+  float* tokproj;           // per-token rows in two steps: [n_modules][N][S][2][16] a', g' of every token, or null
 };
 
 // x' = x @ R'^T for this wave's 16*MTW tokens over all of K, R' fragments read from LDS.
@@ -449,6 +450,49 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
   uint4 v[STAGED ? STREAM_Q : 1][2 * MTW];
   uint4 rq[RFG ? STREAM_Q : 1][2];  // RFG: the fragments that go with v
   bool primed = false;
+  // Two-step per-token rows: a tile leaves 16 * MTW tokens x 32 floats per wave, i.e. 8 * MTW registers per lane.
+  // They stay in registers until KEEP_TILES tiles have gathered or the range ends, and go to the workspace then:
+  // a store shares the in-order completion counter of the stream's loads, so the first wait behind a store also
+  // waits for the store's acknowledgement, which under this read load takes several microseconds -- once per
+  // tile that was a sixth of the kernel's time; at the end of a range nothing waits behind it.
+  // (Deferring wave 0's p x p partial of the per-sequence launches the same way changed nothing: 171.6 us either way.)
+  constexpr int KEEP_TILES = PER_TOKEN ? 8 : 1;
+  f32x4 keepA[KEEP_TILES][MTW], keepG[KEEP_TILES][MTW];
+  int64_t keep_at[KEEP_TILES];  // element offset of the tile's first token in tokproj
+  int keep_rows[KEEP_TILES];
+  int kept = 0;
+  auto flush_kept = [&]() {
+    if constexpr (PER_TOKEN) {
+      const int part = lane & 7;  // 16-byte piece of a token's 128 bytes: 0-3 = a', 4-7 = g'
+#pragma unroll
+      for (int j = 0; j < KEEP_TILES; ++j) {
+        if (j < kept) {
+          // tok[wave] is private to the wave, and a wave's LDS operations complete in order: no workgroup
+          // barrier, only the compiler must keep the writes, the reads and the next tile's writes in order
+          __builtin_amdgcn_wave_barrier();
+#pragma unroll
+          for (int mt = 0; mt < MTW; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              tok[wave][0][mt * 16 + q * 4 + i][c] = keepA[j][mt][i];
+              tok[wave][1][mt * 16 + q * 4 + i][c] = keepG[j][mt][i];
+            }
+          __builtin_amdgcn_wave_barrier();
+          float* dstp = pa.tokproj + keep_at[j];
+#pragma unroll
+          for (int k = 0; k < WAVE_T / 8; ++k) {
+            const int t = k * 8 + (lane >> 3);
+            const float4 val = *reinterpret_cast<const float4*>(&tok[wave][part >> 2][t][(part & 3) * 4]);
+            if (t < keep_rows[j]) {
+              typedef float raw4 __attribute__((ext_vector_type(4)));
+              *reinterpret_cast<raw4*>(dstp + t * 32 + part * 4) = raw4{val.x, val.y, val.z, val.w};
+            }
+          }
+        }
+      }
+      kept = 0;
+    }
+  };
   for (int idx = item0; idx < item1; ++idx) {
     // With the fragments in a global table nothing ties a workgroup to consecutive items (no projections staged
     // per module), so the host deals the items out one by one for even loads and passes the resulting list.
@@ -573,6 +617,31 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
       }
       parity ^= 1;  // the next tile writes the other buffer, so one barrier per tile is enough
     } else {
+      if (pa.tokproj != nullptr) {
+        // two-step rows: the wave's a', g' -- 128 bytes per token -- go to the workspace (later: flush_kept), and
+        // token_rows_kernel writes the store rows from them, a whole row at a time
+        if (rows_valid > 0) {
+#pragma unroll
+          for (int j = KEEP_TILES - 1; j > 0; --j) {
+#pragma unroll
+            for (int mt = 0; mt < MTW; ++mt) {
+              keepA[j][mt] = keepA[j - 1][mt];
+              keepG[j][mt] = keepG[j - 1][mt];
+            }
+            keep_at[j] = keep_at[j - 1];
+            keep_rows[j] = keep_rows[j - 1];
+          }
+#pragma unroll
+          for (int mt = 0; mt < MTW; ++mt) {
+            keepA[0][mt] = accA[mt];
+            keepG[0][mt] = accG[mt];
+          }
+          keep_at[0] = ((((int64_t)m * args.N + n) * args.S) + s0 + wave * WAVE_T) * 32;
+          keep_rows[0] = rows_valid;
+          if (++kept == KEEP_TILES) flush_kept();
+        }
+        continue;
+      }
       // tok[wave] is private to the wave, and a wave's LDS operations complete in order: no workgroup
       // barrier, only the compiler must keep the writes, the reads and the next tile's writes in order
       __builtin_amdgcn_wave_barrier();
@@ -626,6 +695,41 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
         }
       }
     }
+  }
+  flush_kept();
+}
+
+// Second step of the two-step per-token rows: one workgroup per token writes that token's whole store row --
+// every module's p x p block clamp(g'[i] * a'[j]), the arithmetic of the one-step kernel -- from the 128 bytes per
+// module the collection kernel left in `tokproj`.  The blocks of a row are written where the descriptors say
+// (adjacent blocks make one contiguous stretch: 24 KB for 48 modules at p = 16), a lane stores 8 consecutive
+// columns with one 16-byte store, and the projections come out of L2.
+template <int DT>
+__global__ __launch_bounds__(256) void token_rows_kernel(const bgx_module_desc* __restrict__ mods, int n_modules,
+                                                         const float* __restrict__ tokproj,
+                                                         const int32_t* __restrict__ lengths,
+                                                         const int64_t* __restrict__ row_offsets, int N, int S, int p,
+                                                         void* out, int64_t out_row_stride, float lo, float hi) {
+  const int s = blockIdx.x;
+  const int n = blockIdx.y;
+  if (s >= seq_token_limit(lengths, n, S)) return;
+  const int64_t row = row_offsets[n] + s;
+  const int jg = p >> 3;                 // 8-column groups per block row: 1 or 2
+  const int tasks_pm = p * jg;           // 16-byte pieces of a module's block
+  const int tasks = n_modules * tasks_pm;
+  for (int task = threadIdx.x; task < tasks; task += 256) {
+    const int m = task / tasks_pm;
+    const int rem = task - m * tasks_pm;
+    const int i = rem / jg;
+    const int j0 = (rem - i * jg) << 3;
+    const float* src = tokproj + (((int64_t)m * N + n) * S + s) * 32;
+    const float gv = src[16 + i];
+    const float4 a_lo = *reinterpret_cast<const float4*>(src + j0);
+    const float4 a_hi = *reinterpret_cast<const float4*>(src + j0 + 4);
+    const float o[8] = {clampf(gv * a_lo.x, lo, hi), clampf(gv * a_lo.y, lo, hi), clampf(gv * a_lo.z, lo, hi),
+                        clampf(gv * a_lo.w, lo, hi), clampf(gv * a_hi.x, lo, hi), clampf(gv * a_hi.y, lo, hi),
+                        clampf(gv * a_hi.z, lo, hi), clampf(gv * a_hi.w, lo, hi)};
+    store8_as<DT>(out, row * out_row_stride + mods[m].out_col + i * p + j0, o);
   }
 }
 
@@ -834,14 +938,32 @@ static size_t item_list_bytes(int n_modules, int N, int S) {
   return (size_t)n_modules * (size_t)N * (size_t)((S + 63) / 64) * sizeof(int32_t);
 }
 
+// Projected activations and output gradients of every token (a', g': 2 x 16 floats per module and token), the
+// intermediate of the two-step per-token rows; 0 where that route does not apply (p other than 8 or 16).
+static size_t token_projection_bytes(int n_modules, int N, int S, int p) {
+  if (p != 8 && p != 16) return 0;
+  return (size_t)n_modules * (size_t)N * (size_t)S * 32 * sizeof(float);
+}
+
+// Where the parts of the larger workspace start.
+struct WorkspaceLayout {
+  size_t frag, order, tokproj, total;
+};
+static WorkspaceLayout workspace_layout(size_t base, size_t table, int n_modules, int N, int S, int p) {
+  WorkspaceLayout l;
+  l.frag = align_up(base, 256);
+  l.order = align_up(l.frag + table, 256);
+  l.tokproj = align_up(l.order + (table ? item_list_bytes(n_modules, N, S) : 0), 256);
+  l.total = l.tokproj + token_projection_bytes(n_modules, N, S, p);
+  return l;
+}
+
 size_t collect_workspace_bytes_for(const bgx_module_desc* mods, int n_modules, int N, int S, int p, int in_dtype) {
   const size_t base = collect_workspace_bytes(n_modules, N, S, p);
   if (base == 0 || mods == nullptr) return base;
-  const size_t table = fragment_table_bytes(mods, n_modules, p, in_dtype);
-  if (table == 0) return align_up(base, 256);
-  // behind the table: the list of (module, tile) items in the order the workgroups take them, at most one per 64
-  // tokens of a sequence and module
-  return align_up(align_up(base, 256) + table, 256) + item_list_bytes(n_modules, N, S);
+  // behind the minimum: the fragment table, the list of (module, tile) items in the order the workgroups take them
+  // (at most one per 64 tokens of a sequence and module; only with a table), the tokens' projections
+  return workspace_layout(base, fragment_table_bytes(mods, n_modules, p, in_dtype), n_modules, N, S, p).total;
 }
 
 template <typename T, int PB, bool ALIGNED, int MT, int U>
@@ -1022,7 +1144,8 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   // Modules too wide for LDS: the streamed kernel with the fragments in a global table, when the caller's
   // workspace has room for it (bgx_collect_workspace_bytes_for) -- else the tile kernel.
   const size_t frag_bytes = fragment_table_bytes(sorted.data(), n_modules, p, in_dtype);
-  const size_t frag_ws_off = align_up(need, 256);
+  const WorkspaceLayout lay = workspace_layout(need, frag_bytes, n_modules, N, S, p);
+  const size_t frag_ws_off = lay.frag;
   bool rfg = !persist && pb == 1 && aligned && !any_bias && tiles * n_modules <= 0x7fffffffLL && frag_bytes > 0 &&
              ws_bytes >= frag_ws_off + frag_bytes;
   rfg = rfg && switches().collect_staged;
@@ -1038,7 +1161,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   std::vector<unsigned char> head((size_t)n_modules * sizeof(bgx_module_desc));
   memcpy(head.data(), sorted.data(), head.size());
   // table variant: room behind the table for the item list that lets the workgroups take items out of order
-  const size_t order_ws_off = align_up(frag_ws_off + frag_bytes, 256);
+  const size_t order_ws_off = lay.order;
   const bool rfg_order = rfg && ws_bytes >= order_ws_off + (size_t)tiles * n_modules * sizeof(int32_t) &&
                          !switches().collect_lpt_off;
   std::vector<int32_t> order;
@@ -1156,6 +1279,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   args.hi = hi;
 
   const dim3 grid((unsigned)tiles, (unsigned)n_modules);
+  bool two_step = false;
   hipEvent_t ev_start, ev_stop;
   const bool timed = claim_timing_pair(&ev_start, &ev_stop);
   if (timed) BGX_HIP(hipEventRecord(ev_start, st));
@@ -1173,6 +1297,11 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     bool vec8 = per_token && (p == 8 || p == 16) && (uintptr_t)out % 16 == 0 && (out_row_stride * out_elem) % 16 == 0;
     for (int m = 0; m < n_modules && vec8; ++m) vec8 = (sorted[m].out_col * out_elem) % 16 == 0;
     pa.out_vec8 = vec8 ? 1 : 0;
+    // per-token rows in two steps when the blocks can be written 16 bytes at a time and the caller's workspace has
+    // room for the tokens' projections (bgx_collect_workspace_bytes_for)
+    two_step = vec8 && lay.total > lay.tokproj && ws_bytes >= lay.total && N <= 65535 &&
+               !switches().collect_two_step_off;
+    pa.tokproj = two_step ? (float*)((char*)ws + lay.tokproj) : nullptr;
     int rc;
     if (in_dtype == BGX_F32)
       rc = launch_persist<float>(staged, rfg, per_token, tile_tokens, wgs, persist_lds, st, pa);
@@ -1191,6 +1320,20 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   }
   BGX_HIP(hipGetLastError());
   if (!persist) note_kernel(FAMILY_COLLECT, "collect_tile");
+  if (two_step) {
+    const dim3 tgrid((unsigned)S, (unsigned)N);
+    const float* tp = (const float*)((const char*)ws + lay.tokproj);
+    if (out_dtype == BGX_F32)
+      hipLaunchKernelGGL(token_rows_kernel<BGX_F32>, tgrid, dim3(256), 0, st, mods_dev, n_modules, tp, lengths,
+                         rows_or_offsets, N, S, p, out, out_row_stride, lo, hi);
+    else if (out_dtype == BGX_F16)
+      hipLaunchKernelGGL(token_rows_kernel<BGX_F16>, tgrid, dim3(256), 0, st, mods_dev, n_modules, tp, lengths,
+                         rows_or_offsets, N, S, p, out, out_row_stride, lo, hi);
+    else
+      hipLaunchKernelGGL(token_rows_kernel<BGX_BF16>, tgrid, dim3(256), 0, st, mods_dev, n_modules, tp, lengths,
+                         rows_or_offsets, N, S, p, out, out_row_stride, lo, hi);
+    BGX_HIP(hipGetLastError());
+  }
   if (timed) BGX_HIP(hipEventRecord(ev_stop, st));
 
   if (!per_token) {

@@ -38,6 +38,7 @@ struct Switches {
   bool collect_staged = true;     // BGX_COLLECT_STAGED != "0"
   bool collect_persist = true;    // BGX_COLLECT_PERSIST != "0"
   bool collect_lpt_off = false;   // BGX_COLLECT_LPT_OFF set
+  bool collect_two_step_off = false;  // BGX_COLLECT_TWO_STEP_OFF set: per-token rows written by the collection kernel itself
   bool scan_direct_off = false;   // BGX_SCAN_DIRECT_OFF set
   bool scan_stream_off = false;   // BGX_SCAN_STREAM_OFF set
   bool scan_wide_off = false;     // BGX_SCAN_WIDE_OFF set

@@ -86,7 +86,7 @@ const char* bgx_last_error(void);
 
 /* Diagnostics (no counterpart in the reference).  A handful of BGX_*
  * environment variables force a kernel variant, so that tests can compare the
- * variants (BGX_COLLECT_PERSIST=0, BGX_COLLECT_STAGED=0, BGX_COLLECT_LPT_OFF,
+ * variants (BGX_COLLECT_PERSIST=0, BGX_COLLECT_STAGED=0, BGX_COLLECT_LPT_OFF, BGX_COLLECT_TWO_STEP_OFF,
  * BGX_ADAM_FUSED_OFF, BGX_ADAM_DIRECT_OFF, BGX_ADAM_WIDE_OFF, BGX_ADAM_TTX=n, BGX_SCAN_DIRECT_OFF,
  * BGX_SCAN_STREAM_OFF, BGX_SCAN_WIDE_OFF).  The library reads them once, on its first launch;
  * bgx_reload_switches() reads them again.  Launches that are being issued from
@@ -118,13 +118,18 @@ int bgx_adafactor_scales(const float* row_dev, int32_t O, const float* col_dev,
 /* Bytes of device workspace bgx_collect_seq / bgx_collect_tok need.
  * bgx_collect_workspace_bytes is the minimum for any modules of that count.
  * bgx_collect_workspace_bytes_for looks at the modules (only I, O and bias_col
- * of each descriptor are read) and adds room for a table of pre-scaled
- * projection fragments, 32 bytes per input and output feature, and for the
+ * of each descriptor are read) and adds room for (i) a table of pre-scaled
+ * projection fragments, 32 bytes per input and output feature, and the
  * list of work items behind it (4 bytes per module and 64 tokens): with it,
  * modules too wide for their projections to be kept on chip (Llama-3-8B's
  * 4096 x 14336) still run through the streamed persistent kernel; without it
- * such launches use the one-workgroup-per-tile kernel.  Both sizes are
- * accepted by the collect entry points. */
+ * such launches use the one-workgroup-per-tile kernel; (ii) at p = 8 or 16,
+ * the projected activations and output gradients of every token (128 bytes
+ * per module and token): with it bgx_collect_tok writes its rows in two steps
+ * -- the collection kernel leaves those projections in the workspace and a
+ * second kernel writes each token's store row whole -- instead of scattering
+ * one 2 p^2-byte block per module and token from the collection kernel itself
+ * (same values).  Both sizes are accepted by the collect entry points. */
 size_t bgx_collect_workspace_bytes(int32_t n_modules, int32_t N, int32_t S,
                                    int32_t p);
 size_t bgx_collect_workspace_bytes_for(const bgx_module_desc* mods_host,

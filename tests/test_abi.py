@@ -72,10 +72,15 @@ def test_workspace_sizes():
         d.I, d.O = I, O
     base = lib.bgx_collect_workspace_bytes(2, 2, 2048, 16)
     # the table (32 bytes per column of a and g) and, behind it, the list of items: one per 64 tokens and module
+    # and, at p = 8 or 16, 128 bytes per module and token for the two-step per-token rows
+    up = lambda x: -(-x // 256) * 256
+    tokens = 2 * 2 * 2048 * 128
     assert (lib.bgx_collect_workspace_bytes_for(descs, 2, 2, 2048, 16, 2)
-            == -(-base // 256) * 256 + (4096 + 14336 + 4096 + 1024) * 32 + 2 * 2 * (2048 // 64) * 4)
+            == up(up(up(base) + (4096 + 14336 + 4096 + 1024) * 32) + 2 * 2 * (2048 // 64) * 4) + tokens)
     descs[1].O = 1000   # a width the streamed kernel cannot take: no table
-    assert lib.bgx_collect_workspace_bytes_for(descs, 2, 2, 2048, 16, 2) == -(-base // 256) * 256
+    assert lib.bgx_collect_workspace_bytes_for(descs, 2, 2, 2048, 16, 2) == up(base) + tokens
+    base32 = lib.bgx_collect_workspace_bytes(2, 2, 2048, 32)
+    assert lib.bgx_collect_workspace_bytes_for(descs, 2, 2, 2048, 32, 2) == up(base32)   # p = 32: neither
     small = lib.bgx_scan_workspace_bytes(8, 10, 1024)
     assert small >= 8 * 10 * 8 + 8 * 1024 * 8
     assert lib.bgx_scan_workspace_bytes(1024, 100, 0) >= 1024 * 65536 * 8

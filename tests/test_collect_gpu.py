@@ -295,6 +295,35 @@ def test_tok(device, dtype, p):
     assert rel_l2(got, want) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("p", [16, 8])
+def test_two_step_token_rows_equal_the_one_step_rows_bitwise(device, out_dtype, p, bgx_env, kernel_variant):
+    """Per-token rows at p = 8 / 16 are written in two steps by default (the collection kernel leaves every token's
+    a', g' in the workspace, a second kernel writes the store rows whole); BGX_COLLECT_TWO_STEP_OFF makes the
+    collection kernel write them itself.  Same arithmetic, same bits -- on ragged lengths, documents stored out of
+    batch order, several tiles per sequence, and a clamp that bites."""
+    N, S = 4, 300
+    lengths = [300, 2, 131, 257]
+    cases = []
+    for i, (I, O) in enumerate([(128, 256), (256, 64), (64, 192)]):
+        a, g, left, right, norm = make_case(N, S, I, O, p, torch.bfloat16, seed=220 + i,
+                                            normalizer="adafactor" if i == 1 else None, name=f"layers.{i}.w")
+        cases.append((a, g * (30.0 if i == 2 else 1.0), left, right, norm))
+    counts = [l - 1 for l in lengths]
+    order = [3, 1, 0, 2]
+    offs, r = {}, 0
+    for d in order:
+        offs[d] = r
+        r += counts[d]
+    kw = dict(lengths=lengths, per_token=True, row_offsets=[offs[n] for n in range(N)], n_rows=r, lo=-2.0, hi=2.0)
+    two = run_kernel(device, cases, p, out_dtype, **kw)
+    bgx_env("BGX_COLLECT_TWO_STEP_OFF", "1")
+    one = run_kernel(device, cases, p, out_dtype, **kw)
+    bgx_env("BGX_COLLECT_TWO_STEP_OFF", None)
+    assert torch.equal(two, one)
+    assert two.abs().max().item() == 2.0 and (two != 0).any(dim=1).all()   # the clamp bit; every row was written
+
+
 def test_tok_rows_sum_to_seq_row(device):
     # sum over tokens of the per-token rows equals the per-sequence row (fp32)
     N, S, p = 2, 77, 16
