@@ -11,7 +11,7 @@ from pathlib import Path
 LIB_PATH = Path(__file__).resolve().parent / "libbergson_amd.so"
 
 BGX_F32, BGX_F16, BGX_BF16 = 0, 1, 2
-ABI_VERSION = 10
+ABI_VERSION = 11
 STATIC_SCRATCH_BYTES = 16 << 20
 
 
@@ -76,10 +76,11 @@ SIGNATURES: dict[str, tuple] = {
         [C.POINTER(ModuleDesc), C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p,
          C.c_void_p, C.c_int64, C.c_int32, C.c_float, C.c_float, C.c_void_p],
     ),
-    "bgx_adam_table_bytes": (C.c_size_t, [C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
-    "bgx_adam_prepare": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p,
-                                   C.c_void_p]),
-    "bgx_collect_adam_workspace_bytes": (C.c_size_t, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int64]),
+    "bgx_adam_table_bytes": (C.c_size_t, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
+    "bgx_adam_prepare": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32,
+                                   C.c_int32, C.c_void_p, C.c_void_p]),
+    "bgx_collect_adam_workspace_bytes": (C.c_size_t, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
+                                                      C.c_int32, C.c_int64]),
     "bgx_collect_adam": (
         C.c_int,
         [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32,

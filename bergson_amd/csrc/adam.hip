@@ -17,6 +17,8 @@
 
 #include <stdlib.h>
 
+#include <algorithm>
+
 #include <type_traits>
 
 #include "common.hpp"
@@ -29,25 +31,74 @@ namespace bgx {
 int gemm_scores(const void* rows, int64_t n_rows, int64_t D, int64_t stride, int dtype, const void* queries, int Q,
                 float* scores, hipStream_t st);
 
-// table[(j * O + o) * I + k] = round_T(R[j, k] / (sqrt(v[o, k]) + 1e-8))
+// The table's shape.  16-bit models with p <= 32 run on the fused kernels, which want whole 256-feature chunks of
+// O and whole 64-element K tiles of I: their table is padded with zero rows up to O_pad and zero columns up to
+// I_pad, and when the bias gradient is collected the bias is one more input feature -- column I of the table holds
+// bias_col[j] * bias_scale[o], and the activations get a column of ones there (see adam_pad_kernel), so that
+//   sum_o L[i,o] g_t[o] (H_t[o,j] + 1 * bias_col[j] bias_scale[o]) = P_t[i,j] + (sum_o L[i,o] g_t[o] bias_scale[o]) bias_col[j],
+// which is the bias column of the reference's [grad | bias_grad] projection (collector.py:626-644).  Zero rows and
+// columns add exact zeros.  Other models (fp32, p > 32) keep the plain [p * O, I] table and take the bias as two
+// vectors.
+struct AdamDims {
+  int O_pad, I_pad;
+  bool padded;     // the table is not the plain [p * O, I] one
+  bool bias_in_k;  // the bias travels as input feature I
+};
+static AdamDims adam_dims(int O, int I, int p, int dtype, bool bias) {
+  AdamDims d{O, I, false, false};
+  if (dtype == BGX_F32 || p > 32) return d;
+  d.O_pad = (O + 255) / 256 * 256;
+  d.I_pad = (I + (bias ? 1 : 0) + 63) / 64 * 64;
+  d.bias_in_k = bias;
+  d.padded = d.O_pad != O || d.I_pad != I;
+  return d;
+}
+
+// table[(j * O_pad + o) * I_pad + k] = round_T(R[j, k] / (sqrt(v[o, k]) + 1e-8)) for o < O, k < I;
+// round_T(bias_col[j] * bias_scale[o]) at k = I when the bias is collected; 0 elsewhere
 template <typename T>
-__global__ __launch_bounds__(256) void adam_table_kernel(const T* __restrict__ r_in, const float* __restrict__ v, int O,
-                                                         int I, int p, T* __restrict__ table) {
-  const int64_t total = (int64_t)O * p * I;
+__global__ __launch_bounds__(256) void adam_table_kernel(const T* __restrict__ r_in, const float* __restrict__ v,
+                                                         const float* __restrict__ bias_col,
+                                                         const float* __restrict__ bias_scale, int O, int I, int O_pad,
+                                                         int I_pad, int p, T* __restrict__ table) {
+  const int64_t total = (int64_t)O_pad * p * I_pad;
   for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
        idx += (int64_t)gridDim.x * blockDim.x) {
-    const int k = (int)(idx % I);
-    const int64_t jo = idx / I;
-    const int o = (int)(jo % O);
-    const int j = (int)(jo / O);
-    const float w = 1.0f / (sqrtf(v[(int64_t)o * I + k]) + 1e-8f);
-    const float val = Elem<T>::load(r_in + (int64_t)j * I + k) * w;
+    const int k = (int)(idx % I_pad);
+    const int64_t jo = idx / I_pad;
+    const int o = (int)(jo % O_pad);
+    const int j = (int)(jo / O_pad);
+    float val = 0.f;
+    if (o < O && k < I) {
+      const float w = 1.0f / (sqrtf(v[(int64_t)o * I + k]) + 1e-8f);
+      val = Elem<T>::load(r_in + (int64_t)j * I + k) * w;
+    } else if (o < O && k == I && bias_col != nullptr) {
+      val = bias_col[j] * bias_scale[o];
+    }
     if constexpr (sizeof(T) == 4)
       *(float*)(table + idx) = val;
     else if constexpr (Elem<T>::code == BGX_F16)
       ((uint16_t*)table)[idx] = (uint16_t)f32_to_f16_bits(val);
     else
       ((uint16_t*)table)[idx] = (uint16_t)f32_to_bf16_bits(val);
+  }
+}
+
+// dst[t, c] = src[t, c] for c < cols, `one_at` gets 1 (the bias's input feature; -1 = none), the rest 0:
+// [N, S, cols] rows of any stride into a contiguous [N * S, cols_pad] copy.  16-bit elements.
+__global__ __launch_bounds__(256) void adam_pad_kernel(const uint16_t* __restrict__ src, int64_t seq_stride,
+                                                       int64_t tok_stride, int S, int cols, uint16_t* __restrict__ dst,
+                                                       int cols_pad, int one_at, uint16_t one, int64_t total) {
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int c = (int)(idx % cols_pad);
+    const int64_t t = idx / cols_pad;
+    uint16_t val = 0;
+    if (c < cols)
+      val = src[(t / S) * seq_stride + (t % S) * tok_stride + c];
+    else if (c == one_at)
+      val = one;
+    dst[idx] = val;
   }
 }
 
@@ -1341,28 +1392,35 @@ __global__ void adam_zero_kernel(float* x, int64_t n) {
 // ---- host ---------------------------------------------------------------------------------------
 static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
-size_t adam_table_bytes(int O, int I, int p, int dtype) {
+size_t adam_table_bytes(int O, int I, int p, int dtype, int with_bias) {
   if (O <= 0 || I <= 0 || p <= 0) return 0;
-  return (size_t)O * p * I * dtype_size(dtype);
+  const AdamDims d = adam_dims(O, I, p, dtype, with_bias != 0);
+  return (size_t)d.O_pad * p * d.I_pad * dtype_size(dtype);
 }
 
-int adam_prepare_impl(const void* r_in, const float* v, int O, int I, int p, int dtype, void* table, void* stream) {
+int adam_prepare_impl(const void* r_in, const float* v, const float* bias_col, const float* bias_scale, int O, int I,
+                      int p, int dtype, void* table, void* stream) {
   BGX_REQUIRE(r_in && v && table, BGX_E_ARG, "adam_prepare: null pointer");
+  BGX_REQUIRE((bias_col == nullptr) == (bias_scale == nullptr), BGX_E_ARG,
+              "adam_prepare: bias_col and bias_scale go together");
   BGX_REQUIRE(O > 0 && I > 0 && p >= 1 && p <= 64, BGX_E_SHAPE, "adam_prepare: O=%d I=%d p=%d", O, I, p);
+  BGX_REQUIRE(dtype >= BGX_F32 && dtype <= BGX_BF16, BGX_E_DTYPE, "adam_prepare: dtype=%d", dtype);
   hipStream_t st = (hipStream_t)stream;
-  const int64_t total = (int64_t)O * p * I;
+  const AdamDims d = adam_dims(O, I, p, dtype, bias_col != nullptr);
+  const int64_t total = (int64_t)d.O_pad * p * d.I_pad;
   const unsigned blocks = (unsigned)((total + 255) / 256 > 65536 * 16 ? 65536 * 16 : (total + 255) / 256);
+  // (a table that is not padded leaves the bias to bgx_collect_adam's vectors)
+  const float* bc = d.bias_in_k ? bias_col : nullptr;
+  const float* bs = d.bias_in_k ? bias_scale : nullptr;
   if (dtype == BGX_F32)
-    hipLaunchKernelGGL(adam_table_kernel<float>, dim3(blocks), dim3(256), 0, st, (const float*)r_in, v, O, I, p,
-                       (float*)table);
+    hipLaunchKernelGGL(adam_table_kernel<float>, dim3(blocks), dim3(256), 0, st, (const float*)r_in, v, bc, bs, O, I,
+                       d.O_pad, d.I_pad, p, (float*)table);
   else if (dtype == BGX_F16)
-    hipLaunchKernelGGL(adam_table_kernel<f16_t>, dim3(blocks), dim3(256), 0, st, (const f16_t*)r_in, v, O, I, p,
-                       (f16_t*)table);
-  else if (dtype == BGX_BF16)
-    hipLaunchKernelGGL(adam_table_kernel<bf16_t>, dim3(blocks), dim3(256), 0, st, (const bf16_t*)r_in, v, O, I, p,
-                       (bf16_t*)table);
+    hipLaunchKernelGGL(adam_table_kernel<f16_t>, dim3(blocks), dim3(256), 0, st, (const f16_t*)r_in, v, bc, bs, O, I,
+                       d.O_pad, d.I_pad, p, (f16_t*)table);
   else
-    BGX_REQUIRE(false, BGX_E_DTYPE, "adam_prepare: dtype=%d", dtype);
+    hipLaunchKernelGGL(adam_table_kernel<bf16_t>, dim3(blocks), dim3(256), 0, st, (const bf16_t*)r_in, v, bc, bs, O, I,
+                       d.O_pad, d.I_pad, p, (bf16_t*)table);
   BGX_HIP(hipGetLastError());
   return 0;
 }
@@ -1377,12 +1435,30 @@ static int64_t adam_chunk(int64_t T, int O, int p, int64_t chunk_tokens) {
   return chunk_tokens < T ? chunk_tokens : T;
 }
 
-size_t collect_adam_workspace_bytes(int N, int S, int O, int p, int64_t chunk_tokens) {
-  if (N <= 0 || S <= 0 || O <= 0 || p <= 0) return 0;
+// [H or the fused kernels' per-token results][per-token results][per-sequence sums][slice sums], then the padded
+// copies of a, g and r_out where the table is padded (see adam_dims)
+struct AdamWorkspace {
+  size_t ptok, acc, part, a_pad, g_pad, l_pad, total;
+};
+static AdamWorkspace adam_workspace(int N, int S, int I, int O, int p, int dtype, bool bias, int64_t chunk_tokens) {
+  const AdamDims d = adam_dims(O, I, p, dtype, bias);
   const int64_t T = (int64_t)N * S;
-  const int64_t tc = adam_chunk(T, O, p, chunk_tokens);
-  return align_up((size_t)tc * O * p * 4, 256) + align_up((size_t)tc * p * p * 4, 256) +
-         align_up((size_t)N * p * p * 4, 256) + align_up((size_t)N * SEQ_SLICES * p * p * 4, 256);
+  const int64_t tc = adam_chunk(T, d.O_pad, p, chunk_tokens);
+  const size_t esz = dtype_size(dtype);
+  AdamWorkspace w;
+  w.ptok = align_up((size_t)tc * d.O_pad * p * 4, 256);
+  w.acc = w.ptok + align_up((size_t)tc * p * p * 4, 256);
+  w.part = w.acc + align_up((size_t)N * p * p * 4, 256);
+  w.a_pad = w.part + align_up((size_t)N * SEQ_SLICES * p * p * 4, 256);
+  w.g_pad = w.a_pad + (d.I_pad != I ? align_up((size_t)T * d.I_pad * esz, 256) : 0);
+  w.l_pad = w.g_pad + (d.O_pad != O ? align_up((size_t)T * d.O_pad * esz, 256) : 0);
+  w.total = w.l_pad + (d.O_pad != O ? align_up((size_t)p * d.O_pad * esz, 256) : 0);
+  return w;
+}
+
+size_t collect_adam_workspace_bytes(int N, int S, int I, int O, int p, int dtype, int with_bias, int64_t chunk_tokens) {
+  if (N <= 0 || S <= 0 || I <= 0 || O <= 0 || p <= 0) return 0;
+  return adam_workspace(N, S, I, O, p, dtype, with_bias != 0, chunk_tokens).total;
 }
 
 int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_t a_tok_stride, int64_t g_seq_stride,
@@ -1403,20 +1479,57 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
   BGX_REQUIRE((int64_t)O * p <= 0x7fffffffLL, BGX_E_SHAPE, "collect_adam: O*p too large");
   BGX_REQUIRE(out_col >= 0 && out_col + (int64_t)p * p <= out_row_stride, BGX_E_ARG, "collect_adam: columns do not fit");
   if (per_token) BGX_REQUIRE(lengths && rows, BGX_E_ARG, "collect_adam: per-token mode needs lengths and row_offsets");
-  const size_t need = collect_adam_workspace_bytes(N, S, O, p, chunk_tokens);
-  BGX_REQUIRE(ws_bytes >= need, BGX_E_WORKSPACE, "collect_adam: workspace %zu < %zu bytes", ws_bytes, need);
+  const AdamWorkspace lay = adam_workspace(N, S, I, O, p, dtype, bias_col != nullptr, chunk_tokens);
+  BGX_REQUIRE(ws_bytes >= lay.total, BGX_E_WORKSPACE, "collect_adam: workspace %zu < %zu bytes", ws_bytes, lay.total);
   BGX_REQUIRE(((uintptr_t)ws & 255) == 0, BGX_E_ALIGN, "collect_adam: workspace must be 256-byte aligned");
 
   hipStream_t st = (hipStream_t)stream;
   const int64_t T = (int64_t)N * S;
-  const int64_t tc = adam_chunk(T, O, p, chunk_tokens);
   const int pp = p * p;
   char* w = (char*)ws;
-  float* H = (float*)w;
-  float* ptok = (float*)(w + align_up((size_t)tc * O * p * 4, 256));
-  float* acc = (float*)((char*)ptok + align_up((size_t)tc * pp * 4, 256));
-  float* part = (float*)((char*)acc + align_up((size_t)N * pp * 4, 256));
   const size_t esz = dtype_size(dtype);
+
+  // A padded table (16-bit models, p <= 32; see adam_dims): the operands are brought to its shape -- contiguous
+  // copies of a with I_pad columns (a one in column I when the bias travels there), of g and r_out with O_pad
+  // columns -- and everything below runs on the padded shapes.  One pass over a and g, against p * O * I
+  // multiply-adds per token in the kernel proper.
+  const AdamDims dm = adam_dims(O, I, p, dtype, bias_col != nullptr);
+  if (dm.padded) {
+    const uint16_t one = dtype == BGX_F16 ? 0x3C00 : 0x3F80;
+    auto pad = [&](const void* src, int64_t seq_stride, int64_t tok_stride, int rows_s, int64_t rows, int cols,
+                   void* dst, int cols_pad, int one_at) {
+      const int64_t total = rows * cols_pad;
+      const unsigned blocks = (unsigned)std::min<int64_t>((total + 255) / 256, 65536 * 4);
+      hipLaunchKernelGGL(adam_pad_kernel, dim3(blocks), dim3(256), 0, st, (const uint16_t*)src, seq_stride, tok_stride,
+                         rows_s, cols, (uint16_t*)dst, cols_pad, one_at, one, total);
+    };
+    if (dm.I_pad != I) {
+      void* a_pad = w + lay.a_pad;
+      pad(a, a_seq_stride, a_tok_stride, S, T, I, a_pad, dm.I_pad, dm.bias_in_k ? I : -1);
+      a = a_pad;
+      a_tok_stride = dm.I_pad;
+      a_seq_stride = (int64_t)S * dm.I_pad;
+    }
+    if (dm.O_pad != O) {
+      void* g_pad = w + lay.g_pad;
+      void* l_pad = w + lay.l_pad;
+      pad(g, g_seq_stride, g_tok_stride, S, T, O, g_pad, dm.O_pad, -1);
+      pad(r_out, 0, O, p, p, O, l_pad, dm.O_pad, -1);
+      g = g_pad;
+      g_tok_stride = dm.O_pad;
+      g_seq_stride = (int64_t)S * dm.O_pad;
+      r_out = l_pad;
+    }
+    BGX_HIP(hipGetLastError());
+    I = dm.I_pad;
+    O = dm.O_pad;
+    if (dm.bias_in_k) bias_col = bias_scale = nullptr;  // folded into the table
+  }
+  const int64_t tc = adam_chunk(T, O, p, chunk_tokens);
+  float* H = (float*)w;
+  float* ptok = (float*)(w + lay.ptok);
+  float* acc = (float*)(w + lay.acc);
+  float* part = (float*)(w + lay.part);
 
   if (!per_token) {
     const int64_t nacc = (int64_t)N * pp;

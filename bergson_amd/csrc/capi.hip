@@ -82,9 +82,10 @@ int collect_seq_static_impl(const bgx_module_desc* mods_host, int n_modules, int
                             int out_dtype, float lo, float hi, void* stream);
 int adafactor_scales_impl(const float* row, int O, const float* col, int I, int dtype, float* row_scale,
                           float* col_scale, void* stream);
-size_t adam_table_bytes(int O, int I, int p, int dtype);
-int adam_prepare_impl(const void* r_in, const float* v, int O, int I, int p, int dtype, void* table, void* stream);
-size_t collect_adam_workspace_bytes(int N, int S, int O, int p, int64_t chunk_tokens);
+size_t adam_table_bytes(int O, int I, int p, int dtype, int with_bias);
+int adam_prepare_impl(const void* r_in, const float* v, const float* bias_col, const float* bias_scale, int O, int I,
+                      int p, int dtype, void* table, void* stream);
+size_t collect_adam_workspace_bytes(int N, int S, int I, int O, int p, int dtype, int with_bias, int64_t chunk_tokens);
 int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_t a_tok_stride, int64_t g_seq_stride,
                       int64_t g_tok_stride, int N, int S, int I, int O, int p, int dtype, const void* table,
                       const void* r_out, const float* bias_col, const float* bias_scale, int per_token,
@@ -197,17 +198,20 @@ int bgx_collect_seq_static(const bgx_module_desc* mods_host, int32_t n_modules, 
                                       out_row_stride, out_dtype, clamp_lo, clamp_hi, stream);
 }
 
-size_t bgx_adam_table_bytes(int32_t O, int32_t I, int32_t p, int32_t dtype) {
-  return bgx::adam_table_bytes(O, I, p, dtype);
+size_t bgx_adam_table_bytes(int32_t O, int32_t I, int32_t p, int32_t dtype, int32_t with_bias) {
+  return bgx::adam_table_bytes(O, I, p, dtype, with_bias);
 }
 
-int bgx_adam_prepare(const void* r_in_dev, const float* weight_avg_sq_dev, int32_t O, int32_t I, int32_t p,
-                     int32_t dtype, void* table_dev, void* stream) {
-  return bgx::adam_prepare_impl(r_in_dev, weight_avg_sq_dev, O, I, p, dtype, table_dev, stream);
+int bgx_adam_prepare(const void* r_in_dev, const float* weight_avg_sq_dev, const float* bias_col_dev,
+                     const float* bias_scale_dev, int32_t O, int32_t I, int32_t p, int32_t dtype, void* table_dev,
+                     void* stream) {
+  return bgx::adam_prepare_impl(r_in_dev, weight_avg_sq_dev, bias_col_dev, bias_scale_dev, O, I, p, dtype, table_dev,
+                                stream);
 }
 
-size_t bgx_collect_adam_workspace_bytes(int32_t N, int32_t S, int32_t O, int32_t p, int64_t chunk_tokens) {
-  return bgx::collect_adam_workspace_bytes(N, S, O, p, chunk_tokens);
+size_t bgx_collect_adam_workspace_bytes(int32_t N, int32_t S, int32_t I, int32_t O, int32_t p, int32_t dtype,
+                                        int32_t with_bias, int64_t chunk_tokens) {
+  return bgx::collect_adam_workspace_bytes(N, S, I, O, p, dtype, with_bias, chunk_tokens);
 }
 
 int bgx_collect_adam(const void* a_dev, const void* g_dev, int64_t a_seq_stride, int64_t a_tok_stride,

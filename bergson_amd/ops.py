@@ -348,10 +348,11 @@ class AdamPrepared:
         one pass over the second moments)."""
         if self._table is None:
             lib = _lib.load()
-            nbytes = lib.bgx_adam_table_bytes(self.O, self.I, self.p, dtype_code(self.dtype))
+            bias = int(self.bias_col is not None)
+            nbytes = lib.bgx_adam_table_bytes(self.O, self.I, self.p, dtype_code(self.dtype), bias)
             self._table = torch.empty(nbytes // self.r_in.element_size(), dtype=self.dtype, device=self.r_in.device)
-            rc = lib.bgx_adam_prepare(_ptr(self.r_in), _ptr(self.v), self.O, self.I, self.p, dtype_code(self.dtype),
-                                      _ptr(self._table), _stream())
+            rc = lib.bgx_adam_prepare(_ptr(self.r_in), _ptr(self.v), _ptr(self.bias_col), _ptr(self.bias_scale), self.O,
+                                      self.I, self.p, dtype_code(self.dtype), _ptr(self._table), _stream())
             _lib.check(rc, "bgx_adam_prepare")
         _touch_table(self)
         # the table may be dropped and its memory handed out again while this stream still reads it
@@ -403,12 +404,12 @@ def collect_adam(prep: AdamPrepared, a: Tensor, g: Tensor, out: Tensor, *, per_t
         # fused kernel.  Measured on Pythia-160m shapes the second wins once sequences are shorter than
         # about 3000 / p tokens (16 x 256 tokens at p = 16: 0.84 against 1.08 ms per layer; 32 x 128: 1.57
         # against 1.08).
-        fused_ok = (a.dtype != torch.float32 and O % 256 == 0 and I % 64 == 0 and prep.p <= 32
-                    and prep.bias_col is None)
+        fused_ok = a.dtype != torch.float32 and prep.p <= 32   # the shapes the fused per-token kernels take
         if not (fused_ok and S * prep.p < 3000):
             _collect_adam_seq(prep, a, g, out, lengths, rows, lo, hi)
             return
-    nbytes = lib.bgx_collect_adam_workspace_bytes(N, S, O, prep.p, chunk_tokens)
+    nbytes = lib.bgx_collect_adam_workspace_bytes(N, S, I, O, prep.p, dtype_code(prep.dtype),
+                                                  int(prep.bias_col is not None), chunk_tokens)
     ws = _workspace(out.device, nbytes, "adam")
     rc = lib.bgx_collect_adam(_ptr(a), _ptr(g), a.stride(0), a.stride(1), g.stride(0), g.stride(1), N, S, I, O, prep.p,
                               dtype_code(prep.dtype), _ptr(prep.table), _ptr(prep.r_out), _ptr(prep.bias_col),

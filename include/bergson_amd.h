@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define BGX_ABI_VERSION 10
+#define BGX_ABI_VERSION 11
 
 enum bgx_dtype { BGX_F32 = 0, BGX_F16 = 1, BGX_BF16 = 2 };
 
@@ -207,25 +207,36 @@ int bgx_collect_tok(const bgx_module_desc* mods_host, int32_t n_modules,
  *
  * bgx_adam_prepare builds, once per module, the table
  *   table[(j*O + o), k] = round_dtype(r_in[j, k] / (sqrt(weight_avg_sq[o, k]) + 1e-8))
- * of bgx_adam_table_bytes(O, I, p, dtype) bytes.
+ * of bgx_adam_table_bytes(O, I, p, dtype, with_bias) bytes.
  * bgx_collect_adam then computes, for one module of one batch,
  *   P_t[i, j] = sum_o r_out[i, o] g_t[o] * sum_k a_t[k] table[(j*O + o), k]
  * per token t and writes either every valid token's row (per_token != 0:
  * row row_offsets[n] + s, s < lengths[n] - 1) or the sum over each sequence
  * (per_token == 0: row rows[n], or n when rows is NULL), clamped and cast.
- * bias_col_dev [p] / bias_scale_dev [O] (both or neither): when the bias
- * gradient is collected, column I of the [p, I+1] right projection and
- * 1 / (sqrt(bias_avg_sq) + 1e-8) (gradients.py:390-400); they add
- * (sum_o r_out[i, o] g_t[o] bias_scale[o]) * bias_col[j] to P_t[i, j].
+ * bias_col_dev [p] / bias_scale_dev [O] (both or neither, the same to both
+ * calls): when the bias gradient is collected, column I of the [p, I+1] right
+ * projection and 1 / (sqrt(bias_avg_sq) + 1e-8) (gradients.py:390-400); they
+ * add (sum_o r_out[i, o] g_t[o] bias_scale[o]) * bias_col[j] to P_t[i, j].
+ * For 16-bit models with p <= 32 -- the ones the fused kernels take -- the table
+ * is laid out for those kernels whatever the module's widths: O is padded to a
+ * multiple of 256 and I (+ 1 with the bias, which then travels as one more
+ * input feature: table column I = bias_col[j] * bias_scale[o], against a
+ * column of ones in the activations) to a multiple of 64, with zeros; the
+ * call pads a, g and r_out to match in its workspace.  Zero rows and columns
+ * add exact zeros, so the result is that of the unpadded sums.
  * a must be uniformly strided over the flattened tokens
  * (a_seq_stride == S * a_tok_stride).  chunk_tokens = 0 picks the number of
  * tokens per internal pass. */
-size_t bgx_adam_table_bytes(int32_t O, int32_t I, int32_t p, int32_t dtype);
+size_t bgx_adam_table_bytes(int32_t O, int32_t I, int32_t p, int32_t dtype,
+                            int32_t with_bias);
 int bgx_adam_prepare(const void* r_in_dev, const float* weight_avg_sq_dev,
+                     const float* bias_col_dev, const float* bias_scale_dev,
                      int32_t O, int32_t I, int32_t p, int32_t dtype,
                      void* table_dev, void* stream);
-size_t bgx_collect_adam_workspace_bytes(int32_t N, int32_t S, int32_t O,
-                                        int32_t p, int64_t chunk_tokens);
+size_t bgx_collect_adam_workspace_bytes(int32_t N, int32_t S, int32_t I,
+                                        int32_t O, int32_t p, int32_t dtype,
+                                        int32_t with_bias,
+                                        int64_t chunk_tokens);
 int bgx_collect_adam(const void* a_dev, const void* g_dev,
                      int64_t a_seq_stride, int64_t a_tok_stride,
                      int64_t g_seq_stride, int64_t g_tok_stride, int32_t N,

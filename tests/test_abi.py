@@ -24,7 +24,7 @@ def test_header_symbols_are_exported_and_bound():
     for n in names:
         assert hasattr(lib, n), f"{n} is declared in the header but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes bindings and header disagree"
-    assert lib.bgx_abi_version() == _lib.ABI_VERSION == 10
+    assert lib.bgx_abi_version() == _lib.ABI_VERSION == 11
 
 
 def test_module_desc_layout_matches_header():

@@ -502,6 +502,59 @@ def test_adam_with_bias(device, per_token):
     assert rel_l2(out.cpu(), want) <= 1e-5
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("bias", [False, True])
+@pytest.mark.parametrize("per_token", [False, True])
+@pytest.mark.parametrize("shape", [(2, 300, 128, 320, 32), (1, 512, 256, 1000, 32), (2, 70, 200, 256, 16),
+                                   (3, 40, 96, 40, 8), (1, 256, 1024, 768, 32)])
+def test_adam_fused_kernels_take_any_width_and_the_bias(device, dtype, bias, per_token, shape):
+    """16-bit models with p <= 32 stay on the fused per-token kernels whatever the module's widths: O that is no
+    multiple of 256 (320, 1000, 40), I that is no multiple of 64 (200, 96), and the bias column, which travels as one
+    more input feature.  Rows against the oracle, and the route asserted from what the library ran."""
+    from bergson_amd import _lib, ops
+
+    N, S, I, O, p = shape
+    gen = torch.Generator().manual_seed(300 + O + I)
+    a = torch.randn(N, S, I, generator=gen).to(dtype)
+    g = (torch.randn(N, S, O, generator=gen) * 0.1).to(dtype)
+    lengths = [S, max(2, S // 3), max(2, S - 9)][:N]
+    for n, l in enumerate(lengths):
+        g[n, l - 1:] = 0
+    left, right = module_projections("layers.4.mlp.dense_h_to_4h", p, O, I, dtype, collect_bias=bias)
+    # second moments bounded away from zero keep R / sqrt(v) inside fp16's range; in the model dtype where the
+    # bias is collected, as the reference's arithmetic needs there
+    v = torch.rand(O, I, generator=gen) * 1e-3 + 1e-4
+    bsq = (torch.rand(O, generator=gen) * 1e-3 + 1e-4) if bias else None
+    norm = ohooks.Adam(weight_avg_sq=v.to(dtype) if bias else v, bias_avg_sq=None if bsq is None else bsq.to(dtype))
+    mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+    want = ohooks.module_gradient(a, g, norm, left, right, collect_bias=bias, attribute_tokens=per_token,
+                                  collection_mask=mask if per_token else None).float()
+    r_in = right[:, :I].contiguous() if bias else right
+    prep = ops.AdamPrepared(r_in.to(device), left.to(device), norm.weight_avg_sq.float().to(device), 0,
+                            bias_col=right[:, I].to(device) if bias else None,
+                            bias_avg_sq=norm.bias_avg_sq.float().to(device) if bias else None)
+    ldev = torch.tensor(lengths, dtype=torch.int32, device=device)
+    counts = [l - 1 for l in lengths]
+    if per_token:
+        out = torch.zeros(sum(counts), p * p, dtype=torch.float32, device=device)
+        offs = torch.tensor([sum(counts[:n]) for n in range(N)], dtype=torch.int64, device=device)
+        ops.collect_adam(prep, a.to(device), g.to(device), out, per_token=True, lengths=ldev, rows=offs, lo=-3e38,
+                         hi=3e38)
+        torch.cuda.synchronize()
+        assert _lib.last_kernel(_lib.FAMILY_ADAM).startswith("adam_fused")
+    else:
+        out = torch.zeros(N, p * p, dtype=torch.float32, device=device)
+        ops.collect_adam(prep, a.to(device), g.to(device), out, per_token=False, lengths=ldev, rows=None, lo=-3e38,
+                         hi=3e38)
+        torch.cuda.synchronize()
+    assert out.shape == want.shape and torch.isfinite(out).all()
+    assert rel_l2(out.cpu(), want) <= TOL[dtype]
+    if per_token and S * N <= 600:   # every row on its own, so that a wrong padded column cannot hide in the norm
+        live = want.norm(dim=1) > 1e-3 * want.norm(dim=1).max()
+        per_row = (out.cpu() - want).norm(dim=1) / want.norm(dim=1).clamp_min(1e-30)
+        assert per_row[live].max().item() <= 4 * TOL[dtype]
+
+
 # ---- weight-shaped (unprojected) gradients ----------------------------------------------------------
 def _full_case(N, S, I, O, dtype, kind, bias, seed):
     gen = torch.Generator().manual_seed(seed)
