@@ -384,209 +384,21 @@ __device__ inline uint32_t scaled_pair_bits(float x0, float x1, uint32_t g2) {
   }
 }
 
-template <typename T>
-__global__ __launch_bounds__(512) void adam_fused_kernel(FusedArgs a) {
-  using M = Mma32<T>;
-  static_assert(sizeof(T) == 2, "the fused Adam kernel is for 16-bit model dtypes");
-  constexpr int BM = FUSED_TILE, BN = FUSED_TILE, NT = 512;
-  constexpr int EPL = M::EPL;
-  constexpr int BK = TILE_CHUNKS * EPL;
-  // 8 waves as 4 (tokens) x 2 (output features), 64 x 128 per wave: two 32-token blocks per wave keep the
-  // second pass's accumulators at 32 registers
-  constexpr int WNW = 2, WTM = 64, WTN = 128, TM = 2, TN = 4;
-  constexpr int GCH = BM * TILE_CHUNKS / NT, QCH = BN * TILE_CHUNKS / NT;
-  constexpr int ROWS_PER_PASS = NT / TILE_CHUNKS;
-  constexpr int BUF_BYTES = (BM + BN) * LDS_ROW_BYTES;
-  static_assert((NT / 64 / WNW) * TM * 16 * 64 * 4 <= 2 * BUF_BYTES, "the final reduction reuses the GEMM's LDS buffers");
-  extern __shared__ __align__(16) unsigned char smem[];
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm = wave / WNW, wn = wave % WNW;
-  const int fr = lane & 31;
-  const int fh = lane >> 5;
-  const int lrow = tid / TILE_CHUNKS;
-  const int lcol = tid % TILE_CHUNKS;
-  // Which (token tile, column j) this workgroup takes.  Workgroup b runs on XCD b % 8, and the 32 that an XCD
-  // runs at a time share operands through its L2: `ttx` token tiles x 32 / ttx columns (chosen by the host).
-  // In the plain order every XCD walks the whole table; here it reads only its own columns' share.
-  int tt = blockIdx.x, j = blockIdx.y;
-  if (a.ttx > 0) {
-    const int b = blockIdx.x + gridDim.x * blockIdx.y;
-    const int xcd = b & 7, slot = b >> 3;
-    const int jx = 32 / a.ttx, n_super_tt = gridDim.x / a.ttx;
-    const int super = (slot >> 5) * 8 + xcd, within = slot & 31;
-    tt = (super % n_super_tt) * a.ttx + within % a.ttx;
-    j = (super / n_super_tt) * jx + within / a.ttx;
-  }
-  const int t_row0 = tt * BM;  // chunk-local first token of the tile
-  const int p = a.p, O = a.O, pp = p * p;
-  const int64_t I = a.I;
-  const int rows_here = a.tokens - t_row0;  // valid tokens of this tile (may exceed BM)
-
-  const T* act = (const T*)a.a + (int64_t)t_row0 * a.a_tok_stride;
-
-  // Second pass, straight from the accumulators.  The GEMM blocks are accumulated transposed (the table's
-  // fragment as the A operand): lane (fr, fh) then holds token fr of a block, and its 16 accumulators are rows
-  // q*8 + fh*4 + c (q, c = 0..3) of the 32 table rows of the block.  The loader puts table row
-  // fh*16 + q*4 + c at that place of the LDS tile, so those 16 accumulators are 16 consecutive output features,
-  // fh*16 + e: a k-step of the second pass takes e = 8s .. 8s+7, one 16-byte piece of the token's g row and of
-  // a row of L per lane (the order of k inside an MFMA is free as long as both operands use the same one).
-  // H never leaves the registers: no staged tile in LDS, no barrier around the second pass, and the K-tile
-  // pipeline runs on across the chunks of output features.
-  const T* g_row[TM];
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int tl = t_row0 + wm * WTM + i * 32 + fr;
-    const int64_t t = a.t0 + (tl < a.tokens ? tl : a.tokens - 1);
-    const int n = (int)(t / a.S);
-    const int sp = (int)(t - (int64_t)n * a.S);
-    g_row[i] = (const T*)a.g + (int64_t)n * a.g_seq_stride + (int64_t)sp * a.g_tok_stride + wn * WTN + fh * 16;
-  }
-  const T* l_row = (const T*)a.r_out + (int64_t)min(fr, p - 1) * O + wn * WTN + fh * 16;
-
-  f32x16 pacc[TM];
-  f32x16 acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-#pragma unroll
-    for (int e = 0; e < 16; ++e) pacc[i][e] = 0.f;
-#pragma unroll
-    for (int jj = 0; jj < TN; ++jj)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][jj][e] = 0.f;
-  }
-
-  const int KT = (int)(I / BK);
-  const int total = KT * (O / BN);  // K tiles of all chunks, one pipeline
-
-  // the loader runs two tiles ahead of the MFMAs and has its own position
-  int ld_kt = 0;
-  const T* ld_tab = (const T*)a.table + (int64_t)j * O * I;
-  uint4 gr[GCH], qr[QCH];
-  // table row that goes to LDS row lrow (+ multiples of 64): bits (q1 q0 h c1 c0) -> (h q1 q0 c1 c0)
-  const int prow = (lrow & ~31) | ((lrow & 4) << 2) | ((lrow & 24) >> 1) | (lrow & 3);
-  auto gload = [&]() {
-    const int64_t k = (int64_t)ld_kt * BK + lcol * EPL;
-#pragma unroll
-    for (int i = 0; i < GCH; ++i)
-      gr[i] = load_chunk<T, true>(act, lrow + i * ROWS_PER_PASS, rows_here, a.a_tok_stride, k, I);
-#pragma unroll
-    for (int i = 0; i < QCH; ++i) qr[i] = load_chunk<T, true>(ld_tab, prow + i * ROWS_PER_PASS, BN, I, k, I);
-    if (++ld_kt == KT) {
-      ld_kt = 0;
-      ld_tab += (int64_t)BN * I;
-    }
-  };
-  auto lstore = [&](int buf) {
-    unsigned char* base = smem + buf * BUF_BYTES;
-#pragma unroll
-    for (int i = 0; i < GCH; ++i)
-      *reinterpret_cast<uint4*>(base + (lrow + i * ROWS_PER_PASS) * LDS_ROW_BYTES + lcol * 16) = gr[i];
-#pragma unroll
-    for (int i = 0; i < QCH; ++i)
-      *reinterpret_cast<uint4*>(base + (BM + lrow + i * ROWS_PER_PASS) * LDS_ROW_BYTES + lcol * 16) = qr[i];
-  };
-  auto mma_step = [&](const unsigned char* gb, const unsigned char* qb, int kk) {
-    uint4 af[TM], bf[TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const uint4*>(gb + i * 32 * LDS_ROW_BYTES + kk * 32);
-#pragma unroll
-    for (int jj = 0; jj < TN; ++jj) bf[jj] = *reinterpret_cast<const uint4*>(qb + jj * 32 * LDS_ROW_BYTES + kk * 32);
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int jj = 0; jj < TN; ++jj) M::mma(bf[jj], af[i], acc[i][jj]);  // transposed block: rows = o
-  };
-
-  // same pipeline as the store scan: MFMAs of tile t from buffer t&1 while tile t+1 goes to the other
-  // buffer and the loads of tile t+2 are in flight; one barrier per tile
-  gload();
-  lstore(0);
-  if (total > 1) gload();
-  __syncthreads();
-  int kt = 0, oc = 0;
-  for (int t = 0; t < total; ++t) {
-    const int buf = t & 1;
-    const unsigned char* gb = smem + buf * BUF_BYTES + (wm * WTM + fr) * LDS_ROW_BYTES + fh * 16;
-    const unsigned char* qb = smem + buf * BUF_BYTES + (BM + wn * WTN + fr) * LDS_ROW_BYTES + fh * 16;
-    mma_step(gb, qb, 0);
-    if (t + 1 < total) lstore(buf ^ 1);
-    if (t + 2 < total) gload();
-#pragma unroll
-    for (int kk = 1; kk < TILE_CHUNKS / 2; ++kk) mma_step(gb, qb, kk);
-    if (++kt == KT) {
-      // the chunk's H is complete: pacc[t, i] += sum_o (H[t, o] * g[t, o]) * L[i, o] over this wave's 128 o
-      kt = 0;
-      // group = (jj, s): 16 output features per lane pair; the operands of group n + 1 are asked for before
-      // the MFMAs of group n, so one round trip to L2 is exposed per chunk, not one per group
-      // one 32-token block after the other: the eight pieces of a token's g row (two 128-byte lines) are then
-      // asked for back to back, while the lines are still in the L1
-      uint4 lq[2], gq[2];
-      auto ask = [&](int n, int slot) {  // n = i * 8 + group
-        const int grp = n & 7;
-        const int off = oc + (grp >> 1) * 32 + (grp & 1) * 8;
-        lq[slot] = load16_global(l_row + off);
-        gq[slot] = load16_global(g_row[n >> 3] + off);
-      };
-      ask(0, 0);
-#pragma unroll
-      for (int n = 0; n < TM * 2 * TN; ++n) {
-        const int slot = n & 1, i = n >> 3, grp = n & 7, jj = grp >> 1, s = grp & 1;
-        if (n + 1 < TM * 2 * TN) ask(n + 1, slot ^ 1);
-        const f32x16& h = acc[i][jj];
-        uint4 af;
-        af.x = scaled_pair_bits<T>(h[8 * s + 0], h[8 * s + 1], gq[slot].x);
-        af.y = scaled_pair_bits<T>(h[8 * s + 2], h[8 * s + 3], gq[slot].y);
-        af.z = scaled_pair_bits<T>(h[8 * s + 4], h[8 * s + 5], gq[slot].z);
-        af.w = scaled_pair_bits<T>(h[8 * s + 6], h[8 * s + 7], gq[slot].w);
-        M::mma(af, lq[slot], pacc[i]);
-      }
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int jj = 0; jj < TN; ++jj)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) acc[i][jj][e] = 0.f;
-      oc += BN;
-    }
-    __syncthreads();
-  }
-
-  // the two waves that share 64 tokens add their halves of the sum over o, in a fixed order
-  float* red = reinterpret_cast<float*>(smem);
-  if (wn == 1) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) red[((wm * TM + i) * 16 + e) * 64 + lane] = pacc[i][e];
-  }
-  __syncthreads();
-  if (wn == 0) {
-    // pacc[i][e] = P[token (e>>2)*8 + fh*4 + (e&3) of block i of this wave][row fr], column j
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int tl = t_row0 + wm * WTM + i * 32 + (e >> 2) * 8 + fh * 4 + (e & 3);
-        if (tl < a.tokens && fr < p) {
-          bool valid = true;
-          if (a.lengths != nullptr) {
-            const int64_t t = a.t0 + tl;
-            const int n = (int)(t / a.S);
-            valid = (int)(t - (int64_t)n * a.S) < a.lengths[n] - 1;
-          }
-          const float v = pacc[i][e] + red[((wm * TM + i) * 16 + e) * 64 + lane];
-          a.ptok[(int64_t)tl * pp + fr * p + j] = valid ? v : 0.f;
-        }
-      }
-  }
-}
-
 // ---- fused path, tiles loaded straight into LDS ------------------------------------------------------------
-// The same computation as adam_fused_kernel with the store scan's direct-to-LDS pipeline (direct.hpp) and the
-// second pass fed from LDS as well:
+// A workgroup owns (256 tokens, column j of P) and walks the output features in chunks of 256.  Per chunk it runs a
+// 256 x 256 tile GEMM over K = I (H[t, o] = sum_k a[t, k] table[(j, o), k]) on the store scan's direct-to-LDS
+// pipeline (direct.hpp), and a second MFMA pass adds pacc[t, i] += sum_o (H[t, o] g[t, o]) L[i, o] straight from
+// the accumulators: the GEMM blocks are accumulated transposed (the table's fragment as the A operand), so lane
+// (fr, fh) holds token fr of a block and its 16 accumulators are rows q*8 + fh*4 + c (q, c = 0..3) of the block's 32
+// table rows; the loader puts table row fh*16 + q*4 + c at that place of the LDS tile, which makes those 16
+// accumulators 16 consecutive output features, fh*16 + e.  A k-step of the second pass takes e = 8s .. 8s+7, one
+// 16-byte piece of the token's g row and of a row of L per lane (the order of k inside an MFMA is free as long as
+// both operands use the same one).  H never leaves the registers, and the K tiles of all chunks form one pipeline.
+// Which (token tile, column j) a workgroup takes: workgroup b runs on XCD b % 8, and the 32 that an XCD runs at a
+// time share operands through its L2 -- `ttx` token tiles x 32 / ttx columns (chosen by the host); in the plain
+// order every XCD would walk the whole table.  The workgroup writes its column of the per-token p x p blocks to
+// `ptok` (fp32 [tokens][p * p]); rows past `tokens` and positions from a sequence's last token on are left zero.
+//  * the second pass is fed from LDS as well:
 //  * eight waves as 4 x 2: a wave owns 64 tokens against 128 table rows of the chunk (2 x 4 blocks of 32 x 32,
 //    128 accumulators), so that a K tile costs the workgroup 192 KB of fragment reads -- with 8 x 1 (every wave
 //    reading all 256 table rows) it was 288 KB, and together with the 64 KB the loads write that is more LDS time
@@ -603,7 +415,6 @@ __global__ __launch_bounds__(512) void adam_fused_kernel(FusedArgs a) {
 //    memory, and its loads travel two tiles ahead like all others;
 //  * loads are uniform base + 32-bit lane offset (sw_load_lds16), fragment reads and waits are spelled out as in
 //    scan_direct_kernel.
-// Token tile x column mapping to workgroups (ttx), validity masking and the ptok layout are the old kernel's.
 constexpr int FD_A_BYTES = FUSED_TILE * SD_ROW, FD_B_BYTES = FUSED_TILE * SD_ROW;
 constexpr int FD_LDS_BYTES = 3 * FD_A_BYTES + 2 * FD_B_BYTES;
 constexpr int FD_GSLICES = 4;  // slices of 64 output features per chunk of 256
@@ -1450,9 +1261,10 @@ static AdamWorkspace adam_workspace(int N, int S, int I, int O, int p, int dtype
   w.acc = w.ptok + align_up((size_t)tc * p * p * 4, 256);
   w.part = w.acc + align_up((size_t)N * p * p * 4, 256);
   w.a_pad = w.part + align_up((size_t)N * SEQ_SLICES * p * p * 4, 256);
-  w.g_pad = w.a_pad + (d.I_pad != I ? align_up((size_t)T * d.I_pad * esz, 256) : 0);
-  w.l_pad = w.g_pad + (d.O_pad != O ? align_up((size_t)T * d.O_pad * esz, 256) : 0);
-  w.total = w.l_pad + (d.O_pad != O ? align_up((size_t)p * d.O_pad * esz, 256) : 0);
+  const bool family = dtype != BGX_F32 && p <= 32;  // room for the copies whatever the operands turn out to look like
+  w.g_pad = w.a_pad + (family ? align_up((size_t)T * d.I_pad * esz, 256) : 0);
+  w.l_pad = w.g_pad + (family ? align_up((size_t)T * d.O_pad * esz, 256) : 0);
+  w.total = w.l_pad + (family ? align_up((size_t)p * d.O_pad * esz, 256) : 0);
   return w;
 }
 
@@ -1494,7 +1306,13 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
   // columns -- and everything below runs on the padded shapes.  One pass over a and g, against p * O * I
   // multiply-adds per token in the kernel proper.
   const AdamDims dm = adam_dims(O, I, p, dtype, bias_col != nullptr);
-  if (dm.padded) {
+  const bool family = dtype != BGX_F32 && p <= 32;  // the fused kernels' shapes (adam_dims pads to them)
+  // the fused kernels load whole 16-byte pieces with 32-bit offsets from rows that are uniformly strided over the
+  // flattened tokens: operands that are not like that (an odd view of a wider tensor) are copied as well
+  const bool a_odd = family && ((uintptr_t)a % 16 != 0 || a_tok_stride % 8 != 0);
+  const bool g_odd = family && ((uintptr_t)g % 16 != 0 || g_tok_stride % 8 != 0 ||
+                                (N > 1 && g_seq_stride != (int64_t)S * g_tok_stride));
+  if (dm.padded || a_odd || g_odd) {
     const uint16_t one = dtype == BGX_F16 ? 0x3C00 : 0x3F80;
     auto pad = [&](const void* src, int64_t seq_stride, int64_t tok_stride, int rows_s, int64_t rows, int cols,
                    void* dst, int cols_pad, int one_at) {
@@ -1503,21 +1321,23 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
       hipLaunchKernelGGL(adam_pad_kernel, dim3(blocks), dim3(256), 0, st, (const uint16_t*)src, seq_stride, tok_stride,
                          rows_s, cols, (uint16_t*)dst, cols_pad, one_at, one, total);
     };
-    if (dm.I_pad != I) {
+    if (dm.I_pad != I || a_odd) {
       void* a_pad = w + lay.a_pad;
       pad(a, a_seq_stride, a_tok_stride, S, T, I, a_pad, dm.I_pad, dm.bias_in_k ? I : -1);
       a = a_pad;
       a_tok_stride = dm.I_pad;
       a_seq_stride = (int64_t)S * dm.I_pad;
     }
-    if (dm.O_pad != O) {
+    if (dm.O_pad != O || g_odd) {
       void* g_pad = w + lay.g_pad;
-      void* l_pad = w + lay.l_pad;
       pad(g, g_seq_stride, g_tok_stride, S, T, O, g_pad, dm.O_pad, -1);
-      pad(r_out, 0, O, p, p, O, l_pad, dm.O_pad, -1);
       g = g_pad;
       g_tok_stride = dm.O_pad;
       g_seq_stride = (int64_t)S * dm.O_pad;
+    }
+    if (dm.O_pad != O) {
+      void* l_pad = w + lay.l_pad;
+      pad(r_out, 0, O, p, p, O, l_pad, dm.O_pad, -1);
       r_out = l_pad;
     }
     BGX_HIP(hipGetLastError());
@@ -1537,10 +1357,14 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
     BGX_HIP(hipGetLastError());
   }
   // ---- fused path ------------------------------------------------------------------------------
-  const bool fused = dtype != BGX_F32 && O % FUSED_TILE == 0 && I % 64 == 0 && p <= 32 && bias_col == nullptr &&
-                     (uintptr_t)a % 16 == 0 && (uintptr_t)g % 16 == 0 && (uintptr_t)r_out % 16 == 0 &&
-                     (uintptr_t)table % 16 == 0 && a_tok_stride % 8 == 0 && g_seq_stride % 8 == 0 &&
-                     g_tok_stride % 8 == 0 && !switches().adam_fused_off;
+  // (after the padding above O is a multiple of the 256-feature chunk, I of the 64-element K tile, the bias is in
+  // the table and a, g are aligned and uniformly strided; what is left to check are the 32-bit offsets)
+  const bool fused = family && O % FUSED_TILE == 0 && I % 64 == 0 && bias_col == nullptr &&
+                     (uintptr_t)r_out % 16 == 0 && (uintptr_t)table % 16 == 0 &&
+                     (int64_t)FUSED_TILE * a_tok_stride * 2 < ((int64_t)1 << 32) &&
+                     (int64_t)FUSED_TILE * g_tok_stride * 2 < ((int64_t)1 << 32) &&
+                     (int64_t)FUSED_TILE * I * 2 < ((int64_t)1 << 32) && (int64_t)p * O * 2 < ((int64_t)1 << 32) &&
+                     !switches().adam_fused_off;
   if (fused) {
     // no H: the region reserved for it holds the per-token fp32 results, so a chunk can be much larger
     // (tc * O / p tokens; O >= 256 and p <= 32 make that at least 8 tc, so a batch smaller than one tile is
@@ -1549,7 +1373,6 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
     int64_t fc = cap >= T ? T : cap / FUSED_TILE * FUSED_TILE;
     if (fc <= 0) fc = cap;
     float* ptok_f = (float*)w;
-    constexpr size_t smem = 2 * (size_t)(2 * FUSED_TILE) * LDS_ROW_BYTES;
     for (int64_t t0 = 0; t0 < T; t0 += fc) {
       const int64_t rows_c = T - t0 < fc ? T - t0 : fc;
       FusedArgs f;
@@ -1586,14 +1409,8 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
         }
       }
       f.ttx = ttx;
-      // tiles straight into LDS, the second pass fed from LDS: needs g uniformly strided over the flattened tokens
-      // and 32-bit byte offsets within a tile
-      const bool direct = !switches().adam_direct_off && (N == 1 || g_seq_stride == (int64_t)S * g_tok_stride) &&
-                          (int64_t)FUSED_TILE * a_tok_stride * 2 < ((int64_t)1 << 32) &&
-                          (int64_t)FUSED_TILE * g_tok_stride * 2 < ((int64_t)1 << 32) &&
-                          (int64_t)FUSED_TILE * I * 2 < ((int64_t)1 << 32) && (int64_t)p * O * 2 < ((int64_t)1 << 32);
-      // one wave per SIMD: whole token tiles, at least four K tiles per chunk
-      const bool wide = direct && !switches().adam_wide_off && rows_c % FUSED_TILE == 0 && I >= 256;
+      // one wave per SIMD: whole token tiles, at least four K tiles per chunk; else eight waves
+      const bool wide = !switches().adam_wide_off && rows_c % FUSED_TILE == 0 && I >= 256;
       if (wide) {
         if (dtype == BGX_F16) {
           auto kern = adam_fused_wide_kernel<f16_t>;
@@ -1604,27 +1421,17 @@ int collect_adam_impl(const void* a, const void* g, int64_t a_seq_stride, int64_
           BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, FD_LDS_BYTES));
           hipLaunchKernelGGL(kern, grid, dim3(FW_THREADS), FD_LDS_BYTES, st, f);
         }
-      } else if (direct) {
-        if (dtype == BGX_F16) {
-          auto kern = adam_fused_direct_kernel<f16_t>;
-          BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, FD_LDS_BYTES));
-          hipLaunchKernelGGL(kern, grid, dim3(512), FD_LDS_BYTES, st, f);
-        } else {
-          auto kern = adam_fused_direct_kernel<bf16_t>;
-          BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, FD_LDS_BYTES));
-          hipLaunchKernelGGL(kern, grid, dim3(512), FD_LDS_BYTES, st, f);
-        }
       } else if (dtype == BGX_F16) {
-        auto kern = adam_fused_kernel<f16_t>;
-        BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        hipLaunchKernelGGL(kern, grid, dim3(512), smem, st, f);
+        auto kern = adam_fused_direct_kernel<f16_t>;
+        BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, FD_LDS_BYTES));
+        hipLaunchKernelGGL(kern, grid, dim3(512), FD_LDS_BYTES, st, f);
       } else {
-        auto kern = adam_fused_kernel<bf16_t>;
-        BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        hipLaunchKernelGGL(kern, grid, dim3(512), smem, st, f);
+        auto kern = adam_fused_direct_kernel<bf16_t>;
+        BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, FD_LDS_BYTES));
+        hipLaunchKernelGGL(kern, grid, dim3(512), FD_LDS_BYTES, st, f);
       }
       BGX_HIP(hipGetLastError());
-      note_kernel(FAMILY_ADAM, wide ? "adam_fused_wide" : direct ? "adam_fused_direct" : "adam_fused_staged");
+      note_kernel(FAMILY_ADAM, wide ? "adam_fused_wide" : "adam_fused_direct");
       if (per_token) {
         hipLaunchKernelGGL(adam_tok_finalize_kernel, dim3((unsigned)rows_c), dim3(256), 0, st, ptok_f, t0, (int)rows_c,
                            S, pp, lengths, rows, out, out_row_stride, out_col, out_dtype, lo, hi);

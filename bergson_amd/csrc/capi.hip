@@ -40,7 +40,6 @@ static const Switches* read_switches() {
     return e != nullptr && e[0] == '0';
   };
   s->adam_fused_off = getenv("BGX_ADAM_FUSED_OFF") != nullptr;
-  s->adam_direct_off = getenv("BGX_ADAM_DIRECT_OFF") != nullptr;
   s->adam_wide_off = getenv("BGX_ADAM_WIDE_OFF") != nullptr;
   if (const char* e = getenv("BGX_ADAM_TTX")) s->adam_ttx = atoi(e);
   s->collect_staged = !off("BGX_COLLECT_STAGED");

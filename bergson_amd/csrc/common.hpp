@@ -32,7 +32,6 @@ int hip_fail(hipError_t e, const char* what);
 // on first use, into an immutable record; bgx_reload_switches() publishes a fresh one.
 struct Switches {
   bool adam_fused_off = false;    // BGX_ADAM_FUSED_OFF set
-  bool adam_direct_off = false;   // BGX_ADAM_DIRECT_OFF set
   bool adam_wide_off = false;     // BGX_ADAM_WIDE_OFF set: eight waves of 64 x 128 where four of 128 x 128 would run
   int adam_ttx = -1;              // BGX_ADAM_TTX (token tiles per XCD group), -1 = unset
   bool collect_staged = true;     // BGX_COLLECT_STAGED != "0"

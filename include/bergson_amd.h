@@ -87,7 +87,7 @@ const char* bgx_last_error(void);
 /* Diagnostics (no counterpart in the reference).  A handful of BGX_*
  * environment variables force a kernel variant, so that tests can compare the
  * variants (BGX_COLLECT_PERSIST=0, BGX_COLLECT_STAGED=0, BGX_COLLECT_LPT_OFF, BGX_COLLECT_TWO_STEP_OFF,
- * BGX_ADAM_FUSED_OFF, BGX_ADAM_DIRECT_OFF, BGX_ADAM_WIDE_OFF, BGX_ADAM_TTX=n, BGX_SCAN_DIRECT_OFF,
+ * BGX_ADAM_FUSED_OFF, BGX_ADAM_WIDE_OFF, BGX_ADAM_TTX=n, BGX_SCAN_DIRECT_OFF,
  * BGX_SCAN_STREAM_OFF, BGX_SCAN_WIDE_OFF).  The library reads them once, on its first launch;
  * bgx_reload_switches() reads them again.  Launches that are being issued from
  * other threads at that moment see either the old or the new settings. */
@@ -98,7 +98,7 @@ int bgx_reload_switches(void);
  * family 0 = bgx_collect_seq/_tok/_static ("collect_persist_lds",
  * "collect_persist_table", "collect_persist_direct", "collect_tile"),
  * 1 = bgx_collect_adam ("adam_fused_wide", "adam_fused_direct",
- * "adam_fused_staged", "adam_two_kernel"), 2 = bgx_scan* (the kernel of the
+ * "adam_two_kernel"), 2 = bgx_scan* (the kernel of the
  * longest pass: "scan_wide", "scan_wide_known_norms", "scan_direct", "scan_stream",
  * "scan_gemm"), 3 = bgx_fullgrad_* / bgx_project_rows.  The pointer is to a
  * string literal. */

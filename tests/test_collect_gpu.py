@@ -868,10 +868,13 @@ def test_adam_wide_tiles_equal_the_eight_wave_kernel_bitwise(device, dtype, shap
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("shape", [(2, 700, 256, 512, 32), (1, 1024, 1024, 1024, 32), (3, 300, 192, 768, 16)])
-def test_adam_direct_tiles_against_register_staged_kernel(device, dtype, shape, bgx_env):
-    """The fused Adam kernel whose operands all travel through LDS tiles loaded directly from global memory, on
-    shapes with several K tiles, several chunks of output features and ragged lengths: per-token rows against
-    the oracle where it is quick, and against the register-staged fused kernel (BGX_ADAM_DIRECT_OFF) everywhere."""
+def test_adam_direct_tiles_against_oracle_and_two_kernel_path(device, dtype, shape, bgx_env):
+    """The eight-wave fused Adam kernel (partial token tiles, or fewer than four K tiles) on shapes with several K
+    tiles, several chunks of output features and ragged lengths: per-token rows against the oracle on a sample of
+    each sequence's tokens (rows do not depend on each other), and every row against the path that materialises H
+    (BGX_ADAM_FUSED_OFF), an independent implementation of the same sums."""
+    from bergson_amd import _lib
+
     N, S, I, O, p = shape
     case = _adam_case(N, S, I, O, p, dtype, seed=83)
     a, g, left, right, norm = case
@@ -886,14 +889,58 @@ def test_adam_direct_tiles_against_register_staged_kernel(device, dtype, shape, 
     offs = [sum(counts[:n]) for n in range(N)]
     kw = dict(per_token=True, lengths=lengths, row_offsets=offs, n_rows=sum(counts))
     got = _run_adam(device, case, p, dtype, **kw)
-    bgx_env("BGX_ADAM_DIRECT_OFF", "1")
-    staged = _run_adam(device, case, p, dtype, **kw)
-    assert rel_l2(got, staged) <= TOL[dtype]
+    assert _lib.last_kernel(_lib.FAMILY_ADAM) in ("adam_fused_direct", "adam_fused_wide")
+    bgx_env("BGX_ADAM_FUSED_OFF", "1")
+    two = _run_adam(device, case, p, dtype, **kw)
+    assert _lib.last_kernel(_lib.FAMILY_ADAM) == "adam_two_kernel"
+    assert rel_l2(got, two) <= TOL[dtype]
     assert bool(torch.isfinite(got.float()).all())
-    if I * O <= 256 * 768:
-        mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
-        want = ohooks.module_gradient(a, g, norm, left, right, attribute_tokens=True, collection_mask=mask)
-        assert rel_l2(got, want) <= TOL[dtype]
+    gen = torch.Generator().manual_seed(1)
+    for n in range(N):
+        last = counts[n] - 1
+        idx = sorted({0, last, last // 2, min(255, last), min(256, last)} | set(torch.randint(0, last + 1, (6,), generator=gen).tolist()))
+        ones = torch.ones(1, len(idx), dtype=torch.bool)
+        want = ohooks.module_gradient(a[n:n + 1, idx], g[n:n + 1, idx], norm, left, right, attribute_tokens=True,
+                                      collection_mask=ones)
+        assert rel_l2(got[torch.tensor(idx) + offs[n]], want) <= TOL[dtype], n
+
+
+@pytest.mark.parametrize("view", ["g_slice_of_qkv", "a_offset_by_one", "g_sequences_apart"])
+def test_adam_fused_kernels_take_odd_views(device, view):
+    """Operands the fused kernels cannot load in 16-byte pieces from uniformly strided rows -- g as a slice of a
+    wider tensor at an odd offset, a starting one element into its storage, sequences of g that lie apart -- are
+    brought into shape by the call itself and stay on the fused kernels."""
+    from bergson_amd import _lib, ops
+
+    N, S, I, O, p = 2, 256, 128, 256, 16
+    a, g, left, right, norm = _adam_case(N, S, I, O, p, torch.bfloat16, seed=91)
+    norm = ohooks.Adam(weight_avg_sq=norm.weight_avg_sq * 100 + 1e-6)
+    lengths = [256, 100]
+    for n, l in enumerate(lengths):
+        g[n, l - 1:] = 0
+    ad, gd = a.to(device), g.to(device)
+    if view == "g_slice_of_qkv":
+        wide = torch.zeros(N, S, 3 * O + 3, dtype=torch.bfloat16, device=device)
+        wide[:, :, O + 3:2 * O + 3] = gd
+        gd = wide[:, :, O + 3:2 * O + 3]
+    elif view == "a_offset_by_one":
+        flat = torch.zeros(N * S * I + 1, dtype=torch.bfloat16, device=device)
+        flat[1:] = ad.flatten()
+        ad = flat[1:].view(N, S, I)
+    else:
+        apart = torch.zeros(N, S + 5, O, dtype=torch.bfloat16, device=device)
+        apart[:, :S] = gd
+        gd = apart[:, :S]
+    prep = ops.AdamPrepared(right.to(device), left.to(device), norm.weight_avg_sq.to(device), 0)
+    counts = [l - 1 for l in lengths]
+    out = torch.zeros(sum(counts), p * p, dtype=torch.float32, device=device)
+    ops.collect_adam(prep, ad, gd, out, per_token=True, lengths=torch.tensor(lengths, dtype=torch.int32, device=device),
+                     rows=torch.tensor([0, counts[0]], dtype=torch.int64, device=device), lo=-3e38, hi=3e38)
+    torch.cuda.synchronize()
+    assert _lib.last_kernel(_lib.FAMILY_ADAM).startswith("adam_fused")
+    mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+    want = ohooks.module_gradient(a, g, norm, left, right, attribute_tokens=True, collection_mask=mask)
+    assert rel_l2(out.cpu(), want) <= TOL[torch.bfloat16]
 
 
 def test_adam_seq_many_short_sequences(device):
