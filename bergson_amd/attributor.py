@@ -146,7 +146,7 @@ class Attributor:
             res = ops.scan(self.store, qd, unit_norm=self.unit_norm, k=k, query_scale=2.0 ** (-shift), row_sumsq=norms)
             values, indices = res.topk_values, res.topk_indices
         else:
-            # beyond the fused selection's capacity (k = None asks for a full ranking of the store): the
+            # beyond the fused selection's capacity of 65 536 (k = None asks for a full ranking of the store): the
             # scan writes every score, in slices of queries so that [n, Q'] fp32 stays near 4 GB, and the
             # ranking is the library's
             step = max(1, (1 << 30) // max(1, self.N))

@@ -1385,6 +1385,119 @@ __global__ __launch_bounds__(THREADS) void scan_select_kernel(SelectArgs a) {
   }
 }
 
+// ---- selection for k beyond what one workgroup sorts in LDS ------------------------------------------------
+constexpr int SCAN_KMAX_LARGE = 65536;
+constexpr int SELECT_THREADS_LARGE = 1024;
+
+// dst[dst_base ...] = the keys of src[0, n) that are >= bound, in their order; returns how many.  Every thread of
+// the workgroup calls it.  src == dst with dst_base == 0 compacts in place: a step's survivors are written only
+// after every thread has read the step, at positions no later step reads from.
+template <int THREADS>
+__device__ uint32_t compact_keys(const uint64_t* src, uint32_t n, uint64_t bound, uint64_t* dst, uint32_t dst_base,
+                                 SelectShared& sh) {
+  constexpr int NW = THREADS / 64;
+  constexpr int U = SELECT_COMPACT_KEYS / THREADS;
+  static_assert(U * NW == 64, "the offsets are one wave's prefix sum");
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  uint32_t w_base = dst_base;
+  for (uint32_t base = 0; base < n; base += SELECT_COMPACT_KEYS) {
+    uint64_t key[U];
+    uint32_t lane_off[U];
+    bool keep[U];
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      const uint32_t i = base + j * THREADS + tid;
+      key[j] = i < n ? src[i] : 0ull;
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      const uint32_t i = base + j * THREADS + tid;
+      keep[j] = i < n && key[j] >= bound;
+      const uint64_t ballot = __ballot(keep[j]);
+      lane_off[j] = __popcll(ballot & ((1ull << lane) - 1ull));
+      if (lane == 0) sh.part[j * NW + wave] = __popcll(ballot);
+    }
+    __syncthreads();
+    if (tid < 64) {
+      const uint32_t own = sh.part[tid];
+      uint32_t incl = own;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t o = __shfl_up(incl, d);
+        if (tid >= d) incl += o;
+      }
+      sh.part[tid] = incl - own;
+      if (tid == 63) sh.part[64] = incl;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < U; ++j)
+      if (keep[j]) dst[w_base + sh.part[j * NW + wave] + lane_off[j]] = key[j];
+    w_base += sh.part[64];
+    __syncthreads();
+  }
+  __threadfence_block();
+  __syncthreads();
+  return w_base - dst_base;
+}
+
+// scan_select_kernel for k > SCAN_KMAX: the running top-k of a query stays in global memory, unsorted -- after every
+// pass it is the k largest keys seen so far (exact: the k-th largest of old entries and candidates by radix
+// selection, then both lists cut at it) -- and is sorted once, when the scan is over (scan_sort_top_kernel).
+__global__ __launch_bounds__(SELECT_THREADS_LARGE) void scan_select_large_kernel(SelectArgs a, int64_t top_stride) {
+  __shared__ SelectShared sh;
+  const int q = blockIdx.x;
+  const uint32_t k = (uint32_t)a.k;
+  uint64_t* top = a.top + (int64_t)q * top_stride;
+  uint64_t* cand = a.cand + (int64_t)q * a.cand_cap;
+  const uint32_t ntop = a.top_count[q];
+  uint32_t ncand = a.cand_count[q];
+  if ((int64_t)ncand > a.cand_cap) ncand = (uint32_t)a.cand_cap;
+  if (ncand == 0) return;
+  const uint32_t total = ntop + ncand;
+  auto elem = [&](uint32_t i) -> uint64_t { return i < ntop ? top[i] : cand[i - ntop]; };
+  uint64_t kth = 1;  // entry 0 of a by-row list is an empty one
+  if (total > k) {
+    const uint64_t found = radix_kth<SELECT_THREADS_LARGE>(elem, total, k, sh);
+    kth = found > 1 ? found : 1;
+  }
+  uint32_t kept = compact_keys<SELECT_THREADS_LARGE>(top, ntop, kth, top, 0, sh);
+  kept += compact_keys<SELECT_THREADS_LARGE>(cand, ncand, kth, top, kept, sh);
+  if (threadIdx.x == 0) {
+    a.top_count[q] = kept;
+    a.cand_count[q] = 0;
+    if (kept == k) a.thr[q] = ordered_f32((uint32_t)(kth >> 32));
+  }
+}
+
+// Sorts each query's top[0, top_count) in place, descending: bitonic network over the next power of two (the row
+// has room for it; padded with zeros, which sort last), one workgroup per query.
+__global__ __launch_bounds__(1024) void scan_sort_top_kernel(uint64_t* top, const uint32_t* top_count, int64_t top_stride) {
+  uint64_t* keys = top + (int64_t)blockIdx.x * top_stride;
+  const uint32_t kept = top_count[blockIdx.x];
+  uint32_t n2 = 1;
+  while (n2 < kept) n2 <<= 1;
+  for (uint32_t i = kept + threadIdx.x; i < n2; i += 1024) keys[i] = 0;
+  __threadfence_block();
+  __syncthreads();
+  for (uint32_t size = 2; size <= n2; size <<= 1) {
+    for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+      for (uint32_t i = threadIdx.x; i < n2 / 2; i += 1024) {
+        const uint32_t lo = 2 * i - (i & (stride - 1));
+        const uint32_t hi = lo + stride;
+        const bool desc = (lo & size) == 0;
+        const uint64_t x = keys[lo], y = keys[hi];
+        if ((x < y) == desc) {
+          keys[lo] = y;
+          keys[hi] = x;
+        }
+      }
+      __threadfence_block();
+      __syncthreads();
+    }
+  }
+}
+
 __global__ void scan_init_kernel(uint32_t* top_count, uint32_t* cand_count, float* thr, int Q, uint32_t* row_max_enc,
                                  int64_t n_rows) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -1397,13 +1510,13 @@ __global__ void scan_init_kernel(uint32_t* top_count, uint32_t* cand_count, floa
 }
 
 // A query with fewer than k selectable scores (NaN and -inf are never selected) gets (-inf, -1) in the rest.
-__global__ void scan_finish_kernel(const uint64_t* top, const uint32_t* top_count, int Q, int k, int64_t row_base,
-                                   float* topk_val, int64_t* topk_idx, const uint32_t* row_max_enc, float* row_max,
-                                   int64_t n_rows) {
+__global__ void scan_finish_kernel(const uint64_t* top, const uint32_t* top_count, int64_t top_stride, int Q, int k,
+                                   int64_t row_base, float* topk_val, int64_t* topk_idx, const uint32_t* row_max_enc,
+                                   float* row_max, int64_t n_rows) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (top != nullptr && i < (int64_t)Q * k) {
     const bool filled = (uint32_t)(i % k) < top_count[i / k];
-    const uint64_t key = filled ? top[i] : 0ull;
+    const uint64_t key = filled ? top[(i / k) * top_stride + i % k] : 0ull;
     topk_val[i] = filled ? ordered_f32((uint32_t)(key >> 32)) : -INFINITY;
     topk_idx[i] = filled ? (int64_t)(0xffffffffu - (uint32_t)key) + row_base : (int64_t)-1;
   }
@@ -1463,11 +1576,20 @@ struct ScanLayout {
   size_t top, top_count, cand_count, thr, row_part, cand, total;
 };
 
+// Entries of a query's row of the running top-k: k, or beyond SCAN_KMAX the next power of two (the final sort pads
+// the row to it).
+static int64_t scan_top_stride(int k) {
+  if (k <= SCAN_KMAX) return k > 0 ? k : 0;
+  int64_t n2 = 1;
+  while (n2 < k) n2 <<= 1;
+  return n2;
+}
+
 static ScanLayout scan_layout(int Q, int k, int64_t chunk_rows) {
   ScanLayout l;
   size_t off = 0;
   l.top = off;
-  off += align_up((size_t)Q * (size_t)(k > 0 ? k : 0) * 8, 256);
+  off += align_up((size_t)Q * (size_t)scan_top_stride(k) * 8, 256);
   l.top_count = off;
   off += align_up((size_t)Q * 4, 256);
   l.cand_count = off;
@@ -1696,13 +1818,14 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
   const bool want_topk = topk_val != nullptr || topk_idx != nullptr;
   if (want_topk) {
     BGX_REQUIRE(topk_val && topk_idx, BGX_E_ARG, "scan: topk_val and topk_idx go together");
-    BGX_REQUIRE(k >= 1 && k <= SCAN_KMAX && k <= n_rows, BGX_E_SHAPE, "scan: k=%d outside 1..min(%d, n_rows=%lld)", k,
-                SCAN_KMAX, (long long)n_rows);
+    BGX_REQUIRE(k >= 1 && k <= SCAN_KMAX_LARGE && k <= n_rows, BGX_E_SHAPE, "scan: k=%d outside 1..min(%d, n_rows=%lld)",
+                k, SCAN_KMAX_LARGE, (long long)n_rows);
   } else {
     k = 0;
   }
   const int64_t chunk = effective_chunk(chunk_rows, Q);
   const ScanLayout lay = scan_layout(Q, k, chunk);
+  const int64_t top_stride = scan_top_stride(k);
   const bool need_init = want_topk || row_max != nullptr;
   if (want_topk || row_mean != nullptr) {
     BGX_REQUIRE(ws != nullptr, BGX_E_WORKSPACE, "scan: workspace required for top-k and row means");
@@ -1849,7 +1972,9 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
       s.thr = thr;
       s.cand_cap = chunk;
       s.k = k;
-      if (a.first_pass)
+      if (k > SCAN_KMAX)
+        hipLaunchKernelGGL(scan_select_large_kernel, dim3((unsigned)Q), dim3(SELECT_THREADS_LARGE), 0, st, s, top_stride);
+      else if (a.first_pass)
         hipLaunchKernelGGL(scan_select_kernel<SELECT_THREADS_LONG>, dim3((unsigned)Q), dim3(SELECT_THREADS_LONG), 0, st, s);
       else
         hipLaunchKernelGGL(scan_select_kernel<SELECT_THREADS_SHORT>, dim3((unsigned)Q), dim3(SELECT_THREADS_SHORT), 0, st, s);
@@ -1858,11 +1983,16 @@ int scan_impl(const void* store, int64_t n_rows, int64_t D, int64_t stride, int 
     done += rows;
   }
   note_kernel(FAMILY_SCAN, main_kernel);
+  if (want_topk && k > SCAN_KMAX) {
+    hipLaunchKernelGGL(scan_sort_top_kernel, dim3((unsigned)Q), dim3(1024), 0, st, top, (const uint32_t*)top_count,
+                       top_stride);
+    BGX_HIP(hipGetLastError());
+  }
 
   if (need_init) {
     const int64_t n_fin = ((int64_t)Q * k > (row_max ? n_rows : 0)) ? (int64_t)Q * k : n_rows;
     hipLaunchKernelGGL(scan_finish_kernel, dim3((unsigned)((n_fin + 255) / 256)), dim3(256), 0, st,
-                       (const uint64_t*)top, (const uint32_t*)top_count, Q, k, row_base, topk_val, topk_idx,
+                       (const uint64_t*)top, (const uint32_t*)top_count, top_stride, Q, k, row_base, topk_val, topk_idx,
                        (const uint32_t*)row_max_enc, row_max, row_max ? n_rows : 0);
     BGX_HIP(hipGetLastError());
   }

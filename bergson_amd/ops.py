@@ -14,7 +14,7 @@ from torch import Tensor
 from . import _lib
 from ._lib import BGX_BF16, BGX_F16, BGX_F32, BlockDesc, ModuleDesc
 
-SCAN_KMAX = 2048  # largest k of the scan's fused top-k selection
+SCAN_KMAX = 65536  # largest k of the scan's fused top-k selection (sorted in LDS up to 2048, in global memory beyond)
 
 DTYPE_CODE = {torch.float32: BGX_F32, torch.float16: BGX_F16, torch.bfloat16: BGX_BF16}
 

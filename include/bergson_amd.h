@@ -377,7 +377,9 @@ size_t bgx_scan_workspace_bytes_for(int32_t Q, int32_t k, int64_t chunk_rows,
  * Outputs, each optional (NULL to skip):
  *   topk_val_dev [Q, k] fp32, topk_idx_dev [Q, k] int64: per query the k
  *     largest scores in descending order, ties broken by lower row index
- *     (torch.topk, attributor.py:229-235); requires k <= n_rows, k <= 2048.
+ *     (torch.topk, attributor.py:229-235); requires k <= n_rows, k <= 65536
+ *     (up to 2048 the running top-k of a query is kept sorted on chip; beyond,
+ *     it lives in the workspace and is sorted once at the end).
  *     Scores that are NaN or -inf are never selected, whichever pass or
  *     kernel meets them (torch.topk would rank NaN first); a query with
  *     fewer than k selectable scores gets (-inf, -1) in its last entries
