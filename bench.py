@@ -93,6 +93,9 @@ def parse_args():
     ap.add_argument("--plain-loop", action="store_true",
                     help="time the reference's loop shape (forward, backward, hooks, one batch at a time) instead "
                          "of the overlapped loop that CollectorComputer runs by default")
+    ap.add_argument("--kernels-only", action="store_true",
+                    help="leave out the legs that add no kernel of this library to a counter run: the stock-PyTorch "
+                         "baseline, configs[0], configs[3] end to end and the CPU baselines")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy (reads 1 GiB, writes 1 GiB): the known-size "
                          "kernel that hardware byte counters are scaled by")
@@ -494,7 +497,7 @@ def adam_leg(args, torch, device):
     torch.cuda.empty_cache()
     return {"workload": "configs[3]: one Pythia-410m layer, 4 x 1024 tokens, p=32, Adam, per-token rows (bf16) "
                         "written as blocks of the configuration's 98 304-wide store rows",
-            "end_to_end": adam_end_to_end(torch, device),
+            "end_to_end": None if args.kernels_only else adam_end_to_end(torch, device),
             "ms_per_layer": total_ms, "tokens_per_s_24_layers_hooks_only": N * S / (total_ms * 24e-3),
             "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": tf / MFMA_F16_PEAK_TFLOPS, "traffic": ADAM_TRAFFIC_BYTES_PER_LAYER,
@@ -705,15 +708,18 @@ def main():
     if args.per_token_only:
         print(json.dumps({"per_token": per_token_leg(args, torch, device)}))
         return
+    if args.kernels_only:
+        args.no_cpu_baseline = True
     coll, docs, lengths, extra = collection_leg(args, torch, device)
-    gpu_torch = None if args.no_scan else gpu_torch_baseline_leg(args, torch, device, docs, lengths, extra)
+    gpu_torch = None if args.no_scan or args.kernels_only else gpu_torch_baseline_leg(args, torch, device, docs, lengths,
+                                                                                     extra)
     del extra
     torch.cuda.empty_cache()
     scan = None if args.no_scan else scan_leg(args, torch, device)
     per_token = None if args.no_scan else per_token_leg(args, torch, device)
     llama = None if args.no_scan else llama_leg(args, torch, device)
     adam = None if args.no_scan else adam_leg(args, torch, device)
-    config1 = None if args.no_scan else config1_leg(args, torch, device)
+    config1 = None if args.no_scan or args.kernels_only else config1_leg(args, torch, device)
     cpu = None if args.no_cpu_baseline else cpu_baseline_leg(args, torch, docs, lengths)
 
     value = coll["tokens"] / coll["seconds"]
