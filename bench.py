@@ -53,7 +53,7 @@ COLLECT_TRAFFIC_RATIO = 1.036
 # at most 32 queries; and for per-token collection and the Llama-3-8B-shaped layers
 SCAN_TRAFFIC_RATIO_Q1024 = 1.345
 SCAN_TRAFFIC_RATIO_FEW = 1.0016
-PER_TOKEN_TRAFFIC_RATIO = 1.030
+PER_TOKEN_TRAFFIC_RATIO = 1.068
 LLAMA_TRAFFIC_RATIO = 1.007
 # bytes the four fused Adam launches of one layer fetch through the L2s and write, from the same counters
 # (profiles/adam_fused_pythia410m_layer_p32.txt): 5.19 GB + 0.07 GB, against 0.94 GB read once each
@@ -389,7 +389,9 @@ def per_token_leg(args, torch, device):
     return {"workload": "configs[1] modules, per-token rows: 48 Pythia-160m modules, 2 x 2048 tokens, p=16, Adafactor, "
                         "bf16 rows of 12288",
             "ms_per_launch": ms, "tokens_per_s_hooks_only": N * S / (ms * 1e-3),
-            "roofline": {"bound": "hbm", "kernel": "bgx::collect_persist_kernel<bf16_t, true, 2, 4, true, false>",
+            "roofline": {"bound": "hbm", "kernel": "bgx::collect_persist_kernel<bf16_t, true, 2, 4, true, false> (every token's "
+                                                  "projections, written contiguously) + bgx::token_rows_kernel (whole store "
+                                                  "rows from them), one event pair around both",
                          "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
                          "bytes_read": read, "bytes_written": written,
                          "traffic": (read + written) * PER_TOKEN_TRAFFIC_RATIO}}
