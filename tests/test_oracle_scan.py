@@ -75,3 +75,25 @@ def test_attributor_search_self_match_reverse_and_k():
     v2, i2 = S.attributor_search(index, queries, mods, 60)
     G = torch.cat([index[m] for m in mods], 1)
     torch.testing.assert_close(v2, torch.sort(G[picks] @ G.T, dim=1, descending=True).values)
+
+
+def test_attributor_index_normalisation_hand_worked():
+    """`attributor_normalize_index` and `attributor_search` on numbers worked out by hand: the norm runs over all
+    modules of a row together (3-4-12 -> 13), a zero row becomes zeros (0/0 -> NaN -> 0), and the search's cosines
+    and order follow."""
+    idx = {"a": torch.tensor([[3.0, 4.0], [0.0, 0.0], [0.0, 5.0], [-6.0, 0.0]]),
+           "b": torch.tensor([[12.0], [0.0], [0.0], [8.0]])}
+    norm = S.attributor_normalize_index(idx, ["a", "b"])
+    assert torch.allclose(norm["a"], torch.tensor([[3 / 13, 4 / 13], [0.0, 0.0], [0.0, 1.0], [-0.6, 0.0]]))
+    assert torch.allclose(norm["b"], torch.tensor([[12 / 13], [0.0], [0.0], [0.8]]))
+    # one query along (0, 1 | 0): cosines 4/13, 0, 1, 0 -> rows 2, 0, then the two zeros (their order is not defined)
+    q = {"a": torch.tensor([[0.0, 2.0]]), "b": torch.tensor([[0.0]])}
+    vals, rows = S.attributor_search(idx, q, ["a", "b"], 4, unit_norm=True)
+    assert rows[0, :2].tolist() == [2, 0] and sorted(rows[0, 2:].tolist()) == [1, 3]
+    assert torch.allclose(vals, torch.tensor([[1.0, 4 / 13, 0.0, 0.0]]), atol=1e-6)
+    # without unit norms: plain inner products 8, 0, 10, 0; reverse = smallest first
+    vals, rows = S.attributor_search(idx, q, ["a", "b"], 2, unit_norm=False)
+    assert rows.tolist() == [[2, 0]] and vals.tolist() == [[10.0, 8.0]]
+    vals, rows = S.attributor_search(idx, {"a": torch.tensor([[1.0, 1.0]]), "b": torch.tensor([[1.0]])}, ["a", "b"], 2,
+                                         unit_norm=False, reverse=True)
+    assert rows.tolist() == [[1, 3]] and vals.tolist() == [[0.0, 2.0]]   # 19, 0, 5, 2 -> smallest first
