@@ -59,48 +59,42 @@ def _allocate_file(path: Path, nbytes: int) -> None:
         os.fsync(f.fileno())
 
 
-def create_token_index(root: Path, num_token_grads: np.ndarray, grad_sizes: dict[str, int], dtype
-                       ) -> tuple[np.memmap, np.ndarray]:
-    """Ragged per-token store: gradients.bin + offsets.npy + info.json (bergson/data.py:65-137)."""
+def _create_store(root: Path, n_rows: int, grad_sizes: dict[str, int], dtype, *, num_items: int,
+                  offsets: np.ndarray | None) -> np.ndarray:
+    """The files of a gradient store and a writable map of its rows: `gradients.bin` (n_rows x sum(grad_sizes) raw
+    values, sized without writing zeros and synced before any other rank maps it), `info.json`, and for a ragged
+    per-token store `offsets.npy` (bergson/data.py:65-137, :392-445).  Rank 0 creates, everyone maps."""
     root = Path(root)
     name = _dtype_name(dtype)
     np_dtype = storage_np_dtype(name)
-    total_grad_dim = sum(grad_sizes.values())
-    offsets = np.zeros(len(num_token_grads) + 1, dtype=np.int64)
-    np.cumsum(num_token_grads, out=offsets[1:])
-    total_tokens = int(offsets[-1])
-    grad_path = root / "gradients.bin"
+    width = sum(grad_sizes.values())
+    rows_file = root / "gradients.bin"
     if _rank() == 0:
         root.mkdir(parents=True, exist_ok=True)
-        _allocate_file(grad_path, np_dtype.itemsize * total_tokens * total_grad_dim)
-        np.save(root / "offsets.npy", offsets)
-        with (root / "info.json").open("w") as f:
-            json.dump({"attribute_tokens": True, "num_items": len(num_token_grads), "num_grads": total_tokens,
-                       "grad_sizes": grad_sizes, "base_dtype": name}, f, indent=2)
+        _allocate_file(rows_file, n_rows * width * np_dtype.itemsize)
+        if offsets is not None:
+            np.save(root / "offsets.npy", offsets)
+        info = {"attribute_tokens": offsets is not None, "num_items": num_items, "num_grads": n_rows,
+                "grad_sizes": grad_sizes, "base_dtype": name}
+        (root / "info.json").write_text(json.dumps(info, indent=2))
     if dist.is_initialized():
         dist.barrier()
-    if total_tokens == 0:
-        return np.zeros((0, total_grad_dim), dtype=np_dtype), offsets  # type: ignore[return-value]
-    mmap = np.memmap(grad_path, dtype=np_dtype, mode="r+", shape=(total_tokens, total_grad_dim))
-    return mmap, offsets
+    if n_rows == 0:  # an empty file cannot be mapped
+        return np.zeros((0, width), dtype=np_dtype)
+    return np.memmap(rows_file, dtype=np_dtype, mode="r+", shape=(n_rows, width))
+
+
+def create_token_index(root: Path, num_token_grads: np.ndarray, grad_sizes: dict[str, int], dtype
+                       ) -> tuple[np.memmap, np.ndarray]:
+    """Ragged per-token store: rows offsets[i] .. offsets[i + 1] belong to example i (bergson/data.py:65-137)."""
+    offsets = np.concatenate(([0], np.cumsum(num_token_grads, dtype=np.int64))).astype(np.int64)
+    rows = _create_store(root, int(offsets[-1]), grad_sizes, dtype, num_items=len(num_token_grads), offsets=offsets)
+    return rows, offsets  # type: ignore[return-value]
 
 
 def create_index(root: Path, num_grads: int, grad_sizes: dict[str, int], dtype) -> np.memmap:
-    """Flat [num_grads, total_grad_dim] store: gradients.bin + info.json (bergson/data.py:392-445)."""
-    root = Path(root)
-    name = _dtype_name(dtype)
-    np_dtype = storage_np_dtype(name)
-    total = sum(grad_sizes.values())
-    grad_path = root / "gradients.bin"
-    if _rank() == 0:
-        root.mkdir(parents=True, exist_ok=True)
-        _allocate_file(grad_path, np_dtype.itemsize * total * num_grads)
-        with (root / "info.json").open("w") as f:
-            json.dump({"attribute_tokens": False, "num_items": num_grads, "num_grads": num_grads,
-                       "grad_sizes": grad_sizes, "base_dtype": name}, f, indent=2)
-    if dist.is_initialized():
-        dist.barrier()
-    return np.memmap(grad_path, dtype=np_dtype, mode="r+", shape=(num_grads, total))
+    """Flat store: row i is example i (bergson/data.py:392-445)."""
+    return _create_store(root, num_grads, grad_sizes, dtype, num_items=num_grads, offsets=None)  # type: ignore[return-value]
 
 
 def column_offsets(grad_sizes: dict[str, int]) -> dict[str, tuple[int, int]]:
@@ -341,23 +335,28 @@ def pad_and_tensor(sequences: list[list[int]], labels: list[list[int]] | None = 
     """(padded ids, padded labels (-100), shift_loss_masks, collection_masks) (bergson/data.py:743-806).
 
     collection_masks[n, s] = s + 1 < len(sequences[n]): every real position but the last.
+    shift_loss_masks[n, s] = labels[n, s + 1] is supervised (False in the last column).
+    Everything is laid out on the host -- two [N, S] integer arrays filled row by row -- and uploaded once; the
+    masks are computed on the device from the uploaded labels and lengths.
     """
-    if labels is None:
-        labels = sequences
-    max_len = max(len(seq) for seq in sequences)
+    labels = sequences if labels is None else labels
+    lengths = [len(seq) for seq in sequences]
+    width = max(lengths)
     if sync_max_len and dist.is_initialized():
-        t = torch.tensor(max_len, device=device)
-        dist.all_reduce(t, op=dist.ReduceOp.MAX)
-        max_len = int(t)
-    padded = [list(seq) + [padding_value] * (max_len - len(seq)) for seq in sequences]
-    padded_labels = [list(label) + [-100] * (max_len - len(label)) for label in labels]
-    # built on the host and moved once: one H2D copy per tensor instead of device-side construction
-    tokens = torch.tensor(padded, dtype=dtype).to(device, non_blocking=True)
-    labels_t = torch.tensor(padded_labels, dtype=dtype).to(device, non_blocking=True)
-    N, S = tokens.shape
-    shift_loss_masks = torch.zeros(N, S, dtype=torch.bool, device=device)
-    shift_loss_masks[:, :-1] = labels_t[:, 1:] != -100
-    lengths = torch.tensor([len(seq) for seq in sequences]).to(device, non_blocking=True)
-    positions = torch.arange(S, device=device)
-    collection_masks = (positions.unsqueeze(0) + 1) < lengths.unsqueeze(1)
-    return tokens, labels_t, shift_loss_masks, collection_masks
+        widest = torch.tensor(width, device=device)
+        dist.all_reduce(widest, op=dist.ReduceOp.MAX)
+        width = int(widest)
+    ids = np.full((len(sequences), width), padding_value, dtype=np.int64)
+    lab = np.full((len(sequences), width), -100, dtype=np.int64)
+    for n, (seq, label) in enumerate(zip(sequences, labels)):
+        ids[n, :len(seq)] = seq
+        lab[n, :len(label)] = label
+    tokens, labels_t = torch.from_numpy(ids), torch.from_numpy(lab)
+    if dtype is not None and dtype != torch.long:
+        tokens, labels_t = tokens.to(dtype), labels_t.to(dtype)
+    tokens = tokens.to(device, non_blocking=True)
+    labels_t = labels_t.to(device, non_blocking=True)
+    supervised_next = torch.nn.functional.pad(labels_t[:, 1:] != -100, (0, 1), value=False)
+    lengths_t = torch.tensor(lengths).to(device, non_blocking=True)
+    collection_masks = torch.arange(1, width + 1, device=device).unsqueeze(0) < lengths_t.unsqueeze(1)
+    return tokens, labels_t, supervised_next, collection_masks

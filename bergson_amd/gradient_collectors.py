@@ -31,6 +31,22 @@ from .utils import DeviceIndexRing, get_gradient_dtype
 class _DeferredBatchMixin:
     """Shared batch logic of the collectors that write rows of all modules in one launch."""
 
+    def _prepare_collection(self, save_dtype: torch.dtype | None = None) -> dict[str, int]:
+        """What a row-writing collector fixes before its first batch: per-token or per-sequence rows, the dtype the
+        rows are saved in with its clamp range (`save_dtype`, default the model's gradient dtype), and the
+        per-document loss vector; returns the column width of every stored block, in store order."""
+        device = self.model.device
+        if not isinstance(device, torch.device):
+            raise AssertionError("Model device is not set correctly")
+        self.attribute_tokens = bool(self.cfg.attribute_tokens)
+        if self.attribute_tokens and self.preprocess_cfg.aggregation != "none":
+            raise AssertionError("attribute_tokens is incompatible with reduce mode.")
+        self.save_dtype = save_dtype or get_gradient_dtype(self.model)
+        limits = torch.finfo(self.save_dtype)
+        self.lo, self.hi = limits.min, limits.max
+        self.per_doc_losses = torch.zeros(len(self.data), dtype=torch.float32, device=device)
+        return {name: math.prod(shape) for name, shape in self.shapes().items()}
+
     def _column_of(self, name: str) -> int:
         cols = getattr(self, "_columns", None)
         if cols is None:
@@ -122,24 +138,14 @@ class GradientCollector(_DeferredBatchMixin, HookCollectorBase):
     come from its training callback, bergson/huggingface.py:41.)"""
 
     def setup(self) -> None:
-        assert isinstance(self.model.device, torch.device), "Model device is not set correctly"
-        self.attribute_tokens = self.cfg.attribute_tokens
-        if self.cfg.attribute_tokens:
-            assert self.preprocess_cfg.aggregation == "none", "attribute_tokens is incompatible with reduce mode."
-        self.save_dtype = self.store_dtype or get_gradient_dtype(self.model)
-        self.lo = torch.finfo(self.save_dtype).min
-        self.hi = torch.finfo(self.save_dtype).max
-        self.per_doc_losses = torch.full((len(self.data),), device=self.model.device, dtype=torch.float32,
-                                         fill_value=0.0)
+        grad_sizes = self._prepare_collection(self.store_dtype)
         self.save_index = self.scorer is None and not self.skip_index
+        self.builder = None
         if self.save_index:
-            grad_sizes = {name: math.prod(s) for name, s in self.shapes().items()}
             self.builder = Builder(self.data, grad_sizes, self.save_dtype, self.preprocess_cfg,
-                                   attribute_tokens=self.cfg.attribute_tokens,
+                                   attribute_tokens=self.attribute_tokens,
                                    path=self.cfg.partial_run_path if self.cfg.run_path else None,
                                    device=self.model.device, device_store_bytes=self.device_store_bytes)
-        else:
-            self.builder = None
 
     @HookCollectorBase.split_attention_heads
     def backward_hook(self, module: nn.Module, g: Tensor):

@@ -44,24 +44,14 @@ class InMemoryCollector(_DeferredBatchMixin, HookCollectorBase):
         super().__post_init__()
 
     def setup(self) -> None:
-        assert isinstance(self.model.device, torch.device), "Model device is not set correctly"
         if not self.skip_hessians and self.processor.projection_target == "global":
             raise NotImplementedError("autocorrelation statistics of a global projection")
         self._gram_blocks = None
-        self.attribute_tokens = self.cfg.attribute_tokens
-        if self.cfg.attribute_tokens:
-            assert self.preprocess_cfg.aggregation == "none", "attribute_tokens is incompatible with reduce mode."
-        self.save_dtype = get_gradient_dtype(self.model)
-        self.lo = torch.finfo(self.save_dtype).min
-        self.hi = torch.finfo(self.save_dtype).max
-        self.per_doc_losses = torch.full((len(self.data),), device=self.model.device, dtype=torch.float32,
-                                         fill_value=0.0)
-        self.gradients = {}
-        self.scores = None
-        if self.builder is None and self.scorer is None:
-            grad_sizes = {name: math.prod(s) for name, s in self.shapes().items()}
+        grad_sizes = self._prepare_collection()
+        self.gradients, self.scores = {}, None
+        if self.builder is None and self.scorer is None:  # rows stay in memory: a Builder without a path
             self.builder = Builder(self.data, grad_sizes, self.save_dtype, self.preprocess_cfg,
-                                   attribute_tokens=self.cfg.attribute_tokens, device=self.model.device)
+                                   attribute_tokens=self.attribute_tokens, device=self.model.device)
 
     @HookCollectorBase.split_attention_heads
     def backward_hook(self, module: nn.Module, g: Tensor) -> None:
@@ -109,22 +99,24 @@ class InMemoryCollector(_DeferredBatchMixin, HookCollectorBase):
         return len(self.data)
 
     def teardown(self) -> None:
+        """Detaches from the model, finishes the autocorrelation statistics and exposes what was gathered:
+        `gradients[name]` = the module's columns of the in-memory store, `scores` = the scorer's."""
         self.remove_hooks()
         if dist.is_initialized():
             dist.reduce(self.per_doc_losses, dst=0)
-        grad_sizes = {name: math.prod(s) for name, s in self.shapes().items()}
+        widths = {name: math.prod(shape) for name, shape in self.shapes().items()}
         if not self.skip_hessians and self.processor.hessians:
             from .hessians import process_autocorrelation_matrices
 
             if dist.is_initialized() and dist.get_world_size() > 1:
                 raise NotImplementedError("autocorrelation statistics across ranks")
-            process_autocorrelation_matrices(self.processor, self.processor.hessians, self.num_rows(), grad_sizes)
+            process_autocorrelation_matrices(self.processor, self.processor.hessians, self.num_rows(), widths)
         if self.builder is not None:
+            from .data import column_offsets
+
             self.builder.teardown()
-            buf = self.builder.grad_buffer
-            offset = 0
-            for name, dim in grad_sizes.items():
-                self.gradients[name] = numpy_to_tensor(buf[:, offset:offset + dim], self.builder.base_dtype)
-                offset += dim
+            rows = self.builder.grad_buffer
+            self.gradients.update({name: numpy_to_tensor(rows[:, lo:hi], self.builder.base_dtype)
+                                   for name, (lo, hi) in column_offsets(widths).items()})
         if self.scorer is not None:
             self.scores = self.scorer.writer.scores
