@@ -279,15 +279,21 @@ __device__ __forceinline__ void scan_block_epilogue_full(const ScanArgs& args, f
 #pragma unroll
     for (int e = 1; e < 16; ++e) cmax = fmaxf(cmax, acc_row[j][e]);
     if (__builtin_expect(cmax > thr[j], 0)) {
+      // the lane's candidates of this block are counted and their places reserved with one atomic: one wait for the
+      // wave per query block (an atomic per candidate is one wait per row in which any lane has one -- most of the
+      // sixteen while the thresholds are still loose)
       const int64_t q = q_b + j * 32;
-      uint32_t* const cnt = args.cand_count + q;
       uint64_t* const list = args.cand + q * args.cand_cap;
+      uint32_t n = 0;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) n += acc_row[j][e] > thr[j] ? 1u : 0u;
+      uint32_t pos = atomicAdd(args.cand_count + q, n);
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const float v = acc_row[j][e];
         if (v > thr[j]) {
-          const uint32_t pos = atomicAdd(cnt, 1u);
           if ((int64_t)pos < args.cand_cap) list[pos] = make_key(v, (uint32_t)(grow_b + (e >> 2) * 8 + (e & 3)));
+          ++pos;
         }
       }
     }
