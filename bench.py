@@ -236,6 +236,55 @@ def gpu_torch_baseline_leg(args, torch, device, docs, lengths, extra):
                     "device) on the same model, batches and GPU"}
 
 
+class BoardPower:
+    """Samples the board's power sensor (hwmon `power1_input`, microwatts) every 20 ms while the block runs.
+
+    The matrix-bound kernels run the chip into its power limit (`power1_cap`), which is what sets their clocks:
+    the legs that time them report the power they drew beside their rate.  `report()` is None where the sensor
+    cannot be read."""
+
+    def __init__(self):
+        import glob
+        import threading
+
+        found = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input"))
+        self.path = found[0] if found else None
+        self.samples: list[float] = []
+        self._stop = threading.Event()
+        self._thread = threading.Thread(target=self._run, daemon=True)
+
+    def _read(self, path):
+        try:
+            with open(path) as f:
+                return int(f.read()) / 1e6
+        except (OSError, ValueError):
+            return None
+
+    def _run(self):
+        while not self._stop.is_set():
+            w = self._read(self.path)
+            if w is not None:
+                self.samples.append(w)
+            self._stop.wait(0.02)
+
+    def __enter__(self):
+        if self.path is not None:
+            self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop.set()
+        if self.path is not None:
+            self._thread.join()
+
+    def report(self):
+        if not self.samples:
+            return None
+        cap = self._read(self.path.replace("power1_input", "power1_cap"))
+        return {"mean_w": sum(self.samples) / len(self.samples), "max_w": max(self.samples), "cap_w": cap,
+                "samples": len(self.samples)}
+
+
 def scan_leg(args, torch, device):
     from bergson_amd import ops
 
@@ -263,11 +312,12 @@ def scan_leg(args, torch, device):
     torch.cuda.synchronize()
     reps = 10  # the first scans of a burst run ~1 % slower (the chip's clocks settle under sustained load)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(reps):
-        res = run()
-    e1.record()
-    torch.cuda.synchronize()
+    with BoardPower() as power:
+        e0.record()
+        for _ in range(reps):
+            res = run()
+        e1.record()
+        torch.cuda.synchronize()
     ms = e0.elapsed_time(e1) / reps
     flops = 2.0 * n * D * Q
     out = {
@@ -278,6 +328,7 @@ def scan_leg(args, torch, device):
                      "kernel": "bgx::scan_wide_kernel<f16_t> (384 x 256 tiles, operands loaded straight into LDS)"},
         "hbm_gbs": n * D * 2 / (ms * 1e-3) / 1e9,
         "top1_mean": float(res.topk_values[:Q, 0].mean().item()),
+        "board_power": power.report(),
     }
     # the same scan with the store's row norms known from an earlier scan, as Attributor runs every search after
     # its first (the reference normalises an index once, when it loads it): the tile kernel's K loop without the
@@ -288,20 +339,40 @@ def scan_leg(args, torch, device):
 
     res_known = run_known()
     torch.cuda.synchronize()
-    e0.record()
-    for _ in range(reps):
-        run_known()
-    e1.record()
-    torch.cuda.synchronize()
+    with BoardPower() as power:
+        e0.record()
+        for _ in range(reps):
+            run_known()
+        e1.record()
+        torch.cuda.synchronize()
     ms_known = e0.elapsed_time(e1) / reps
     out["known_row_norms"] = {
         "ms": ms_known, "rows_per_s": n / (ms_known * 1e-3),
         "roofline": {"bound": "mfma", "achieved": flops / (ms_known * 1e-3) / 1e12, "peak": MFMA_F16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": flops / (ms_known * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS},
         "same_top_k": bool(torch.equal(res_known.topk_indices, res.topk_indices)),
+        "board_power": power.report(),
         "what": "bgx_scan_known_norms: row sums of squares taken from an earlier scan of the store instead of "
                 "being summed again in the K loop",
     }
+    # for scale: the library's GEMM (hipBLASLt through torch.matmul) on the scan's shape -- scores only, no norms,
+    # no selection; 2 GB of fp16 scores written.  Both run the chip into its power limit, which sets the clocks.
+    dense = torch.empty((n, Q), dtype=torch.float16, device=device)
+    qt = qd.T  # a view: both operands contiguous along D, the layout the library is fastest on
+    torch.matmul(store, qt, out=dense)
+    torch.cuda.synchronize()
+    with BoardPower() as power:
+        e0.record()
+        for _ in range(reps):
+            torch.matmul(store, qt, out=dense)
+        e1.record()
+        torch.cuda.synchronize()
+    ms_lib = e0.elapsed_time(e1) / reps
+    out["library_gemm_same_shape"] = {"ms": ms_lib, "tflops": flops / (ms_lib * 1e-3) / 1e12,
+                                      "frac_of_peak": flops / (ms_lib * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
+                                      "board_power": power.report(),
+                                      "what": "torch.matmul(store [n, D] fp16, queries^T [D, Q]) -> [n, Q] fp16"}
+    del dense, qt
     # the one pass that forms those sums when an index is loaded (Attributor: the reference normalises the index
     # at load time), bit-equal to the sums the scan hands out
     loaded = ops.row_sumsq(store)
@@ -472,6 +543,8 @@ def adam_leg(args, torch, device):
     # 30 timed launches behind 5 untimed ones per module: the first launches of a burst run at lower clocks (5 timed
     # launches read 7 % slower than 60), and the configuration this stands for issues 96 of them per batch
     reps, total_ms, total_flops, modules = 30, 0.0, 0.0, {}
+    power = BoardPower()
+    power.__enter__()
     for block, (name, (I, O)) in enumerate((("query_key_value", (d, 3 * d)), ("dense", (d, d)),
                                             ("dense_h_to_4h", (d, 4 * d)), ("dense_4h_to_h", (4 * d, d)))):
         a = rnd(N, S, I).to(torch.bfloat16)
@@ -494,6 +567,7 @@ def adam_leg(args, torch, device):
         total_ms += ms
         total_flops += flops
         del a, g, v, prep
+    power.__exit__()
     tf = total_flops / (total_ms * 1e-3) / 1e12
     del out
     torch.cuda.empty_cache()
@@ -501,6 +575,7 @@ def adam_leg(args, torch, device):
                         "written as blocks of the configuration's 98 304-wide store rows",
             "end_to_end": None if args.kernels_only else adam_end_to_end(torch, device),
             "ms_per_layer": total_ms, "tokens_per_s_24_layers_hooks_only": N * S / (total_ms * 24e-3),
+            "board_power": power.report(),
             "roofline": {"bound": "mfma", "achieved": tf, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": tf / MFMA_F16_PEAK_TFLOPS, "traffic": ADAM_TRAFFIC_BYTES_PER_LAYER,
                          "kernel": "bgx::adam_fused_wide_kernel<bf16_t>"},

@@ -248,21 +248,30 @@ class Builder:
             self.grad_buffer.flush()
 
     def teardown(self) -> None:
+        """Everything staged reaches the store, then the store is completed: one row per item needs nothing more
+        on disk (an in-memory store is summed over the ranks, each of which filled its own rows); an aggregated
+        store is the one row `_finish_aggregate` writes (builder.py:196-232)."""
         self.flush()
-        if self.preprocess_cfg.aggregation == "none":
-            if dist.is_initialized() and not isinstance(self.grad_buffer, np.memmap):
-                if self.grad_buffer.dtype == np.uint16:
-                    raise NotImplementedError("gathering an in-memory bfloat16 store across ranks")
-                dist.all_reduce(torch.from_numpy(self.grad_buffer), op=dist.ReduceOp.SUM)
-            return
-        assert self.in_memory_grad_buffer is not None
-        if dist.is_initialized():
-            dist.reduce(self.in_memory_grad_buffer, dst=0, op=dist.ReduceOp.SUM)
+        ranks = dist.is_initialized()
+        if self.preprocess_cfg.aggregation != "none":
+            self._finish_aggregate(ranks)
+        elif ranks and not isinstance(self.grad_buffer, np.memmap):
+            if self.grad_buffer.dtype == np.uint16:
+                raise NotImplementedError("gathering an in-memory bfloat16 store across ranks")
+            dist.all_reduce(torch.from_numpy(self.grad_buffer), op=dist.ReduceOp.SUM)
+
+    def _finish_aggregate(self, ranks: bool) -> None:
+        """The running sum on the device becomes the store's single row: summed onto rank 0, divided by the item
+        count for a mean, scaled to unit length if asked, and written by rank 0 in the store's dtype."""
+        total = self.in_memory_grad_buffer
+        if total is None:
+            raise AssertionError("an aggregating Builder has no running sum")
+        if ranks:
+            dist.reduce(total, dst=0, op=dist.ReduceOp.SUM)
         if self.preprocess_cfg.aggregation == "mean":
-            self.in_memory_grad_buffer /= self.num_items
+            total /= self.num_items
         if self.preprocess_cfg.normalize_aggregated_grad:
-            ops.unit_normalize_rows_(self.in_memory_grad_buffer)
-        self.in_memory_grad_buffer = self.in_memory_grad_buffer.cpu()
-        rank = dist.get_rank() if dist.is_initialized() else 0
-        if rank == 0:
-            self.grad_buffer[:] = self.in_memory_grad_buffer.numpy().astype(self.grad_buffer.dtype)
+            ops.unit_normalize_rows_(total)
+        self.in_memory_grad_buffer = host = total.cpu()
+        if not ranks or dist.get_rank() == 0:
+            self.grad_buffer[:] = host.numpy().astype(self.grad_buffer.dtype)
