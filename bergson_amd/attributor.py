@@ -60,7 +60,7 @@ class Attributor:
 
     def __init__(self, index_path: str | Path, device: str = "cuda", dtype: torch.dtype = torch.float32,
                  unit_norm: bool = False, faiss_cfg=None, inversion_cfg=None, hessian_path: str | Path | None = None,
-                 ev_correction: bool = False):
+                 ev_correction: bool = False, device_store_bytes: int | None = None):
         if faiss_cfg is not None:
             raise NotImplementedError("FAISS search is outside this package; the exact scan replaces the Flat index")
         self.device = torch.device(device)
@@ -92,17 +92,48 @@ class Attributor:
             raise TypeError("float64 stores are not supported by the scan kernels")
         self._row_sumsq: Tensor | None = None
         self._row_sumsq_of: tuple | None = None
-        self.store = upload_store(load_gradients(index_path), base, self.device)
-        self.N = self.store.shape[0]
-        if self.preconditioner is not None and unit_norm:
-            # split mode: the index rows are transformed once, before the scan normalises them.  The
-            # transformed store is fp32 (what g.float() @ H gives) when a second, fp32 copy fits in half of the
-            # free memory, else it keeps the store's dtype.
-            free, _ = torch.cuda.mem_get_info(self.device)
-            out_dtype = torch.float32 if self.store.numel() * 4 <= free // 2 else self.store.dtype
-            self.store = self.preconditioner.apply_rows(self.store, self.grad_sizes, out_dtype=out_dtype)
-        if unit_norm:
-            self.row_sumsq()  # the reference normalises the index when it loads it (attributor.py:137-167)
+        mapped = load_gradients(index_path)
+        self.N = mapped.shape[0]
+        # The store lives in HBM when it fits (`device_store_bytes`, default four fifths of the free memory).  A
+        # larger one stays mapped on the host and every search streams it through the device in slabs of rows,
+        # each scanned like a store of its own (`row_base` = its first row) and merged into the running top-k.
+        free, _ = torch.cuda.mem_get_info(self.device)
+        budget = int(free * 0.8) if device_store_bytes is None else int(device_store_bytes)
+        self._base = base
+        self._mapped = None
+        self._slab_rows = 0
+        self._slab_sumsq: dict[int, Tensor] = {}
+        split = self.preconditioner is not None and unit_norm
+        if mapped.size * mapped.dtype.itemsize <= budget:
+            self.store = upload_store(mapped, base, self.device)
+            if split:
+                # split mode: the index rows are transformed once, before the scan normalises them.  The
+                # transformed store is fp32 (what g.float() @ H gives) when a second, fp32 copy fits in half of the
+                # free memory, else it keeps the store's dtype.
+                free, _ = torch.cuda.mem_get_info(self.device)
+                out_dtype = torch.float32 if self.store.numel() * 4 <= free // 2 else self.store.dtype
+                self.store = self.preconditioner.apply_rows(self.store, self.grad_sizes, out_dtype=out_dtype)
+            if unit_norm:
+                self.row_sumsq()  # the reference normalises the index when it loads it (attributor.py:137-167)
+        else:
+            self.store = None
+            self._mapped = mapped
+            row_bytes = mapped.shape[1] * mapped.dtype.itemsize * (2 if split else 1)  # split mode: slab + its transform
+            self._slab_rows = max(1, budget // row_bytes)
+
+    def _slabs(self):
+        """(first row, device rows, their sums of squares or None) for every slab of a store that is streamed."""
+        for lo in range(0, self.N, self._slab_rows):
+            hi = min(self.N, lo + self._slab_rows)
+            rows = upload_store(self._mapped[lo:hi], self._base, self.device)
+            if self.preconditioner is not None and self.unit_norm:
+                rows = self.preconditioner.apply_rows(rows, self.grad_sizes, out_dtype=rows.dtype)
+            norms = None
+            if self.unit_norm:
+                if lo not in self._slab_sumsq:  # 4 bytes per row: kept for the next search
+                    self._slab_sumsq[lo] = ops.row_sumsq(rows)
+                norms = self._slab_sumsq[lo]
+            yield lo, rows, norms
 
     def row_sumsq(self) -> Tensor:
         """Sums of squares of the store's rows (one HBM-bound pass), kept for every search: the index-side
@@ -110,6 +141,8 @@ class Attributor:
         multipliers the scan takes instead of summing the squares of every row again.  Recomputed when `store`
         has been replaced or written to since (its storage, shape or version counter changed)."""
         store = self.store
+        if store is None:
+            raise RuntimeError("this store is streamed from the host in slabs; its row sums are kept per slab")
         state = (store.data_ptr(), tuple(store.shape), store.dtype, store._version)
         if self._row_sumsq is None or self._row_sumsq_of != state:
             self._row_sumsq = ops.row_sumsq(store)
@@ -119,6 +152,8 @@ class Attributor:
     @property
     def grads(self) -> dict[str, Tensor]:
         """Per-module column views of the device store (raw rows; normalisation happens inside the scan)."""
+        if self.store is None:
+            raise RuntimeError("this store is streamed from the host in slabs and has no device-resident views")
         return {name: self.store[:, lo:hi] for name, (lo, hi) in self._columns.items()}
 
     def search(self, queries: dict[str, Tensor], k: int | None, modules: set[str] | None = None,
@@ -140,27 +175,43 @@ class Attributor:
         # a power-of-two rescale keeps small query entries clear of the fp16 subnormal range
         qmax = float(q.abs().max().item())
         shift = 0 if qmax == 0 or not math.isfinite(qmax) else -math.frexp(qmax)[1]
-        qd = (q * (2.0 ** shift)).to(self.store.dtype)
-        norms = self.row_sumsq() if self.unit_norm else None
-        if k <= ops.SCAN_KMAX:
-            res = ops.scan(self.store, qd, unit_norm=self.unit_norm, k=k, query_scale=2.0 ** (-shift), row_sumsq=norms)
-            values, indices = res.topk_values, res.topk_indices
+        if self.store is not None:
+            norms = self.row_sumsq() if self.unit_norm else None
+            values, indices = self._search_rows(self.store, 0, norms, q, shift, k)
         else:
-            # beyond the fused selection's capacity of 65 536 (k = None asks for a full ranking of the store): the
-            # scan writes every score, in slices of queries so that [n, Q'] fp32 stays near 4 GB, and the
-            # ranking is the library's
-            step = max(1, (1 << 30) // max(1, self.N))
-            vals, idxs = [], []
-            for lo in range(0, qd.shape[0], step):
-                res = ops.scan(self.store, qd[lo:lo + step].contiguous(), unit_norm=self.unit_norm,
-                               query_scale=2.0 ** (-shift), want_scores=True, row_sumsq=norms)
-                v, i = torch.topk(res.scores.T, k, dim=1)
-                vals.append(v)
-                idxs.append(i)
-            values, indices = torch.cat(vals), torch.cat(idxs)
+            values = indices = None
+            for lo, rows, norms in self._slabs():
+                v, i = self._search_rows(rows, lo, norms, q, shift, min(k, rows.shape[0]))
+                if values is not None:  # the running top-k and the slab's, merged
+                    v, i = torch.cat([values, v], dim=1), torch.cat([indices, i], dim=1)
+                    v, pick = torch.topk(v, min(k, v.shape[1]), dim=1)
+                    i = torch.gather(i, 1, pick)
+                values, indices = v, i
+                del rows
         if reverse:
             values = -values
         return torch.return_types.topk((values.to(self.dtype), indices))
+
+    def _search_rows(self, rows: Tensor, row_base: int, norms: Tensor | None, q: Tensor, shift: int, k: int):
+        """Top-k of `rows` (store rows `row_base` onwards) for fp32 queries `q`: (values, store row numbers)."""
+        qd = (q * (2.0 ** shift)).to(rows.dtype)
+        scale = 2.0 ** (-shift)
+        if k <= ops.SCAN_KMAX:
+            res = ops.scan(rows, qd, unit_norm=self.unit_norm, k=k, query_scale=scale, row_base=row_base,
+                           row_sumsq=norms)
+            return res.topk_values, res.topk_indices
+        # beyond the fused selection's capacity of 65 536 (k = None asks for a full ranking of the store): the
+        # scan writes every score, in slices of queries so that [n, Q'] fp32 stays near 4 GB, and the
+        # ranking is the library's
+        step = max(1, (1 << 30) // max(1, rows.shape[0]))
+        vals, idxs = [], []
+        for lo in range(0, qd.shape[0], step):
+            res = ops.scan(rows, qd[lo:lo + step].contiguous(), unit_norm=self.unit_norm, query_scale=scale,
+                           want_scores=True, row_sumsq=norms)
+            v, i = torch.topk(res.scores.T, k, dim=1)
+            vals.append(v)
+            idxs.append(i + row_base)
+        return torch.cat(vals), torch.cat(idxs)
 
     @contextmanager
     def trace(self, module: nn.Module, k: int | None, *, modules: set[str] | None = None, reverse: bool = False

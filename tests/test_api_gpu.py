@@ -332,6 +332,44 @@ def test_build_then_score_entry_points(device, tmp_path):
         assert (got - want).abs().max().item() <= 1e-3
 
 
+@pytest.mark.parametrize("unit_norm", [True, False])
+def test_attributor_streams_a_store_that_does_not_fit(device, tmp_path, unit_norm):
+    """A store larger than the device budget stays mapped on the host and is searched in slabs of rows: the
+    resident store's values to fp32 rounding (a slab of 700 rows and a store of 5000 go to different kernels,
+    which add up over D in different orders), the same rows up to swaps of scores that close, row numbers counted
+    over the whole store; k above a slab's row count and a second search (the slabs' row norms are kept)
+    included."""
+    from bergson_amd import Attributor, GradientProcessor
+    from bergson_amd.data import create_index
+
+    n, sizes = 5000, {"a": 192, "b": 64}
+    gen = torch.Generator().manual_seed(21)
+    rows = torch.randn(n, 256, generator=gen) * (torch.rand(n, 1, generator=gen) * 2 + 0.2)
+    path = tmp_path / "slabs"
+    mm = create_index(path, n, sizes, "float16")
+    mm[:] = rows.to(torch.float16).numpy()
+    mm.flush()
+    GradientProcessor(projection_dim=None).save(path)
+    resident = Attributor(path, device="cuda:0", unit_norm=unit_norm)
+    streamed = Attributor(path, device="cuda:0", unit_norm=unit_norm, device_store_bytes=700 * 256 * 2)
+    assert resident.store is not None and streamed.store is None and streamed._slab_rows == 700
+    with pytest.raises(RuntimeError, match="slabs"):
+        streamed.grads
+    picks = torch.tensor([3, 699, 700, 2500, 4999])
+    q = rows[picks] + 0.05 * torch.randn(5, 256, generator=gen)
+    queries = {"a": q[:, :192].to(device), "b": q[:, 192:].to(device)}
+    for k in (1, 10, 900, 10):
+        v0, i0 = resident.search(queries, k)
+        v1, i1 = streamed.search(queries, k)
+        assert v1.shape == (5, k) and torch.allclose(v0, v1, rtol=1e-5, atol=2e-5)
+        assert (i0 == i1).float().mean().item() >= 0.98
+        assert not unit_norm or (i1[:, 0].cpu() == picks).all()  # by cosine a noisy copy finds its original
+    assert sorted(streamed._slab_sumsq) == (list(range(0, n, 700)) if unit_norm else [])
+    rv0, ri0 = resident.search(queries, 4, reverse=True)
+    rv1, ri1 = streamed.search(queries, 4, reverse=True)
+    assert torch.allclose(rv0, rv1, rtol=1e-5, atol=2e-5) and (ri0 == ri1).float().mean().item() >= 0.9
+
+
 def test_attributor_full_ranking_beyond_the_fused_top_k(device, tmp_path):
     """k = None ranks the whole store (attributor.py:229-235 with k = None -> N); past the fused selection's
     2048 entries the scan writes every score and the ranking is torch.topk's."""
