@@ -107,6 +107,14 @@ int fullgrad_seq_gemm_impl(const void* a, const void* g, int64_t a_seq_stride, i
                            const float* row_scale, const float* col_scale, const float* adam_v, int collect_bias,
                            const float* bias_scale, const int32_t* lengths, const int64_t* out_rows, void* out,
                            int64_t out_row_stride, int64_t out_col, int out_dtype, float lo, float hi, void* stream);
+size_t collect_seq_weight_workspace_bytes(int N, int I, int O, int p);
+int collect_seq_weight_impl(const void* a, const void* g, int64_t a_seq_stride, int64_t a_tok_stride,
+                            int64_t g_seq_stride, int64_t g_tok_stride, int N, int S, int I, int O, int p, int dtype,
+                            const float* row_scale, const float* col_scale, const float* adam_v, const void* left,
+                            const void* right, int64_t right_stride, const float* bias_col, const float* bias_scale,
+                            const int32_t* lengths, const int64_t* out_rows, void* out, int64_t out_row_stride,
+                            int64_t out_col, int out_dtype, float lo, float hi, void* ws, size_t ws_bytes,
+                            void* stream);
 size_t project_rows_workspace_bytes(int64_t M, int64_t W, int P, int dtype);
 int project_rows_impl(const void* rows, int64_t M, int64_t W, int64_t row_stride, int dtype, const void* proj, int P,
                       float* acc, int64_t acc_stride, void* ws, size_t ws_bytes, void* stream);
@@ -264,6 +272,25 @@ int bgx_fullgrad_seq_gemm(const void* a_dev, const void* g_dev, int64_t a_seq_st
                                      dtype, row_scale_dev, col_scale_dev, adam_v_dev, collect_bias, bias_scale_dev,
                                      lengths_dev, out_rows_dev, out_dev, out_row_stride, out_col, out_dtype, clamp_lo,
                                      clamp_hi, stream);
+}
+
+size_t bgx_collect_seq_weight_workspace_bytes(int32_t N, int32_t I, int32_t O, int32_t p) {
+  return bgx::collect_seq_weight_workspace_bytes(N, I, O, p);
+}
+
+int bgx_collect_seq_weight(const void* a_dev, const void* g_dev, int64_t a_seq_stride, int64_t a_tok_stride,
+                           int64_t g_seq_stride, int64_t g_tok_stride, int32_t N, int32_t S, int32_t I, int32_t O,
+                           int32_t p, int32_t dtype, const float* row_scale_dev, const float* col_scale_dev,
+                           const float* adam_v_dev, const void* left_dev, const void* right_dev, int64_t right_stride,
+                           const float* bias_col_dev, const float* bias_scale_dev, const int32_t* lengths_dev,
+                           const int64_t* out_rows_dev, void* out_dev, int64_t out_row_stride, int64_t out_col,
+                           int32_t out_dtype, float clamp_lo, float clamp_hi, void* workspace_dev,
+                           size_t workspace_bytes, void* stream) {
+  return bgx::collect_seq_weight_impl(a_dev, g_dev, a_seq_stride, a_tok_stride, g_seq_stride, g_tok_stride, N, S, I, O,
+                                      p, dtype, row_scale_dev, col_scale_dev, adam_v_dev, left_dev, right_dev,
+                                      right_stride, bias_col_dev, bias_scale_dev, lengths_dev, out_rows_dev, out_dev,
+                                      out_row_stride, out_col, out_dtype, clamp_lo, clamp_hi, workspace_dev,
+                                      workspace_bytes, stream);
 }
 
 size_t bgx_project_rows_workspace_bytes(int64_t n_rows, int64_t width, int32_t P, int32_t dtype) {

@@ -11,6 +11,7 @@
 // and writes it straight to the token's row.  Both are bound by the bytes they write.
 
 #include <algorithm>
+#include <type_traits>
 
 #include "common.hpp"
 #include "mma32.hpp"
@@ -151,6 +152,21 @@ struct WgradIn {
   int tiles_i;
 };
 
+// The projected variant (PROJECT): the tile does not leave as weight-shaped values.  Its normalised values, rounded
+// to the model dtype as the reference's are (collector.py:623-634), are projected from both sides inside the
+// workgroup -- Z = L[:, tile's output features] Q_tile R[:, tile's input features]^T, three small MFMA products through
+// LDS -- and the p x p result goes to partial[sequence][tile]; wgrad_project_sum_kernel adds a sequence's tiles in a
+// fixed order, clamps, casts and writes the row.  Nothing of size [N, O, I] is written or read back.
+struct WgradProject {
+  const void* left;    // [p, O]   model dtype
+  const void* right;   // [p, right_stride]: columns 0 .. I - 1
+  const float* bias_col;  // [p] or NULL: the right projection's column for the bias gradient
+  int64_t right_stride;
+  int p;
+  int left_whole, right_whole;  // rows of left / right can be loaded in whole 16-byte pieces
+  float* partial;      // [N][tiles][p * p]
+};
+
 constexpr int WG_BT = 64;            // tile edge
 constexpr int WG_OUT_PITCH = 68;     // floats per row of the staged result tile
 
@@ -184,8 +200,8 @@ __device__ inline uint2 lds_read_tr16(const unsigned char* p) {
   return __builtin_bit_cast(uint2, v);
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void wgrad_seq_kernel(FullArgs a, WgradIn in) {
+template <typename T, bool PROJECT>
+__global__ __launch_bounds__(256) void wgrad_seq_kernel(FullArgs a, WgradIn in, WgradProject pj) {
   using L = WgradTile<T>;
   constexpr int BT = WG_BT, BK = L::BK, VEC = L::VEC, NCH = L::NCH;
   constexpr int CPR = BT / VEC;  // 16-byte pieces per tile row
@@ -286,6 +302,20 @@ __global__ __launch_bounds__(256) void wgrad_seq_kernel(FullArgs a, WgradIn in) 
     load_stage(0);
     store_stage(0);
   }
+  // (projected variant) this lane's fragments of L and R for the tile's four k-steps: asked for now, used behind the
+  // K loop
+  uint4 lf[PROJECT ? BT / 16 : 1], rf[PROJECT ? BT / 16 : 1];
+  if constexpr (PROJECT) {
+    const T* left = (const T*)pj.left;
+    const T* right = (const T*)pj.right;
+#pragma unroll
+    for (int q = 0; q < BT / 16; ++q) {
+      lf[q] = pj.left_whole ? load_chunk<T, true>(left, fr, pj.p, a.O, o0 + q * 16 + 8 * fh, a.O)
+                            : load_chunk<T, false>(left, fr, pj.p, a.O, o0 + q * 16 + 8 * fh, a.O);
+      rf[q] = pj.right_whole ? load_chunk<T, true>(right, fr, pj.p, pj.right_stride, i0 + q * 16 + 8 * fh, a.I)
+                             : load_chunk<T, false>(right, fr, pj.p, pj.right_stride, i0 + q * 16 + 8 * fh, a.I);
+    }
+  }
   __syncthreads();
   for (int kt = 0; kt < KT; ++kt) {
     if (kt + 1 < KT) load_stage(kt + 1);
@@ -294,6 +324,102 @@ __global__ __launch_bounds__(256) void wgrad_seq_kernel(FullArgs a, WgradIn in) 
     __syncthreads();
   }
 
+  if constexpr (PROJECT) {
+    static_assert(!L::F32, "the projected epilogue multiplies on the 16-bit matrix instructions");
+    // LDS: [0, 8 KB) the normalised tile as an operand tile (rows = output features, the contraction index of the
+    // first product); behind it the bias partial sums, the bias values, L b, and the two halves of W
+    constexpr int W_PITCH = 144;  // bytes per row of W: 64 values and 16 bytes against bank conflicts
+    unsigned char* qt = smem;
+    float* red = reinterpret_cast<float*>(smem + L::OPERAND);   // [PARTS][64]
+    float* bvec = red + 256;                                     // [64]
+    float* wb = bvec + 64;                                       // [32]
+    unsigned char* w_hi = reinterpret_cast<unsigned char*>(wb + 32);
+    unsigned char* w_lo = w_hi + 32 * W_PITCH;
+    static_assert(L::OPERAND + (256 + 64 + 32) * 4 + 2 * 32 * W_PITCH <= 2 * L::STAGE, "projected epilogue in LDS");
+    auto to_bits = [](float v) -> uint16_t {
+      return (uint16_t)(std::is_same<T, bf16_t>::value ? f32_to_bf16_bits(v) : f32_to_f16_bits(v));
+    };
+    {
+      const int il = wn * 32 + fr, i = i0 + il;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int ol = wm * 32 + 8 * (e >> 2) + 4 * fh + (e & 3), o = o0 + ol;
+        float v = 0.f;
+        if (o < a.O && i < a.I) v = round_to_dtype(normalise_weight(a, round_to_dtype(acc[e], a.dtype), o, i), a.dtype);
+        *reinterpret_cast<uint16_t*>(qt + L::off(ol, il)) = to_bits(v);
+      }
+    }
+    if (with_bias) red[b_part * BT + b_col] = bias_part;
+    __syncthreads();
+    const T* left = (const T*)pj.left;
+    if (wm == 0) {
+      // W[j', i] = sum_o L[j', o0 + o] Q[o, i] for the wave's 32 input features: A from global memory, B through the
+      // transposing read, as in the K loop
+      f32x16 w;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) w[e] = 0.f;
+      const int rk = 8 * fh + ((lane & 15) >> 2);
+      const int rc = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+#pragma unroll
+      for (int ks = 0; ks < BT; ks += 16) {
+        const uint2 q0 = lds_read_tr16(qt + L::off(ks + rk, wn * 32 + rc));
+        const uint2 q1 = lds_read_tr16(qt + L::off(ks + rk + 4, wn * 32 + rc));
+        Mma32<T>::mma(lf[ks / 16], make_uint4(q0.x, q0.y, q1.x, q1.y), w);
+      }
+      // W = hi + lo in the model dtype: the second product then sees W to twice the dtype's precision
+      const int il = wn * 32 + fr;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int jl = 8 * (e >> 2) + 4 * fh + (e & 3);
+        const uint16_t hb = to_bits(w[e]);
+        const float hf = std::is_same<T, bf16_t>::value ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb);
+        *reinterpret_cast<uint16_t*>(w_hi + jl * W_PITCH + il * 2) = hb;
+        *reinterpret_cast<uint16_t*>(w_lo + jl * W_PITCH + il * 2) = to_bits(w[e] - hf);
+      }
+    } else if (with_bias && wave == 2) {
+      // the tile's bias gradients: summed over the tokens, scaled, rounded to the model dtype
+      float t = 0.f;
+#pragma unroll
+      for (int q = 0; q < PARTS; ++q) t += red[q * BT + lane];
+      const int o = o0 + lane;
+      if (a.bias_scale != nullptr && o < a.O) t *= a.bias_scale[o];
+      bvec[lane] = o < a.O ? round_to_dtype(t, a.dtype) : 0.f;
+    }
+    __syncthreads();
+    f32x16 z;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) z[e] = 0.f;
+    if (wave == 0) {
+      // Z[j', j] = sum_i W[j', i] R[j, i0 + i]
+#pragma unroll
+      for (int ks = 0; ks < BT; ks += 16) {
+        const uint4 hi4 = *reinterpret_cast<const uint4*>(w_hi + fr * W_PITCH + (ks + 8 * fh) * 2);
+        const uint4 lo4 = *reinterpret_cast<const uint4*>(w_lo + fr * W_PITCH + (ks + 8 * fh) * 2);
+        Mma32<T>::mma(hi4, rf[ks / 16], z);
+        Mma32<T>::mma(lo4, rf[ks / 16], z);
+      }
+    } else if (with_bias && wave == 2 && lane < 32) {
+      // (L b)[j'] over the tile's output features
+      float t = 0.f;
+      if (lane < pj.p)
+        for (int o = 0; o < BT && o0 + o < a.O; ++o) t += Elem<T>::load(left + (int64_t)lane * a.O + o0 + o) * bvec[o];
+      wb[lane] = t;
+    }
+    if (with_bias) __syncthreads();
+    if (wave == 0) {
+      const int tiles = (int)gridDim.x;
+      float* dst = pj.partial + ((int64_t)n * tiles + blockIdx.x) * pj.p * pj.p;
+      const int j = fr;
+      float rb = 0.f;
+      if (with_bias && j < pj.p) rb = pj.bias_col[j];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int jl = 8 * (e >> 2) + 4 * fh + (e & 3);
+        if (jl < pj.p && j < pj.p) dst[jl * pj.p + j] = z[e] + (with_bias ? wb[jl] * rb : 0.f);
+      }
+    }
+    return;
+  }
   // ---- epilogue: normalise in place, stage the tile in LDS (the operand stages are done with: the loop ends on a
   // barrier), then every lane stores 8 consecutive values of a row
   const int64_t row = in.out_rows ? in.out_rows[n] : (int64_t)n;
@@ -547,7 +673,146 @@ template <typename T>
 static void launch_wgrad(const FullArgs& fa, WgradIn in, int N, hipStream_t st) {
   in.tiles_i = (fa.I + WG_BT - 1) / WG_BT;
   const unsigned tiles = (unsigned)(((fa.O + WG_BT - 1) / WG_BT) * in.tiles_i);
-  hipLaunchKernelGGL(wgrad_seq_kernel<T>, dim3(tiles, (unsigned)N), dim3(256), 0, st, fa, in);
+  hipLaunchKernelGGL((wgrad_seq_kernel<T, false>), dim3(tiles, (unsigned)N), dim3(256), 0, st, fa, in, WgradProject{});
+}
+
+// Adds a sequence's tiles in two steps, each in an order that depends on the shape alone.  A workgroup takes 64
+// values e and one group of consecutive tiles; four threads per value each add every fourth tile of the group and
+// meet in LDS.  Step 1 (groups > 1): sums[n][group][e] = sum of the group's tiles of partial[n].  Step 2 (one group):
+// out[row(n), out_col + e] = clamp(sum), cast.
+constexpr int WG_SUM_GROUP = 16;  // tiles per group in step 1
+__global__ __launch_bounds__(256) void wgrad_project_sum_kernel(const float* __restrict__ src, int tiles, int pp,
+                                                                int per_group, float* __restrict__ sums,
+                                                                const int64_t* __restrict__ out_rows, void* out,
+                                                                int64_t out_row_stride, int64_t out_col, int out_dtype,
+                                                                float lo, float hi) {
+  __shared__ float red[4][64];
+  const int n = blockIdx.y, grp = blockIdx.z, groups = gridDim.z;
+  const int el = threadIdx.x & 63, q = threadIdx.x >> 6;
+  const int e = blockIdx.x * 64 + el;
+  const int t0 = grp * per_group, t1 = min(tiles, t0 + per_group);
+  float s = 0.f;
+  if (e < pp) {
+    const float* base = src + (int64_t)n * tiles * pp + e;
+    for (int t = t0 + q; t < t1; t += 4) s += base[(int64_t)t * pp];
+  }
+  red[q][el] = s;
+  __syncthreads();
+  if (q != 0 || e >= pp) return;
+  const float total = (red[0][el] + red[1][el]) + (red[2][el] + red[3][el]);
+  if (sums != nullptr) {
+    sums[((int64_t)n * groups + grp) * pp + e] = total;
+  } else {
+    const int64_t row = out_rows ? out_rows[n] : (int64_t)n;
+    store_as(out, row * out_row_stride + out_col + e, clampf(total, lo, hi), out_dtype);
+  }
+}
+
+static int64_t wgrad_sum_groups(int64_t tiles) { return (tiles + WG_SUM_GROUP - 1) / WG_SUM_GROUP; }
+
+size_t collect_seq_weight_workspace_bytes(int N, int I, int O, int p) {
+  if (N <= 0 || I <= 0 || O <= 0 || p <= 0) return 0;
+  const size_t tiles = (size_t)((O + WG_BT - 1) / WG_BT) * (size_t)((I + WG_BT - 1) / WG_BT);
+  // the tiles' contributions, and behind them the sums of groups of tiles
+  return ((size_t)N * (tiles + (size_t)wgrad_sum_groups((int64_t)tiles)) * (size_t)p * p * 4 + 255) / 256 * 256;
+}
+
+// Per-sequence rows of a module whose normaliser acts on the weight-shaped gradient (Adam's second moments, or
+// Adafactor's factors): out[row(n), out_col : + p * p] = clamp(L normalise(g[n]^T a[n] [| bias]) R^T)
+// (collector.py:609-644 with a projection, per sequence).  16-bit models, p <= 32.
+int collect_seq_weight_impl(const void* a, const void* g, int64_t a_seq_stride, int64_t a_tok_stride,
+                            int64_t g_seq_stride, int64_t g_tok_stride, int N, int S, int I, int O, int p, int dtype,
+                            const float* row_scale, const float* col_scale, const float* adam_v, const void* left,
+                            const void* right, int64_t right_stride, const float* bias_col, const float* bias_scale,
+                            const int32_t* lengths, const int64_t* out_rows, void* out, int64_t out_row_stride,
+                            int64_t out_col, int out_dtype, float lo, float hi, void* ws, size_t ws_bytes,
+                            void* stream) {
+  const int collect_bias = bias_col != nullptr;
+  BGX_REQUIRE(a && g && left && right && out, BGX_E_ARG, "collect_seq_weight: null pointer");
+  BGX_REQUIRE(N > 0 && S > 0 && N <= 65535 && I > 0 && O > 0, BGX_E_SHAPE, "collect_seq_weight: N=%d S=%d I=%d O=%d", N,
+              S, I, O);
+  BGX_REQUIRE(p >= 1 && p <= 32, BGX_E_SHAPE, "collect_seq_weight: p=%d outside 1..32", p);
+  BGX_REQUIRE(dtype == BGX_F16 || dtype == BGX_BF16, BGX_E_DTYPE, "collect_seq_weight: dtype=%d (16-bit models only)",
+              dtype);
+  BGX_REQUIRE(dtype_ok(out_dtype), BGX_E_DTYPE, "collect_seq_weight: out_dtype=%d", out_dtype);
+  BGX_REQUIRE(a_tok_stride >= I && g_tok_stride >= O && a_seq_stride >= 0 && g_seq_stride >= 0 &&
+                  right_stride >= I,
+              BGX_E_ARG, "collect_seq_weight: strides a (%lld, %lld) g (%lld, %lld) right %lld", (long long)a_seq_stride,
+              (long long)a_tok_stride, (long long)g_seq_stride, (long long)g_tok_stride, (long long)right_stride);
+  BGX_REQUIRE(adam_v == nullptr || (row_scale == nullptr && col_scale == nullptr), BGX_E_ARG,
+              "collect_seq_weight: Adam moments and Adafactor factors are exclusive");
+  BGX_REQUIRE(out_col >= 0 && out_col + (int64_t)p * p <= out_row_stride, BGX_E_ARG,
+              "collect_seq_weight: columns [%lld, +%d) do not fit a row of %lld", (long long)out_col, p * p,
+              (long long)out_row_stride);
+  const size_t need = collect_seq_weight_workspace_bytes(N, I, O, p);
+  BGX_REQUIRE(ws != nullptr && ((uintptr_t)ws & 255) == 0 && ws_bytes >= need, BGX_E_WORKSPACE,
+              "collect_seq_weight: workspace %zu < %zu bytes (or not 256-byte aligned)", ws_bytes, need);
+  const int64_t n_tiles = (int64_t)((O + WG_BT - 1) / WG_BT) * ((I + WG_BT - 1) / WG_BT);
+  BGX_REQUIRE(n_tiles <= 0x7fffffff, BGX_E_SHAPE, "collect_seq_weight: O=%d I=%d", O, I);
+  FullArgs fa;
+  fa.O = O;
+  fa.I = I;
+  fa.Iw = I + (collect_bias ? 1 : 0);
+  fa.dtype = dtype;
+  fa.row_scale = row_scale;
+  fa.col_scale = col_scale;
+  fa.adam_v = adam_v;
+  fa.bias_scale = bias_scale;
+  fa.out = nullptr;
+  fa.out_row_stride = 0;
+  fa.out_col = 0;
+  fa.out_dtype = out_dtype;
+  fa.lo = lo;
+  fa.hi = hi;
+  WgradIn in;
+  in.act = a;
+  in.g = g;
+  in.a_seq_stride = a_seq_stride;
+  in.a_tok_stride = a_tok_stride;
+  in.g_seq_stride = g_seq_stride;
+  in.g_tok_stride = g_tok_stride;
+  in.S = S;
+  in.lengths = lengths;
+  in.out_rows = nullptr;
+  const int64_t es = 2;
+  auto whole = [&](const void* q, int64_t s0, int64_t s1) {
+    return ((uintptr_t)q % 16 == 0) && (s0 * es) % 16 == 0 && (s1 * es) % 16 == 0;
+  };
+  in.aligned = whole(a, a_seq_stride, a_tok_stride) && whole(g, g_seq_stride, g_tok_stride);
+  in.tiles_i = (I + WG_BT - 1) / WG_BT;
+  WgradProject pj;
+  pj.left = left;
+  pj.right = right;
+  pj.bias_col = bias_col;
+  pj.right_stride = right_stride;
+  pj.p = p;
+  pj.partial = (float*)ws;
+  // whole 16-byte pieces: aligned rows, and a width of whole pieces (a piece never straddles the end of a row)
+  pj.left_whole = (uintptr_t)left % 16 == 0 && O % 8 == 0;
+  pj.right_whole = (uintptr_t)right % 16 == 0 && right_stride % 8 == 0 && I % 8 == 0;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == BGX_F16)
+    hipLaunchKernelGGL((wgrad_seq_kernel<f16_t, true>), dim3((unsigned)n_tiles, (unsigned)N), dim3(256), 0, st, fa, in, pj);
+  else
+    hipLaunchKernelGGL((wgrad_seq_kernel<bf16_t, true>), dim3((unsigned)n_tiles, (unsigned)N), dim3(256), 0, st, fa, in, pj);
+  BGX_HIP(hipGetLastError());
+  const int pp = p * p;
+  const int groups = (int)wgrad_sum_groups(n_tiles);
+  float* sums = (float*)ws + (size_t)N * (size_t)n_tiles * pp;
+  const unsigned ex = (unsigned)((pp + 63) / 64);
+  if (groups > 1) {
+    BGX_REQUIRE(groups <= 65535, BGX_E_SHAPE, "collect_seq_weight: O=%d I=%d", O, I);
+    hipLaunchKernelGGL(wgrad_project_sum_kernel, dim3(ex, (unsigned)N, (unsigned)groups), dim3(256), 0, st,
+                       (const float*)ws, (int)n_tiles, pp, WG_SUM_GROUP, sums, nullptr, nullptr, 0, 0, out_dtype, lo, hi);
+    hipLaunchKernelGGL(wgrad_project_sum_kernel, dim3(ex, (unsigned)N, 1u), dim3(256), 0, st, (const float*)sums, groups,
+                       pp, groups, nullptr, out_rows, out, out_row_stride, out_col, out_dtype, lo, hi);
+  } else {
+    hipLaunchKernelGGL(wgrad_project_sum_kernel, dim3(ex, (unsigned)N, 1u), dim3(256), 0, st, (const float*)ws,
+                       (int)n_tiles, pp, (int)n_tiles, nullptr, out_rows, out, out_row_stride, out_col, out_dtype, lo, hi);
+  }
+  BGX_HIP(hipGetLastError());
+  note_kernel(FAMILY_FULLGRAD, "wgrad_seq_projected");
+  return 0;
 }
 
 int fullgrad_seq_gemm_impl(const void* a, const void* g, int64_t a_seq_stride, int64_t a_tok_stride,

@@ -399,13 +399,14 @@ def collect_adam(prep: AdamPrepared, a: Tensor, g: Tensor, out: Tensor, *, per_t
         raise ValueError("per-token collection needs lengths and row offsets")
     _check_batch_vectors(lengths, rows, N, out.device)
     if not per_token and chunk_tokens == 0:
-        # Two ways to the per-sequence rows.  Normalising the summed gradient costs ~ N * O * I (bound by the
-        # bytes of the [N, O, I] gradient); summing per-token results costs ~ N * S * p * O * I flops on the
-        # fused kernel.  Measured on Pythia-160m shapes the second wins once sequences are shorter than
-        # about 3000 / p tokens (16 x 256 tokens at p = 16: 0.84 against 1.08 ms per layer; 32 x 128: 1.57
-        # against 1.08).
+        # Two ways to the per-sequence rows.  Normalising the summed gradient costs ~ N * S * O * I flops for the
+        # product over the tokens plus a projection per 64 x 64 tile and sequence; summing per-token results costs
+        # ~ N * S * p * O * I flops on the fused kernel, whatever the sequences' length.  Measured per layer of
+        # Pythia-160m shapes on 4096 tokens, first against second: 0.27 / 0.88 ms (4 x 1024, p = 16), 0.44 / 0.83
+        # (16 x 256), 0.64 / 0.82 (32 x 128), 1.08 / 0.82 (64 x 64); at p = 32: 0.74 / 1.63 (32 x 128), 1.33 / 1.66
+        # (64 x 64), 2.56 / 1.66 (128 x 32) -- the second wins once sequences are shorter than about 1500 / p tokens.
         fused_ok = a.dtype != torch.float32 and prep.p <= 32   # the shapes the fused per-token kernels take
-        if not (fused_ok and S * prep.p < 3000):
+        if not (fused_ok and S * prep.p < 1500):
             _collect_adam_seq(prep, a, g, out, lengths, rows, lo, hi)
             return
     nbytes = lib.bgx_collect_adam_workspace_bytes(N, S, I, O, prep.p, dtype_code(prep.dtype),
@@ -504,16 +505,28 @@ def project_rows(rows: Tensor, proj: Tensor, acc: Tensor) -> None:
 
 
 def _collect_adam_seq(prep: AdamPrepared, a: Tensor, g: Tensor, out: Tensor, lengths: Tensor | None,
-                      rows: Tensor | None, lo: float, hi: float) -> None:
+                      rows: Tensor | None, lo: float, hi: float, through_memory: bool = False) -> None:
     """Per-sequence Adam without anything per token: the normalisation is applied to the summed gradient, as
     the reference does (collector.py:634-644):
-        Q[n] = (g[n]^T a[n]) / (sqrt(v) + 1e-8)  [| bias column]     bgx_fullgrad_seq_gemm
-        P[n] = L Q[n] R^T                                            bgx_collect_seq with the output features
-    in the role of tokens: "a" = Q[n] ([O, I(+1)] rows), projected by R; "g" = L^T ([O, p], shared by all n,
-    sequence stride 0) with an identity projection; the token reduction is the sum over output features.
+        Q[n] = (g[n]^T a[n]) / (sqrt(v) + 1e-8)  [| bias column],   P[n] = L Q[n] R^T.
+    16-bit models with p <= 32: one launch forms Q tile by tile and projects every tile where it is
+    (bgx_collect_seq_weight).  Otherwise Q goes through memory: bgx_fullgrad_seq_gemm, then bgx_collect_seq with
+    the output features in the role of tokens -- "a" = Q[n] ([O, I(+1)] rows), projected by R; "g" = L^T ([O, p],
+    shared by all n, sequence stride 0) with an identity projection; the token reduction is the sum over output
+    features.
     """
     N, S, _ = a.shape
     full, r_in, lt, eye = prep.seq_state()
+    if prep.dtype != torch.float32 and prep.p <= 32 and not through_memory:
+        lib = _lib.load()
+        ws = _workspace(out.device, lib.bgx_collect_seq_weight_workspace_bytes(N, prep.I, prep.O, prep.p), "adam_seq")
+        rc = lib.bgx_collect_seq_weight(_ptr(a), _ptr(g), a.stride(0), a.stride(1), g.stride(0), g.stride(1), N, S,
+                                        prep.I, prep.O, prep.p, dtype_code(prep.dtype), None, None, _ptr(full.adam_v),
+                                        _ptr(prep.r_out), _ptr(prep.r_in), prep.r_in.stride(0), _ptr(prep.bias_col),
+                                        _ptr(full.bias_scale), _ptr(lengths), _ptr(rows), _ptr(out), out.stride(0),
+                                        prep.out_col, dtype_code(out.dtype), lo, hi, _ptr(ws), ws.numel(), _stream())
+        _lib.check(rc, "bgx_collect_seq_weight")
+        return
     q = torch.empty((N, full.width), dtype=prep.dtype, device=a.device)
     # positions from len-1 on carry no label: the kernel leaves them out of the sum
     full_gradient(full, a, g, q, per_token=False, lengths=lengths, rows=None, lo=float("-inf"), hi=float("inf"))

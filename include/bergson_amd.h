@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define BGX_ABI_VERSION 11
+#define BGX_ABI_VERSION 12
 
 enum bgx_dtype { BGX_F32 = 0, BGX_F16 = 1, BGX_BF16 = 2 };
 
@@ -303,6 +303,43 @@ int bgx_fullgrad_seq_gemm(const void* a_dev, const void* g_dev,
                           int64_t out_row_stride, int64_t out_col,
                           int32_t out_dtype, float clamp_lo, float clamp_hi,
                           void* stream);
+/* bgx_collect_seq_weight: per-sequence rows of one module whose normaliser acts
+ * on the weight-shaped gradient -- Adam's second moments (adam_v_dev), or
+ * Adafactor's factors -- with a projection:
+ *   out[row(n), out_col : out_col + p*p] =
+ *       clamp(L normalise(g[n]^T a[n] [| bias gradient]) R^T)
+ * i.e. the reference's per-sequence branch of _compute_gradient with an Adam
+ * normaliser (bergson/collector/collector.py:609-644 with
+ * reduce over the tokens; bergson/gradients.py:380-400): `g.mT @ a` over the
+ * tokens s < lengths[n] - 1, rounded to the model dtype, divided by
+ * sqrt(v) + 1e-8, the bias column appended, projected by L = left_dev [p, O]
+ * and R = right_dev [p, right_stride] (columns 0 .. I-1) with bias_col_dev [p]
+ * (fp32, or NULL when the bias is not collected) as the column that multiplies
+ * the bias gradient sum_s g[n, s, :] * bias_scale_dev (NULL = 1).  One launch forms the product over
+ * the tokens on 64 x 64 tiles and projects each tile where it is; nothing
+ * weight-shaped reaches memory.  The tiles' p x p contributions meet in the
+ * workspace (bgx_collect_seq_weight_workspace_bytes, 256-byte aligned) and are
+ * added in a fixed order.  16-bit models (BGX_F16 / BGX_BF16), p <= 32; other
+ * cases go through bgx_fullgrad_seq_gemm and bgx_collect_seq. */
+size_t bgx_collect_seq_weight_workspace_bytes(int32_t N, int32_t I, int32_t O,
+                                              int32_t p);
+int bgx_collect_seq_weight(const void* a_dev, const void* g_dev,
+                           int64_t a_seq_stride, int64_t a_tok_stride,
+                           int64_t g_seq_stride, int64_t g_tok_stride,
+                           int32_t N, int32_t S, int32_t I, int32_t O,
+                           int32_t p, int32_t dtype,
+                           const float* row_scale_dev,
+                           const float* col_scale_dev,
+                           const float* adam_v_dev, const void* left_dev,
+                           const void* right_dev, int64_t right_stride,
+                           const float* bias_col_dev,
+                           const float* bias_scale_dev,
+                           const int32_t* lengths_dev,
+                           const int64_t* out_rows_dev, void* out_dev,
+                           int64_t out_row_stride, int64_t out_col,
+                           int32_t out_dtype, float clamp_lo, float clamp_hi,
+                           void* workspace_dev, size_t workspace_bytes,
+                           void* stream);
 /* The global projection (projection_target = "global",
  * collector.py:364-390: `grad.flatten(1) @ proj.T` per module, summed over
  * the modules): acc_dev[m, j] += sum_k rows_dev[m, k] * proj_dev[j, k] for

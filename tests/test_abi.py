@@ -24,7 +24,7 @@ def test_header_symbols_are_exported_and_bound():
     for n in names:
         assert hasattr(lib, n), f"{n} is declared in the header but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes bindings and header disagree"
-    assert lib.bgx_abi_version() == _lib.ABI_VERSION == 11
+    assert lib.bgx_abi_version() == _lib.ABI_VERSION == 12
 
 
 def test_module_desc_layout_matches_header():
@@ -91,6 +91,12 @@ def test_workspace_sizes():
     assert lib.bgx_scan_workspace_bytes_for(20, 100, 0, 12288, 0) == padded + 2 * (12288 // 16) * 1024
     assert lib.bgx_scan_workspace_bytes_for(33, 100, 0, 12288, 1) == -(-lib.bgx_scan_workspace_bytes(33, 100, 0) // 256) * 256
     assert lib.bgx_scan_workspace_bytes_for(20, 100, 0, 12288 + 32, 1) == padded   # not two k-steps: no table
+    # per-sequence rows through the weight-shaped gradient: p * p fp32 values per sequence and 64 x 64 tile, and
+    # per group of 16 tiles
+    tiles = (3072 // 64) * (768 // 64)
+    assert lib.bgx_collect_seq_weight_workspace_bytes(4, 768, 3072, 16) == 4 * (tiles + tiles // 16) * 256 * 4
+    assert lib.bgx_collect_seq_weight_workspace_bytes(1, 70, 61, 7) == up(1 * (2 * 1 + 1) * 49 * 4)
+    assert lib.bgx_collect_seq_weight_workspace_bytes(0, 64, 64, 16) == 0
 
 
 def test_argument_errors_before_any_launch():
@@ -113,6 +119,14 @@ def test_argument_errors_before_any_launch():
     rc = lib.bgx_scan(C.c_void_p(256), 10, 8, 8, 1, C.c_void_p(256), 2, 1.0, 1, 11, 0, C.c_void_p(256), C.c_void_p(256),
                       None, None, None, None, C.c_void_p(256), 1 << 30, 0, None)
     assert rc == -3 and b"k=11" in lib.bgx_last_error()
+    P = C.c_void_p(256)
+    seq_weight = lambda p, dtype, ws, ws_bytes: lib.bgx_collect_seq_weight(
+        P, P, 64 * 8, 64, 64 * 8, 64, 2, 8, 64, 64, p, dtype, None, None, P, P, P, 64, None, None, None, None, P, 1024,
+        0, 2, 0.0, 0.0, ws, ws_bytes, None)
+    assert seq_weight(33, 2, P, 1 << 20) == -3 and b"p=33" in lib.bgx_last_error()
+    assert seq_weight(16, 0, P, 1 << 20) == -2 and b"16-bit" in lib.bgx_last_error()
+    assert seq_weight(16, 2, P, 16) == -4 and b"workspace" in lib.bgx_last_error()
+    assert seq_weight(16, 2, None, 0) == -4
     rc = lib.bgx_unit_normalize_rows(None, 1, 1, 1, 0, None)
     assert rc == -1
     with pytest.raises(_lib.BergsonAmdError, match="code -1"):

@@ -619,7 +619,8 @@ def _wgrad_reference(a, g, lengths):
 @pytest.mark.parametrize("shape", [
     (3, 37, 24, 40),       # one ragged 64-wide tile, tokens not a multiple of a stage
     (2, 130, 200, 136),    # several 64-wide tiles with ragged edges
-    (3, 96, 1024, 1024),   # 128-wide tiles (64 tiles x 3 sequences)
+    (3, 96, 1024, 1024),   # whole tiles, many of them
+    (8, 70, 700, 650),     # many tiles with ragged edges and rows that are not whole 16-byte pieces
     (1, 70, 70, 61),       # odd widths: pieces of 16 bytes cannot be loaded whole
     (4, 1, 64, 64),        # a single token
 ])
@@ -632,7 +633,7 @@ def test_fullgrad_seq_gemm_against_float64(device, dtype, shape):
     gen = torch.Generator().manual_seed(91)
     a = torch.randn(N, S, I, generator=gen).to(dtype)
     g = (torch.randn(N, S, O, generator=gen) * 0.1).to(dtype)
-    lengths = [S + 1, max(1, S // 2), 1, S][:N]
+    lengths = ([S + 1, max(1, S // 2), 1, S] * 2)[:N]
     want = _wgrad_reference(a, g, lengths).reshape(N, O * I)
     out = torch.full((N + 1, 3 + O * I), 7.0, dtype=torch.float32, device=device)
     rows = torch.tensor(list(range(N, 0, -1)), dtype=torch.int64, device=device)
@@ -756,6 +757,55 @@ def test_fullgrad_tok(device, dtype, kind, bias):
                       rows=torch.tensor(offs, dtype=torch.int64, device=device), lo=lo, hi=hi)
     torch.cuda.synchronize()
     assert rel_l2(out.cpu(), want) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("bias", [False, True])
+@pytest.mark.parametrize("shape", [(3, 150, 192, 256, 16), (4, 70, 200, 330, 32), (2, 130, 77, 61, 7),
+                                   (5, 64, 64, 64, 32), (2, 300, 1024, 520, 16)])
+def test_adam_seq_projected_in_the_tile_kernel(device, dtype, bias, shape):
+    """Per-sequence Adam on 16-bit models: the weight-shaped gradient is formed tile by tile and projected where
+    it is (bgx_collect_seq_weight).  Against the oracle's op sequence, and against the route through memory
+    (bgx_fullgrad_seq_gemm + bgx_collect_seq: the same rounding of the normalised gradient, the projections summed
+    in another order); ragged tiles, odd widths, short and empty sequences, scattered rows, the bias column."""
+    from bergson_amd import _lib, ops
+
+    N, S, I, O, p = shape
+    gen = torch.Generator().manual_seed(77)
+    a = torch.randn(N, S, I, generator=gen).to(dtype)
+    g = (torch.randn(N, S, O, generator=gen) * 0.1).to(dtype)
+    lengths = ([S + 1, max(2, S // 3), 1, S, 2] * 2)[:N]
+    gz = g.clone()
+    for n, l in enumerate(lengths):
+        gz[n, max(l - 1, 0):] = 0
+    left, right = module_projections("layers.1.mlp.dense_h_to_4h", p, O, I, dtype, collect_bias=bias)
+    # second moments bounded away from zero keep the normalised gradient inside fp16's range; in the model dtype
+    # where the bias is collected, as the reference's arithmetic needs there
+    v = torch.rand(O, I, generator=gen) * 1e-3 + 1e-4
+    bsq = (torch.rand(O, generator=gen) * 1e-3 + 1e-4) if bias else None
+    norm = ohooks.Adam(weight_avg_sq=v.to(dtype) if bias else v, bias_avg_sq=None if bsq is None else bsq.to(dtype))
+    want = ohooks.module_gradient(a, gz, norm, left, right, collect_bias=bias)
+    kw = dict(bias_col=right[:, I].to(device), bias_avg_sq=norm.bias_avg_sq.float().to(device)) if bias else {}
+    prep = ops.AdamPrepared(right[:, :I].contiguous().to(device), left.to(device),
+                            norm.weight_avg_sq.float().to(device), 3, **kw)
+    ldev = torch.tensor(lengths, dtype=torch.int32, device=device)
+    rows = torch.tensor(list(range(N, 0, -1)), dtype=torch.int64, device=device)
+    lo, hi = torch.finfo(dtype).min, torch.finfo(dtype).max
+    outs = []
+    for through_memory in (False, True):
+        out = torch.full((N + 1, 3 + p * p + 2), 5.0, dtype=dtype, device=device)
+        ops._collect_adam_seq(prep, a.to(device), g.to(device), out, ldev, rows, lo, hi, through_memory=through_memory)
+        torch.cuda.synchronize()
+        if not through_memory:
+            assert _lib.last_kernel(_lib.FAMILY_FULLGRAD) == "wgrad_seq_projected"
+        outs.append(out.cpu())
+    got = outs[0]
+    assert bool((got[0] == 5).all()) and bool((got[:, :3] == 5).all()) and bool((got[:, 3 + p * p:] == 5).all())
+    block = got[list(range(N, 0, -1)), 3:3 + p * p].float()
+    assert rel_l2(block, want.float()) <= TOL[dtype]
+    assert rel_l2(block, outs[1][list(range(N, 0, -1)), 3:3 + p * p].float()) <= TOL[dtype] / 2
+    if N >= 3:
+        assert block[2].abs().sum() == 0  # the sequence of length 1 has no labelled token
 
 
 def test_adam_seq_with_lengths_and_rows(device):
