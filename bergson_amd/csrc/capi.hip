@@ -49,6 +49,7 @@ static const Switches* read_switches() {
   s->scan_direct_off = getenv("BGX_SCAN_DIRECT_OFF") != nullptr;
   s->scan_stream_off = getenv("BGX_SCAN_STREAM_OFF") != nullptr;
   s->scan_wide_off = getenv("BGX_SCAN_WIDE_OFF") != nullptr;
+  s->wgrad_big_off = getenv("BGX_WGRAD_BIG_OFF") != nullptr;
   return s;
 }
 

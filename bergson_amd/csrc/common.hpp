@@ -41,6 +41,7 @@ struct Switches {
   bool scan_direct_off = false;   // BGX_SCAN_DIRECT_OFF set
   bool scan_stream_off = false;   // BGX_SCAN_STREAM_OFF set
   bool scan_wide_off = false;     // BGX_SCAN_WIDE_OFF set
+  bool wgrad_big_off = false;     // BGX_WGRAD_BIG_OFF set: per-sequence weight gradients on 64 x 64 tiles only
 };
 const Switches& switches();
 

@@ -167,27 +167,33 @@ struct WgradProject {
   float* partial;      // [N][tiles][p * p]
 };
 
-constexpr int WG_BT = 64;            // tile edge
-constexpr int WG_OUT_PITCH = 68;     // floats per row of the staged result tile
+constexpr int WG_OUT_PITCH_PAD = 4;  // floats added to a row of the staged result tile
 
-template <typename T>
+// TB: 32 x 32 blocks per wave and side -- the tile is 64 TB square on 2 x 2 waves.
+template <typename T, int TB>
 struct WgradTile {
   static constexpr bool F32 = sizeof(T) == 4;
+  static constexpr int BT = 64 * TB;                     // tile edge
   static constexpr int BK = F32 ? 32 : 64;               // tokens per stage
   static constexpr int VEC = 16 / (int)sizeof(T);        // elements per 16-byte piece
-  static constexpr int PITCH = WG_BT * (int)sizeof(T);   // bytes per token row of a tile
-  static constexpr int OPERAND = BK * PITCH;             // 8 KB
+  static constexpr int PITCH = BT * (int)sizeof(T);      // bytes per token row of a tile
+  static constexpr int OPERAND = BK * PITCH;             // 8 KB (TB = 1), 16 KB (TB = 2)
   static constexpr int STAGE = 2 * OPERAND;              // g tile, then a tile
-  static constexpr int NCH = BK * (WG_BT / VEC) / 256;   // 16-byte pieces per thread, operand and stage
-  // byte offset of element (token k, feature c) inside an operand tile.  16-bit: the two 64-byte halves of a row
-  // swap on every second pair of token rows, so that the four rows a transposing read touches fall into different
-  // banks; fp32: odd token rows are shifted by half the banks, for the two rows a K = 2 operand reads.
+  static constexpr int NCH = BK * (BT / VEC) / 256;      // 16-byte pieces per thread, operand and stage
+  static constexpr int OUT_PITCH = BT + WG_OUT_PITCH_PAD;
+  // byte offset of element (token k, feature c) inside an operand tile.  16-bit: a transposing read of half a
+  // wave touches 64 bytes of each of four consecutive token rows, which must fall into different banks: with
+  // 128-byte rows (TB = 1) consecutive rows are half the banks apart already and the two 64-byte halves of a row
+  // swap on every second pair of rows; with 256-byte rows (TB = 2) every row starts at bank 0 and the four 64-byte
+  // units of row k are permuted by k mod 4.  fp32: odd token rows are shifted by half the banks, for the two rows a
+  // K = 2 operand reads.
   __device__ static int off(int k, int c) {
     if constexpr (F32) {
       return k * PITCH + ((c ^ ((k & 1) << 5)) << 2);
     } else {
       const int b = c * 2;
-      return k * PITCH + (((b >> 6) ^ ((k >> 1) & 1)) << 6) + (b & 63);
+      const int perm = TB == 1 ? ((k >> 1) & 1) : (k & 3);
+      return k * PITCH + (((b >> 6) ^ perm) << 6) + (b & 63);
     }
   }
 };
@@ -200,12 +206,22 @@ __device__ inline uint2 lds_read_tr16(const unsigned char* p) {
   return __builtin_bit_cast(uint2, v);
 }
 
-template <typename T, bool PROJECT>
-__global__ __launch_bounds__(256) void wgrad_seq_kernel(FullArgs a, WgradIn in, WgradProject pj) {
-  using L = WgradTile<T>;
-  constexpr int BT = WG_BT, BK = L::BK, VEC = L::VEC, NCH = L::NCH;
+// Two tile sizes.  A 64 x 64 tile (one 32 x 32 block per wave) asks the L2s for 16 KB per 0.52 MFLOP, and on
+// Pythia-sized modules that is what bounds it (~300 TFLOP/s at ~10 TB/s from the L2s); 128 x 128 (2 x 2 blocks per
+// wave) asks for half as much per flop and half as much of LDS per MFMA.  The small tile keeps the few-sequence
+// batches of small modules spread over the chip.
+// WHOLE: both operands can be loaded in whole 16-byte pieces (aligned rows, widths of whole pieces).  The loads are
+// then unconditional -- a piece past the end of the sequence or of the row is fetched from a clamped address and
+// zeroed afterwards -- so that the compiler sees straight-line code and lets the two register sets' loads stay in
+// flight past each other (around conditional loads it waits for all of them).
+template <typename T, int TB, bool PROJECT, bool WHOLE>
+__global__ __launch_bounds__(256, 2) void wgrad_seq_kernel(FullArgs a, WgradIn in, WgradProject pj) {
+  using L = WgradTile<T, TB>;
+  constexpr int BT = L::BT, BK = L::BK, VEC = L::VEC, NCH = L::NCH, OUT_PITCH = L::OUT_PITCH;
   constexpr int CPR = BT / VEC;  // 16-byte pieces per tile row
-  static_assert(2 * L::STAGE >= BT * WG_OUT_PITCH * 4, "the staged result tile reuses the operand stages");
+  constexpr int WT = 32 * TB;    // rows / columns of a wave's part of the tile
+  // the result leaves through LDS 64 rows at a time (block row i of the two wave rows), the bias partial sums behind
+  static_assert(2 * L::STAGE >= (64 * OUT_PITCH + 256) * 4, "the staged result rows reuse the operand stages");
   __shared__ __align__(16) unsigned char smem[2 * L::STAGE];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -222,13 +238,33 @@ __global__ __launch_bounds__(256) void wgrad_seq_kernel(FullArgs a, WgradIn in, 
   const T* ap = (const T*)in.act + (int64_t)n * in.a_seq_stride;
 
   // ---- loader: piece c of a stage is 16 bytes of token row c / CPR
-  uint4 gv[NCH], av[NCH];
-  auto fetch = [&](const T* base, int64_t tok_stride, int width, int col0, int kt, int j) -> uint4 {
+  // two register sets: a stage is asked for three iterations before it is computed on and written to LDS two
+  // iterations later, so that its loads have two iterations' time to arrive
+  uint4 gv[2][NCH], av[2][NCH];
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
+  // what does not change from stage to stage is worked out once per thread: piece j is token row p_row[j] of a
+  // stage, its columns start at p_gcol[j] / p_acol[j] (clamped into the row for the unconditional loads of WHOLE)
+  int p_row[NCH], p_gcol[NCH], p_acol[NCH], p_lds[NCH];
+  bool p_gok[NCH], p_aok[NCH];
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
     const int c = tid + 256 * j;
-    const int k = c / CPR, col = col0 + (c % CPR) * VEC;
-    const int s = kt * BK + k;
+    p_row[j] = c / CPR;
+    const int col = (c % CPR) * VEC;
+    p_gok[j] = o0 + col < a.O;
+    p_aok[j] = i0 + col < a.I;
+    p_gcol[j] = WHOLE ? min(o0 + col, a.O - VEC) : o0 + col;
+    p_acol[j] = WHOLE ? min(i0 + col, a.I - VEC) : i0 + col;
+    p_lds[j] = L::off(c / CPR, col);
+  }
+  auto fetch = [&](const T* base, int64_t tok_stride, int width, int col, bool col_ok, int s) -> uint4 {
     uint4 v = make_uint4(0u, 0u, 0u, 0u);
-    if (s < Sn && col < width) {
+    if constexpr (WHOLE) {
+      // (what lies outside is zeroed when the piece is written to LDS, not here: touching the value now would
+      // mean waiting for it now)
+      v = load16_global(base + (int64_t)min(s, Sn - 1) * tok_stride + col);
+    } else if (s < Sn && col_ok) {
       const T* src = base + (int64_t)s * tok_stride + col;
       if (in.aligned && col + VEC <= width) {
         v = load16_global(src);
@@ -243,53 +279,93 @@ __global__ __launch_bounds__(256) void wgrad_seq_kernel(FullArgs a, WgradIn in, 
     }
     return v;
   };
-  auto load_stage = [&](int kt) {
+  int set_kt[2] = {0, 0};  // the stage each register set holds
+  auto load_stage = [&](int kt, auto set_tag) {
+    constexpr int SET = decltype(set_tag)::value;
+    set_kt[SET] = kt;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
-      gv[j] = fetch(gp, in.g_tok_stride, a.O, o0, kt, j);
-      av[j] = fetch(ap, in.a_tok_stride, a.I, i0, kt, j);
+      const int sj = kt * BK + p_row[j];
+      gv[SET][j] = fetch(gp, in.g_tok_stride, a.O, p_gcol[j], p_gok[j], sj);
+      av[SET][j] = fetch(ap, in.a_tok_stride, a.I, p_acol[j], p_aok[j], sj);
     }
   };
-  auto store_stage = [&](int st) {
+  auto store_stage = [&](int st, auto set_tag) {
+    constexpr int SET = decltype(set_tag)::value;
     unsigned char* base = smem + st * L::STAGE;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
-      const int c = tid + 256 * j;
-      const int off = L::off(c / CPR, (c % CPR) * VEC);
-      *reinterpret_cast<uint4*>(base + off) = gv[j];
-      *reinterpret_cast<uint4*>(base + L::OPERAND + off) = av[j];
+      uint4 gw = gv[SET][j], aw = av[SET][j];
+      if constexpr (WHOLE) {
+        const bool row_ok = set_kt[SET] * BK + p_row[j] < Sn;
+        const bool g_ok = row_ok && p_gok[j], a_ok = row_ok && p_aok[j];
+        gw = make_uint4(g_ok ? gw.x : 0u, g_ok ? gw.y : 0u, g_ok ? gw.z : 0u, g_ok ? gw.w : 0u);
+        aw = make_uint4(a_ok ? aw.x : 0u, a_ok ? aw.y : 0u, a_ok ? aw.z : 0u, a_ok ? aw.w : 0u);
+      }
+      *reinterpret_cast<uint4*>(base + p_lds[j]) = gw;
+      *reinterpret_cast<uint4*>(base + L::OPERAND + p_lds[j]) = aw;
     }
   };
 
-  f32x16 acc;
+  f32x16 acc[TB][TB];
 #pragma unroll
-  for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+  for (int i = 0; i < TB; ++i)
+#pragma unroll
+    for (int j = 0; j < TB; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
   float bias_part = 0.f;
   constexpr int PARTS = 256 / BT;  // threads per output feature for the bias sum
   const int b_col = tid % BT, b_part = tid / BT;
 
+  // place of this lane's transposing reads: token (lane % 16) / 4 of its K = 4 group, features 4 (lane % 4) .. + 3 of
+  // the 16 its group of lanes covers
+  const int rk = 8 * fh + ((lane & 15) >> 2);
+  const int rc = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  int g_rd[TB], a_rd[TB];
+#pragma unroll
+  for (int i = 0; i < TB; ++i) {
+    g_rd[i] = L::off(rk, wm * WT + i * 32 + rc);
+    a_rd[i] = L::off(rk, wn * WT + i * 32 + rc);
+  }
   auto compute = [&](int st) {
     const unsigned char* gt = smem + st * L::STAGE;
     const unsigned char* at = gt + L::OPERAND;
     if constexpr (L::F32) {
 #pragma unroll
       for (int kk = 0; kk < BK; kk += 2) {
-        const float af = *reinterpret_cast<const float*>(gt + L::off(kk + fh, wm * 32 + fr));
-        const float bf = *reinterpret_cast<const float*>(at + L::off(kk + fh, wn * 32 + fr));
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af, bf, acc, 0, 0, 0);
+        float gf[TB], af[TB];
+#pragma unroll
+        for (int i = 0; i < TB; ++i) gf[i] = *reinterpret_cast<const float*>(gt + L::off(kk + fh, wm * WT + i * 32 + fr));
+#pragma unroll
+        for (int j = 0; j < TB; ++j) af[j] = *reinterpret_cast<const float*>(at + L::off(kk + fh, wn * WT + j * 32 + fr));
+#pragma unroll
+        for (int i = 0; i < TB; ++i)
+#pragma unroll
+          for (int j = 0; j < TB; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(gf[i], af[j], acc[i][j], 0, 0, 0);
       }
     } else {
-      // place of this lane's read: token (lane % 16) / 4 of its K = 4 group, features 4 (lane % 4) .. + 3 of the 16
-      // its group of lanes covers
-      const int rk = 8 * fh + ((lane & 15) >> 2);
-      const int rc = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+      // (token rows ks + rk and ks + rk + 4 of a k-step permute their 64-byte units like row rk does, whatever ks:
+      // a read's address is the lane's address in row rk plus a constant)
 #pragma unroll
       for (int ks = 0; ks < BK; ks += 16) {
-        const uint2 g0 = lds_read_tr16(gt + L::off(ks + rk, wm * 32 + rc));
-        const uint2 g1 = lds_read_tr16(gt + L::off(ks + rk + 4, wm * 32 + rc));
-        const uint2 a0 = lds_read_tr16(at + L::off(ks + rk, wn * 32 + rc));
-        const uint2 a1 = lds_read_tr16(at + L::off(ks + rk + 4, wn * 32 + rc));
-        Mma32<T>::mma(make_uint4(g0.x, g0.y, g1.x, g1.y), make_uint4(a0.x, a0.y, a1.x, a1.y), acc);
+        uint4 gf[TB], af[TB];
+#pragma unroll
+        for (int i = 0; i < TB; ++i) {
+          const uint2 g0 = lds_read_tr16(gt + g_rd[i] + ks * L::PITCH);
+          const uint2 g1 = lds_read_tr16(gt + g_rd[i] + (ks + 4) * L::PITCH);
+          gf[i] = make_uint4(g0.x, g0.y, g1.x, g1.y);
+        }
+#pragma unroll
+        for (int j = 0; j < TB; ++j) {
+          const uint2 a0 = lds_read_tr16(at + a_rd[j] + ks * L::PITCH);
+          const uint2 a1 = lds_read_tr16(at + a_rd[j] + (ks + 4) * L::PITCH);
+          af[j] = make_uint4(a0.x, a0.y, a1.x, a1.y);
+        }
+#pragma unroll
+        for (int i = 0; i < TB; ++i)
+#pragma unroll
+          for (int j = 0; j < TB; ++j) Mma32<T>::mma(gf[i], af[j], acc[i][j]);
       }
     }
     if (with_bias) {
@@ -299,17 +375,20 @@ __global__ __launch_bounds__(256) void wgrad_seq_kernel(FullArgs a, WgradIn in, 
   };
 
   if (KT > 0) {
-    load_stage(0);
-    store_stage(0);
+    load_stage(0, Set0{});
+    store_stage(0, Set0{});
   }
-  // (projected variant) this lane's fragments of L and R for the tile's four k-steps: asked for now, used behind the
-  // K loop
-  uint4 lf[PROJECT ? BT / 16 : 1], rf[PROJECT ? BT / 16 : 1];
+  if (WHOLE ? KT > 0 : KT > 1) load_stage(1, Set0{});
+  if (WHOLE ? KT > 0 : KT > 2) load_stage(2, Set1{});
+  // (projected variant) this lane's fragments of L and R for the tile's k-steps: asked for now, used behind the K
+  // loop
+  constexpr int KSTEPS = BT / 16;
+  uint4 lf[PROJECT ? KSTEPS : 1], rf[PROJECT ? KSTEPS : 1];
   if constexpr (PROJECT) {
     const T* left = (const T*)pj.left;
     const T* right = (const T*)pj.right;
 #pragma unroll
-    for (int q = 0; q < BT / 16; ++q) {
+    for (int q = 0; q < KSTEPS; ++q) {
       lf[q] = pj.left_whole ? load_chunk<T, true>(left, fr, pj.p, a.O, o0 + q * 16 + 8 * fh, a.O)
                             : load_chunk<T, false>(left, fr, pj.p, a.O, o0 + q * 16 + 8 * fh, a.O);
       rf[q] = pj.right_whole ? load_chunk<T, true>(right, fr, pj.p, pj.right_stride, i0 + q * 16 + 8 * fh, a.I)
@@ -317,73 +396,111 @@ __global__ __launch_bounds__(256) void wgrad_seq_kernel(FullArgs a, WgradIn in, 
     }
   }
   __syncthreads();
-  for (int kt = 0; kt < KT; ++kt) {
-    if (kt + 1 < KT) load_stage(kt + 1);
-    compute(kt & 1);
-    if (kt + 1 < KT) store_stage((kt + 1) & 1);
-    __syncthreads();
+  // iteration kt: stage kt + 1 (asked for two iterations ago) goes to the LDS stage that iteration kt - 1 read, its
+  // register set takes stage kt + 3, then the MFMAs of stage kt
+  if constexpr (WHOLE) {
+    // no branch inside: a stage past the end of the sequence is fetched from its last row and written as zeros (so
+    // that an odd number of stages runs as the next even one), and the compiler can count the loads in flight
+    for (int kt = 0; kt < KT; kt += 2) {
+      store_stage(1, Set0{});
+      load_stage(kt + 3, Set0{});
+      compute(0);
+      __syncthreads();
+      store_stage(0, Set1{});
+      load_stage(kt + 4, Set1{});
+      compute(1);
+      __syncthreads();
+    }
+  } else {
+    for (int kt = 0; kt < KT; kt += 2) {
+      if (kt + 1 < KT) store_stage(1, Set0{});
+      if (kt + 3 < KT) load_stage(kt + 3, Set0{});
+      compute(0);
+      __syncthreads();
+      if (kt + 1 < KT) {
+        if (kt + 2 < KT) store_stage(0, Set1{});
+        if (kt + 4 < KT) load_stage(kt + 4, Set1{});
+        compute(1);
+        __syncthreads();
+      }
+    }
   }
 
   if constexpr (PROJECT) {
     static_assert(!L::F32, "the projected epilogue multiplies on the 16-bit matrix instructions");
-    // LDS: [0, 8 KB) the normalised tile as an operand tile (rows = output features, the contraction index of the
-    // first product); behind it the bias partial sums, the bias values, L b, and the two halves of W
-    constexpr int W_PITCH = 144;  // bytes per row of W: 64 values and 16 bytes against bank conflicts
+    // LDS: the normalised tile, transposed -- Qt[i][o], rows of BT output features: a lane of the K loop's
+    // accumulators holds one input feature and runs of four consecutive output features, which are one 8-byte write
+    // each this way round, and the first product's operand (32 input features x 16 output features per k-step) is a
+    // plain 16-byte read; behind it the bias partial sums, the bias values, L b, and the two halves of W[j'][i]
+    constexpr int Q_PITCH = BT * 2 + 16;  // bytes per row: BT values and 16 bytes against bank conflicts
+    constexpr int QT_BYTES = BT * Q_PITCH;
     unsigned char* qt = smem;
-    float* red = reinterpret_cast<float*>(smem + L::OPERAND);   // [PARTS][64]
-    float* bvec = red + 256;                                     // [64]
-    float* wb = bvec + 64;                                       // [32]
+    float* red = reinterpret_cast<float*>(smem + QT_BYTES);  // [PARTS][BT]
+    float* bvec = red + 256;                                  // [BT]
+    float* wb = bvec + BT;                                    // [32]
     unsigned char* w_hi = reinterpret_cast<unsigned char*>(wb + 32);
-    unsigned char* w_lo = w_hi + 32 * W_PITCH;
-    static_assert(L::OPERAND + (256 + 64 + 32) * 4 + 2 * 32 * W_PITCH <= 2 * L::STAGE, "projected epilogue in LDS");
-    auto to_bits = [](float v) -> uint16_t {
-      return (uint16_t)(std::is_same<T, bf16_t>::value ? f32_to_bf16_bits(v) : f32_to_f16_bits(v));
+    unsigned char* w_lo = w_hi + 32 * Q_PITCH;
+    static_assert(QT_BYTES + (256 + BT + 32) * 4 + 2 * 32 * Q_PITCH <= 2 * L::STAGE, "projected epilogue in LDS");
+    auto pack2 = [](float x, float y) -> uint32_t {
+      return std::is_same<T, bf16_t>::value ? f32x2_to_bf16x2_bits(x, y) : f32x2_to_f16x2_bits(x, y);
     };
-    {
-      const int il = wn * 32 + fr, i = i0 + il;
+    auto unpack_lo = [](uint32_t w) -> float {
+      return std::is_same<T, bf16_t>::value ? bf16_bits_to_f32(w & 0xffffu) : f16_bits_to_f32(w & 0xffffu);
+    };
+    auto unpack_hi = [](uint32_t w) -> float {
+      return std::is_same<T, bf16_t>::value ? bf16_bits_to_f32(w >> 16) : f16_bits_to_f32(w >> 16);
+    };
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int ol = wm * 32 + 8 * (e >> 2) + 4 * fh + (e & 3), o = o0 + ol;
-        float v = 0.f;
-        if (o < a.O && i < a.I) v = round_to_dtype(normalise_weight(a, round_to_dtype(acc[e], a.dtype), o, i), a.dtype);
-        *reinterpret_cast<uint16_t*>(qt + L::off(ol, il)) = to_bits(v);
+    for (int i = 0; i < TB; ++i)
+#pragma unroll
+      for (int j = 0; j < TB; ++j) {
+        const int il = wn * WT + j * 32 + fr, ii = i0 + il;
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+          const int ol = wm * WT + i * 32 + 8 * gq + 4 * fh;  // four consecutive output features from here
+          float v[4];
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const int o = o0 + ol + c;
+            v[c] = 0.f;
+            if (o < a.O && ii < a.I)
+              v[c] = round_to_dtype(normalise_weight(a, round_to_dtype(acc[i][j][gq * 4 + c], a.dtype), o, ii), a.dtype);
+          }
+          *reinterpret_cast<uint2*>(qt + il * Q_PITCH + ol * 2) = make_uint2(pack2(v[0], v[1]), pack2(v[2], v[3]));
+        }
       }
-    }
     if (with_bias) red[b_part * BT + b_col] = bias_part;
     __syncthreads();
     const T* left = (const T*)pj.left;
-    if (wm == 0) {
-      // W[j', i] = sum_o L[j', o0 + o] Q[o, i] for the wave's 32 input features: A from global memory, B through the
-      // transposing read, as in the K loop
+    if (wave < 2 * TB) {
+      // Wt[i, j'] = sum_o Qt[i][o] L[j', o0 + o] for the wave's 32 input features
       f32x16 w;
 #pragma unroll
       for (int e = 0; e < 16; ++e) w[e] = 0.f;
-      const int rk = 8 * fh + ((lane & 15) >> 2);
-      const int rc = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+      const unsigned char* q_rd = qt + (wave * 32 + fr) * Q_PITCH + 8 * fh * 2;
 #pragma unroll
-      for (int ks = 0; ks < BT; ks += 16) {
-        const uint2 q0 = lds_read_tr16(qt + L::off(ks + rk, wn * 32 + rc));
-        const uint2 q1 = lds_read_tr16(qt + L::off(ks + rk + 4, wn * 32 + rc));
-        Mma32<T>::mma(lf[ks / 16], make_uint4(q0.x, q0.y, q1.x, q1.y), w);
-      }
-      // W = hi + lo in the model dtype: the second product then sees W to twice the dtype's precision
-      const int il = wn * 32 + fr;
+      for (int ks = 0; ks < BT; ks += 16)
+        Mma32<T>::mma(*reinterpret_cast<const uint4*>(q_rd + ks * 2), lf[ks / 16], w);
+      // W = hi + lo in the model dtype (the second product then sees W to twice the dtype's precision), written as
+      // W[j'][i]: this lane is j' = fr and holds runs of four consecutive input features
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int jl = 8 * (e >> 2) + 4 * fh + (e & 3);
-        const uint16_t hb = to_bits(w[e]);
-        const float hf = std::is_same<T, bf16_t>::value ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb);
-        *reinterpret_cast<uint16_t*>(w_hi + jl * W_PITCH + il * 2) = hb;
-        *reinterpret_cast<uint16_t*>(w_lo + jl * W_PITCH + il * 2) = to_bits(w[e] - hf);
+      for (int gq = 0; gq < 4; ++gq) {
+        const int il = wave * 32 + 8 * gq + 4 * fh;
+        const uint32_t h01 = pack2(w[gq * 4 + 0], w[gq * 4 + 1]), h23 = pack2(w[gq * 4 + 2], w[gq * 4 + 3]);
+        const uint32_t l01 = pack2(w[gq * 4 + 0] - unpack_lo(h01), w[gq * 4 + 1] - unpack_hi(h01));
+        const uint32_t l23 = pack2(w[gq * 4 + 2] - unpack_lo(h23), w[gq * 4 + 3] - unpack_hi(h23));
+        *reinterpret_cast<uint2*>(w_hi + fr * Q_PITCH + il * 2) = make_uint2(h01, h23);
+        *reinterpret_cast<uint2*>(w_lo + fr * Q_PITCH + il * 2) = make_uint2(l01, l23);
       }
-    } else if (with_bias && wave == 2) {
+    }
+    if (with_bias && tid < BT) {
       // the tile's bias gradients: summed over the tokens, scaled, rounded to the model dtype
       float t = 0.f;
 #pragma unroll
-      for (int q = 0; q < PARTS; ++q) t += red[q * BT + lane];
-      const int o = o0 + lane;
+      for (int q = 0; q < PARTS; ++q) t += red[q * BT + tid];
+      const int o = o0 + tid;
       if (a.bias_scale != nullptr && o < a.O) t *= a.bias_scale[o];
-      bvec[lane] = o < a.O ? round_to_dtype(t, a.dtype) : 0.f;
+      bvec[tid] = o < a.O ? round_to_dtype(t, a.dtype) : 0.f;
     }
     __syncthreads();
     f32x16 z;
@@ -393,12 +510,12 @@ __global__ __launch_bounds__(256) void wgrad_seq_kernel(FullArgs a, WgradIn in, 
       // Z[j', j] = sum_i W[j', i] R[j, i0 + i]
 #pragma unroll
       for (int ks = 0; ks < BT; ks += 16) {
-        const uint4 hi4 = *reinterpret_cast<const uint4*>(w_hi + fr * W_PITCH + (ks + 8 * fh) * 2);
-        const uint4 lo4 = *reinterpret_cast<const uint4*>(w_lo + fr * W_PITCH + (ks + 8 * fh) * 2);
+        const uint4 hi4 = *reinterpret_cast<const uint4*>(w_hi + fr * Q_PITCH + (ks + 8 * fh) * 2);
+        const uint4 lo4 = *reinterpret_cast<const uint4*>(w_lo + fr * Q_PITCH + (ks + 8 * fh) * 2);
         Mma32<T>::mma(hi4, rf[ks / 16], z);
         Mma32<T>::mma(lo4, rf[ks / 16], z);
       }
-    } else if (with_bias && wave == 2 && lane < 32) {
+    } else if (with_bias && wave == 1 && lane < 32) {
       // (L b)[j'] over the tile's output features
       float t = 0.f;
       if (lane < pj.p)
@@ -420,64 +537,67 @@ __global__ __launch_bounds__(256) void wgrad_seq_kernel(FullArgs a, WgradIn in, 
     }
     return;
   }
-  // ---- epilogue: normalise in place, stage the tile in LDS (the operand stages are done with: the loop ends on a
-  // barrier), then every lane stores 8 consecutive values of a row
+  // ---- epilogue: normalise in place, stage 64 rows of the tile in LDS at a time (the operand stages are done
+  // with: the loop ends on a barrier) -- block row i of both wave rows -- then every lane stores 8 consecutive
+  // values of a row
   const int64_t row = in.out_rows ? in.out_rows[n] : (int64_t)n;
   const int64_t dst0 = row * a.out_row_stride + a.out_col;
   float* tile = reinterpret_cast<float*>(smem);
-  {
-    // acc[e] = sum for output feature o0 + 32 wm + 8 (e / 4) + 4 fh + e % 4, input feature i0 + 32 wn + fr
-    const int il = wn * 32 + fr, i = i0 + il;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int ol = wm * 32 + 8 * (e >> 2) + 4 * fh + (e & 3), o = o0 + ol;
-      float v = 0.f;
-      if (o < a.O && i < a.I) {
-        v = round_to_dtype(acc[e], a.dtype);
-        v = clampf(round_to_dtype(normalise_weight(a, v, o, i), a.dtype), a.lo, a.hi);
-      }
-      tile[ol * WG_OUT_PITCH + il] = v;
-    }
-  }
-  float bias_total = 0.f;
-  if (with_bias) {
-    // the bias sums take the rows of the tile array behind the tile itself
-    float* red = tile + BT * WG_OUT_PITCH;
-    static_assert(2 * L::STAGE >= (BT * WG_OUT_PITCH + 256) * 4, "room for the bias partial sums");
-    red[b_part * BT + b_col] = bias_part;
-  }
-  __syncthreads();
+  float* red = tile + 64 * OUT_PITCH;  // the bias partial sums, behind the staged rows
+  if (with_bias) red[b_part * BT + b_col] = bias_part;
   const int es = (int)dtype_size(a.out_dtype);
   // rows of the tile start on 16-byte boundaries of the output when the row pitch and the tile's first element do
   const bool rows_aligned = ((uintptr_t)a.out + (uintptr_t)(dst0 + (int64_t)o0 * a.Iw + i0) * es) % 16 == 0 &&
                             ((int64_t)a.Iw * es) % 16 == 0;
 #pragma unroll
-  for (int q = 0; q < 2; ++q) {
-    const int piece = tid + 256 * q;
-    const int ol = piece >> 3, il = (piece & 7) * 8;
-    const int o = o0 + ol, i = i0 + il;
-    if (o >= a.O || i >= a.I) continue;
-    float v[8];
-    const f32x4 lo4 = *reinterpret_cast<const f32x4*>(tile + ol * WG_OUT_PITCH + il);
-    const f32x4 hi4 = *reinterpret_cast<const f32x4*>(tile + ol * WG_OUT_PITCH + il + 4);
-    v[0] = lo4[0], v[1] = lo4[1], v[2] = lo4[2], v[3] = lo4[3];
-    v[4] = hi4[0], v[5] = hi4[1], v[6] = hi4[2], v[7] = hi4[3];
-    const int64_t dst = dst0 + (int64_t)o * a.Iw + i;
-    if (rows_aligned && i + 8 <= a.I) {
-      if (a.out_dtype == BGX_F32)
-        store8_as<BGX_F32>(a.out, dst, v);
-      else if (a.out_dtype == BGX_F16)
-        store8_as<BGX_F16>(a.out, dst, v);
-      else
-        store8_as<BGX_BF16>(a.out, dst, v);
-    } else {
+  for (int i = 0; i < TB; ++i) {
+    if (i > 0) __syncthreads();  // the rows staged before have been stored
+    // acc[i][j][e]: output feature o0 + WT wm + 32 i + 8 (e / 4) + 4 fh + e % 4, input feature i0 + WT wn + 32 j + fr
 #pragma unroll
-      for (int e = 0; e < 8; ++e)
-        if (i + e < a.I) store_as(a.out, dst + e, v[e], a.out_dtype);
+    for (int j = 0; j < TB; ++j) {
+      const int il = wn * WT + j * 32 + fr, ii = i0 + il;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int sl = wm * 32 + 8 * (e >> 2) + 4 * fh + (e & 3);  // staged row
+        const int o = o0 + wm * WT + i * 32 + (sl - wm * 32);
+        float v = 0.f;
+        if (o < a.O && ii < a.I) {
+          v = round_to_dtype(acc[i][j][e], a.dtype);
+          v = clampf(round_to_dtype(normalise_weight(a, v, o, ii), a.dtype), a.lo, a.hi);
+        }
+        tile[sl * OUT_PITCH + il] = v;
+      }
+    }
+    __syncthreads();
+    constexpr int PIECES = 64 * (BT / 8) / 256;  // 8-value pieces per thread
+#pragma unroll
+    for (int q = 0; q < PIECES; ++q) {
+      const int piece = tid + 256 * q;
+      const int sl = piece / (BT / 8), il = (piece % (BT / 8)) * 8;
+      const int o = o0 + (sl >> 5) * WT + i * 32 + (sl & 31), ii = i0 + il;
+      if (o >= a.O || ii >= a.I) continue;
+      float v[8];
+      const f32x4 lo4 = *reinterpret_cast<const f32x4*>(tile + sl * OUT_PITCH + il);
+      const f32x4 hi4 = *reinterpret_cast<const f32x4*>(tile + sl * OUT_PITCH + il + 4);
+      v[0] = lo4[0], v[1] = lo4[1], v[2] = lo4[2], v[3] = lo4[3];
+      v[4] = hi4[0], v[5] = hi4[1], v[6] = hi4[2], v[7] = hi4[3];
+      const int64_t dst = dst0 + (int64_t)o * a.Iw + ii;
+      if (rows_aligned && ii + 8 <= a.I) {
+        if (a.out_dtype == BGX_F32)
+          store8_as<BGX_F32>(a.out, dst, v);
+        else if (a.out_dtype == BGX_F16)
+          store8_as<BGX_F16>(a.out, dst, v);
+        else
+          store8_as<BGX_BF16>(a.out, dst, v);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (ii + e < a.I) store_as(a.out, dst + e, v[e], a.out_dtype);
+      }
     }
   }
   if (with_bias && b_part == 0 && o0 + b_col < a.O) {
-    const float* red = tile + BT * WG_OUT_PITCH;
+    float bias_total = 0.f;
 #pragma unroll
     for (int q = 0; q < PARTS; ++q) bias_total += red[q * BT + b_col];
     const int o = o0 + b_col;
@@ -669,11 +789,35 @@ int fullgrad_seq_impl(const void* P, int N, int O, int I, int dtype, const float
   return 0;
 }
 
-template <typename T>
-static void launch_wgrad(const FullArgs& fa, WgradIn in, int N, hipStream_t st) {
-  in.tiles_i = (fa.I + WG_BT - 1) / WG_BT;
-  const unsigned tiles = (unsigned)(((fa.O + WG_BT - 1) / WG_BT) * in.tiles_i);
-  hipLaunchKernelGGL((wgrad_seq_kernel<T, false>), dim3(tiles, (unsigned)N), dim3(256), 0, st, fa, in, WgradProject{});
+// Tile edge of a launch: 128 for long sequences of modules with enough tiles of that size for two rounds of the chip
+// (two workgroups to a CU).  With fewer the last, partly filled round costs more than the larger tile saves, and
+// with short sequences its longer epilogue does: by the tracer, 4 x 1024 tokens of a 1024 x 4096 module (1024 large
+// tiles) take 110 us against 123 us on the small tiles, of a 768 x 3072 module (576 large tiles, 1.1 rounds) 88 us
+// against 73.
+static int wgrad_tile_edge(int O, int I, int N, int S) {
+  const int64_t big = (int64_t)((O + 127) / 128) * ((I + 127) / 128);
+  return O >= 128 && I >= 128 && S >= 512 && big * N >= 1024 && !switches().wgrad_big_off ? 128 : 64;
+}
+
+template <typename T, bool PROJECT>
+static int64_t launch_wgrad(const FullArgs& fa, WgradIn in, const WgradProject& pj, int N, hipStream_t st) {
+  const int bt = wgrad_tile_edge(fa.O, fa.I, N, in.S);
+  in.tiles_i = (fa.I + bt - 1) / bt;
+  const int64_t tiles = (int64_t)((fa.O + bt - 1) / bt) * in.tiles_i;
+  constexpr int VEC = 16 / (int)sizeof(T);
+  const bool whole = in.aligned && fa.O % VEC == 0 && fa.I % VEC == 0;
+  const dim3 grid((unsigned)tiles, (unsigned)N), block(256);
+  if (bt == 128 && whole)
+    hipLaunchKernelGGL((wgrad_seq_kernel<T, 2, PROJECT, true>), grid, block, 0, st, fa, in, pj);
+  else if (bt == 128)
+    hipLaunchKernelGGL((wgrad_seq_kernel<T, 2, PROJECT, false>), grid, block, 0, st, fa, in, pj);
+  else if (whole)
+    hipLaunchKernelGGL((wgrad_seq_kernel<T, 1, PROJECT, true>), grid, block, 0, st, fa, in, pj);
+  else
+    hipLaunchKernelGGL((wgrad_seq_kernel<T, 1, PROJECT, false>), grid, block, 0, st, fa, in, pj);
+  note_kernel(FAMILY_FULLGRAD, PROJECT ? (bt == 128 ? "wgrad_seq_projected_128" : "wgrad_seq_projected_64")
+                                       : (bt == 128 ? "wgrad_seq_128" : "wgrad_seq_64"));
+  return tiles;
 }
 
 // Adds a sequence's tiles in two steps, each in an order that depends on the shape alone.  A workgroup takes 64
@@ -712,7 +856,8 @@ static int64_t wgrad_sum_groups(int64_t tiles) { return (tiles + WG_SUM_GROUP - 
 
 size_t collect_seq_weight_workspace_bytes(int N, int I, int O, int p) {
   if (N <= 0 || I <= 0 || O <= 0 || p <= 0) return 0;
-  const size_t tiles = (size_t)((O + WG_BT - 1) / WG_BT) * (size_t)((I + WG_BT - 1) / WG_BT);
+  // (sized for 64 x 64 tiles; a launch on 128 x 128 tiles uses a quarter)
+  const size_t tiles = (size_t)((O + 63) / 64) * (size_t)((I + 63) / 64);
   // the tiles' contributions, and behind them the sums of groups of tiles
   return ((size_t)N * (tiles + (size_t)wgrad_sum_groups((int64_t)tiles)) * (size_t)p * p * 4 + 255) / 256 * 256;
 }
@@ -747,8 +892,8 @@ int collect_seq_weight_impl(const void* a, const void* g, int64_t a_seq_stride, 
   const size_t need = collect_seq_weight_workspace_bytes(N, I, O, p);
   BGX_REQUIRE(ws != nullptr && ((uintptr_t)ws & 255) == 0 && ws_bytes >= need, BGX_E_WORKSPACE,
               "collect_seq_weight: workspace %zu < %zu bytes (or not 256-byte aligned)", ws_bytes, need);
-  const int64_t n_tiles = (int64_t)((O + WG_BT - 1) / WG_BT) * ((I + WG_BT - 1) / WG_BT);
-  BGX_REQUIRE(n_tiles <= 0x7fffffff, BGX_E_SHAPE, "collect_seq_weight: O=%d I=%d", O, I);
+  BGX_REQUIRE((int64_t)((O + 63) / 64) * ((I + 63) / 64) <= 0x7fffffff, BGX_E_SHAPE, "collect_seq_weight: O=%d I=%d", O,
+              I);
   FullArgs fa;
   fa.O = O;
   fa.I = I;
@@ -779,7 +924,7 @@ int collect_seq_weight_impl(const void* a, const void* g, int64_t a_seq_stride, 
     return ((uintptr_t)q % 16 == 0) && (s0 * es) % 16 == 0 && (s1 * es) % 16 == 0;
   };
   in.aligned = whole(a, a_seq_stride, a_tok_stride) && whole(g, g_seq_stride, g_tok_stride);
-  in.tiles_i = (I + WG_BT - 1) / WG_BT;
+  in.tiles_i = 0;
   WgradProject pj;
   pj.left = left;
   pj.right = right;
@@ -791,10 +936,8 @@ int collect_seq_weight_impl(const void* a, const void* g, int64_t a_seq_stride, 
   pj.left_whole = (uintptr_t)left % 16 == 0 && O % 8 == 0;
   pj.right_whole = (uintptr_t)right % 16 == 0 && right_stride % 8 == 0 && I % 8 == 0;
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == BGX_F16)
-    hipLaunchKernelGGL((wgrad_seq_kernel<f16_t, true>), dim3((unsigned)n_tiles, (unsigned)N), dim3(256), 0, st, fa, in, pj);
-  else
-    hipLaunchKernelGGL((wgrad_seq_kernel<bf16_t, true>), dim3((unsigned)n_tiles, (unsigned)N), dim3(256), 0, st, fa, in, pj);
+  const int64_t n_tiles = dtype == BGX_F16 ? launch_wgrad<f16_t, true>(fa, in, pj, N, st)
+                                           : launch_wgrad<bf16_t, true>(fa, in, pj, N, st);
   BGX_HIP(hipGetLastError());
   const int pp = p * p;
   const int groups = (int)wgrad_sum_groups(n_tiles);
@@ -811,7 +954,6 @@ int collect_seq_weight_impl(const void* a, const void* g, int64_t a_seq_stride, 
                        (int)n_tiles, pp, (int)n_tiles, nullptr, out_rows, out, out_row_stride, out_col, out_dtype, lo, hi);
   }
   BGX_HIP(hipGetLastError());
-  note_kernel(FAMILY_FULLGRAD, "wgrad_seq_projected");
   return 0;
 }
 
@@ -849,11 +991,11 @@ int fullgrad_seq_gemm_impl(const void* a, const void* g, int64_t a_seq_stride, i
   in.tiles_i = 0;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == BGX_F32)
-    launch_wgrad<float>(fa, in, N, st);
+    launch_wgrad<float, false>(fa, in, WgradProject{}, N, st);
   else if (dtype == BGX_F16)
-    launch_wgrad<f16_t>(fa, in, N, st);
+    launch_wgrad<f16_t, false>(fa, in, WgradProject{}, N, st);
   else
-    launch_wgrad<bf16_t>(fa, in, N, st);
+    launch_wgrad<bf16_t, false>(fa, in, WgradProject{}, N, st);
   BGX_HIP(hipGetLastError());
   return 0;
 }

@@ -619,8 +619,9 @@ def _wgrad_reference(a, g, lengths):
 @pytest.mark.parametrize("shape", [
     (3, 37, 24, 40),       # one ragged 64-wide tile, tokens not a multiple of a stage
     (2, 130, 200, 136),    # several 64-wide tiles with ragged edges
-    (3, 96, 1024, 1024),   # whole tiles, many of them
-    (8, 70, 700, 650),     # many tiles with ragged edges and rows that are not whole 16-byte pieces
+    (3, 96, 1024, 1024),   # whole 64-wide tiles, many of them
+    (16, 520, 1024, 1024), # 128-wide tiles (long sequences, 64 tiles x 16 sequences: two rounds of the chip)
+    (29, 530, 700, 650),   # 128-wide tiles with ragged edges and rows that are not whole 16-byte pieces
     (1, 70, 70, 61),       # odd widths: pieces of 16 bytes cannot be loaded whole
     (4, 1, 64, 64),        # a single token
 ])
@@ -633,7 +634,7 @@ def test_fullgrad_seq_gemm_against_float64(device, dtype, shape):
     gen = torch.Generator().manual_seed(91)
     a = torch.randn(N, S, I, generator=gen).to(dtype)
     g = (torch.randn(N, S, O, generator=gen) * 0.1).to(dtype)
-    lengths = ([S + 1, max(1, S // 2), 1, S] * 2)[:N]
+    lengths = [[S + 1, max(1, S // 2), 1, S][n % 4] for n in range(N)]
     want = _wgrad_reference(a, g, lengths).reshape(N, O * I)
     out = torch.full((N + 1, 3 + O * I), 7.0, dtype=torch.float32, device=device)
     rows = torch.tensor(list(range(N, 0, -1)), dtype=torch.int64, device=device)
@@ -646,6 +647,41 @@ def test_fullgrad_seq_gemm_against_float64(device, dtype, shape):
     assert rel_l2(got[list(range(N, 0, -1)), 3:].double(), want) <= TOL[dtype]
     if N >= 3:
         assert got[N - 2, 3:].abs().sum() == 0  # the sequence of length 1 has no labelled token
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("kind,bias", [(None, False), ("adam", True), ("adafactor", True)])
+def test_fullgrad_seq_gemm_128_tiles_equal_64_tiles_bitwise(device, dtype, kind, bias, monkeypatch):
+    """Modules with enough 128 x 128 tiles to go round take them (wgrad_seq_128); every element is the same
+    sequence of MFMAs over the tokens as on 64 x 64 tiles, the normalisation behind it is the same code: identical
+    bits, ragged edges and short sequences included.  (The bias column is a plain sum over the tokens, added up by
+    four threads per feature on the small tiles and two on the large ones: equal to rounding.)"""
+    from bergson_amd import _lib, ops
+
+    N, S, I, O = 52, 600, 520, 392
+    a, g, norm = _full_case(N, S, I, O, dtype, kind, bias, seed=97)
+    mod = _full_module(device, a, g, norm, bias, 5)
+    a, g = a.to(device), g.to(device)
+    lengths = torch.tensor([S + 1, 77, 1, S, 2, 65, 64, 130, 17, S, S, 533, 100] * 4, dtype=torch.int32, device=device)
+    lo, hi = torch.finfo(dtype).min, torch.finfo(dtype).max
+    outs = {}
+    for tiles in ("wgrad_seq_128", "wgrad_seq_64"):
+        if tiles == "wgrad_seq_64":
+            monkeypatch.setenv("BGX_WGRAD_BIG_OFF", "1")
+            _lib.reload_switches()
+        out = torch.zeros(N, 5 + mod.width, dtype=dtype, device=device)
+        ops.full_gradient(mod, a, g, out, per_token=False, lengths=lengths, rows=None, lo=lo, hi=hi)
+        torch.cuda.synchronize()
+        assert _lib.last_kernel(_lib.FAMILY_FULLGRAD) == tiles
+        outs[tiles] = out
+    monkeypatch.delenv("BGX_WGRAD_BIG_OFF")
+    _lib.reload_switches()
+    Iw = I + int(bias)
+    big, small = (outs[t][:, 5:].reshape(N, O, Iw) for t in ("wgrad_seq_128", "wgrad_seq_64"))
+    assert torch.equal(big[:, :, :I], small[:, :, :I]) and torch.equal(outs["wgrad_seq_128"][:, :5], outs["wgrad_seq_64"][:, :5])
+    if bias:
+        assert rel_l2(big[:, :, I].float().cpu(), small[:, :, I].float().cpu()) <= 1e-6 + TOL[dtype] / 10
+    assert big[0].abs().sum() > 0 and big[2].abs().sum() == 0
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -762,7 +798,8 @@ def test_fullgrad_tok(device, dtype, kind, bias):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("bias", [False, True])
 @pytest.mark.parametrize("shape", [(3, 150, 192, 256, 16), (4, 70, 200, 330, 32), (2, 130, 77, 61, 7),
-                                   (5, 64, 64, 64, 32), (2, 300, 1024, 520, 16)])
+                                   (5, 64, 64, 64, 32), (2, 300, 1024, 520, 16),
+                                   (16, 520, 1024, 1024, 32), (29, 530, 700, 650, 16)])  # the last two: 128 x 128 tiles
 def test_adam_seq_projected_in_the_tile_kernel(device, dtype, bias, shape):
     """Per-sequence Adam on 16-bit models: the weight-shaped gradient is formed tile by tile and projected where
     it is (bgx_collect_seq_weight).  Against the oracle's op sequence, and against the route through memory
@@ -774,7 +811,7 @@ def test_adam_seq_projected_in_the_tile_kernel(device, dtype, bias, shape):
     gen = torch.Generator().manual_seed(77)
     a = torch.randn(N, S, I, generator=gen).to(dtype)
     g = (torch.randn(N, S, O, generator=gen) * 0.1).to(dtype)
-    lengths = ([S + 1, max(2, S // 3), 1, S, 2] * 2)[:N]
+    lengths = [[S + 1, max(2, S // 3), 1, S, 2][n % 5] for n in range(N)]
     gz = g.clone()
     for n, l in enumerate(lengths):
         gz[n, max(l - 1, 0):] = 0
@@ -797,7 +834,8 @@ def test_adam_seq_projected_in_the_tile_kernel(device, dtype, bias, shape):
         ops._collect_adam_seq(prep, a.to(device), g.to(device), out, ldev, rows, lo, hi, through_memory=through_memory)
         torch.cuda.synchronize()
         if not through_memory:
-            assert _lib.last_kernel(_lib.FAMILY_FULLGRAD) == "wgrad_seq_projected"
+            big = -(-O // 128) * -(-I // 128) * N >= 1024 and S >= 512
+            assert _lib.last_kernel(_lib.FAMILY_FULLGRAD) == ("wgrad_seq_projected_128" if big else "wgrad_seq_projected_64")
         outs.append(out.cpu())
     got = outs[0]
     assert bool((got[0] == 5).all()) and bool((got[:, :3] == 5).all()) and bool((got[:, 3 + p * p:] == 5).all())
