@@ -88,7 +88,8 @@ const char* bgx_last_error(void);
  * environment variables force a kernel variant, so that tests can compare the
  * variants (BGX_COLLECT_PERSIST=0, BGX_COLLECT_STAGED=0, BGX_COLLECT_LPT_OFF, BGX_COLLECT_TWO_STEP_OFF,
  * BGX_ADAM_FUSED_OFF, BGX_ADAM_WIDE_OFF, BGX_ADAM_TTX=n, BGX_SCAN_DIRECT_OFF,
- * BGX_SCAN_STREAM_OFF, BGX_SCAN_WIDE_OFF).  The library reads them once, on its first launch;
+ * BGX_SCAN_STREAM_OFF, BGX_SCAN_WIDE_OFF, BGX_WGRAD_BIG_OFF).  The library reads them once, on its
+ * first launch;
  * bgx_reload_switches() reads them again.  Launches that are being issued from
  * other threads at that moment see either the old or the new settings. */
 int bgx_reload_switches(void);
