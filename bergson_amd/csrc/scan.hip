@@ -1036,6 +1036,7 @@ __global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
 constexpr int SS_MTW = 4;                // 16-row blocks per wave
 constexpr int SS_WAVE_ROWS = 16 * SS_MTW;
 constexpr int SS_TILE_ROWS = 4 * SS_WAVE_ROWS;
+constexpr int SS_MAX_QUERIES = 48;       // up to three blocks of 16 queries (a fourth gains nothing over the tiles)
 
 template <typename T>
 __global__ __launch_bounds__(COLLECT_THREADS) void scan_query_fragments_kernel(const T* __restrict__ queries, int Q,
@@ -1635,7 +1636,7 @@ size_t scan_workspace_bytes(int Q, int k, int64_t chunk_rows) {
 // Bytes of the query fragment table of the streaming kernel (1 KB per k-step and block of 16 queries), or 0
 // where that kernel does not apply: more than 32 queries, a row length that is no multiple of two k-steps.
 static size_t query_table_bytes(int Q, int64_t D, int dtype) {
-  if (Q <= 0 || Q > 32) return 0;
+  if (Q <= 0 || Q > SS_MAX_QUERIES) return 0;
   const int kstep = dtype == BGX_F32 ? 16 : 32;
   if (D <= 0 || D % (2 * kstep) != 0) return 0;
   return (size_t)((Q + 15) / 16) * (size_t)(D / kstep) * 1024;
@@ -1651,15 +1652,14 @@ static int launch_stream(const ScanArgs& a, int blocks, const uint4* table, int 
   // stage slots, score blocks (pitch 16 * blocks + 1 floats), row multipliers
   const size_t smem = 4 * Stream<SS_MTW>::BYTES_PER_WAVE +
                       4 * SS_WAVE_ROWS * (size_t)(16 * blocks + 1) * sizeof(float) + 4 * SS_WAVE_ROWS * sizeof(float);
-  if (blocks == 1) {
-    auto kern = scan_stream_kernel<T, 1>;
+  auto go = [&](auto kern) -> int {
     BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(COLLECT_THREADS), smem, st, a, table);
-  } else {
-    auto kern = scan_stream_kernel<T, 2>;
-    BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(COLLECT_THREADS), smem, st, a, table);
-  }
+    return 0;
+  };
+  const int rc = blocks == 1 ? go(scan_stream_kernel<T, 1>) : blocks == 2 ? go(scan_stream_kernel<T, 2>)
+                                                              : go(scan_stream_kernel<T, 3>);
+  if (rc != 0) return rc;
   BGX_HIP(hipGetLastError());
   return 0;
 }

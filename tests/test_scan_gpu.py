@@ -180,16 +180,17 @@ def test_scan_row_mean_alone(device, Q):
 
 
 # ---- few queries over a long store: the streaming kernel ------------------------------------------------
-# At most 32 queries, a row length that is a multiple of two MFMA k-steps and at least two tiles of 256 rows
+# At most 48 queries, a row length that is a multiple of two MFMA k-steps and at least two tiles of 256 rows
 # per compute unit route the scan through the streaming kernel: a first pass of one tile per compute unit
 # without thresholds (one candidate per row, cut down by the select kernel's sample bound), then the rest.
 STREAM_ROWS = 2 * 256 * 256 + 9001  # past the minimum, with a ragged last tile
 
 
 @pytest.mark.parametrize("dtype,D,Q", [(torch.float16, 128, 5), (torch.float16, 320, 32), (torch.bfloat16, 192, 16),
-                                       (torch.bfloat16, 64, 23), (torch.float32, 96, 8), (torch.float32, 32, 32)])
+                                       (torch.bfloat16, 64, 23), (torch.float32, 96, 8), (torch.float32, 32, 32),
+                                       (torch.float16, 128, 33), (torch.bfloat16, 192, 48), (torch.float32, 64, 41)])
 def test_scan_streamed_few_queries(device, dtype, D, Q):
-    from bergson_amd import ops
+    from bergson_amd import _lib, ops
 
     n, k = STREAM_ROWS, 100
     store, queries = make_store(n, D, Q, dtype, seed=D + Q)
@@ -200,6 +201,7 @@ def test_scan_streamed_few_queries(device, dtype, D, Q):
     res = ops.scan(dev_store, dev_q, unit_norm=True, k=k, want_row_max=True, want_row_mean=True, want_scores=True,
                    want_sumsq=True)
     torch.cuda.synchronize()
+    assert _lib.last_kernel(_lib.FAMILY_SCAN) == "scan_stream"
     assert (res.scores.cpu().T - ref).abs().max().item() <= COS_TOL
     assert res.scores[12345].abs().max().item() == 0
     assert (res.row_mean.cpu() - ref.mean(0)).abs().max().item() <= COS_TOL
