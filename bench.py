@@ -26,6 +26,7 @@ One JSON line is printed.  It also carries
                 with unit-norm cosine, top-100 per query and the per-row max; its own cpu_baseline is the
                 reference's search on a slice of the store;
   per_token     configs[1]'s modules with one row per token (attribute_tokens), kernel only;
+  wide_projection  configs[1]'s modules with per-sequence rows at p = 32 and p = 64, kernel only;
   llama8b_layers  configs[4]'s module shapes through a 4-layer Llama-3-8B-shaped model;
   adam_per_token  configs[3]'s hot kernel, and `end_to_end`: the product loop on a Pythia-410m-shaped model over a
                 slice of that configuration, into the real 98 304-wide per-token store;
@@ -468,6 +469,48 @@ def per_token_leg(args, torch, device):
                          "traffic": (read + written) * PER_TOKEN_TRAFFIC_RATIO}}
 
 
+def wide_projection_leg(args, torch, device):
+    """configs[1]'s 48 modules, per-sequence rows at projection dimensions above 16: the streamed collection kernel
+    with two (p = 32) or four (p = 64) blocks of 16 projection columns per k-step, fragments from the table in global
+    memory, 4 x 1024 tokens per launch.  Kernel only, synthetic a / g; the event pair spans the collection kernel,
+    not the table's preparation before it nor the sum of the tiles' partial blocks behind it."""
+    from bergson_amd import _lib, ops
+
+    N, S, d = 4, 1024, 768
+    gen = torch.Generator(device=device).manual_seed(4)
+    rnd = lambda *shape: torch.randn(*shape, generator=gen, device=device)
+    shapes = [(d, 3 * d), (d, d), (d, 4 * d), (4 * d, d)] * 12
+    acts = [(rnd(N, S, I).to(torch.bfloat16), (rnd(N, S, O) * 0.01).to(torch.bfloat16)) for I, O in shapes]
+    lengths = torch.full((N,), S, dtype=torch.int32, device=device)
+    read = N * S * sum(I + O for I, O in shapes) * 2
+    out = {"workload": "configs[1] modules, per-sequence rows at p = 32 and 64: 48 Pythia-160m modules, 4 x 1024 "
+                       "tokens, Adafactor, fp16 rows", "bytes_read": read}
+    reps = 10
+    for p in (32, 64):
+        mods, col = [], 0
+        for (I, O), (a, g) in zip(shapes, acts):
+            rs, cs = ops.adafactor_scales(rnd(O).abs() * 1e-4 + 1e-12, rnd(I).abs() * 1e-4 + 1e-12, torch.bfloat16)
+            mods.append(ops.ModuleInput(a=a, g=g, r_in=(rnd(p, I) / 4).to(torch.bfloat16),
+                                        r_out=(rnd(p, O) / 4).to(torch.bfloat16), out_col=col, col_scale=cs, row_scale=rs))
+            col += p * p
+        rows = torch.zeros(N, col, device=device, dtype=torch.float16)
+        ops.collect_seq(mods, p, rows, lengths=lengths, lo=-6e4, hi=6e4)
+        torch.cuda.synchronize()
+        ops.collect_timing_start(reps)
+        for _ in range(reps):
+            ops.collect_seq(mods, p, rows, lengths=lengths, lo=-6e4, hi=6e4)
+        torch.cuda.synchronize()
+        ms = ops.collect_timing_stop()
+        ms = sum(ms) / len(ms)
+        gbs = read / (ms * 1e-3) / 1e9
+        out[f"p{p}"] = {"ms_per_launch": ms, "kernel": _lib.last_kernel(_lib.FAMILY_COLLECT),
+                        "tokens_per_s_hooks_only": N * S / (ms * 1e-3),
+                        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                     "frac": gbs / HBM_PEAK_GBS, "traffic": None}}
+        del mods, rows
+    return out
+
+
 def llama_leg(args, torch, device):
     """configs[4]'s module shapes through a model: four layers of a Llama-3-8B-shaped decoder (28 hooked modules
     of 4096 x {4096, 1024, 14336}), batches of 2 x 2048 tokens, p = 16, Adafactor, fp16 store.  The roofline entry
@@ -794,6 +837,7 @@ def main():
     torch.cuda.empty_cache()
     scan = None if args.no_scan else scan_leg(args, torch, device)
     per_token = None if args.no_scan else per_token_leg(args, torch, device)
+    wide = None if args.no_scan else wide_projection_leg(args, torch, device)
     llama = None if args.no_scan else llama_leg(args, torch, device)
     adam = None if args.no_scan else adam_leg(args, torch, device)
     config1 = None if args.no_scan or args.kernels_only else config1_leg(args, torch, device)
@@ -852,6 +896,7 @@ def main():
         "gpu_torch_baseline": gpu_torch,
         "store_scan": scan,
         "per_token": per_token,
+        "wide_projection": wide,
         "llama8b_layers": llama,
         "adam_per_token": adam,
         "config1": config1,

@@ -345,7 +345,7 @@ struct PersistArgs {
   int scratch_bytes;        // LDS between the fragments and the staging rings (exchange / per-token tiles)
   int out_vec8;             // per-token rows: every p x p block starts 16-byte aligned and p is 8 or 16
   const uint4* frag;        // RFG: scaled projection fragments of every module in global memory
-  const int64_t* frag_off;  // RFG: [n_modules] first k-step of a module's fragments (r_in's, then r_out's)
+  const int64_t* frag_off;  // RFG: [n_modules] first fragment (1 KB) of a module in the table (r_in's, then r_out's)
   const int32_t* order;     // RFG: the items in the order the workgroups take them (wg_first indexes this list), or null
   float* tokproj;           // per-token rows in two steps: [n_modules][N][S][2][16] a', g' of every token, or null
 };
@@ -396,7 +396,8 @@ __device__ inline int seq_token_limit_uniform(const int32_t* lengths, int n, int
   return lengths ? min(max(load_uniform(lengths + n) - 1, 0), S) : S;
 }
 
-// Fills the global fragment table of the RFG variant: block (m, 0, z) writes the scaled fragments of k-steps
+// Fills the global fragment table of the RFG variant (nblk blocks of 16 projection rows per k-step, those past
+// row p - 1 repeating it): block (m, 0, z) writes the scaled fragments of k-steps
 // [z, z + 1) * FRAG_STEPS_PER_WG of module m's r_in, block (m, 1, z) those of its r_out, in the order
 // stage_projection gives them in LDS.
 constexpr int FRAG_STEPS_PER_WG = 4 * STAGE_B;  // one round of loads per thread
@@ -404,22 +405,29 @@ constexpr int FRAG_STEPS_PER_WG = 4 * STAGE_B;  // one round of loads per thread
 template <typename T>
 __global__ __launch_bounds__(COLLECT_THREADS) void frag_prepare_kernel(const bgx_module_desc* __restrict__ mods,
                                                                        const int64_t* __restrict__ frag_off,
-                                                                       uint4* __restrict__ frag, int p) {
+                                                                       uint4* __restrict__ frag, int p, int nblk) {
   const bgx_module_desc d = mods[blockIdx.x];
   const int ks0 = blockIdx.z * FRAG_STEPS_PER_WG;
   const int K = blockIdx.y == 0 ? d.I : d.O;
   if (ks0 * Mma<T>::KS >= K) return;
   uint4* dst = frag + frag_off[blockIdx.x] * WAVE;
-  if (blockIdx.y == 0)
-    stage_projection<T>((const T*)d.r_in, d.col_scale, d.I, p, dst, threadIdx.x, ks0, ks0 + FRAG_STEPS_PER_WG);
-  else
-    stage_projection<T>((const T*)d.r_out, d.row_scale, d.O, p, dst + (size_t)(d.I / Mma<T>::KS) * WAVE, threadIdx.x,
-                        ks0, ks0 + FRAG_STEPS_PER_WG);
+  for (int blk = 0; blk < nblk; ++blk) {  // blocks of 16 projection rows, interleaved per k-step
+    if (blockIdx.y == 0)
+      stage_projection<T>((const T*)d.r_in, d.col_scale, d.I, p, dst, threadIdx.x, ks0, ks0 + FRAG_STEPS_PER_WG, blk,
+                          nblk, blk * 16);
+    else
+      stage_projection<T>((const T*)d.r_out, d.row_scale, d.O, p, dst + (size_t)(d.I / Mma<T>::KS) * nblk * WAVE,
+                          threadIdx.x, ks0, ks0 + FRAG_STEPS_PER_WG, blk, nblk, blk * 16);
+  }
 }
 
-template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED = false, bool RFG = false>
+// PB = blocks of 16 projection columns (p <= 16 * PB).  More than one only with the fragments in the global table
+// (two projections to 32 columns do not fit LDS at the usual widths) and for per-sequence rows: a tile then gives
+// PB x PB blocks of P.
+template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED = false, bool RFG = false, int PB = 1>
 __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(PersistArgs pa) {
   static_assert(STAGED || !RFG, "the global fragment table is read through the stream's queue");
+  static_assert(PB == 1 || (RFG && !PER_TOKEN), "wider projections: table fragments, per-sequence rows");
   using M = Mma<T>;
   constexpr int WAVE_T = 16 * MTW;      // tokens per wave
   constexpr int TILE_T = 4 * WAVE_T;    // tokens per workgroup
@@ -428,7 +436,7 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
   uint4* rfrag = reinterpret_cast<uint4*>(smem_raw);
   unsigned char* scratch = smem_raw + (size_t)pa.r_steps * WAVE * 16;
   // per-sequence: the P blocks of waves 1..3, double-buffered by tile parity; per-token: a', g' of each wave
-  f32x4 (*pred)[3][WAVE] = reinterpret_cast<f32x4 (*)[3][WAVE]>(scratch);
+  f32x4 (*pred)[3][PB * PB][WAVE] = reinterpret_cast<f32x4 (*)[3][PB * PB][WAVE]>(scratch);
   float (*tok)[2][WAVE_T][LDP] = reinterpret_cast<float (*)[2][WAVE_T][LDP]>(scratch);
 
   const CollectArgs& args = pa.c;
@@ -448,7 +456,7 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
   // STAGED: the register queue of the wave's input stream, and whether it holds the first block of the
   // tile that comes next
   uint4 v[STAGED ? STREAM_Q : 1][2 * MTW];
-  uint4 rq[RFG ? STREAM_Q : 1][2];  // RFG: the fragments that go with v
+  uint4 rq[RFG ? STREAM_Q : 1][2 * PB];  // RFG: the fragments that go with v
   bool primed = false;
   // Two-step per-token rows: a tile leaves 16 * MTW tokens x 32 floats per wave, i.e. 8 * MTW registers per lane.
   // They stay in registers until KEEP_TILES tiles have gathered or the range ends, and go to the workspace then:
@@ -513,7 +521,7 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
     const int nA = d.I / M::KS;
     const uint4* rfA = rfrag;  // fragments of r_in, then of r_out: in LDS, or (RFG) in the global table
     if constexpr (RFG) rfA = pa.frag + load_uniform(pa.frag_off + m) * WAVE;
-    const uint4* rfG = rfA + (size_t)nA * WAVE;
+    const uint4* rfG = rfA + (size_t)nA * PB * WAVE;
     const int64_t t0 = s0 + wave * WAVE_T;
     const T* a0 = (const T*)d.a + (int64_t)n * d.a_seq_stride + t0 * d.a_tok_stride;
     const T* g0 = (const T*)d.g + (int64_t)n * d.g_seq_stride + t0 * d.g_tok_stride;
@@ -523,7 +531,7 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
       if (rows_valid > 0 && !primed) {
         const T* ua[2 * MTW];
         stream_rows<T, MTW>(a0, d.a_tok_stride, rows_valid, lane, ua);
-        stream_prime<T, MTW, RFG>(ua, d.I / (2 * M::KS), rfA, lane, v, rq);
+        stream_prime<T, MTW, RFG, PB>(ua, d.I / (2 * M::KS), rfA, lane, v, rq);
         primed = true;
       }
     }
@@ -539,10 +547,10 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
       __syncthreads();
     }
 
-    f32x4 accA[MTW];
-    f32x4 accG[MTW];
+    f32x4 accA[MTW * PB];  // [mt * PB + pb]
+    f32x4 accG[MTW * PB];
 #pragma unroll
-    for (int mt = 0; mt < MTW; ++mt) {
+    for (int mt = 0; mt < MTW * PB; ++mt) {
       accA[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
       accG[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
@@ -555,7 +563,7 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
         const T* un[RG];
         stream_rows<T, MTW>(a0, d.a_tok_stride, rows_valid, lane, ua);
         stream_rows<T, MTW>(g0, d.g_tok_stride, rows_valid, lane, ug);
-        stream_segment<T, MTW, RFG>(ua, nkpA, ug, nkpG, rfA, rfG, stage, lane, v, rq, accA);
+        stream_segment<T, MTW, RFG, PB>(ua, nkpA, ug, nkpG, rfA, rfG, stage, lane, v, rq, accA);
         // what follows g: the a rows of the next tile of the range, where this wave has tokens in it
         int nkpN = 0;
         const uint4* rfN = rfG;  // RFG: the next tile's r_in fragments (any readable address when none follows)
@@ -581,9 +589,9 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
             if constexpr (RFG) rfN = pa.frag + load_uniform(pa.frag_off + m2) * WAVE;
           }
         }
-        stream_segment<T, MTW, RFG>(ug, nkpG, un, nkpN, rfG, rfN, stage, lane, v, rq, accG);
+        stream_segment<T, MTW, RFG, PB>(ug, nkpG, un, nkpN, rfG, rfN, stage, lane, v, rq, accG);
         primed = nkpN > 0;
-      } else {
+      } else if constexpr (PB == 1) {
         project_tokens_lds<T, MTW, U>(a0, d.a_tok_stride, rows_valid, d.I, rfA, lane, accA);
         project_tokens_lds<T, MTW, U>(g0, d.g_tok_stride, rows_valid, d.O, rfG, lane, accG);
       }
@@ -591,29 +599,49 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
 #pragma unroll
       for (int mt = 0; mt < MTW; ++mt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (mt * 16 + q * 4 + i >= rows_valid) accG[mt][i] = 0.f;
+        for (int pb = 0; pb < PB; ++pb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (mt * 16 + q * 4 + i >= rows_valid) accG[mt * PB + pb][i] = 0.f;
     } else {
       primed = false;
     }
 
     if constexpr (!PER_TOKEN) {
-      // P[i, j] = sum_t g'[t, i] * a'[t, j] over this wave's tokens; lane (c, q) gets P[4q + e][c]
-      f32x4 P = f32x4{0.f, 0.f, 0.f, 0.f};
+      // P[i, j] = sum_t g'[t, i] * a'[t, j] over this wave's tokens, in blocks of 16 x 16; lane (c, q) gets
+      // P[16 ib + 4q + e][16 jb + c] of block (ib, jb)
+      f32x4 P[PB * PB];
 #pragma unroll
-      for (int mt = 0; mt < MTW; ++mt)
+      for (int ib = 0; ib < PB; ++ib)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) P = __builtin_amdgcn_mfma_f32_16x16x4f32(accG[mt][i], accA[mt][i], P, 0, 0, 0);
-      if (wave > 0) pred[parity][wave - 1][lane] = P;
+        for (int jb = 0; jb < PB; ++jb) {
+          f32x4 blk = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int mt = 0; mt < MTW; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              blk = __builtin_amdgcn_mfma_f32_16x16x4f32(accG[mt * PB + ib][i], accA[mt * PB + jb][i], blk, 0, 0, 0);
+          P[ib * PB + jb] = blk;
+        }
+      if (wave > 0) {
+#pragma unroll
+        for (int b = 0; b < PB * PB; ++b) pred[parity][wave - 1][b][lane] = P[b];
+      }
       __syncthreads();
       if (wave == 0) {
-        const f32x4 p1 = pred[parity][0][lane], p2 = pred[parity][1][lane], p3 = pred[parity][2][lane];
         float* dst = args.partials + (((int64_t)m * args.N + n) * args.tiles_per_seq + ts) * pp;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int i = q * 4 + e;
-          if (i < p && c < p) dst[i * p + c] = (P[e] + p1[e]) + (p2[e] + p3[e]);
-        }
+        for (int ib = 0; ib < PB; ++ib)
+#pragma unroll
+          for (int jb = 0; jb < PB; ++jb) {
+            const int b = ib * PB + jb;
+            const f32x4 p1 = pred[parity][0][b][lane], p2 = pred[parity][1][b][lane], p3 = pred[parity][2][b][lane];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int i = ib * 16 + q * 4 + e, j = jb * 16 + c;
+              if (i < p && j < p) dst[i * p + j] = (P[b][e] + p1[e]) + (p2[e] + p3[e]);
+            }
+          }
       }
       parity ^= 1;  // the next tile writes the other buffer, so one barrier per tile is enough
     } else {
@@ -919,10 +947,16 @@ size_t collect_workspace_bytes(int n_modules, int N, int S, int p) {
   return desc_bytes(n_modules) + (size_t)n_modules * N * tiles * p * p * sizeof(float);
 }
 
-// Bytes of the global fragment table for these modules (1 KB per k-step of I + O), or 0 when the table
-// cannot be used: a width that is not a multiple of two k-steps, p > 16, a bias column.
+constexpr int PERSIST_MAX_PB = 4;  // blocks of 16 projection columns the streamed kernel is built for: 1, 2 or 4
+static int table_blocks(int p) {
+  const int pb = (p + 15) / 16;
+  return pb == 3 ? 4 : pb;
+}
+
+// Bytes of the global fragment table for these modules (1 KB per k-step of I + O and block of 16 projection
+// columns), or 0 when the table cannot be used: a width that is not a multiple of two k-steps, p > 32, a bias column.
 static size_t fragment_table_bytes(const bgx_module_desc* mods, int n_modules, int p, int in_dtype) {
-  if (p > 16) return 0;
+  if (p > 16 * PERSIST_MAX_PB) return 0;
   const int kstep = in_dtype == BGX_F32 ? 16 : 32;
   size_t steps = 0;
   for (int m = 0; m < n_modules; ++m) {
@@ -930,7 +964,7 @@ static size_t fragment_table_bytes(const bgx_module_desc* mods, int n_modules, i
       return 0;
     steps += (size_t)(mods[m].I + mods[m].O) / kstep;
   }
-  return steps * 1024;
+  return steps * 1024 * (size_t)table_blocks(p);
 }
 
 // The workspace that also holds the fragment table, for launches whose modules are too wide for LDS.
@@ -1023,9 +1057,9 @@ static int compute_units(int* out) {
   return 0;
 }
 
-template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED, bool RFG>
+template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED, bool RFG, int PB = 1>
 static int launch_persist_one(int wgs, size_t lds, hipStream_t st, const PersistArgs& pa) {
-  auto kern = collect_persist_kernel<T, PER_TOKEN, MTW, U, STAGED, RFG>;
+  auto kern = collect_persist_kernel<T, PER_TOKEN, MTW, U, STAGED, RFG, PB>;
   // the opt-in to more than 64 KB of dynamic LDS is per kernel and per device; do it once for each
   static std::atomic<bool> opted_in[MAX_DEVICES];
   int dev = 0;
@@ -1048,10 +1082,15 @@ static int launch_persist_s(bool per_token, int tile_tokens, int wgs, size_t lds
                    : launch_persist_one<T, false, 1, 8, STAGED, RFG>(wgs, lds, st, pa);
 }
 
-// staged: streamed token rows; rfg: (staged only) projection fragments from the global table
+// staged: streamed token rows; rfg: (staged only) projection fragments from the global table; pb: blocks of 16
+// projection columns (more than one: table fragments and per-sequence rows only, tiles of 128 or 256 tokens)
 template <typename T>
-static int launch_persist(bool staged, bool rfg, bool per_token, int tile_tokens, int wgs, size_t lds, hipStream_t st,
-                          const PersistArgs& pa) {
+static int launch_persist(bool staged, bool rfg, bool per_token, int pb, int tile_tokens, int wgs, size_t lds,
+                          hipStream_t st, const PersistArgs& pa) {
+  if (pb == 2)
+    return tile_tokens == 256 ? launch_persist_one<T, false, 4, 4, true, true, 2>(wgs, lds, st, pa)
+                              : launch_persist_one<T, false, 2, 4, true, true, 2>(wgs, lds, st, pa);
+  if (pb > 2) return launch_persist_one<T, false, 2, 4, true, true, 4>(wgs, lds, st, pa);  // 256 tokens: registers spill
   if (rfg) return launch_persist_s<T, true, true>(per_token, tile_tokens, wgs, lds, st, pa);
   return staged ? launch_persist_s<T, true, false>(per_token, tile_tokens, wgs, lds, st, pa)
                 : launch_persist_s<T, false, false>(per_token, tile_tokens, wgs, lds, st, pa);
@@ -1121,7 +1160,19 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   args.S = S;
   args.p = p;
   const int pb = (p + 15) / 16;
-  const int tile_tokens = tile_tokens_for(pb, aligned, any_bias, S);
+  // Projections wider than 16 columns: per-sequence rows go through the streamed kernel with the fragments in the
+  // global table, when the caller's workspace has room for it, on tiles of 128 or 256 tokens (a wave then loads
+  // as many bytes of fragments as of tokens, or half as many).
+  const size_t frag_bytes = fragment_table_bytes(sorted.data(), n_modules, p, in_dtype);
+  const WorkspaceLayout lay = workspace_layout(need, frag_bytes, n_modules, N, S, p);
+  const bool wide = pb > 1 && pb <= PERSIST_MAX_PB && !per_token && aligned && !any_bias && frag_bytes > 0 &&
+                    ws_bytes >= lay.frag + frag_bytes && switches().collect_staged && switches().collect_persist;
+  int tile_tokens = tile_tokens_for(pb, aligned, any_bias, S);
+  if (wide) {
+    // 256 tokens where the sequence length wastes little of a wave's 64 (measured 209 us against 231 us at p = 32
+    // on 4 x 1024 tokens of 48 modules); with four blocks the registers hold a wave's 32 tokens only
+    tile_tokens = pb == 2 && (int64_t)((S + 63) / 64 * 64) * 100 <= (int64_t)S * 104 ? 256 : 128;
+  }
   args.tiles_per_seq = (S + tile_tokens - 1) / tile_tokens;
   const int64_t tiles = (int64_t)N * args.tiles_per_seq;
   BGX_REQUIRE(tiles <= 0x7fffffffLL, BGX_E_SHAPE, "collect: %lld tiles exceed the grid limit", (long long)tiles);
@@ -1130,12 +1181,16 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   // fit in LDS beside its exchange buffers.
   int r_steps = 0;
   for (int m = 0; m < n_modules; ++m) r_steps = std::max(r_steps, (sorted[m].I + sorted[m].O) / kstep);
-  const size_t scratch_bytes = per_token ? persist_scratch_bytes(tile_tokens) : (size_t)2 * 3 * WAVE * 16;
+  const size_t scratch_bytes =
+      per_token ? persist_scratch_bytes(tile_tokens)
+                : (size_t)2 * 3 * WAVE * 16 * (wide ? table_blocks(p) * table_blocks(p) : 1);
   size_t persist_lds = (size_t)r_steps * 1024 + scratch_bytes;
   bool persist = pb == 1 && aligned && !any_bias && persist_lds <= LDS_PER_WG &&
                  tiles * n_modules <= 0x7fffffffLL;
   // staging rings for fully coalesced loads: every K a multiple of two k-steps, and 32 KB more of LDS
-  const size_t stage_bytes = (size_t)4 * (tile_tokens == 128 ? Stream<2>::BYTES_PER_WAVE : Stream<1>::BYTES_PER_WAVE);
+  const size_t stage_bytes = (size_t)4 * (tile_tokens == 256   ? Stream<4>::BYTES_PER_WAVE
+                                          : tile_tokens == 128 ? Stream<2>::BYTES_PER_WAVE
+                                                               : Stream<1>::BYTES_PER_WAVE);
   bool staged = persist && persist_lds + stage_bytes <= LDS_PER_WG;
   for (int m = 0; m < n_modules && staged; ++m)
     staged = sorted[m].I % (2 * kstep) == 0 && sorted[m].O % (2 * kstep) == 0;
@@ -1143,10 +1198,8 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   if (staged) persist_lds += stage_bytes;
   // Modules too wide for LDS: the streamed kernel with the fragments in a global table, when the caller's
   // workspace has room for it (bgx_collect_workspace_bytes_for) -- else the tile kernel.
-  const size_t frag_bytes = fragment_table_bytes(sorted.data(), n_modules, p, in_dtype);
-  const WorkspaceLayout lay = workspace_layout(need, frag_bytes, n_modules, N, S, p);
   const size_t frag_ws_off = lay.frag;
-  bool rfg = !persist && pb == 1 && aligned && !any_bias && tiles * n_modules <= 0x7fffffffLL && frag_bytes > 0 &&
+  bool rfg = !persist && (pb == 1 || wide) && aligned && !any_bias && tiles * n_modules <= 0x7fffffffLL && frag_bytes > 0 &&
              ws_bytes >= frag_ws_off + frag_bytes;
   rfg = rfg && switches().collect_staged;
   if (rfg) {
@@ -1241,12 +1294,12 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     }
     head.resize(desc_bytes(n_modules), 0);
     memcpy(head.data() + ranges_offset(n_modules), first.data(), first.size() * sizeof(int32_t));
-    if (rfg) {  // where each module's fragments start, in k-steps
+    if (rfg) {  // where each module's fragments start, in fragments of 1 KB
       std::vector<int64_t> foff((size_t)n_modules);
       int64_t steps = 0;
       for (int m = 0; m < n_modules; ++m) {
         foff[m] = steps;
-        steps += (sorted[m].I + sorted[m].O) / kstep;
+        steps += (int64_t)(sorted[m].I + sorted[m].O) / kstep * table_blocks(p);
       }
       memcpy(head.data() + frag_off_offset(n_modules), foff.data(), foff.size() * sizeof(int64_t));
     }
@@ -1263,11 +1316,14 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     for (int m = 0; m < n_modules; ++m) widest = std::max(widest, std::max(sorted[m].I, sorted[m].O) / kstep);
     const dim3 pgrid((unsigned)n_modules, 2, (unsigned)((widest + FRAG_STEPS_PER_WG - 1) / FRAG_STEPS_PER_WG));
     if (in_dtype == BGX_F32)
-      hipLaunchKernelGGL(frag_prepare_kernel<float>, pgrid, dim3(COLLECT_THREADS), 0, st, mods_dev, frag_off_dev, frag_dev, p);
+      hipLaunchKernelGGL(frag_prepare_kernel<float>, pgrid, dim3(COLLECT_THREADS), 0, st, mods_dev, frag_off_dev, frag_dev, p,
+                         table_blocks(p));
     else if (in_dtype == BGX_F16)
-      hipLaunchKernelGGL(frag_prepare_kernel<f16_t>, pgrid, dim3(COLLECT_THREADS), 0, st, mods_dev, frag_off_dev, frag_dev, p);
+      hipLaunchKernelGGL(frag_prepare_kernel<f16_t>, pgrid, dim3(COLLECT_THREADS), 0, st, mods_dev, frag_off_dev, frag_dev, p,
+                         table_blocks(p));
     else
-      hipLaunchKernelGGL(frag_prepare_kernel<bf16_t>, pgrid, dim3(COLLECT_THREADS), 0, st, mods_dev, frag_off_dev, frag_dev, p);
+      hipLaunchKernelGGL(frag_prepare_kernel<bf16_t>, pgrid, dim3(COLLECT_THREADS), 0, st, mods_dev, frag_off_dev, frag_dev, p,
+                         table_blocks(p));
     BGX_HIP(hipGetLastError());
   }
   args.partials = (float*)((char*)ws + desc_bytes(n_modules));
@@ -1304,11 +1360,11 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     pa.tokproj = two_step ? (float*)((char*)ws + lay.tokproj) : nullptr;
     int rc;
     if (in_dtype == BGX_F32)
-      rc = launch_persist<float>(staged, rfg, per_token, tile_tokens, wgs, persist_lds, st, pa);
+      rc = launch_persist<float>(staged, rfg, per_token, pb, tile_tokens, wgs, persist_lds, st, pa);
     else if (in_dtype == BGX_F16)
-      rc = launch_persist<f16_t>(staged, rfg, per_token, tile_tokens, wgs, persist_lds, st, pa);
+      rc = launch_persist<f16_t>(staged, rfg, per_token, pb, tile_tokens, wgs, persist_lds, st, pa);
     else
-      rc = launch_persist<bf16_t>(staged, rfg, per_token, tile_tokens, wgs, persist_lds, st, pa);
+      rc = launch_persist<bf16_t>(staged, rfg, per_token, pb, tile_tokens, wgs, persist_lds, st, pa);
     if (rc != 0) return rc;
     note_kernel(FAMILY_COLLECT, rfg ? "collect_persist_table" : staged ? "collect_persist_lds" : "collect_persist_direct");
   } else if (in_dtype == BGX_F32) {

@@ -15,11 +15,12 @@ constexpr int COLLECT_THREADS = 256;  // the workgroup size these helpers are wr
 constexpr int STAGE_B = 6;            // fragments a thread keeps in flight while staging a projection
 
 // k-steps [ks0, ks1) of the matrix; the whole of it by default.  The fragment of k-step ks goes to
-// dst[(ks * nblk + blk) * 64 + lane]: nblk matrices of 16 rows interleaved per k-step (one by default).
+// dst[(ks * nblk + blk) * 64 + lane]: nblk matrices of 16 rows interleaved per k-step (one by default).  The 16
+// rows are rows row0 .. row0 + 15 of R, those past the last (p - 1) repeating it.
 template <typename T>
 __device__ inline void stage_projection(const T* __restrict__ R, const float* __restrict__ scale, int K, int p,
                                         uint4* __restrict__ dst, int tid, int ks0 = 0, int ks1 = -1, int blk = 0,
-                                        int nblk = 1) {
+                                        int nblk = 1, int row0 = 0) {
   using M = Mma<T>;
   const int nfrag = (ks1 < 0 ? K / M::KS : min(ks1, K / M::KS)) * WAVE;
   constexpr int B = STAGE_B;  // fragments per thread in flight
@@ -32,7 +33,7 @@ __device__ inline void stage_projection(const T* __restrict__ R, const float* __
       const int ks = f >> 6, l = f & 63;
       const int r = l & 15, q = l >> 4;
       const int k0 = ks * M::KS + q * M::EPL;
-      v[b] = load16_global(R + (int64_t)min(r, p - 1) * K + k0);
+      v[b] = load16_global(R + (int64_t)min(row0 + r, p - 1) * K + k0);
       if (scale != nullptr) {
 #pragma unroll
         for (int e = 0; e < M::EPL / 4; ++e) s4[b][e] = load16_global(scale + k0 + 4 * e);

@@ -120,11 +120,13 @@ int bgx_adafactor_scales(const float* row_dev, int32_t O, const float* col_dev,
  * bgx_collect_workspace_bytes is the minimum for any modules of that count.
  * bgx_collect_workspace_bytes_for looks at the modules (only I, O and bias_col
  * of each descriptor are read) and adds room for (i) a table of pre-scaled
- * projection fragments, 32 bytes per input and output feature, and the
- * list of work items behind it (4 bytes per module and 64 tokens): with it,
- * modules too wide for their projections to be kept on chip (Llama-3-8B's
- * 4096 x 14336) still run through the streamed persistent kernel; without it
- * such launches use the one-workgroup-per-tile kernel; (ii) at p = 8 or 16,
+ * projection fragments, 32 bytes per input and output feature (64 for
+ * 16 < p <= 32, 128 for 32 < p <= 64), and the list of work items behind it
+ * (4 bytes per module and 64 tokens): with it, modules too wide for their
+ * projections to be kept on chip (Llama-3-8B's 4096 x 14336) and per-sequence
+ * launches at p > 16 still run through the streamed persistent kernel;
+ * without it such launches use the one-workgroup-per-tile kernel, which is a
+ * third to a half slower; (ii) at p = 8 or 16,
  * the projected activations and output gradients of every token (128 bytes
  * per module and token): with it bgx_collect_tok writes its rows in two steps
  * -- the collection kernel leaves those projections in the workspace and a

@@ -265,6 +265,34 @@ def test_wide_modules(device, dtype, per_token):
     assert rel_l2(got, want) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("p,S", [(32, 512), (32, 300), (20, 257), (64, 500), (50, 130)])
+def test_seq_wide_projections(device, dtype, p, S, kernel_variant):
+    """p > 16: per-sequence rows come from the streamed kernel with two or four blocks of 16 projection columns per
+    k-step (the default variant; tiles of 256 tokens where the sequence length wastes little of them, else of 128),
+    or from the tile kernel (the other two).  Ragged lengths, a projection dimension that is no multiple of 16, a
+    normalizer folded into the fragments, out_rows."""
+    from bergson_amd import _lib
+
+    N = 4
+    lengths = [S, (2 * S) // 3, 65, 2]
+    cases = []
+    for i, (I, O) in enumerate([(256, 768), (64, 64), (384, 128)]):
+        a, g, left, right, norm = make_case(N, S, I, O, p, dtype, seed=70 + i, normalizer="adafactor" if i == 0 else None,
+                                            name=f"layers.{i}.p{p}")
+        if norm is not None:
+            g = g * 1e-3  # keeps every value inside the fp16 range of the store
+        for n, l in enumerate(lengths):
+            g[n, l - 1:] = 0
+        cases.append((a, g, left, right, norm))
+    out_rows = [3, 0, 4, 1]
+    got = run_kernel(device, cases, p, dtype, lengths=lengths, out_rows=out_rows, n_rows=5)
+    assert _lib.last_kernel(_lib.FAMILY_COLLECT) == ("collect_persist_table" if kernel_variant == "streamed" else "collect_tile")
+    want = oracle_rows(cases, dtype)
+    assert rel_l2(got[out_rows], want) <= TOL[dtype]
+    assert got[2].abs().sum() == 0
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("p", [16, 32, 8])
 def test_tok(device, dtype, p):
