@@ -436,7 +436,8 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
   uint4* rfrag = reinterpret_cast<uint4*>(smem_raw);
   unsigned char* scratch = smem_raw + (size_t)pa.r_steps * WAVE * 16;
   // per-sequence: the P blocks of waves 1..3, double-buffered by tile parity; per-token: a', g' of each wave
-  f32x4 (*pred)[3][PB * PB][WAVE] = reinterpret_cast<f32x4 (*)[3][PB * PB][WAVE]>(scratch);
+  f32x4 (*pred)[3][WAVE] = reinterpret_cast<f32x4 (*)[3][WAVE]>(scratch);
+  f32x4 (*pblk)[PB * PB][WAVE] = reinterpret_cast<f32x4 (*)[PB * PB][WAVE]>(scratch);  // PB > 1: [wave][block][lane]
   float (*tok)[2][WAVE_T][LDP] = reinterpret_cast<float (*)[2][WAVE_T][LDP]>(scratch);
 
   const CollectArgs& args = pa.c;
@@ -610,40 +611,53 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
     if constexpr (!PER_TOKEN) {
       // P[i, j] = sum_t g'[t, i] * a'[t, j] over this wave's tokens, in blocks of 16 x 16; lane (c, q) gets
       // P[16 ib + 4q + e][16 jb + c] of block (ib, jb)
-      f32x4 P[PB * PB];
+      float* dst = args.partials + (((int64_t)m * args.N + n) * args.tiles_per_seq + ts) * pp;
+      if constexpr (PB == 1) {
+        f32x4 P = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ib = 0; ib < PB; ++ib)
+        for (int mt = 0; mt < MTW; ++mt)
 #pragma unroll
-        for (int jb = 0; jb < PB; ++jb) {
-          f32x4 blk = f32x4{0.f, 0.f, 0.f, 0.f};
+          for (int i = 0; i < 4; ++i) P = __builtin_amdgcn_mfma_f32_16x16x4f32(accG[mt][i], accA[mt][i], P, 0, 0, 0);
+        if (wave > 0) pred[parity][wave - 1][lane] = P;
+        __syncthreads();
+        if (wave == 0) {
+          const f32x4 p1 = pred[parity][0][lane], p2 = pred[parity][1][lane], p3 = pred[parity][2][lane];
 #pragma unroll
-          for (int mt = 0; mt < MTW; ++mt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              blk = __builtin_amdgcn_mfma_f32_16x16x4f32(accG[mt * PB + ib][i], accA[mt * PB + jb][i], blk, 0, 0, 0);
-          P[ib * PB + jb] = blk;
+          for (int e = 0; e < 4; ++e) {
+            const int i = q * 4 + e;
+            if (i < p && c < p) dst[i * p + c] = (P[e] + p1[e]) + (p2[e] + p3[e]);
+          }
         }
-      if (wave > 0) {
-#pragma unroll
-        for (int b = 0; b < PB * PB; ++b) pred[parity][wave - 1][b][lane] = P[b];
-      }
-      __syncthreads();
-      if (wave == 0) {
-        float* dst = args.partials + (((int64_t)m * args.N + n) * args.tiles_per_seq + ts) * pp;
+        parity ^= 1;  // the next tile writes the other buffer, so one barrier per tile is enough
+      } else {
+        // every wave leaves its PB x PB blocks in LDS as it makes them (none is kept in registers), and the four
+        // waves share the sums: wave w adds up blocks w, w + 4, ...
 #pragma unroll
         for (int ib = 0; ib < PB; ++ib)
 #pragma unroll
           for (int jb = 0; jb < PB; ++jb) {
-            const int b = ib * PB + jb;
-            const f32x4 p1 = pred[parity][0][b][lane], p2 = pred[parity][1][b][lane], p3 = pred[parity][2][b][lane];
+            f32x4 blk = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int i = ib * 16 + q * 4 + e, j = jb * 16 + c;
-              if (i < p && j < p) dst[i * p + j] = (P[b][e] + p1[e]) + (p2[e] + p3[e]);
-            }
+            for (int mt = 0; mt < MTW; ++mt)
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                blk = __builtin_amdgcn_mfma_f32_16x16x4f32(accG[mt * PB + ib][i], accA[mt * PB + jb][i], blk, 0, 0, 0);
+            pblk[wave][ib * PB + jb][lane] = blk;
           }
+        __syncthreads();
+#pragma unroll
+        for (int bb = 0; bb < PB * PB / 4; ++bb) {
+          const int b = bb * 4 + wave;
+          const int ib = b / PB, jb = b - ib * PB;
+          const f32x4 p0 = pblk[0][b][lane], p1 = pblk[1][b][lane], p2 = pblk[2][b][lane], p3 = pblk[3][b][lane];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int i = ib * 16 + q * 4 + e, j = jb * 16 + c;
+            if (i < p && j < p) dst[i * p + j] = (p0[e] + p1[e]) + (p2[e] + p3[e]);
+          }
+        }
+        __syncthreads();  // the next tile's blocks go to the same place
       }
-      parity ^= 1;  // the next tile writes the other buffer, so one barrier per tile is enough
     } else {
       if (pa.tokproj != nullptr) {
         // two-step rows: the wave's a', g' -- 128 bytes per token -- go to the workspace (later: flush_kept), and
@@ -1090,7 +1104,8 @@ static int launch_persist(bool staged, bool rfg, bool per_token, int pb, int til
   if (pb == 2)
     return tile_tokens == 256 ? launch_persist_one<T, false, 4, 4, true, true, 2>(wgs, lds, st, pa)
                               : launch_persist_one<T, false, 2, 4, true, true, 2>(wgs, lds, st, pa);
-  if (pb > 2) return launch_persist_one<T, false, 2, 4, true, true, 4>(wgs, lds, st, pa);  // 256 tokens: registers spill
+  // four blocks: 128 tokens (with 256 the registers spill 260 bytes, and the kernel gains 4 %: 289 us against 302)
+  if (pb > 2) return launch_persist_one<T, false, 2, 4, true, true, 4>(wgs, lds, st, pa);
   if (rfg) return launch_persist_s<T, true, true>(per_token, tile_tokens, wgs, lds, st, pa);
   return staged ? launch_persist_s<T, true, false>(per_token, tile_tokens, wgs, lds, st, pa)
                 : launch_persist_s<T, false, false>(per_token, tile_tokens, wgs, lds, st, pa);
@@ -1169,7 +1184,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
                     ws_bytes >= lay.frag + frag_bytes && switches().collect_staged && switches().collect_persist;
   int tile_tokens = tile_tokens_for(pb, aligned, any_bias, S);
   if (wide) {
-    // 256 tokens where the sequence length wastes little of a wave's 64 (measured 209 us against 231 us at p = 32
+    // 256 tokens where the sequence length wastes little of a wave's 64 (measured 208 us against 225 us at p = 32
     // on 4 x 1024 tokens of 48 modules); with four blocks the registers hold a wave's 32 tokens only
     tile_tokens = pb == 2 && (int64_t)((S + 63) / 64 * 64) * 100 <= (int64_t)S * 104 ? 256 : 128;
   }
@@ -1183,7 +1198,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   for (int m = 0; m < n_modules; ++m) r_steps = std::max(r_steps, (sorted[m].I + sorted[m].O) / kstep);
   const size_t scratch_bytes =
       per_token ? persist_scratch_bytes(tile_tokens)
-                : (size_t)2 * 3 * WAVE * 16 * (wide ? table_blocks(p) * table_blocks(p) : 1);
+                : (wide ? (size_t)4 * WAVE * 16 * table_blocks(p) * table_blocks(p) : (size_t)2 * 3 * WAVE * 16);
   size_t persist_lds = (size_t)r_steps * 1024 + scratch_bytes;
   bool persist = pb == 1 && aligned && !any_bias && persist_lds <= LDS_PER_WG &&
                  tiles * n_modules <= 0x7fffffffLL;
