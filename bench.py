@@ -471,10 +471,11 @@ def per_token_leg(args, torch, device):
 
 
 def wide_projection_leg(args, torch, device):
-    """configs[1]'s 48 modules, per-sequence rows at projection dimensions above 16: the streamed collection kernel
-    with two (p = 32) or four (p = 64) blocks of 16 projection columns per k-step, fragments from the table in global
-    memory, 4 x 1024 tokens per launch.  Kernel only, synthetic a / g; the event pair spans the collection kernel,
-    not the table's preparation before it nor the sum of the tiles' partial blocks behind it."""
+    """configs[1]'s 48 modules at projection dimensions above 16: the streamed collection kernel with two (p = 32)
+    or four (p = 64) blocks of 16 projection columns per k-step, fragments from the table in global memory, 4 x 1024
+    tokens per launch; per-sequence rows, and per-token rows (at p = 32; in two steps, bf16 rows of 49 152 values).
+    Kernel only, synthetic a / g; the event pair spans the collection kernel (and, per token, the kernel that writes
+    the rows), not the table's preparation before it nor the sum of the tiles' partial blocks behind it."""
     from bergson_amd import _lib, ops
 
     N, S, d = 4, 1024, 768
@@ -508,6 +509,25 @@ def wide_projection_leg(args, torch, device):
                         "tokens_per_s_hooks_only": N * S / (ms * 1e-3),
                         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                      "frac": gbs / HBM_PEAK_GBS, "traffic": read * WIDE_TRAFFIC_RATIO[p]}}
+        if p == 32:
+            offsets = torch.arange(N, device=device, dtype=torch.int64) * (S - 1)
+            tok_rows = torch.zeros(N * (S - 1), col, device=device, dtype=torch.bfloat16)
+            run = lambda: ops.collect_tok(mods, p, tok_rows, lengths=lengths, row_offsets=offsets, lo=-3e38, hi=3e38)
+            run()
+            torch.cuda.synchronize()
+            ops.collect_timing_start(reps)
+            for _ in range(reps):
+                run()
+            torch.cuda.synchronize()
+            ms = ops.collect_timing_stop()
+            ms = sum(ms) / len(ms)
+            written = tok_rows.numel() * 2
+            gbs = (read + written) / (ms * 1e-3) / 1e9
+            out["p32_per_token"] = {"ms_per_launch": ms, "kernel": _lib.last_kernel(_lib.FAMILY_COLLECT),
+                                    "bytes_written": written,
+                                    "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                                 "frac": gbs / HBM_PEAK_GBS, "traffic": None}}
+            del tok_rows
         del mods, rows
     return out
 

@@ -422,16 +422,16 @@ __global__ __launch_bounds__(COLLECT_THREADS) void frag_prepare_kernel(const bgx
 }
 
 // PB = blocks of 16 projection columns (p <= 16 * PB).  More than one only with the fragments in the global table
-// (two projections to 32 columns do not fit LDS at the usual widths) and for per-sequence rows: a tile then gives
-// PB x PB blocks of P.
+// (two projections to 32 columns do not fit LDS at the usual widths): a tile then gives PB x PB blocks of P, or,
+// per token, a' and g' of 16 * PB columns each for the two-step rows (the only per-token route with PB > 1).
 template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED = false, bool RFG = false, int PB = 1>
 __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(PersistArgs pa) {
   static_assert(STAGED || !RFG, "the global fragment table is read through the stream's queue");
-  static_assert(PB == 1 || (RFG && !PER_TOKEN), "wider projections: table fragments, per-sequence rows");
+  static_assert(PB == 1 || RFG, "wider projections: fragments from the table");
   using M = Mma<T>;
   constexpr int WAVE_T = 16 * MTW;      // tokens per wave
   constexpr int TILE_T = 4 * WAVE_T;    // tokens per workgroup
-  constexpr int LDP = 20;  // row of a' or g' in LDS: 16 floats, padded so that rows stay 16-byte aligned
+  constexpr int LDP = 16 * PB + 4;  // row of a' or g' in LDS: 16 * PB floats, padded so that rows stay 16-byte aligned
   extern __shared__ __align__(16) unsigned char smem_raw[];
   uint4* rfrag = reinterpret_cast<uint4*>(smem_raw);
   unsigned char* scratch = smem_raw + (size_t)pa.r_steps * WAVE * 16;
@@ -465,14 +465,16 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
   // waits for the store's acknowledgement, which under this read load takes several microseconds -- once per
   // tile that was a sixth of the kernel's time; at the end of a range nothing waits behind it.
   // (Deferring wave 0's p x p partial of the per-sequence launches the same way changed nothing: 171.6 us either way.)
-  constexpr int KEEP_TILES = PER_TOKEN ? 8 : 1;
-  f32x4 keepA[KEEP_TILES][MTW], keepG[KEEP_TILES][MTW];
+  constexpr int KEEP_TILES = PER_TOKEN && PB == 1 ? 8 : 1;  // wider projections: no registers to spare
+  f32x4 keepA[KEEP_TILES][MTW * PB], keepG[KEEP_TILES][MTW * PB];
   int64_t keep_at[KEEP_TILES];  // element offset of the tile's first token in tokproj
   int keep_rows[KEEP_TILES];
   int kept = 0;
   auto flush_kept = [&]() {
     if constexpr (PER_TOKEN) {
-      const int part = lane & 7;  // 16-byte piece of a token's 128 bytes: 0-3 = a', 4-7 = g'
+      // 16-byte piece of a token's 128 * PB bytes: the first 4 * PB are a', the others g'
+      constexpr int PIECES = 8 * PB;
+      const int part = lane & (PIECES - 1);
 #pragma unroll
       for (int j = 0; j < KEEP_TILES; ++j) {
         if (j < kept) {
@@ -482,19 +484,23 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
 #pragma unroll
           for (int mt = 0; mt < MTW; ++mt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              tok[wave][0][mt * 16 + q * 4 + i][c] = keepA[j][mt][i];
-              tok[wave][1][mt * 16 + q * 4 + i][c] = keepG[j][mt][i];
-            }
+            for (int pb = 0; pb < PB; ++pb)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                tok[wave][0][mt * 16 + q * 4 + i][pb * 16 + c] = keepA[j][mt * PB + pb][i];
+                tok[wave][1][mt * 16 + q * 4 + i][pb * 16 + c] = keepG[j][mt * PB + pb][i];
+              }
           __builtin_amdgcn_wave_barrier();
           float* dstp = pa.tokproj + keep_at[j];
+          constexpr int TOK_PER_PASS = WAVE / PIECES;
 #pragma unroll
-          for (int k = 0; k < WAVE_T / 8; ++k) {
-            const int t = k * 8 + (lane >> 3);
-            const float4 val = *reinterpret_cast<const float4*>(&tok[wave][part >> 2][t][(part & 3) * 4]);
+          for (int k = 0; k < WAVE_T / TOK_PER_PASS; ++k) {
+            const int t = k * TOK_PER_PASS + lane / PIECES;
+            const float4 val =
+                *reinterpret_cast<const float4*>(&tok[wave][part / (4 * PB)][t][(part % (4 * PB)) * 4]);
             if (t < keep_rows[j]) {
               typedef float raw4 __attribute__((ext_vector_type(4)));
-              *reinterpret_cast<raw4*>(dstp + t * 32 + part * 4) = raw4{val.x, val.y, val.z, val.w};
+              *reinterpret_cast<raw4*>(dstp + t * (32 * PB) + part * 4) = raw4{val.x, val.y, val.z, val.w};
             }
           }
         }
@@ -659,14 +665,14 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
         __syncthreads();  // the next tile's blocks go to the same place
       }
     } else {
-      if (pa.tokproj != nullptr) {
-        // two-step rows: the wave's a', g' -- 128 bytes per token -- go to the workspace (later: flush_kept), and
+      if (PB > 1 || pa.tokproj != nullptr) {
+        // two-step rows: the wave's a', g' -- 128 * PB bytes per token -- go to the workspace (later: flush_kept), and
         // token_rows_kernel writes the store rows from them, a whole row at a time
         if (rows_valid > 0) {
 #pragma unroll
           for (int j = KEEP_TILES - 1; j > 0; --j) {
 #pragma unroll
-            for (int mt = 0; mt < MTW; ++mt) {
+            for (int mt = 0; mt < MTW * PB; ++mt) {
               keepA[j][mt] = keepA[j - 1][mt];
               keepG[j][mt] = keepG[j - 1][mt];
             }
@@ -674,11 +680,11 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
             keep_rows[j] = keep_rows[j - 1];
           }
 #pragma unroll
-          for (int mt = 0; mt < MTW; ++mt) {
+          for (int mt = 0; mt < MTW * PB; ++mt) {
             keepA[0][mt] = accA[mt];
             keepG[0][mt] = accG[mt];
           }
-          keep_at[0] = ((((int64_t)m * args.N + n) * args.S) + s0 + wave * WAVE_T) * 32;
+          keep_at[0] = ((((int64_t)m * args.N + n) * args.S) + s0 + wave * WAVE_T) * (32 * PB);
           keep_rows[0] = rows_valid;
           if (++kept == KEEP_TILES) flush_kept();
         }
@@ -742,8 +748,8 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
 }
 
 // Second step of the two-step per-token rows: one workgroup per token writes that token's whole store row --
-// every module's p x p block clamp(g'[i] * a'[j]), the arithmetic of the one-step kernel -- from the 128 bytes per
-// module the collection kernel left in `tokproj`.  The blocks of a row are written where the descriptors say
+// every module's p x p block clamp(g'[i] * a'[j]), the arithmetic of the one-step kernel -- from the 2 * pcols
+// floats per module (pcols = 16 for p <= 16, else 32 or 64) the collection kernel left in `tokproj`.  The blocks of a row are written where the descriptors say
 // (adjacent blocks make one contiguous stretch: 24 KB for 48 modules at p = 16), a lane stores 8 consecutive
 // columns with one 16-byte store, and the projections come out of L2.
 template <int DT>
@@ -751,12 +757,13 @@ __global__ __launch_bounds__(256) void token_rows_kernel(const bgx_module_desc* 
                                                          const float* __restrict__ tokproj,
                                                          const int32_t* __restrict__ lengths,
                                                          const int64_t* __restrict__ row_offsets, int N, int S, int p,
-                                                         void* out, int64_t out_row_stride, float lo, float hi) {
+                                                         int pcols, void* out, int64_t out_row_stride, float lo,
+                                                         float hi) {
   const int s = blockIdx.x;
   const int n = blockIdx.y;
   if (s >= seq_token_limit(lengths, n, S)) return;
   const int64_t row = row_offsets[n] + s;
-  const int jg = p >> 3;                 // 8-column groups per block row: 1 or 2
+  const int jg = p >> 3;                 // 8-column groups per block row (p is a multiple of 8)
   const int tasks_pm = p * jg;           // 16-byte pieces of a module's block
   const int tasks = n_modules * tasks_pm;
   for (int task = threadIdx.x; task < tasks; task += 256) {
@@ -764,8 +771,8 @@ __global__ __launch_bounds__(256) void token_rows_kernel(const bgx_module_desc* 
     const int rem = task - m * tasks_pm;
     const int i = rem / jg;
     const int j0 = (rem - i * jg) << 3;
-    const float* src = tokproj + (((int64_t)m * N + n) * S + s) * 32;
-    const float gv = src[16 + i];
+    const float* src = tokproj + (((int64_t)m * N + n) * S + s) * (2 * pcols);  // a' (pcols floats), then g'
+    const float gv = src[pcols + i];
     const float4 a_lo = *reinterpret_cast<const float4*>(src + j0);
     const float4 a_hi = *reinterpret_cast<const float4*>(src + j0 + 4);
     const float o[8] = {clampf(gv * a_lo.x, lo, hi), clampf(gv * a_lo.y, lo, hi), clampf(gv * a_lo.z, lo, hi),
@@ -968,7 +975,7 @@ static int table_blocks(int p) {
 }
 
 // Bytes of the global fragment table for these modules (1 KB per k-step of I + O and block of 16 projection
-// columns), or 0 when the table cannot be used: a width that is not a multiple of two k-steps, p > 32, a bias column.
+// columns), or 0 when the table cannot be used: a width that is not a multiple of two k-steps, p > 64, a bias column.
 static size_t fragment_table_bytes(const bgx_module_desc* mods, int n_modules, int p, int in_dtype) {
   if (p > 16 * PERSIST_MAX_PB) return 0;
   const int kstep = in_dtype == BGX_F32 ? 16 : 32;
@@ -986,11 +993,12 @@ static size_t item_list_bytes(int n_modules, int N, int S) {
   return (size_t)n_modules * (size_t)N * (size_t)((S + 63) / 64) * sizeof(int32_t);
 }
 
-// Projected activations and output gradients of every token (a', g': 2 x 16 floats per module and token), the
-// intermediate of the two-step per-token rows; 0 where that route does not apply (p other than 8 or 16).
+// Projected activations and output gradients of every token (a', g': 2 x 16 floats per module and token, 2 x 32 or
+// 2 x 64 for p > 16), the intermediate of the two-step per-token rows; 0 where that route does not apply (p other
+// than 8, 16 or a multiple of 8 up to 64).
 static size_t token_projection_bytes(int n_modules, int N, int S, int p) {
-  if (p != 8 && p != 16) return 0;
-  return (size_t)n_modules * (size_t)N * (size_t)S * 32 * sizeof(float);
+  if (p != 8 && p != 16 && !(p > 16 && p <= 16 * PERSIST_MAX_PB && p % 8 == 0)) return 0;
+  return (size_t)n_modules * (size_t)N * (size_t)S * 32 * table_blocks(p) * sizeof(float);
 }
 
 // Where the parts of the larger workspace start.
@@ -1002,7 +1010,8 @@ static WorkspaceLayout workspace_layout(size_t base, size_t table, int n_modules
   l.frag = align_up(base, 256);
   l.order = align_up(l.frag + table, 256);
   l.tokproj = align_up(l.order + (table ? item_list_bytes(n_modules, N, S) : 0), 256);
-  l.total = l.tokproj + token_projection_bytes(n_modules, N, S, p);
+  // wider projections reach the two-step rows only through the table
+  l.total = l.tokproj + (p > 16 && table == 0 ? 0 : token_projection_bytes(n_modules, N, S, p));
   return l;
 }
 
@@ -1097,10 +1106,12 @@ static int launch_persist_s(bool per_token, int tile_tokens, int wgs, size_t lds
 }
 
 // staged: streamed token rows; rfg: (staged only) projection fragments from the global table; pb: blocks of 16
-// projection columns (more than one: table fragments and per-sequence rows only, tiles of 128 or 256 tokens)
+// projection columns (more than one: table fragments only, tiles of 128 or 256 tokens; per token 128, two-step rows)
 template <typename T>
 static int launch_persist(bool staged, bool rfg, bool per_token, int pb, int tile_tokens, int wgs, size_t lds,
                           hipStream_t st, const PersistArgs& pa) {
+  if (pb == 2 && per_token) return launch_persist_one<T, true, 2, 4, true, true, 2>(wgs, lds, st, pa);
+  if (pb > 2 && per_token) return launch_persist_one<T, true, 2, 4, true, true, 4>(wgs, lds, st, pa);
   if (pb == 2)
     return tile_tokens == 256 ? launch_persist_one<T, false, 4, 4, true, true, 2>(wgs, lds, st, pa)
                               : launch_persist_one<T, false, 2, 4, true, true, 2>(wgs, lds, st, pa);
@@ -1112,8 +1123,8 @@ static int launch_persist(bool staged, bool rfg, bool per_token, int pb, int til
 }
 
 // LDS beside the projection fragments: the larger of the P exchange buffers and the per-token a', g' tiles
-static size_t persist_scratch_bytes(int tile_tokens) {
-  return std::max((size_t)2 * 3 * WAVE * 16, (size_t)2 * tile_tokens * 20 * sizeof(float));
+static size_t persist_scratch_bytes(int tile_tokens, int blocks = 1) {
+  return std::max((size_t)2 * 3 * WAVE * 16, (size_t)2 * tile_tokens * (16 * blocks + 4) * sizeof(float));
 }
 
 int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules, int N, int S,
@@ -1180,10 +1191,18 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   // as many bytes of fragments as of tokens, or half as many).
   const size_t frag_bytes = fragment_table_bytes(sorted.data(), n_modules, p, in_dtype);
   const WorkspaceLayout lay = workspace_layout(need, frag_bytes, n_modules, N, S, p);
-  const bool wide = pb > 1 && pb <= PERSIST_MAX_PB && !per_token && aligned && !any_bias && frag_bytes > 0 &&
-                    ws_bytes >= lay.frag + frag_bytes && switches().collect_staged && switches().collect_persist;
+  // Per-token rows take it only in two steps (projections of every token to the workspace, whole rows from there).
+  const int64_t out_elem = out_dtype == BGX_F32 ? 4 : 2;
+  bool wide_tok = per_token && pb > 1 && p % 8 == 0 && (uintptr_t)out % 16 == 0 &&
+                  (out_row_stride * out_elem) % 16 == 0 && lay.total > lay.tokproj && ws_bytes >= lay.total &&
+                  N <= 65535 && !switches().collect_two_step_off;
+  for (int m = 0; m < n_modules && wide_tok; ++m) wide_tok = (sorted[m].out_col * out_elem) % 16 == 0;
+  const bool wide = pb > 1 && pb <= PERSIST_MAX_PB && (!per_token || wide_tok) && aligned && !any_bias &&
+                    frag_bytes > 0 && ws_bytes >= lay.frag + frag_bytes && switches().collect_staged &&
+                    switches().collect_persist;
   int tile_tokens = tile_tokens_for(pb, aligned, any_bias, S);
-  if (wide) {
+  if (wide && per_token) tile_tokens = 128;
+  if (wide && !per_token) {
     // 256 tokens where the sequence length wastes little of a wave's 64 (measured 208 us against 225 us at p = 32
     // on 4 x 1024 tokens of 48 modules); with four blocks the registers hold a wave's 32 tokens only
     tile_tokens = pb == 2 && (int64_t)((S + 63) / 64 * 64) * 100 <= (int64_t)S * 104 ? 256 : 128;
@@ -1197,7 +1216,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   int r_steps = 0;
   for (int m = 0; m < n_modules; ++m) r_steps = std::max(r_steps, (sorted[m].I + sorted[m].O) / kstep);
   const size_t scratch_bytes =
-      per_token ? persist_scratch_bytes(tile_tokens)
+      per_token ? persist_scratch_bytes(tile_tokens, wide ? table_blocks(p) : 1)
                 : (wide ? (size_t)4 * WAVE * 16 * table_blocks(p) * table_blocks(p) : (size_t)2 * 3 * WAVE * 16);
   size_t persist_lds = (size_t)r_steps * 1024 + scratch_bytes;
   bool persist = pb == 1 && aligned && !any_bias && persist_lds <= LDS_PER_WG &&
@@ -1364,8 +1383,8 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     pa.tiles_pm = (int)tiles;
     pa.r_steps = r_steps;
     pa.scratch_bytes = (int)scratch_bytes;
-    const int64_t out_elem = out_dtype == BGX_F32 ? 4 : 2;
-    bool vec8 = per_token && (p == 8 || p == 16) && (uintptr_t)out % 16 == 0 && (out_row_stride * out_elem) % 16 == 0;
+    bool vec8 = per_token && (p == 8 || p == 16 || wide) && (uintptr_t)out % 16 == 0 &&
+                (out_row_stride * out_elem) % 16 == 0;
     for (int m = 0; m < n_modules && vec8; ++m) vec8 = (sorted[m].out_col * out_elem) % 16 == 0;
     pa.out_vec8 = vec8 ? 1 : 0;
     // per-token rows in two steps when the blocks can be written 16 bytes at a time and the caller's workspace has
@@ -1396,13 +1415,13 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     const float* tp = (const float*)((const char*)ws + lay.tokproj);
     if (out_dtype == BGX_F32)
       hipLaunchKernelGGL(token_rows_kernel<BGX_F32>, tgrid, dim3(256), 0, st, mods_dev, n_modules, tp, lengths,
-                         rows_or_offsets, N, S, p, out, out_row_stride, lo, hi);
+                         rows_or_offsets, N, S, p, 16 * table_blocks(p), out, out_row_stride, lo, hi);
     else if (out_dtype == BGX_F16)
       hipLaunchKernelGGL(token_rows_kernel<BGX_F16>, tgrid, dim3(256), 0, st, mods_dev, n_modules, tp, lengths,
-                         rows_or_offsets, N, S, p, out, out_row_stride, lo, hi);
+                         rows_or_offsets, N, S, p, 16 * table_blocks(p), out, out_row_stride, lo, hi);
     else
       hipLaunchKernelGGL(token_rows_kernel<BGX_BF16>, tgrid, dim3(256), 0, st, mods_dev, n_modules, tp, lengths,
-                         rows_or_offsets, N, S, p, out, out_row_stride, lo, hi);
+                         rows_or_offsets, N, S, p, 16 * table_blocks(p), out, out_row_stride, lo, hi);
     BGX_HIP(hipGetLastError());
   }
   if (timed) BGX_HIP(hipEventRecord(ev_stop, st));

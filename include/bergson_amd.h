@@ -123,10 +123,11 @@ int bgx_adafactor_scales(const float* row_dev, int32_t O, const float* col_dev,
  * projection fragments, 32 bytes per input and output feature (64 for
  * 16 < p <= 32, 128 for 32 < p <= 64), and the list of work items behind it
  * (4 bytes per module and 64 tokens): with it, modules too wide for their
- * projections to be kept on chip (Llama-3-8B's 4096 x 14336) and per-sequence
- * launches at p > 16 still run through the streamed persistent kernel;
+ * projections to be kept on chip (Llama-3-8B's 4096 x 14336) and launches
+ * at p > 16 still run through the streamed persistent kernel;
  * without it such launches use the one-workgroup-per-tile kernel, which is a
- * third to a half slower; (ii) at p = 8 or 16,
+ * third to a half slower; (ii) at p = 8 or 16 (and, with the table, at any
+ * multiple of 8 up to 64: 256 or 512 bytes per module and token),
  * the projected activations and output gradients of every token (128 bytes
  * per module and token): with it bgx_collect_tok writes its rows in two steps
  * -- the collection kernel leaves those projections in the workspace and a

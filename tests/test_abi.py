@@ -81,11 +81,12 @@ def test_workspace_sizes():
     assert lib.bgx_collect_workspace_bytes_for(descs, 2, 2, 2048, 16, 2) == up(base) + tokens
     base32 = lib.bgx_collect_workspace_bytes(2, 2, 2048, 32)
     assert lib.bgx_collect_workspace_bytes_for(descs, 2, 2, 2048, 32, 2) == up(base32)   # p = 32: neither
-    descs[1].O = 1024   # p = 32, 64: the table holds two, four blocks of 16 projection columns; no per-token rows
-    for p, blocks in ((32, 2), (48, 4), (50, 4), (64, 4)):
+    descs[1].O = 1024   # p = 32, 64: the table holds two, four blocks of 16 projection columns; the tokens' projections
+    for p, blocks in ((32, 2), (48, 4), (50, 4), (64, 4)):   # are 128 bytes per block (p a multiple of 8 only)
         basep = lib.bgx_collect_workspace_bytes(2, 2, 2048, p)
         assert (lib.bgx_collect_workspace_bytes_for(descs, 2, 2, 2048, p, 2)
-                == up(up(up(basep) + (4096 + 14336 + 4096 + 1024) * 32 * blocks) + 2 * 2 * (2048 // 64) * 4))
+                == up(up(up(basep) + (4096 + 14336 + 4096 + 1024) * 32 * blocks) + 2 * 2 * (2048 // 64) * 4)
+                + (tokens * blocks if p % 8 == 0 else 0))
     small = lib.bgx_scan_workspace_bytes(8, 10, 1024)
     assert small >= 8 * 10 * 8 + 8 * 1024 * 8
     assert lib.bgx_scan_workspace_bytes(1024, 100, 0) >= 1024 * 65536 * 8

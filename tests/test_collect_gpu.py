@@ -293,6 +293,34 @@ def test_seq_wide_projections(device, dtype, p, S, kernel_variant):
     assert got[2].abs().sum() == 0
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("p,S", [(32, 300), (64, 200), (24, 129), (40, 70), (20, 90)])
+def test_tok_wide_projections(device, dtype, p, S, kernel_variant):
+    """Per-token rows at p > 16: with p a multiple of 8 the streamed kernel leaves every token's a', g' (32 or 64
+    columns each) in the workspace and token_rows_kernel writes the rows (the default variant); other p, and the other
+    two variants, take the tile kernel.  Ragged lengths, two modules."""
+    from bergson_amd import _lib
+
+    N = 3
+    lengths = [S, S // 2 + 1, 2]
+    cases = []
+    for i, (I, O) in enumerate([(128, 256), (64, 64)]):
+        a, g, left, right, norm = make_case(N, S, I, O, p, dtype, seed=80 + i, normalizer="adafactor" if i == 1 else None,
+                                            name=f"layers.{i}.tok{p}")
+        for n, l in enumerate(lengths):
+            g[n, l - 1:] = 0
+        cases.append((a, g, left, right, norm))
+    counts = [l - 1 for l in lengths]
+    row_offsets = [sum(counts[:n]) for n in range(N)]
+    mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+    got = run_kernel(device, cases, p, dtype, lengths=lengths, per_token=True, row_offsets=row_offsets, n_rows=sum(counts))
+    streamed = kernel_variant == "streamed" and p % 8 == 0
+    assert _lib.last_kernel(_lib.FAMILY_COLLECT) == ("collect_persist_table" if streamed else "collect_tile")
+    want = oracle_rows(cases, dtype, attribute_tokens=True, collection_mask=mask)
+    assert got.shape == want.shape
+    assert rel_l2(got, want) <= TOL[dtype]
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("p", [16, 32, 8])
 def test_tok(device, dtype, p):
