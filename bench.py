@@ -56,6 +56,7 @@ SCAN_TRAFFIC_RATIO_Q1024 = 1.345
 SCAN_TRAFFIC_RATIO_FEW = 1.0016
 PER_TOKEN_TRAFFIC_RATIO = 1.068
 WIDE_TRAFFIC_RATIO = {32: 1.078, 64: 1.151}
+WIDE_TOK_TRAFFIC_RATIO = 1.113
 LLAMA_TRAFFIC_RATIO = 1.007
 # bytes the four fused Adam launches of one layer fetch through the L2s and write, from the same counters
 # (profiles/adam_fused_pythia410m_layer_p32.txt): 5.19 GB + 0.07 GB, against 0.94 GB read once each
@@ -526,7 +527,8 @@ def wide_projection_leg(args, torch, device):
             out["p32_per_token"] = {"ms_per_launch": ms, "kernel": _lib.last_kernel(_lib.FAMILY_COLLECT),
                                     "bytes_written": written,
                                     "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                                 "frac": gbs / HBM_PEAK_GBS, "traffic": None}}
+                                                 "frac": gbs / HBM_PEAK_GBS,
+                                                 "traffic": (read + written) * WIDE_TOK_TRAFFIC_RATIO}}
             del tok_rows
         del mods, rows
     return out
