@@ -774,7 +774,6 @@ __device__ inline void fw_static_for(std::integer_sequence<int, Is...>, F&& f) {
 
 template <typename T>
 __global__ __launch_bounds__(FW_THREADS) void adam_fused_wide_kernel(FusedArgs a) {
-  using M = Mma32<T>;
   static_assert(sizeof(T) == 2, "the fused Adam kernel is for 16-bit model dtypes");
   constexpr int BM = FUSED_TILE, BN = FUSED_TILE, BK = 64;
   constexpr int TM = 4, TN = 4;
@@ -799,8 +798,6 @@ __global__ __launch_bounds__(FW_THREADS) void adam_fused_wide_kernel(FusedArgs a
   const int p = a.p, O = a.O, pp = p * p;
   const int KT = a.I / BK;  // at least 4 (host)
   const int n_chunks = O / BN;
-  const int per_chunk = KT + FD_GSLICES;
-  const int total = per_chunk * n_chunks;
 
   // ---- the load stream
   const uint32_t a_row_bytes = (uint32_t)(a.a_tok_stride * sizeof(T));

@@ -854,7 +854,7 @@ __global__ __launch_bounds__(256) void unit_normalize_kernel(T* rows, int64_t n_
   }
   red[threadIdx.x] = s;
   __syncthreads();
-  for (int w = 128; w > 0; w >>= 1) {
+  for (unsigned w = 128; w > 0; w >>= 1) {
     if (threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
     __syncthreads();
   }
