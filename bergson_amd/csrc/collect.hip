@@ -424,10 +424,14 @@ __global__ __launch_bounds__(COLLECT_THREADS) void frag_prepare_kernel(const bgx
 // PB = blocks of 16 projection columns (p <= 16 * PB).  More than one only with the fragments in the global table
 // (two projections to 32 columns do not fit LDS at the usual widths): a tile then gives PB x PB blocks of P, or,
 // per token, a' and g' of 16 * PB columns each for the two-step rows (the only per-token route with PB > 1).
+// With RFG the workgroup's waves load each block of table fragments once between them and pass it round through LDS
+// (stream_segment_shared: SHARE below) instead of each loading all of it; all four then stream in step, tile after
+// tile, and a wave without tokens in a tile streams that tile's first row and discards what it gets.
 template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED = false, bool RFG = false, int PB = 1>
 __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(PersistArgs pa) {
   static_assert(STAGED || !RFG, "the global fragment table is read through the stream's queue");
   static_assert(PB == 1 || RFG, "wider projections: fragments from the table");
+  constexpr bool SHARE = RFG;
   using M = Mma<T>;
   constexpr int WAVE_T = 16 * MTW;      // tokens per wave
   constexpr int TILE_T = 4 * WAVE_T;    // tokens per workgroup
@@ -457,7 +461,10 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
   // STAGED: the register queue of the wave's input stream, and whether it holds the first block of the
   // tile that comes next
   uint4 v[STAGED ? STREAM_Q : 1][2 * MTW];
-  uint4 rq[RFG ? STREAM_Q : 1][2 * PB];  // RFG: the fragments that go with v
+  uint4 rq[1][2 * PB];  // (the per-wave fragment queue of stream_segment<RFG>: not used here)
+  uint4 rs[2 * PB];  // SHARE: this wave's k-pair of the block of fragments that comes next
+  uint4* ring = reinterpret_cast<uint4*>(scratch + pa.scratch_bytes + 4 * Stream<MTW>::BYTES_PER_WAVE);  // SHARE
+  int ring_slot = 0;
   bool primed = false;
   // Two-step per-token rows: a tile leaves 16 * MTW tokens x 32 floats per wave, i.e. 8 * MTW registers per lane.
   // They stay in registers until KEEP_TILES tiles have gathered or the range ends, and go to the workspace then:
@@ -523,22 +530,27 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
     const int s_limit = seq_token_limit_uniform(args.lengths, n, args.S);
     if (s0 >= s_limit) continue;  // whole tile is padding (uniform over the workgroup); nothing ran ahead into it
     const int rows_valid = min(WAVE_T, s_limit - s0 - wave * WAVE_T);  // of this wave; may be <= 0
+    // rows the wave streams: its own, or (SHARE, none of its own) the tile's first
+    const int rows_eff = SHARE ? max(rows_valid, 1) : rows_valid;
 
     const bgx_module_desc d = load_uniform(args.mods + m);
     const int nA = d.I / M::KS;
     const uint4* rfA = rfrag;  // fragments of r_in, then of r_out: in LDS, or (RFG) in the global table
     if constexpr (RFG) rfA = pa.frag + load_uniform(pa.frag_off + m) * WAVE;
     const uint4* rfG = rfA + (size_t)nA * PB * WAVE;
-    const int64_t t0 = s0 + wave * WAVE_T;
+    const int64_t t0 = s0 + (SHARE && rows_valid <= 0 ? 0 : wave * WAVE_T);
     const T* a0 = (const T*)d.a + (int64_t)n * d.a_seq_stride + t0 * d.a_tok_stride;
     const T* g0 = (const T*)d.g + (int64_t)n * d.g_seq_stride + t0 * d.g_tok_stride;
     if constexpr (STAGED) {
       // a tile nothing ran ahead into (the first of the range, or after padding): its first loads go out
       // before the projections are staged
-      if (rows_valid > 0 && !primed) {
+      if (rows_eff > 0 && !primed) {
         const T* ua[2 * MTW];
-        stream_rows<T, MTW>(a0, d.a_tok_stride, rows_valid, lane, ua);
-        stream_prime<T, MTW, RFG, PB>(ua, d.I / (2 * M::KS), rfA, lane, v, rq);
+        stream_rows<T, MTW>(a0, d.a_tok_stride, rows_eff, lane, ua);
+        if constexpr (SHARE)
+          stream_prime_shared<T, MTW, PB>(ua, d.I / (2 * M::KS), rfA, lane, wave, v, rs);
+        else
+          stream_prime<T, MTW, false, PB>(ua, d.I / (2 * M::KS), rfA, lane, v, rq);
         primed = true;
       }
     }
@@ -561,16 +573,19 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
       accA[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
       accG[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
-    if (rows_valid > 0) {
+    if (rows_eff > 0) {
       if constexpr (STAGED) {
         constexpr int RG = 2 * MTW;
         const int nkpA = d.I / (2 * M::KS), nkpG = d.O / (2 * M::KS);
         const T* ua[RG];
         const T* ug[RG];
         const T* un[RG];
-        stream_rows<T, MTW>(a0, d.a_tok_stride, rows_valid, lane, ua);
-        stream_rows<T, MTW>(g0, d.g_tok_stride, rows_valid, lane, ug);
-        stream_segment<T, MTW, RFG, PB>(ua, nkpA, ug, nkpG, rfA, rfG, stage, lane, v, rq, accA);
+        stream_rows<T, MTW>(a0, d.a_tok_stride, rows_eff, lane, ua);
+        stream_rows<T, MTW>(g0, d.g_tok_stride, rows_eff, lane, ug);
+        if constexpr (SHARE)
+          stream_segment_shared<T, MTW, PB>(ua, nkpA, ug, nkpG, rfA, rfG, stage, ring, ring_slot, lane, wave, v, rs, accA);
+        else
+          stream_segment<T, MTW, false, PB>(ua, nkpA, ug, nkpG, rfA, rfG, stage, lane, v, rq, accA);
         // what follows g: the a rows of the next tile of the range, where this wave has tokens in it
         int nkpN = 0;
         const uint4* rfN = rfG;  // RFG: the next tile's r_in fragments (any readable address when none follows)
@@ -585,18 +600,23 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
           const int tile2 = item2 - m2 * pa.tiles_pm;
           const int n2 = tile2 / args.tiles_per_seq;
           const int s02 = (tile2 - n2 * args.tiles_per_seq) * TILE_T;
-          const int rows2 = min(WAVE_T, seq_token_limit_uniform(args.lengths, n2, args.S) - s02 - wave * WAVE_T);
-          if (rows2 > 0) {  // implies that the tile is not all padding
+          const int limit2 = seq_token_limit_uniform(args.lengths, n2, args.S);
+          const int rows2 = min(WAVE_T, limit2 - s02 - wave * WAVE_T);
+          // SHARE: whenever the tile is not all padding, the waves without tokens in it with its first row
+          if (SHARE ? s02 < limit2 : rows2 > 0) {  // rows2 > 0 implies that the tile is not all padding
             const bgx_module_desc* d2 = args.mods + m2;
             const int64_t stride2 = load_uniform(&d2->a_tok_stride);
             const T* a2 = (const T*)load_uniform(&d2->a) + (int64_t)n2 * load_uniform(&d2->a_seq_stride) +
-                          (int64_t)(s02 + wave * WAVE_T) * stride2;
-            stream_rows<T, MTW>(a2, stride2, rows2, lane, un);
+                          (int64_t)(s02 + (rows2 > 0 ? wave * WAVE_T : 0)) * stride2;
+            stream_rows<T, MTW>(a2, stride2, max(rows2, 1), lane, un);
             nkpN = load_uniform(&d2->I) / (2 * M::KS);
             if constexpr (RFG) rfN = pa.frag + load_uniform(pa.frag_off + m2) * WAVE;
           }
         }
-        stream_segment<T, MTW, RFG, PB>(ug, nkpG, un, nkpN, rfG, rfN, stage, lane, v, rq, accG);
+        if constexpr (SHARE)
+          stream_segment_shared<T, MTW, PB>(ug, nkpG, un, nkpN, rfG, rfN, stage, ring, ring_slot, lane, wave, v, rs, accG);
+        else
+          stream_segment<T, MTW, false, PB>(ug, nkpG, un, nkpN, rfG, rfN, stage, lane, v, rq, accG);
         primed = nkpN > 0;
       } else if constexpr (PB == 1) {
         project_tokens_lds<T, MTW, U>(a0, d.a_tok_stride, rows_valid, d.I, rfA, lane, accA);
@@ -1105,19 +1125,33 @@ static int launch_persist_s(bool per_token, int tile_tokens, int wgs, size_t lds
                    : launch_persist_one<T, false, 1, 8, STAGED, RFG>(wgs, lds, st, pa);
 }
 
-// staged: streamed token rows; rfg: (staged only) projection fragments from the global table; pb: blocks of 16
-// projection columns (more than one: table fragments only, tiles of 128 or 256 tokens; per token 128, two-step rows)
+// the variants with the fragments in the global table; pb: blocks of 16 projection columns (more than one: tiles of
+// 128 or 256 tokens; per token 128, two-step rows)
+template <typename T>
+static int launch_persist_table(bool per_token, int pb, int tile_tokens, int wgs, size_t lds, hipStream_t st,
+                                const PersistArgs& pa) {
+  if (pb == 1) {
+    if (tile_tokens == 128)
+      return per_token ? launch_persist_one<T, true, 2, 4, true, true, 1>(wgs, lds, st, pa)
+                       : launch_persist_one<T, false, 2, 4, true, true, 1>(wgs, lds, st, pa);
+    return per_token ? launch_persist_one<T, true, 1, 8, true, true, 1>(wgs, lds, st, pa)
+                     : launch_persist_one<T, false, 1, 8, true, true, 1>(wgs, lds, st, pa);
+  }
+  if (pb == 2) {
+    if (per_token) return launch_persist_one<T, true, 2, 4, true, true, 2>(wgs, lds, st, pa);
+    return tile_tokens == 256 ? launch_persist_one<T, false, 4, 4, true, true, 2>(wgs, lds, st, pa)
+                              : launch_persist_one<T, false, 2, 4, true, true, 2>(wgs, lds, st, pa);
+  }
+  // four blocks: 128 tokens (with 256 the registers spill 200 bytes)
+  return per_token ? launch_persist_one<T, true, 2, 4, true, true, 4>(wgs, lds, st, pa)
+                   : launch_persist_one<T, false, 2, 4, true, true, 4>(wgs, lds, st, pa);
+}
+
+// staged: streamed token rows; rfg: (staged only) projection fragments from the global table
 template <typename T>
 static int launch_persist(bool staged, bool rfg, bool per_token, int pb, int tile_tokens, int wgs, size_t lds,
                           hipStream_t st, const PersistArgs& pa) {
-  if (pb == 2 && per_token) return launch_persist_one<T, true, 2, 4, true, true, 2>(wgs, lds, st, pa);
-  if (pb > 2 && per_token) return launch_persist_one<T, true, 2, 4, true, true, 4>(wgs, lds, st, pa);
-  if (pb == 2)
-    return tile_tokens == 256 ? launch_persist_one<T, false, 4, 4, true, true, 2>(wgs, lds, st, pa)
-                              : launch_persist_one<T, false, 2, 4, true, true, 2>(wgs, lds, st, pa);
-  // four blocks: 128 tokens (with 256 the registers spill 260 bytes, and the kernel gains 4 %: 289 us against 302)
-  if (pb > 2) return launch_persist_one<T, false, 2, 4, true, true, 4>(wgs, lds, st, pa);
-  if (rfg) return launch_persist_s<T, true, true>(per_token, tile_tokens, wgs, lds, st, pa);
+  if (rfg) return launch_persist_table<T>(per_token, pb, tile_tokens, wgs, lds, st, pa);
   return staged ? launch_persist_s<T, true, false>(per_token, tile_tokens, wgs, lds, st, pa)
                 : launch_persist_s<T, false, false>(per_token, tile_tokens, wgs, lds, st, pa);
 }
@@ -1236,10 +1270,10 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   bool rfg = !persist && (pb == 1 || wide) && aligned && !any_bias && tiles * n_modules <= 0x7fffffffLL && frag_bytes > 0 &&
              ws_bytes >= frag_ws_off + frag_bytes;
   rfg = rfg && switches().collect_staged;
-  if (rfg) {
+  if (rfg) {  // beside the rest: the ring through which the workgroup shares the table's fragments
     persist = staged = true;
     r_steps = 0;
-    persist_lds = scratch_bytes + stage_bytes;
+    persist_lds = scratch_bytes + stage_bytes + (size_t)stream_ring_bytes(table_blocks(p));
   }
   // BGX_COLLECT_PERSIST=0 in the environment forces the one-workgroup-per-tile kernel (tests, comparisons)
   persist = persist && switches().collect_persist;

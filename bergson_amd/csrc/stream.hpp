@@ -247,5 +247,119 @@ __device__ inline void stream_segment(const T* const (&cur)[2 * MTW], int nkp, c
 }
 static_assert(STREAM_Q == 4, "stream_segment spells out its four steps");
 
+// ---- table fragments shared by the workgroup --------------------------------------------------------------------
+// With the fragments in the global table each wave of stream_segment<RFG> loads every fragment for itself: 2 * QB KB
+// per k-pair and wave beside its 2 * MTW KB of rows.  Those loads hit in the L2s, but they pass through the compute
+// unit's one vector memory pipeline behind the rows' misses, and what they cost is its time (about 21 cycles per
+// 1 KB load, added to a step whose rows take HBM's time: four waves at QB = 4 spend 670 of a step's 2170 cycles on
+// them).  Here the four waves of a workgroup -- which walk the same k-pairs of the same module at the same time --
+// load each fragment once: of a block of STREAM_Q = 4 k-pairs wave w fetches k-pair w (2 * QB loads into rs, one
+// block ahead like the rows), writes it to one of two LDS slots at the start of the block, and after a barrier
+// every wave reads the block's fragments from there.  One barrier per block: the slot written for block b + 1 was
+// last read during block b - 1, which every wave has left when it has passed the barrier of block b.
+// Every wave of the workgroup must call these with the same nkp / nkp_next sequence (the barrier); a wave without
+// rows of its own passes rows that are safe to read and discards what it accumulates.
+constexpr int stream_ring_bytes(int qb) { return 2 * STREAM_Q * 2 * qb * WAVE * 16; }
+
+// bare barrier: the LDS writes of this wave are done, the global loads in flight stay in flight
+__device__ inline void stream_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <typename T, int MTW, int QB>
+__device__ inline void stream_prime_shared(const T* const (&urow)[2 * MTW], int nkp, const uint4* __restrict__ rf,
+                                           int lane, int wave, uint4 (&v)[STREAM_Q][2 * MTW], uint4 (&rs)[2 * QB]) {
+  // the fragments first, as in a block of the segment: on every path into a block its fragment loads then have
+  // exactly the block's STREAM_Q * 2 * MTW row loads behind them, and the wait in front of the ring write is that count
+  const int wj = wave < nkp ? wave : 0;
+#pragma unroll
+  for (int s = 0; s < 2 * QB; ++s) rs[s] = load16_global(rf + (wj * 2 * QB + s) * WAVE + lane);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int j = 0; j < STREAM_Q; ++j) {
+    const int jj = j < nkp ? j : 0;
+#pragma unroll
+    for (int rg = 0; rg < 2 * MTW; ++rg) v[j][rg] = load16_global_stream(urow[rg] + jj * 2 * Mma<T>::KS);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+// ring: the two LDS slots (stream_ring_bytes); ring_slot: which of them the block that comes next uses (kept by the
+// caller across segments)
+template <typename T, int MTW, int QB>
+__device__ inline void stream_segment_shared(const T* const (&cur)[2 * MTW], int nkp, const T* const (&nxt)[2 * MTW],
+                                             int nkp_next, const uint4* __restrict__ rf,
+                                             const uint4* __restrict__ rf_next, unsigned char* __restrict__ stage,
+                                             uint4* __restrict__ ring, int& ring_slot, int lane, int wave,
+                                             uint4 (&v)[STREAM_Q][2 * MTW], uint4 (&rs)[2 * QB],
+                                             f32x4 (&acc)[MTW * QB]) {
+  using M = Mma<T>;
+  using St = Stream<MTW>;
+  constexpr int RG = St::RG;
+  constexpr int Q = STREAM_Q;
+  constexpr int SLOT = Q * 2 * QB * WAVE;  // uint4 entries of a ring slot
+  const int r = lane & 15;
+  const int q = lane >> 4;
+  int foff[MTW][2];  // fragment of 16-row block mt, k-step s of the pair, inside a slot
+#pragma unroll
+  for (int mt = 0; mt < MTW; ++mt)
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+      foff[mt][s] = (mt * 2 + (r >> 3)) * 1024 + (r & 7) * 128 + (((s * 4 + q) ^ (r & 7) ^ (r >> 3)) << 4);
+
+  for (int kp0 = 0; kp0 < nkp; kp0 += Q) {
+    const int len = min(Q, nkp - kp0);
+    const bool last = kp0 + Q >= nkp;
+    const int len_next = last ? min(Q, nkp_next) : min(Q, nkp - kp0 - Q);
+    const T* nptr[RG];
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg) nptr[rg] = last ? nxt[rg] : cur[rg] + (kp0 + Q) * 2 * M::KS;
+    const uint4* nrf = last ? rf_next : rf + (kp0 + Q) * 2 * QB * WAVE;
+
+    // this wave's k-pair of the block goes to the ring; behind the barrier the whole block is there
+    uint4* slotf = ring + ring_slot * SLOT;
+#pragma unroll
+    for (int s = 0; s < 2 * QB; ++s) slotf[(wave * 2 * QB + s) * WAVE + lane] = rs[s];
+    stream_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    {  // its k-pair of the block that follows (k-pair 0 again where that block is shorter: never used)
+      const int wj = wave < len_next ? wave : 0;
+#pragma unroll
+      for (int s = 0; s < 2 * QB; ++s) rs[s] = load16_global(nrf + (wj * 2 * QB + s) * WAVE + lane);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    auto step = [&](auto j_tag) {
+      constexpr int j = decltype(j_tag)::value;
+      if (j < len) {
+#pragma unroll
+        for (int rg = 0; rg < RG; ++rg) *reinterpret_cast<uint4*>(stage + rg * 1024 + lane * 16) = v[j][rg];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      const int jj = j < len_next ? j : 0;
+#pragma unroll
+      for (int rg = 0; rg < RG; ++rg) v[j][rg] = load16_global_stream(nptr[rg] + jj * 2 * M::KS);
+      __builtin_amdgcn_sched_barrier(0);
+      if (j < len) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+          uint4 rfv[QB];
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb) rfv[qb] = slotf[((j * 2 + s) * QB + qb) * WAVE + lane];
+#pragma unroll
+          for (int mt = 0; mt < MTW; ++mt) {
+            const uint4 xf = *reinterpret_cast<const uint4*>(stage + foff[mt][s]);
+#pragma unroll
+            for (int qb = 0; qb < QB; ++qb) M::mma(xf, rfv[qb], acc[mt * QB + qb]);
+          }
+        }
+      }
+    };
+    step(std::integral_constant<int, 0>{});
+    step(std::integral_constant<int, 1>{});
+    step(std::integral_constant<int, 2>{});
+    step(std::integral_constant<int, 3>{});
+    ring_slot ^= 1;
+  }
+}
+
 
 }  // namespace bgx
