@@ -1031,7 +1031,11 @@ __global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
 // rows at a time over all of D with whole-line non-temporal loads through its register queue and its own
 // LDS slot, the queries come as MFMA fragments from a table in global memory (built once per scan; every
 // wave reads the same table, so it lives in L2), the row norms are summed from the data on its way to LDS.
-// No workgroup barrier anywhere.  Scores land in 16 x 16 accumulators: lane (c, q4) holds rows 4 q4 + e of
+// With one or two blocks of 16 queries every wave loads the table's fragments for itself and no workgroup barrier
+// is anywhere; with three (SHARE) the waves of a workgroup load each fragment once between them and share it through
+// LDS (stream_segment_shared: one barrier per four k-pairs, the waves stream in step).  Same box, 10^6 x 12288 fp16:
+// 48 queries 4.10 ms shared against 4.32, 32 queries 4.00 either way, 16 queries 4.01 against 3.92 -- the waves then
+// wait for each other's selection loops, and there is little to save.  Scores land in 16 x 16 accumulators: lane (c, q4) holds rows 4 q4 + e of
 // each 16-row block against query 16 qb + c.
 constexpr int SS_MTW = 4;                // 16-row blocks per wave
 constexpr int SS_WAVE_ROWS = 16 * SS_MTW;
@@ -1049,7 +1053,7 @@ __global__ __launch_bounds__(COLLECT_THREADS) void scan_query_fragments_kernel(c
                       ks0 + 4 * STAGE_B, blk, nblk);
 }
 
-template <typename T, int QB>
+template <typename T, int QB, bool SHARE = (QB >= 3)>
 __global__ __launch_bounds__(COLLECT_THREADS, 1) void scan_stream_kernel(ScanArgs args, const uint4* __restrict__ qfrag) {
   using M = Mma<T>;
   using St = Stream<SS_MTW>;
@@ -1063,6 +1067,10 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void scan_stream_kernel(ScanArg
   float* sc = reinterpret_cast<float*>(smem + 4 * St::BYTES_PER_WAVE) + wave * (SS_WAVE_ROWS * SC_PITCH);
   float* wrow = reinterpret_cast<float*>(smem + 4 * St::BYTES_PER_WAVE) + 4 * (SS_WAVE_ROWS * SC_PITCH) +
                 wave * SS_WAVE_ROWS;  // row multipliers
+  // behind them: the two slots through which the workgroup's waves share the table's fragments
+  uint4* ring = reinterpret_cast<uint4*>(smem + 4 * St::BYTES_PER_WAVE + 4 * (SS_WAVE_ROWS * SC_PITCH) * sizeof(float) +
+                                         4 * SS_WAVE_ROWS * sizeof(float));
+  int ring_slot = 0;
   const int c = lane & 15;
   const int q4 = lane >> 4;
   const int rho = lane >> 3;
@@ -1076,20 +1084,25 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void scan_stream_kernel(ScanArg
   const int64_t r_first = ((int64_t)gw * args.units_per_wave + min(gw, args.units_rem)) * 16;
   const int64_t r_last =
       min(args.rows, r_first + ((int64_t)args.units_per_wave + (gw < args.units_rem ? 1 : 0)) * 16);
-  const int n_steps = (int)((r_last - r_first + SS_WAVE_ROWS - 1) / SS_WAVE_ROWS);
+  // SHARE: the waves of a workgroup stream in step: all take as many steps as its first wave, which has the most
+  // rows; a wave whose rows have run out streams the pass's first row and drops the result.
+  const int gw0 = SHARE ? blockIdx.x * 4 : gw;
+  const int n_steps = (int)((((int64_t)args.units_per_wave + (gw0 < args.units_rem ? 1 : 0)) * 16 + SS_WAVE_ROWS - 1) /
+                            SS_WAVE_ROWS);
 
   if (args.first_pass && blockIdx.x == 0 && tid < args.Q) args.cand_count[tid] = (uint32_t)args.rows;
 
-  // Every wave walks D from its own starting k-pair (a multiple of the queue length) and wraps around: at any
-  // moment the waves of the chip then read different parts of the query table, whose 4 KB stretches would
-  // otherwise each be wanted by every wave at once.  A step is two segments, [rot, nkp) and [0, rot).
-  const int rot = stream_rotation(nkp, gw);
+  // Every wave (SHARE: every workgroup) walks D from its own starting k-pair (a multiple of the queue length) and
+  // wraps around: at any moment the waves of the chip then read different parts of the query table, whose 4 KB
+  // stretches would otherwise each be wanted by all of them at once.  A step is two segments, [rot, nkp) and [0, rot).
+  const int rot = stream_rotation(nkp, SHARE ? (int)blockIdx.x : gw);
   const int nseg = rot > 0 ? 2 : 1;
   constexpr int KP = 2 * M::KS;        // elements of a k-pair
   constexpr int FP = 2 * QB * WAVE;    // table entries of a k-pair
 
   uint4 v[STREAM_Q][RG];
-  uint4 rq[STREAM_Q][2 * QB];
+  uint4 rq[SHARE ? 1 : STREAM_Q][2 * QB];  // per-wave fragment queue
+  uint4 rs[2 * QB];                        // SHARE: this wave's k-pair of the next block of fragments
   f32x4 acc[SS_MTW * QB];
   float ssq[RG];
   bool primed = false;
@@ -1097,26 +1110,34 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void scan_stream_kernel(ScanArg
     const int step = item / nseg;
     const int sg = item - step * nseg;
     const int64_t prow0 = r_first + (int64_t)step * SS_WAVE_ROWS;  // pass-local first row of this step
-    const int rows_valid = (int)min((int64_t)SS_WAVE_ROWS, r_last - prow0);
+    const int rows_valid = (int)min((int64_t)SS_WAVE_ROWS, r_last - prow0);  // <= 0: none left for this wave
+    const int64_t srow0 = rows_valid > 0 ? prow0 : 0;  // the rows it streams
+    const int srows = max(rows_valid, 1);
     const int k0 = sg == 0 ? rot : 0;
     const int len = nseg == 1 ? nkp : (sg == 0 ? nkp - rot : rot);
     const T* ur[RG];
     const T* un[RG];
-    stream_rows<T, SS_MTW>(store + prow0 * args.store_stride + k0 * KP, args.store_stride, rows_valid, lane, ur);
-    if (!primed) stream_prime<T, SS_MTW, true, QB>(ur, len, qfrag + k0 * FP, lane, v, rq);
+    stream_rows<T, SS_MTW>(store + srow0 * args.store_stride + k0 * KP, args.store_stride, srows, lane, ur);
+    if (!primed) {
+      if constexpr (SHARE)
+        stream_prime_shared<T, SS_MTW, QB>(ur, len, qfrag + k0 * FP, lane, wave, v, rs);
+      else
+        stream_prime<T, SS_MTW, true, QB>(ur, len, qfrag + k0 * FP, lane, v, rq);
+    }
     int len_next = 0;
     int k1 = 0;
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg) un[rg] = ur[rg];
     if (sg + 1 < nseg) {
       // the same rows from k-pair 0
-      stream_rows<T, SS_MTW>(store + prow0 * args.store_stride, args.store_stride, rows_valid, lane, un);
+      stream_rows<T, SS_MTW>(store + srow0 * args.store_stride, args.store_stride, srows, lane, un);
       len_next = rot;
     } else if (step + 1 < n_steps) {
       const int64_t prow1 = prow0 + SS_WAVE_ROWS;
       const int rows1 = (int)min((int64_t)SS_WAVE_ROWS, r_last - prow1);
       k1 = rot;
-      stream_rows<T, SS_MTW>(store + prow1 * args.store_stride + k1 * KP, args.store_stride, rows1, lane, un);
+      stream_rows<T, SS_MTW>(store + (rows1 > 0 ? prow1 : 0) * args.store_stride + k1 * KP, args.store_stride,
+                             max(rows1, 1), lane, un);
       len_next = nkp - rot;
     }
     if (sg == 0) {
@@ -1125,10 +1146,15 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void scan_stream_kernel(ScanArg
 #pragma unroll
       for (int rg = 0; rg < RG; ++rg) ssq[rg] = 0.f;
     }
-    stream_segment<T, SS_MTW, true, QB, true>(ur, len, un, len_next, qfrag + k0 * FP, qfrag + k1 * FP, stage, lane, v, rq,
-                                              acc, ssq);
+    if constexpr (SHARE)
+      stream_segment_shared<T, SS_MTW, QB, true>(ur, len, un, len_next, qfrag + k0 * FP, qfrag + k1 * FP, stage, ring,
+                                                 ring_slot, lane, wave, v, rs, acc, ssq);
+    else
+      stream_segment<T, SS_MTW, true, QB, true>(ur, len, un, len_next, qfrag + k0 * FP, qfrag + k1 * FP, stage, lane, v,
+                                                rq, acc, ssq);
     primed = len_next > 0;
     if (sg + 1 < nseg) continue;
+    if (rows_valid <= 0) continue;  // nothing of this wave's in the step (no workgroup barrier below)
 
     // ---- row norms: lane (rho, sig) carried slot sig of row rg * 8 + rho; a row's 8 lanes add up ----
     __builtin_amdgcn_wave_barrier();
@@ -1649,9 +1675,10 @@ size_t scan_workspace_bytes_for(int Q, int k, int64_t chunk_rows, int64_t D, int
 
 template <typename T>
 static int launch_stream(const ScanArgs& a, int blocks, const uint4* table, int wgs, hipStream_t st) {
-  // stage slots, score blocks (pitch 16 * blocks + 1 floats), row multipliers
+  // stage slots, score blocks (pitch 16 * blocks + 1 floats), row multipliers, the fragment ring (three blocks)
   const size_t smem = 4 * Stream<SS_MTW>::BYTES_PER_WAVE +
-                      4 * SS_WAVE_ROWS * (size_t)(16 * blocks + 1) * sizeof(float) + 4 * SS_WAVE_ROWS * sizeof(float);
+                      4 * SS_WAVE_ROWS * (size_t)(16 * blocks + 1) * sizeof(float) + 4 * SS_WAVE_ROWS * sizeof(float) +
+                      (blocks >= 3 ? (size_t)stream_ring_bytes(blocks) : 0);
   auto go = [&](auto kern) -> int {
     BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(COLLECT_THREADS), smem, st, a, table);

@@ -284,13 +284,13 @@ __device__ inline void stream_prime_shared(const T* const (&urow)[2 * MTW], int 
 
 // ring: the two LDS slots (stream_ring_bytes); ring_slot: which of them the block that comes next uses (kept by the
 // caller across segments)
-template <typename T, int MTW, int QB>
+template <typename T, int MTW, int QB, bool SUMSQ = false>
 __device__ inline void stream_segment_shared(const T* const (&cur)[2 * MTW], int nkp, const T* const (&nxt)[2 * MTW],
                                              int nkp_next, const uint4* __restrict__ rf,
                                              const uint4* __restrict__ rf_next, unsigned char* __restrict__ stage,
                                              uint4* __restrict__ ring, int& ring_slot, int lane, int wave,
                                              uint4 (&v)[STREAM_Q][2 * MTW], uint4 (&rs)[2 * QB],
-                                             f32x4 (&acc)[MTW * QB]) {
+                                             f32x4 (&acc)[MTW * QB], float* __restrict__ ssq = nullptr) {
   using M = Mma<T>;
   using St = Stream<MTW>;
   constexpr int RG = St::RG;
@@ -331,7 +331,10 @@ __device__ inline void stream_segment_shared(const T* const (&cur)[2 * MTW], int
       constexpr int j = decltype(j_tag)::value;
       if (j < len) {
 #pragma unroll
-        for (int rg = 0; rg < RG; ++rg) *reinterpret_cast<uint4*>(stage + rg * 1024 + lane * 16) = v[j][rg];
+        for (int rg = 0; rg < RG; ++rg) {
+          *reinterpret_cast<uint4*>(stage + rg * 1024 + lane * 16) = v[j][rg];
+          if constexpr (SUMSQ) ssq[rg] = Mma32<T>::sumsq(v[j][rg], ssq[rg]);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
       const int jj = j < len_next ? j : 0;
