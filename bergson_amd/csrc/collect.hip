@@ -429,7 +429,7 @@ __global__ __launch_bounds__(COLLECT_THREADS) void frag_prepare_kernel(const bgx
 // tile, and a wave without tokens in a tile streams that tile's first row and discards what it gets.
 template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED = false, bool RFG = false, int PB = 1>
 __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(PersistArgs pa) {
-  static_assert(STAGED || !RFG, "the global fragment table is read through the stream's queue");
+  static_assert(STAGED || !RFG, "the global fragment table goes with the streamed rows");
   static_assert(PB == 1 || RFG, "wider projections: fragments from the table");
   constexpr bool SHARE = RFG;
   using M = Mma<T>;

@@ -127,10 +127,10 @@ __device__ inline int stream_rotation(int nkp, int gw) {
 // at its worst case, a full drain).  For module widths that are multiples of STREAM_Q k-pairs the only
 // such repeats are at the end of a wave's last tile.
 //
-// With RFG the projection fragments do not sit in LDS (modules too wide for it) but in a table in global
-// memory, in the same fragment order, written by frag_prepare_kernel before the launch; they then travel
-// through the same queue: two 1 KB fragment loads per k-pair behind the wave's 2 * MTW row loads.  They are
-// ordinary cached loads -- every workgroup of a module reads the same table.
+// With RFG the fragments do not sit in LDS but in a table in global memory, in the same fragment order (the
+// few-queries scan's query table; the collection kernel uses stream_segment_shared below for its projection
+// table); they then travel through the same queue: two 1 KB fragment loads per k-pair and block of columns behind
+// the wave's 2 * MTW row loads.  They are ordinary cached loads -- every wave reads the same table.
 //
 // QB = fragment blocks of 16 columns per k-step (1 for a projection to p <= 16; the few-queries scan uses one
 // block per 16 queries): acc[mt * QB + qb], table fragment ((k-step) * QB + qb).  SUMSQ also accumulates, per
