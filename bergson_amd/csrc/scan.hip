@@ -1040,7 +1040,9 @@ __global__ __launch_bounds__(SW_THREADS) void scan_wide_kernel(ScanArgs args) {
 constexpr int SS_MTW = 4;                // 16-row blocks per wave
 constexpr int SS_WAVE_ROWS = 16 * SS_MTW;
 constexpr int SS_TILE_ROWS = 4 * SS_WAVE_ROWS;
-constexpr int SS_MAX_QUERIES = 48;       // up to three blocks of 16 queries (a fourth gains nothing over the tiles)
+constexpr int SS_MAX_QUERIES = 96;       // up to six blocks of 16 queries (LDS: the fragment ring is 16 KB per block)
+// blocks of 16 queries whose scores pass through LDS together on their way to the rows' lanes
+constexpr int ss_score_blocks(int qb) { return qb <= 3 ? qb : (qb <= 5 ? 2 : 1); }
 
 template <typename T>
 __global__ __launch_bounds__(COLLECT_THREADS) void scan_query_fragments_kernel(const T* __restrict__ queries, int Q,
@@ -1063,7 +1065,8 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void scan_stream_kernel(ScanArg
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   unsigned char* stage = smem + wave * St::BYTES_PER_WAVE;
-  constexpr int SC_PITCH = 16 * QB + 1;  // floats per row of the wave's score block in LDS (odd: no bank conflicts)
+  constexpr int EB = ss_score_blocks(QB);
+  constexpr int SC_PITCH = 16 * EB + 1;  // floats per row of the wave's score block in LDS (odd: no bank conflicts)
   float* sc = reinterpret_cast<float*>(smem + 4 * St::BYTES_PER_WAVE) + wave * (SS_WAVE_ROWS * SC_PITCH);
   float* wrow = reinterpret_cast<float*>(smem + 4 * St::BYTES_PER_WAVE) + 4 * (SS_WAVE_ROWS * SC_PITCH) +
                 wave * SS_WAVE_ROWS;  // row multipliers
@@ -1174,24 +1177,30 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void scan_stream_kernel(ScanArg
     }
     __builtin_amdgcn_wave_barrier();
 
-    // ---- scores: through LDS, so that lane l owns row l and walks the queries in a plain loop -------------
+    // ---- scores: through LDS, EB blocks of queries at a time, so that lane l owns row l and walks the queries
+    // in a plain loop -------------
+    const int row = lane;
+    const bool row_ok = row < rows_valid;
+    const int64_t prow = prow0 + row;
+    const int64_t grow = args.row0 + prow;
+    const float w = wrow[row];
+    float rmax = -INFINITY;
+    float rsum = 0.f;
 #pragma unroll
-    for (int mt = 0; mt < SS_MTW; ++mt)
+    for (int g0 = 0; g0 < QB; g0 += EB) {
+      if (g0 > 0) __builtin_amdgcn_wave_barrier();  // the lanes have read the blocks before
 #pragma unroll
-      for (int qb = 0; qb < QB; ++qb)
+      for (int mt = 0; mt < SS_MTW; ++mt)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) sc[(mt * 16 + q4 * 4 + e) * SC_PITCH + qb * 16 + c] = acc[mt * QB + qb][e];
-    __builtin_amdgcn_wave_barrier();
-    {
-      const int row = lane;
-      const bool row_ok = row < rows_valid;
-      const int64_t prow = prow0 + row;
-      const int64_t grow = args.row0 + prow;
-      const float w = wrow[row];
-      float rmax = -INFINITY;
-      float rsum = 0.f;
-      for (int qi = 0; qi < args.Q; ++qi) {
-        const float val = sc[row * SC_PITCH + qi] * w;
+        for (int eb = 0; eb < EB; ++eb)
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (g0 + eb < QB)
+              sc[(mt * 16 + q4 * 4 + e) * SC_PITCH + eb * 16 + c] = acc[mt * QB + g0 + eb][e];
+      __builtin_amdgcn_wave_barrier();
+      const int q_end = min(args.Q, (g0 + EB) * 16);
+      for (int qi = g0 * 16; qi < q_end; ++qi) {
+        const float val = sc[row * SC_PITCH + qi - g0 * 16] * w;
         const float thr = args.thr != nullptr ? args.thr[qi] : INFINITY;
         if (row_ok) {
           rmax = fmaxf(rmax, val);
@@ -1205,10 +1214,10 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void scan_stream_kernel(ScanArg
           }
         }
       }
-      if (row_ok) {
-        if (args.row_max_enc != nullptr) atomicMax(&args.row_max_enc[grow], f32_ordered(rmax));
-        if (args.row_sum_part != nullptr) args.row_sum_part[prow * args.n_parts] = rsum;
-      }
+    }
+    if (row_ok) {
+      if (args.row_max_enc != nullptr) atomicMax(&args.row_max_enc[grow], f32_ordered(rmax));
+      if (args.row_sum_part != nullptr) args.row_sum_part[prow * args.n_parts] = rsum;
     }
     __builtin_amdgcn_wave_barrier();  // sc and wrow are rewritten by the next tile
   }
@@ -1675,17 +1684,22 @@ size_t scan_workspace_bytes_for(int Q, int k, int64_t chunk_rows, int64_t D, int
 
 template <typename T>
 static int launch_stream(const ScanArgs& a, int blocks, const uint4* table, int wgs, hipStream_t st) {
-  // stage slots, score blocks (pitch 16 * blocks + 1 floats), row multipliers, the fragment ring (three blocks)
+  // stage slots, score blocks (pitch 16 * ss_score_blocks + 1 floats), row multipliers, the fragment ring (three
+  // blocks and more)
   const size_t smem = 4 * Stream<SS_MTW>::BYTES_PER_WAVE +
-                      4 * SS_WAVE_ROWS * (size_t)(16 * blocks + 1) * sizeof(float) + 4 * SS_WAVE_ROWS * sizeof(float) +
-                      (blocks >= 3 ? (size_t)stream_ring_bytes(blocks) : 0);
+                      4 * SS_WAVE_ROWS * (size_t)(16 * ss_score_blocks(blocks) + 1) * sizeof(float) +
+                      4 * SS_WAVE_ROWS * sizeof(float) + (blocks >= 3 ? (size_t)stream_ring_bytes(blocks) : 0);
   auto go = [&](auto kern) -> int {
     BGX_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(COLLECT_THREADS), smem, st, a, table);
     return 0;
   };
-  const int rc = blocks == 1 ? go(scan_stream_kernel<T, 1>) : blocks == 2 ? go(scan_stream_kernel<T, 2>)
-                                                              : go(scan_stream_kernel<T, 3>);
+  const int rc = blocks == 1   ? go(scan_stream_kernel<T, 1>)
+                 : blocks == 2 ? go(scan_stream_kernel<T, 2>)
+                 : blocks == 3 ? go(scan_stream_kernel<T, 3>)
+                 : blocks == 4 ? go(scan_stream_kernel<T, 4>)
+                 : blocks == 5 ? go(scan_stream_kernel<T, 5>)
+                               : go(scan_stream_kernel<T, 6>);
   if (rc != 0) return rc;
   BGX_HIP(hipGetLastError());
   return 0;

@@ -682,7 +682,7 @@ def scan(store: Tensor, queries: Tensor, *, unit_norm: bool, k: int = 0, query_s
     if want_sumsq and row_sumsq is None:
         res.sumsq = torch.empty((n,), dtype=torch.float32, device=dev)
     ws = None
-    if k or want_row_mean or Q <= 48:  # few queries: the streaming kernel keeps its query fragments there
+    if k or want_row_mean or Q <= 96:  # few queries: the streaming kernel keeps its query fragments there
         ws = _workspace(dev, lib.bgx_scan_workspace_bytes_for(Q, k, chunk_rows, D, dtype_code(store.dtype)), "scan")
     if row_sumsq is not None:
         _need_gpu(row_sumsq, "row_sumsq")

@@ -398,7 +398,7 @@ int bgx_unit_normalize_rows(void* rows_dev, int64_t n_rows, int64_t D,
 size_t bgx_scan_workspace_bytes(int32_t Q, int32_t k, int64_t chunk_rows);
 /* The same plus room for a table of the queries as matrix-core fragments
  * (1 KB per block of 16 queries and k-step: 32 elements of D at 16 bits, 16 at
- * fp32): with it, scans with at most 48 queries over at least 512 rows per
+ * fp32): with it, scans with at most 96 queries over at least 512 rows per
  * compute unit, D a multiple of two k-steps, stream the store with the
  * few-queries kernel; without it they use the tiled kernel.  A workspace is then needed
  * even when neither top-k nor row means are asked for.  bgx_scan accepts

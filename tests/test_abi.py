@@ -97,7 +97,9 @@ def test_workspace_sizes():
     assert lib.bgx_scan_workspace_bytes_for(20, 100, 0, 12288, 0) == padded + 2 * (12288 // 16) * 1024
     base33 = -(-lib.bgx_scan_workspace_bytes(33, 100, 0) // 256) * 256
     assert lib.bgx_scan_workspace_bytes_for(33, 100, 0, 12288, 1) == base33 + 3 * (12288 // 32) * 1024   # three blocks
-    assert lib.bgx_scan_workspace_bytes_for(49, 100, 0, 12288, 1) == -(-lib.bgx_scan_workspace_bytes(49, 100, 0) // 256) * 256
+    base96 = -(-lib.bgx_scan_workspace_bytes(96, 100, 0) // 256) * 256
+    assert lib.bgx_scan_workspace_bytes_for(96, 100, 0, 12288, 1) == base96 + 6 * (12288 // 32) * 1024   # six: the most
+    assert lib.bgx_scan_workspace_bytes_for(97, 100, 0, 12288, 1) == -(-lib.bgx_scan_workspace_bytes(97, 100, 0) // 256) * 256
     assert lib.bgx_scan_workspace_bytes_for(20, 100, 0, 12288 + 32, 1) == padded   # not two k-steps: no table
     # per-sequence rows through the weight-shaped gradient: p * p fp32 values per sequence and 64 x 64 tile, and
     # per group of 16 tiles

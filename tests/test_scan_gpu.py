@@ -180,7 +180,7 @@ def test_scan_row_mean_alone(device, Q):
 
 
 # ---- few queries over a long store: the streaming kernel ------------------------------------------------
-# At most 48 queries, a row length that is a multiple of two MFMA k-steps and at least two tiles of 256 rows
+# At most 96 queries, a row length that is a multiple of two MFMA k-steps and at least two tiles of 256 rows
 # per compute unit route the scan through the streaming kernel: a first pass of one tile per compute unit
 # without thresholds (one candidate per row, cut down by the select kernel's sample bound), then the rest.
 STREAM_ROWS = 2 * 256 * 256 + 9001  # past the minimum, with a ragged last tile
@@ -188,7 +188,9 @@ STREAM_ROWS = 2 * 256 * 256 + 9001  # past the minimum, with a ragged last tile
 
 @pytest.mark.parametrize("dtype,D,Q", [(torch.float16, 128, 5), (torch.float16, 320, 32), (torch.bfloat16, 192, 16),
                                        (torch.bfloat16, 64, 23), (torch.float32, 96, 8), (torch.float32, 32, 32),
-                                       (torch.float16, 128, 33), (torch.bfloat16, 192, 48), (torch.float32, 64, 41)])
+                                       (torch.float16, 128, 33), (torch.bfloat16, 192, 48), (torch.float32, 64, 41),
+                                       (torch.float16, 192, 49), (torch.bfloat16, 128, 64), (torch.float32, 64, 70),
+                                       (torch.float16, 64, 80), (torch.bfloat16, 320, 96), (torch.float32, 32, 91)])
 def test_scan_streamed_few_queries(device, dtype, D, Q):
     from bergson_amd import _lib, ops
 
