@@ -380,6 +380,30 @@ def test_two_step_token_rows_equal_the_one_step_rows_bitwise(device, out_dtype, 
     assert two.abs().max().item() == 2.0 and (two != 0).any(dim=1).all()   # the clamp bit; every row was written
 
 
+def test_two_step_token_rows_of_wide_modules_equal_the_one_step_rows_bitwise(device, bgx_env, kernel_variant):
+    """The same for modules whose projections do not fit LDS (fragments from the table in global memory, shared by the
+    workgroup's waves): several tiles per sequence, ragged lengths, waves without tokens in the last tile."""
+    from bergson_amd import _lib
+
+    N, S, p = 3, 330, 16
+    lengths = [330, 3, 140]
+    cases = []
+    for i, (I, O) in enumerate([(4096, 1024), (512, 4608)]):
+        a, g, left, right, norm = make_case(N, S, I, O, p, torch.bfloat16, seed=230 + i,
+                                            normalizer="adafactor" if i == 0 else None, name=f"layers.{i}.wide")
+        cases.append((a, g, left, right, norm))
+    counts = [l - 1 for l in lengths]
+    kw = dict(lengths=lengths, per_token=True, row_offsets=[sum(counts[:n]) for n in range(N)], n_rows=sum(counts))
+    two = run_kernel(device, cases, p, torch.bfloat16, **kw)
+    route = _lib.last_kernel(_lib.FAMILY_COLLECT)
+    bgx_env("BGX_COLLECT_TWO_STEP_OFF", "1")
+    one = run_kernel(device, cases, p, torch.bfloat16, **kw)
+    bgx_env("BGX_COLLECT_TWO_STEP_OFF", None)
+    assert route == ("collect_persist_table" if kernel_variant == "streamed" else "collect_tile")
+    assert torch.equal(two, one)
+    assert (two != 0).any(dim=1).all()
+
+
 def test_tok_rows_sum_to_seq_row(device):
     # sum over tokens of the per-token rows equals the per-sequence row (fp32)
     N, S, p = 2, 77, 16
