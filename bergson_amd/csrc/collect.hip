@@ -427,8 +427,12 @@ __global__ __launch_bounds__(COLLECT_THREADS) void frag_prepare_kernel(const bgx
 // With RFG the workgroup's waves load each block of table fragments once between them and pass it round through LDS
 // (stream_segment_shared: SHARE below) instead of each loading all of it; all four then stream in step, tile after
 // tile, and a wave without tokens in a tile streams that tile's first row and discards what it gets.
-template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED = false, bool RFG = false, int PB = 1>
+// BIAS: the launch has modules with a bias column and no bias factor of their own (bias_col without bias_scale):
+// their P is sum_t g'_t (x) (a'_t + bias_col), so the column is added to a' of every token before the reduction.
+template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED = false, bool RFG = false, int PB = 1,
+          bool BIAS = false>
 __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(PersistArgs pa) {
+  static_assert(!BIAS || (STAGED && PB == 1), "the bias column goes with the streamed kernels at p <= 16");
   static_assert(STAGED || !RFG, "the global fragment table goes with the streamed rows");
   static_assert(PB == 1 || RFG, "wider projections: fragments from the table");
   constexpr bool SHARE = RFG;
@@ -541,6 +545,14 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
     const int64_t t0 = s0 + (SHARE && rows_valid <= 0 ? 0 : wave * WAVE_T);
     const T* a0 = (const T*)d.a + (int64_t)n * d.a_seq_stride + t0 * d.a_tok_stride;
     const T* g0 = (const T*)d.g + (int64_t)n * d.g_seq_stride + t0 * d.g_tok_stride;
+    // BIAS: this lane's entry of the bias column, loaded here, ahead of the tile's stream, so that the wait for it
+    // further down has none of the stream's loads in front of it; unconditionally (a load behind a branch would
+    // make every wait at the join a full drain): a module without the column reads the descriptor table instead
+    float bias_v = 0.f;
+    if constexpr (BIAS) {
+      const float* bp = d.bias_col != nullptr ? d.bias_col : reinterpret_cast<const float*>(args.mods);
+      bias_v = bp[min(c, p - 1)];
+    }
     if constexpr (STAGED) {
       // a tile nothing ran ahead into (the first of the range, or after padding): its first loads go out
       // before the projections are staged
@@ -621,6 +633,13 @@ __global__ __launch_bounds__(COLLECT_THREADS, 1) void collect_persist_kernel(Per
       } else if constexpr (PB == 1) {
         project_tokens_lds<T, MTW, U>(a0, d.a_tok_stride, rows_valid, d.I, rfA, lane, accA);
         project_tokens_lds<T, MTW, U>(g0, d.g_tok_stride, rows_valid, d.O, rfG, lane, accG);
+      }
+      if constexpr (BIAS) {
+        const float b = d.bias_col != nullptr && c < p ? bias_v : 0.f;
+#pragma unroll
+        for (int mt = 0; mt < MTW; ++mt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) accA[mt][i] += b;
       }
       // token rows past the last valid one hold garbage: zero them in g' (that removes their products)
 #pragma unroll
@@ -995,13 +1014,13 @@ static int table_blocks(int p) {
 }
 
 // Bytes of the global fragment table for these modules (1 KB per k-step of I + O and block of 16 projection
-// columns), or 0 when the table cannot be used: a width that is not a multiple of two k-steps, p > 64, a bias column.
+// columns), or 0 when the table cannot be used: a width that is not a multiple of two k-steps, p > 64, a bias column with a factor of its own.
 static size_t fragment_table_bytes(const bgx_module_desc* mods, int n_modules, int p, int in_dtype) {
   if (p > 16 * PERSIST_MAX_PB) return 0;
   const int kstep = in_dtype == BGX_F32 ? 16 : 32;
   size_t steps = 0;
   for (int m = 0; m < n_modules; ++m) {
-    if (mods[m].I <= 0 || mods[m].O <= 0 || mods[m].I % (2 * kstep) || mods[m].O % (2 * kstep) || mods[m].bias_col)
+    if (mods[m].I <= 0 || mods[m].O <= 0 || mods[m].I % (2 * kstep) || mods[m].O % (2 * kstep) || mods[m].bias_scale)
       return 0;
     steps += (size_t)(mods[m].I + mods[m].O) / kstep;
   }
@@ -1100,9 +1119,9 @@ static int compute_units(int* out) {
   return 0;
 }
 
-template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED, bool RFG, int PB = 1>
+template <typename T, bool PER_TOKEN, int MTW, int U, bool STAGED, bool RFG, int PB = 1, bool BIAS = false>
 static int launch_persist_one(int wgs, size_t lds, hipStream_t st, const PersistArgs& pa) {
-  auto kern = collect_persist_kernel<T, PER_TOKEN, MTW, U, STAGED, RFG, PB>;
+  auto kern = collect_persist_kernel<T, PER_TOKEN, MTW, U, STAGED, RFG, PB, BIAS>;
   // the opt-in to more than 64 KB of dynamic LDS is per kernel and per device; do it once for each
   static std::atomic<bool> opted_in[MAX_DEVICES];
   int dev = 0;
@@ -1115,14 +1134,14 @@ static int launch_persist_one(int wgs, size_t lds, hipStream_t st, const Persist
   return 0;
 }
 
-template <typename T, bool STAGED, bool RFG>
+template <typename T, bool STAGED, bool RFG, bool BIAS = false>
 static int launch_persist_s(bool per_token, int tile_tokens, int wgs, size_t lds, hipStream_t st,
                             const PersistArgs& pa) {
   if (tile_tokens == 128)
-    return per_token ? launch_persist_one<T, true, 2, 4, STAGED, RFG>(wgs, lds, st, pa)
-                     : launch_persist_one<T, false, 2, 4, STAGED, RFG>(wgs, lds, st, pa);
-  return per_token ? launch_persist_one<T, true, 1, 8, STAGED, RFG>(wgs, lds, st, pa)
-                   : launch_persist_one<T, false, 1, 8, STAGED, RFG>(wgs, lds, st, pa);
+    return per_token ? launch_persist_one<T, true, 2, 4, STAGED, RFG, 1, BIAS>(wgs, lds, st, pa)
+                     : launch_persist_one<T, false, 2, 4, STAGED, RFG, 1, BIAS>(wgs, lds, st, pa);
+  return per_token ? launch_persist_one<T, true, 1, 8, STAGED, RFG, 1, BIAS>(wgs, lds, st, pa)
+                   : launch_persist_one<T, false, 1, 8, STAGED, RFG, 1, BIAS>(wgs, lds, st, pa);
 }
 
 // the variants with the fragments in the global table; pb: blocks of 16 projection columns (more than one: tiles of
@@ -1148,9 +1167,13 @@ static int launch_persist_table(bool per_token, int pb, int tile_tokens, int wgs
 }
 
 // staged: streamed token rows; rfg: (staged only) projection fragments from the global table
+// bias: modules with a bias column in the launch (streamed variants at p <= 16 only: the caller routes so)
 template <typename T>
-static int launch_persist(bool staged, bool rfg, bool per_token, int pb, int tile_tokens, int wgs, size_t lds,
-                          hipStream_t st, const PersistArgs& pa) {
+static int launch_persist(bool staged, bool rfg, bool bias, bool per_token, int pb, int tile_tokens, int wgs,
+                          size_t lds, hipStream_t st, const PersistArgs& pa) {
+  if (bias)
+    return rfg ? launch_persist_s<T, true, true, true>(per_token, tile_tokens, wgs, lds, st, pa)
+               : launch_persist_s<T, true, false, true>(per_token, tile_tokens, wgs, lds, st, pa);
   if (rfg) return launch_persist_table<T>(per_token, pb, tile_tokens, wgs, lds, st, pa);
   return staged ? launch_persist_s<T, true, false>(per_token, tile_tokens, wgs, lds, st, pa)
                 : launch_persist_s<T, false, false>(per_token, tile_tokens, wgs, lds, st, pa);
@@ -1181,7 +1204,8 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   const int epl = in_dtype == BGX_F32 ? 4 : 8;
   const int kstep = in_dtype == BGX_F32 ? 16 : 32;
   bool aligned = true;
-  bool any_bias = false;
+  bool any_bias = false;     // modules with a bias column ...
+  bool scaled_bias = false;  // ... and with a factor of its own on it (a second projection of g: tile kernel only)
   for (int m = 0; m < n_modules; ++m) {
     const bgx_module_desc& d = mods_host[m];
     BGX_REQUIRE(d.a && d.g && d.r_in && d.r_out, BGX_E_ARG, "collect: module %d has a null a/g/r_in/r_out", m);
@@ -1192,6 +1216,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     BGX_REQUIRE(d.bias_col != nullptr || d.bias_scale == nullptr, BGX_E_ARG,
                 "collect: module %d has a bias_scale but no bias_col", m);
     any_bias = any_bias || d.bias_col != nullptr;
+    scaled_bias = scaled_bias || d.bias_scale != nullptr;
     const bool ok = ((uintptr_t)d.a % 16 == 0) && ((uintptr_t)d.g % 16 == 0) &&
                     ((uintptr_t)d.r_in % 16 == 0) && ((uintptr_t)d.r_out % 16 == 0) &&
                     (d.I % kstep == 0) && (d.O % kstep == 0) && (d.a_seq_stride % epl == 0) &&
@@ -1234,7 +1259,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   const bool wide = pb > 1 && pb <= PERSIST_MAX_PB && (!per_token || wide_tok) && aligned && !any_bias &&
                     frag_bytes > 0 && ws_bytes >= lay.frag + frag_bytes && switches().collect_staged &&
                     switches().collect_persist;
-  int tile_tokens = tile_tokens_for(pb, aligned, any_bias, S);
+  int tile_tokens = tile_tokens_for(pb, aligned, scaled_bias, S);
   if (wide && per_token) tile_tokens = 128;
   if (wide && !per_token) {
     // 256 tokens where the sequence length wastes little of a wave's 64 (measured 208 us against 225 us at p = 32
@@ -1242,7 +1267,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     tile_tokens = pb == 2 && (int64_t)((S + 63) / 64 * 64) * 100 <= (int64_t)S * 104 ? 256 : 128;
   }
   args.tiles_per_seq = (S + tile_tokens - 1) / tile_tokens;
-  const int64_t tiles = (int64_t)N * args.tiles_per_seq;
+  int64_t tiles = (int64_t)N * args.tiles_per_seq;
   BGX_REQUIRE(tiles <= 0x7fffffffLL, BGX_E_SHAPE, "collect: %lld tiles exceed the grid limit", (long long)tiles);
 
   // The persistent variant needs every module's projection fragments (16 rows x (I + O) elements) to
@@ -1253,7 +1278,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
       per_token ? persist_scratch_bytes(tile_tokens, wide ? table_blocks(p) : 1)
                 : (wide ? (size_t)4 * WAVE * 16 * table_blocks(p) * table_blocks(p) : (size_t)2 * 3 * WAVE * 16);
   size_t persist_lds = (size_t)r_steps * 1024 + scratch_bytes;
-  bool persist = pb == 1 && aligned && !any_bias && persist_lds <= LDS_PER_WG &&
+  bool persist = pb == 1 && aligned && !scaled_bias && persist_lds <= LDS_PER_WG &&
                  tiles * n_modules <= 0x7fffffffLL;
   // staging rings for fully coalesced loads: every K a multiple of two k-steps, and 32 KB more of LDS
   const size_t stage_bytes = (size_t)4 * (tile_tokens == 256   ? Stream<4>::BYTES_PER_WAVE
@@ -1267,7 +1292,7 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   // Modules too wide for LDS: the streamed kernel with the fragments in a global table, when the caller's
   // workspace has room for it (bgx_collect_workspace_bytes_for) -- else the tile kernel.
   const size_t frag_ws_off = lay.frag;
-  bool rfg = !persist && (pb == 1 || wide) && aligned && !any_bias && tiles * n_modules <= 0x7fffffffLL && frag_bytes > 0 &&
+  bool rfg = !persist && (pb == 1 || wide) && aligned && !scaled_bias && tiles * n_modules <= 0x7fffffffLL && frag_bytes > 0 &&
              ws_bytes >= frag_ws_off + frag_bytes;
   rfg = rfg && switches().collect_staged;
   if (rfg) {  // beside the rest: the ring through which the workgroup shares the table's fragments
@@ -1277,7 +1302,15 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
   }
   // BGX_COLLECT_PERSIST=0 in the environment forces the one-workgroup-per-tile kernel (tests, comparisons)
   persist = persist && switches().collect_persist;
+  // a bias column goes with the streamed variants only
+  if (any_bias && !staged) persist = false;
   rfg = rfg && persist;
+  if (!persist && any_bias && tile_tokens != 64) {  // the tile kernel's bias variant runs on 64-token tiles
+    tile_tokens = 64;
+    args.tiles_per_seq = (S + tile_tokens - 1) / tile_tokens;
+    tiles = (int64_t)N * args.tiles_per_seq;
+    BGX_REQUIRE(tiles <= 0x7fffffffLL, BGX_E_SHAPE, "collect: %lld tiles exceed the grid limit", (long long)tiles);
+  }
 
   std::vector<unsigned char> head((size_t)n_modules * sizeof(bgx_module_desc));
   memcpy(head.data(), sorted.data(), head.size());
@@ -1428,11 +1461,11 @@ int collect_impl(bool per_token, const bgx_module_desc* mods_host, int n_modules
     pa.tokproj = two_step ? (float*)((char*)ws + lay.tokproj) : nullptr;
     int rc;
     if (in_dtype == BGX_F32)
-      rc = launch_persist<float>(staged, rfg, per_token, pb, tile_tokens, wgs, persist_lds, st, pa);
+      rc = launch_persist<float>(staged, rfg, any_bias, per_token, pb, tile_tokens, wgs, persist_lds, st, pa);
     else if (in_dtype == BGX_F16)
-      rc = launch_persist<f16_t>(staged, rfg, per_token, pb, tile_tokens, wgs, persist_lds, st, pa);
+      rc = launch_persist<f16_t>(staged, rfg, any_bias, per_token, pb, tile_tokens, wgs, persist_lds, st, pa);
     else
-      rc = launch_persist<bf16_t>(staged, rfg, per_token, pb, tile_tokens, wgs, persist_lds, st, pa);
+      rc = launch_persist<bf16_t>(staged, rfg, any_bias, per_token, pb, tile_tokens, wgs, persist_lds, st, pa);
     if (rc != 0) return rc;
     note_kernel(FAMILY_COLLECT, rfg ? "collect_persist_table" : staged ? "collect_persist_lds" : "collect_persist_direct");
   } else if (in_dtype == BGX_F32) {

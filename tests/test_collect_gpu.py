@@ -550,6 +550,52 @@ def test_bias_column(device, dtype, normalizer, per_token):
     assert rel_l2(out.cpu(), want) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("per_token", [False, True])
+@pytest.mark.parametrize("wide", [False, True])
+def test_bias_column_without_a_factor_on_the_streamed_kernels(device, dtype, per_token, wide, kernel_variant):
+    """A bias column with no factor of its own (no normalizer, or none on the bias) is a constant added to every
+    token's projected activation, which the streamed kernels do in registers; the launch mixes a module with the column
+    and one without, ragged lengths, and (wide) a module whose projections come from the table in global memory."""
+    from bergson_amd import _lib, ops
+
+    N, S, p = 3, 200, 16
+    lengths = [200, 77, 2]
+    shapes = [(128, 192, True), (64, 64, False)]
+    if wide:
+        shapes.append((4096 if dtype == torch.bfloat16 else 2048, 1024, True))
+    gen = torch.Generator().manual_seed(61)
+    mask = (torch.arange(S).unsqueeze(0) + 1) < torch.tensor(lengths).unsqueeze(1)
+    mods, wants, col = [], [], 0
+    for i, (I, O, bias) in enumerate(shapes):
+        a = torch.randn(N, S, I, generator=gen).to(dtype)
+        g = (torch.randn(N, S, O, generator=gen) * 0.1).to(dtype)
+        for n, l in enumerate(lengths):
+            g[n, l - 1:] = 0
+        left, right = module_projections(f"layers.{i}.b", p, O, I, dtype, collect_bias=bias)
+        wants.append(ohooks.module_gradient(a, g, None, left, right, collect_bias=bias, attribute_tokens=per_token,
+                                            collection_mask=mask if per_token else None))
+        mods.append(ops.ModuleInput(a=a.to(device), g=g.to(device), r_in=right[:, :I].contiguous().to(device),
+                                    r_out=left.to(device), out_col=col,
+                                    bias_col=right[:, I].float().contiguous().to(device) if bias else None))
+        col += p * p
+    want = torch.cat(wants, dim=1)
+    ldev = torch.tensor(lengths, dtype=torch.int32, device=device)
+    if per_token:
+        counts = [l - 1 for l in lengths]
+        out = torch.zeros(sum(counts), col, dtype=dtype, device=device)
+        ops.collect_tok(mods, p, out, lengths=ldev,
+                        row_offsets=torch.tensor([sum(counts[:n]) for n in range(N)], dtype=torch.int64, device=device))
+    else:
+        out = torch.zeros(N, col, dtype=dtype, device=device)
+        ops.collect_seq(mods, p, out, lengths=ldev)
+    torch.cuda.synchronize()
+    route = _lib.last_kernel(_lib.FAMILY_COLLECT)
+    assert route == {"streamed": "collect_persist_table" if wide else "collect_persist_lds"}.get(kernel_variant, "collect_tile")
+    assert out.shape == want.shape
+    assert rel_l2(out.cpu(), want) <= TOL[dtype]
+
+
 @pytest.mark.parametrize("per_token", [False, True])
 def test_adam_with_bias(device, per_token):
     from bergson_amd import ops
