@@ -118,8 +118,8 @@ int bgx_adafactor_scales(const float* row_dev, int32_t O, const float* col_dev,
 
 /* Bytes of device workspace bgx_collect_seq / bgx_collect_tok need.
  * bgx_collect_workspace_bytes is the minimum for any modules of that count.
- * bgx_collect_workspace_bytes_for looks at the modules (only I, O and bias_col
- * of each descriptor are read) and adds room for (i) a table of pre-scaled
+ * bgx_collect_workspace_bytes_for looks at the modules (only I, O and
+ * bias_scale of each descriptor are read) and adds room for (i) a table of pre-scaled
  * projection fragments, 32 bytes per input and output feature (64 for
  * 16 < p <= 32, 128 for 32 < p <= 64), and the list of work items behind it
  * (4 bytes per module and 64 tokens): with it, modules too wide for their
