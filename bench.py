@@ -463,7 +463,7 @@ def per_token_leg(args, torch, device):
     return {"workload": "configs[1] modules, per-token rows: 48 Pythia-160m modules, 2 x 2048 tokens, p=16, Adafactor, "
                         "bf16 rows of 12288",
             "ms_per_launch": ms, "tokens_per_s_hooks_only": N * S / (ms * 1e-3),
-            "roofline": {"bound": "hbm", "kernel": "bgx::collect_persist_kernel<bf16_t, true, 2, 4, true, false, 1> (every token's "
+            "roofline": {"bound": "hbm", "kernel": "bgx::collect_persist_kernel<bf16_t, true, 2, 4, true, false, 1, false> (every token's "
                                                   "projections, written contiguously) + bgx::token_rows_kernel (whole store "
                                                   "rows from them), one event pair around both",
                          "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
@@ -579,7 +579,7 @@ def llama_leg(args, torch, device):
     out = {"workload": f"configs[4] shapes: {layers} layers of a Llama-3-8B-shaped decoder (28 modules), 2 x 2048-token "
                        "batches, p=16, Adafactor, fp16 store",
            "tokens_per_s_this_4_layer_model": 4096 * n_batches / dt, "ms_per_step": dt / n_batches * 1e3,
-           "roofline": {"bound": "hbm", "kernel": "bgx::collect_persist_kernel<bf16_t, false, 2, 4, true, true, 1> "
+           "roofline": {"bound": "hbm", "kernel": "bgx::collect_persist_kernel<bf16_t, false, 2, 4, true, true, 1, false> "
                                                   "(streamed loads, projection fragments from a global table, shared by the workgroup through LDS)",
                         "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
                         "bytes_per_launch": nbytes, "ms_per_launch": ms_launch, "launches": len(ms),
@@ -903,7 +903,7 @@ def main():
                               "store flush only"},
         "roofline": {
             "bound": "hbm",
-            "kernel": "bgx::collect_persist_kernel<bf16_t, false, 2, 4, true, false, 1> and <bf16_t, false, 1, 8, true, false, 1> (128- and 64-token tiles, streamed loads, projections in LDS)",
+            "kernel": "bgx::collect_persist_kernel<bf16_t, false, 2, 4, true, false, 1, false> and <bf16_t, false, 1, 8, true, false, 1, false> (128- and 64-token tiles, streamed loads, projections in LDS)",
             "achieved": coll["achieved_gbs"],
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
